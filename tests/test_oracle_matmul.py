@@ -1,0 +1,294 @@
+"""Pins the oracle's matmul / reorder against what the mathematics fixes.
+
+No stored golden tensors exist in the reference (its tests compute expected
+values on the fly), so each check here is chosen so that a plausible mistake
+(dropped zero-point, wrong group index, transposed operand, swapped scale
+order, wrong broadcast) fails it:
+  * exact integer dot products by brute force (numpy int64),
+  * the zero-point compensation identity of
+    src/cpu/matmul/gemm_x8s8s32x_matmul.cpp:165-193,
+  * integer-valued data with power-of-two scales, where every intermediate is
+    exactly representable so any evaluation order gives the same bits (the
+    reason benchdnn can compare matmul with a zero threshold,
+    tests/benchdnn/utils/compare.hpp:74),
+  * pure-Python loops with hand-written index arithmetic for grouped scales
+    and zero points,
+  * a sequential float32 accumulation written with numpy for the float path.
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+
+SWISH, RELU, LINEAR = 0x2C, 0x20, 0x26
+ADD, MUL = 0x1FFF0, 0x1FFF1
+
+
+def T(dt, arr, strides=None, dims=None):
+    arr = np.ascontiguousarray(arr)
+    return O.Tensor(dt, dims if dims is not None else arr.shape, arr, strides)
+
+
+def test_s32_accumulators_are_the_exact_integer_dot_product():
+    rng = np.random.default_rng(0)
+    M, K, N = 7, 96, 10
+    src = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    wei = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    dst = np.zeros((M, N), np.int32)
+    zp = np.array([131], np.int32)
+    acc = O.matmul_s32_acc(T(O.U8, src), T(O.S8, wei), T(O.S32, dst),
+                           zps={O.Q_SRC: O.Quant(0, O.S32, zp)})
+    want = (src.astype(np.int64) - 131) @ wei.astype(np.int64)
+    assert np.array_equal(acc, want)
+    # compensation identity: sum((s-zp)*w) == sum(s*w) - zp*colsum(w)
+    plain = O.matmul_s32_acc(T(O.U8, src), T(O.S8, wei), T(O.S32, dst))
+    assert np.array_equal(acc, plain - 131 * wei.astype(np.int64).sum(0))
+    # a transposed operand must not pass: strides select the layout
+    wt = np.ascontiguousarray(wei.T)
+    acc_t = O.matmul_s32_acc(T(O.U8, src), O.Tensor(O.S8, (K, N), wt, (1, K)), T(O.S32, dst),
+                             zps={O.Q_SRC: O.Quant(0, O.S32, zp)})
+    assert np.array_equal(acc_t, want)
+
+
+def test_int8_exact_arithmetic_any_order():
+    """Small integers and power-of-two scales: all intermediates exact."""
+    rng = np.random.default_rng(1)
+    B, M, K, N = 3, 5, 64, 6
+    src = rng.integers(-4, 5, (B, M, K)).astype(np.int8)
+    wei = rng.integers(-4, 5, (B, K, N)).astype(np.int8)
+    ws = (2.0 ** rng.integers(-2, 3, N)).astype(np.float32)
+    ss = np.array([0.5], np.float32)
+    bias = rng.integers(-8, 9, (1, 1, N)).astype(np.float32)
+    dzp = np.array([3], np.int32)
+    dsc = np.array([2.0], np.float32)
+    dst = np.zeros((B, M, N), np.int8)
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.S8, dst), bias=T(O.F32, bias),
+             scales={O.Q_SRC: O.Quant(0, O.F32, ss), O.Q_WEI: O.Quant(1 << 2, O.F32, ws),
+                     O.Q_DST: O.Quant(0, O.F32, dsc)},
+             zps={O.Q_DST: O.Quant(0, O.S32, dzp)},
+             post_ops=[{"kind": "eltwise", "alg": RELU, "alpha": 0.0}])
+    acc = np.einsum("bmk,bkn->bmn", src.astype(np.float64), wei.astype(np.float64))
+    want = np.maximum(acc * 0.5 * ws + bias, 0) / 2.0 + 3
+    want = np.clip(np.rint(want), -128, 127).astype(np.int8)
+    assert np.array_equal(dst, want)
+
+
+def _py_int8_reference(src, wei, ss, ws, sz, wz, gs, gw, gsz, gwz):
+    """Pure-Python int8 matmul with K-grouped src/wei scales and zero points.
+    Layouts: src quant [M, K/g], wei quant [K/g, N] (row-major)."""
+    M, K = src.shape
+    N = wei.shape[1]
+    gk = min(gs, gw, gsz, gwz)
+    out = np.zeros((M, N), np.float32)
+    for m in range(M):
+        for n in range(N):
+            d = np.float32(0)
+            for g in range(K // gk):
+                acc = 0
+                for k in range(g * gk, (g + 1) * gk):
+                    s = int(src[m, k]) - int(sz[m, k // gsz])
+                    w = int(wei[k, n]) - int(wz[k // gwz, n])
+                    acc += s * w
+                k_last = (g + 1) * gk - 1
+                a = np.float32(acc)
+                a = a * ss[m, k_last // gs]
+                a = a * ws[k_last // gw, n]
+                d = d + a
+            out[m, n] = d
+    return out
+
+
+def test_int8_grouped_scales_and_zero_points_indexing():
+    rng = np.random.default_rng(2)
+    M, K, N = 4, 128, 6
+    gs, gw, gsz, gwz = 64, 32, 128, 64
+    src = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    wei = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    ss = rng.uniform(0.01, 0.1, (M, K // gs)).astype(np.float32)
+    ws = rng.uniform(0.01, 0.1, (K // gw, N)).astype(np.float32)
+    sz = rng.integers(-5, 6, (M, K // gsz)).astype(np.int32)
+    wz = rng.integers(-5, 6, (K // gwz, N)).astype(np.int8)
+    dst = np.zeros((M, N), np.float32)
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.F32, dst),
+             scales={O.Q_SRC: O.Quant(3, O.F32, ss, (1, gs)), O.Q_WEI: O.Quant(3, O.F32, ws, (gw, 1))},
+             zps={O.Q_SRC: O.Quant(3, O.S32, sz, (1, gsz)), O.Q_WEI: O.Quant(3, O.S8, wz, (gwz, 1))})
+    want = _py_int8_reference(src, wei, ss, ws, sz, wz, gs, gw, gsz, gwz)
+    assert np.array_equal(dst.view(np.uint32), want.view(np.uint32))
+
+
+def test_int8_scale_order_is_src_then_weights():
+    """((float)acc * s_src) * s_wei, not acc * (s_src * s_wei):
+    src/cpu/matmul/ref_matmul_int8.cpp:195-218."""
+    rng = np.random.default_rng(3)
+    M, K, N = 64, 256, 64
+    src = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wei = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    ss = rng.uniform(0.005, 0.05, (M, 1)).astype(np.float32)
+    ws = rng.uniform(0.0005, 0.005, N).astype(np.float32)
+    dst = np.zeros((M, N), np.float32)
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.F32, dst),
+             scales={O.Q_SRC: O.Quant(3, O.F32, ss, (1, K)), O.Q_WEI: O.Quant(2, O.F32, ws)})
+    acc = (src.astype(np.int64) @ wei.astype(np.int64)).astype(np.float32)
+    want = (acc * ss) * ws[None, :]
+    other = acc * (ss * ws[None, :])
+    assert np.array_equal(dst.view(np.uint32), want.view(np.uint32))
+    assert not np.array_equal(want.view(np.uint32), other.view(np.uint32))
+
+
+def test_int8_literal_k_grouping_sums_in_f32_one_k_at_a_time():
+    """As written, v3.8 closes the K group after every k when an entry carries no
+    explicit groups (src/cpu/matmul/ref_matmul_int8.cpp:139-144 with
+    src/common/primitive_attr_quant.hpp:83-90): d = sum_k f32(s*w)*ss*ws in f32."""
+    rng = np.random.default_rng(33)
+    M, K, N = 5, 200, 6
+    src = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    wei = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    ss = np.array([0.02], np.float32)
+    zp = np.array([128], np.int32)
+    dst = np.zeros((M, N), np.float32)
+    args = dict(scales={O.Q_SRC: O.Quant(0, O.F32, ss), O.Q_WEI: O.Quant(2, O.F32, ws)},
+                zps={O.Q_SRC: O.Quant(0, O.S32, zp)})
+    O.matmul(T(O.U8, src), T(O.S8, wei), T(O.F32, dst), k_group_mode=O.KGROUP_LITERAL, **args)
+    d = np.zeros((M, N), np.float32)
+    for k in range(K):
+        prod = ((src[:, k].astype(np.int32) - 128)[:, None] * wei[k].astype(np.int32)[None, :]).astype(np.float32)
+        d = d + (prod * ss[0]) * ws[None, :]
+    assert np.array_equal(dst.view(np.uint32), d.view(np.uint32))
+    # the whole-K integer accumulation differs only by f32 summation error
+    dst2 = np.zeros((M, N), np.float32)
+    O.matmul(T(O.U8, src), T(O.S8, wei), T(O.F32, dst2), **args)
+    acc = ((src.astype(np.int64) - 128) @ wei.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(dst2.view(np.uint32), ((acc * ss[0]) * ws[None, :]).view(np.uint32))
+    scale = (np.abs(src.astype(np.float64) - 128) @ np.abs(wei.astype(np.float64))) * 0.02 * ws[None, :]
+    assert np.max(np.abs(dst - dst2) / scale) < 1e-6
+    assert not np.array_equal(dst, dst2)
+
+
+def test_int8_accumulator_rounds_to_f32_above_2_pow_24():
+    K = 4096
+    src = np.full((1, K), 127, np.int8)
+    wei = np.full((K, 2), 127, np.int8)
+    wei[0, 1] = 126  # 66064383 is not representable in f32
+    dst = np.zeros((1, 2), np.float32)
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.F32, dst))
+    assert dst[0, 0] == np.float32(127 * 127 * K)
+    assert 127 * 127 * K - 127 == 66064257 and int(dst[0, 1]) == 66064256  # f32 spacing is 4 there
+
+
+def _bf16(a):
+    return O.from_f32(O.BF16, np.asarray(a, np.float32))
+
+
+def test_weights_decompression_sequential_f32():
+    """bf16 x u4 with group-K f16 scales and u4 zero points, f32 accumulate in k
+    order: src/cpu/matmul/ref_matmul.cpp:140-173."""
+    rng = np.random.default_rng(4)
+    M, K, N, G = 3, 256, 16, 128
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    a_bf = _bf16(a)
+    a = O.to_f32(O.BF16, a_bf)
+    w = rng.integers(0, 16, (K, N))
+    sc = O.from_f32(O.F16, rng.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
+    zp = rng.integers(6, 10, (K // G, N))
+    dst = np.zeros((M, N), np.uint16)
+    O.matmul(T(O.BF16, a_bf), O.Tensor(O.U4, (K, N), O.pack4(w)), T(O.BF16, dst),
+             scales={O.Q_WEI: O.Quant(3, O.F16, sc, (G, 1))},
+             zps={O.Q_WEI: O.Quant(3, O.U4, O.pack4(zp), (G, 1))}, apply_to_int=True)
+    scf = sc.view(np.float16).astype(np.float32)
+    acc = np.zeros((M, N), np.float32)
+    for k in range(K):
+        wk = (w[k].astype(np.float32) - zp[k // G].astype(np.float32)) * scf[k // G]
+        acc = acc + a[:, k, None] * wk[None, :]
+    assert np.array_equal(dst, _bf16(acc))
+    # dropping the zero point or using the wrong group must change the answer
+    acc2 = a @ ((w - 8) * scf.repeat(G, 0)).astype(np.float32)
+    assert not np.array_equal(dst, _bf16(acc2))
+
+
+def test_fp8_path_and_sum_post_op():
+    rng = np.random.default_rng(5)
+    M, K, N = 8, 64, 8
+    a8 = O.from_f32(O.F8_E4M3, np.clip(rng.standard_normal((M, K)) * 4, -448, 448).astype(np.float32))
+    b8 = O.from_f32(O.F8_E4M3, np.clip(rng.standard_normal((K, N)) * 4, -448, 448).astype(np.float32))
+    old = _bf16(rng.standard_normal((M, N)))
+    dst = old.copy()
+    O.matmul(T(O.F8_E4M3, a8), T(O.F8_E4M3, b8), T(O.BF16, dst),
+             scales={O.Q_SRC: O.Quant(0, O.F32, np.array([0.5], np.float32)),
+                     O.Q_WEI: O.Quant(0, O.F32, np.array([0.25], np.float32))},
+             post_ops=[{"kind": "sum", "scale": 1.0}])
+    a, b = O.to_f32(O.F8_E4M3, a8), O.to_f32(O.F8_E4M3, b8)
+    acc = np.zeros((M, N), np.float32)
+    for k in range(K):
+        acc = acc + a[:, k, None] * b[None, k, :]
+    want = (acc * np.float32(0.5)) * np.float32(0.25) + O.to_f32(O.BF16, old)
+    assert np.array_equal(dst, _bf16(want))
+
+
+def test_binary_post_op_broadcast_and_batch():
+    rng = np.random.default_rng(6)
+    B, M, K, N = 4, 6, 32, 5
+    q = rng.integers(-127, 128, (B, M, K)).astype(np.int8)
+    kt = rng.integers(-127, 128, (B, N, K)).astype(np.int8)  # stored as K^T: acb view
+    mask = np.where(np.arange(N)[None, :] > np.arange(M)[:, None], -1e4, 0).astype(np.float32)[None]
+    dst = np.zeros((B, M, N), np.float32)
+    wei = O.Tensor(O.S8, (B, K, N), kt, (N * K, 1, K))
+    O.matmul(T(O.S8, q), wei, T(O.F32, dst),
+             scales={O.Q_SRC: O.Quant(0, O.F32, np.array([0.01], np.float32)),
+                     O.Q_WEI: O.Quant(0, O.F32, np.array([0.012], np.float32))},
+             post_ops=[{"kind": "binary", "alg": ADD, "src1": T(O.F32, mask)}])
+    acc = np.einsum("bmk,bnk->bmn", q.astype(np.int64), kt.astype(np.int64)).astype(np.float32)
+    want = (acc * np.float32(0.01)) * np.float32(0.012) + mask
+    assert np.array_equal(dst.view(np.uint32), want.view(np.uint32))
+    # batch broadcast of the weights (dims 1 on the batch axis)
+    dst2 = np.zeros((B, M, N), np.float32)
+    O.matmul(T(O.S8, q), O.Tensor(O.S8, (1, K, N), kt[:1], (N * K, 1, K)), T(O.F32, dst2))
+    want2 = np.einsum("bmk,nk->bmn", q.astype(np.int64), kt[0].astype(np.int64)).astype(np.float32)
+    assert np.array_equal(dst2, want2)
+
+
+def test_post_op_chain_order_bias_and_prelu():
+    rng = np.random.default_rng(7)
+    M, K, N = 5, 32, 7
+    src = rng.integers(-8, 9, (M, K)).astype(np.int8)
+    wei = rng.integers(-8, 9, (K, N)).astype(np.int8)
+    bias = rng.integers(-4, 5, (1, N)).astype(np.int32)
+    col = rng.integers(1, 4, (1, N)).astype(np.float32)
+    pw = (2.0 ** rng.integers(-2, 2, N)).astype(np.float32)
+    old = rng.integers(-10, 10, (M, N)).astype(np.float32)
+    dst = old.copy()
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.F32, dst), bias=T(O.S32, bias),
+             post_ops=[{"kind": "binary", "alg": MUL, "src1": T(O.F32, col)},
+                       {"kind": "sum", "scale": 0.5},
+                       {"kind": "prelu", "mask": 2, "weights": pw},
+                       {"kind": "eltwise", "alg": LINEAR, "alpha": 2.0, "beta": 1.0, "scale": 0.25}])
+    acc = (src.astype(np.int64) @ wei.astype(np.int64)).astype(np.float64)
+    v = (acc + bias) * col + 0.5 * old
+    v = np.where(v < 0, v * pw[None, :], v)
+    v = (2.0 * v + 1.0) * 0.25
+    assert np.array_equal(dst, v.astype(np.float32))
+
+
+def test_zero_dim_is_a_no_op():
+    dst = np.full((0, 4), 7, np.float32)
+    O.matmul(T(O.S8, np.zeros((0, 8), np.int8)), T(O.S8, np.zeros((8, 4), np.int8)), T(O.F32, dst, dims=(0, 4)))
+    dst = np.full((3, 4), 7, np.float32)
+    O.matmul(O.Tensor(O.S8, (3, 0), np.zeros(1, np.int8)), O.Tensor(O.S8, (0, 4), np.zeros(1, np.int8)), T(O.F32, dst))
+    assert np.all(dst == 7)  # src/cpu/matmul/ref_matmul_int8.cpp:64-66
+
+
+def test_reorder_quantize_and_transpose():
+    rng = np.random.default_rng(8)
+    K, N = 64, 12
+    w = (rng.standard_normal((K, N)) * 3).astype(np.float32)
+    sc = (2.0 ** rng.integers(-3, 0, N)).astype(np.float32)
+    out = np.zeros((N, K), np.int8)  # ba layout of a [K, N] tensor
+    O.reorder(T(O.F32, w), O.Tensor(O.S8, (K, N), out, (1, K)),
+              dst_scale=O.Quant(2, O.F32, sc))
+    want = np.clip(np.rint(w / sc[None, :]), -128, 127).astype(np.int8)
+    assert np.array_equal(out.T, want)
+    # u4 <- s8 pure conversion keeps nibble order
+    v = rng.integers(0, 16, (K, N)).astype(np.int8)
+    out4 = np.zeros(K * N // 2, np.uint8)
+    O.reorder(T(O.S8, v), O.Tensor(O.U4, (K, N), out4))
+    assert np.array_equal(out4, O.pack4(v))
