@@ -1,0 +1,160 @@
+/*
+ * Thin C ABI over the gfx950 HIP kernels of the quantized matmul path.
+ *
+ * This is the only interface the .hip translation units export. The dnnl_*
+ * entry points (include/oneapi/dnnl/dnnl.h) are host C++ on top of it: a
+ * primitive descriptor picks an implementation with qmm_matmul_impl_supports(),
+ * a primitive owns a plan, and execute() is one qmm_matmul_launch() on the
+ * stream's HIP stream. Plain-old-data only: dims, strides, data-type codes,
+ * masks, groups, the post-op list and device pointers. No call here allocates
+ * except plan creation (one small device copy of the descriptor).
+ *
+ * Reference interfaces this layer stands in for:
+ *   - primitive_t::execute(const exec_ctx_t &) of a matmul implementation
+ *     (src/common/primitive.hpp:43-80, src/gpu/amd/miopen_matmul.hpp:35-165),
+ *   - pd_t::init() returning status::unimplemented for unsupported cases so
+ *     the implementation list falls through
+ *     (src/common/primitive_desc_iterator.hpp:67-94,
+ *      src/gpu/gpu_matmul_list.cpp:45-62),
+ *   - the reorder implementation list entry used for weights prepacking
+ *     (src/cpu/x64/matmul/brgemm_matmul_reorders.hpp:28-76).
+ *
+ * Data-type, algorithm and primitive-kind codes are the dnnl ones
+ * (dnnl_data_type_t, dnnl_alg_kind_t, dnnl_primitive_kind_t).
+ */
+#ifndef QMM_HIP_H
+#define QMM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QMM_MAX_NDIMS 12
+#define QMM_MAX_POST_OPS 32
+#define QMM_API __attribute__((visibility("default")))
+
+/* status codes: 0 ok; the rest map 1:1 onto dnnl_status_t */
+enum {
+    QMM_OK = 0,
+    QMM_OUT_OF_MEMORY = 1,
+    QMM_INVALID_ARGUMENTS = 2,
+    QMM_UNIMPLEMENTED = 3,
+    QMM_RUNTIME_ERROR = 5
+};
+
+/* Physical layouts of a weights tensor. */
+enum {
+    QMM_LAYOUT_PLAIN = 0, /* strided, strides in elements */
+    /* 1-byte elements (s8/u8/f8) in MFMA operand order: per batch,
+     * [N/32][K/32][64 lanes][16 bytes], lane = 32*((k%32)/16) + n%32,
+     * byte = k%16; K padded to 128 and N to 32 with zeros; followed (256-byte
+     * aligned) by s32 column sums [batch][Npad] for integer weights. */
+    QMM_LAYOUT_MFMA_B8 = 1,
+    /* 4-bit elements for the decode kernel: per batch,
+     * [N/16][K/128][64 lanes][16 bytes], lane = 16*c + n%16 holds
+     * k = 128*g + 32*s + 8*c + j for dword s = 0..3, and inside a dword the
+     * nibble at bits 4*p..4*p+3 is j = perm(p) = (p%2)*4 + p/2 ... see
+     * qmm_w4_nibble_pos(); K padded to 128 and N to 16 with zeros. */
+    QMM_LAYOUT_MFMA_W4 = 2
+};
+
+typedef struct {
+    int32_t dt;
+    int32_t ndims;
+    int64_t dims[QMM_MAX_NDIMS];
+    int64_t strides[QMM_MAX_NDIMS]; /* elements; ignored for packed layouts */
+} qmm_tensor_t;
+
+/* One scales or zero-points entry (dnnl_primitive_attr_set_scales /
+ * _set_zero_points): the buffer is a dense row-major tensor over the masked
+ * dims of the quantized tensor with its last two dims divided by the groups
+ * (src/cpu/matmul/matmul_utils.hpp:156-196). */
+typedef struct {
+    int32_t set; /* 0: default value (scale 1, zero point 0) */
+    int32_t mask;
+    int32_t dt;
+    int32_t has_groups;
+    int64_t g0, g1; /* groups over the last two dims; 1 when absent */
+} qmm_quant_t;
+
+typedef struct {
+    int32_t kind; /* dnnl_sum / dnnl_eltwise / dnnl_binary / dnnl_prelu */
+    int32_t alg;
+    float alpha, beta, scale;
+    int32_t zero_point;
+    int32_t dt; /* sum: data type dst is read as (0 = dst's own) */
+    int32_t mask; /* prelu */
+    qmm_tensor_t src1; /* binary operand descriptor (plain) */
+} qmm_postop_t;
+
+enum { QMM_SRC = 0, QMM_WEI = 1, QMM_DST = 2 };
+
+typedef struct {
+    qmm_tensor_t src, wei, bias, dst; /* bias.ndims == 0: no bias */
+    int32_t wei_layout;
+    int32_t apply_to_int; /* fpmath_mode apply_to_int */
+    qmm_quant_t scales[3];
+    qmm_quant_t zps[3];
+    int32_t npo;
+    int32_t reserved;
+    qmm_postop_t po[QMM_MAX_POST_OPS];
+} qmm_matmul_desc_t;
+
+typedef struct {
+    const void *src, *wei, *bias;
+    void *dst;
+    const void *scales[3];
+    const void *zps[3];
+    const void *po_arg[QMM_MAX_POST_OPS]; /* binary src1 / prelu weights */
+    void *scratch; /* qmm_matmul_scratch_size() bytes, or NULL when 0 */
+} qmm_matmul_args_t;
+
+typedef struct qmm_plan qmm_plan_t;
+
+/* ---- matmul implementations, in dispatch order ---- */
+QMM_API int qmm_matmul_impl_count(void);
+QMM_API const char *qmm_matmul_impl_name(int impl);
+/* QMM_OK if implementation `impl` computes `desc`; QMM_UNIMPLEMENTED if not */
+QMM_API int qmm_matmul_impl_supports(int impl, const qmm_matmul_desc_t *desc);
+QMM_API size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc);
+QMM_API int qmm_matmul_plan_create(
+        qmm_plan_t **plan, int impl, const qmm_matmul_desc_t *desc);
+QMM_API void qmm_matmul_plan_destroy(qmm_plan_t *plan);
+/* Enqueue on `hip_stream` (a hipStream_t); asynchronous. */
+QMM_API int qmm_matmul_launch(const qmm_plan_t *plan,
+        const qmm_matmul_args_t *args, void *hip_stream);
+
+/* ---- packed weights layouts ---- */
+/* Bytes a weights tensor [batch..., K, N] of type dt occupies in `layout`. */
+QMM_API size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N);
+/* Layout format_tag any resolves to for this problem, or QMM_LAYOUT_PLAIN. */
+QMM_API int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc);
+
+/* ---- reorder ---- */
+typedef struct {
+    qmm_tensor_t src, dst; /* same logical dims */
+    int32_t src_layout, dst_layout;
+    qmm_quant_t src_scale, dst_scale, src_zp, dst_zp;
+} qmm_reorder_desc_t;
+
+typedef struct {
+    const void *src;
+    void *dst;
+    const void *src_scale, *dst_scale, *src_zp, *dst_zp;
+} qmm_reorder_args_t;
+
+QMM_API int qmm_reorder_supports(const qmm_reorder_desc_t *desc);
+QMM_API int qmm_reorder_launch(const qmm_reorder_desc_t *desc,
+        const qmm_reorder_args_t *args, void *hip_stream);
+
+/* ---- device queries used by the engine ---- */
+QMM_API int qmm_device_count(void);
+QMM_API const char *qmm_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,75 @@
+"""Builds the shared library of the MI355X quantized-matmul path.
+
+hipcc cross-compiles every translation unit for gfx950 (no GPU needed) and
+links one in-tree shared object, onednn_amd/libdnnl_amd.so, which exports the
+dnnl_* C API subset and the qmm_* kernel-level C ABI.
+
+Flags of note:
+  -ffp-contract=off   the epilogue must round every float step separately;
+  -Xclang -target-feature -Xclang -packed-fp32-ops
+                      keeps the compiler from forming packed FP32 instructions.
+"""
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(HERE, "libdnnl_amd.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+          "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+          "-Wall", "-Wno-unused-function", "-Wno-pass-failed"]
+DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+# (source, object suffix, extra defines)
+UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
+         ("qmm_pack.hip", "", []), ("qmm_dispatch.hip", "", []),
+         ("qmm_gemm_b8.hip", "", []),
+         ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]
+# the tiled GEMM is instantiated once per tile configuration, each in its own
+# object so the instantiations compile in parallel
+GEMM_VARIANTS = [1, 2, 3, 4, 5]
+for v in GEMM_VARIANTS:
+    UNITS.append(("qmm_gemm_b8.hip", "_v%d" % v, ["-DQMM_GEMM_VARIANT=%d" % v]))
+
+
+def _compile(unit):
+    src, suffix, defs = unit
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
+    cmd = [HIPCC] + COMMON + defs
+    if src.endswith(".hip"):
+        cmd += DEVICE
+    else:
+        cmd += ["-x", "hip", "--offload-host-only"] if False else []
+    cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                       text=True)
+    out = "\n".join(l for l in r.stdout.splitlines()
+                    if "packed-fp32-ops" not in l and "warning generated" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), out))
+    return obj, out
+
+
+def build(verbose=False, jobs=None):
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 4)
+    objs = []
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for obj, out in ex.map(_compile, UNITS):
+            objs.append(obj)
+            if verbose and out.strip():
+                print(out)
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,480 @@
+// Device-side scalar layer shared by every kernel of the quantized matmul path:
+// typed loads/stores with the reference's conversions, eltwise / binary
+// formulas and the ordered epilogue (bias, post-ops, dst scale, dst zero point,
+// saturating store).
+//
+// All float steps here must round separately (the translation units are built
+// with -ffp-contract=off): the reference's scalar code is compiled for an ISA
+// without FMA, and s8/u8 results are compared bit for bit.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qmm_hip.h"
+
+namespace qmm {
+
+// dnnl_data_type_t codes (include/oneapi/dnnl/dnnl_common_types.h:76-115)
+enum : int {
+    dt_undef = 0, dt_f16 = 1, dt_bf16 = 2, dt_f32 = 3, dt_s32 = 4, dt_s8 = 5,
+    dt_u8 = 6, dt_f8_e5m2 = 9, dt_f8_e4m3 = 10, dt_s4 = 11, dt_u4 = 12,
+    dt_e8m0 = 13
+};
+// dnnl_primitive_kind_t codes used for post-ops
+enum : int { pk_sum = 4, pk_eltwise = 7, pk_binary = 13, pk_prelu = 18 };
+
+#define QMM_HD __host__ __device__ __forceinline__
+#define QMM_D __device__ __forceinline__
+
+QMM_HD uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+QMM_HD float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// ---- bf16: src/common/bfloat16.cpp:22-56 ----
+QMM_HD uint16_t f32_to_bf16(float f) {
+    const uint32_t u = f2u(f);
+    const uint32_t e = (u >> 23) & 0xFF;
+    const uint16_t hi = (uint16_t)(u >> 16);
+    if (e == 0) return hi & 0x8000; // zero and denormals: signed zero
+    if (e == 0xFF) return (u & 0x7FFFFF) ? (uint16_t)(hi | 0x40) : hi;
+    return (uint16_t)((u + 0x7FFFu + (hi & 1u)) >> 16);
+}
+QMM_HD float bf16_to_f32(uint16_t r) { return u2f((uint32_t)r << 16); }
+
+// ---- f16: src/common/float16.hpp:52-127 ----
+QMM_HD uint16_t f32_to_f16(float f) {
+    const uint32_t i = f2u(f);
+    const uint32_t s = i >> 31, e = (i >> 23) & 0xFF, m = i & 0x7FFFFF;
+    uint32_t mm = m >> 13, ee = 0;
+    const uint32_t r = m & 0x1FFF;
+    const int32_t eee = (int32_t)e - 127 + 15;
+    if (e == 0) {
+        mm = 0;
+    } else if (e == 0xFF) {
+        ee = 0x1F;
+        if (m != 0) mm |= 0x200;
+    } else if (eee > 0 && eee < 0x1F) {
+        ee = (uint32_t)eee;
+        if (r > (0x1000 - (mm & 1))) {
+            mm++;
+            if (mm == 0x400) {
+                mm = 0;
+                ee++;
+            }
+        }
+    } else if (eee >= 0x1F) {
+        ee = 0x1F;
+        mm = 0;
+    } else {
+        const float ff = u2f(i & 0x7FFFFFFFu) + 0.5f;
+        mm = f2u(ff) & 0x7FF;
+    }
+    return (uint16_t)((s << 15) | (ee << 10) | mm);
+}
+QMM_HD float f16_to_f32(uint16_t raw) {
+    const uint32_t ss = raw >> 15, ee = (raw >> 10) & 0x1F, mm = raw & 0x3FF;
+    uint32_t m = mm << 13, e;
+    if (ee == 0) {
+        if (mm == 0) return u2f(ss << 31);
+        // subnormal half: mm * 2^-24, exact in f32
+        const float v = (float)mm * u2f(0x33800000u);
+        return ss ? -v : v;
+    } else if (ee == 0x1F) {
+        e = 0xFF;
+        if (m != 0) m |= 0x400000;
+    } else
+        e = ee - 15 + 127;
+    return u2f((ss << 31) | (e << 23) | m);
+}
+
+// ---- f8: src/common/float8.cpp:43-190 ----
+QMM_HD uint8_t f16_to_e4m3(uint16_t h) {
+    int fraw = h;
+    const unsigned s8 = (fraw & 0x8000) >> 8;
+    fraw &= 0x7fff;
+    if (fraw > 0x5f40) return (uint8_t)(s8 | 0x7f);
+    if (fraw <= 0x1400) return (uint8_t)s8;
+    uint16_t shifter = (uint16_t)((fraw & 0x7c00) + 0x1c00);
+    const bool is_denorm = shifter < 0x4000;
+    if (is_denorm) shifter = 0x4000;
+    uint16_t rounded
+            = f32_to_f16(f16_to_f32((uint16_t)fraw) + f16_to_f32(shifter));
+    rounded = f32_to_f16(f16_to_f32(rounded) - f16_to_f32(shifter));
+    int e8 = ((rounded & 0x7c00) >> 10) - 8;
+    uint8_t m8 = (uint8_t)((rounded & 0x03ff) >> 7);
+    if (is_denorm) {
+        m8 = (uint8_t)((m8 | 0x8) >> (-e8 + 1));
+        e8 = 0;
+    }
+    return (uint8_t)(s8 | (e8 << 3) | m8);
+}
+QMM_HD uint16_t e4m3_to_f16(uint8_t r) {
+    const uint16_t s8 = (r & 0x80) >> 7, e8 = (r & 0x78) >> 3, m8 = r & 0x7;
+    uint16_t e16 = e8 + 8, m16 = m8;
+    if (e8 == 0 && m8 != 0) {
+        uint16_t count = 2;
+        count = m8 > 0x1 ? 1 : count;
+        count = m8 > 0x3 ? 0 : count;
+        e16 -= count;
+        m16 = (m16 << (count + 1)) & 0x7;
+    } else if (e8 == 0 && m8 == 0) {
+        e16 = 0;
+    } else if (e8 == 0xf && m8 == 0x7) {
+        e16 = 0x1f;
+        m16 = 0x4;
+    }
+    return (uint16_t)((s8 << 15) | (e16 << 10) | (m16 << 7));
+}
+QMM_HD uint8_t f16_to_e5m2(uint16_t fraw) {
+    const bool is_special = (fraw & 0x7c00) == 0x7c00;
+    const bool is_nan = is_special && (fraw & 0x03ff);
+    if (is_nan) return (uint8_t)((fraw >> 8) | 0x02);
+    if (is_special) return (uint8_t)(fraw >> 8);
+    fraw = (uint16_t)(fraw + 0x007f + ((fraw & 0x0100) >> 8));
+    return (uint8_t)(fraw >> 8);
+}
+QMM_HD float e5m2_to_f32(uint8_t r) {
+    const uint8_t raw = ((r & 0x7d) == 0x7d) ? (r | 0x02) : r;
+    return f16_to_f32((uint16_t)(raw << 8));
+}
+QMM_HD float e8m0_to_f32(uint8_t r) {
+    return r == 0xff ? u2f(0xffc00000u) : u2f((uint32_t)r << 23);
+}
+
+// ---- typed element access: src/cpu/ref_io_helper.hpp:33-154 ----
+QMM_HD int nibble_at(const void *p, int64_t idx) {
+    const uint8_t b = ((const uint8_t *)p)[idx >> 1];
+    return (idx & 1) ? (b >> 4) : (b & 0xf); // even index = low nibble
+}
+QMM_HD int s4_value(int nib) { return (nib & 8) ? nib - 16 : nib; }
+
+QMM_HD int load_int(int dt, const void *p, int64_t idx) {
+    switch (dt) {
+        case dt_s32: return ((const int32_t *)p)[idx];
+        case dt_s8: return ((const int8_t *)p)[idx];
+        case dt_u8: return ((const uint8_t *)p)[idx];
+        case dt_s4: return s4_value(nibble_at(p, idx));
+        case dt_u4: return nibble_at(p, idx);
+        default: return 0x7fffffff;
+    }
+}
+
+QMM_HD float load_float(int dt, const void *p, int64_t idx) {
+    switch (dt) {
+        case dt_f32: return ((const float *)p)[idx];
+        case dt_bf16: return bf16_to_f32(((const uint16_t *)p)[idx]);
+        case dt_f16: return f16_to_f32(((const uint16_t *)p)[idx]);
+        case dt_f8_e4m3:
+            return f16_to_f32(e4m3_to_f16(((const uint8_t *)p)[idx]));
+        case dt_f8_e5m2: return e5m2_to_f32(((const uint8_t *)p)[idx]);
+        case dt_s32: return (float)((const int32_t *)p)[idx];
+        case dt_s8: return (float)((const int8_t *)p)[idx];
+        case dt_u8: return (float)((const uint8_t *)p)[idx];
+        case dt_e8m0: return e8m0_to_f32(((const uint8_t *)p)[idx]);
+        case dt_s4: return (float)s4_value(nibble_at(p, idx));
+        case dt_u4: return (float)nibble_at(p, idx);
+        default: return u2f(0x7fc00000u);
+    }
+}
+
+// clamp then round half to even (src/cpu/simple_q10n.hpp:41-81); a NaN passes
+// the clamps and converts to the x86 "integer indefinite" value
+QMM_HD int round_sat(float v, float lo, float hi) {
+    if (v < lo) v = lo;
+    if (v > hi) v = hi;
+    if (v != v) return (int)0x80000000;
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (int)__builtin_rintf(v);
+#else
+    return (int)__builtin_nearbyintf(v);
+#endif
+}
+
+QMM_HD void store_float(int dt, float v, void *p, int64_t idx) {
+    switch (dt) {
+        case dt_f32: ((float *)p)[idx] = v; break;
+        case dt_bf16: ((uint16_t *)p)[idx] = f32_to_bf16(v); break;
+        case dt_f16: ((uint16_t *)p)[idx] = f32_to_f16(v); break;
+        case dt_f8_e4m3:
+            ((uint8_t *)p)[idx] = f16_to_e4m3(f32_to_f16(v));
+            break;
+        case dt_f8_e5m2:
+            ((uint8_t *)p)[idx] = f16_to_e5m2(f32_to_f16(v));
+            break;
+        case dt_s32:
+            ((int32_t *)p)[idx] = round_sat(v, -2147483648.f, 2147483520.f);
+            break;
+        case dt_s8: ((int8_t *)p)[idx] = (int8_t)round_sat(v, -128.f, 127.f); break;
+        case dt_u8: ((uint8_t *)p)[idx] = (uint8_t)round_sat(v, 0.f, 255.f); break;
+        default: break;
+    }
+}
+
+// ---- eltwise forward: src/common/math_utils.hpp:129-416 ----
+enum : int {
+    alg_relu = 0x20, alg_tanh, alg_elu, alg_square, alg_abs, alg_sqrt,
+    alg_linear, alg_soft_relu, alg_hardsigmoid, alg_logistic, alg_exp,
+    alg_gelu_tanh, alg_swish, alg_log, alg_clip, alg_clip_v2, alg_pow,
+    alg_gelu_erf, alg_round, alg_mish, alg_hardswish,
+    alg_relu_dst = 0x100, alg_tanh_dst, alg_elu_dst, alg_sqrt_dst,
+    alg_logistic_dst, alg_exp_dst, alg_clip_v2_dst,
+    alg_bin_add = 0x1fff0, alg_bin_mul, alg_bin_max, alg_bin_min, alg_bin_div,
+    alg_bin_sub, alg_bin_ge, alg_bin_gt, alg_bin_le, alg_bin_lt, alg_bin_eq,
+    alg_bin_ne
+};
+
+QMM_D float logistic_f(float s) {
+    const float bound = 88.72283172607421875f;
+    const float in = -s;
+    return in < bound ? 1.f / (1.f + expf(in)) : 0.f;
+}
+QMM_D float soft_relu_f(float s, float alpha) {
+    const float bound = 88.72283172607421875f;
+    const float in = s * alpha;
+    const float v = in < bound ? log1pf(expf(in)) : in;
+    return v / alpha;
+}
+QMM_D float hardsigmoid_f(float s, float alpha, float beta) {
+    const float v = alpha * s + beta;
+    return v <= 0.f ? 0.f : v >= 1.f ? 1.f : v;
+}
+
+QMM_D float eltwise_fwd(int alg, float s, float alpha, float beta) {
+    switch (alg) {
+        case alg_relu:
+        case alg_relu_dst: return s > 0 ? s : s * alpha;
+        case alg_tanh:
+        case alg_tanh_dst: return tanhf(s);
+        case alg_elu:
+        case alg_elu_dst: return s > 0 ? s : alpha * expm1f(s);
+        case alg_square: return s * s;
+        case alg_abs: return s > 0 ? s : -s;
+        case alg_sqrt:
+        case alg_sqrt_dst: return sqrtf(s);
+        case alg_linear: return alpha * s + beta;
+        case alg_soft_relu: return soft_relu_f(s, alpha);
+        case alg_hardsigmoid: return hardsigmoid_f(s, alpha, beta);
+        case alg_logistic:
+        case alg_logistic_dst: return logistic_f(s);
+        case alg_exp:
+        case alg_exp_dst: return expf(s);
+        case alg_gelu_tanh: {
+            const float sqrt_2_over_pi = 0.79788458347320556640625f;
+            const float fitting_const = 0.044715f;
+            const float v = tanhf(
+                    sqrt_2_over_pi * s * (1 + fitting_const * s * s));
+            return (float)(0.5 * s * (1. + v));
+        }
+        case alg_swish: return s * logistic_f(alpha * s);
+        case alg_log: return logf(s);
+        case alg_clip: {
+            s = s > alpha ? s : alpha;
+            return s > beta ? beta : s;
+        }
+        case alg_clip_v2:
+        case alg_clip_v2_dst: {
+            s = s > alpha ? s : alpha;
+            return s < beta ? s : beta;
+        }
+        case alg_pow: return alpha * powf(s, beta);
+        case alg_gelu_erf: {
+            const float sqrt_2_over_2 = 0.707106769084930419921875f;
+            const float v = s * sqrt_2_over_2;
+            return 0.5f * s * (1.f + erff(v));
+        }
+        case alg_round: return __builtin_rintf(s);
+        case alg_mish: return s * tanhf(soft_relu_f(s, 1.f));
+        case alg_hardswish: return s * hardsigmoid_f(s, alpha, beta);
+        default: return u2f(0x7fc00000u);
+    }
+}
+
+// src/cpu/primitive_attr_postops.cpp:29-46
+QMM_D float binary_op(int alg, float x, float y) {
+    switch (alg) {
+        case alg_bin_add: return x + y;
+        case alg_bin_div: return x / y;
+        case alg_bin_max: return x > y ? x : y;
+        case alg_bin_min: return x < y ? x : y;
+        case alg_bin_mul: return x * y;
+        case alg_bin_sub: return x - y;
+        case alg_bin_ge: return x >= y;
+        case alg_bin_gt: return x > y;
+        case alg_bin_le: return x <= y;
+        case alg_bin_lt: return x < y;
+        case alg_bin_eq: return x == y;
+        case alg_bin_ne: return x != y;
+        default: return u2f(0x7fc00000u);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Compact epilogue description used by the tiled kernels. The host folds the
+// problem to (batch, m, n) coordinates: every tensor touched after the
+// accumulation is addressed as base + b*sb + m*sm + n*sn with zero strides on
+// broadcast dims.
+struct ep_tensor_t {
+    const void *ptr;
+    int64_t sb, sm, sn;
+    int32_t dt;
+    int32_t pad_;
+};
+
+struct ep_postop_t {
+    int32_t kind, alg;
+    float alpha, beta, scale;
+    int32_t zero_point;
+    ep_tensor_t t; // binary operand, prelu weights (f32) or dst-as-sum_dt
+};
+
+constexpr int EP_MAX_PO = 6;
+
+struct epilogue_t {
+    ep_tensor_t dst;
+    ep_tensor_t bias; // ptr == nullptr: none
+    ep_tensor_t src_scale; // per-tensor or per-m (sm != 0); nullptr: none
+    ep_tensor_t wei_scale; // per-tensor or per-n (sn != 0); nullptr: none
+    const void *dst_scale; // single value, inverted in the kernel
+    int32_t dst_scale_dt;
+    int32_t npo;
+    const int32_t *dst_zp; // s32; index dst_zp_sn * n
+    int64_t dst_zp_sn;
+    ep_postop_t po[EP_MAX_PO];
+};
+
+QMM_D float ep_load(const ep_tensor_t &t, int64_t b, int64_t m, int64_t n) {
+    return load_float(t.dt, t.ptr, b * t.sb + m * t.sm + n * t.sn);
+}
+
+// Ordered tail of the reference kernels, starting after the K reduction:
+//   integer path   src/cpu/matmul/ref_matmul_int8.cpp:195-259
+//   float path     src/cpu/matmul/ref_matmul.cpp:199-229
+// `acc` is (float)s32 for the integer path or the f32 accumulator.
+QMM_D void epilogue_apply_store(const epilogue_t &ep, float acc, int64_t b,
+        int64_t m, int64_t n) {
+    float d = acc;
+    if (ep.src_scale.ptr) d *= ep_load(ep.src_scale, b, m, 0);
+    if (ep.wei_scale.ptr) d *= ep_load(ep.wei_scale, b, 0, n);
+    if (ep.bias.ptr) d += ep_load(ep.bias, b, m, n);
+    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n * ep.dst.sn;
+#pragma unroll 1
+    for (int i = 0; i < ep.npo; i++) {
+        const ep_postop_t &e = ep.po[i];
+        if (e.kind == pk_eltwise) {
+            d = eltwise_fwd(e.alg, d, e.alpha, e.beta) * e.scale;
+        } else if (e.kind == pk_sum) {
+            const float old = load_float(e.t.dt, ep.dst.ptr, dst_off);
+            d += e.scale * (old - (float)e.zero_point);
+        } else if (e.kind == pk_binary) {
+            d = binary_op(e.alg, d, ep_load(e.t, b, m, n));
+        } else if (e.kind == pk_prelu) {
+            if (d < 0) d = ep_load(e.t, b, m, n) * d;
+        }
+    }
+    if (ep.dst_scale) d *= 1.f / load_float(ep.dst_scale_dt, ep.dst_scale, 0);
+    if (ep.dst_zp) d += (float)ep.dst_zp[ep.dst_zp_sn * n];
+    store_float(ep.dst.dt, d, (void *)ep.dst.ptr, dst_off);
+}
+
+// Four consecutive n at once (n % 4 == 0): the tiled GEMM hands its results
+// over row-wise so that a lane owns 4 neighbours of a dst row and 16 lanes
+// cover 64 columns; stores are 4-element vectors when the row is dense and
+// aligned. `nvalid` (1..4) masks the tail of a row.
+QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
+        int64_t b, int64_t m, int64_t n, int nvalid) {
+    if (ep.src_scale.ptr) {
+        const float s = ep_load(ep.src_scale, b, m, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= s;
+    }
+    if (ep.wei_scale.ptr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < nvalid) d[i] *= ep_load(ep.wei_scale, b, 0, n + i);
+    }
+    if (ep.bias.ptr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < nvalid) d[i] += ep_load(ep.bias, b, m, n + i);
+    }
+    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n * ep.dst.sn;
+#pragma unroll 1
+    for (int pi = 0; pi < ep.npo; pi++) {
+        const ep_postop_t &e = ep.po[pi];
+        if (e.kind == pk_eltwise) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] = eltwise_fwd(e.alg, d[i], e.alpha, e.beta) * e.scale;
+        } else if (e.kind == pk_sum) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid) {
+                    const float old = load_float(
+                            e.t.dt, ep.dst.ptr, dst_off + i * ep.dst.sn);
+                    d[i] += e.scale * (old - (float)e.zero_point);
+                }
+        } else if (e.kind == pk_binary) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid)
+                    d[i] = binary_op(e.alg, d[i], ep_load(e.t, b, m, n + i));
+        } else if (e.kind == pk_prelu) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid && d[i] < 0)
+                    d[i] = ep_load(e.t, b, m, n + i) * d[i];
+        }
+    }
+    if (ep.dst_scale) {
+        const float inv = 1.f / load_float(ep.dst_scale_dt, ep.dst_scale, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= inv;
+    }
+    if (ep.dst_zp) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < nvalid) d[i] += (float)ep.dst_zp[ep.dst_zp_sn * (n + i)];
+    }
+    void *dst = (void *)ep.dst.ptr;
+    const int dt = ep.dst.dt;
+    if (nvalid == 4 && ep.dst.sn == 1) {
+        if (dt == dt_bf16 || dt == dt_f16) {
+            uint16_t *q = (uint16_t *)dst + dst_off;
+            if (((uintptr_t)q & 7) == 0) {
+                uint16_t h[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    h[i] = dt == dt_bf16 ? f32_to_bf16(d[i]) : f32_to_f16(d[i]);
+                *(uint2 *)q = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16),
+                        (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+                return;
+            }
+        } else if (dt == dt_f32) {
+            float *q = (float *)dst + dst_off;
+            if (((uintptr_t)q & 15) == 0) {
+                *(float4 *)q = make_float4(d[0], d[1], d[2], d[3]);
+                return;
+            }
+        } else if (dt == dt_s8 || dt == dt_u8) {
+            uint8_t *q = (uint8_t *)dst + dst_off;
+            if (((uintptr_t)q & 3) == 0) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = dt == dt_s8 ? round_sat(d[i], -128.f, 127.f)
+                                              : round_sat(d[i], 0.f, 255.f);
+                    w |= (uint32_t)(r & 0xff) << (8 * i);
+                }
+                *(uint32_t *)q = w;
+                return;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (i < nvalid) store_float(dt, d[i], dst, dst_off + i * ep.dst.sn);
+}
+
+} // namespace qmm

@@ -1,0 +1,805 @@
+// Host side of the thin C ABI (include/qmm_hip.h): implementation selection,
+// plan creation and kernel launches. Pure host code apart from the HIP runtime
+// calls; it never computes a result itself.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "qmm_device.hpp"
+#include "qmm_hip.h"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+void launch_matmul_generic(const generic_params_t *dev_params,
+        const generic_params_t &host_params, const qmm_matmul_args_t &args,
+        hipStream_t stream);
+void launch_reorder_generic(const generic_reorder_params_t &params,
+        const qmm_reorder_args_t &args, hipStream_t stream);
+void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
+        hipStream_t stream);
+void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
+void launch_pack_b8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        bool with_colsum, hipStream_t stream);
+void launch_unpack_b8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
+void launch_pack_w4(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
+void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
+} // namespace qmm
+
+using namespace qmm;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char *msg) {
+    g_last_error = msg;
+    return code;
+}
+int hip_fail(hipError_t e, const char *what) {
+    g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+    return QMM_RUNTIME_ERROR;
+}
+
+bool is_int8(int dt) { return dt == dt_s8 || dt == dt_u8; }
+bool is_int4(int dt) { return dt == dt_s4 || dt == dt_u4; }
+bool is_wei_int(int dt) { return is_int8(dt) || is_int4(dt); }
+bool one_of(int v, std::initializer_list<int> l) {
+    for (int x : l)
+        if (v == x) return true;
+    return false;
+}
+
+int dims_mask(const int64_t *d1, const int64_t *d2, int nd) {
+    int mask = 0;
+    for (int d = 0; d < nd; d++)
+        if (d1[d] == d2[d]) mask |= 1 << d;
+    return mask;
+}
+
+// geometry of a scales / zero-points buffer over tensor dims `tdims`
+void quant_geom(generic_quant_t &q, const qmm_quant_t &a, int nd,
+        const int64_t *tdims, int64_t g0, int64_t g1) {
+    std::memset(&q, 0, sizeof(q));
+    q.g0 = g0 > 0 ? g0 : 1;
+    q.g1 = g1 > 0 ? g1 : 1;
+    q.nelems = 1;
+    if (!a.set) return;
+    int64_t dims[QMM_MAX_NDIMS];
+    for (int d = 0; d < nd; d++)
+        dims[d] = (a.mask & (1 << d)) ? tdims[d] : 1;
+    if (nd >= 2) {
+        dims[nd - 1] /= q.g1;
+        dims[nd - 2] /= q.g0;
+    }
+    int64_t s = 1;
+    for (int d = nd - 1; d >= 0; d--) {
+        q.strides[d] = (a.mask & (1 << d)) ? s : 0;
+        s *= dims[d] > 0 ? dims[d] : 1;
+    }
+    q.nelems = s;
+    q.indexed = s > 1;
+}
+
+int64_t group_or(const qmm_quant_t &a, int which, int64_t dflt) {
+    if (!a.set || !a.has_groups) return dflt;
+    const int64_t g = which == 0 ? a.g0 : a.g1;
+    return g > 0 ? g : dflt;
+}
+
+void prelu_strides(int64_t *strides, const qmm_tensor_t &dst, int mask) {
+    // prelu weights: f32, dims = masked dst dims, layout a/ab/acb/acdb/acdeb
+    // (src/cpu/primitive_attr_postops.cpp:196-225)
+    static const int perm[6][5] = {{0}, {0}, {0, 1}, {0, 2, 1}, {0, 2, 3, 1},
+            {0, 2, 3, 4, 1}};
+    const int nd = dst.ndims;
+    int64_t s = 1;
+    for (int i = nd - 1; i >= 0; i--) {
+        const int d = nd <= 5 ? perm[nd][i] : i;
+        const int64_t dim = (mask & (1 << d)) ? dst.dims[d] : 0;
+        strides[d] = s;
+        s *= dim > 0 ? dim : 1;
+    }
+}
+
+void build_generic(generic_params_t &P, const qmm_matmul_desc_t &D) {
+    std::memset(&P, 0, sizeof(P));
+    P.desc = D;
+    const int nd = D.dst.ndims;
+    P.M = D.dst.dims[nd - 2];
+    P.N = D.dst.dims[nd - 1];
+    P.K = D.src.dims[nd - 1];
+    P.batch = 1;
+    for (int d = 0; d < nd - 2; d++)
+        P.batch *= D.dst.dims[d];
+    P.src_mask = dims_mask(D.dst.dims, D.src.dims, nd);
+    P.wei_mask = dims_mask(D.dst.dims, D.wei.dims, nd);
+    P.bia_mask = D.bias.ndims ? dims_mask(D.dst.dims, D.bias.dims, nd) : 0;
+    P.int_path = is_int8(D.src.dt);
+    P.decompress = !P.int_path && is_wei_int(D.wei.dt) && D.apply_to_int;
+    P.sum_dt = D.dst.dt;
+    for (int i = 0; i < D.npo; i++) {
+        if (D.po[i].kind == pk_sum && !P.has_sum) {
+            P.has_sum = 1;
+            if (D.po[i].dt != dt_undef) P.sum_dt = D.po[i].dt;
+        }
+        if (D.po[i].kind == pk_prelu)
+            prelu_strides(P.desc.po[i].src1.strides, D.dst, D.po[i].mask);
+    }
+    P.dst_zp_mult = D.zps[QMM_DST].set && D.zps[QMM_DST].mask > 0;
+    const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
+    const qmm_quant_t &sz = D.zps[QMM_SRC], &wz = D.zps[QMM_WEI];
+    quant_geom(P.q_src_scale, ss, nd, D.src.dims, 1, group_or(ss, 1, 1));
+    quant_geom(P.q_src_zp, sz, nd, D.src.dims, 1, group_or(sz, 1, 1));
+    quant_geom(P.q_wei_scale, ws, nd, D.wei.dims, group_or(ws, 0, 1),
+            group_or(ws, 1, 1));
+    quant_geom(P.q_wei_zp, wz, nd, D.wei.dims, group_or(wz, 0, 1),
+            group_or(wz, 1, 1));
+    // K groups of the integer path: the smallest group over the four entries.
+    // An entry without explicit groups varies per k if its mask covers K
+    // (group of 1) and otherwise spans all of K.
+    int64_t ng = 1;
+    if (P.K > 0) {
+        const int64_t K = P.K;
+        const int src_kbit = 1 << (nd - 1), wei_kbit = 1 << (nd - 2);
+        auto kgroup = [&](const qmm_quant_t &a, int which, int kbit) {
+            if (!a.set) return K;
+            if (a.has_groups) return group_or(a, which, K);
+            return (a.mask & kbit) ? (int64_t)1 : K;
+        };
+        int64_t t;
+        t = K / kgroup(sz, 1, src_kbit);
+        if (t > ng) ng = t;
+        t = K / kgroup(wz, 0, wei_kbit);
+        if (t > ng) ng = t;
+        t = K / kgroup(ss, 1, src_kbit);
+        if (t > ng) ng = t;
+        t = K / kgroup(ws, 0, wei_kbit);
+        if (t > ng) ng = t;
+    }
+    P.ngroups_k = ng;
+    P.group_k = P.K > 0 ? P.K / ng : 0;
+    P.wei_scale_stride_n = (ws.set && (ws.mask & (1 << (nd - 1)))) ? 1 : 0;
+}
+
+// Fold the batch dims of `t` (dims relative to dst's) into one linear stride.
+// Returns false if no single stride describes it.
+bool fold_batch(const qmm_tensor_t &t, const qmm_tensor_t &dst, int64_t &sb) {
+    const int nd = dst.ndims;
+    sb = 0;
+    if (nd <= 2) return true;
+    // effective stride per batch dim (0 where broadcast)
+    int64_t es[QMM_MAX_NDIMS];
+    for (int d = 0; d < nd - 2; d++)
+        es[d] = (t.dims[d] == dst.dims[d] && dst.dims[d] > 1) ? t.strides[d] : 0;
+    // innermost non-unit batch dim sets the stride, outer ones must nest
+    int64_t expect = -1;
+    for (int d = nd - 3; d >= 0; d--) {
+        if (dst.dims[d] == 1) continue;
+        if (expect < 0) {
+            sb = es[d];
+            expect = es[d] * dst.dims[d];
+        } else {
+            if (es[d] != expect) return false;
+            expect *= dst.dims[d];
+        }
+    }
+    return true;
+}
+
+bool fold_tensor(ep_tensor_t &e, const qmm_tensor_t &t,
+        const qmm_tensor_t &dst, const void *ptr) {
+    const int nd = dst.ndims;
+    e.ptr = ptr;
+    e.dt = t.dt;
+    e.sm = t.dims[nd - 2] == dst.dims[nd - 2] ? t.strides[nd - 2] : 0;
+    e.sn = t.dims[nd - 1] == dst.dims[nd - 1] ? t.strides[nd - 1] : 0;
+    return fold_batch(t, dst, e.sb);
+}
+
+// a quant buffer seen as a (b, m, n) tensor over the dst coordinates;
+// `is_src`: dims are (.., M, K) else (.., K, N). Only single-K-group buffers.
+bool fold_quant(ep_tensor_t &e, const generic_quant_t &q, const qmm_quant_t &a,
+        const qmm_tensor_t &t, const qmm_tensor_t &dst, bool is_src,
+        const void *ptr) {
+    const int nd = dst.ndims;
+    e.ptr = ptr;
+    e.dt = a.dt;
+    e.sb = e.sm = e.sn = 0;
+    if (!q.indexed) return true;
+    if (is_src) {
+        e.sm = q.strides[nd - 2];
+    } else {
+        if (q.g1 != 1) return false;
+        e.sn = q.strides[nd - 1];
+    }
+    qmm_tensor_t qt = t;
+    for (int d = 0; d < nd; d++)
+        qt.strides[d] = q.strides[d];
+    for (int d = 0; d < nd - 2; d++)
+        if (!(a.mask & (1 << d))) qt.dims[d] = 1; // broadcast
+    return fold_batch(qt, dst, e.sb);
+}
+
+// Build the compact epilogue; false if the problem does not fit it.
+bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
+        const qmm_matmul_args_t *A) {
+    const qmm_matmul_desc_t &D = P.desc;
+    const int nd = D.dst.ndims;
+    std::memset(&ep, 0, sizeof(ep));
+    const qmm_matmul_args_t zero_args = {};
+    if (!A) A = &zero_args;
+    if (!fold_tensor(ep.dst, D.dst, D.dst, A->dst)) return false;
+    if (D.bias.ndims) {
+        if (!fold_tensor(ep.bias, D.bias, D.dst, A->bias)) return false;
+        if (!A->bias) ep.bias.ptr = (const void *)1; // shape check only
+    }
+    const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
+    if (ss.set) {
+        if (P.q_src_scale.g1 != P.K && (ss.mask & (1 << (nd - 1))))
+            return false; // K-grouped src scales
+        if (!fold_quant(ep.src_scale, P.q_src_scale, ss, D.src, D.dst, true,
+                    A->scales[QMM_SRC]))
+            return false;
+        if (!A->scales[QMM_SRC]) ep.src_scale.ptr = (const void *)1;
+    }
+    if (ws.set && !P.decompress) {
+        if ((ws.mask & (1 << (nd - 2))) && P.q_wei_scale.g0 != P.K)
+            return false; // K-grouped weights scales
+        if (!fold_quant(ep.wei_scale, P.q_wei_scale, ws, D.wei, D.dst, false,
+                    A->scales[QMM_WEI]))
+            return false;
+        if (!A->scales[QMM_WEI]) ep.wei_scale.ptr = (const void *)1;
+    }
+    if (D.scales[QMM_DST].set) {
+        if (D.scales[QMM_DST].mask != 0) return false;
+        ep.dst_scale = A->scales[QMM_DST] ? A->scales[QMM_DST] : (const void *)1;
+        ep.dst_scale_dt = D.scales[QMM_DST].dt;
+    }
+    if (D.zps[QMM_DST].set) {
+        if (D.zps[QMM_DST].dt != dt_s32) return false;
+        ep.dst_zp = A->zps[QMM_DST] ? (const int32_t *)A->zps[QMM_DST]
+                                    : (const int32_t *)1;
+        ep.dst_zp_sn = P.dst_zp_mult;
+    }
+    if (D.npo > EP_MAX_PO) return false;
+    ep.npo = D.npo;
+    for (int i = 0; i < D.npo; i++) {
+        const qmm_postop_t &e = P.desc.po[i];
+        ep_postop_t &o = ep.po[i];
+        o.kind = e.kind;
+        o.alg = e.alg;
+        o.alpha = e.alpha;
+        o.beta = e.beta;
+        o.scale = e.scale;
+        o.zero_point = e.zero_point;
+        if (e.kind == pk_binary) {
+            if (!fold_tensor(o.t, e.src1, D.dst, A->po_arg[i])) return false;
+        } else if (e.kind == pk_prelu) {
+            qmm_tensor_t w = D.dst;
+            w.dt = dt_f32;
+            for (int d = 0; d < nd; d++) {
+                // -1 never equals a dst dim: masked-out dims broadcast
+                w.dims[d] = (e.mask & (1 << d)) ? D.dst.dims[d] : -1;
+                w.strides[d] = e.src1.strides[d];
+            }
+            if (!fold_tensor(o.t, w, D.dst, A->po_arg[i])) return false;
+        } else if (e.kind == pk_sum) {
+            o.t.dt = P.sum_dt;
+        } else if (e.kind != pk_eltwise) {
+            return false;
+        }
+    }
+    return true;
+}
+
+// ---------------------------------------------------------------------------
+bool plain_wei_strides(const qmm_matmul_desc_t &D, int64_t &sb, int64_t &sk,
+        int64_t &sn) {
+    const int nd = D.wei.ndims;
+    sk = D.wei.strides[nd - 2];
+    sn = D.wei.strides[nd - 1];
+    return fold_batch(D.wei, D.dst, sb);
+}
+
+int64_t wei_batch(const qmm_matmul_desc_t &D) {
+    int64_t b = 1;
+    for (int d = 0; d < D.wei.ndims - 2; d++)
+        b *= D.wei.dims[d];
+    return b;
+}
+
+int supports_gemm_b8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    const int nd = D.dst.ndims;
+    const bool i8 = is_int8(D.src.dt) && D.wei.dt == dt_s8;
+    const bool f8 = D.src.dt == dt_f8_e4m3 && D.wei.dt == dt_f8_e4m3;
+    if (!i8 && !f8) return QMM_UNIMPLEMENTED;
+    if (i8 && !one_of(D.dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s32, dt_s8, dt_u8}))
+        return QMM_UNIMPLEMENTED;
+    if (f8 && !one_of(D.dst.dt, {dt_f32, dt_bf16, dt_f16, dt_f8_e4m3, dt_f8_e5m2}))
+        return QMM_UNIMPLEMENTED;
+    if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
+    if (P.M > INT32_MAX || P.N > INT32_MAX || P.K > INT32_MAX
+            || P.batch > 65535)
+        return QMM_UNIMPLEMENTED;
+    if (!one_of(D.wei_layout, {QMM_LAYOUT_PLAIN, QMM_LAYOUT_MFMA_B8}))
+        return QMM_UNIMPLEMENTED;
+    // weights batch dims: all present or all broadcast
+    const int64_t wb = wei_batch(D);
+    if (wb != 1 && wb != P.batch) return QMM_UNIMPLEMENTED;
+    if (D.wei_layout == QMM_LAYOUT_PLAIN) {
+        int64_t sb, sk, sn;
+        if (!plain_wei_strides(D, sb, sk, sn)) return QMM_UNIMPLEMENTED;
+    }
+    // source rows K-contiguous, 16-byte granular
+    if (D.src.strides[nd - 1] != 1 || P.K % 16 != 0
+            || D.src.strides[nd - 2] % 16 != 0)
+        return QMM_UNIMPLEMENTED;
+    int64_t a_sb;
+    if (!fold_batch(D.src, D.dst, a_sb) || a_sb % 16 != 0)
+        return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_WEI].set) return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_SRC].set) {
+        if (!i8 || D.zps[QMM_SRC].mask != 0) return QMM_UNIMPLEMENTED;
+        if (!one_of(D.zps[QMM_SRC].dt, {dt_s32, dt_s8, dt_u8}))
+            return QMM_UNIMPLEMENTED;
+    }
+    if (f8 && D.scales[QMM_SRC].set && D.scales[QMM_SRC].mask != 0)
+        return QMM_UNIMPLEMENTED;
+    if (f8 && D.scales[QMM_WEI].set
+            && (D.scales[QMM_WEI].mask & ~(1 << (nd - 1))))
+        return QMM_UNIMPLEMENTED;
+    if (f8 && D.zps[QMM_DST].set) return QMM_UNIMPLEMENTED;
+    epilogue_t ep;
+    if (!build_epilogue(ep, P, nullptr)) return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
+int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    const int nd = D.dst.ndims;
+    if (nd != 2) return QMM_UNIMPLEMENTED;
+    if (!one_of(D.src.dt, {dt_bf16, dt_f16}) || !is_int4(D.wei.dt)
+            || !D.apply_to_int)
+        return QMM_UNIMPLEMENTED;
+    if (D.src.dt == dt_bf16 && !one_of(D.dst.dt, {dt_bf16, dt_f32}))
+        return QMM_UNIMPLEMENTED;
+    if (D.src.dt == dt_f16 && !one_of(D.dst.dt, {dt_f16, dt_f32}))
+        return QMM_UNIMPLEMENTED;
+    if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
+    if (P.M > INT32_MAX || P.N > INT32_MAX || P.K > INT32_MAX)
+        return QMM_UNIMPLEMENTED;
+    if (!one_of(D.wei_layout, {QMM_LAYOUT_PLAIN, QMM_LAYOUT_MFMA_W4}))
+        return QMM_UNIMPLEMENTED;
+    if (D.src.strides[1] != 1 || P.K % 8 != 0 || D.src.strides[0] % 8 != 0)
+        return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_SRC].set || D.zps[QMM_DST].set) return QMM_UNIMPLEMENTED;
+    if (D.scales[QMM_SRC].set && D.scales[QMM_SRC].mask != 0)
+        return QMM_UNIMPLEMENTED;
+    const qmm_quant_t &ws = D.scales[QMM_WEI], &wz = D.zps[QMM_WEI];
+    if (ws.set) {
+        if (!one_of(ws.dt, {dt_f32, dt_f16, dt_bf16})) return QMM_UNIMPLEMENTED;
+        if (P.q_wei_scale.g1 != 1) return QMM_UNIMPLEMENTED; // N groups
+        if ((ws.mask & 1) && (P.q_wei_scale.g0 % 32 != 0))
+            return QMM_UNIMPLEMENTED;
+        if ((ws.mask & 1) && P.K % P.q_wei_scale.g0 != 0)
+            return QMM_UNIMPLEMENTED;
+    }
+    if (wz.set) {
+        if (!one_of(wz.dt, {dt_s32, dt_s8, dt_u8, dt_s4, dt_u4}))
+            return QMM_UNIMPLEMENTED;
+        if (P.q_wei_zp.g1 != 1) return QMM_UNIMPLEMENTED;
+        if ((wz.mask & 1) && (P.q_wei_zp.g0 % 32 != 0)) return QMM_UNIMPLEMENTED;
+        if ((wz.mask & 1) && P.K % P.q_wei_zp.g0 != 0) return QMM_UNIMPLEMENTED;
+    }
+    epilogue_t ep;
+    if (!build_epilogue(ep, P, nullptr)) return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
+int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    if (D.wei_layout != QMM_LAYOUT_PLAIN) return QMM_UNIMPLEMENTED;
+    const int s = D.src.dt, w = D.wei.dt, d = D.dst.dt;
+    if (is_int8(s)) {
+        // src/cpu/matmul/ref_matmul_int8.hpp:43-129
+        if (!is_wei_int(w)) return QMM_UNIMPLEMENTED;
+        if (!one_of(d, {dt_f32, dt_bf16, dt_f16, dt_s32, dt_s8, dt_u8}))
+            return QMM_UNIMPLEMENTED;
+    } else {
+        // src/cpu/matmul/ref_matmul.hpp:44-157
+        if (!one_of(s, {dt_f32, dt_bf16, dt_f16, dt_f8_e5m2, dt_f8_e4m3}))
+            return QMM_UNIMPLEMENTED;
+        if (!one_of(w, {dt_f32, dt_bf16, dt_f16, dt_f8_e5m2, dt_f8_e4m3, dt_u8,
+                    dt_s8, dt_u4, dt_s4}))
+            return QMM_UNIMPLEMENTED;
+        if (!one_of(d, {dt_f32, dt_bf16, dt_f16, dt_f8_e5m2, dt_f8_e4m3}))
+            return QMM_UNIMPLEMENTED;
+        if (!(s == w || one_of(w, {dt_bf16, dt_f16, dt_u8, dt_s8, dt_u4, dt_s4})))
+            return QMM_UNIMPLEMENTED;
+        if (is_int8(w) && !D.apply_to_int) return QMM_UNIMPLEMENTED;
+        if (s == dt_f32 && d != dt_f32) return QMM_UNIMPLEMENTED;
+        if (s == dt_bf16 && !one_of(d, {dt_f32, dt_bf16})) return QMM_UNIMPLEMENTED;
+        if (s == dt_f16 && !one_of(d, {dt_f32, dt_f16})) return QMM_UNIMPLEMENTED;
+        if (D.zps[QMM_SRC].set || D.zps[QMM_DST].set) return QMM_UNIMPLEMENTED;
+        if (D.scales[QMM_SRC].set && D.scales[QMM_SRC].mask != 0)
+            return QMM_UNIMPLEMENTED;
+        if (D.scales[QMM_WEI].set && !P.decompress
+                && (D.scales[QMM_WEI].mask & ~(1 << (D.dst.ndims - 1))))
+            return QMM_UNIMPLEMENTED;
+    }
+    if (D.scales[QMM_DST].set && D.scales[QMM_DST].mask != 0)
+        return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_DST].set && D.zps[QMM_DST].dt != dt_s32)
+        return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
+const char *impl_names[impl_count]
+        = {"hip:gfx950:mfma_b8", "hip:gfx950:decode_w4", "hip:gfx950:generic"};
+
+int g_gemm_variant = 0;
+
+} // namespace
+
+extern "C" {
+
+const char *qmm_last_error(void) {
+    return g_last_error.c_str();
+}
+
+int qmm_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int qmm_matmul_impl_count(void) {
+    return impl_count;
+}
+const char *qmm_matmul_impl_name(int impl) {
+    return impl >= 0 && impl < impl_count ? impl_names[impl] : "";
+}
+
+int qmm_matmul_impl_supports(int impl, const qmm_matmul_desc_t *desc) {
+    if (!desc || desc->dst.ndims < 2 || desc->dst.ndims > QMM_MAX_NDIMS)
+        return QMM_INVALID_ARGUMENTS;
+    generic_params_t P;
+    build_generic(P, *desc);
+    switch (impl) {
+        case impl_gemm_b8: return supports_gemm_b8(*desc, P);
+        case impl_gemv_w4: return supports_gemv_w4(*desc, P);
+        case impl_generic: return supports_generic(*desc, P);
+        default: return QMM_INVALID_ARGUMENTS;
+    }
+}
+
+size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N) {
+    (void)dt;
+    if (layout == QMM_LAYOUT_MFMA_B8)
+        return (size_t)b8_geom(batch, K, N).total_bytes;
+    if (layout == QMM_LAYOUT_MFMA_W4)
+        return (size_t)w4_geom(batch, K, N).total_bytes;
+    return 0;
+}
+
+int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
+    qmm_matmul_desc_t d = *desc;
+    // strides of an undecided weights tensor are not meaningful yet
+    d.wei_layout = QMM_LAYOUT_MFMA_B8;
+    if (qmm_matmul_impl_supports(impl_gemm_b8, &d) == QMM_OK)
+        return QMM_LAYOUT_MFMA_B8;
+    d.wei_layout = QMM_LAYOUT_MFMA_W4;
+    if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
+        return QMM_LAYOUT_MFMA_W4;
+    return QMM_LAYOUT_PLAIN;
+}
+
+size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
+    if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
+    const int nd = desc->wei.ndims;
+    const int64_t K = desc->wei.dims[nd - 2], N = desc->wei.dims[nd - 1];
+    if (impl == impl_gemm_b8)
+        return qmm_packed_size(
+                QMM_LAYOUT_MFMA_B8, desc->wei.dt, wei_batch(*desc), K, N);
+    if (impl == impl_gemv_w4)
+        return qmm_packed_size(QMM_LAYOUT_MFMA_W4, desc->wei.dt, 1, K, N);
+    return 0;
+}
+
+int qmm_matmul_plan_create(
+        qmm_plan_t **plan, int impl, const qmm_matmul_desc_t *desc) {
+    if (!plan || !desc) return QMM_INVALID_ARGUMENTS;
+    const int st = qmm_matmul_impl_supports(impl, desc);
+    if (st != QMM_OK) return st;
+    qmm_plan *p = new (std::nothrow) qmm_plan();
+    if (!p) return QMM_OUT_OF_MEMORY;
+    p->impl = impl;
+    p->desc = *desc;
+    p->dev = nullptr;
+    build_generic(p->host, *desc);
+    p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
+    // the generic kernel reads its (large) descriptor from device memory; the
+    // tiled kernels fall back to it for operands they cannot address (pointers
+    // that are not 16-byte aligned), so every plan over plain weights keeps one
+    if (desc->wei_layout == QMM_LAYOUT_PLAIN
+            && supports_generic(*desc, p->host) == QMM_OK) {
+        hipError_t e = hipMalloc((void **)&p->dev, sizeof(generic_params_t));
+        if (e != hipSuccess) {
+            delete p;
+            return hip_fail(e, "hipMalloc(plan)");
+        }
+        e = hipMemcpy(p->dev, &p->host, sizeof(generic_params_t),
+                hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(p->dev);
+            delete p;
+            return hip_fail(e, "hipMemcpy(plan)");
+        }
+    }
+    *plan = p;
+    return QMM_OK;
+}
+
+void qmm_matmul_plan_destroy(qmm_plan_t *plan) {
+    if (!plan) return;
+    if (plan->dev) (void)hipFree(plan->dev);
+    delete plan;
+}
+
+static bool aligned16(const void *p) {
+    return ((uintptr_t)p & 15) == 0;
+}
+
+int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
+        void *hip_stream) {
+    if (!plan || !args) return QMM_INVALID_ARGUMENTS;
+    hipStream_t stream = (hipStream_t)hip_stream;
+    const qmm_matmul_desc_t &D = plan->desc;
+    const generic_params_t &P = plan->host;
+    const int nd = D.dst.ndims;
+    if (P.M == 0 || P.N == 0 || P.batch == 0) return QMM_OK;
+    if (!args->src || !args->wei || !args->dst)
+        return fail(QMM_INVALID_ARGUMENTS, "null src/weights/dst pointer");
+    for (int i = 0; i < 3; i++) {
+        if (D.scales[i].set && !args->scales[i])
+            return fail(QMM_INVALID_ARGUMENTS, "scales buffer is missing");
+        if (D.zps[i].set && !args->zps[i])
+            return fail(QMM_INVALID_ARGUMENTS, "zero points buffer is missing");
+    }
+    for (int i = 0; i < D.npo; i++)
+        if ((D.po[i].kind == pk_binary || D.po[i].kind == pk_prelu)
+                && !args->po_arg[i])
+            return fail(QMM_INVALID_ARGUMENTS, "post-op argument is missing");
+    if (D.bias.ndims && !args->bias)
+        return fail(QMM_INVALID_ARGUMENTS, "bias pointer is missing");
+    if (plan->scratch_bytes && !args->scratch)
+        return fail(QMM_INVALID_ARGUMENTS, "scratch buffer is missing");
+
+    int impl = plan->impl;
+    if (impl != impl_generic && !aligned16(args->src)) {
+        if (!plan->dev)
+            return fail(QMM_INVALID_ARGUMENTS,
+                    "source pointer must be 16-byte aligned");
+        impl = impl_generic;
+    }
+
+    if (impl == impl_generic) {
+        if (!plan->dev) return fail(QMM_RUNTIME_ERROR, "plan has no device copy");
+        launch_matmul_generic(plan->dev, P, *args, stream);
+    } else if (impl == impl_gemm_b8) {
+        const bool f8 = D.src.dt == dt_f8_e4m3;
+        gemm_params_t g;
+        std::memset(&g, 0, sizeof(g));
+        if (!build_epilogue(g.ep, P, args))
+            return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
+        g.A = (const uint8_t *)args->src;
+        g.lda = D.src.strides[nd - 2];
+        fold_batch(D.src, D.dst, g.a_sb);
+        const int64_t wb = wei_batch(D);
+        const b8_geom_t geom = b8_geom(wb, P.K, P.N);
+        const uint8_t *packed = (const uint8_t *)args->wei;
+        if (D.wei_layout == QMM_LAYOUT_PLAIN) {
+            int64_t sb, sk, sn;
+            plain_wei_strides(D, sb, sk, sn);
+            if (wb == 1) sb = 0;
+            launch_pack_b8(args->wei, args->scratch, D.wei.dt, wb, P.K, P.N, sb,
+                    sk, sn, !f8, stream);
+            packed = (const uint8_t *)args->scratch;
+        }
+        g.B = packed;
+        g.b_sb = wb == 1 ? 0 : geom.batch_bytes;
+        g.colsum = f8 ? nullptr : (const int32_t *)(packed + geom.colsum_off);
+        g.colsum_sb = wb == 1 ? 0 : geom.Npad;
+        g.src_zp = D.zps[QMM_SRC].set ? args->zps[QMM_SRC] : nullptr;
+        g.src_zp_dt = D.zps[QMM_SRC].dt;
+        g.a_is_u8 = D.src.dt == dt_u8;
+        g.M = (int32_t)P.M;
+        g.N = (int32_t)P.N;
+        g.K = (int32_t)P.K;
+        g.batch = (int32_t)P.batch;
+        g.kb32 = (int32_t)geom.kb32;
+        g.nb32 = (int32_t)geom.nb32;
+        launch_gemm_b8(g, f8, g_gemm_variant, stream);
+    } else if (impl == impl_gemv_w4) {
+        gemv_params_t g;
+        std::memset(&g, 0, sizeof(g));
+        if (!build_epilogue(g.ep, P, args))
+            return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
+        const w4_geom_t geom = w4_geom(1, P.K, P.N);
+        const uint8_t *packed = (const uint8_t *)args->wei;
+        if (D.wei_layout == QMM_LAYOUT_PLAIN) {
+            launch_pack_w4(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N, 0,
+                    D.wei.strides[0], D.wei.strides[1], stream);
+            packed = (const uint8_t *)args->scratch;
+        }
+        g.A = (const uint16_t *)args->src;
+        g.lda = D.src.strides[0];
+        g.B = packed;
+        const qmm_quant_t &ws = D.scales[QMM_WEI], &wz = D.zps[QMM_WEI];
+        const int Kpad = (int)geom.Kpad;
+        g.scales = ws.set ? args->scales[QMM_WEI] : nullptr;
+        g.scale_dt = ws.dt;
+        g.gs = (ws.set && (ws.mask & 1)) ? (int)P.q_wei_scale.g0 : Kpad;
+        g.scale_per_n = ws.set && (ws.mask & 2);
+        g.zps = wz.set ? args->zps[QMM_WEI] : nullptr;
+        g.zp_dt = wz.dt;
+        g.gz = (wz.set && (wz.mask & 1)) ? (int)P.q_wei_zp.g0 : 0;
+        g.zp_per_n = wz.set && (wz.mask & 2);
+        g.M = (int32_t)P.M;
+        g.N = (int32_t)P.N;
+        g.K = (int32_t)P.K;
+        g.kg128 = (int32_t)geom.kg128;
+        g.nb16 = (int32_t)geom.nb16;
+        g.wei_signed = D.wei.dt == dt_s4;
+        g.act_f16 = D.src.dt == dt_f16;
+        g.m0 = 0;
+        launch_gemv_w4(g, stream);
+    } else {
+        return fail(QMM_INVALID_ARGUMENTS, "unknown implementation");
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "kernel launch");
+    return QMM_OK;
+}
+
+// tuning hook used by the benchmark sweep: tile configuration of mfma_b8
+QMM_API void qmm_set_gemm_variant(int v) {
+    g_gemm_variant = v;
+}
+
+// ---------------------------------------------------------------------------
+static bool is_plain_copy_dt(int a, int b) {
+    return a == b;
+}
+
+int qmm_reorder_supports(const qmm_reorder_desc_t *d) {
+    if (!d) return QMM_INVALID_ARGUMENTS;
+    const int nd = d->src.ndims;
+    if (nd != d->dst.ndims || nd < 1 || nd > QMM_MAX_NDIMS)
+        return QMM_INVALID_ARGUMENTS;
+    const bool quant = d->src_scale.set || d->dst_scale.set || d->src_zp.set
+            || d->dst_zp.set;
+    if (d->src_layout == QMM_LAYOUT_PLAIN && d->dst_layout == QMM_LAYOUT_PLAIN) {
+        const int s = d->src.dt, t = d->dst.dt;
+        if (!one_of(s, {dt_f32, dt_bf16, dt_f16, dt_f8_e4m3, dt_f8_e5m2, dt_s32,
+                    dt_s8, dt_u8, dt_s4, dt_u4}))
+            return QMM_UNIMPLEMENTED;
+        if (!one_of(t, {dt_f32, dt_bf16, dt_f16, dt_f8_e4m3, dt_f8_e5m2, dt_s32,
+                    dt_s8, dt_u8, dt_s4, dt_u4}))
+            return QMM_UNIMPLEMENTED;
+        if (is_int4(t)) {
+            // the pair owner scheme needs a stride-1 dim of even extent
+            bool ok = false;
+            for (int i = 0; i < nd; i++)
+                if (d->dst.strides[i] == 1 && d->dst.dims[i] % 2 == 0) ok = true;
+            if (!ok) return QMM_UNIMPLEMENTED;
+        }
+        if (d->dst_zp.set && d->dst_zp.mask != 0) return QMM_UNIMPLEMENTED;
+        return QMM_OK;
+    }
+    // packing / unpacking: same data type, no quantization, >= 2 dims
+    if (quant || nd < 2 || !is_plain_copy_dt(d->src.dt, d->dst.dt))
+        return QMM_UNIMPLEMENTED;
+    const int packed
+            = d->src_layout == QMM_LAYOUT_PLAIN ? d->dst_layout : d->src_layout;
+    if (d->src_layout != QMM_LAYOUT_PLAIN && d->dst_layout != QMM_LAYOUT_PLAIN)
+        return QMM_UNIMPLEMENTED;
+    const qmm_tensor_t &pl
+            = d->src_layout == QMM_LAYOUT_PLAIN ? d->src : d->dst;
+    // batch dims of the plain side must nest densely
+    qmm_tensor_t shape = pl;
+    int64_t sb;
+    if (!fold_batch(pl, shape, sb)) return QMM_UNIMPLEMENTED;
+    if (packed == QMM_LAYOUT_MFMA_B8) {
+        if (!one_of(pl.dt, {dt_s8, dt_u8, dt_f8_e4m3, dt_f8_e5m2}))
+            return QMM_UNIMPLEMENTED;
+        return QMM_OK;
+    }
+    if (packed == QMM_LAYOUT_MFMA_W4) {
+        if (!is_int4(pl.dt)) return QMM_UNIMPLEMENTED;
+        if (d->dst_layout == QMM_LAYOUT_PLAIN) {
+            // unpack writes byte pairs along the stride-1 dim
+            const bool n_inner = pl.strides[nd - 1] == 1
+                    && pl.dims[nd - 1] % 2 == 0;
+            const bool k_inner = pl.strides[nd - 2] == 1
+                    && pl.dims[nd - 2] % 2 == 0;
+            if (!n_inner && !k_inner) return QMM_UNIMPLEMENTED;
+        }
+        return QMM_OK;
+    }
+    return QMM_UNIMPLEMENTED;
+}
+
+int qmm_reorder_launch(const qmm_reorder_desc_t *d,
+        const qmm_reorder_args_t *args, void *hip_stream) {
+    const int st = qmm_reorder_supports(d);
+    if (st != QMM_OK) return st;
+    if (!args || !args->src || !args->dst)
+        return fail(QMM_INVALID_ARGUMENTS, "null reorder pointer");
+    hipStream_t stream = (hipStream_t)hip_stream;
+    const int nd = d->src.ndims;
+    int64_t nelems = 1;
+    for (int i = 0; i < nd; i++)
+        nelems *= d->src.dims[i];
+    if (nelems == 0) return QMM_OK;
+
+    if (d->src_layout == QMM_LAYOUT_PLAIN && d->dst_layout == QMM_LAYOUT_PLAIN) {
+        generic_reorder_params_t P;
+        std::memset(&P, 0, sizeof(P));
+        P.desc = *d;
+        P.nelems = nelems;
+        for (int i = 0; i < nd; i++)
+            if (d->dst.strides[i] == 1 && d->dst.dims[i] % 2 == 0) P.pair_dim = i;
+        quant_geom(P.q_src_scale, d->src_scale, nd, d->src.dims,
+                group_or(d->src_scale, 0, 1), group_or(d->src_scale, 1, 1));
+        quant_geom(P.q_dst_scale, d->dst_scale, nd, d->src.dims, 1, 1);
+        quant_geom(P.q_src_zp, d->src_zp, nd, d->src.dims,
+                group_or(d->src_zp, 0, 1), group_or(d->src_zp, 1, 1));
+        if ((d->src_scale.set && !args->src_scale)
+                || (d->dst_scale.set && !args->dst_scale)
+                || (d->src_zp.set && !args->src_zp)
+                || (d->dst_zp.set && !args->dst_zp))
+            return fail(QMM_INVALID_ARGUMENTS, "reorder attribute buffer missing");
+        launch_reorder_generic(P, *args, stream);
+    } else {
+        const bool packing = d->src_layout == QMM_LAYOUT_PLAIN;
+        const qmm_tensor_t &pl = packing ? d->src : d->dst;
+        const int packed = packing ? d->dst_layout : d->src_layout;
+        const int64_t K = pl.dims[nd - 2], N = pl.dims[nd - 1];
+        int64_t batch = 1;
+        for (int i = 0; i < nd - 2; i++)
+            batch *= pl.dims[i];
+        int64_t sb = 0;
+        qmm_tensor_t shape = pl;
+        fold_batch(pl, shape, sb);
+        const int64_t sk = pl.strides[nd - 2], sn = pl.strides[nd - 1];
+        if (packed == QMM_LAYOUT_MFMA_B8) {
+            if (packing)
+                launch_pack_b8(args->src, args->dst, pl.dt, batch, K, N, sb, sk,
+                        sn, pl.dt == dt_s8 || pl.dt == dt_u8, stream);
+            else
+                launch_unpack_b8(args->src, args->dst, pl.dt, batch, K, N, sb,
+                        sk, sn, stream);
+        } else {
+            if (packing)
+                launch_pack_w4(args->src, args->dst, pl.dt, batch, K, N, sb, sk,
+                        sn, stream);
+            else
+                launch_unpack_w4(args->src, args->dst, pl.dt, batch, K, N, sb,
+                        sk, sn, stream);
+        }
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "reorder launch");
+    return QMM_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,382 @@
+// hip:gfx950:mfma_b8 -- int8 (u8/s8 x s8 -> s32) and fp8 (e4m3 x e4m3 -> f32)
+// GEMM on the CDNA4 matrix cores with a fused epilogue.
+//
+// Layout of the work:
+//   * weights arrive prepacked in MFMA operand order (QMM_LAYOUT_MFMA_B8): a
+//     32-column x 32-k fragment is 1 KiB, lane l holds column l%32 and the 16
+//     k-bytes of half l/32, so a tile of the B operand is a plain contiguous
+//     copy global -> LDS and the ds_read_b128 of a wave is conflict free;
+//   * the source rows are staged row-major in LDS with an XOR swizzle of the
+//     16-byte chunks, which keeps both the coalesced global load (a row's
+//     BK bytes by consecutive lanes) and the fragment reads (32 rows x 16 B)
+//     spread over all 64 banks;
+//   * a block of 4 waves owns a BM x BN tile, each wave WM x WN of it as
+//     FM x FN v_mfma_i32_32x32x32_i8 (or v_mfma_f32_32x32x64_f8f6f4)
+//     accumulators; LDS is double buffered, the next tile's global loads are
+//     in flight while the current one is multiplied;
+//   * u8 sources are turned into s8 by flipping the top bit and the missing
+//     128 * colsum(W)[n] (and the source zero point, -zp * colsum(W)[n]) is
+//     added to the s32 accumulator from the column sums stored behind the
+//     packed weights (identity of
+//     src/cpu/matmul/gemm_x8s8s32x_matmul.cpp:165-193) -- exact in s32;
+//   * the epilogue follows src/cpu/matmul/ref_matmul_int8.cpp:195-259 step by
+//     step: (float)acc, * src scale, * weights scale, + bias, post-ops,
+//     * 1/dst scale, + dst zero point, saturating store.
+//
+// Blocks are numbered so that the eight XCDs (each with its own L2) work on
+// disjoint column ranges of the weights, and consecutive blocks of an XCD
+// share source rows.
+#include <type_traits>
+
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <bool F8>
+struct acc_traits;
+template <>
+struct acc_traits<false> {
+    typedef v16i type;
+};
+template <>
+struct acc_traits<true> {
+    typedef v16f type;
+};
+
+// compile-time loop: the body sees its index as a constant, so accumulator
+// arrays indexed by it stay in registers whatever the optimizer decides about
+// the loops inside the body
+template <int N, typename F>
+QMM_D void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1> {});
+    }
+}
+
+// chunk swizzle of the row-major A tile: CH 16-byte chunks per row
+template <int CH>
+QMM_D int a_swz(int row, int q) {
+    constexpr int ROWS_PER_256B = 16 / CH;
+    return q ^ ((row / ROWS_PER_256B) % CH);
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, bool F8>
+__global__ void __launch_bounds__(WGM *WGN * 64, (BM * BN <= 256 * 128) ? 2 : 1)
+gemm_b8_kernel(const gemm_params_t p) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int FM = WM / 32, FN = WN / 32;
+    constexpr int KF = BK / 32; // k32 fragments per tile
+    constexpr int CH = BK / 16; // 16-byte chunks per A row
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int A_CH = A_BYTES / 16 / NT, B_CH = B_BYTES / 16 / NT;
+    static_assert(A_CH * 16 * NT == A_BYTES && B_CH * 16 * NT == B_BYTES, "");
+    static_assert(!F8 || (KF % 2 == 0), "fp8 MFMA consumes 64 k per step");
+    typedef typename acc_traits<F8>::type acc_t;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *const As0 = lds;
+    uint8_t *const Bs0 = lds + 2 * A_BYTES;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm0 = (wave / WGN) * WM;
+    const int wn0 = (wave % WGN) * WN;
+
+    // ---- XCD-aware tile order ----
+    // Hardware hands consecutive block ids to the 8 XCDs round robin. Give
+    // XCD x the logical tiles [x*per, (x+1)*per): consecutive logical tiles
+    // run on one XCD and share its L2. Logical order is n-major within groups
+    // of GROUP_M row tiles, so neighbours share weight columns and src rows.
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt = blockIdx.x;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        if (ntiles >= 64) {
+            lt = xcd * per + slot;
+            if (slot >= per || lt >= ntiles) return;
+        }
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const uint8_t *__restrict__ A = p.A + (int64_t)bz * p.a_sb;
+    const uint8_t *__restrict__ B = p.B + (int64_t)bz * p.b_sb;
+
+    acc_t acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0;
+
+    const int KT = (p.K + BK - 1) / BK;
+    uint4 ra[A_CH], rb[B_CH];
+
+    auto gload = [&](int kt) {
+#pragma unroll
+        for (int j = 0; j < A_CH; j++) {
+            const int c = tid + j * NT;
+            const int row = c / CH, q = c % CH;
+            const int gm = m0 + row;
+            const int gk = kt * BK + q * 16;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (gm < p.M && gk < p.K)
+                v = *(const uint4 *)(A + (int64_t)gm * p.lda + gk);
+            ra[j] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < B_CH; j++) {
+            const int c = tid + j * NT;
+            const int nbl = c / (KF * 64), rem = c % (KF * 64);
+            const int nb = n0 / 32 + nbl;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (nb < p.nb32)
+                v = *(const uint4 *)(B
+                        + ((int64_t)nb * p.kb32 + (int64_t)kt * KF) * 1024
+                        + rem * 16);
+            rb[j] = v;
+        }
+    };
+    auto lstore = [&](int stage) {
+        uint8_t *As = As0 + stage * A_BYTES;
+        uint8_t *Bs = Bs0 + stage * B_BYTES;
+#pragma unroll
+        for (int j = 0; j < A_CH; j++) {
+            const int c = tid + j * NT;
+            const int row = c / CH, q = c % CH;
+            *(uint4 *)(As + row * BK + a_swz<CH>(row, q) * 16) = ra[j];
+        }
+#pragma unroll
+        for (int j = 0; j < B_CH; j++) {
+            const int c = tid + j * NT;
+            *(uint4 *)(Bs + c * 16) = rb[j];
+        }
+    };
+
+    gload(0);
+    lstore(0);
+    __syncthreads();
+
+    const uint32_t flip = p.a_is_u8 ? 0x80808080u : 0u;
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int stage = kt & 1;
+        if (kt + 1 < KT) gload(kt + 1);
+        const uint8_t *As = As0 + stage * A_BYTES;
+        const uint8_t *Bs = Bs0 + stage * B_BYTES;
+        if constexpr (!F8) {
+#pragma unroll
+            for (int ki = 0; ki < KF; ki++) {
+                v4i a[FM], b[FN];
+#pragma unroll
+                for (int i = 0; i < FM; i++) {
+                    const int row = wm0 + i * 32 + (lane & 31);
+                    const int q = ki * 2 + (lane >> 5);
+                    uint4 v = *(const uint4 *)(As + row * BK
+                            + a_swz<CH>(row, q) * 16);
+                    v.x ^= flip;
+                    v.y ^= flip;
+                    v.z ^= flip;
+                    v.w ^= flip;
+                    a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                }
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    const uint4 v = *(const uint4 *)(Bs
+                            + ((((wn0 >> 5) + j) * KF + ki) * 64 + lane) * 16);
+                    b[j] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                }
+#pragma unroll
+                for (int i = 0; i < FM; i++)
+#pragma unroll
+                    for (int j = 0; j < FN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int ki = 0; ki < KF; ki += 2) {
+                v8i a[FM], b[FN];
+#pragma unroll
+                for (int i = 0; i < FM; i++) {
+                    const int row = wm0 + i * 32 + (lane & 31);
+                    const int q0 = ki * 2 + (lane >> 5);
+                    const uint4 v0 = *(const uint4 *)(As + row * BK
+                            + a_swz<CH>(row, q0) * 16);
+                    const uint4 v1 = *(const uint4 *)(As + row * BK
+                            + a_swz<CH>(row, q0 + 2) * 16);
+                    a[i] = v8i {(int)v0.x, (int)v0.y, (int)v0.z, (int)v0.w,
+                            (int)v1.x, (int)v1.y, (int)v1.z, (int)v1.w};
+                }
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    const uint8_t *bp = Bs
+                            + ((((wn0 >> 5) + j) * KF + ki) * 64 + lane) * 16;
+                    const uint4 v0 = *(const uint4 *)bp;
+                    const uint4 v1 = *(const uint4 *)(bp + 1024);
+                    b[j] = v8i {(int)v0.x, (int)v0.y, (int)v0.z, (int)v0.w,
+                            (int)v1.x, (int)v1.y, (int)v1.z, (int)v1.w};
+                }
+#pragma unroll
+                for (int i = 0; i < FM; i++)
+#pragma unroll
+                    for (int j = 0; j < FN; j++)
+                        acc[i][j]
+                                = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                                        a[i], b[j], acc[i][j], 0, 0, 0, 0, 0,
+                                        0);
+            }
+        }
+        if (kt + 1 < KT) lstore(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- zero-point compensation (integer path) ----
+    int comp = 0;
+    if constexpr (!F8) {
+        comp = p.a_is_u8 ? 128 : 0;
+        if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+    }
+
+    // ---- epilogue ----
+    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column
+    // l%32 of its 32x32 fragment: a lane owns one column. The results of one
+    // 32-row band of the wave tile go through a wave-private LDS tile and come
+    // back row-wise, 4 neighbouring columns per lane, so that the post-op code
+    // exists once (run-time loop) and every store is a dense vector.
+    float *const stg = (float *)lds + wave * (32 * WN);
+    int cs[FN];
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+        cs[j] = 0;
+        if constexpr (!F8) {
+            const int n = n0 + wn0 + j * 32 + (lane & 31);
+            if (n < p.N && comp != 0 && p.colsum)
+                cs[j] = comp * p.colsum[(int64_t)bz * p.colsum_sb + n];
+        }
+    }
+    constexpr int ROWS_PER_IT = 256 / WN; // 64 lanes x 4 columns
+    static_for<FM>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                float v;
+                if constexpr (F8)
+                    v = acc[i][j][r];
+                else
+                    v = (float)(int32_t)((uint32_t)acc[i][j][r]
+                            + (uint32_t)cs[j]);
+                stg[row * WN + j * 32 + (lane & 31)] = v;
+            }
+        }
+#pragma unroll 1
+        for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+            const int row = it * ROWS_PER_IT + lane / (WN / 4);
+            const int col = (lane % (WN / 4)) * 4;
+            const float4 t = *(const float4 *)&stg[row * WN + col];
+            const int m = m0 + wm0 + i * 32 + row;
+            const int n = n0 + wn0 + col;
+            if (m < p.M && n < p.N) {
+                float v[4] = {t.x, t.y, t.z, t.w};
+                epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
+            }
+        }
+    });
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, bool F8>
+static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
+    gemm_params_t q = p;
+    q.tiles_m = (p.M + BM - 1) / BM;
+    q.tiles_n = (p.N + BN - 1) / BN;
+    const int ntiles = q.tiles_m * q.tiles_n;
+    // with the XCD remap every XCD gets ceil(ntiles/8) slots
+    const int grid_x = ntiles >= 64 ? ((ntiles + 7) / 8) * 8 : ntiles;
+    constexpr size_t lds_main = 2 * (size_t)(BM + BN) * BK;
+    constexpr size_t lds_ep
+            = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
+    constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
+    auto kern = gemm_b8_kernel<BM, BN, BK, WGM, WGN, F8>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void *)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(WGM * WGN * 64), lds,
+            stream, q);
+}
+
+// One tile configuration per translation unit (QMM_GEMM_VARIANT), so the
+// instantiations build in parallel; the unit without the macro holds the
+// dispatcher.
+#if defined(QMM_GEMM_VARIANT)
+#if QMM_GEMM_VARIANT == 1
+#define QMM_CFG 256, 128, 64, 2, 2
+#elif QMM_GEMM_VARIANT == 2
+#define QMM_CFG 128, 128, 64, 2, 2
+#elif QMM_GEMM_VARIANT == 3
+#define QMM_CFG 256, 256, 64, 2, 2
+#elif QMM_GEMM_VARIANT == 4
+#define QMM_CFG 128, 256, 64, 2, 2
+#elif QMM_GEMM_VARIANT == 5
+#define QMM_CFG 256, 128, 128, 2, 2
+#endif
+#define QMM_CAT_(a, b) a##b
+#define QMM_CAT(a, b) QMM_CAT_(a, b)
+void QMM_CAT(launch_gemm_b8_v, QMM_GEMM_VARIANT)(
+        const gemm_params_t &p, bool f8, hipStream_t stream) {
+    if (f8)
+        launch_cfg<QMM_CFG, true>(p, stream);
+    else
+        launch_cfg<QMM_CFG, false>(p, stream);
+}
+#else
+void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);
+void launch_gemm_b8_v2(const gemm_params_t &p, bool f8, hipStream_t stream);
+void launch_gemm_b8_v3(const gemm_params_t &p, bool f8, hipStream_t stream);
+void launch_gemm_b8_v4(const gemm_params_t &p, bool f8, hipStream_t stream);
+void launch_gemm_b8_v5(const gemm_params_t &p, bool f8, hipStream_t stream);
+
+// variant: 0 = heuristic; others pick a tile configuration explicitly (used by
+// the tuning sweep)
+void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
+        hipStream_t stream) {
+    if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return;
+    if (variant == 0) {
+        const int64_t big = (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128)
+                * p.batch;
+        variant = big >= 256 ? 1 : 2;
+    }
+    switch (variant) {
+        case 1: launch_gemm_b8_v1(p, f8, stream); break;
+        case 3: launch_gemm_b8_v3(p, f8, stream); break;
+        case 4: launch_gemm_b8_v4(p, f8, stream); break;
+        case 5: launch_gemm_b8_v5(p, f8, stream); break;
+        default: launch_gemm_b8_v2(p, f8, stream); break;
+    }
+}
+#endif
+
+} // namespace qmm

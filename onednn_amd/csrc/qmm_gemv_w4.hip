@@ -1,0 +1,244 @@
+// hip:gfx950:decode_w4 -- weights-decompression matmul for small M (the decode
+// step of an LLM linear layer): 16-bit activations [M,K] x 4-bit weights [K,N]
+// with K-grouped scales and zero points, f32 accumulation
+// (semantics: src/cpu/matmul/ref_matmul.cpp:140-173 with
+// fpmath_mode apply_to_int).
+//
+// The kernel is bound by the HBM stream of the packed weights, so everything
+// is arranged around one 128-bit load per lane:
+//   * weights are prepacked (QMM_LAYOUT_MFMA_W4) in 1 KiB tiles of 16 columns
+//     x 128 k; lane 16*c + n holds, per 32-k step s, the eight nibbles of
+//     column n for k = 32*s + 8*c + 0..7, ordered so that
+//     (dword >> 4i) & 0x000F000F is the pair (2i, 2i+1);
+//   * a pair of nibbles becomes a pair of bf16 (or f16) values 128+w
+//     (1024+w) with a single v_and_or_b32 on the exponent pattern -- no
+//     integer-to-float conversions in the stream;
+//   * the 16 x 16 x 32 MFMA multiplies 16 activation rows by the 16 columns of
+//     the tile; a second MFMA against a vector of ones yields the row sums of
+//     the activations, which remove both the magic offset and the zero point
+//     when a scale group closes:
+//         out += scale[g,n] * (P - (offset + zp[g,n]) * S);
+//   * a block owns 16 columns and all of K; its waves take the k tiles round
+//     robin and issue their loads before touching the activations, which are
+//     staged once per block in LDS in MFMA operand order.
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr int GEMV_WAVES = 8;
+constexpr int GEMV_LDS_BUDGET = 128 * 1024;
+
+template <bool F16>
+QMM_D v4f mfma16(const v4u &a, const v4u &b, const v4f &c) {
+    if constexpr (F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                __builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0,
+                0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0,
+                0, 0);
+}
+
+// weights are read exactly once: keep them from displacing reusable lines
+QMM_D uint4 ld_stream(const uint8_t *ptr) {
+    const v4u v = __builtin_nontemporal_load((const v4u *)ptr);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <bool F16>
+__global__ void __launch_bounds__(GEMV_WAVES * 64)
+gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // lds: activations [KC/8 chunks][MR rows][16 bytes]; later reused for the
+    // cross-wave reduction [GEMV_WAVES][64 lanes][4 floats]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nb = blockIdx.x;
+    const int m_base = p.m0 + blockIdx.y * 16;
+    const int rows = min(16, p.M - m_base);
+    const int c = lane >> 4; // k chunk of the lane
+    const int r = lane & 15; // activation row (A operand) / column (B operand)
+    const int n = nb * 16 + r;
+
+    constexpr uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    constexpr float OFFSET = F16 ? 1024.f : 128.f;
+    constexpr uint32_t ONE2 = F16 ? 0x3C003C00u : 0x3F803F80u;
+    const v4u ones = {ONE2, ONE2, ONE2, ONE2};
+    const uint32_t sflip = p.wei_signed ? 0x88888888u : 0u;
+    const float soff = p.wei_signed ? 8.f : 0.f;
+
+    // flush granularity: the scale and zero-point groups both close there
+    int fl = p.gs;
+    if (p.gz > 0) {
+        int a = p.gs, b = p.gz;
+        while (b) {
+            const int t = a % b;
+            a = b;
+            b = t;
+        }
+        fl = a;
+    }
+
+    v4f out = {0.f, 0.f, 0.f, 0.f};
+    v4f P = {0.f, 0.f, 0.f, 0.f}, S = {0.f, 0.f, 0.f, 0.f};
+
+    const uint8_t *__restrict__ Bt
+            = p.B + ((int64_t)nb * p.kg128) * 1024 + lane * 16;
+    const int Kpad = p.kg128 * 128;
+
+    for (int kc0 = 0; kc0 < Kpad; kc0 += KC) {
+        const int kc_len = min(KC, Kpad - kc0);
+        const int tiles = kc_len / 128;
+        const int g0 = kc0 / 128;
+        // first batch of weight loads goes out before the activations
+        constexpr int UNR = 4;
+        uint4 wt[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            const int t = wave + u * GEMV_WAVES;
+            wt[u] = make_uint4(0, 0, 0, 0);
+            if (t < tiles)
+                wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
+        }
+        if (kc0 > 0) __syncthreads(); // previous chunk fully consumed
+        // stage activations: chunk kc (8 values) of row m -> (kc*MR + m)*16
+        for (int i = tid; i < (kc_len / 8) * MR; i += GEMV_WAVES * 64) {
+            const int kc = i / MR, m = i % MR;
+            const int k = kc0 + kc * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (m < rows && k < p.K)
+                v = *(const uint4 *)(p.A + (int64_t)(m_base + m) * p.lda + k);
+            *(uint4 *)(lds + (size_t)i * 16) = v;
+        }
+        __syncthreads();
+
+        for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
+            if (tb > 0) {
+#pragma unroll
+                for (int u = 0; u < UNR; u++) {
+                    const int t = tb + wave + u * GEMV_WAVES;
+                    wt[u] = make_uint4(0, 0, 0, 0);
+                    if (t < tiles)
+                        wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int t = tb + wave + u * GEMV_WAVES;
+                if (t >= tiles) break;
+                const uint32_t wd[4] = {wt[u].x ^ sflip, wt[u].y ^ sflip,
+                        wt[u].z ^ sflip, wt[u].w ^ sflip};
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const uint32_t d = wd[s];
+                    v4u b;
+                    b.x = (d & 0x000F000Fu) | MAGIC;
+                    b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
+                    b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
+                    b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
+                    v4u a = {0u, 0u, 0u, 0u};
+                    if (r < MR) {
+                        const uint4 av = *(const uint4 *)(lds
+                                + ((size_t)(t * 16 + s * 4 + c) * MR + r) * 16);
+                        a = v4u {av.x, av.y, av.z, av.w};
+                    }
+                    P = mfma16<F16>(a, b, P);
+                    S = mfma16<F16>(a, ones, S);
+                    const int k_end = kc0 + t * 128 + (s + 1) * 32;
+                    // A wave's tiles are not adjacent in k, so the partial
+                    // sums are folded at every tile end as well as where a
+                    // scale / zero-point group closes inside a tile (folding
+                    // early is exact in structure: both factors are constant
+                    // over the folded range).
+                    if (s == 3 || k_end % fl == 0) {
+                        // the range just folded contains k_end - 1
+                        const int kq = min(k_end, p.K) - 1;
+                        float sc = 1.f, zp = 0.f;
+                        if (n < p.N) {
+                            if (p.scales)
+                                sc = load_float(p.scale_dt, p.scales,
+                                        p.scale_per_n
+                                                ? (int64_t)(kq / p.gs) * p.N + n
+                                                : (int64_t)(kq / p.gs));
+                            if (p.zps)
+                                zp = (float)load_int(p.zp_dt, p.zps,
+                                        p.gz > 0 ? (p.zp_per_n
+                                                        ? (int64_t)(kq / p.gz)
+                                                                        * p.N
+                                                                + n
+                                                        : (int64_t)(kq / p.gz))
+                                                 : (p.zp_per_n ? (int64_t)n
+                                                               : 0));
+                        }
+                        const float off = OFFSET + soff + zp;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            out[j] = __builtin_fmaf(
+                                    sc, P[j] - off * S[j], out[j]);
+                            P[j] = 0.f;
+                            S[j] = 0.f;
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- reduce the waves' partial sums and finish ----
+    __syncthreads();
+    float *red = (float *)lds;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        red[(wave * 64 + lane) * 4 + j] = out[j];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float v = 0.f;
+            for (int w = 0; w < GEMV_WAVES; w++)
+                v += red[(w * 64 + lane) * 4 + j];
+            // MFMA output: register j of lane l is row 4*(l/16)+j, column l%16
+            const int m = m_base + 4 * c + j;
+            if (m < p.M && n < p.N && 4 * c + j < rows)
+                epilogue_apply_store(p.ep, v, 0, m, n);
+        }
+    }
+}
+
+void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
+    if (p.M <= 0 || p.N <= 0) return;
+    const int rows = p.M < 16 ? p.M : 16;
+    int MR = 1;
+    while (MR < rows) MR *= 2;
+    const int Kpad = p.kg128 * 128;
+    int KC = GEMV_LDS_BUDGET / (2 * MR);
+    KC = KC / 128 * 128;
+    if (KC > Kpad) KC = Kpad;
+    size_t lds = (size_t)KC * 2 * MR;
+    const size_t red = (size_t)GEMV_WAVES * 64 * 4 * sizeof(float);
+    if (lds < red) lds = red;
+    dim3 grid(p.nb16, (p.M + 15) / 16);
+    auto launch = [&](auto kern) {
+        static bool attr_done = false;
+        if (!attr_done) {
+            (void)hipFuncSetAttribute((const void *)kern,
+                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                    GEMV_LDS_BUDGET);
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, p,
+                MR, KC);
+    };
+    if (p.act_f16)
+        launch(gemv_w4_kernel<true>);
+    else
+        launch(gemv_w4_kernel<false>);
+}
+
+} // namespace qmm

@@ -1,0 +1,190 @@
+// Weights prepacking: plain strided tensors -> the MFMA operand layouts
+// (QMM_LAYOUT_MFMA_B8 with s32 column sums, QMM_LAYOUT_MFMA_W4) and back.
+// This is the reorder a user runs once per weights tensor after asking the
+// matmul primitive descriptor for its weights layout through format_tag any
+// (the role of src/cpu/x64/matmul/brgemm_matmul_reorders.cpp:29-53 in the
+// reference). Values are copied bit for bit; padding is zero.
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+
+struct pack_params_t {
+    const uint8_t *src;
+    uint8_t *dst;
+    int64_t batch, K, N;
+    int64_t sb, sk, sn; // plain side strides, elements
+    int32_t dt;
+    int32_t pad_;
+};
+
+// one thread per 16-byte chunk of the packed tensor
+__global__ void __launch_bounds__(256)
+pack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
+    const int64_t chunks = p.batch * g.batch_bytes / 16;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks;
+            c += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t per_b = g.batch_bytes / 16;
+        const int64_t b = c / per_b, cb = c % per_b;
+        const int lane = (int)(cb % 64);
+        const int64_t frag = cb / 64;
+        const int64_t nb = frag / g.kb32, kb = frag % g.kb32;
+        const int64_t n = nb * 32 + (lane & 31);
+        const int64_t k0 = kb * 32 + (lane >> 5) * 16;
+        uint32_t w[4] = {0, 0, 0, 0};
+        if (n < p.N) {
+            const uint8_t *s = p.src + b * p.sb + n * p.sn;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t k = k0 + i;
+                const uint32_t v = k < p.K ? s[k * p.sk] : 0u;
+                w[i / 4] |= v << (8 * (i % 4));
+            }
+        }
+        *(uint4 *)(p.dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// column sums of the (signed or unsigned) 8-bit weights, one thread per column
+__global__ void __launch_bounds__(256)
+colsum_kernel(const pack_params_t p, const b8_geom_t g) {
+    const int64_t total = p.batch * g.Npad;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t b = i / g.Npad, n = i % g.Npad;
+        int32_t acc = 0;
+        if (n < p.N) {
+            const uint8_t *s = p.src + b * p.sb + n * p.sn;
+            for (int64_t k = 0; k < p.K; k++) {
+                const uint8_t v = s[k * p.sk];
+                acc += p.dt == dt_s8 ? (int32_t)(int8_t)v : (int32_t)v;
+            }
+        }
+        ((int32_t *)(p.dst + g.colsum_off))[i] = acc;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+unpack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
+    // p.src: packed, p.dst: plain
+    const int64_t total = p.batch * p.K * p.N;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t n = i % p.N, k = (i / p.N) % p.K, b = i / (p.N * p.K);
+        p.dst[b * p.sb + k * p.sk + n * p.sn]
+                = p.src[b * g.batch_bytes + b8_offset(g, k, n)];
+    }
+}
+
+// one thread per packed dword (8 nibbles)
+__global__ void __launch_bounds__(256)
+pack_w4_kernel(const pack_params_t p, const w4_geom_t g) {
+    const int64_t dwords = p.batch * g.batch_bytes / 4;
+    for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < dwords;
+            d += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t per_b = g.batch_bytes / 4;
+        const int64_t b = d / per_b, db = d % per_b;
+        const int s = (int)(db % 4);
+        const int lane = (int)((db / 4) % 64);
+        const int64_t tile = db / 256;
+        const int64_t nbk = tile / g.kg128, kg = tile % g.kg128;
+        const int64_t n = nbk * 16 + (lane & 15);
+        const int64_t kbase = kg * 128 + 32 * s + 8 * (lane >> 4);
+        uint32_t w = 0;
+        if (n < p.N) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int64_t k = kbase + j;
+                if (k >= p.K) continue;
+                const int64_t e = b * p.sb + k * p.sk + n * p.sn;
+                const uint32_t nib = (uint32_t)nibble_at(p.src, e);
+                const int pos = j / 2 + 4 * (j % 2);
+                w |= nib << (4 * pos);
+            }
+        }
+        ((uint32_t *)p.dst)[d] = w;
+    }
+}
+
+// one thread per destination byte: the two nibbles are neighbours along the
+// plain tensor's stride-1 dim (n for ab, k for ba)
+__global__ void __launch_bounds__(256)
+unpack_w4_kernel(const pack_params_t p, const w4_geom_t g) {
+    const bool n_inner = p.sn == 1;
+    const int64_t total = p.batch * p.K * p.N / 2;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        uint8_t out = 0;
+        int64_t e0 = 0;
+        for (int h = 0; h < 2; h++) {
+            const int64_t l = 2 * i + h;
+            int64_t b, k, n;
+            if (n_inner) {
+                n = l % p.N;
+                k = (l / p.N) % p.K;
+                b = l / (p.N * p.K);
+            } else {
+                k = l % p.K;
+                n = (l / p.K) % p.N;
+                b = l / (p.N * p.K);
+            }
+            const int64_t e = b * p.sb + k * p.sk + n * p.sn;
+            if (h == 0) e0 = e;
+            const int64_t ni = b * g.batch_bytes * 2 + w4_nibble_index(g, k, n);
+            out |= (uint8_t)(nibble_at(p.src, ni) << (4 * (int)(e & 1)));
+        }
+        p.dst[e0 >> 1] = out;
+    }
+}
+
+static unsigned grid_for(int64_t n) {
+    int64_t b = (n + 255) / 256;
+    if (b < 1) b = 1;
+    if (b > 262144) b = 262144;
+    return (unsigned)b;
+}
+
+void launch_pack_b8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        bool with_colsum, hipStream_t stream) {
+    const b8_geom_t g = b8_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(pack_b8_kernel, dim3(grid_for(batch * g.batch_bytes / 16)),
+            dim3(256), 0, stream, p, g);
+    if (with_colsum)
+        hipLaunchKernelGGL(colsum_kernel, dim3(grid_for(batch * g.Npad)),
+                dim3(256), 0, stream, p, g);
+}
+
+void launch_unpack_b8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const b8_geom_t g = b8_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(unpack_b8_kernel, dim3(grid_for(batch * K * N)),
+            dim3(256), 0, stream, p, g);
+}
+
+void launch_pack_w4(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4_geom_t g = w4_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(pack_w4_kernel, dim3(grid_for(batch * g.batch_bytes / 4)),
+            dim3(256), 0, stream, p, g);
+}
+
+void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4_geom_t g = w4_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(unpack_w4_kernel, dim3(grid_for(batch * K * N / 2)),
+            dim3(256), 0, stream, p, g);
+}
+
+} // namespace qmm

@@ -1,0 +1,153 @@
+// Host/device parameter blocks of the kernels and the plan object behind
+// qmm_matmul_plan_create(). Shared by the .hip kernels and the host dispatch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qmm_device.hpp"
+#include "qmm_hip.h"
+
+namespace qmm {
+
+// A scales / zero-points buffer as the generic kernels index it: dense
+// row-major over the masked dims, last two dims divided by the groups
+// (src/cpu/matmul/matmul_utils.hpp:156-196). strides[d] == 0 where the mask
+// bit is clear.
+struct generic_quant_t {
+    int32_t indexed; // 0: single element at offset 0
+    int32_t pad_;
+    int64_t g0, g1;
+    int64_t strides[QMM_MAX_NDIMS];
+    int64_t nelems;
+};
+
+struct generic_params_t {
+    qmm_matmul_desc_t desc;
+    int64_t M, N, K, batch;
+    int32_t src_mask, wei_mask, bia_mask; // dims equal to dst's
+    int32_t int_path, decompress, has_sum, sum_dt, dst_zp_mult;
+    int64_t ngroups_k, group_k;
+    int64_t wei_scale_stride_n;
+    generic_quant_t q_src_scale, q_wei_scale, q_src_zp, q_wei_zp;
+};
+
+struct generic_reorder_params_t {
+    qmm_reorder_desc_t desc;
+    int64_t nelems;
+    int32_t pair_dim; // 4-bit dst: the stride-1 dim
+    int32_t pad_;
+    generic_quant_t q_src_scale, q_dst_scale, q_src_zp;
+};
+
+// ---- packed layouts -------------------------------------------------------
+// QMM_LAYOUT_MFMA_B8: byte offset of element (k, n) inside one batch slice.
+struct b8_geom_t {
+    int64_t K, N, Kpad, Npad, kb32, nb32;
+    int64_t batch_bytes; // data bytes per batch slice
+    int64_t colsum_off; // byte offset of the s32 column sums (all batches)
+    int64_t total_bytes;
+};
+QMM_HD int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
+QMM_HD b8_geom_t b8_geom(int64_t batch, int64_t K, int64_t N) {
+    b8_geom_t g;
+    g.K = K;
+    g.N = N;
+    g.Kpad = round_up(K, 128);
+    g.Npad = round_up(N, 32);
+    g.kb32 = g.Kpad / 32;
+    g.nb32 = g.Npad / 32;
+    g.batch_bytes = g.Kpad * g.Npad;
+    g.colsum_off = round_up(batch * g.batch_bytes, 256);
+    g.total_bytes = g.colsum_off + batch * g.Npad * 4;
+    return g;
+}
+QMM_HD int64_t b8_offset(const b8_geom_t &g, int64_t k, int64_t n) {
+    const int64_t lane = 32 * ((k % 32) / 16) + (n % 32);
+    return (((n / 32) * g.kb32 + k / 32) * 64 + lane) * 16 + (k % 16);
+}
+
+// QMM_LAYOUT_MFMA_W4: nibble index of element (k, n) inside one batch slice.
+struct w4_geom_t {
+    int64_t K, N, Kpad, Npad, kg128, nb16;
+    int64_t batch_bytes, total_bytes;
+};
+QMM_HD w4_geom_t w4_geom(int64_t batch, int64_t K, int64_t N) {
+    w4_geom_t g;
+    g.K = K;
+    g.N = N;
+    g.Kpad = round_up(K, 128);
+    g.Npad = round_up(N, 16);
+    g.kg128 = g.Kpad / 128;
+    g.nb16 = g.Npad / 16;
+    g.batch_bytes = g.Kpad * g.Npad / 2;
+    g.total_bytes = batch * g.batch_bytes;
+    return g;
+}
+// One 16-column x 128-k tile is 1024 bytes = 64 lanes x 4 dwords. Lane
+// 16*c + n%16 holds, in dword s, the eight values k = 128*g + 32*s + 8*c + j;
+// value j sits in the nibble at bit 4*p with p = j/2 + 4*(j%2), so that
+// (dword >> 4*i) & 0x000F000F yields the pair (j = 2i, j = 2i+1) in the low
+// and high half-words.
+QMM_HD int64_t w4_nibble_index(const w4_geom_t &g, int64_t k, int64_t n) {
+    const int64_t tile = (n / 16) * g.kg128 + k / 128;
+    const int64_t kk = k % 128;
+    const int64_t s = kk / 32, c = (kk % 32) / 8, j = kk % 8;
+    const int64_t lane = 16 * c + (n % 16);
+    const int64_t p = j / 2 + 4 * (j % 2);
+    return ((tile * 64 + lane) * 4 + s) * 8 + p;
+}
+
+// ---- MFMA GEMM (int8 / fp8) -----------------------------------------------
+struct gemm_params_t {
+    const uint8_t *A; // src, rows K-contiguous
+    int64_t lda, a_sb; // bytes
+    const uint8_t *B; // QMM_LAYOUT_MFMA_B8
+    int64_t b_sb; // bytes between batch slices (0: broadcast)
+    const int32_t *colsum; // [batch][Npad] or nullptr
+    int64_t colsum_sb; // elements
+    const void *src_zp; // single value or nullptr
+    int32_t src_zp_dt;
+    int32_t a_is_u8;
+    int32_t M, N, K, batch;
+    int32_t kb32; // K blocks of 32 in the packed weights
+    int32_t nb32;
+    int32_t tiles_m, tiles_n;
+    int32_t pad_;
+    epilogue_t ep;
+};
+
+// ---- decode kernel (4-bit / 8-bit weights, 16-bit activations) -------------
+struct gemv_params_t {
+    const uint16_t *A; // activations [M][K], bf16 or f16
+    int64_t lda; // elements
+    const uint8_t *B; // QMM_LAYOUT_MFMA_W4
+    const void *scales; // [K/gs][N]
+    const void *zps; // [K/gz][N] or single or nullptr
+    int32_t scale_dt, zp_dt;
+    int32_t gs, gz; // K group sizes (multiples of 32); gz == 0: single zp
+    int32_t scale_per_n, zp_per_n; // 0: broadcast over n
+    int32_t M, N, K;
+    int32_t kg128, nb16;
+    int32_t wei_signed; // s4 weights
+    int32_t act_f16; // activations are f16 (else bf16)
+    int32_t m0; // first row handled by this launch
+    epilogue_t ep;
+};
+
+enum impl_id_t : int {
+    impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
+    impl_gemv_w4 = 1, // decode: 4-bit weights, M small
+    impl_generic = 2,
+    impl_count = 3
+};
+
+} // namespace qmm
+
+struct qmm_plan {
+    int impl;
+    qmm::generic_params_t host; // generic parameters (always filled)
+    qmm::generic_params_t *dev; // device copy, used by the generic kernel
+    qmm_matmul_desc_t desc;
+    size_t scratch_bytes;
+};

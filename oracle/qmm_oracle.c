@@ -587,16 +587,23 @@ static void mm_ctx_init(mm_ctx_t *c, const orc_matmul_t *p) {
      * integer accumulation every other implementation of the reference
      * performs (gemm_x8s8s32x_matmul.cpp:165-193, brgemm). */
     int64_t K = c->K, ng = 1, t;
-    const int64_t dflt = p->k_group_mode == ORC_KGROUP_WHOLE ? (K > 0 ? K : 1) : 1;
     if (K > 0) {
-        t = K / (sz->set && sz->g1 > 0 ? sz->g1 : dflt);
+        const int whole = p->k_group_mode == ORC_KGROUP_WHOLE;
+        const int src_kbit = 1 << (nd - 1), wei_kbit = 1 << (nd - 2);
+        /* WHOLE: an entry without groups still varies per k when its mask
+         * covers the K dim (one value per k: group of 1) */
+#define KGROUP(q, g, kbit) \
+    ((q)->set && (g) > 0 ? (g) \
+                         : (whole && !((q)->set && ((q)->mask & (kbit))) ? K : 1))
+        t = K / KGROUP(sz, sz->g1, src_kbit);
         if (t > ng) ng = t;
-        t = K / (wz->set && wz->g0 > 0 ? wz->g0 : dflt);
+        t = K / KGROUP(wz, wz->g0, wei_kbit);
         if (t > ng) ng = t;
-        t = K / (ss->set && ss->g1 > 0 ? ss->g1 : dflt);
+        t = K / KGROUP(ss, ss->g1, src_kbit);
         if (t > ng) ng = t;
-        t = K / (ws->set && ws->g0 > 0 ? ws->g0 : dflt);
+        t = K / KGROUP(ws, ws->g0, wei_kbit);
         if (t > ng) ng = t;
+#undef KGROUP
     }
     c->ngroups_k = ng;
     c->group_k = K > 0 ? K / ng : 0;
