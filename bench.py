@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matmul path on one MI355X.
+
+A "step" is one execute() of the primitive over one batch of synthetic input
+already resident in HBM. The headline workload is BASELINE.json's config 2
+(W8A8 LLM linear layer: s8 [4096,4096] x s8 [4096,14336], per-token src scales,
+per-N weights scales, swish, bf16 dst); the decode GEMV (config 3) and the fp8
+GEMM (config 5) are measured in the same run and reported as extra objects of
+the same JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_INT8 = 5000.0  # TOP/s, dense MFMA int8 (published MI355X figure)
+PEAK_FP8 = 5000.0  # TFLOP/s, dense MFMA fp8
+PEAK_HBM = 8000.0  # GB/s
+
+
+def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
+    """Config 2: returns (problem tensors on host, attr builder)."""
+    r = np.random.default_rng(seed)
+    src = np.clip(np.rint(r.standard_normal((M, K)) * 32), -127, 127).astype(np.int8)
+    wei = r.integers(-127, 128, (K, N), dtype=np.int8)
+    ss = r.uniform(0.005, 0.05, M).astype(np.float32)
+    ws = r.uniform(0.0005, 0.005, N).astype(np.float32)
+    return src, wei, ss, ws
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=["c2"])
+    ap.add_argument("--variant", type=int, default=0, help="mfma_b8 tile configuration (0 = heuristic)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the decode / fp8 side measurements")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=192, help="rows of config 2 timed on the CPU oracle")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the path shards "
+              "along N without any exchange, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import onednn_amd as dnnl
+    from onednn_amd import _capi, hiprt, memory
+    from qmm_harness import T, assert_bf16_within_1ulp
+    dt = memory.data_type
+    tag = memory.format_tag
+    A = dnnl
+
+    eng = dnnl.engine(dnnl.engine.kind.gpu, 0)
+    strm = dnnl.stream(eng)
+    hs = C_stream(strm)
+    _capi.lib().qmm_set_gemm_variant(args.variant)
+
+    # ------------------------------------------------------------------ c2
+    M, K, N = 4096, 4096, 14336
+    src, wei, ss, ws = build_c2(dnnl, dt, T)
+    attr = A.primitive_attr()
+    attr.set_scales(A.DNNL_ARG_SRC, 3, [1, K], dt.f32)
+    attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 2)
+    po = A.post_ops()
+    po.append_eltwise(A.algorithm.eltwise_swish, 1.0, 0.0)
+    attr.set_post_ops(po)
+    pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.s8, T("ab")), memory.desc([K, N], dt.s8, tag.any),
+                                 memory.desc([M, N], dt.bf16, T("ab")), attr=attr)
+    prim = A.matmul(pd)
+    m_src = memory(pd.src_desc(), eng).write(src)
+    m_plain = memory(memory.desc([K, N], dt.s8, T("ab")), eng).write(wei)
+    m_wei = memory(pd.weights_desc(), eng)
+    A.reorder(m_plain, m_wei).execute(strm, m_plain, m_wei)  # prepack, once, untimed
+    m_dst = memory(pd.dst_desc(), eng)
+    m_ss = memory(memory.desc([M], dt.f32, T("a")), eng).write(ss)
+    m_ws = memory(memory.desc([N], dt.f32, T("a")), eng).write(ws)
+    exec_args = {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: m_wei, A.DNNL_ARG_DST: m_dst,
+                 A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: m_ss, A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: m_ws}
+    strm.wait()
+    del m_plain
+
+    for _ in range(args.warmup):
+        prim.execute(strm, exec_args)
+    strm.wait()
+    hiprt.device_synchronize()
+    e0, e1 = hiprt.Event(), hiprt.Event()
+    t0 = time.perf_counter()
+    e0.record(hs)
+    for _ in range(args.steps):
+        prim.execute(strm, exec_args)
+    e1.record(hs)
+    strm.wait()
+    hiprt.device_synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = e1.elapsed_ms(e0) / args.steps
+    ops = 2.0 * M * K * N
+    tops = ops / (wall_ms * 1e-3) / 1e12
+    kern_tops = ops / (ev_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "int8/fp8 matmul TOPS + % MFMA peak; int4-weight GEMV HBM GB/s, 1 MI355X",
+        "value": round(tops, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "s8", "data": "synthetic",
+        "config": {"workload": "config 2: W8A8 linear, s8[4096,4096] x s8[4096,14336] -> bf16, per-token src scales, "
+                               "per-N weights scales, swish; weights prepacked via format_tag any",
+                   "impl": pd.impl_info_str(), "tile_variant": args.variant},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TFLOP/s",
+                     "frac": round(kern_tops / PEAK_INT8, 4), "traffic": None,
+                     "kernel": "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
+                     "algorithmic_ops_per_launch": ops},
+    }
+
+    # ------------------------------------------------------- CPU baseline
+    if not args.no_cpu_baseline:
+        import oracle as O
+        rows = min(args.cpu_rows, M)
+        sel = np.linspace(0, M - 1, rows).astype(np.int64)
+        s_sub = np.ascontiguousarray(src[sel])
+        d_sub = np.zeros((rows, N), np.uint16)
+        ncores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        t = time.perf_counter()
+        O.matmul(O.Tensor(O.S8, [rows, K], s_sub), O.Tensor(O.S8, [K, N], wei), O.Tensor(O.BF16, [rows, N], d_sub),
+                 scales={O.Q_SRC: O.Quant(3, O.F32, np.ascontiguousarray(ss[sel]), (1, K)), O.Q_WEI: O.Quant(2, O.F32, ws)},
+                 post_ops=[{"kind": "eltwise", "alg": A.algorithm.eltwise_swish, "alpha": 1.0}], nthreads=ncores)
+        cpu_s = time.perf_counter() - t
+        out["cpu_baseline"] = {"value": round(2.0 * rows * K * N / cpu_s / 1e12, 5), "unit": "TOP/s", "cores": ncores,
+                               "kind": "port",
+                               "sample": "%d of the 4096 rows of config 2 (evenly spaced), full K and N, "
+                                         "scalar C oracle with OpenMP, %.1f s" % (rows, cpu_s)}
+        # the same rows double as a parity check of the timed kernel's output
+        got = m_dst.read(np.uint16, (M, N))[sel]
+        frac = assert_bf16_within_1ulp(got, d_sub, "bench parity sample")
+        out["parity_sample"] = {"rows": rows, "max_bf16_ulp": 1, "frac_off_by_one": round(frac, 6)}
+
+    if not args.no_extras:
+        out["decode_gemv"] = bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt)
+        out["fp8_gemm"] = bench_fp8(A, memory, dt, tag, T, eng, strm, hs, hiprt)
+    print(json.dumps(out))
+
+
+def C_stream(strm):
+    import ctypes as C
+    from onednn_amd import _capi
+    p = C.c_void_p()
+    _capi.call("dnnl_hip_interop_stream_get_stream", strm._h, C.byref(p))
+    return p.value
+
+
+def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20):
+    """Config 3: bf16 x u4 GEMV, G=128 f16 scales + u4 zero points. The 8.7 MB
+    of one weights set would sit in the last-level cache, so `sets` distinct
+    copies are cycled; the launches are replayed from a HIP graph so that the
+    host does not pace them."""
+    import oracle as O
+    K = N = 4096
+    G = 128
+    r = np.random.default_rng(3)
+    res = {}
+    w = O.pack4(r.integers(0, 16, (K, N)))
+    sc = O.from_f32(O.F16, r.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
+    zp = O.pack4(r.integers(6, 10, (K // G, N)))
+    for M in (1, 16):
+        attr = A.primitive_attr()
+        attr.set_fpmath_mode(A.fpmath_mode.bf16, True)
+        attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
+        attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.u4)
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.bf16, T("ab")), memory.desc([K, N], dt.u4, tag.any),
+                                     memory.desc([M, N], dt.bf16, T("ab")), attr=attr)
+        prim = A.matmul(pd)
+        a = O.from_f32(O.BF16, r.standard_normal((M, K)).astype(np.float32))
+        m_src = memory(pd.src_desc(), eng).write(a)
+        m_dst = memory(pd.dst_desc(), eng)
+        plain = memory(memory.desc([K, N], dt.u4, T("ab")), eng).write(w)
+        first = memory(pd.weights_desc(), eng)
+        A.reorder(plain, first).execute(strm, plain, first)
+        strm.wait()
+        wsets, ssets, zsets = [first], [], []
+        nb = pd.weights_desc().get_size()
+        for i in range(sets):
+            if i:
+                m = memory(pd.weights_desc(), eng)
+                hiprt.memcpy_dtod(m.get_data_handle(), first.get_data_handle(), nb)
+                wsets.append(m)
+            ssets.append(memory(memory.desc([sc.nbytes], dt.u8, T("a")), eng).write(sc))
+            zsets.append(memory(memory.desc([zp.nbytes], dt.u8, T("a")), eng).write(zp))
+
+        def one(i):
+            prim.execute(strm, {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: wsets[i], A.DNNL_ARG_DST: m_dst,
+                                A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: ssets[i],
+                                A.DNNL_ARG_ATTR_ZERO_POINTS | A.DNNL_ARG_WEIGHTS: zsets[i]})
+
+        for i in range(sets):
+            one(i)
+        strm.wait()
+        graph = hiprt.Graph(hs, lambda: [one(i) for i in range(sets)])
+        graph.launch()
+        strm.wait()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(hs)
+        for _ in range(reps):
+            graph.launch()
+        e1.record(hs)
+        strm.wait()
+        us = e1.elapsed_ms(e0) * 1e3 / (reps * sets)
+        nbytes = K * N // 2 + sc.nbytes + zp.nbytes + M * K * 2 + M * N * 2
+        res["M%d" % M] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
+                          "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
+                          "impl": pd.impl_info_str(), "weight_sets": sets, "timing": "hip graph of %d launches x %d" % (sets, reps)}
+    return res
+
+
+def bench_fp8(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=10):
+    """Config 5: f8_e4m3 8192^3, scales 0.5 / 0.25, sum post-op, bf16 dst."""
+    import oracle as O
+    n = 8192
+    r = np.random.default_rng(5)
+    # e4m3 codes drawn directly: clip(N(0,1)*4) quantised with the reference rounding on a 1M sample, tiled
+    base = O.from_f32(O.F8_E4M3, np.clip(r.standard_normal(1 << 20) * 4, -448, 448).astype(np.float32))
+    a = np.resize(base, n * n)
+    b = np.resize(np.roll(base, 12345), n * n)
+    attr = A.primitive_attr()
+    attr.set_scales_mask(A.DNNL_ARG_SRC, 0)
+    attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 0)
+    po = A.post_ops()
+    po.append_sum(1.0)
+    attr.set_post_ops(po)
+    pd = A.matmul.primitive_desc(eng, memory.desc([n, n], dt.f8_e4m3, T("ab")), memory.desc([n, n], dt.f8_e4m3, tag.any),
+                                 memory.desc([n, n], dt.bf16, T("ab")), attr=attr)
+    prim = A.matmul(pd)
+    m_src = memory(pd.src_desc(), eng).write(a)
+    plain = memory(memory.desc([n, n], dt.f8_e4m3, T("ab")), eng).write(b)
+    m_wei = memory(pd.weights_desc(), eng)
+    A.reorder(plain, m_wei).execute(strm, plain, m_wei)
+    strm.wait()
+    del plain
+    m_dst = memory(pd.dst_desc(), eng).write(O.from_f32(O.BF16, np.resize(r.standard_normal(1 << 20).astype(np.float32), n * n)))
+    m_s = memory(memory.desc([1], dt.f32, T("a")), eng).write(np.array([0.5], np.float32))
+    m_w = memory(memory.desc([1], dt.f32, T("a")), eng).write(np.array([0.25], np.float32))
+    ex = {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: m_wei, A.DNNL_ARG_DST: m_dst,
+          A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: m_s, A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: m_w}
+    for _ in range(3):
+        prim.execute(strm, ex)
+    strm.wait()
+    e0, e1 = hiprt.Event(), hiprt.Event()
+    e0.record(hs)
+    for _ in range(steps):
+        prim.execute(strm, ex)
+    e1.record(hs)
+    strm.wait()
+    ms = e1.elapsed_ms(e0) / steps
+    tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    return {"ms_per_launch": round(ms, 4), "TFLOPs": round(tf, 1), "frac_of_fp8_peak": round(tf / PEAK_FP8, 4),
+            "impl": pd.impl_info_str()}
+
+
+if __name__ == "__main__":
+    main()

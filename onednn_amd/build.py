@@ -21,7 +21,7 @@ OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libdnnl_amd.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wno-inline-asm",
           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
           "-Wall", "-Wno-unused-function", "-Wno-pass-failed"]
 DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",

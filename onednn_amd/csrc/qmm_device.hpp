@@ -339,7 +339,22 @@ struct epilogue_t {
     int32_t npo;
     const int32_t *dst_zp; // s32; index dst_zp_sn * n
     int64_t dst_zp_sn;
+    int32_t fast; // EP_FAST_* shape recognised by the host, 0: interpret
+    int32_t pad_;
     ep_postop_t po[EP_MAX_PO];
+};
+
+// Epilogue shapes the tiled GEMM handles with straight-line code instead of
+// the post-op interpreter: f32 scales (per-tensor / per-m source, per-tensor /
+// per-n weights), no bias, no dst scale / zero point, a dense bf16 or f32 dst
+// row and at most one post-op of the kinds below.
+enum : int {
+    EP_FAST_NONE = 0,
+    EP_FAST_PLAIN = 1, // no post-op
+    EP_FAST_RELU = 2, // eltwise relu(alpha)
+    EP_FAST_SWISH = 3, // eltwise swish(alpha)
+    EP_FAST_ADD = 4, // binary add with an f32 operand, dense along n
+    EP_FAST_SUM = 5 // sum with zero point 0 read in dst's own type
 };
 
 QMM_D float ep_load(const ep_tensor_t &t, int64_t b, int64_t m, int64_t n) {
@@ -475,6 +490,89 @@ QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
 #pragma unroll
     for (int i = 0; i < 4; i++)
         if (i < nvalid) store_float(dt, d[i], dst, dst_off + i * ep.dst.sn);
+}
+
+// Straight-line epilogue for the EP_FAST_* shapes: d[i] is (float)acc of four
+// neighbouring columns n..n+3 of row m. ss / ws are the source and weights
+// scales (1.0 when absent is NOT substituted: the flags say whether to
+// multiply, so the operation sequence equals the reference's). Everything but
+// swish is operation-for-operation the interpreter's arithmetic; swish uses
+// the hardware exp2 / rcp (relative error ~4e-7, far inside the 1e-5 / 1 bf16
+// ulp bars that any exp implementation other than the reference's libm needs).
+QMM_D void epilogue_fast4(const epilogue_t &ep, float (&d)[4], bool has_ss,
+        float ss, bool has_ws, const float (&ws)[4], int64_t b, int64_t m,
+        int64_t n, int nvalid) {
+    if (has_ss) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= ss;
+    }
+    if (has_ws) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= ws[i];
+    }
+    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n;
+    const int fast = ep.fast;
+    if (fast == EP_FAST_RELU) {
+        const float alpha = ep.po[0].alpha;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = d[i] > 0 ? d[i] : d[i] * alpha;
+    } else if (fast == EP_FAST_SWISH) {
+        const float na = -ep.po[0].alpha * 1.44269504088896340736f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float e = __builtin_amdgcn_exp2f(d[i] * na);
+            d[i] = d[i] * __builtin_amdgcn_rcpf(1.0f + e);
+        }
+    } else if (fast == EP_FAST_ADD) {
+        const float *q = (const float *)ep.po[0].t.ptr + b * ep.po[0].t.sb
+                + m * ep.po[0].t.sm + n;
+        if (nvalid == 4 && (((uintptr_t)q) & 15) == 0) {
+            const float4 y = *(const float4 *)q;
+            d[0] += y.x;
+            d[1] += y.y;
+            d[2] += y.z;
+            d[3] += y.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid) d[i] += q[i];
+        }
+    } else if (fast == EP_FAST_SUM) {
+        const float sc = ep.po[0].scale;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < nvalid) {
+                const float old = load_float(ep.dst.dt, ep.dst.ptr, dst_off + i);
+                d[i] += sc * (old - 0.f);
+            }
+    }
+    if (ep.dst.dt == dt_bf16) {
+        uint16_t *q = (uint16_t *)ep.dst.ptr + dst_off;
+        uint16_t h[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            h[i] = f32_to_bf16(d[i]);
+        if (nvalid == 4 && (((uintptr_t)q) & 7) == 0) {
+            *(uint2 *)q = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16),
+                    (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid) q[i] = h[i];
+        }
+    } else { // f32
+        float *q = (float *)ep.dst.ptr + dst_off;
+        if (nvalid == 4 && (((uintptr_t)q) & 15) == 0) {
+            *(float4 *)q = make_float4(d[0], d[1], d[2], d[3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (i < nvalid) q[i] = d[i];
+        }
+    }
 }
 
 } // namespace qmm

@@ -299,6 +299,30 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
             return false;
         }
     }
+    // straight-line shapes (see EP_FAST_* in qmm_device.hpp)
+    ep.fast = EP_FAST_NONE;
+    const bool scales_f32 = (!ep.src_scale.ptr || ep.src_scale.dt == dt_f32)
+            && (!ep.wei_scale.ptr || ep.wei_scale.dt == dt_f32);
+    if (scales_f32 && !ep.bias.ptr && !ep.dst_scale && !ep.dst_zp
+            && ep.dst.sn == 1 && (ep.dst.dt == dt_bf16 || ep.dst.dt == dt_f32)
+            && ep.npo <= 1) {
+        if (ep.npo == 0) {
+            ep.fast = EP_FAST_PLAIN;
+        } else {
+            const ep_postop_t &o = ep.po[0];
+            if (o.kind == pk_eltwise && o.scale == 1.f && o.alg == alg_relu)
+                ep.fast = EP_FAST_RELU;
+            else if (o.kind == pk_eltwise && o.scale == 1.f
+                    && o.alg == alg_swish)
+                ep.fast = EP_FAST_SWISH;
+            else if (o.kind == pk_binary && o.alg == alg_bin_add
+                    && o.t.dt == dt_f32 && o.t.sn == 1)
+                ep.fast = EP_FAST_ADD;
+            else if (o.kind == pk_sum && o.zero_point == 0
+                    && o.t.dt == ep.dst.dt)
+                ep.fast = EP_FAST_SUM;
+        }
+    }
     return true;
 }
 

@@ -67,8 +67,31 @@ QMM_D int a_swz(int row, int q) {
     return q ^ ((row / ROWS_PER_256B) % CH);
 }
 
-template <int BM, int BN, int BK, int WGM, int WGN, bool F8>
-__global__ void __launch_bounds__(WGM *WGN * 64, (BM * BN <= 256 * 128) ? 2 : 1)
+// One lane's 16 bytes from global memory straight into LDS: the wave's 64 lanes
+// fill the 1 KiB at `lds_addr` (wave-uniform byte address) in lane order.
+// Written as assembly on purpose: the compiler orders every later LDS read
+// after a direct-to-LDS load it knows about with a full vmcnt(0), which would
+// serialise the pipeline below; completion is tracked by hand with
+// wait_vmcnt() + the block barrier.
+QMM_D void load_to_lds16(const void *gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+// s_waitcnt immediate for "at most n vector-memory operations outstanding"
+// (gfx9 encoding: vmcnt in bits 3:0 and 15:14; expcnt / lgkmcnt left open)
+constexpr int vmcnt_imm(int n) {
+    return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8);
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, bool F8,
+        bool U8A>
+__global__ void __launch_bounds__(WGM *WGN * 64,
+        (BM / WGM) * (BN / WGN) <= 128 * 64 ? 2 : 1)
 gemm_b8_kernel(const gemm_params_t p) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -76,18 +99,20 @@ gemm_b8_kernel(const gemm_params_t p) {
     constexpr int KF = BK / 32; // k32 fragments per tile
     constexpr int CH = BK / 16; // 16-byte chunks per A row
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     constexpr int A_CH = A_BYTES / 16 / NT, B_CH = B_BYTES / 16 / NT;
+    constexpr int LOADS = A_CH + B_CH; // vector loads per thread and tile
     static_assert(A_CH * 16 * NT == A_BYTES && B_CH * 16 * NT == B_BYTES, "");
     static_assert(!F8 || (KF % 2 == 0), "fp8 MFMA consumes 64 k per step");
+    static_assert(STAGES >= 2 && STAGES <= 4, "");
     typedef typename acc_traits<F8>::type acc_t;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *const As0 = lds;
-    uint8_t *const Bs0 = lds + 2 * A_BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WGN) * WM;
     const int wn0 = (wave % WGN) * WN;
 
@@ -127,61 +152,73 @@ gemm_b8_kernel(const gemm_params_t p) {
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0;
 
+    // ---- global -> LDS without registers ----
+    // A wave-wide global_load_lds_dwordx4 drops lane l's 16 bytes at
+    // M0-base + 16*l: the LDS image of one instruction is 1 KiB contiguous and
+    // any permutation has to happen on the global side. For the weights the
+    // packed layout already is the LDS image. For the source tile the image is
+    // [row][BK] with the 16-byte chunks of a row XOR-swizzled, so the lane that
+    // fills chunk position cp of row r fetches chunk cp ^ swz(r) of that row:
+    // still the same BK contiguous bytes per row, fully coalesced.
+    // Loads carry no predicate: rows past M and column blocks past the packed
+    // N re-read the last valid ones (their accumulators are never stored), k
+    // past K re-reads the row's last 16 valid bytes, which meet the zero
+    // padding of the packed weights (fp8 launches have K % BK == 0).
     const int KT = (p.K + BK - 1) / BK;
-    uint4 ra[A_CH], rb[B_CH];
+    const uint8_t *a_ptr[A_CH];
+    int a_k[A_CH];
+#pragma unroll
+    for (int j = 0; j < A_CH; j++) {
+        const int c = tid + j * NT;
+        const int row = c / CH, cp = c % CH;
+        const int gm = min(m0 + row, p.M - 1);
+        a_ptr[j] = A + (int64_t)gm * p.lda;
+        a_k[j] = a_swz<CH>(row, cp) * 16;
+    }
+    const uint8_t *b_ptr[B_CH];
+#pragma unroll
+    for (int j = 0; j < B_CH; j++) {
+        const int c = tid + j * NT;
+        const int nbl = c / (KF * 64), rem = c % (KF * 64);
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1);
+        b_ptr[j] = B + (int64_t)nb * p.kb32 * 1024 + rem * 16;
+    }
 
-    auto gload = [&](int kt) {
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    auto issue = [&](int kt) {
+        const int stage = kt % STAGES;
+        const uint32_t As = lds_base + stage * STAGE_BYTES;
+        const uint32_t Bs = As + A_BYTES;
 #pragma unroll
         for (int j = 0; j < A_CH; j++) {
-            const int c = tid + j * NT;
-            const int row = c / CH, q = c % CH;
-            const int gm = m0 + row;
-            const int gk = kt * BK + q * 16;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (gm < p.M && gk < p.K)
-                v = *(const uint4 *)(A + (int64_t)gm * p.lda + gk);
-            ra[j] = v;
+            const int gk = min(kt * BK + a_k[j], p.K - 16);
+            load_to_lds16(a_ptr[j] + gk, As + (j * NT + wave * 64) * 16);
         }
 #pragma unroll
-        for (int j = 0; j < B_CH; j++) {
-            const int c = tid + j * NT;
-            const int nbl = c / (KF * 64), rem = c % (KF * 64);
-            const int nb = n0 / 32 + nbl;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (nb < p.nb32)
-                v = *(const uint4 *)(B
-                        + ((int64_t)nb * p.kb32 + (int64_t)kt * KF) * 1024
-                        + rem * 16);
-            rb[j] = v;
-        }
-    };
-    auto lstore = [&](int stage) {
-        uint8_t *As = As0 + stage * A_BYTES;
-        uint8_t *Bs = Bs0 + stage * B_BYTES;
-#pragma unroll
-        for (int j = 0; j < A_CH; j++) {
-            const int c = tid + j * NT;
-            const int row = c / CH, q = c % CH;
-            *(uint4 *)(As + row * BK + a_swz<CH>(row, q) * 16) = ra[j];
-        }
-#pragma unroll
-        for (int j = 0; j < B_CH; j++) {
-            const int c = tid + j * NT;
-            *(uint4 *)(Bs + c * 16) = rb[j];
-        }
+        for (int j = 0; j < B_CH; j++)
+            load_to_lds16(b_ptr[j] + (int64_t)kt * (KF * 1024),
+                    Bs + (j * NT + wave * 64) * 16);
     };
 
-    gload(0);
-    lstore(0);
-    __syncthreads();
-
-    const uint32_t flip = p.a_is_u8 ? 0x80808080u : 0u;
+    // prologue: STAGES-1 tiles in flight
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; s++)
+        if (s < KT) issue(s);
 
     for (int kt = 0; kt < KT; kt++) {
-        const int stage = kt & 1;
-        if (kt + 1 < KT) gload(kt + 1);
-        const uint8_t *As = As0 + stage * A_BYTES;
-        const uint8_t *Bs = Bs0 + stage * B_BYTES;
+        // tile kt has landed once at most the loads of the younger tiles in
+        // flight remain; the barrier publishes it to the other waves and
+        // guarantees everybody is done with the stage that is refilled next
+        if (kt + STAGES - 2 < KT)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * LOADS));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        if (kt + STAGES - 1 < KT) issue(kt + STAGES - 1);
+
+        const uint8_t *As = lds + (kt % STAGES) * STAGE_BYTES;
+        const uint8_t *Bs = As + A_BYTES;
         if constexpr (!F8) {
 #pragma unroll
             for (int ki = 0; ki < KF; ki++) {
@@ -192,10 +229,12 @@ gemm_b8_kernel(const gemm_params_t p) {
                     const int q = ki * 2 + (lane >> 5);
                     uint4 v = *(const uint4 *)(As + row * BK
                             + a_swz<CH>(row, q) * 16);
-                    v.x ^= flip;
-                    v.y ^= flip;
-                    v.z ^= flip;
-                    v.w ^= flip;
+                    if constexpr (U8A) { // u8 source -> s8: flip the top bits
+                        v.x ^= 0x80808080u;
+                        v.y ^= 0x80808080u;
+                        v.z ^= 0x80808080u;
+                        v.w ^= 0x80808080u;
+                    }
                     a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
                 }
 #pragma unroll
@@ -245,9 +284,8 @@ gemm_b8_kernel(const gemm_params_t p) {
                                         0);
             }
         }
-        if (kt + 1 < KT) lstore(stage ^ 1);
-        __syncthreads();
     }
+    __syncthreads(); // LDS is reused by the epilogue
 
     // ---- zero-point compensation (integer path) ----
     int comp = 0;
@@ -274,6 +312,20 @@ gemm_b8_kernel(const gemm_params_t p) {
         }
     }
     constexpr int ROWS_PER_IT = 256 / WN; // 64 lanes x 4 columns
+    // on the way back a lane owns columns ecol..ecol+3 of every row it visits
+    const int ecol = (lane % (WN / 4)) * 4;
+    const int en = n0 + wn0 + ecol;
+    const int envalid = min(4, p.N - en);
+    const bool has_ss = p.ep.src_scale.ptr != nullptr;
+    const bool has_ws = p.ep.wei_scale.ptr != nullptr;
+    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
+    if (p.ep.fast != EP_FAST_NONE && has_ws) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < envalid)
+                ws4[i] = ((const float *)p.ep.wei_scale.ptr)[bz * p.ep.wei_scale.sb
+                        + (int64_t)(en + i) * p.ep.wei_scale.sn];
+    }
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
 #pragma unroll
@@ -293,19 +345,26 @@ gemm_b8_kernel(const gemm_params_t p) {
 #pragma unroll 1
         for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
             const int row = it * ROWS_PER_IT + lane / (WN / 4);
-            const int col = (lane % (WN / 4)) * 4;
-            const float4 t = *(const float4 *)&stg[row * WN + col];
+            const float4 t = *(const float4 *)&stg[row * WN + ecol];
             const int m = m0 + wm0 + i * 32 + row;
-            const int n = n0 + wn0 + col;
-            if (m < p.M && n < p.N) {
+            if (m < p.M && en < p.N) {
                 float v[4] = {t.x, t.y, t.z, t.w};
-                epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
+                if (p.ep.fast != EP_FAST_NONE) {
+                    float ss = 1.f;
+                    if (has_ss)
+                        ss = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
+                                + m * p.ep.src_scale.sm];
+                    epilogue_fast4(
+                            p.ep, v, has_ss, ss, has_ws, ws4, bz, m, en, envalid);
+                } else
+                    epilogue_apply_store4(p.ep, v, bz, m, en, envalid);
             }
         }
     });
 }
 
-template <int BM, int BN, int BK, int WGM, int WGN, bool F8>
+template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, bool F8,
+        bool U8A>
 static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
     gemm_params_t q = p;
     q.tiles_m = (p.M + BM - 1) / BM;
@@ -313,11 +372,11 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
     const int ntiles = q.tiles_m * q.tiles_n;
     // with the XCD remap every XCD gets ceil(ntiles/8) slots
     const int grid_x = ntiles >= 64 ? ((ntiles + 7) / 8) * 8 : ntiles;
-    constexpr size_t lds_main = 2 * (size_t)(BM + BN) * BK;
+    constexpr size_t lds_main = (size_t)STAGES * (BM + BN) * BK;
     constexpr size_t lds_ep
             = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
     constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
-    auto kern = gemm_b8_kernel<BM, BN, BK, WGM, WGN, F8>;
+    auto kern = gemm_b8_kernel<BM, BN, BK, WGM, WGN, STAGES, F8, U8A>;
     static bool attr_done = false;
     if (!attr_done) {
         (void)hipFuncSetAttribute((const void *)kern,
@@ -332,25 +391,28 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
 // instantiations build in parallel; the unit without the macro holds the
 // dispatcher.
 #if defined(QMM_GEMM_VARIANT)
+// BM, BN, BK, waves along M, waves along N, LDS stages
 #if QMM_GEMM_VARIANT == 1
-#define QMM_CFG 256, 128, 64, 2, 2
+#define QMM_CFG 256, 128, 64, 2, 2, 3
 #elif QMM_GEMM_VARIANT == 2
-#define QMM_CFG 128, 128, 64, 2, 2
+#define QMM_CFG 128, 128, 64, 2, 2, 3
 #elif QMM_GEMM_VARIANT == 3
-#define QMM_CFG 256, 256, 64, 2, 2
+#define QMM_CFG 256, 256, 64, 2, 4, 3
 #elif QMM_GEMM_VARIANT == 4
-#define QMM_CFG 128, 256, 64, 2, 2
+#define QMM_CFG 256, 256, 64, 2, 4, 4
 #elif QMM_GEMM_VARIANT == 5
-#define QMM_CFG 256, 128, 128, 2, 2
+#define QMM_CFG 256, 128, 64, 2, 2, 4
 #endif
 #define QMM_CAT_(a, b) a##b
 #define QMM_CAT(a, b) QMM_CAT_(a, b)
 void QMM_CAT(launch_gemm_b8_v, QMM_GEMM_VARIANT)(
         const gemm_params_t &p, bool f8, hipStream_t stream) {
     if (f8)
-        launch_cfg<QMM_CFG, true>(p, stream);
+        launch_cfg<QMM_CFG, true, false>(p, stream);
+    else if (p.a_is_u8)
+        launch_cfg<QMM_CFG, false, true>(p, stream);
     else
-        launch_cfg<QMM_CFG, false>(p, stream);
+        launch_cfg<QMM_CFG, false, false>(p, stream);
 }
 #else
 void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);

@@ -52,7 +52,12 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <bool F16>
+// FAST: one 16-bit scale and at most one byte-sized (4- or 8-bit) zero point
+// per column and 128-k tile. Every load of that variant is unconditional
+// (out-of-range tiles re-read the last valid one, absent buffers are replaced
+// by the weights pointer), so the number of loads in flight is known at
+// compile time and no wait has to drain the whole queue.
+template <bool F16, bool FAST>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -92,42 +97,127 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
             = p.B + ((int64_t)nb * p.kg128) * 1024 + lane * 16;
     const int Kpad = p.kg128 * 128;
 
+    // Scale / zero point of the group that contains k (this lane's column).
+    // Loading and decoding are split: the raw bits are fetched without any
+    // dependent instruction, so the compiler can leave the loads in flight
+    // next to the weights stream and convert when the value is needed.
+    const int64_t sN = p.scale_per_n ? p.N : 0, zN = p.zp_per_n ? p.N : 0;
+    const bool lane_ok = n < p.N;
+    auto scale_raw = [&](int kq) -> uint32_t {
+        if (!p.scales || !lane_ok) return 0u;
+        const int64_t idx = (int64_t)(kq / p.gs) * (p.scale_per_n ? p.N : 1)
+                + (p.scale_per_n ? n : 0);
+        return p.scale_dt == dt_f32 ? ((const uint32_t *)p.scales)[idx]
+                                    : (uint32_t)((const uint16_t *)p.scales)[idx];
+    };
+    auto scale_cvt = [&](uint32_t raw) -> float {
+        if (!p.scales || !lane_ok) return 1.f;
+        if (p.scale_dt == dt_f32) return u2f(raw);
+        if (p.scale_dt == dt_bf16) return u2f(raw << 16);
+        return f16_to_f32((uint16_t)raw);
+    };
+    auto zp_index = [&](int kq) -> int64_t {
+        const int64_t g = p.gz > 0 ? kq / p.gz : 0;
+        return g * (p.zp_per_n ? p.N : 1) + (p.zp_per_n ? n : 0);
+    };
+    auto zp_raw = [&](int kq) -> uint32_t {
+        if (!p.zps || !lane_ok) return 0u;
+        const int64_t idx = zp_index(kq);
+        if (p.zp_dt == dt_s32) return ((const uint32_t *)p.zps)[idx];
+        if (p.zp_dt == dt_s4 || p.zp_dt == dt_u4)
+            return ((const uint8_t *)p.zps)[idx >> 1];
+        return ((const uint8_t *)p.zps)[idx];
+    };
+    auto zp_cvt = [&](uint32_t raw, int kq) -> float {
+        if (!p.zps || !lane_ok) return 0.f;
+        switch (p.zp_dt) {
+            case dt_s32: return (float)(int32_t)raw;
+            case dt_s8: return (float)(int8_t)raw;
+            case dt_u8: return (float)(uint8_t)raw;
+            default: {
+                const int nib = (zp_index(kq) & 1) ? (raw >> 4) & 0xf : raw & 0xf;
+                return (float)(p.zp_dt == dt_s4 ? s4_value(nib) : nib);
+            }
+        }
+    };
+    // When no group closes inside a 128-k tile, a tile has one scale and one
+    // zero point per column: they are fetched together with the tile so that
+    // their latency overlaps the weights stream instead of following it.
+    const bool per_tile = FAST || fl % 128 == 0;
+    const uint16_t *const fast_sc = (const uint16_t *)p.scales;
+    const uint8_t *const fast_zp = p.zps ? (const uint8_t *)p.zps : p.B;
+    const bool zp4 = p.zp_dt == dt_s4 || p.zp_dt == dt_u4;
+
     for (int kc0 = 0; kc0 < Kpad; kc0 += KC) {
         const int kc_len = min(KC, Kpad - kc0);
         const int tiles = kc_len / 128;
         const int g0 = kc0 / 128;
-        // first batch of weight loads goes out before the activations
         constexpr int UNR = 4;
         uint4 wt[UNR];
+        uint32_t scp[UNR], zpp[UNR]; // raw scale / zero-point bits per tile
+        auto fetch = [&](int tb) {
 #pragma unroll
-        for (int u = 0; u < UNR; u++) {
-            const int t = wave + u * GEMV_WAVES;
-            wt[u] = make_uint4(0, 0, 0, 0);
-            if (t < tiles)
-                wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
-        }
+            for (int u = 0; u < UNR; u++) {
+                const int t = tb + wave + u * GEMV_WAVES;
+                wt[u] = make_uint4(0, 0, 0, 0);
+                if constexpr (FAST) {
+                    const int tc = min(t, tiles - 1);
+                    wt[u] = ld_stream(Bt + (int64_t)(g0 + tc) * 1024);
+                    const int kq = min(kc0 + (tc + 1) * 128, p.K) - 1;
+                    const int nn = min(n, p.N - 1);
+                    scp[u] = fast_sc[(int64_t)(kq / p.gs) * sN
+                            + (p.scale_per_n ? nn : 0)];
+                    const int64_t zi = p.zps
+                            ? (int64_t)(p.gz > 0 ? kq / p.gz : 0) * zN
+                                    + (p.zp_per_n ? nn : 0)
+                            : 0;
+                    zpp[u] = fast_zp[zp4 ? zi >> 1 : zi];
+                    continue;
+                }
+                scp[u] = 0u;
+                zpp[u] = 0u;
+                if (t < tiles) {
+                    wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
+                    if (per_tile) {
+                        const int kq = min(kc0 + (t + 1) * 128, p.K) - 1;
+                        scp[u] = scale_raw(kq);
+                        zpp[u] = zp_raw(kq);
+                    }
+                }
+            }
+        };
+        // Vector-memory results return in issue order, so the activation
+        // chunks this thread stages are requested first and the weights right
+        // behind them: waiting for the activations then leaves the weights in
+        // flight. Chunk kc (8 values) of row m lands at (kc*MR + m)*16.
         if (kc0 > 0) __syncthreads(); // previous chunk fully consumed
-        // stage activations: chunk kc (8 values) of row m -> (kc*MR + m)*16
-        for (int i = tid; i < (kc_len / 8) * MR; i += GEMV_WAVES * 64) {
+        const int nchunks = (kc_len / 8) * MR;
+        auto act_load = [&](int i) -> uint4 {
             const int kc = i / MR, m = i % MR;
             const int k = kc0 + kc * 8;
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (m < rows && k < p.K)
+            if (i < nchunks && m < rows && k < p.K)
                 v = *(const uint4 *)(p.A + (int64_t)(m_base + m) * p.lda + k);
-            *(uint4 *)(lds + (size_t)i * 16) = v;
+            return v;
+        };
+        constexpr int ACT_PRE = 2;
+        uint4 areg[ACT_PRE];
+#pragma unroll
+        for (int q = 0; q < ACT_PRE; q++)
+            areg[q] = act_load(tid + q * GEMV_WAVES * 64);
+        fetch(0);
+#pragma unroll
+        for (int q = 0; q < ACT_PRE; q++) {
+            const int i = tid + q * GEMV_WAVES * 64;
+            if (i < nchunks) *(uint4 *)(lds + (size_t)i * 16) = areg[q];
         }
+        for (int i = tid + ACT_PRE * GEMV_WAVES * 64; i < nchunks;
+                i += GEMV_WAVES * 64)
+            *(uint4 *)(lds + (size_t)i * 16) = act_load(i);
         __syncthreads();
 
         for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
-            if (tb > 0) {
-#pragma unroll
-                for (int u = 0; u < UNR; u++) {
-                    const int t = tb + wave + u * GEMV_WAVES;
-                    wt[u] = make_uint4(0, 0, 0, 0);
-                    if (t < tiles)
-                        wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
-                }
-            }
+            if (tb > 0) fetch(tb);
 #pragma unroll
             for (int u = 0; u < UNR; u++) {
                 const int t = tb + wave + u * GEMV_WAVES;
@@ -156,25 +246,17 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                     // scale / zero-point group closes inside a tile (folding
                     // early is exact in structure: both factors are constant
                     // over the folded range).
-                    if (s == 3 || k_end % fl == 0) {
+                    if (s == 3 || (!per_tile && k_end % fl == 0)) {
                         // the range just folded contains k_end - 1
-                        const int kq = min(k_end, p.K) - 1;
-                        float sc = 1.f, zp = 0.f;
-                        if (n < p.N) {
-                            if (p.scales)
-                                sc = load_float(p.scale_dt, p.scales,
-                                        p.scale_per_n
-                                                ? (int64_t)(kq / p.gs) * p.N + n
-                                                : (int64_t)(kq / p.gs));
-                            if (p.zps)
-                                zp = (float)load_int(p.zp_dt, p.zps,
-                                        p.gz > 0 ? (p.zp_per_n
-                                                        ? (int64_t)(kq / p.gz)
-                                                                        * p.N
-                                                                + n
-                                                        : (int64_t)(kq / p.gz))
-                                                 : (p.zp_per_n ? (int64_t)n
-                                                               : 0));
+                        float sc, zp;
+                        if (per_tile) {
+                            const int kq = min(kc0 + (t + 1) * 128, p.K) - 1;
+                            sc = scale_cvt(scp[u]);
+                            zp = zp_cvt(zpp[u], kq);
+                        } else {
+                            const int kq = min(k_end, p.K) - 1;
+                            sc = scale_cvt(scale_raw(kq));
+                            zp = zp_cvt(zp_raw(kq), kq);
                         }
                         const float off = OFFSET + soff + zp;
 #pragma unroll
@@ -235,10 +317,31 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, p,
                 MR, KC);
     };
-    if (p.act_f16)
-        launch(gemv_w4_kernel<true>);
-    else
-        launch(gemv_w4_kernel<false>);
+    // the all-unconditional-loads variant (see the kernel's FAST parameter)
+    int fl = p.gs;
+    if (p.gz > 0) {
+        int a = p.gs, b = p.gz;
+        while (b) {
+            const int t = a % b;
+            a = b;
+            b = t;
+        }
+        fl = a;
+    }
+    const bool fast = p.scales && fl % 128 == 0
+            && (p.scale_dt == dt_f16 || p.scale_dt == dt_bf16)
+            && (!p.zps || p.zp_dt != dt_s32);
+    if (p.act_f16) {
+        if (fast)
+            launch(gemv_w4_kernel<true, true>);
+        else
+            launch(gemv_w4_kernel<true, false>);
+    } else {
+        if (fast)
+            launch(gemv_w4_kernel<false, true>);
+        else
+            launch(gemv_w4_kernel<false, false>);
+    }
 }
 
 } // namespace qmm

@@ -1,0 +1,436 @@
+"""GPU parity: every kernel against the CPU oracle on the same seeded inputs,
+through the C ABI (dnnl_* entry points of libdnnl_amd.so).
+
+Bars (written per assertion): s32 / s8 / u8 dst bit-exact; f32 dst rel 1e-5;
+bf16 dst within 1 bf16 ulp; int4 decompression rel 1e-2 (measured far below).
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import onednn_amd as dnnl
+import oracle as O
+from onednn_amd import memory
+from qmm_harness import (Problem, T, TensorSpec, assert_bf16_within_1ulp, assert_bit_exact,
+                         assert_f32_close, dt, tag)
+
+pytestmark = pytest.mark.gpu
+
+A = dnnl.algorithm
+GENERIC, MFMA, DECODE = "hip:gfx950:generic", "hip:gfx950:mfma_b8", "hip:gfx950:decode_w4"
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    eng = dnnl.engine(dnnl.engine.kind.gpu, 0)
+    return eng, dnnl.stream(eng)
+
+
+def rnd(seed):
+    return np.random.default_rng(seed)
+
+
+# ---------------------------------------------------------------------------
+# problem builders (value distributions of the benchmark configurations)
+def int8_linear(M, K, N, seed, src_dt=dt.u8, dst_dt=dt.f32, src_zp=128, src_scale=0.02,
+                per_token=False, post_ops=None, bias_dt=None, dst_scale=None, dst_zp=None,
+                dst_zp_per_n=False, wei_layout="ab", batch=()):
+    r = rnd(seed)
+    b = list(batch)
+    if src_dt == dt.u8:
+        s = r.integers(0, 256, b + [M, K])
+    else:
+        s = np.clip(np.rint(r.standard_normal(b + [M, K]) * 32), -127, 127)
+    w = r.integers(-127, 128, b + [K, N])
+    nd = len(b) + 2
+    letters = list("abcdefghijkl"[:nd])
+    if wei_layout == "ba":
+        letters[-2], letters[-1] = letters[-1], letters[-2]
+    wl = "".join(letters)
+    src = TensorSpec(src_dt, b + [M, K], None, s)
+    wei = TensorSpec(dt.s8, b + [K, N], wl, w)
+    dst = TensorSpec(dst_dt, b + [M, N])
+    scales = {"wei": (1 << (nd - 1), dt.f32, None, r.uniform(0.001, 0.01, N))}
+    if per_token:
+        scales["src"] = ((1 << (nd - 2)) | (1 << (nd - 1)), dt.f32, (1, K), r.uniform(0.005, 0.05, M))
+    elif src_scale is not None:
+        scales["src"] = (0, dt.f32, None, [src_scale])
+    zps = {}
+    if src_zp is not None:
+        zps["src"] = (0, dt.s32, None, [src_zp])
+    if dst_scale is not None:
+        scales["dst"] = (0, dt.f32, None, [dst_scale])
+    if dst_zp is not None:
+        zps["dst"] = (2 if dst_zp_per_n else 0, dt.s32, None, dst_zp)
+    bias = None
+    if bias_dt is not None:
+        bias = TensorSpec(bias_dt, [1] * (nd - 1) + [N], None, r.integers(-20, 20, N))
+    return Problem(src, wei, dst, bias=bias, scales=scales, zps=zps, post_ops=post_ops)
+
+
+def decode_w4(M, K, N, seed, G=128, act_dt=dt.bf16, wei_dt=dt.u4, zp_dt=dt.u4, scale_dt=dt.f16,
+              with_zp=True, zp_group=None, post_ops=None):
+    r = rnd(seed)
+    a = r.standard_normal((M, K)).astype(np.float32)
+    lo, hi = (0, 16) if wei_dt == dt.u4 else (-8, 8)
+    w = r.integers(lo, hi, (K, N))
+    src = TensorSpec(act_dt, [M, K], None, a)
+    wei = TensorSpec(wei_dt, [K, N], None, w)
+    dst = TensorSpec(act_dt, [M, N])
+    scales = {"wei": (3, scale_dt, (G, 1), r.uniform(0.005, 0.02, (K // G, N)))}
+    zps = {}
+    if with_zp:
+        zg = zp_group or G
+        zlo, zhi = (6, 10) if zp_dt != dt.s4 else (-2, 3)
+        zps["wei"] = (3, zp_dt, (zg, 1), r.integers(zlo, zhi, (K // zg, N)))
+    return Problem(src, wei, dst, scales=scales, zps=zps, post_ops=post_ops, apply_to_int=True,
+                   fpmath=dnnl.fpmath_mode.bf16 if act_dt == dt.bf16 else dnnl.fpmath_mode.f16)
+
+
+def fp8_gemm(M, K, N, seed, dst_dt=dt.bf16, with_sum=True):
+    r = rnd(seed)
+    a = np.clip(r.standard_normal((M, K)) * 4, -448, 448).astype(np.float32)
+    b = np.clip(r.standard_normal((K, N)) * 4, -448, 448).astype(np.float32)
+    src = TensorSpec(dt.f8_e4m3, [M, K], None, a)
+    wei = TensorSpec(dt.f8_e4m3, [K, N], None, b)
+    dst = TensorSpec(dst_dt, [M, N], None, r.standard_normal((M, N)).astype(np.float32))
+    scales = {"src": (0, dt.f32, None, [0.5]), "wei": (0, dt.f32, None, [0.25])}
+    po = [{"kind": "sum", "scale": 1.0}] if with_sum else []
+    return Problem(src, wei, dst, scales=scales, post_ops=po)
+
+
+def decode_term_scale(p):
+    """sum_k |a| * |w - zp| * scale per output of a weights-decompression problem."""
+    a = np.abs(p.src.logical().astype(np.float64))
+    w = p.wei.logical().astype(np.float64)
+    K, N = w.shape
+    mask, code, groups, vals = p.scales["wei"]
+    sc = O.to_f32(code, Problem._quant_raw(code, vals)).astype(np.float64).reshape(K // groups[0], N)
+    if "wei" in p.zps:
+        zm, zc, zg, zv = p.zps["wei"]
+        w = w - np.repeat(np.asarray(zv, np.float64).reshape(K // zg[0], N), zg[0], 0)
+    return a @ (np.abs(w) * np.repeat(sc, groups[0], 0))
+
+
+def term_scale(p):
+    """Magnitude of the summed terms per output: |src - zp| @ |wei| * scales."""
+    s = np.abs(p.src.logical().astype(np.float64))
+    if "src" in p.zps:
+        s = np.abs(p.src.logical().astype(np.float64) - np.asarray(p.zps["src"][3], np.float64).reshape(-1)[0])
+    w = np.abs(p.wei.logical().astype(np.float64))
+    t = s @ w
+    if "src" in p.scales:
+        v = np.asarray(p.scales["src"][3], np.float64).reshape(-1)
+        t = t * (v[:, None] if v.size > 1 else v[0])
+    if "wei" in p.scales:
+        v = np.asarray(p.scales["wei"][3], np.float64).reshape(-1)
+        t = t * (v[None, :] if v.size > 1 else v[0])
+    return t
+
+
+# ---------------------------------------------------------------------------
+# the generic kernel: operation-for-operation restatement, bit-exact everywhere
+GENERIC_CASES = {
+    "c1_small": lambda: int8_linear(24, 96, 40, 1),
+    "s8_per_token_swish_bf16": lambda: int8_linear(17, 128, 24, 2, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True,
+                                                   post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.1}]),
+    "u8_dst_with_zp_scale_bias": lambda: int8_linear(9, 64, 33, 3, dst_dt=dt.u8, bias_dt=dt.f32, dst_scale=3.0,
+                                                     dst_zp=[7], post_ops=[{"kind": "eltwise", "alg": A.eltwise_linear, "alpha": 0.5, "beta": 1.0}]),
+    "s8_dst_per_n_dst_zp": lambda: int8_linear(9, 64, 32, 4, dst_dt=dt.s8, dst_scale=2.0, dst_zp=rnd(4).integers(-5, 5, 32), dst_zp_per_n=True),
+    "s32_dst": lambda: int8_linear(5, 48, 16, 5, dst_dt=dt.s32, src_scale=None),
+    "batched_ba_weights": lambda: int8_linear(7, 32, 12, 6, src_dt=dt.s8, src_zp=None, wei_layout="ba", batch=(2, 3)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(GENERIC_CASES))
+def test_generic_int8_bit_exact(ctx, name):
+    eng, strm = ctx
+    say("generic " + name)
+    p = GENERIC_CASES[name]()
+    got = p.run_gpu(eng, strm, impl=GENERIC)
+    assert_bit_exact(got, p.run_oracle(), name)
+
+
+def test_generic_grouped_dynamic_quant_and_chain(ctx):
+    eng, strm = ctx
+    say("generic grouped s8 x u4, grouped src/wei scales and zero points, post-op chain")
+    r = rnd(11)
+    M, K, N = 6, 128, 16
+    src = TensorSpec(dt.s8, [M, K], None, r.integers(-128, 128, (M, K)))
+    wei = TensorSpec(dt.u4, [K, N], None, r.integers(0, 16, (K, N)))
+    dst = TensorSpec(dt.f32, [M, N], None, r.integers(-5, 5, (M, N)).astype(np.float32))
+    col = TensorSpec(dt.f32, [1, N], None, r.uniform(0.5, 2, N).astype(np.float32))
+    p = Problem(src, wei, dst,
+                scales={"src": (3, dt.f16, (1, 64), r.uniform(0.01, 0.1, (M, 2))),
+                        "wei": (3, dt.bf16, (32, 1), r.uniform(0.01, 0.1, (4, N)))},
+                zps={"src": (3, dt.s8, (1, 128), r.integers(-3, 3, (M, 1))),
+                     "wei": (3, dt.u4, (64, 1), r.integers(6, 10, (2, N)))},
+                post_ops=[{"kind": "binary", "alg": A.binary_mul, "src1": col},
+                          {"kind": "sum", "scale": 0.5},
+                          {"kind": "prelu", "mask": 2, "weights": 2.0 ** r.integers(-2, 2, N)},
+                          {"kind": "eltwise", "alg": A.eltwise_clip_v2, "alpha": -3.0, "beta": 4.0}])
+    got = p.run_gpu(eng, strm, impl=GENERIC)
+    assert_bit_exact(got, p.run_oracle(), "grouped chain")
+
+
+@pytest.mark.parametrize("act,wei,zp", [(dt.bf16, dt.u4, dt.u4), (dt.f16, dt.s4, dt.s8), (dt.bf16, dt.s8, None)])
+def test_generic_float_paths_bit_exact(ctx, act, wei, zp):
+    """Sequential f32 accumulation in k order, as the reference's float path."""
+    eng, strm = ctx
+    say("generic decompression %d x %d" % (act, wei))
+    if wei == dt.s8:
+        r = rnd(21)
+        M, K, N = 3, 64, 8
+        p = Problem(TensorSpec(act, [M, K], None, r.standard_normal((M, K)).astype(np.float32)),
+                    TensorSpec(dt.s8, [K, N], None, r.integers(-128, 128, (K, N))),
+                    TensorSpec(act, [M, N]),
+                    scales={"wei": (2, dt.f32, None, r.uniform(0.001, 0.01, N))},
+                    apply_to_int=True, fpmath=dnnl.fpmath_mode.bf16)
+    else:
+        p = decode_w4(3, 256, 16, 22, act_dt=act, wei_dt=wei, zp_dt=zp)
+    got = p.run_gpu(eng, strm, impl=GENERIC)
+    assert_bit_exact(got, p.run_oracle(), "float path")
+
+
+def test_generic_fp8_and_f32(ctx):
+    eng, strm = ctx
+    say("generic fp8 sum + plain f32")
+    p = fp8_gemm(8, 64, 8, 31)
+    assert_bit_exact(p.run_gpu(eng, strm, impl=GENERIC), p.run_oracle(), "fp8")
+    r = rnd(32)
+    p = Problem(TensorSpec(dt.f32, [4, 33], None, r.standard_normal((4, 33)).astype(np.float32)),
+                TensorSpec(dt.f32, [33, 5], "ba", r.standard_normal((33, 5)).astype(np.float32)),
+                TensorSpec(dt.f32, [4, 5]))
+    assert_bit_exact(p.run_gpu(eng, strm), p.run_oracle(), "f32")
+
+
+# ---------------------------------------------------------------------------
+# MFMA int8 GEMM: exact s32 accumulation + reference-ordered epilogue
+MFMA_CASES = {
+    # name: (builder, exact) -- exact=False when a transcendental post-op is involved
+    "c1_shape": (lambda: int8_linear(256, 1024, 1024, 41), True),
+    "c1_tails": (lambda: int8_linear(200, 272, 150, 42), True),
+    "c1_plain_weights_ba": (lambda: int8_linear(64, 128, 96, 43, wei_layout="ba"), True),
+    "u8_zp_7_s8_dst": (lambda: int8_linear(130, 256, 260, 44, dst_dt=dt.s8, src_zp=7, dst_scale=40.0, dst_zp=[3], bias_dt=dt.s32), True),
+    "s8_u8_dst_relu": (lambda: int8_linear(96, 512, 128, 45, src_dt=dt.s8, dst_dt=dt.u8, src_zp=None, dst_scale=25.0,
+                                            post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]), True),
+    "s8_s32_dst_no_scales": (lambda: int8_linear(64, 4096, 64, 46, src_dt=dt.s8, dst_dt=dt.s32, src_zp=None, src_scale=None), True),
+    "c2_slice_per_token_bf16": (lambda: int8_linear(384, 4096, 512, 47, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True), True),
+    "c2_slice_swish": (lambda: int8_linear(256, 1024, 256, 48, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True,
+                                            post_ops=[{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]), False),
+}
+
+
+@pytest.mark.parametrize("name", sorted(MFMA_CASES))
+@pytest.mark.parametrize("weights_any", [True, False])
+def test_mfma_int8(ctx, name, weights_any):
+    eng, strm = ctx
+    say("mfma_b8 %s any=%s" % (name, weights_any))
+    build, exact = MFMA_CASES[name]
+    p = build()
+    got, pd = p.run_gpu(eng, strm, weights_any=weights_any, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    want = p.run_oracle()
+    if exact:
+        assert_bit_exact(got, want, name)  # integer dst and f32/bf16 after exact ops: bit-exact
+    else:
+        assert_bf16_within_1ulp(got, want, name)  # device expf vs libm: 1 bf16 ulp
+
+
+def test_mfma_int8_s32_accumulators_are_exact(ctx):
+    eng, strm = ctx
+    say("mfma_b8 s32 accumulators, u8 with zero point, K=4096")
+    p = int8_linear(64, 4096, 96, 51, dst_dt=dt.s32, src_zp=119, src_scale=None)
+    p.scales = {}
+    got = p.run_gpu(eng, strm, weights_any=True).view(np.int32).reshape(64, 96)
+    exact = (p.src.logical().astype(np.int64) - 119) @ p.wei.logical().astype(np.int64)
+    # below 2^24 the f32 detour of the store is exact too
+    small = np.abs(exact) < 2 ** 24
+    assert small.any() and np.array_equal(got[small], exact[small])
+    assert_bit_exact(got, p.run_oracle().view(np.int32).reshape(64, 96), "s32 dst")
+
+
+def test_mfma_int8_against_literal_v38_reference(ctx):
+    """The v3.8 source, read literally, sums scaled products in f32 one k at a
+    time; the integer accumulation used here differs from it by f32 summation
+    error only: within 1e-5 of the magnitude of the summed terms."""
+    eng, strm = ctx
+    say("mfma_b8 vs literal k-by-k f32 reference")
+    p = int8_linear(64, 1024, 128, 52)
+    got = p.run_gpu(eng, strm, weights_any=True).view(np.float32).reshape(64, 128)
+    want = p.run_oracle(k_group_mode=O.KGROUP_LITERAL).view(np.float32).reshape(64, 128)
+    assert_f32_close(got, want, rel=1e-5, scale=term_scale(p), what="literal")
+
+
+def test_mfma_batched_scores_with_mask(ctx):
+    eng, strm = ctx
+    say("mfma_b8 batched scores (config 4 shape, fewer heads) + binary add mask, K^T weights view")
+    r = rnd(53)
+    B, S, D = 3, 256, 128
+    q = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127)
+    k = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127)
+    mask = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], -1e4, 0).astype(np.float32)[None]
+    for wl, wv in (("abc", np.transpose(k, (0, 2, 1))), ("acb", np.transpose(k, (0, 2, 1)))):
+        p = Problem(TensorSpec(dt.s8, [B, S, D], None, q), TensorSpec(dt.s8, [B, D, S], wl, wv),
+                    TensorSpec(dt.f32, [B, S, S]),
+                    scales={"src": (0, dt.f32, None, [0.01]), "wei": (0, dt.f32, None, [0.012])},
+                    post_ops=[{"kind": "binary", "alg": A.binary_add, "src1": TensorSpec(dt.f32, [1, S, S], None, mask)}])
+        for any_ in (True, False):
+            got, pd = p.run_gpu(eng, strm, weights_any=any_, return_pd=True)
+            assert pd.impl_info_str() == MFMA
+            assert_bit_exact(got, p.run_oracle(), "scores %s any=%s" % (wl, any_))
+
+
+def test_mfma_fp8(ctx):
+    eng, strm = ctx
+    for (M, K, N, dd) in ((128, 256, 128, dt.bf16), (200, 512, 136, dt.f32)):
+        say("mfma_b8 fp8 %dx%dx%d" % (M, K, N))
+        p = fp8_gemm(M, K, N, 61, dst_dt=dd)
+        for any_ in (True, False):
+            got, pd = p.run_gpu(eng, strm, weights_any=any_, return_pd=True)
+            assert pd.impl_info_str() == MFMA
+            want = p.run_oracle()
+            a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
+            if dd == dt.bf16:
+                # MFMA sums in another order than the reference's k loop: 1 bf16 ulp,
+                # or the f32 bar (1e-5 of the summed magnitudes) where the result cancels
+                assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
+            else:
+                assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
+                                 rel=1e-5, scale=a, what="fp8 f32")
+
+
+# ---------------------------------------------------------------------------
+# decode: 4-bit weights
+@pytest.mark.parametrize("M", [1, 2, 16, 19])
+@pytest.mark.parametrize("weights_any", [True, False])
+def test_decode_w4_config3(ctx, M, weights_any):
+    eng, strm = ctx
+    say("decode_w4 M=%d K=N=1024 G=128 any=%s" % (M, weights_any))
+    p = decode_w4(M, 1024, 1024, 70 + M)
+    got, pd = p.run_gpu(eng, strm, weights_any=weights_any, return_pd=True)
+    assert pd.impl_info_str() == DECODE
+    want = p.run_oracle()
+    g = O.to_f32(dt.bf16, got).reshape(M, 1024)
+    w = O.to_f32(dt.bf16, want).reshape(M, 1024)
+    # rel 1e-2 is the bar of the int4 bf16-math path
+    assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="decode")
+    # what the kernel actually achieves: 1 bf16 ulp, or 2e-5 of the summed
+    # magnitudes where the result cancels (f32 accumulation in another order)
+    assert_bf16_within_1ulp(got, want, "decode bf16", abs_slack=2e-5 * decode_term_scale(p))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(act_dt=dt.f16, wei_dt=dt.s4, zp_dt=dt.s8, scale_dt=dt.f32, G=64),
+    dict(act_dt=dt.bf16, wei_dt=dt.u4, zp_dt=dt.u8, G=32, zp_group=128),
+    dict(act_dt=dt.bf16, wei_dt=dt.s4, with_zp=False, scale_dt=dt.bf16, G=256),
+    dict(act_dt=dt.bf16, wei_dt=dt.u4, zp_dt=dt.u4, G=128,
+         post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]),
+])
+def test_decode_w4_variants(ctx, kw):
+    eng, strm = ctx
+    say("decode_w4 variant %r" % (kw,))
+    p = decode_w4(5, 512, 272, 80, **kw)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == DECODE
+    want = p.run_oracle()
+    code = kw.get("act_dt", dt.bf16)
+    g, w = O.to_f32(code, got), O.to_f32(code, want)
+    assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="decode variant")
+
+
+# ---------------------------------------------------------------------------
+# reorder
+def test_prepack_round_trip(ctx):
+    eng, strm = ctx
+    say("prepack round trips")
+    r = rnd(90)
+    for code, dims, layout in ((dt.s8, [208, 150], "ab"), (dt.s8, [2, 96, 70], "acb"), (dt.f8_e4m3, [64, 64], "ba"),
+                               (dt.u4, [256, 48], "ab"), (dt.s4, [136, 34], "ba")):
+        vals = r.integers(0, 16, dims) if code in (dt.u4,) else r.integers(-8, 8, dims)
+        t = TensorSpec(code, dims, layout, vals if code not in (dt.f8_e4m3,) else vals.astype(np.float32))
+        if code in (dt.u4, dt.s4):
+            src_md = memory.desc([1, dims[0]], dt.bf16, T("ab"))
+            attr = dnnl.primitive_attr()
+            attr.set_fpmath_mode(dnnl.fpmath_mode.bf16, True)
+            pd = dnnl.matmul.primitive_desc(eng, src_md, memory.desc(dims, code, tag.any),
+                                            memory.desc([1, dims[1]], dt.bf16, T("ab")), attr=attr)
+        else:
+            sdt = dt.s8 if code == dt.s8 else code
+            b = dims[:-2]
+            pd = dnnl.matmul.primitive_desc(eng, memory.desc(b + [16, dims[-2]], sdt, T("abc"[:len(dims)])),
+                                            memory.desc(dims, code, tag.any),
+                                            memory.desc(b + [16, dims[-1]], dt.f32, T("abc"[:len(dims)])))
+        wmd = pd.weights_desc()
+        assert wmd.get_format_kind() == memory.format_kind.opaque
+        plain = memory(t.md(), eng).write(t.raw)
+        packed = memory(wmd, eng)
+        back = memory(t.md(), eng).write(np.zeros_like(t.raw))
+        dnnl.reorder(plain, packed).execute(strm, plain, packed)
+        dnnl.reorder(packed, back).execute(strm, packed, back)
+        strm.wait()
+        got = t.logical(back.read(t.raw.dtype))
+        assert np.array_equal(got, t.logical()), (code, dims, layout)
+
+
+def test_generic_reorder_matches_oracle(ctx):
+    eng, strm = ctx
+    say("quantizing reorder f32 -> s8 (ba) with per-column scales, f32 -> u4")
+    r = rnd(91)
+    K, N = 64, 24
+    w = (r.standard_normal((K, N)) * 3).astype(np.float32)
+    sc = (2.0 ** r.integers(-3, 0, N)).astype(np.float32)
+    src = TensorSpec(dt.f32, [K, N], None, w)
+    for code, layout in ((dt.s8, "ba"), (dt.u4, "ab"), (dt.bf16, "ab")):
+        dst = TensorSpec(code, [K, N], layout)
+        attr = dnnl.primitive_attr()
+        attr.set_scales_mask(dnnl.DNNL_ARG_DST, 2)
+        pd = dnnl.reorder.primitive_desc(eng, src.md(), eng, dst.md(), attr=attr)
+        s_mem = memory(src.md(), eng).write(src.raw)
+        d_mem = memory(dst.md(), eng).write(dst.raw)
+        sc_mem = memory(memory.desc([N], dt.f32, T("a")), eng).write(sc)
+        dnnl.reorder(pd).execute(strm, {dnnl.DNNL_ARG_FROM: s_mem, dnnl.DNNL_ARG_TO: d_mem,
+                                        dnnl.DNNL_ARG_ATTR_SCALES | dnnl.DNNL_ARG_DST: sc_mem})
+        strm.wait()
+        want = dst.raw.copy()
+        O.reorder(src.oracle(), dst.oracle(want), dst_scale=O.Quant(2, dt.f32, sc))
+        assert_bit_exact(d_mem.read(dst.raw.dtype), want, "reorder %d" % code)
+
+
+# ---------------------------------------------------------------------------
+# execution contract
+def test_execute_argument_errors_and_zero_dims(ctx):
+    eng, strm = ctx
+    say("execute argument checks")
+    p = int8_linear(16, 64, 32, 95)
+    pd = p.primitive_desc(eng)
+    prim = dnnl.matmul(pd)
+    src = memory(pd.src_desc(), eng).write(p.src.raw)
+    wei = memory(pd.weights_desc(), eng).write(p.wei.raw)
+    dst = memory(pd.dst_desc(), eng)
+    with pytest.raises(dnnl.error) as e:  # scales / zero-point memories missing
+        prim.execute(strm, {dnnl.DNNL_ARG_SRC: src, dnnl.DNNL_ARG_WEIGHTS: wei, dnnl.DNNL_ARG_DST: dst})
+    assert e.value.status == dnnl.status.invalid_arguments
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, {dnnl.DNNL_ARG_SRC: src, dnnl.DNNL_ARG_DST: dst})
+    assert e.value.status == dnnl.status.invalid_arguments
+    # zero-dim problems are successful no-ops (src/cpu/matmul/ref_matmul_int8.cpp:64-66)
+    md0 = memory.desc([0, 64], dt.s8, T("ab"))
+    pd0 = dnnl.matmul.primitive_desc(eng, md0, memory.desc([64, 8], dt.s8, T("ab")), memory.desc([0, 8], dt.f32, T("ab")))
+    dnnl.matmul(pd0).execute(strm, {dnnl.DNNL_ARG_SRC: memory(md0, eng), dnnl.DNNL_ARG_WEIGHTS: memory(memory.desc([64, 8], dt.s8, T("ab")), eng),
+                                    dnnl.DNNL_ARG_DST: memory(memory.desc([0, 8], dt.f32, T("ab")), eng)})
+    strm.wait()
+
+
+def test_user_scratchpad_mode(ctx):
+    eng, strm = ctx
+    say("user-managed scratchpad for on-the-fly packing")
+    p = int8_linear(64, 128, 96, 96)
+    got = p.run_gpu(eng, strm, weights_any=False, scratchpad_user=True)
+    assert_bit_exact(got, p.run_oracle(), "user scratchpad")
