@@ -396,12 +396,6 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
 #define QMM_CFG 256, 128, 64, 2, 2, 3
 #elif QMM_GEMM_VARIANT == 2
 #define QMM_CFG 128, 128, 64, 2, 2, 3
-#elif QMM_GEMM_VARIANT == 3
-#define QMM_CFG 256, 256, 64, 2, 4, 3
-#elif QMM_GEMM_VARIANT == 4
-#define QMM_CFG 256, 256, 64, 2, 4, 4
-#elif QMM_GEMM_VARIANT == 5
-#define QMM_CFG 256, 128, 64, 2, 2, 4
 #endif
 #define QMM_CAT_(a, b) a##b
 #define QMM_CAT(a, b) QMM_CAT_(a, b)
@@ -417,15 +411,23 @@ void QMM_CAT(launch_gemm_b8_v, QMM_GEMM_VARIANT)(
 #else
 void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);
 void launch_gemm_b8_v2(const gemm_params_t &p, bool f8, hipStream_t stream);
-void launch_gemm_b8_v3(const gemm_params_t &p, bool f8, hipStream_t stream);
-void launch_gemm_b8_v4(const gemm_params_t &p, bool f8, hipStream_t stream);
-void launch_gemm_b8_v5(const gemm_params_t &p, bool f8, hipStream_t stream);
+// 256 x 256 tile kernel with the hand-ordered main loop (qmm_gemm_b8x.hip)
+bool gemm_b8x_eligible(const gemm_params_t &p, bool f8);
+void launch_gemm_b8x(const gemm_params_t &p, hipStream_t stream);
 
 // variant: 0 = heuristic; others pick a tile configuration explicitly (used by
-// the tuning sweep)
+// the tuning sweep; 6 = the 256 x 256 kernel where it applies)
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return;
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
+            * p.batch;
+    if ((variant == 6 || (variant == 0 && tiles256 >= 192))
+            && gemm_b8x_eligible(p, f8)) {
+        launch_gemm_b8x(p, stream);
+        return;
+    }
+    if (variant == 6) variant = 0;
     if (variant == 0) {
         const int64_t big = (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128)
                 * p.batch;
@@ -433,9 +435,6 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
     }
     switch (variant) {
         case 1: launch_gemm_b8_v1(p, f8, stream); break;
-        case 3: launch_gemm_b8_v3(p, f8, stream); break;
-        case 4: launch_gemm_b8_v4(p, f8, stream); break;
-        case 5: launch_gemm_b8_v5(p, f8, stream); break;
         default: launch_gemm_b8_v2(p, f8, stream); break;
     }
 }

@@ -1,0 +1,476 @@
+// hip:gfx950:mfma_b8, large-problem kernel: int8 (s8 x s8 -> s32) GEMM with
+// a 256 x 256 x 64 block tile, four waves of 128 x 128 each (one per SIMD, the
+// 256 accumulator registers of a wave hold its tile), and a hand-ordered main
+// loop.
+//
+// Why this shape. With one wave per SIMD nothing hides a stalled instruction,
+// so the loop is written as an explicit sequence: every v_mfma_i32_32x32x32_i8
+// (32 cycles of matrix-core time) is followed by at most two cheap
+// instructions, the LDS fragment reads for the next 16 MFMAs and the
+// global -> LDS loads two tiles ahead are spread between the MFMAs, and the
+// waits are counted (lgkmcnt / vmcnt) instead of full. Measured on MI355X the
+// loop then runs at the MFMA issue rate (65.5 k of 74 k cycles per tile); what
+// remains is the clock the chip sustains while matrix cores and the L2 -> LDS
+// stream are both busy, and the 256 x 256 tile is what minimises that stream
+// per MFMA (32 KiB per 128 MFMAs and CU).
+//
+// Pipeline (k-step = 64 k, two MFMA sub-steps of 32 k):
+//   LDS ring of 4 stages x (A 256x64 + B 256x64 bytes). The A half of tile t+2
+//   is requested in the second sub-step of k-step t-1... in general: k-step kt
+//   first finishes tile kt-1 (second sub-step) while requesting the A half of
+//   tile kt+2, then starts tile kt (first sub-step) while requesting the B half
+//   of tile kt+2. One barrier per k-step, preceded by vmcnt(8): tile kt has
+//   landed for every wave and the stage that tile kt+2 goes to (last read in
+//   k-step kt-2) is free. Fragments are double buffered in registers and read
+//   one sub-step ahead.
+//
+// Semantics are those of qmm_gemm_b8.hip (same packed weights, same source
+// zero-point compensation through the stored column sums, same epilogue
+// arithmetic as src/cpu/matmul/ref_matmul_int8.cpp:195-259); only epilogues of
+// the straight-line kinds (EP_FAST_*) are handled here, everything else stays
+// with the general kernel.
+#include <type_traits>
+
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace b8x {
+
+constexpr int BM = 256, BN = 256, BK = 64, NT = 256;
+constexpr int STAGES = 4;
+constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+constexpr uint32_t RING = STAGES * STAGE_BYTES; // 128 KiB, power of two
+constexpr int SS_OFF = RING; // 256 per-row source scales (f32)
+constexpr int STG_WAVE = 64 * 128 * 4; // epilogue staging of one wave (in the ring)
+constexpr int LDS_TOTAL = RING + 1024;
+
+template <int N, typename F>
+QMM_D void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1> {});
+    }
+}
+
+// chunk swizzle of the row-major A tile (4 chunks of 16 bytes per row)
+QMM_D int a_swz(int row, int q) {
+    return q ^ ((row >> 2) & 3);
+}
+
+} // namespace b8x
+
+// The main loop is assembled from these pieces. The memory instructions are
+// inline assembly so that they stay exactly where they are written and carry
+// no compiler-inserted waits; the MFMAs are builtins (the compiler knows their
+// latency when it later reads the accumulators) pinned in place by scheduling
+// barriers.
+#define QX_SB() __builtin_amdgcn_sched_barrier(0)
+#define QX_MF(i, j, cb) \
+    { \
+        QX_SB(); \
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8( \
+                fa[cb][i], fb[cb][j], acc[i][j], 0, 0, 0); \
+        QX_SB(); \
+    }
+#define QX_DSR(dst, addr, off) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" \
+                 : "=v"(dst) \
+                 : "v"(addr), "n"(off))
+#define QX_WL(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
+#define QX_WV(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+// LDS destination of a direct load = M0 + 16 * lane
+#define QX_M0(sreg, imm) \
+    asm volatile("s_add_u32 m0, %0, %1" ::"s"(sreg), "n"(imm) : "m0", "scc")
+#define QX_DMA(voff, sbase) \
+    asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase) \
+                 : "memory")
+#define QX_RD_A(nb, va, i) QX_DSR(fa[nb][i], va, (i)*2048)
+#define QX_RD_B(nb, vb, nki, j) QX_DSR(fb[nb][j], vb, ((j)*2 + (nki)) * 1024)
+
+// 16 MFMAs on fragment buffer CB. The 8 fragments of the next sub-step are
+// read into buffer NB in the order a0 b0 b1 b2 b3 a1 a2 a3 (the order the next
+// sub-step's counted waits assume); D0..D3 are direct loads (or empty).
+#define QX_SUB(CB, NB, NA, NBA, NKI, D0, D1, D2, D3) \
+    QX_WL(3); \
+    QX_MF(0, 0, CB); QX_RD_A(NB, NA, 0); \
+    QX_MF(0, 1, CB); QX_RD_B(NB, NBA, NKI, 0); \
+    QX_MF(0, 2, CB); QX_RD_B(NB, NBA, NKI, 1); \
+    QX_MF(0, 3, CB); QX_RD_B(NB, NBA, NKI, 2); \
+    QX_WL(6); \
+    QX_MF(1, 0, CB); QX_RD_B(NB, NBA, NKI, 3); \
+    D0; QX_MF(1, 1, CB); D1; QX_MF(1, 2, CB); D2; QX_MF(1, 3, CB); \
+    QX_WL(6); \
+    D3; QX_MF(2, 0, CB); \
+    QX_MF(2, 1, CB); QX_MF(2, 2, CB); QX_RD_A(NB, NA, 1); QX_MF(2, 3, CB); \
+    QX_WL(6); \
+    QX_MF(3, 0, CB); QX_RD_A(NB, NA, 2); QX_MF(3, 1, CB); \
+    QX_MF(3, 2, CB); QX_RD_A(NB, NA, 3); QX_MF(3, 3, CB);
+// the four direct loads of one tile half (V: per-lane offsets, SB: base
+// pointer, SD: LDS destination of the wave); each M0 write sits one MFMA before
+// the load that uses it
+#define QX_D0(V, SB, SD) QX_M0(SD, 0 * 4096)
+#define QX_D1(V, SB, SD) \
+    QX_DMA(V[0], SB); \
+    QX_M0(SD, 1 * 4096)
+#define QX_D2(V, SB, SD) \
+    QX_DMA(V[1], SB); \
+    QX_M0(SD, 2 * 4096)
+#define QX_D3(V, SB, SD) \
+    QX_DMA(V[2], SB); \
+    QX_M0(SD, 3 * 4096)
+#define QX_D4(V, SB, SD) QX_DMA(V[3], SB)
+#define QX_SUB_D(CB, NB, NA, NBA, NKI, V, SB, SD) \
+    QX_WL(3); \
+    QX_MF(0, 0, CB); QX_RD_A(NB, NA, 0); \
+    QX_MF(0, 1, CB); QX_RD_B(NB, NBA, NKI, 0); \
+    QX_MF(0, 2, CB); QX_RD_B(NB, NBA, NKI, 1); \
+    QX_MF(0, 3, CB); QX_RD_B(NB, NBA, NKI, 2); \
+    QX_WL(6); \
+    QX_MF(1, 0, CB); QX_RD_B(NB, NBA, NKI, 3); \
+    QX_D0(V, SB, SD); QX_MF(1, 1, CB); QX_D1(V, SB, SD); QX_MF(1, 2, CB); \
+    QX_D2(V, SB, SD); QX_MF(1, 3, CB); \
+    QX_WL(6); \
+    QX_D3(V, SB, SD); QX_MF(2, 0, CB); QX_D4(V, SB, SD); \
+    QX_MF(2, 1, CB); QX_MF(2, 2, CB); QX_RD_A(NB, NA, 1); QX_MF(2, 3, CB); \
+    QX_WL(6); \
+    QX_MF(3, 0, CB); QX_RD_A(NB, NA, 2); QX_MF(3, 1, CB); \
+    QX_MF(3, 2, CB); QX_RD_A(NB, NA, 3); QX_MF(3, 3, CB);
+#define QX_SUB_LAST(CB) \
+    QX_WL(0); \
+    QX_MF(0, 0, CB); QX_MF(0, 1, CB); QX_MF(0, 2, CB); QX_MF(0, 3, CB); \
+    QX_MF(1, 0, CB); QX_MF(1, 1, CB); QX_MF(1, 2, CB); QX_MF(1, 3, CB); \
+    QX_MF(2, 0, CB); QX_MF(2, 1, CB); QX_MF(2, 2, CB); QX_MF(2, 3, CB); \
+    QX_MF(3, 0, CB); QX_MF(3, 1, CB); QX_MF(3, 2, CB); QX_MF(3, 3, CB);
+
+// epilogue_fast4 for a full group of four bf16 results: same arithmetic, the
+// conversion done by v_cvt_pk_bf16_f32 (round to nearest even; the caller runs
+// with f32 denormals flushed, which reproduces the reference's subnormal -> 0).
+QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
+        float ss, bool has_ws, const float (&ws)[4], int64_t b, int64_t m,
+        int64_t n) {
+    if (has_ss) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= ss;
+    }
+    if (has_ws) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] *= ws[i];
+    }
+    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n;
+    uint16_t *q = (uint16_t *)ep.dst.ptr + dst_off;
+    const int fast = ep.fast;
+    if (fast == EP_FAST_RELU) {
+        const float alpha = ep.po[0].alpha;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = d[i] > 0 ? d[i] : d[i] * alpha;
+    } else if (fast == EP_FAST_SWISH) {
+        const float na = -ep.po[0].alpha * 1.44269504088896340736f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float e = __builtin_amdgcn_exp2f(d[i] * na);
+            d[i] = d[i] * __builtin_amdgcn_rcpf(1.0f + e);
+        }
+    } else if (fast == EP_FAST_ADD) {
+        const float *y = (const float *)ep.po[0].t.ptr + b * ep.po[0].t.sb
+                + m * ep.po[0].t.sm + n;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] += y[i];
+    } else if (fast == EP_FAST_SUM) {
+        const float sc = ep.po[0].scale;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] += sc * (bf16_to_f32(q[i]) - 0.f);
+    }
+    uint32_t h0, h1;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(h0) : "v"(d[0]), "v"(d[1]));
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(h1) : "v"(d[2]), "v"(d[3]));
+    if ((((uintptr_t)q) & 7) == 0) {
+        *(uint2 *)q = make_uint2(h0, h1);
+    } else {
+        q[0] = (uint16_t)h0;
+        q[1] = (uint16_t)(h0 >> 16);
+        q[2] = (uint16_t)h1;
+        q[3] = (uint16_t)(h1 >> 16);
+    }
+}
+
+__global__ void __launch_bounds__(b8x::NT, 1)
+gemm_b8x_kernel(const gemm_params_t p) {
+    using namespace b8x;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+    // ---- XCD-aware tile order (see qmm_gemm_b8.hip) ----
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        lt = xcd * per + slot;
+        if (slot >= per || lt >= ntiles) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const int KT = p.K / BK; // host guarantees K % 64 == 0 and KT >= 4
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+
+    // Per-lane 32-bit offsets from the tile's base pointers. Chunk c = tid +
+    // 256 j of the A tile is row c / 4, LDS chunk position c % 4, and holds
+    // the row's chunk (c % 4) ^ swz(row): the swizzle is applied on the global
+    // side because a direct load fills LDS in lane order. Rows past M and
+    // column blocks past the packed N re-read the last valid ones.
+    uint32_t a_vo[4], b_vo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tid + j * NT;
+        const int row = c >> 2, cp = c & 3;
+        const int gm = min(m0 + row, p.M - 1) - m0;
+        a_vo[j] = (uint32_t)gm * (uint32_t)p.lda + a_swz(row, cp) * 16;
+        const int nbl = c >> 7, rem = c & 127;
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1) - n0 / 32;
+        b_vo[j] = (uint32_t)nb * (uint32_t)p.kb32 * 1024u + rem * 16;
+    }
+    auto sgpr_ptr = [](const uint8_t *q) {
+        const uint64_t v = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi
+                = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+    };
+    // next tile half to request: global base and this wave's LDS slot
+    const uint8_t *sa = sgpr_ptr(
+            p.A + (int64_t)bz * p.a_sb + (int64_t)m0 * p.lda);
+    const uint8_t *sb = sgpr_ptr(p.B + (int64_t)bz * p.b_sb
+            + (int64_t)(n0 / 32) * p.kb32 * 1024);
+    uint32_t dA = lds_base + wave * 1024;
+    uint32_t dB = dA + A_BYTES;
+#define QX_ADV_A() \
+    { \
+        sa += BK; \
+        dA = ((dA - lds_base + STAGE_BYTES) & (RING - 1)) + lds_base; \
+    }
+#define QX_ADV_B() \
+    { \
+        sb += 2048; \
+        dB = ((dB - lds_base + STAGE_BYTES) & (RING - 1)) + lds_base; \
+    }
+#define QX_FETCH(V, SB, SD) \
+    { \
+        QX_M0(SD, 0 * 4096); asm volatile("s_nop 0"); QX_DMA(V[0], SB); \
+        QX_M0(SD, 1 * 4096); asm volatile("s_nop 0"); QX_DMA(V[1], SB); \
+        QX_M0(SD, 2 * 4096); asm volatile("s_nop 0"); QX_DMA(V[2], SB); \
+        QX_M0(SD, 3 * 4096); asm volatile("s_nop 0"); QX_DMA(V[3], SB); \
+    }
+
+    // fragment addresses inside stage 0
+    const int arow = wm0 + (lane & 31);
+    const uint32_t a_off0
+            = lds_base + arow * BK + a_swz(arow, (lane >> 5)) * 16;
+    const uint32_t a_off1
+            = lds_base + arow * BK + a_swz(arow, 2 + (lane >> 5)) * 16;
+    const uint32_t b_off = lds_base + A_BYTES + ((wn0 >> 5) * 128 + lane) * 16;
+
+    v16i acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0;
+    v4i fa[2][4], fb[2][4];
+
+    // per-row source scales of the tile (1.0 when there are none)
+    {
+        float s = 1.f;
+        if (p.ep.src_scale.ptr)
+            s = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
+                    + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm];
+        ((float *)(lds + SS_OFF))[tid] = s;
+    }
+
+    // ---- prologue: tiles 0 and 1 and the A half of tile 2 ----
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_WV(12);
+    __syncthreads();
+    QX_RD_A(0, a_off0, 0);
+    QX_RD_B(0, b_off, 0, 0);
+    QX_RD_B(0, b_off, 0, 1);
+    QX_RD_B(0, b_off, 0, 2);
+    QX_RD_B(0, b_off, 0, 3);
+    QX_RD_A(0, a_off0, 1);
+    QX_RD_A(0, a_off0, 2);
+    QX_RD_A(0, a_off0, 3);
+    uint32_t st = 0; // ring offset of the tile whose first half was started
+    {
+        const uint32_t va1 = a_off1, vb = b_off;
+        QX_SUB_D(0, 1, va1, vb, 1, b_vo, sb, dB) // B half of tile 2
+        QX_ADV_B();
+    }
+    // k-step kt: second half of tile kt-1 (requesting the A half of tile
+    // kt+2), then first half of tile kt (requesting the B half of tile kt+2)
+    for (int kt = 1; kt <= KT - 3; kt++) {
+        const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
+        const uint32_t van = a_off0 + stn, vbn = b_off + stn,
+                       va1 = a_off1 + stn;
+        QX_WV(8); // tile kt has landed
+        __builtin_amdgcn_s_barrier();
+        QX_SUB_D(1, 0, van, vbn, 0, a_vo, sa, dA)
+        QX_ADV_A();
+        QX_SUB_D(0, 1, va1, vbn, 1, b_vo, sb, dB)
+        QX_ADV_B();
+        st = stn;
+    }
+#pragma unroll 1
+    for (int kt = KT - 2; kt <= KT - 1; kt++) {
+        const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
+        const uint32_t van = a_off0 + stn, vbn = b_off + stn,
+                       va1 = a_off1 + stn;
+        QX_WV(0);
+        __builtin_amdgcn_s_barrier();
+        QX_SUB(1, 0, van, vbn, 0, , , , )
+        QX_SUB(0, 1, va1, vbn, 1, , , , )
+        st = stn;
+    }
+    QX_SUB_LAST(1)
+    __syncthreads();
+
+    // ---- epilogue ----
+    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
+    // column l%32 of its 32x32 fragment. The wave tile goes through LDS in two
+    // halves of 64 rows x 128 columns (the ring is free now, every wave takes a
+    // quarter of it), straight from the accumulator registers, and comes back
+    // row-wise, 4 neighbouring columns per lane, so that the arithmetic exists
+    // once per half and every store is a dense vector. A wave reads back only
+    // what it wrote itself: LDS executes a wave's instructions in order, no
+    // barrier is involved.
+    const epilogue_t &ep = p.ep;
+    const uint32_t stg_w = lds_base + wave * STG_WAVE
+            + (4 * (lane >> 5) * 128 + (lane & 31)) * 4;
+    const int *const stg_r = (const int *)lds + wave * (STG_WAVE / 4);
+    const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
+    const int ecol = (lane & 31) * 4;
+    const int en = n0 + wn0 + ecol;
+    const int envalid = min(4, p.N - en);
+    const bool has_ss = ep.src_scale.ptr != nullptr;
+    const bool has_ws = ep.wei_scale.ptr != nullptr;
+    const bool to_bf16 = ep.dst.dt == dt_bf16;
+    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
+    int cs4[4] = {0, 0, 0, 0};
+    {
+        int comp = 0;
+        if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < envalid) {
+                if (has_ws)
+                    ws4[i] = ((const float *)ep.wei_scale.ptr)[bz * ep.wei_scale.sb
+                            + (int64_t)(en + i) * ep.wei_scale.sn];
+                if (comp != 0 && p.colsum)
+                    cs4[i] = comp
+                            * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
+            }
+    }
+    // bf16 results: the reference conversion maps f32 subnormals to +-0
+    // (src/common/bfloat16.cpp:22-56). With single-precision denormals flushed
+    // for the rest of the wave's life, the last multiply of the chain (or the
+    // packed conversion's input stage) produces that zero and
+    // v_cvt_pk_bf16_f32 does the round-to-nearest-even.
+    if (to_bf16) __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
+    static_for<2>([&](auto H) {
+        constexpr int h = decltype(H)::value;
+#pragma unroll
+        for (int i2 = 0; i2 < 2; i2++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
+                                 "a"(acc[2 * h + i2][j][r]),
+                                 "n"(((i2 * 32 + 8 * (r / 4) + (r % 4)) * 128
+                                             + j * 32)
+                                         * 4)
+                                 : "memory");
+#pragma unroll 2
+        for (int it = 0; it < 32; it++) {
+            const int row = it * 2 + (lane >> 5);
+            const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
+            const int lrow = h * 64 + row;
+            const int m = m0 + wm0 + lrow;
+            const float ss = ssl[lrow];
+            if (m < p.M && envalid > 0) {
+                float v[4];
+                v[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
+                v[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
+                v[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
+                v[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+                if (to_bf16 && envalid == 4)
+                    epilogue_fast4_bf16(ep, v, has_ss, ss, has_ws, ws4, bz, m, en);
+                else
+                    epilogue_fast4(ep, v, has_ss, ss, has_ws, ws4, bz, m, en,
+                            envalid);
+            }
+        }
+    });
+}
+
+static void launch_b8x(const gemm_params_t &p, hipStream_t stream) {
+    using namespace b8x;
+    gemm_params_t q = p;
+    q.tiles_m = (p.M + BM - 1) / BM;
+    q.tiles_n = (p.N + BN - 1) / BN;
+    const int ntiles = q.tiles_m * q.tiles_n;
+    const int grid_x = ((ntiles + 7) / 8) * 8;
+    auto kern = gemm_b8x_kernel;
+    static bool attr_done = false;
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void *)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(NT), LDS_TOTAL,
+            stream, q);
+}
+
+// Problems the kernel takes: s8 sources, K a multiple of 64 with at least 4
+// k-steps, a straight-line epilogue, 32-bit addressable tiles, and enough
+// 256 x 256 tiles to occupy the chip.
+bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
+    if (f8 || p.a_is_u8 || p.ep.fast == EP_FAST_NONE) return false;
+    if (p.K % 64 != 0 || p.K < 4 * 64) return false;
+    if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;
+    if ((int64_t)8 * p.kb32 * 1024 >= ((int64_t)1 << 32)) return false;
+    return true;
+}
+
+void launch_gemm_b8x(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(p, stream);
+}
+
+} // namespace qmm
