@@ -268,6 +268,76 @@ def test_mfma_int8_against_literal_v38_reference(ctx):
     assert_f32_close(got, want, rel=1e-5, scale=term_scale(p), what="literal")
 
 
+# ---------------------------------------------------------------------------
+# the 256 x 256 tile kernel of mfma_b8 (picked by itself only for large problems):
+# forced here so that edge tiles, every straight-line epilogue and the bf16
+# subnormal rule are checked at sizes the oracle finishes quickly
+@pytest.fixture
+def tile256():
+    from onednn_amd import _capi
+    _capi.lib().qmm_set_gemm_variant(6)
+    yield
+    _capi.lib().qmm_set_gemm_variant(0)
+
+
+def _tiny_scale_problem():
+    p = int8_linear(256, 256, 256, 76, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, src_scale=1e-30)
+    # |acc| <= 256 * 127 * 127, so acc * 1e-30 * 3e-15 spans f32 subnormals and normals
+    p.scales["wei"] = (2, dt.f32, None, rnd(76).uniform(1e-15, 3e-15, 256))
+    return p
+
+
+TILE256_CASES = {
+    "edges_per_token_bf16": (lambda: int8_linear(300, 256, 502, 71, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True), True),
+    "src_zp_relu_f32": (lambda: int8_linear(260, 320, 384, 72, src_dt=dt.s8, dst_dt=dt.f32, src_zp=5,
+                                            post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.1}]), True),
+    "swish_bf16_full_tiles": (lambda: int8_linear(512, 512, 512, 73, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True,
+                                                  post_ops=[{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]), False),
+    "swish_f32_edges": (lambda: int8_linear(130, 256, 250, 74, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None,
+                                            post_ops=[{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]), False),
+    "plain_f32_batched": (lambda: int8_linear(256, 256, 256, 75, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, batch=(2,)), True),
+    "bf16_subnormal_results_are_zero": (_tiny_scale_problem, True),
+}
+
+
+@pytest.mark.parametrize("name", sorted(TILE256_CASES))
+def test_mfma_int8_tile256_kernel(ctx, tile256, name):
+    eng, strm = ctx
+    say("mfma_b8 256x256 kernel %s" % name)
+    build, exact = TILE256_CASES[name]
+    p = build()
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    want = p.run_oracle()
+    if exact:
+        assert_bit_exact(got, want, name)
+    elif p.dst.dt == dt.bf16:
+        assert_bf16_within_1ulp(got, want, name, abs_slack=1e-30)  # device exp2/rcp vs libm expf
+    else:
+        M, N = p.dst.dims[-2:]
+        assert_f32_close(got.view(np.float32).reshape(-1, N), want.view(np.float32).reshape(-1, N),
+                         rel=1e-5, scale=np.abs(want.view(np.float32).reshape(-1, N)) + 1e-30, what=name)
+
+
+def test_mfma_int8_tile256_binary_add_and_sum(ctx, tile256):
+    eng, strm = ctx
+    r = rnd(77)
+    M, K, N = 300, 256, 260
+    for dd in (dt.f32, dt.bf16):
+        say("mfma_b8 256x256 kernel binary add / sum, dst %s" % dd)
+        s = np.clip(np.rint(r.standard_normal((M, K)) * 32), -127, 127)
+        w = r.integers(-127, 128, (K, N))
+        sc = {"src": (0, dt.f32, None, [0.01]), "wei": (2, dt.f32, None, r.uniform(0.001, 0.01, N))}
+        add = Problem(TensorSpec(dt.s8, [M, K], None, s), TensorSpec(dt.s8, [K, N], None, w), TensorSpec(dd, [M, N]),
+                      scales=sc, post_ops=[{"kind": "binary", "alg": A.binary_add,
+                                            "src1": TensorSpec(dt.f32, [M, N], None, r.standard_normal((M, N)).astype(np.float32))}])
+        assert_bit_exact(add.run_gpu(eng, strm, weights_any=True), add.run_oracle(), "binary add")
+        acc = Problem(TensorSpec(dt.s8, [M, K], None, s), TensorSpec(dt.s8, [K, N], None, w),
+                      TensorSpec(dd, [M, N], None, r.standard_normal((M, N)).astype(np.float32)),
+                      scales=sc, post_ops=[{"kind": "sum", "scale": 1.0}])
+        assert_bit_exact(acc.run_gpu(eng, strm, weights_any=True), acc.run_oracle(), "sum")
+
+
 def test_mfma_batched_scores_with_mask(ctx):
     eng, strm = ctx
     say("mfma_b8 batched scores (config 4 shape, fewer heads) + binary add mask, K^T weights view")
