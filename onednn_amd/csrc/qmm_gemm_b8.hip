@@ -413,7 +413,7 @@ void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);
 void launch_gemm_b8_v2(const gemm_params_t &p, bool f8, hipStream_t stream);
 // 256 x 256 tile kernel with the hand-ordered main loop (qmm_gemm_b8x.hip)
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8);
-void launch_gemm_b8x(const gemm_params_t &p, hipStream_t stream);
+void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream);
 
 // variant: 0 = heuristic; others pick a tile configuration explicitly (used by
 // the tuning sweep; 6 = the 256 x 256 kernel where it applies)
@@ -424,7 +424,7 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
             * p.batch;
     if ((variant == 6 || (variant == 0 && tiles256 >= 192))
             && gemm_b8x_eligible(p, f8)) {
-        launch_gemm_b8x(p, stream);
+        launch_gemm_b8x(p, f8, stream);
         return;
     }
     if (variant == 6) variant = 0;

@@ -207,7 +207,7 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 // Epilogue of 64 staged rows when the wave's 128 x 128 tile lies fully inside
 // the matrix and the dst rows are vector-aligned: no per-lane conditions, so
 // the rows pipeline. FAST is the recognised epilogue shape, BF16 the dst type.
-template <int FAST, bool BF16>
+template <int FAST, bool BF16, bool F8>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const float (&ws4)[4],
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
@@ -224,10 +224,17 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float ss = ssl[row];
         const int64_t m = m_first + row;
         float d[4];
-        d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
-        d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
-        d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
-        d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+        if constexpr (F8) { // f32 accumulators, staged as bits
+            d[0] = u2f((uint32_t)t.x);
+            d[1] = u2f((uint32_t)t.y);
+            d[2] = u2f((uint32_t)t.z);
+            d[3] = u2f((uint32_t)t.w);
+        } else {
+            d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
+            d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
+            d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
+            d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+        }
         // absent scales are 1.0 (exact)
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -281,6 +288,127 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
                     = make_float4(d[0], d[1], d[2], d[3]);
         }
     }
+}
+
+// Epilogue of one 256 x 256 block tile, shared by the int8 and fp8 kernels.
+template <bool F8, typename AccT>
+QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
+        uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
+        int wm0, int wn0, int bz) {
+    using namespace b8x;
+    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
+    // column l%32 of its 32x32 fragment. The wave tile goes through LDS in two
+    // halves of 64 rows x 128 columns (the ring is free now, every wave takes a
+    // quarter of it), straight from the accumulator registers, and comes back
+    // row-wise, 4 neighbouring columns per lane, so that the arithmetic exists
+    // once per half and every store is a dense vector. A wave reads back only
+    // what it wrote itself: LDS executes a wave's instructions in order, no
+    // barrier is involved.
+    const epilogue_t &ep = p.ep;
+    const uint32_t stg_w = lds_base + wave * STG_WAVE
+            + (4 * (lane >> 5) * 128 + (lane & 31)) * 4;
+    const int *const stg_r = (const int *)lds + wave * (STG_WAVE / 4);
+    const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
+    const int ecol = (lane & 31) * 4;
+    const int en = n0 + wn0 + ecol;
+    const int envalid = min(4, p.N - en);
+    const bool has_ss = ep.src_scale.ptr != nullptr;
+    const bool has_ws = ep.wei_scale.ptr != nullptr;
+    const bool to_bf16 = ep.dst.dt == dt_bf16;
+    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
+    int cs4[4] = {0, 0, 0, 0};
+    {
+        int comp = 0;
+        if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < envalid) {
+                if (has_ws)
+                    ws4[i] = ((const float *)ep.wei_scale.ptr)[bz * ep.wei_scale.sb
+                            + (int64_t)(en + i) * ep.wei_scale.sn];
+                if (comp != 0 && p.colsum)
+                    cs4[i] = comp
+                            * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
+            }
+    }
+    // bf16 results: the reference conversion maps f32 subnormals to +-0
+    // (src/common/bfloat16.cpp:22-56). With single-precision denormals flushed
+    // for the rest of the wave's life, the last multiply of the chain (or the
+    // packed conversion's input stage) produces that zero and
+    // v_cvt_pk_bf16_f32 does the round-to-nearest-even.
+    if (to_bf16) __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
+    // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
+    // operand's rows) aligned for vector access
+    bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
+            && (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
+            && ((uintptr_t)ep.dst.ptr & 15) == 0;
+    if (ep.fast == EP_FAST_ADD)
+        full = full && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
+                && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;
+    static_for<2>([&](auto H) {
+        constexpr int h = decltype(H)::value;
+#pragma unroll
+        for (int i2 = 0; i2 < 2; i2++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
+                                 "a"(acc[2 * h + i2][j][r]),
+                                 "n"(((i2 * 32 + 8 * (r / 4) + (r % 4)) * 128
+                                             + j * 32)
+                                         * 4)
+                                 : "memory");
+        if (full) {
+            const int64_t m_first = m0 + wm0 + h * 64;
+            const float *const ssh = ssl + h * 64;
+#define QX_EP_CASE(F) \
+    case F: \
+        if (to_bf16) \
+            ep_rows_full<F, true, F8>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
+        else \
+            ep_rows_full<F, false, F8>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
+        break;
+            switch (ep.fast) {
+                QX_EP_CASE(EP_FAST_PLAIN)
+                QX_EP_CASE(EP_FAST_RELU)
+                QX_EP_CASE(EP_FAST_SWISH)
+                QX_EP_CASE(EP_FAST_ADD)
+                QX_EP_CASE(EP_FAST_SUM)
+                default: break;
+            }
+#undef QX_EP_CASE
+        } else {
+#pragma unroll 1
+            for (int it = 0; it < 32; it++) {
+                const int row = it * 2 + (lane >> 5);
+                const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
+                const int lrow = h * 64 + row;
+                const int m = m0 + wm0 + lrow;
+                const float ss = ssl[lrow];
+                if (m < p.M && envalid > 0) {
+                    float v[4];
+                    if constexpr (F8) {
+                        v[0] = u2f((uint32_t)t.x);
+                        v[1] = u2f((uint32_t)t.y);
+                        v[2] = u2f((uint32_t)t.z);
+                        v[3] = u2f((uint32_t)t.w);
+                    } else {
+                        v[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
+                        v[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
+                        v[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
+                        v[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+                    }
+                    if (to_bf16 && envalid == 4)
+                        epilogue_fast4_bf16(
+                                ep, v, has_ss, ss, has_ws, ws4, bz, m, en);
+                    else
+                        epilogue_fast4(ep, v, has_ss, ss, has_ws, ws4, bz, m,
+                                en, envalid);
+                }
+            }
+        }
+    });
 }
 
 __global__ void __launch_bounds__(b8x::NT, 1)
@@ -440,123 +568,203 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QX_SUB_LAST(1)
     __syncthreads();
 
-    // ---- epilogue ----
-    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
-    // column l%32 of its 32x32 fragment. The wave tile goes through LDS in two
-    // halves of 64 rows x 128 columns (the ring is free now, every wave takes a
-    // quarter of it), straight from the accumulator registers, and comes back
-    // row-wise, 4 neighbouring columns per lane, so that the arithmetic exists
-    // once per half and every store is a dense vector. A wave reads back only
-    // what it wrote itself: LDS executes a wave's instructions in order, no
-    // barrier is involved.
-    const epilogue_t &ep = p.ep;
-    const uint32_t stg_w = lds_base + wave * STG_WAVE
-            + (4 * (lane >> 5) * 128 + (lane & 31)) * 4;
-    const int *const stg_r = (const int *)lds + wave * (STG_WAVE / 4);
-    const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
-    const int ecol = (lane & 31) * 4;
-    const int en = n0 + wn0 + ecol;
-    const int envalid = min(4, p.N - en);
-    const bool has_ss = ep.src_scale.ptr != nullptr;
-    const bool has_ws = ep.wei_scale.ptr != nullptr;
-    const bool to_bf16 = ep.dst.dt == dt_bf16;
-    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
-    int cs4[4] = {0, 0, 0, 0};
-    {
-        int comp = 0;
-        if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < envalid) {
-                if (has_ws)
-                    ws4[i] = ((const float *)ep.wei_scale.ptr)[bz * ep.wei_scale.sb
-                            + (int64_t)(en + i) * ep.wei_scale.sn];
-                if (comp != 0 && p.colsum)
-                    cs4[i] = comp
-                            * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
-            }
-    }
-    // bf16 results: the reference conversion maps f32 subnormals to +-0
-    // (src/common/bfloat16.cpp:22-56). With single-precision denormals flushed
-    // for the rest of the wave's life, the last multiply of the chain (or the
-    // packed conversion's input stage) produces that zero and
-    // v_cvt_pk_bf16_f32 does the round-to-nearest-even.
-    if (to_bf16) __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
-    // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
-    // operand's rows) aligned for vector access
-    bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
-            && (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
-            && ((uintptr_t)ep.dst.ptr & 15) == 0;
-    if (ep.fast == EP_FAST_ADD)
-        full = full && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
-                && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;
-    static_for<2>([&](auto H) {
-        constexpr int h = decltype(H)::value;
-#pragma unroll
-        for (int i2 = 0; i2 < 2; i2++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
-                                 "a"(acc[2 * h + i2][j][r]),
-                                 "n"(((i2 * 32 + 8 * (r / 4) + (r % 4)) * 128
-                                             + j * 32)
-                                         * 4)
-                                 : "memory");
-        if (full) {
-            const int64_t m_first = m0 + wm0 + h * 64;
-            const float *const ssh = ssl + h * 64;
-#define QX_EP_CASE(F) \
-    case F: \
-        if (to_bf16) \
-            ep_rows_full<F, true>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
-        else \
-            ep_rows_full<F, false>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
-        break;
-            switch (ep.fast) {
-                QX_EP_CASE(EP_FAST_PLAIN)
-                QX_EP_CASE(EP_FAST_RELU)
-                QX_EP_CASE(EP_FAST_SWISH)
-                QX_EP_CASE(EP_FAST_ADD)
-                QX_EP_CASE(EP_FAST_SUM)
-                default: break;
-            }
-#undef QX_EP_CASE
-        } else {
-#pragma unroll 1
-            for (int it = 0; it < 32; it++) {
-                const int row = it * 2 + (lane >> 5);
-                const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
-                const int lrow = h * 64 + row;
-                const int m = m0 + wm0 + lrow;
-                const float ss = ssl[lrow];
-                if (m < p.M && envalid > 0) {
-                    float v[4];
-                    v[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
-                    v[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
-                    v[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
-                    v[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
-                    if (to_bf16 && envalid == 4)
-                        epilogue_fast4_bf16(
-                                ep, v, has_ss, ss, has_ws, ws4, bz, m, en);
-                    else
-                        epilogue_fast4(ep, v, has_ss, ss, has_ws, ws4, bz, m,
-                                en, envalid);
-                }
-            }
-        }
-    });
+    tile_epilogue<false>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
 }
 
-static void launch_b8x(const gemm_params_t &p, hipStream_t stream) {
+// ---- fp8 (e4m3 x e4m3 -> f32) ----------------------------------------------
+// Same tile, ring and epilogue. v_mfma_f32_32x32x64_f8f6f4 consumes a whole
+// 64-k tile per instruction (64 cycles), so a k-step is one group of 16 MFMAs
+// on the fragments read during the previous k-step; the 16 fragment reads of
+// the next tile and the 8 direct loads two tiles further on are spread between
+// them. The fragment reads are ordinary LDS loads here (the compiler counts
+// their waits itself; it does not see the direct loads, so it adds no vmcnt);
+// the scheduling barriers keep everything where it is written. An operand is
+// the pair (k 0..31 fragment, k 32..63 fragment) of the int8 path, i.e. lane
+// half h holds k 16h..16h+15 and 32+16h..32+16h+15 -- the same permutation on
+// both operands.
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define QF_MF(i, j, cb) \
+    { \
+        QX_SB(); \
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4( \
+                __builtin_shufflevector(fa[cb][0][i], fa[cb][1][i], 0, 1, 2, \
+                        3, 4, 5, 6, 7), \
+                __builtin_shufflevector(fb[cb][0][j], fb[cb][1][j], 0, 1, 2, \
+                        3, 4, 5, 6, 7), \
+                acc[i][j], 0, 0, 0, 0, 0, 0); \
+        QX_SB(); \
+    }
+#define QF_RA(nb, h, i) \
+    { \
+        fa[nb][h][i] = *(const v4i *)(ldsn + (h ? a_rel1 : a_rel0) + (i)*2048); \
+        QX_SB(); \
+    }
+#define QF_RB(nb, h, j) \
+    { \
+        fb[nb][h][j] = *(const v4i *)(ldsn + b_rel + ((j)*2 + (h)) * 1024); \
+        QX_SB(); \
+    }
+// one k-step: 16 MFMAs on buffer CB, the next tile's fragments into buffer NB
+// (order a0 b0 b1 b2 b3 a1 a2 a3, both halves each); D*: direct loads or empty
+#define QF_STEP(CB, NB, DA0, DA1, DA2, DA3, DA4, DB0, DB1, DB2, DB3, DB4) \
+    QF_MF(0, 0, CB); QF_RA(NB, 0, 0); QF_RA(NB, 1, 0); \
+    QF_MF(0, 1, CB); QF_RB(NB, 0, 0); QF_RB(NB, 1, 0); \
+    QF_MF(0, 2, CB); QF_RB(NB, 0, 1); QF_RB(NB, 1, 1); \
+    QF_MF(0, 3, CB); QF_RB(NB, 0, 2); QF_RB(NB, 1, 2); \
+    DA0; QF_MF(1, 0, CB); DA1; QF_RB(NB, 0, 3); \
+    QF_MF(1, 1, CB); DA2; QF_RB(NB, 1, 3); \
+    QF_MF(1, 2, CB); DA3; QF_RA(NB, 0, 1); \
+    QF_MF(1, 3, CB); DA4; QF_RA(NB, 1, 1); \
+    DB0; QF_MF(2, 0, CB); DB1; QF_RA(NB, 0, 2); \
+    QF_MF(2, 1, CB); DB2; QF_RA(NB, 1, 2); \
+    QF_MF(2, 2, CB); DB3; QF_RA(NB, 0, 3); \
+    QF_MF(2, 3, CB); DB4; QF_RA(NB, 1, 3); \
+    QF_MF(3, 0, CB); QF_MF(3, 1, CB); QF_MF(3, 2, CB); QF_MF(3, 3, CB);
+#define QF_STEP_D(CB, NB) \
+    QF_STEP(CB, NB, QX_D0(a_vo, sa, dA), QX_D1(a_vo, sa, dA), \
+            QX_D2(a_vo, sa, dA), QX_D3(a_vo, sa, dA), QX_D4(a_vo, sa, dA), \
+            QX_D0(b_vo, sb, dB), QX_D1(b_vo, sb, dB), QX_D2(b_vo, sb, dB), \
+            QX_D3(b_vo, sb, dB), QX_D4(b_vo, sb, dB))
+#define QF_STEP_ND(CB, NB) QF_STEP(CB, NB, , , , , , , , , , )
+#define QF_LAST(CB) \
+    QF_MF(0, 0, CB); QF_MF(0, 1, CB); QF_MF(0, 2, CB); QF_MF(0, 3, CB); \
+    QF_MF(1, 0, CB); QF_MF(1, 1, CB); QF_MF(1, 2, CB); QF_MF(1, 3, CB); \
+    QF_MF(2, 0, CB); QF_MF(2, 1, CB); QF_MF(2, 2, CB); QF_MF(2, 3, CB); \
+    QF_MF(3, 0, CB); QF_MF(3, 1, CB); QF_MF(3, 2, CB); QF_MF(3, 3, CB);
+
+__global__ void __launch_bounds__(b8x::NT, 1)
+gemm_f8x_kernel(const gemm_params_t p) {
+    using namespace b8x;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        lt = xcd * per + slot;
+        if (slot >= per || lt >= ntiles) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const int KT = p.K / BK; // host guarantees K % 128 == 0 and KT >= 6
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+
+    uint32_t a_vo[4], b_vo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tid + j * NT;
+        const int row = c >> 2, cp = c & 3;
+        const int gm = min(m0 + row, p.M - 1) - m0;
+        a_vo[j] = (uint32_t)gm * (uint32_t)p.lda + a_swz(row, cp) * 16;
+        const int nbl = c >> 7, rem = c & 127;
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1) - n0 / 32;
+        b_vo[j] = (uint32_t)nb * (uint32_t)p.kb32 * 1024u + rem * 16;
+    }
+    auto sgpr_ptr = [](const uint8_t *q) {
+        const uint64_t v = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi
+                = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+    };
+    const uint8_t *sa = sgpr_ptr(
+            p.A + (int64_t)bz * p.a_sb + (int64_t)m0 * p.lda);
+    const uint8_t *sb = sgpr_ptr(p.B + (int64_t)bz * p.b_sb
+            + (int64_t)(n0 / 32) * p.kb32 * 1024);
+    uint32_t dA = lds_base + wave * 1024;
+    uint32_t dB = dA + A_BYTES;
+
+    // fragment offsets inside a stage
+    const int arow = wm0 + (lane & 31);
+    const int a_rel0 = arow * BK + a_swz(arow, (lane >> 5)) * 16;
+    const int a_rel1 = arow * BK + a_swz(arow, 2 + (lane >> 5)) * 16;
+    const int b_rel = A_BYTES + ((wn0 >> 5) * 128 + lane) * 16;
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.f;
+    v4i fa[2][2][4], fb[2][2][4];
+
+    {
+        float s = 1.f;
+        if (p.ep.src_scale.ptr)
+            s = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
+                    + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm];
+        ((float *)(lds + SS_OFF))[tid] = s;
+    }
+
+    // ---- prologue: tiles 0, 1, 2 requested; tile 0's fragments read ----
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_WV(16);
+    __syncthreads();
+    uint32_t st = 0; // ring offset of the tile whose fragments are read next
+    {
+        const uint8_t *ldsn = lds;
+        QX_SB();
+        QF_RA(0, 0, 0); QF_RA(0, 1, 0);
+        QF_RB(0, 0, 0); QF_RB(0, 1, 0); QF_RB(0, 0, 1); QF_RB(0, 1, 1);
+        QF_RB(0, 0, 2); QF_RB(0, 1, 2); QF_RB(0, 0, 3); QF_RB(0, 1, 3);
+        QF_RA(0, 0, 1); QF_RA(0, 1, 1); QF_RA(0, 0, 2); QF_RA(0, 1, 2);
+        QF_RA(0, 0, 3); QF_RA(0, 1, 3);
+    }
+    // k-step kt: multiplies tile kt-1 (buffer (kt-1)&1), reads tile kt's
+    // fragments, requests tile kt+2
+#define QF_KSTEP(WAITV, BODY) \
+    { \
+        st = (st + STAGE_BYTES) & (RING - 1); \
+        const uint8_t *ldsn = lds + st; \
+        QX_WV(WAITV); \
+        __builtin_amdgcn_s_barrier(); \
+        QX_SB(); \
+        BODY \
+    }
+    for (int kt = 1; kt <= KT - 4; kt += 2) {
+        QF_KSTEP(8, QF_STEP_D(0, 1) QX_ADV_A(); QX_ADV_B();)
+        QF_KSTEP(8, QF_STEP_D(1, 0) QX_ADV_A(); QX_ADV_B();)
+    }
+    QF_KSTEP(8, QF_STEP_D(0, 1)) // kt = KT-3: requests tile KT-1
+    QF_KSTEP(0, QF_STEP_ND(1, 0)) // kt = KT-2
+    QF_KSTEP(0, QF_STEP_ND(0, 1)) // kt = KT-1
+    QF_LAST(1)
+    __syncthreads();
+
+    tile_epilogue<true>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+}
+
+template <typename K>
+static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
     using namespace b8x;
     gemm_params_t q = p;
     q.tiles_m = (p.M + BM - 1) / BM;
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ((ntiles + 7) / 8) * 8;
-    auto kern = gemm_b8x_kernel;
     static bool attr_done = false;
     if (!attr_done) {
         (void)hipFuncSetAttribute((const void *)kern,
@@ -567,19 +775,23 @@ static void launch_b8x(const gemm_params_t &p, hipStream_t stream) {
             stream, q);
 }
 
-// Problems the kernel takes: s8 sources, K a multiple of 64 with at least 4
-// k-steps, a straight-line epilogue, 32-bit addressable tiles, and enough
+// Problems the kernels take: s8 or fp8 sources, K a multiple of 64 (fp8: 128)
+// with at least 4 (6) k-steps, a straight-line epilogue, 32-bit addressable tiles, and enough
 // 256 x 256 tiles to occupy the chip.
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
-    if (f8 || p.a_is_u8 || p.ep.fast == EP_FAST_NONE) return false;
+    if (p.a_is_u8 || p.ep.fast == EP_FAST_NONE) return false;
+    if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
     if (p.K % 64 != 0 || p.K < 4 * 64) return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;
     if ((int64_t)8 * p.kb32 * 1024 >= ((int64_t)1 << 32)) return false;
     return true;
 }
 
-void launch_gemm_b8x(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(p, stream);
+void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
+    if (f8)
+        launch_b8x(gemm_f8x_kernel, p, stream);
+    else
+        launch_b8x(gemm_b8x_kernel, p, stream);
 }
 
 } // namespace qmm

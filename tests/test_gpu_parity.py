@@ -319,6 +319,24 @@ def test_mfma_int8_tile256_kernel(ctx, tile256, name):
                          rel=1e-5, scale=np.abs(want.view(np.float32).reshape(-1, N)) + 1e-30, what=name)
 
 
+def test_mfma_fp8_tile256_kernel(ctx, tile256):
+    eng, strm = ctx
+    for (M, K, N, dd, with_sum) in ((256, 512, 256, dt.bf16, True), (300, 384, 260, dt.f32, False), (128, 1024, 512, dt.bf16, False)):
+        say("mfma_b8 256x256 fp8 kernel %dx%dx%d" % (M, K, N))
+        p = fp8_gemm(M, K, N, 78, dst_dt=dd, with_sum=with_sum)
+        got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+        assert pd.impl_info_str() == MFMA
+        want = p.run_oracle()
+        a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
+        if dd == dt.bf16:
+            # another summation order than the reference's k loop: 1 bf16 ulp, or the
+            # f32 bar (1e-5 of the summed magnitudes) where the result cancels
+            assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
+        else:
+            assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
+                             rel=1e-5, scale=a, what="fp8 f32")
+
+
 def test_mfma_int8_tile256_binary_add_and_sum(ctx, tile256):
     eng, strm = ctx
     r = rnd(77)
