@@ -26,6 +26,10 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 PEAK_INT8 = 5000.0  # TOP/s, dense MFMA int8 (published MI355X figure)
 PEAK_FP8 = 5000.0  # TFLOP/s, dense MFMA fp8
 PEAK_HBM = 8000.0  # GB/s
+# HBM bytes per launch of the config-2 kernel: rocprofv3 FETCH_SIZE and WRITE_SIZE
+# (KiB per dispatch), each scaled by what the same counter reads for a 1 GiB
+# device copy (--calibrate-copy): 188,820 KiB x 2.000 + 114,690 KiB x 1.000
+TRAFFIC_C2_BYTES = 386.7e6 + 117.4e6
 
 
 def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
@@ -47,12 +51,26 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="mfma_b8 tile configuration (0 = heuristic)")
     ap.add_argument("--no-extras", action="store_true", help="skip the decode / fp8 side measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=192, help="rows of config 2 timed on the CPU oracle")
+    ap.add_argument("--cpu-rows", type=int, default=640, help="rows of config 2 timed on the CPU oracle")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a 1 GiB device-to-device copy (reference point for the rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the path shards "
               "along N without any exchange, see DESIGN.md); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.calibrate_copy:
+        import torch
+        n = 1 << 30
+        a = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": n, "launches": 3}))
+        return
 
     import onednn_amd as dnnl
     from onednn_amd import _capi, hiprt, memory
@@ -117,8 +135,9 @@ def main():
                                "per-N weights scales, swish; weights prepacked via format_tag any",
                    "impl": pd.impl_info_str(), "tile_variant": args.variant},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TFLOP/s",
-                     "frac": round(kern_tops / PEAK_INT8, 4), "traffic": None,
-                     "kernel": "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
+                     "frac": round(kern_tops / PEAK_INT8, 4),
+                     "traffic": TRAFFIC_C2_BYTES if args.variant == 0 else None,
+                     "kernel": "gemm_b8x_kernel (int8, 256x256 tile)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }
 
