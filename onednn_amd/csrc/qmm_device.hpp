@@ -575,4 +575,90 @@ QMM_D void epilogue_fast4(const epilogue_t &ep, float (&d)[4], bool has_ss,
     }
 }
 
+// Straight-line epilogue of four neighbouring results of one row when nothing
+// has to be checked per lane: the four columns exist, dst (and a binary
+// operand) can be accessed as one vector. FAST is the recognised shape, BF16
+// the dst type. bf16 results are packed by v_cvt_pk_bf16_f32 (round to nearest
+// even); the caller runs with f32 denormals flushed (see
+// epilogue_flush_denormals), which reproduces the reference conversion's
+// subnormal -> +-0 (src/common/bfloat16.cpp:22-56). Absent scales are passed
+// as 1.0, which is exact.
+QMM_D void epilogue_flush_denormals() {
+    // MODE register, FP_DENORM field for single precision (bits 5:4) = flush
+    __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
+}
+
+template <int FAST, bool BF16>
+QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
+        const float (&ws4)[4], int64_t bz, int64_t m, int64_t en) {
+    const float alpha = FAST == EP_FAST_RELU || FAST == EP_FAST_SWISH
+            ? ep.po[0].alpha
+            : 0.f;
+    const float na = -alpha * 1.44269504088896340736f;
+    const float sum_scale = FAST == EP_FAST_SUM ? ep.po[0].scale : 0.f;
+    // absent scales are 1.0 (exact)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        d[i] = d[i] * ss * ws4[i];
+    const int64_t dst_off = bz * ep.dst.sb + m * ep.dst.sm + en;
+    if constexpr (FAST == EP_FAST_RELU) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = d[i] > 0 ? d[i] : d[i] * alpha;
+    } else if constexpr (FAST == EP_FAST_SWISH) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float e = __builtin_amdgcn_exp2f(d[i] * na);
+            d[i] = d[i] * __builtin_amdgcn_rcpf(1.0f + e);
+        }
+    } else if constexpr (FAST == EP_FAST_ADD) {
+        const float4 y = *(const float4 *)((const float *)ep.po[0].t.ptr
+                + bz * ep.po[0].t.sb + m * ep.po[0].t.sm + en);
+        d[0] += y.x;
+        d[1] += y.y;
+        d[2] += y.z;
+        d[3] += y.w;
+    } else if constexpr (FAST == EP_FAST_SUM) {
+        if constexpr (BF16) {
+            const uint2 o = *(const uint2 *)((const uint16_t *)ep.dst.ptr
+                    + dst_off);
+            d[0] += sum_scale * (u2f(o.x << 16) - 0.f);
+            d[1] += sum_scale * (u2f(o.x & 0xFFFF0000u) - 0.f);
+            d[2] += sum_scale * (u2f(o.y << 16) - 0.f);
+            d[3] += sum_scale * (u2f(o.y & 0xFFFF0000u) - 0.f);
+        } else {
+            const float4 o = *(const float4 *)((const float *)ep.dst.ptr
+                    + dst_off);
+            d[0] += sum_scale * (o.x - 0.f);
+            d[1] += sum_scale * (o.y - 0.f);
+            d[2] += sum_scale * (o.z - 0.f);
+            d[3] += sum_scale * (o.w - 0.f);
+        }
+    }
+    if constexpr (BF16) {
+        uint32_t h0, h1;
+        asm("v_cvt_pk_bf16_f32 %0, %1, %2"
+                : "=v"(h0)
+                : "v"(d[0]), "v"(d[1]));
+        asm("v_cvt_pk_bf16_f32 %0, %1, %2"
+                : "=v"(h1)
+                : "v"(d[2]), "v"(d[3]));
+        *(uint2 *)((uint16_t *)ep.dst.ptr + dst_off) = make_uint2(h0, h1);
+    } else {
+        *(float4 *)((float *)ep.dst.ptr + dst_off)
+                = make_float4(d[0], d[1], d[2], d[3]);
+    }
+}
+
+// wave-uniform test for epilogue_full4: dst rows (and a binary operand's)
+// aligned for vector access
+QMM_D bool epilogue_full4_ok(const epilogue_t &ep) {
+    bool ok = (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
+            && ((uintptr_t)ep.dst.ptr & 15) == 0;
+    if (ep.fast == EP_FAST_ADD)
+        ok = ok && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
+                && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;
+    return ok;
+}
+
 } // namespace qmm

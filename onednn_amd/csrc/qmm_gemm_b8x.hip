@@ -212,11 +212,6 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const float (&ws4)[4],
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
     const int ecol = (lane & 31) * 4;
-    const float alpha = FAST == EP_FAST_RELU || FAST == EP_FAST_SWISH
-            ? ep.po[0].alpha
-            : 0.f;
-    const float na = -alpha * 1.44269504088896340736f;
-    const float sum_scale = FAST == EP_FAST_SUM ? ep.po[0].scale : 0.f;
 #pragma unroll 8
     for (int it = 0; it < 32; it++) {
         const int row = it * 2 + (lane >> 5);
@@ -235,58 +230,7 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
             d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
             d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
         }
-        // absent scales are 1.0 (exact)
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            d[i] = d[i] * ss * ws4[i];
-        const int64_t dst_off = bz * ep.dst.sb + m * ep.dst.sm + en;
-        if constexpr (FAST == EP_FAST_RELU) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                d[i] = d[i] > 0 ? d[i] : d[i] * alpha;
-        } else if constexpr (FAST == EP_FAST_SWISH) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float e = __builtin_amdgcn_exp2f(d[i] * na);
-                d[i] = d[i] * __builtin_amdgcn_rcpf(1.0f + e);
-            }
-        } else if constexpr (FAST == EP_FAST_ADD) {
-            const float4 y = *(const float4 *)((const float *)ep.po[0].t.ptr
-                    + bz * ep.po[0].t.sb + m * ep.po[0].t.sm + en);
-            d[0] += y.x;
-            d[1] += y.y;
-            d[2] += y.z;
-            d[3] += y.w;
-        } else if constexpr (FAST == EP_FAST_SUM) {
-            if constexpr (BF16) {
-                const uint2 o = *(const uint2 *)((const uint16_t *)ep.dst.ptr
-                        + dst_off);
-                d[0] += sum_scale * (u2f(o.x << 16) - 0.f);
-                d[1] += sum_scale * (u2f(o.x & 0xFFFF0000u) - 0.f);
-                d[2] += sum_scale * (u2f(o.y << 16) - 0.f);
-                d[3] += sum_scale * (u2f(o.y & 0xFFFF0000u) - 0.f);
-            } else {
-                const float4 o = *(const float4 *)((const float *)ep.dst.ptr
-                        + dst_off);
-                d[0] += sum_scale * (o.x - 0.f);
-                d[1] += sum_scale * (o.y - 0.f);
-                d[2] += sum_scale * (o.z - 0.f);
-                d[3] += sum_scale * (o.w - 0.f);
-            }
-        }
-        if constexpr (BF16) {
-            uint32_t h0, h1;
-            asm("v_cvt_pk_bf16_f32 %0, %1, %2"
-                    : "=v"(h0)
-                    : "v"(d[0]), "v"(d[1]));
-            asm("v_cvt_pk_bf16_f32 %0, %1, %2"
-                    : "=v"(h1)
-                    : "v"(d[2]), "v"(d[3]));
-            *(uint2 *)((uint16_t *)ep.dst.ptr + dst_off) = make_uint2(h0, h1);
-        } else {
-            *(float4 *)((float *)ep.dst.ptr + dst_off)
-                    = make_float4(d[0], d[1], d[2], d[3]);
-        }
+        epilogue_full4<FAST, BF16>(ep, d, ss, ws4, bz, m, en);
     }
 }
 
@@ -336,15 +280,11 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     // for the rest of the wave's life, the last multiply of the chain (or the
     // packed conversion's input stage) produces that zero and
     // v_cvt_pk_bf16_f32 does the round-to-nearest-even.
-    if (to_bf16) __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
+    if (to_bf16) epilogue_flush_denormals();
     // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
     // operand's rows) aligned for vector access
-    bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
-            && (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
-            && ((uintptr_t)ep.dst.ptr & 15) == 0;
-    if (ep.fast == EP_FAST_ADD)
-        full = full && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
-                && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;
+    const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
+            && epilogue_full4_ok(ep);
     static_for<2>([&](auto H) {
         constexpr int h = decltype(H)::value;
 #pragma unroll
