@@ -326,10 +326,6 @@ gemm_b8_kernel(const gemm_params_t p) {
                 ws4[i] = ((const float *)p.ep.wei_scale.ptr)[bz * p.ep.wei_scale.sb
                         + (int64_t)(en + i) * p.ep.wei_scale.sn];
     }
-    const bool to_bf16 = p.ep.dst.dt == dt_bf16;
-    const bool full = p.ep.fast != EP_FAST_NONE && m0 + wm0 + WM <= p.M
-            && n0 + wn0 + WN <= p.N && epilogue_full4_ok(p.ep);
-    if (full && to_bf16) epilogue_flush_denormals();
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
 #pragma unroll
@@ -346,60 +342,22 @@ gemm_b8_kernel(const gemm_params_t p) {
                 stg[row * WN + j * 32 + (lane & 31)] = v;
             }
         }
-        if (full) {
-            // whole wave tile inside the matrix, vector-aligned rows: no
-            // per-lane conditions, the rows of the band pipeline
-            const int64_t m_first = m0 + wm0 + i * 32;
-            auto rows = [&](auto FK, auto BF) {
-                constexpr int FAST = decltype(FK)::value;
-                constexpr bool BF16 = decltype(BF)::value;
-#pragma unroll
-                for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
-                    const int row = it * ROWS_PER_IT + lane / (WN / 4);
-                    const float4 t = *(const float4 *)&stg[row * WN + ecol];
-                    const int64_t m = m_first + row;
+#pragma unroll 1
+        for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+            const int row = it * ROWS_PER_IT + lane / (WN / 4);
+            const float4 t = *(const float4 *)&stg[row * WN + ecol];
+            const int m = m0 + wm0 + i * 32 + row;
+            if (m < p.M && en < p.N) {
+                float v[4] = {t.x, t.y, t.z, t.w};
+                if (p.ep.fast != EP_FAST_NONE) {
                     float ss = 1.f;
                     if (has_ss)
                         ss = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
                                 + m * p.ep.src_scale.sm];
-                    float v[4] = {t.x, t.y, t.z, t.w};
-                    epilogue_full4<FAST, BF16>(p.ep, v, ss, ws4, bz, m, en);
-                }
-            };
-#define QMM_EP_CASE(F) \
-    case F: \
-        if (to_bf16) \
-            rows(std::integral_constant<int, F> {}, std::true_type {}); \
-        else \
-            rows(std::integral_constant<int, F> {}, std::false_type {}); \
-        break;
-            switch (p.ep.fast) {
-                QMM_EP_CASE(EP_FAST_PLAIN)
-                QMM_EP_CASE(EP_FAST_RELU)
-                QMM_EP_CASE(EP_FAST_SWISH)
-                QMM_EP_CASE(EP_FAST_ADD)
-                QMM_EP_CASE(EP_FAST_SUM)
-                default: break;
-            }
-#undef QMM_EP_CASE
-        } else {
-#pragma unroll 1
-            for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
-                const int row = it * ROWS_PER_IT + lane / (WN / 4);
-                const float4 t = *(const float4 *)&stg[row * WN + ecol];
-                const int m = m0 + wm0 + i * 32 + row;
-                if (m < p.M && en < p.N) {
-                    float v[4] = {t.x, t.y, t.z, t.w};
-                    if (p.ep.fast != EP_FAST_NONE) {
-                        float ss = 1.f;
-                        if (has_ss)
-                            ss = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
-                                    + m * p.ep.src_scale.sm];
-                        epilogue_fast4(
-                                p.ep, v, has_ss, ss, has_ws, ws4, bz, m, en, envalid);
-                    } else
-                        epilogue_apply_store4(p.ep, v, bz, m, en, envalid);
-                }
+                    epilogue_fast4(
+                            p.ep, v, has_ss, ss, has_ws, ws4, bz, m, en, envalid);
+                } else
+                    epilogue_apply_store4(p.ep, v, bz, m, en, envalid);
             }
         }
     });
