@@ -262,7 +262,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     float ws4[4] = {1.f, 1.f, 1.f, 1.f};
     int cs4[4] = {0, 0, 0, 0};
     {
-        int comp = 0;
+        int comp = p.a_is_u8 ? 128 : 0;
         if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -351,6 +351,12 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     });
 }
 
+// SHORTK: K of at most 4 k-steps (attention-score shapes): all of K fits the
+// LDS ring, so every tile is requested at once and multiplied after a single
+// wait; these problems are bound by the dst stream and share the epilogue.
+// u8 sources (top bits flipped after the fragment read, +128 * colsum in the
+// epilogue) are taken on that path only.
+template <bool SHORTK>
 __global__ void __launch_bounds__(b8x::NT, 1)
 gemm_b8x_kernel(const gemm_params_t p) {
     using namespace b8x;
@@ -458,55 +464,92 @@ gemm_b8x_kernel(const gemm_params_t p) {
         ((float *)(lds + SS_OFF))[tid] = s;
     }
 
-    // ---- prologue: tiles 0 and 1 and the A half of tile 2 ----
-    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
-    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
-    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
-    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
-    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
-    QX_WV(12);
-    __syncthreads();
-    QX_RD_A(0, a_off0, 0);
-    QX_RD_B(0, b_off, 0, 0);
-    QX_RD_B(0, b_off, 0, 1);
-    QX_RD_B(0, b_off, 0, 2);
-    QX_RD_B(0, b_off, 0, 3);
-    QX_RD_A(0, a_off0, 1);
-    QX_RD_A(0, a_off0, 2);
-    QX_RD_A(0, a_off0, 3);
-    uint32_t st = 0; // ring offset of the tile whose first half was started
-    {
-        const uint32_t va1 = a_off1, vb = b_off;
-        QX_SUB_D(0, 1, va1, vb, 1, b_vo, sb, dB) // B half of tile 2
-        QX_ADV_B();
-    }
-    // k-step kt: second half of tile kt-1 (requesting the A half of tile
-    // kt+2), then first half of tile kt (requesting the B half of tile kt+2)
-    for (int kt = 1; kt <= KT - 3; kt++) {
-        const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
-        const uint32_t van = a_off0 + stn, vbn = b_off + stn,
-                       va1 = a_off1 + stn;
-        QX_WV(8); // tile kt has landed
-        __builtin_amdgcn_s_barrier();
-        QX_SUB_D(1, 0, van, vbn, 0, a_vo, sa, dA)
-        QX_ADV_A();
-        QX_SUB_D(0, 1, va1, vbn, 1, b_vo, sb, dB)
-        QX_ADV_B();
-        st = stn;
-    }
-#pragma unroll 1
-    for (int kt = KT - 2; kt <= KT - 1; kt++) {
-        const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
-        const uint32_t van = a_off0 + stn, vbn = b_off + stn,
-                       va1 = a_off1 + stn;
+    if constexpr (SHORTK) {
+        for (int t = 0; t < KT; t++) {
+            QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+            QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+        }
         QX_WV(0);
-        __builtin_amdgcn_s_barrier();
-        QX_SUB(1, 0, van, vbn, 0, , , , )
-        QX_SUB(0, 1, va1, vbn, 1, , , , )
-        st = stn;
+        __syncthreads();
+        const uint32_t flip = p.a_is_u8 ? 0x80808080u : 0u;
+        for (int t = 0; t < KT; t++) {
+#pragma unroll
+            for (int ki = 0; ki < 2; ki++) {
+                const uint8_t *S = lds + t * STAGE_BYTES;
+                const int arel = arow * BK + a_swz(arow, 2 * ki + (lane >> 5)) * 16;
+                const int brel = A_BYTES + ((wn0 >> 5) * 128 + lane) * 16 + ki * 1024;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    v4i v = *(const v4i *)(S + arel + i * 2048);
+                    v.x ^= flip;
+                    v.y ^= flip;
+                    v.z ^= flip;
+                    v.w ^= flip;
+                    fa[0][i] = v;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    fb[0][j] = *(const v4i *)(S + brel + j * 2048);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    } else {
+        // ---- prologue: tiles 0 and 1 and the A half of tile 2 ----
+        QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+        QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+        QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+        QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+        QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+        QX_WV(12);
+        __syncthreads();
+        QX_RD_A(0, a_off0, 0);
+        QX_RD_B(0, b_off, 0, 0);
+        QX_RD_B(0, b_off, 0, 1);
+        QX_RD_B(0, b_off, 0, 2);
+        QX_RD_B(0, b_off, 0, 3);
+        QX_RD_A(0, a_off0, 1);
+        QX_RD_A(0, a_off0, 2);
+        QX_RD_A(0, a_off0, 3);
+        uint32_t st = 0; // ring offset of the tile whose first half was started
+        {
+            const uint32_t va1 = a_off1, vb = b_off;
+            QX_SUB_D(0, 1, va1, vb, 1, b_vo, sb, dB) // B half of tile 2
+            QX_ADV_B();
+        }
+        // k-step kt: second half of tile kt-1 (requesting the A half of tile
+        // kt+2), then first half of tile kt (requesting the B half of tile kt+2)
+        for (int kt = 1; kt <= KT - 3; kt++) {
+            const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
+            const uint32_t van = a_off0 + stn, vbn = b_off + stn,
+                           va1 = a_off1 + stn;
+            QX_WV(8); // tile kt has landed
+            __builtin_amdgcn_s_barrier();
+            QX_SUB_D(1, 0, van, vbn, 0, a_vo, sa, dA)
+            QX_ADV_A();
+            QX_SUB_D(0, 1, va1, vbn, 1, b_vo, sb, dB)
+            QX_ADV_B();
+            st = stn;
+        }
+#pragma unroll 1
+        for (int kt = KT - 2; kt <= KT - 1; kt++) {
+            const uint32_t stn = (st + STAGE_BYTES) & (RING - 1);
+            const uint32_t van = a_off0 + stn, vbn = b_off + stn,
+                           va1 = a_off1 + stn;
+            QX_WV(0);
+            __builtin_amdgcn_s_barrier();
+            QX_SUB(1, 0, van, vbn, 0, , , , )
+            QX_SUB(0, 1, va1, vbn, 1, , , , )
+            st = stn;
+        }
+        QX_SUB_LAST(1)
+        __syncthreads();
     }
-    QX_SUB_LAST(1)
-    __syncthreads();
 
     tile_epilogue<false>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
 }
@@ -705,23 +748,35 @@ static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ((ntiles + 7) / 8) * 8;
-    static bool attr_done = false;
-    if (!attr_done) {
+    // one attribute call per kernel (the kernels share this function's type)
+    static const void *done[8] = {};
+    bool seen = false;
+    for (const void *d : done)
+        seen = seen || d == (const void *)kern;
+    if (!seen) {
         (void)hipFuncSetAttribute((const void *)kern,
                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-        attr_done = true;
+        for (const void *&d : done)
+            if (!d) {
+                d = (const void *)kern;
+                break;
+            }
     }
     hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(NT), LDS_TOTAL,
             stream, q);
 }
 
-// Problems the kernels take: s8 or fp8 sources, K a multiple of 64 (fp8: 128)
-// with at least 4 (6) k-steps, a straight-line epilogue, 32-bit addressable tiles, and enough
+// Problems the kernels take: K a multiple of 64; s8 sources (u8 too when K is
+// at most 256), or fp8 sources with K a multiple of 128 and at least 6 k-steps; a straight-line epilogue, 32-bit addressable tiles, and enough
 // 256 x 256 tiles to occupy the chip.
+static bool short_k(const gemm_params_t &p) {
+    return p.K <= 4 * 64;
+}
+
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
-    if (p.a_is_u8 || p.ep.fast == EP_FAST_NONE) return false;
+    if (p.ep.fast == EP_FAST_NONE || p.K % 64 != 0 || p.K < 64) return false;
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
-    if (p.K % 64 != 0 || p.K < 4 * 64) return false;
+    if (p.a_is_u8 && !short_k(p)) return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;
     if ((int64_t)8 * p.kb32 * 1024 >= ((int64_t)1 << 32)) return false;
     return true;
@@ -730,8 +785,10 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     if (f8)
         launch_b8x(gemm_f8x_kernel, p, stream);
+    else if (short_k(p))
+        launch_b8x(gemm_b8x_kernel<true>, p, stream);
     else
-        launch_b8x(gemm_b8x_kernel, p, stream);
+        launch_b8x(gemm_b8x_kernel<false>, p, stream);
 }
 
 } // namespace qmm

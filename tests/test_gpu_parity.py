@@ -297,6 +297,11 @@ TILE256_CASES = {
                                             post_ops=[{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]), False),
     "plain_f32_batched": (lambda: int8_linear(256, 256, 256, 75, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, batch=(2,)), True),
     "bf16_subnormal_results_are_zero": (_tiny_scale_problem, True),
+    # K of at most 256: the all-of-K-in-LDS path, which also takes u8 sources
+    "short_k128_u8_zp128_f32": (lambda: int8_linear(300, 128, 260, 79), True),
+    "short_k256_u8_zp7_bf16": (lambda: int8_linear(256, 256, 512, 80, dst_dt=dt.bf16, src_zp=7, per_token=True), True),
+    "short_k64_s8_relu": (lambda: int8_linear(130, 64, 250, 81, src_dt=dt.s8, src_zp=None,
+                                              post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]), True),
 }
 
 
@@ -317,6 +322,22 @@ def test_mfma_int8_tile256_kernel(ctx, tile256, name):
         M, N = p.dst.dims[-2:]
         assert_f32_close(got.view(np.float32).reshape(-1, N), want.view(np.float32).reshape(-1, N),
                          rel=1e-5, scale=np.abs(want.view(np.float32).reshape(-1, N)) + 1e-30, what=name)
+
+
+def test_mfma_int8_tile256_short_k_batched_scores(ctx, tile256):
+    eng, strm = ctx
+    say("mfma_b8 256x256 kernel, K = 128, batched scores + mask")
+    r = rnd(82)
+    B, S, D = 3, 512, 128
+    q = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127)
+    k = np.clip(np.rint(r.standard_normal((B, D, S)) * 40), -127, 127)
+    mask = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], -1e4, 0).astype(np.float32)[None]
+    p = Problem(TensorSpec(dt.s8, [B, S, D], None, q), TensorSpec(dt.s8, [B, D, S], None, k), TensorSpec(dt.f32, [B, S, S]),
+                scales={"src": (0, dt.f32, None, [0.01]), "wei": (0, dt.f32, None, [0.012])},
+                post_ops=[{"kind": "binary", "alg": A.binary_add, "src1": TensorSpec(dt.f32, [1, S, S], None, mask)}])
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    assert_bit_exact(got, p.run_oracle(), "scores")
 
 
 def test_mfma_fp8_tile256_kernel(ctx, tile256):
