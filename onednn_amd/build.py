@@ -35,7 +35,7 @@ UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
          ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]
 # the tiled GEMM is instantiated once per tile configuration, each in its own
 # object so the instantiations compile in parallel
-GEMM_VARIANTS = [1, 2]
+GEMM_VARIANTS = [1, 2, 3]
 for v in GEMM_VARIANTS:
     UNITS.append(("qmm_gemm_b8.hip", "_v%d" % v, ["-DQMM_GEMM_VARIANT=%d" % v]))
 

@@ -396,6 +396,8 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
 #define QMM_CFG 256, 128, 64, 2, 2, 3
 #elif QMM_GEMM_VARIANT == 2
 #define QMM_CFG 128, 128, 64, 2, 2, 3
+#elif QMM_GEMM_VARIANT == 3
+#define QMM_CFG 64, 64, 64, 2, 2, 3
 #endif
 #define QMM_CAT_(a, b) a##b
 #define QMM_CAT(a, b) QMM_CAT_(a, b)
@@ -411,6 +413,7 @@ void QMM_CAT(launch_gemm_b8_v, QMM_GEMM_VARIANT)(
 #else
 void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);
 void launch_gemm_b8_v2(const gemm_params_t &p, bool f8, hipStream_t stream);
+void launch_gemm_b8_v3(const gemm_params_t &p, bool f8, hipStream_t stream);
 // 256 x 256 tile kernel with the hand-ordered main loop (qmm_gemm_b8x.hip)
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8);
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream);
@@ -431,10 +434,14 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
     if (variant == 0) {
         const int64_t big = (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128)
                 * p.batch;
-        variant = big >= 256 ? 1 : 2;
+        const int64_t mid = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128)
+                * p.batch;
+        // small problems: more, smaller tiles keep more CUs busy
+        variant = big >= 256 ? 1 : (mid >= 64 ? 2 : 3);
     }
     switch (variant) {
         case 1: launch_gemm_b8_v1(p, f8, stream); break;
+        case 3: launch_gemm_b8_v3(p, f8, stream); break;
         default: launch_gemm_b8_v2(p, f8, stream); break;
     }
 }
