@@ -148,132 +148,216 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     const uint8_t *const fast_zp = p.zps ? (const uint8_t *)p.zps : p.B;
     const bool zp4 = p.zp_dt == dt_s4 || p.zp_dt == dt_u4;
 
-    for (int kc0 = 0; kc0 < Kpad; kc0 += KC) {
-        const int kc_len = min(KC, Kpad - kc0);
-        const int tiles = kc_len / 128;
-        const int g0 = kc0 / 128;
+    if constexpr (FAST) {
+        // Waves are independent until the final reduction: each one fetches
+        // its weight tiles, their scales / zero points AND its activation
+        // fragments (lane (r, c) holds row r, k = 32 s + 8 c .. + 7 of a tile)
+        // straight into registers, every load unconditional (clamped
+        // addresses), all issued before the first use. No LDS staging, no
+        // barrier before the arithmetic. Tile and group indices are wave
+        // uniform (scalar arithmetic, shifts instead of divisions). Rows past
+        // M compute on a repeated row and are never stored; only k past K has
+        // to be zeroed (the padded weights decode to the magic offset, not 0).
+        const int uw = __builtin_amdgcn_readfirstlane(wave);
+        const int tiles = Kpad / 128;
+        const int rr = min(r, rows - 1);
+        const uint16_t *__restrict__ Arow
+                = p.A + (int64_t)(m_base + rr) * p.lda;
+        const int nn = min(n, p.N - 1);
+        const uint16_t *const scn = fast_sc + (p.scale_per_n ? nn : 0);
+        const int zcol = p.zp_per_n ? nn : 0;
+        const bool sc_f16 = p.scale_dt == dt_f16;
+        const bool k_tail = (p.K & 127) != 0;
         constexpr int UNR = 4;
-        uint4 wt[UNR];
-        uint32_t scp[UNR], zpp[UNR]; // raw scale / zero-point bits per tile
-        auto fetch = [&](int tb) {
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int t = tb + wave + u * GEMV_WAVES;
-                wt[u] = make_uint4(0, 0, 0, 0);
-                if constexpr (FAST) {
-                    const int tc = min(t, tiles - 1);
-                    wt[u] = ld_stream(Bt + (int64_t)(g0 + tc) * 1024);
-                    const int kq = min(kc0 + (tc + 1) * 128, p.K) - 1;
-                    const int nn = min(n, p.N - 1);
-                    scp[u] = fast_sc[(int64_t)(kq / p.gs) * sN
-                            + (p.scale_per_n ? nn : 0)];
-                    const int64_t zi = p.zps
-                            ? (int64_t)(p.gz > 0 ? kq / p.gz : 0) * zN
-                                    + (p.zp_per_n ? nn : 0)
-                            : 0;
-                    zpp[u] = fast_zp[zp4 ? zi >> 1 : zi];
-                    continue;
-                }
-                scp[u] = 0u;
-                zpp[u] = 0u;
-                if (t < tiles) {
-                    wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
-                    if (per_tile) {
-                        const int kq = min(kc0 + (t + 1) * 128, p.K) - 1;
-                        scp[u] = scale_raw(kq);
-                        zpp[u] = zp_raw(kq);
-                    }
-                }
-            }
-        };
-        // Vector-memory results return in issue order, so the activation
-        // chunks this thread stages are requested first and the weights right
-        // behind them: waiting for the activations then leaves the weights in
-        // flight. Chunk kc (8 values) of row m lands at (kc*MR + m)*16.
-        if (kc0 > 0) __syncthreads(); // previous chunk fully consumed
-        const int nchunks = (kc_len / 8) * MR;
-        auto act_load = [&](int i) -> uint4 {
-            const int kc = i / MR, m = i % MR;
-            const int k = kc0 + kc * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (i < nchunks && m < rows && k < p.K)
-                v = *(const uint4 *)(p.A + (int64_t)(m_base + m) * p.lda + k);
-            return v;
-        };
-        constexpr int ACT_PRE = 2;
-        uint4 areg[ACT_PRE];
-#pragma unroll
-        for (int q = 0; q < ACT_PRE; q++)
-            areg[q] = act_load(tid + q * GEMV_WAVES * 64);
-        fetch(0);
-#pragma unroll
-        for (int q = 0; q < ACT_PRE; q++) {
-            const int i = tid + q * GEMV_WAVES * 64;
-            if (i < nchunks) *(uint4 *)(lds + (size_t)i * 16) = areg[q];
-        }
-        for (int i = tid + ACT_PRE * GEMV_WAVES * 64; i < nchunks;
-                i += GEMV_WAVES * 64)
-            *(uint4 *)(lds + (size_t)i * 16) = act_load(i);
-        __syncthreads();
-
         for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
-            if (tb > 0) fetch(tb);
+            uint4 wt[UNR], av[UNR][4];
+            uint32_t scp[UNR], zpp[UNR];
 #pragma unroll
             for (int u = 0; u < UNR; u++) {
-                const int t = tb + wave + u * GEMV_WAVES;
+                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+                wt[u] = ld_stream(Bt + (int64_t)tc * 1024);
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++) {
+                    // chunks past the row's end re-read its last one
+                    const int k = min(tc * 128 + s4 * 32 + c * 8, p.K - 8);
+                    av[u][s4] = *(const uint4 *)(Arow + k);
+                }
+                const int gsc = p.gs_shift < 0 ? 0 : tc >> p.gs_shift;
+                scp[u] = scn[(int64_t)gsc * sN];
+                const int gzp = p.gz_shift < 0 ? 0 : tc >> p.gz_shift;
+                const int64_t zi = p.zps ? (int64_t)gzp * zN + zcol : 0;
+                zpp[u] = fast_zp[zp4 ? zi >> 1 : zi];
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int t = tb + uw + u * GEMV_WAVES;
                 if (t >= tiles) break;
                 const uint32_t wd[4] = {wt[u].x ^ sflip, wt[u].y ^ sflip,
                         wt[u].z ^ sflip, wt[u].w ^ sflip};
+                if (k_tail && t == tiles - 1) {
 #pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    const uint32_t d = wd[s];
+                    for (int s4 = 0; s4 < 4; s4++)
+                        if (t * 128 + s4 * 32 + c * 8 >= p.K)
+                            av[u][s4] = make_uint4(0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++) {
+                    const uint32_t d = wd[s4];
                     v4u b;
                     b.x = (d & 0x000F000Fu) | MAGIC;
                     b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
                     b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
                     b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
-                    v4u a = {0u, 0u, 0u, 0u};
-                    if (r < MR) {
-                        const uint4 av = *(const uint4 *)(lds
-                                + ((size_t)(t * 16 + s * 4 + c) * MR + r) * 16);
-                        a = v4u {av.x, av.y, av.z, av.w};
-                    }
+                    const v4u a = {av[u][s4].x, av[u][s4].y, av[u][s4].z,
+                            av[u][s4].w};
                     P = mfma16<F16>(a, b, P);
                     S = mfma16<F16>(a, ones, S);
-                    const int k_end = kc0 + t * 128 + (s + 1) * 32;
-                    // A wave's tiles are not adjacent in k, so the partial
-                    // sums are folded at every tile end as well as where a
-                    // scale / zero-point group closes inside a tile (folding
-                    // early is exact in structure: both factors are constant
-                    // over the folded range).
-                    if (s == 3 || (!per_tile && k_end % fl == 0)) {
-                        // the range just folded contains k_end - 1
-                        float sc, zp;
+                }
+                // one scale and one zero point per column and tile: fold here
+                const float sc = sc_f16
+                        ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
+                        : u2f(scp[u] << 16);
+                float zp = 0.f;
+                if (p.zps) {
+                    const int gzp = p.gz_shift < 0 ? 0 : t >> p.gz_shift;
+                    const int64_t zi = (int64_t)gzp * zN + zcol;
+                    const uint32_t raw = zpp[u];
+                    if (zp4) {
+                        const int nib = (zi & 1) ? (raw >> 4) & 0xf : raw & 0xf;
+                        zp = (float)(p.zp_dt == dt_s4 ? s4_value(nib) : nib);
+                    } else {
+                        zp = p.zp_dt == dt_s8 ? (float)(int8_t)raw
+                                              : (float)(uint8_t)raw;
+                    }
+                }
+                const float off = OFFSET + soff + zp;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    out[j] = __builtin_fmaf(sc, P[j] - off * S[j], out[j]);
+                    P[j] = 0.f;
+                    S[j] = 0.f;
+                }
+            }
+        }
+    } else {
+        for (int kc0 = 0; kc0 < Kpad; kc0 += KC) {
+            const int kc_len = min(KC, Kpad - kc0);
+            const int tiles = kc_len / 128;
+            const int g0 = kc0 / 128;
+            constexpr int UNR = 4;
+            uint4 wt[UNR];
+            uint32_t scp[UNR], zpp[UNR]; // raw scale / zero-point bits per tile
+            auto fetch = [&](int tb) {
+    #pragma unroll
+                for (int u = 0; u < UNR; u++) {
+                    const int t = tb + wave + u * GEMV_WAVES;
+                    wt[u] = make_uint4(0, 0, 0, 0);
+                    scp[u] = 0u;
+                    zpp[u] = 0u;
+                    if (t < tiles) {
+                        wt[u] = ld_stream(Bt + (int64_t)(g0 + t) * 1024);
                         if (per_tile) {
                             const int kq = min(kc0 + (t + 1) * 128, p.K) - 1;
-                            sc = scale_cvt(scp[u]);
-                            zp = zp_cvt(zpp[u], kq);
-                        } else {
-                            const int kq = min(k_end, p.K) - 1;
-                            sc = scale_cvt(scale_raw(kq));
-                            zp = zp_cvt(zp_raw(kq), kq);
+                            scp[u] = scale_raw(kq);
+                            zpp[u] = zp_raw(kq);
                         }
-                        const float off = OFFSET + soff + zp;
-#pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            out[j] = __builtin_fmaf(
-                                    sc, P[j] - off * S[j], out[j]);
-                            P[j] = 0.f;
-                            S[j] = 0.f;
+                    }
+                }
+            };
+            // Vector-memory results return in issue order, so the activation
+            // chunks this thread stages are requested first and the weights right
+            // behind them: waiting for the activations then leaves the weights in
+            // flight. Chunk kc (8 values) of row m lands at (kc*MR + m)*16.
+            if (kc0 > 0) __syncthreads(); // previous chunk fully consumed
+            const int nchunks = (kc_len / 8) * MR;
+            auto act_load = [&](int i) -> uint4 {
+                const int kc = i / MR, m = i % MR;
+                const int k = kc0 + kc * 8;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (i < nchunks && m < rows && k < p.K)
+                    v = *(const uint4 *)(p.A + (int64_t)(m_base + m) * p.lda + k);
+                return v;
+            };
+            constexpr int ACT_PRE = 2;
+            uint4 areg[ACT_PRE];
+    #pragma unroll
+            for (int q = 0; q < ACT_PRE; q++)
+                areg[q] = act_load(tid + q * GEMV_WAVES * 64);
+            fetch(0);
+    #pragma unroll
+            for (int q = 0; q < ACT_PRE; q++) {
+                const int i = tid + q * GEMV_WAVES * 64;
+                if (i < nchunks) *(uint4 *)(lds + (size_t)i * 16) = areg[q];
+            }
+            for (int i = tid + ACT_PRE * GEMV_WAVES * 64; i < nchunks;
+                    i += GEMV_WAVES * 64)
+                *(uint4 *)(lds + (size_t)i * 16) = act_load(i);
+            __syncthreads();
+
+            for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
+                if (tb > 0) fetch(tb);
+    #pragma unroll
+                for (int u = 0; u < UNR; u++) {
+                    const int t = tb + wave + u * GEMV_WAVES;
+                    if (t >= tiles) break;
+                    const uint32_t wd[4] = {wt[u].x ^ sflip, wt[u].y ^ sflip,
+                            wt[u].z ^ sflip, wt[u].w ^ sflip};
+    #pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        const uint32_t d = wd[s];
+                        v4u b;
+                        b.x = (d & 0x000F000Fu) | MAGIC;
+                        b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
+                        b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
+                        b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
+                        v4u a = {0u, 0u, 0u, 0u};
+                        if (r < MR) {
+                            const uint4 av = *(const uint4 *)(lds
+                                    + ((size_t)(t * 16 + s * 4 + c) * MR + r) * 16);
+                            a = v4u {av.x, av.y, av.z, av.w};
+                        }
+                        P = mfma16<F16>(a, b, P);
+                        S = mfma16<F16>(a, ones, S);
+                        const int k_end = kc0 + t * 128 + (s + 1) * 32;
+                        // A wave's tiles are not adjacent in k, so the partial
+                        // sums are folded at every tile end as well as where a
+                        // scale / zero-point group closes inside a tile (folding
+                        // early is exact in structure: both factors are constant
+                        // over the folded range).
+                        if (s == 3 || (!per_tile && k_end % fl == 0)) {
+                            // the range just folded contains k_end - 1
+                            float sc, zp;
+                            if (per_tile) {
+                                const int kq = min(kc0 + (t + 1) * 128, p.K) - 1;
+                                sc = scale_cvt(scp[u]);
+                                zp = zp_cvt(zpp[u], kq);
+                            } else {
+                                const int kq = min(k_end, p.K) - 1;
+                                sc = scale_cvt(scale_raw(kq));
+                                zp = zp_cvt(zp_raw(kq), kq);
+                            }
+                            const float off = OFFSET + soff + zp;
+    #pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                out[j] = __builtin_fmaf(
+                                        sc, P[j] - off * S[j], out[j]);
+                                P[j] = 0.f;
+                                S[j] = 0.f;
+                            }
                         }
                     }
                 }
             }
         }
+
     }
 
     // ---- reduce the waves' partial sums and finish ----
-    __syncthreads();
+    if constexpr (!FAST) __syncthreads(); // the staged activations are dead
     float *red = (float *)lds;
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -306,17 +390,6 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
     const size_t red = (size_t)GEMV_WAVES * 64 * 4 * sizeof(float);
     if (lds < red) lds = red;
     dim3 grid(p.nb16, (p.M + 15) / 16);
-    auto launch = [&](auto kern) {
-        static bool attr_done = false;
-        if (!attr_done) {
-            (void)hipFuncSetAttribute((const void *)kern,
-                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                    GEMV_LDS_BUDGET);
-            attr_done = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, p,
-                MR, KC);
-    };
     // the all-unconditional-loads variant (see the kernel's FAST parameter)
     int fl = p.gs;
     if (p.gz > 0) {
@@ -328,9 +401,47 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         }
         fl = a;
     }
+    // group widths of the form 128 << s (or one group over all of K)
+    auto shift_of = [&](int g, int &sh) {
+        if (g >= Kpad) {
+            sh = -1;
+            return true;
+        }
+        if (g % 128 != 0) return false;
+        int q = g / 128;
+        sh = 0;
+        while (q > 1 && q % 2 == 0) {
+            q /= 2;
+            sh++;
+        }
+        return q == 1;
+    };
+    gemv_params_t q = p;
     const bool fast = p.scales && fl % 128 == 0
             && (p.scale_dt == dt_f16 || p.scale_dt == dt_bf16)
-            && (!p.zps || p.zp_dt != dt_s32);
+            && (!p.zps || p.zp_dt != dt_s32) && shift_of(p.gs, q.gs_shift)
+            && (p.gz > 0 ? shift_of(p.gz, q.gz_shift)
+                         : ((q.gz_shift = -1), true));
+    auto launch = [&](auto kern) {
+        // (the four kernels share this lambda's type: one call each)
+        static const void *done[4] = {};
+        bool seen = false;
+        for (const void *d : done)
+            seen = seen || d == (const void *)kern;
+        if (!seen) {
+            (void)hipFuncSetAttribute((const void *)kern,
+                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                    GEMV_LDS_BUDGET);
+            for (const void *&d : done)
+                if (!d) {
+                    d = (const void *)kern;
+                    break;
+                }
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, q,
+                MR, KC);
+    };
+    if (fast) lds = red; // that variant keeps its activations in registers
     if (p.act_f16) {
         if (fast)
             launch(gemv_w4_kernel<true, true>);

@@ -132,6 +132,9 @@ struct gemv_params_t {
     int32_t wei_signed; // s4 weights
     int32_t act_f16; // activations are f16 (else bf16)
     int32_t m0; // first row handled by this launch
+    // fast variant: K groups are 128 << shift wide (host-checked); -1: single
+    int32_t gs_shift, gz_shift;
+    int32_t pad_;
     epilogue_t ep;
 };
 
