@@ -79,8 +79,9 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     const float soff = p.wei_signed ? 8.f : 0.f;
 
     // flush granularity: the scale and zero-point groups both close there
+    // (the fast variant folds once per 128-k tile and does not need it)
     int fl = p.gs;
-    if (p.gz > 0) {
+    if (!FAST && p.gz > 0) {
         int a = p.gs, b = p.gz;
         while (b) {
             const int t = a % b;
@@ -192,21 +193,34 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                 const int64_t zi = p.zps ? (int64_t)gzp * zN + zcol : 0;
                 zpp[u] = fast_zp[zp4 ? zi >> 1 : zi];
             }
+            if (k_tail && tb + UNR * GEMV_WAVES >= tiles) {
+                // zero the activations past K (last tile of the matrix)
 #pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int t = tb + uw + u * GEMV_WAVES;
-                if (t >= tiles) break;
-                const uint32_t wd[4] = {wt[u].x ^ sflip, wt[u].y ^ sflip,
-                        wt[u].z ^ sflip, wt[u].w ^ sflip};
-                if (k_tail && t == tiles - 1) {
+                for (int u = 0; u < UNR; u++) {
+                    const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
 #pragma unroll
                     for (int s4 = 0; s4 < 4; s4++)
-                        if (t * 128 + s4 * 32 + c * 8 >= p.K)
+                        if (tc * 128 + s4 * 32 + c * 8 >= p.K)
                             av[u][s4] = make_uint4(0, 0, 0, 0);
                 }
+            }
+            // the four tiles are independent accumulation chains: a tile past
+            // the end is a repeat of the last one and is folded with scale 0
+            v4f Pu[UNR], Su[UNR];
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++) {
-                    const uint32_t d = wd[s4];
+            for (int u = 0; u < UNR; u++) {
+                Pu[u] = v4f {0.f, 0.f, 0.f, 0.f};
+                Su[u] = v4f {0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+#pragma unroll
+                for (int u = 0; u < UNR; u++) {
+                    const uint32_t d = (s4 == 0 ? wt[u].x
+                                    : s4 == 1   ? wt[u].y
+                                    : s4 == 2   ? wt[u].z
+                                                : wt[u].w)
+                            ^ sflip;
                     v4u b;
                     b.x = (d & 0x000F000Fu) | MAGIC;
                     b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
@@ -214,16 +228,22 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                     b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
                     const v4u a = {av[u][s4].x, av[u][s4].y, av[u][s4].z,
                             av[u][s4].w};
-                    P = mfma16<F16>(a, b, P);
-                    S = mfma16<F16>(a, ones, S);
+                    Pu[u] = mfma16<F16>(a, b, Pu[u]);
+                    Su[u] = mfma16<F16>(a, ones, Su[u]);
                 }
-                // one scale and one zero point per column and tile: fold here
-                const float sc = sc_f16
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int t = tb + uw + u * GEMV_WAVES;
+                const int tc = min(t, tiles - 1);
+                // one scale and one zero point per column and tile
+                float sc = sc_f16
                         ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
                         : u2f(scp[u] << 16);
+                if (t >= tiles) sc = 0.f;
                 float zp = 0.f;
                 if (p.zps) {
-                    const int gzp = p.gz_shift < 0 ? 0 : t >> p.gz_shift;
+                    const int gzp = p.gz_shift < 0 ? 0 : tc >> p.gz_shift;
                     const int64_t zi = (int64_t)gzp * zN + zcol;
                     const uint32_t raw = zpp[u];
                     if (zp4) {
@@ -236,11 +256,8 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                 }
                 const float off = OFFSET + soff + zp;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    out[j] = __builtin_fmaf(sc, P[j] - off * S[j], out[j]);
-                    P[j] = 0.f;
-                    S[j] = 0.f;
-                }
+                for (int j = 0; j < 4; j++)
+                    out[j] = __builtin_fmaf(sc, Pu[u][j] - off * Su[u][j], out[j]);
             }
         }
     } else {
