@@ -18,6 +18,9 @@ void launch_matmul_generic(const generic_params_t *dev_params,
         hipStream_t stream);
 void launch_reorder_generic(const generic_reorder_params_t &params,
         const qmm_reorder_args_t &args, hipStream_t stream);
+bool gemm_b8_uses_tile256(const gemm_params_t &p, bool f8, int variant);
+void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
+        int64_t K, int64_t lda, int64_t a_sb, hipStream_t stream);
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream);
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
@@ -526,13 +529,37 @@ int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
     return QMM_LAYOUT_PLAIN;
 }
 
+// Large u8-source problems go through the 256 x 256 kernel after a pre-pass
+// that rewrites the source as s8: room for that copy, behind the packed weights.
+static size_t u8_copy_bytes(const qmm_matmul_desc_t *desc) {
+    const int nd = desc->dst.ndims;
+    if (desc->src.dt != dt_u8) return 0;
+    const int64_t M = desc->dst.dims[nd - 2], N = desc->dst.dims[nd - 1];
+    const int64_t K = desc->src.dims[nd - 1];
+    int64_t batch = 1;
+    for (int d = 0; d < nd - 2; d++)
+        batch *= desc->dst.dims[d];
+    if (K % 64 != 0 || K <= 256) return 0;
+    if (((M + 255) / 256) * ((N + 255) / 256) * batch < 192) return 0;
+    return (size_t)(batch * M * K);
+}
+
+static size_t round256(size_t v) {
+    return (v + 255) / 256 * 256;
+}
+
 size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
-    if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     const int nd = desc->wei.ndims;
     const int64_t K = desc->wei.dims[nd - 2], N = desc->wei.dims[nd - 1];
-    if (impl == impl_gemm_b8)
-        return qmm_packed_size(
-                QMM_LAYOUT_MFMA_B8, desc->wei.dt, wei_batch(*desc), K, N);
+    if (impl == impl_gemm_b8) {
+        const size_t packed = desc->wei_layout == QMM_LAYOUT_PLAIN
+                ? qmm_packed_size(QMM_LAYOUT_MFMA_B8, desc->wei.dt,
+                        wei_batch(*desc), K, N)
+                : 0;
+        const size_t copy = u8_copy_bytes(desc);
+        return copy ? round256(packed) + copy : packed;
+    }
+    if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     if (impl == impl_gemv_w4)
         return qmm_packed_size(QMM_LAYOUT_MFMA_W4, desc->wei.dt, 1, K, N);
     return 0;
@@ -651,6 +678,22 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.batch = (int32_t)P.batch;
         g.kb32 = (int32_t)geom.kb32;
         g.nb32 = (int32_t)geom.nb32;
+        if (g.a_is_u8 && u8_copy_bytes(&D) && args->scratch) {
+            gemm_params_t h = g;
+            uint8_t *copy = (uint8_t *)args->scratch
+                    + (D.wei_layout == QMM_LAYOUT_PLAIN
+                                    ? round256(geom.total_bytes)
+                                    : 0);
+            h.A = copy;
+            h.lda = P.K;
+            h.a_sb = P.M * P.K;
+            h.a_preflipped = 1;
+            if (gemm_b8_uses_tile256(h, f8, g_gemm_variant)) {
+                launch_flip_u8(g.A, copy, P.batch, P.M, P.K, g.lda, g.a_sb,
+                        stream);
+                g = h;
+            }
+        }
         launch_gemm_b8(g, f8, g_gemm_variant, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;

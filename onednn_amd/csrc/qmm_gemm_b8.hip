@@ -420,13 +420,18 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream);
 
 // variant: 0 = heuristic; others pick a tile configuration explicitly (used by
 // the tuning sweep; 6 = the 256 x 256 kernel where it applies)
+// true when launch_gemm_b8 would hand the problem to the 256 x 256 kernel
+bool gemm_b8_uses_tile256(const gemm_params_t &p, bool f8, int variant) {
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
+            * p.batch;
+    return (variant == 6 || (variant == 0 && tiles256 >= 192))
+            && gemm_b8x_eligible(p, f8);
+}
+
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return;
-    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
-            * p.batch;
-    if ((variant == 6 || (variant == 0 && tiles256 >= 192))
-            && gemm_b8x_eligible(p, f8)) {
+    if (gemm_b8_uses_tile256(p, f8, variant)) {
         launch_gemm_b8x(p, f8, stream);
         return;
     }

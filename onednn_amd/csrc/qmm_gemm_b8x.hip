@@ -355,7 +355,8 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
 // LDS ring, so every tile is requested at once and multiplied after a single
 // wait; these problems are bound by the dst stream and share the epilogue.
 // u8 sources (top bits flipped after the fragment read, +128 * colsum in the
-// epilogue) are taken on that path only.
+// epilogue) are taken on that path only; the pipelined path takes them once a
+// pre-pass has rewritten them as s8 (a_preflipped).
 template <bool SHORTK>
 __global__ void __launch_bounds__(b8x::NT, 1)
 gemm_b8x_kernel(const gemm_params_t p) {
@@ -471,7 +472,8 @@ gemm_b8x_kernel(const gemm_params_t p) {
         }
         QX_WV(0);
         __syncthreads();
-        const uint32_t flip = p.a_is_u8 ? 0x80808080u : 0u;
+        const uint32_t flip
+                = p.a_is_u8 && !p.a_preflipped ? 0x80808080u : 0u;
         for (int t = 0; t < KT; t++) {
 #pragma unroll
             for (int ki = 0; ki < 2; ki++) {
@@ -776,7 +778,7 @@ static bool short_k(const gemm_params_t &p) {
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     if (p.ep.fast == EP_FAST_NONE || p.K % 64 != 0 || p.K < 64) return false;
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
-    if (p.a_is_u8 && !short_k(p)) return false;
+    if (p.a_is_u8 && !p.a_preflipped && !short_k(p)) return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;
     if ((int64_t)8 * p.kb32 * 1024 >= ((int64_t)1 << 32)) return false;
     return true;

@@ -45,22 +45,36 @@ pack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
     }
 }
 
-// column sums of the (signed or unsigned) 8-bit weights, one thread per column
+// column sums of the (signed or unsigned) 8-bit weights: blockIdx.y cuts K into
+// chunks of COLSUM_KCHUNK rows, a thread sums one column of its chunk and adds
+// the partial sum to the (zeroed) s32 result -- integer atomics, so the result
+// does not depend on the order
+constexpr int COLSUM_KCHUNK = 128;
+
+__global__ void __launch_bounds__(256)
+colsum_zero_kernel(const pack_params_t p, const b8_geom_t g) {
+    const int64_t total = p.batch * g.Npad;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x)
+        ((int32_t *)(p.dst + g.colsum_off))[i] = 0;
+}
+
 __global__ void __launch_bounds__(256)
 colsum_kernel(const pack_params_t p, const b8_geom_t g) {
     const int64_t total = p.batch * g.Npad;
+    const int64_t k0 = (int64_t)blockIdx.y * COLSUM_KCHUNK;
+    const int64_t k1 = k0 + COLSUM_KCHUNK < p.K ? k0 + COLSUM_KCHUNK : p.K;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
             i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t b = i / g.Npad, n = i % g.Npad;
+        if (n >= p.N) continue;
+        const uint8_t *s = p.src + b * p.sb + n * p.sn;
         int32_t acc = 0;
-        if (n < p.N) {
-            const uint8_t *s = p.src + b * p.sb + n * p.sn;
-            for (int64_t k = 0; k < p.K; k++) {
-                const uint8_t v = s[k * p.sk];
-                acc += p.dt == dt_s8 ? (int32_t)(int8_t)v : (int32_t)v;
-            }
+        for (int64_t k = k0; k < k1; k++) {
+            const uint8_t v = s[k * p.sk];
+            acc += p.dt == dt_s8 ? (int32_t)(int8_t)v : (int32_t)v;
         }
-        ((int32_t *)(p.dst + g.colsum_off))[i] = acc;
+        atomicAdd((int32_t *)(p.dst + g.colsum_off) + i, acc);
     }
 }
 
@@ -152,9 +166,44 @@ void launch_pack_b8(const void *src, void *dst, int dt, int64_t batch,
             sn, dt, 0};
     hipLaunchKernelGGL(pack_b8_kernel, dim3(grid_for(batch * g.batch_bytes / 16)),
             dim3(256), 0, stream, p, g);
-    if (with_colsum)
-        hipLaunchKernelGGL(colsum_kernel, dim3(grid_for(batch * g.Npad)),
+    if (with_colsum) {
+        hipLaunchKernelGGL(colsum_zero_kernel, dim3(grid_for(batch * g.Npad)),
                 dim3(256), 0, stream, p, g);
+        const int64_t cols = (batch * g.Npad + 255) / 256;
+        const unsigned kchunks
+                = (unsigned)((K + COLSUM_KCHUNK - 1) / COLSUM_KCHUNK);
+        hipLaunchKernelGGL(colsum_kernel,
+                dim3((unsigned)(cols < 65535 ? cols : 65535),
+                        kchunks ? kchunks : 1),
+                dim3(256), 0, stream, p, g);
+    }
+}
+
+// u8 activations -> s8 (x ^ 0x80) into a dense [batch][M][K] buffer: the
+// pre-pass of the 256 x 256 GEMM kernel for u8 sources (the +128 * colsum
+// correction is applied in its epilogue). One thread per 16 bytes.
+__global__ void __launch_bounds__(256)
+flip_u8_kernel(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t K16,
+        int64_t M, int64_t lda, int64_t a_sb) {
+    const int64_t total = rows * K16;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / K16, c = i % K16;
+        const int64_t b = r / M, m = r % M;
+        uint4 v = *(const uint4 *)(src + b * a_sb + m * lda + c * 16);
+        v.x ^= 0x80808080u;
+        v.y ^= 0x80808080u;
+        v.z ^= 0x80808080u;
+        v.w ^= 0x80808080u;
+        *(uint4 *)(dst + i * 16) = v;
+    }
+}
+
+void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
+        int64_t K, int64_t lda, int64_t a_sb, hipStream_t stream) {
+    hipLaunchKernelGGL(flip_u8_kernel, dim3(grid_for(batch * M * K / 16)),
+            dim3(256), 0, stream, (const uint8_t *)src, (uint8_t *)dst,
+            batch * M, K / 16, M, lda, a_sb);
 }
 
 void launch_unpack_b8(const void *src, void *dst, int dt, int64_t batch,

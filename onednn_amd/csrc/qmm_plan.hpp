@@ -113,7 +113,7 @@ struct gemm_params_t {
     int32_t kb32; // K blocks of 32 in the packed weights
     int32_t nb32;
     int32_t tiles_m, tiles_n;
-    int32_t pad_;
+    int32_t a_preflipped; // u8 source already rewritten as s8 (x ^ 0x80)
     epilogue_t ep;
 };
 

@@ -324,6 +324,18 @@ def test_mfma_int8_tile256_kernel(ctx, tile256, name):
                          rel=1e-5, scale=np.abs(want.view(np.float32).reshape(-1, N)) + 1e-30, what=name)
 
 
+def test_mfma_int8_large_u8_source_prepass(ctx):
+    """192 tiles of 256 x 256 with a u8 source: rewritten as s8 by a pre-pass into the
+    scratchpad, then the 256 x 256 kernel with the +128 * colsum correction."""
+    eng, strm = ctx
+    say("mfma_b8 u8 source 4096x320x3072 (library scratchpad)")
+    p = int8_linear(4096, 320, 3072, 84, src_zp=121)
+    for any_ in (True, False):
+        got, pd = p.run_gpu(eng, strm, weights_any=any_, return_pd=True)
+        assert pd.impl_info_str() == MFMA
+        assert_bit_exact(got, p.run_oracle(), "u8 prepass any=%s" % any_)
+
+
 def test_mfma_int8_tile256_short_k_batched_scores(ctx, tile256):
     eng, strm = ctx
     say("mfma_b8 256x256 kernel, K = 128, batched scores + mask")
