@@ -1,5 +1,5 @@
-// hip:gfx950:mfma_b8, large-problem kernel: int8 (s8 x s8 -> s32) GEMM with
-// a 256 x 256 x 64 block tile, four waves of 128 x 128 each (one per SIMD, the
+// hip:gfx950:mfma_b8, large-problem kernels: int8 (s8 x s8 -> s32) and fp8
+// (e4m3 x e4m3 -> f32, further down) GEMM with a 256 x 256 x 64 block tile, four waves of 128 x 128 each (one per SIMD, the
 // 256 accumulator registers of a wave hold its tile), and a hand-ordered main
 // loop.
 //
@@ -15,14 +15,13 @@
 // per MFMA (32 KiB per 128 MFMAs and CU).
 //
 // Pipeline (k-step = 64 k, two MFMA sub-steps of 32 k):
-//   LDS ring of 4 stages x (A 256x64 + B 256x64 bytes). The A half of tile t+2
-//   is requested in the second sub-step of k-step t-1... in general: k-step kt
-//   first finishes tile kt-1 (second sub-step) while requesting the A half of
-//   tile kt+2, then starts tile kt (first sub-step) while requesting the B half
-//   of tile kt+2. One barrier per k-step, preceded by vmcnt(8): tile kt has
-//   landed for every wave and the stage that tile kt+2 goes to (last read in
-//   k-step kt-2) is free. Fragments are double buffered in registers and read
-//   one sub-step ahead.
+//   LDS ring of 4 stages x (A 256x64 + B 256x64 bytes). Loop iteration kt first
+//   finishes tile kt-1 (its second sub-step) while requesting the A half of
+//   tile kt+2, then starts tile kt (its first sub-step) while requesting the B
+//   half of tile kt+2. One barrier per iteration, preceded by vmcnt(8): tile kt
+//   has landed for every wave, and the stage tile kt+2 goes to (last read in
+//   iteration kt-1, by fragments every wave has consumed since) is free.
+//   Fragments are double buffered in registers and read one sub-step ahead.
 //
 // Semantics are those of qmm_gemm_b8.hip (same packed weights, same source
 // zero-point compensation through the stored column sums, same epilogue

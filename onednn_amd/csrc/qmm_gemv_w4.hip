@@ -269,7 +269,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
             uint4 wt[UNR];
             uint32_t scp[UNR], zpp[UNR]; // raw scale / zero-point bits per tile
             auto fetch = [&](int tb) {
-    #pragma unroll
+#pragma unroll
                 for (int u = 0; u < UNR; u++) {
                     const int t = tb + wave + u * GEMV_WAVES;
                     wt[u] = make_uint4(0, 0, 0, 0);
@@ -301,11 +301,11 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
             };
             constexpr int ACT_PRE = 2;
             uint4 areg[ACT_PRE];
-    #pragma unroll
+#pragma unroll
             for (int q = 0; q < ACT_PRE; q++)
                 areg[q] = act_load(tid + q * GEMV_WAVES * 64);
             fetch(0);
-    #pragma unroll
+#pragma unroll
             for (int q = 0; q < ACT_PRE; q++) {
                 const int i = tid + q * GEMV_WAVES * 64;
                 if (i < nchunks) *(uint4 *)(lds + (size_t)i * 16) = areg[q];
@@ -317,13 +317,13 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 
             for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
                 if (tb > 0) fetch(tb);
-    #pragma unroll
+#pragma unroll
                 for (int u = 0; u < UNR; u++) {
                     const int t = tb + wave + u * GEMV_WAVES;
                     if (t >= tiles) break;
                     const uint32_t wd[4] = {wt[u].x ^ sflip, wt[u].y ^ sflip,
                             wt[u].z ^ sflip, wt[u].w ^ sflip};
-    #pragma unroll
+#pragma unroll
                     for (int s = 0; s < 4; s++) {
                         const uint32_t d = wd[s];
                         v4u b;
@@ -358,7 +358,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                                 zp = zp_cvt(zp_raw(kq), kq);
                             }
                             const float off = OFFSET + soff + zp;
-    #pragma unroll
+#pragma unroll
                             for (int j = 0; j < 4; j++) {
                                 out[j] = __builtin_fmaf(
                                         sc, P[j] - off * S[j], out[j]);
