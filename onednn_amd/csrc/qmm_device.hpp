@@ -643,10 +643,12 @@ QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
         asm("v_cvt_pk_bf16_f32 %0, %1, %2"
                 : "=v"(h1)
                 : "v"(d[2]), "v"(d[3]));
-        *(uint2 *)((uint16_t *)ep.dst.ptr + dst_off) = make_uint2(h0, h1);
+        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+        *(v2u *)((uint16_t *)ep.dst.ptr + dst_off) = v2u {h0, h1};
     } else {
-        *(float4 *)((float *)ep.dst.ptr + dst_off)
-                = make_float4(d[0], d[1], d[2], d[3]);
+        typedef float v4fl __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(v4fl {d[0], d[1], d[2], d[3]},
+                (v4fl *)((float *)ep.dst.ptr + dst_off));
     }
 }
 
