@@ -58,7 +58,16 @@ enum {
      * k = 128*g + 32*s + 8*c + j for dword s = 0..3, and inside a dword the
      * nibble at bits 4*p..4*p+3 is j = perm(p) = (p%2)*4 + p/2 ... see
      * qmm_w4_nibble_pos(); K padded to 128 and N to 16 with zeros. */
-    QMM_LAYOUT_MFMA_W4 = 2
+    QMM_LAYOUT_MFMA_W4 = 2,
+    /* 4-bit elements for the int8-activation GEMM: per batch,
+     * [N/32][K/64][64 lanes][16 bytes]; lane = 32*h + n%32 holds, in dword
+     * 2*i + q, the eight values k = 64*t + 32*i + 16*h + 8*q + j (j = 0..7),
+     * value j in the nibble at bits 4*p..4*p+3 with p = 2*(j%4) + j/4, so that
+     * (dword << 4) & 0xF0F0F0F0 and dword & 0xF0F0F0F0 are j = 0..3 and
+     * j = 4..7 as bytes holding 16 * value. Values are stored as signed
+     * nibbles: s4 as is, u4 as (u - 8). K padded to 64 and N to 32 with
+     * zeros. */
+    QMM_LAYOUT_MFMA_W4K64 = 3
 };
 
 typedef struct {

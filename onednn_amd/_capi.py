@@ -130,6 +130,7 @@ _SIGNATURES = {
     "qmm_matmul_impl_count": (_I, []),
     "qmm_matmul_impl_name": (C.c_char_p, [_I]),
     "qmm_set_gemm_variant": (None, [_I]),
+    "qmm_set_w4a8_variant": (None, [_I]),
 }
 
 _lib = None
@@ -149,6 +150,7 @@ def lib():
             f.argtypes = args
             f.restype = _I if res is None else res
         L.qmm_set_gemm_variant.restype = None
+        L.qmm_set_w4a8_variant.restype = None
         _lib = L
     return _lib
 

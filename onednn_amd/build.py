@@ -31,7 +31,7 @@ DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",
 UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
          ("qmm_pack.hip", "", []), ("qmm_dispatch.hip", "", []),
          ("qmm_gemm_b8.hip", "", []),
-         ("qmm_gemm_b8x.hip", "", []),
+         ("qmm_gemm_b8x.hip", "", []), ("qmm_gemm_w4a8.hip", "", []),
          ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]
 # the tiled GEMM is instantiated once per tile configuration, each in its own
 # object so the instantiations compile in parallel

@@ -24,6 +24,14 @@ void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream);
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
+void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
+void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
+void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
+void launch_unpack_w4k(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
 void launch_pack_b8(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         bool with_colsum, hipStream_t stream);
@@ -235,7 +243,7 @@ bool fold_quant(ep_tensor_t &e, const generic_quant_t &q, const qmm_quant_t &a,
 
 // Build the compact epilogue; false if the problem does not fit it.
 bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
-        const qmm_matmul_args_t *A) {
+        const qmm_matmul_args_t *A, bool scales_in_kernel = false) {
     const qmm_matmul_desc_t &D = P.desc;
     const int nd = D.dst.ndims;
     std::memset(&ep, 0, sizeof(ep));
@@ -247,7 +255,7 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
         if (!A->bias) ep.bias.ptr = (const void *)1; // shape check only
     }
     const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
-    if (ss.set) {
+    if (ss.set && !scales_in_kernel) {
         if (P.q_src_scale.g1 != P.K && (ss.mask & (1 << (nd - 1))))
             return false; // K-grouped src scales
         if (!fold_quant(ep.src_scale, P.q_src_scale, ss, D.src, D.dst, true,
@@ -255,7 +263,7 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
             return false;
         if (!A->scales[QMM_SRC]) ep.src_scale.ptr = (const void *)1;
     }
-    if (ws.set && !P.decompress) {
+    if (ws.set && !P.decompress && !scales_in_kernel) {
         if ((ws.mask & (1 << (nd - 2))) && P.q_wei_scale.g0 != P.K)
             return false; // K-grouped weights scales
         if (!fold_quant(ep.wei_scale, P.q_wei_scale, ws, D.wei, D.dst, false,
@@ -391,6 +399,75 @@ int supports_gemm_b8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     return QMM_OK;
 }
 
+// K extent of one entry of a scales / zero-points buffer: the group size if it
+// has K groups, 1 if it varies per k without groups, K if it does not vary
+int64_t k_extent(const qmm_quant_t &a, int which, int kbit, int64_t K) {
+    if (!a.set) return K;
+    if (a.has_groups) return group_or(a, which, K);
+    return (a.mask & kbit) ? (int64_t)1 : K;
+}
+
+int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    const int nd = D.dst.ndims;
+    if (nd != 2) return QMM_UNIMPLEMENTED;
+    if (D.src.dt != dt_s8 || !is_int4(D.wei.dt)) return QMM_UNIMPLEMENTED;
+    if (!one_of(D.dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s32, dt_s8, dt_u8}))
+        return QMM_UNIMPLEMENTED;
+    if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
+    if (P.M > (1 << 30) || P.N > (1 << 30) || P.K > 131072)
+        return QMM_UNIMPLEMENTED;
+    if (!one_of(D.wei_layout, {QMM_LAYOUT_PLAIN, QMM_LAYOUT_MFMA_W4K64}))
+        return QMM_UNIMPLEMENTED;
+    if (D.src.strides[1] != 1 || D.src.strides[0] % 16 != 0)
+        return QMM_UNIMPLEMENTED;
+    // whole 64-k tiles per group, every buffer's K extent a whole number of
+    // groups
+    const int64_t gk = P.group_k;
+    if (P.K % 64 != 0 || gk % 64 != 0 || gk > 32768) return QMM_UNIMPLEMENTED;
+    const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
+    const qmm_quant_t &wz = D.zps[QMM_WEI];
+    if (D.zps[QMM_SRC].set) return QMM_UNIMPLEMENTED;
+    if (k_extent(ss, 1, 2, P.K) % gk || k_extent(ws, 0, 1, P.K) % gk
+            || k_extent(wz, 0, 1, P.K) % gk)
+        return QMM_UNIMPLEMENTED;
+    if (ss.set && !one_of(ss.dt, {dt_f32, dt_f16, dt_bf16}))
+        return QMM_UNIMPLEMENTED;
+    if (ws.set) {
+        if (!one_of(ws.dt, {dt_f32, dt_f16, dt_bf16})) return QMM_UNIMPLEMENTED;
+        if (P.q_wei_scale.g1 != 1) return QMM_UNIMPLEMENTED; // N groups
+    }
+    if (wz.set) {
+        if (!one_of(wz.dt, {dt_s32, dt_s8, dt_u8, dt_s4, dt_u4}))
+            return QMM_UNIMPLEMENTED;
+        if (P.q_wei_zp.g1 != 1) return QMM_UNIMPLEMENTED;
+    }
+    epilogue_t ep;
+    if (!build_epilogue(ep, P, nullptr, true)) return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
+// scratchpad of mfma_w4a8 behind the packed weights: the per-group arrays
+struct w4a8_scratch_t {
+    int64_t Mpad, Npad, ng;
+    bool has_zp;
+    size_t ss_off, rs_off, sw_off, zw_off, total;
+};
+w4a8_scratch_t w4a8_scratch(const qmm_matmul_desc_t &D,
+        const generic_params_t &P) {
+    w4a8_scratch_t s;
+    s.Mpad = round_up(P.M, 256) + 256;
+    s.Npad = round_up(P.N, 256) + 256;
+    s.ng = P.ngroups_k;
+    s.has_zp = D.zps[QMM_WEI].set || D.wei.dt == dt_u4;
+    const size_t rows = (size_t)s.ng * s.Mpad * 4, cols = (size_t)s.ng * s.Npad * 4;
+    s.ss_off = 0;
+    s.sw_off = rows;
+    s.rs_off = rows + cols;
+    s.zw_off = s.rs_off + (s.has_zp ? rows : 0);
+    s.total = s.zw_off + (s.has_zp ? cols : 0);
+    return s;
+}
+
 int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
     if (nd != 2) return QMM_UNIMPLEMENTED;
@@ -469,10 +546,11 @@ int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     return QMM_OK;
 }
 
-const char *impl_names[impl_count]
-        = {"hip:gfx950:mfma_b8", "hip:gfx950:decode_w4", "hip:gfx950:generic"};
+const char *impl_names[impl_count] = {"hip:gfx950:mfma_b8",
+        "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:generic"};
 
 int g_gemm_variant = 0;
+int g_w4a8_variant = 0;
 
 } // namespace
 
@@ -502,6 +580,7 @@ int qmm_matmul_impl_supports(int impl, const qmm_matmul_desc_t *desc) {
     build_generic(P, *desc);
     switch (impl) {
         case impl_gemm_b8: return supports_gemm_b8(*desc, P);
+        case impl_gemm_w4a8: return supports_gemm_w4a8(*desc, P);
         case impl_gemv_w4: return supports_gemv_w4(*desc, P);
         case impl_generic: return supports_generic(*desc, P);
         default: return QMM_INVALID_ARGUMENTS;
@@ -514,6 +593,8 @@ size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N) 
         return (size_t)b8_geom(batch, K, N).total_bytes;
     if (layout == QMM_LAYOUT_MFMA_W4)
         return (size_t)w4_geom(batch, K, N).total_bytes;
+    if (layout == QMM_LAYOUT_MFMA_W4K64)
+        return (size_t)w4k_geom(batch, K, N).total_bytes;
     return 0;
 }
 
@@ -523,6 +604,9 @@ int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
     d.wei_layout = QMM_LAYOUT_MFMA_B8;
     if (qmm_matmul_impl_supports(impl_gemm_b8, &d) == QMM_OK)
         return QMM_LAYOUT_MFMA_B8;
+    d.wei_layout = QMM_LAYOUT_MFMA_W4K64;
+    if (qmm_matmul_impl_supports(impl_gemm_w4a8, &d) == QMM_OK)
+        return QMM_LAYOUT_MFMA_W4K64;
     d.wei_layout = QMM_LAYOUT_MFMA_W4;
     if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
         return QMM_LAYOUT_MFMA_W4;
@@ -558,6 +642,15 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
                 : 0;
         const size_t copy = u8_copy_bytes(desc);
         return copy ? round256(packed) + copy : packed;
+    }
+    if (impl == impl_gemm_w4a8) {
+        generic_params_t P;
+        build_generic(P, *desc);
+        const size_t packed = desc->wei_layout == QMM_LAYOUT_PLAIN
+                ? round256(qmm_packed_size(
+                        QMM_LAYOUT_MFMA_W4K64, desc->wei.dt, 1, K, N))
+                : 0;
+        return packed + w4a8_scratch(*desc, P).total;
     }
     if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     if (impl == impl_gemv_w4)
@@ -695,6 +788,72 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             }
         }
         launch_gemm_b8(g, f8, g_gemm_variant, stream);
+    } else if (impl == impl_gemm_w4a8) {
+        w4a8_params_t g;
+        std::memset(&g, 0, sizeof(g));
+        if (!build_epilogue(g.ep, P, args, true))
+            return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
+        const w4k_geom_t geom = w4k_geom(1, P.K, P.N);
+        const uint8_t *packed = (const uint8_t *)args->wei;
+        uint8_t *arrays = (uint8_t *)args->scratch;
+        if (D.wei_layout == QMM_LAYOUT_PLAIN) {
+            launch_pack_w4k(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N, 0,
+                    D.wei.strides[0], D.wei.strides[1], stream);
+            packed = (const uint8_t *)args->scratch;
+            arrays += round256(geom.total_bytes);
+        }
+        const w4a8_scratch_t sc = w4a8_scratch(D, P);
+        const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
+        const qmm_quant_t &wz = D.zps[QMM_WEI];
+        w4a8_prep_t q;
+        std::memset(&q, 0, sizeof(q));
+        q.A = (const uint8_t *)args->src;
+        q.lda = D.src.strides[0];
+        q.ss = ss.set ? args->scales[QMM_SRC] : nullptr;
+        q.sw = ws.set ? args->scales[QMM_WEI] : nullptr;
+        q.zw = wz.set ? args->zps[QMM_WEI] : nullptr;
+        q.ss_dt = ss.dt;
+        q.sw_dt = ws.dt;
+        q.zw_dt = wz.dt;
+        q.w_off = D.wei.dt == dt_u4 ? 8 : 0;
+        q.ss_sm = P.q_src_scale.strides[0];
+        q.ss_sk = P.q_src_scale.strides[1];
+        q.sw_sk = P.q_wei_scale.strides[0];
+        q.sw_sn = P.q_wei_scale.strides[1];
+        q.zw_sk = P.q_wei_zp.strides[0];
+        q.zw_sn = P.q_wei_zp.strides[1];
+        q.ss_g = (int32_t)k_extent(ss, 1, 2, P.K);
+        q.sw_g = (int32_t)k_extent(ws, 0, 1, P.K);
+        q.zw_g = (int32_t)k_extent(wz, 0, 1, P.K);
+        q.M = (int32_t)P.M;
+        q.N = (int32_t)P.N;
+        q.K = (int32_t)P.K;
+        q.gk = (int32_t)P.group_k;
+        q.ng = (int32_t)sc.ng;
+        q.Mpad = (int32_t)sc.Mpad;
+        q.Npad = (int32_t)sc.Npad;
+        q.ssT = (float *)(arrays + sc.ss_off);
+        q.swT = (float *)(arrays + sc.sw_off);
+        q.rsT = sc.has_zp ? (int32_t *)(arrays + sc.rs_off) : nullptr;
+        q.zwT = sc.has_zp ? (int32_t *)(arrays + sc.zw_off) : nullptr;
+        launch_w4a8_prep(q, stream);
+        g.A = q.A;
+        g.lda = q.lda;
+        g.B = packed;
+        g.ssT = q.ssT;
+        g.rsT = q.rsT;
+        g.swT = q.swT;
+        g.zwT = q.zwT;
+        g.M = q.M;
+        g.N = q.N;
+        g.K = q.K;
+        g.Mpad = q.Mpad;
+        g.Npad = q.Npad;
+        g.kt64 = (int32_t)geom.kt64;
+        g.nb32 = (int32_t)geom.nb32;
+        g.tpg = q.gk / 64;
+        g.ng = q.ng;
+        launch_gemm_w4a8(g, g_w4a8_variant, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;
         std::memset(&g, 0, sizeof(g));
@@ -740,6 +899,10 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
 // tuning hook used by the benchmark sweep: tile configuration of mfma_b8
 QMM_API void qmm_set_gemm_variant(int v) {
     g_gemm_variant = v;
+}
+// same for mfma_w4a8 (0: by problem size, 1..3: tile configuration)
+QMM_API void qmm_set_w4a8_variant(int v) {
+    g_w4a8_variant = v;
 }
 
 // ---------------------------------------------------------------------------
@@ -790,7 +953,7 @@ int qmm_reorder_supports(const qmm_reorder_desc_t *d) {
             return QMM_UNIMPLEMENTED;
         return QMM_OK;
     }
-    if (packed == QMM_LAYOUT_MFMA_W4) {
+    if (packed == QMM_LAYOUT_MFMA_W4 || packed == QMM_LAYOUT_MFMA_W4K64) {
         if (!is_int4(pl.dt)) return QMM_UNIMPLEMENTED;
         if (d->dst_layout == QMM_LAYOUT_PLAIN) {
             // unpack writes byte pairs along the stride-1 dim
@@ -854,6 +1017,13 @@ int qmm_reorder_launch(const qmm_reorder_desc_t *d,
                         sn, pl.dt == dt_s8 || pl.dt == dt_u8, stream);
             else
                 launch_unpack_b8(args->src, args->dst, pl.dt, batch, K, N, sb,
+                        sk, sn, stream);
+        } else if (packed == QMM_LAYOUT_MFMA_W4K64) {
+            if (packing)
+                launch_pack_w4k(args->src, args->dst, pl.dt, batch, K, N, sb, sk,
+                        sn, stream);
+            else
+                launch_unpack_w4k(args->src, args->dst, pl.dt, batch, K, N, sb,
                         sk, sn, stream);
         } else {
             if (packing)

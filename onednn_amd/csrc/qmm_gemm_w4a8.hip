@@ -1,0 +1,452 @@
+// hip:gfx950:mfma_w4a8 -- s8 activations x 4-bit weights (s4 / u4) on the int8
+// matrix cores, with scales that vary along K in groups on both operands
+// (dynamically quantized activations, group-quantized weights) and optional
+// grouped weights zero points.
+//
+// The arithmetic is that of src/cpu/matmul/ref_matmul_int8.cpp:139-219 with the
+// group as the unit: inside a K group the products are summed in s32, the
+// group's sum is converted to f32, multiplied by the source scale of (row,
+// group) and the weights scale of (group, column) and added to an f32
+// accumulator; bias / post-ops / dst quantization follow once at the end.
+//
+//   * weights are prepacked (QMM_LAYOUT_MFMA_W4K64): a 32-column x 64-k tile is
+//     1 KiB, a lane's 16 bytes are its two 32-k operand fragments as nibbles.
+//     Every nibble is a signed value w' (s4 as is, u4 minus 8) and is expanded
+//     to the byte 16 * w' with one shift and two ANDs per eight values, so the
+//     MFMA accumulates 16 * sum(s * w'): the factor is a power of two and is
+//     folded into the weights scales;
+//   * zero points and the u4 offset leave the dot product through the row sums
+//     of the source: sum(s * (w - z)) = sum(s * w') - (z - off) * sum(s), all in
+//     s32 (off = 8 for u4, 0 for s4);
+//   * a pre-pass (w4a8_prep_kernel) rewrites the scale and zero-point buffers of
+//     the launch, whatever their data types and strides, as f32 / s32 arrays
+//     [group][row] and [group][column] in the scratchpad and computes the row
+//     sums, so the GEMM fetches the 1 KiB of each that a group of its tile needs
+//     with one direct-to-LDS load;
+//   * a workgroup owns BM x BN of dst; tiles of 64 k are streamed global -> LDS
+//     through a ring of STAGES, one barrier per tile (the scheme of
+//     qmm_gemm_b8.hip). Each wave keeps two accumulator sets: s32 for the
+//     running group (the first MFMA of a group starts from zero) and f32 for
+//     the result. Two workgroups share a CU so that one can rescale while the
+//     other multiplies.
+#include <type_traits>
+
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+namespace w4a8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <int N, typename F>
+QMM_D void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1> {});
+    }
+}
+
+// 16-byte chunk q of row `row` of the row-major 64-byte-wide source tile
+QMM_D int a_swz(int row, int q) {
+    return q ^ ((row >> 2) & 3);
+}
+
+// lane l's 16 bytes go to lds_addr + 16 * l (wave-uniform lds_addr)
+QMM_D void load_to_lds16(const void *gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+constexpr int vmcnt_imm(int n) {
+    return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8);
+}
+
+constexpr int BK = 64;
+constexpr int X_BYTES = 1024; // one per-group array slice in LDS
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool HAS_ZP>
+__global__ void __launch_bounds__(WGM *WGN * 64, 2)
+gemm_w4a8_kernel(const w4a8_params_t p) {
+    constexpr int NW = WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int FM = WM / 32, FN = WN / 32;
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK / 2;
+    constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    constexpr int NX = HAS_ZP ? 4 : 2; // per-group arrays: ss, sw [, rs, zw]
+    constexpr int XSLOT = NX * X_BYTES;
+    constexpr int X_OFF = STAGES * STAGE_BYTES;
+    // wave-wide 1 KiB loads per tile / per group, spread over the waves; a
+    // wave whose share runs past the end repeats earlier ones (same bytes to
+    // the same place), so that every wave issues the same number
+    constexpr int A_W = A_BYTES / 1024, B_W = B_BYTES / 1024;
+    constexpr int TILE_W = A_W + B_W;
+    constexpr int PER_T = (TILE_W + NW - 1) / NW;
+    constexpr int PER_X = (NX + NW - 1) / NW;
+    static_assert(A_W * 1024 == A_BYTES && B_W * 1024 == B_BYTES, "");
+    static_assert(BM <= 256 && BN <= 256, "group arrays are 1 KiB of f32");
+    static_assert(STAGES == 3, "");
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave / WGN) * WM;
+    const int wn0 = (wave % WGN) * WN;
+
+    // XCD-aware tile order: consecutive logical tiles run on one XCD
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt = blockIdx.x;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        if (ntiles >= 64) {
+            lt = xcd * per + slot;
+            if (slot >= per || lt >= ntiles) return;
+        }
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- addresses of this wave's loads ----
+    // Tile loads: index x < A_W is 16 source rows (4 chunks of 16 bytes each,
+    // XOR-swizzled in LDS), the others one packed 32-column weights block.
+    const uint8_t *t_ptr[PER_T];
+    int t_step[PER_T];
+    uint32_t t_lds[PER_T];
+#pragma unroll
+    for (int j = 0; j < PER_T; j++) {
+        const int x = (wave * PER_T + j) % TILE_W; // wave-uniform
+        if (x < A_W) {
+            const int c = x * 64 + lane;
+            const int row = c >> 2, cp = c & 3;
+            const int gm = min(m0 + row, p.M - 1);
+            t_ptr[j] = p.A + (int64_t)gm * p.lda + a_swz(row, cp) * 16;
+            t_step[j] = BK;
+            t_lds[j] = x * 1024;
+        } else {
+            const int y = x - A_W;
+            const int nb = min(n0 / 32 + y, p.nb32 - 1);
+            t_ptr[j] = p.B + (int64_t)nb * p.kt64 * 1024 + lane * 16;
+            t_step[j] = 1024;
+            t_lds[j] = A_BYTES + y * 1024;
+        }
+    }
+    // Group loads: 256 consecutive f32 / s32 of the transposed arrays from the
+    // tile's first row / column on (the arrays are padded so this stays inside)
+    const uint8_t *x_ptr[PER_X];
+    int64_t x_step[PER_X];
+    uint32_t x_lds[PER_X];
+#pragma unroll
+    for (int j = 0; j < PER_X; j++) {
+        const int x = (wave * PER_X + j) % NX;
+        const bool row_side = (x & 1) == 0; // 0: ss, 1: sw, 2: rs, 3: zw
+        const void *base = x == 0 ? (const void *)p.ssT
+                : x == 1          ? (const void *)p.swT
+                : x == 2          ? (const void *)p.rsT
+                                  : (const void *)p.zwT;
+        x_ptr[j] = (const uint8_t *)base
+                + ((int64_t)(row_side ? m0 : n0) + lane * 4) * 4;
+        x_step[j] = (int64_t)(row_side ? p.Mpad : p.Npad) * 4;
+        x_lds[j] = x * X_BYTES;
+    }
+
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    const int KT = p.kt64;
+    // issue state: tile number, its position in its group, the group
+    int is_kt = 0, is_t = 0, is_g = 0;
+    auto issue = [&]() {
+        if (is_t == 0) {
+            const uint32_t xs = lds_base + X_OFF + (is_g % STAGES) * XSLOT;
+#pragma unroll
+            for (int j = 0; j < PER_X; j++)
+                load_to_lds16(x_ptr[j] + is_g * x_step[j], xs + x_lds[j]);
+        }
+        const uint32_t st = lds_base + (is_kt % STAGES) * STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < PER_T; j++)
+            load_to_lds16(t_ptr[j] + (int64_t)is_kt * t_step[j], st + t_lds[j]);
+        is_kt++;
+        if (++is_t == p.tpg) {
+            is_t = 0;
+            is_g++;
+        }
+    };
+
+    v16i acc[FM][FN];
+    v16f res[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[i][j][r] = 0;
+                res[i][j][r] = 0.f;
+            }
+
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; s++)
+        if (s < KT) issue();
+
+    // one 64-k tile: FIRST starts the group's s32 accumulators from zero
+    auto tile_mma = [&](int kt, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
+        // the tile has landed once only younger tiles' loads are in flight (a
+        // younger tile may carry group loads too: then this waits a little
+        // longer than needed, never shorter)
+        if (kt + STAGES - 2 < KT)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * PER_T));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        if (kt + STAGES - 1 < KT) issue();
+
+        const uint8_t *As = lds + (kt % STAGES) * STAGE_BYTES;
+        const uint8_t *Bs = As + A_BYTES;
+        uint4 braw[FN];
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+            braw[j] = *(const uint4 *)(Bs + (((wn0 >> 5) + j) * 64 + lane) * 16);
+#pragma unroll
+        for (int ki = 0; ki < 2; ki++) {
+            v4i a[FM], b[FN];
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                const int row = wm0 + i * 32 + (lane & 31);
+                const int q = ki * 2 + (lane >> 5);
+                const uint4 v = *(const uint4 *)(As + row * BK
+                        + a_swz(row, q) * 16);
+                a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+            }
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                const uint32_t w0 = ki ? braw[j].z : braw[j].x;
+                const uint32_t w1 = ki ? braw[j].w : braw[j].y;
+                b[j] = v4i {(int)((w0 << 4) & 0xF0F0F0F0u),
+                        (int)(w0 & 0xF0F0F0F0u), (int)((w1 << 4) & 0xF0F0F0F0u),
+                        (int)(w1 & 0xF0F0F0F0u)};
+            }
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    if (FIRST && ki == 0) {
+                        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                0, 0, 0};
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                a[i], b[j], zero, 0, 0, 0);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                a[i], b[j], acc[i][j], 0, 0, 0);
+                    }
+                }
+        }
+    };
+
+    int kt = 0;
+    for (int g = 0; g < p.ng; g++) {
+        tile_mma(kt++, std::true_type {});
+        for (int t = 1; t < p.tpg; t++)
+            tile_mma(kt++, std::false_type {});
+
+        // ---- group end: res += (float)(acc [- z * rowsum]) * ss * sw ----
+        // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
+        // column l%32 of its fragment.
+        const uint8_t *xs = lds + X_OFF + (g % STAGES) * XSLOT;
+        const float *ssl = (const float *)xs;
+        const float *swl = (const float *)(xs + X_BYTES);
+        const int32_t *rsl = (const int32_t *)(xs + 2 * X_BYTES);
+        const int32_t *zwl = (const int32_t *)(xs + 3 * X_BYTES);
+        float sw[FN];
+        int zw[FN];
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+            sw[j] = swl[wn0 + j * 32 + (lane & 31)];
+            zw[j] = HAS_ZP ? zwl[wn0 + j * 32 + (lane & 31)] : 0;
+        }
+        static_for<FM>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            float ss[16];
+            int rs[16];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int row = wm0 + i * 32 + 8 * q + 4 * (lane >> 5);
+                const float4 s4 = *(const float4 *)&ssl[row];
+                ss[4 * q + 0] = s4.x;
+                ss[4 * q + 1] = s4.y;
+                ss[4 * q + 2] = s4.z;
+                ss[4 * q + 3] = s4.w;
+                if constexpr (HAS_ZP) {
+                    const int4 r4 = *(const int4 *)&rsl[row];
+                    rs[4 * q + 0] = r4.x;
+                    rs[4 * q + 1] = r4.y;
+                    rs[4 * q + 2] = r4.z;
+                    rs[4 * q + 3] = r4.w;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int t = acc[i][j][r];
+                    if constexpr (HAS_ZP) t += __mul24(zw[j], rs[r]);
+                    res[i][j][r] = __builtin_fmaf(
+                            (float)t * ss[r], sw[j], res[i][j][r]);
+                }
+        });
+    }
+    __syncthreads(); // LDS is reused by the epilogue
+
+    // ---- epilogue: rows back through a wave-private LDS tile, 4 neighbouring
+    // columns per lane, then bias / post-ops / dst conversion ----
+    float *const stg = (float *)lds + wave * (32 * WN);
+    constexpr int ROWS_PER_IT = 256 / WN;
+    const int ecol = (lane % (WN / 4)) * 4;
+    const int en = n0 + wn0 + ecol;
+    const int envalid = min(4, p.N - en);
+    const float one4[4] = {1.f, 1.f, 1.f, 1.f};
+    static_for<FM>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                stg[row * WN + j * 32 + (lane & 31)] = res[i][j][r];
+            }
+#pragma unroll 1
+        for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+            const int row = it * ROWS_PER_IT + lane / (WN / 4);
+            const float4 t = *(const float4 *)&stg[row * WN + ecol];
+            const int m = m0 + wm0 + i * 32 + row;
+            if (m < p.M && en < p.N) {
+                float v[4] = {t.x, t.y, t.z, t.w};
+                if (p.ep.fast != EP_FAST_NONE)
+                    epilogue_fast4(
+                            p.ep, v, false, 1.f, false, one4, 0, m, en, envalid);
+                else
+                    epilogue_apply_store4(p.ep, v, 0, m, en, envalid);
+            }
+        }
+    });
+}
+
+// ---- pre-pass ----
+// One thread per (group, row) and per (group, column).
+__global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
+    const int64_t rows = (int64_t)p.ng * p.M, cols = (int64_t)p.ng * p.N;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+            i < rows + cols; i += (int64_t)gridDim.x * blockDim.x) {
+        if (i < rows) {
+            const int g = (int)(i / p.M), m = (int)(i % p.M);
+            const int k0 = g * p.gk;
+            p.ssT[(int64_t)g * p.Mpad + m] = p.ss
+                    ? load_float(p.ss_dt, p.ss,
+                            m * p.ss_sm + (k0 / p.ss_g) * p.ss_sk)
+                    : 1.f;
+            if (p.rsT) {
+                const uint8_t *a = p.A + (int64_t)m * p.lda + k0;
+                int sum = 0;
+                for (int k = 0; k < p.gk; k += 16) {
+                    const uint4 v = *(const uint4 *)(a + k);
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                        sum += (int)(int8_t)(w[d] & 0xff)
+                                + (int)(int8_t)((w[d] >> 8) & 0xff)
+                                + (int)(int8_t)((w[d] >> 16) & 0xff)
+                                + (int)(int8_t)(w[d] >> 24);
+                }
+                p.rsT[(int64_t)g * p.Mpad + m] = sum;
+            }
+        } else {
+            const int64_t c = i - rows;
+            const int g = (int)(c / p.N), n = (int)(c % p.N);
+            const int k0 = g * p.gk;
+            const float s = p.sw ? load_float(p.sw_dt, p.sw,
+                                    (k0 / p.sw_g) * p.sw_sk + n * p.sw_sn)
+                                 : 1.f;
+            p.swT[(int64_t)g * p.Npad + n] = s * 0.0625f;
+            if (p.zwT) {
+                const int z = p.zw ? load_int(p.zw_dt, p.zw,
+                                      (k0 / p.zw_g) * p.zw_sk + n * p.zw_sn)
+                                   : 0;
+                p.zwT[(int64_t)g * p.Npad + n] = -16 * (z - p.w_off);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool HAS_ZP>
+static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
+    constexpr int STAGES = 3;
+    w4a8_params_t q = p;
+    q.tiles_m = (p.M + BM - 1) / BM;
+    q.tiles_n = (p.N + BN - 1) / BN;
+    const int ntiles = q.tiles_m * q.tiles_n;
+    const int grid_x = ntiles >= 64 ? ((ntiles + 7) / 8) * 8 : ntiles;
+    constexpr size_t lds_main = (size_t)STAGES
+            * (BM * BK + BN * BK / 2 + (HAS_ZP ? 4 : 2) * X_BYTES);
+    constexpr size_t lds_ep
+            = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
+    constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
+    auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, HAS_ZP>;
+    static bool attr_done = false; // one per instantiation
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void *)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x), dim3(WGM * WGN * 64), lds, stream, q);
+}
+
+template <bool HAS_ZP>
+static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
+    switch (variant) {
+        case 1: launch_cfg<128, 128, 2, 2, HAS_ZP>(p, stream); break;
+        case 2: launch_cfg<64, 128, 2, 2, HAS_ZP>(p, stream); break;
+        default: launch_cfg<32, 64, 1, 2, HAS_ZP>(p, stream); break;
+    }
+}
+
+} // namespace w4a8
+
+void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
+    const int64_t total = (int64_t)p.ng * ((int64_t)p.M + p.N);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(w4a8::w4a8_prep_kernel, dim3((unsigned)blocks), dim3(256),
+            0, stream, p);
+}
+
+// variant: 0 = by problem size; 1: 128 x 128, 2: 64 x 128, 3: 32 x 64 tiles
+void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream) {
+    if (p.M <= 0 || p.N <= 0) return;
+    if (variant < 1 || variant > 3) {
+        const int64_t big = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+        const int64_t mid = (int64_t)((p.M + 63) / 64) * ((p.N + 127) / 128);
+        variant = big >= 256 ? 1 : ((mid >= 128 && p.M > 32) ? 2 : 3);
+        if (variant == 3 && p.M > 64) variant = 2;
+    }
+    if (p.zwT)
+        w4a8::launch_zp<true>(p, variant, stream);
+    else
+        w4a8::launch_zp<false>(p, variant, stream);
+}
+
+} // namespace qmm

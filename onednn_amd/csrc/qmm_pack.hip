@@ -1,9 +1,11 @@
 // Weights prepacking: plain strided tensors -> the MFMA operand layouts
-// (QMM_LAYOUT_MFMA_B8 with s32 column sums, QMM_LAYOUT_MFMA_W4) and back.
+// (QMM_LAYOUT_MFMA_B8 with s32 column sums, QMM_LAYOUT_MFMA_W4,
+// QMM_LAYOUT_MFMA_W4K64) and back.
 // This is the reorder a user runs once per weights tensor after asking the
 // matmul primitive descriptor for its weights layout through format_tag any
 // (the role of src/cpu/x64/matmul/brgemm_matmul_reorders.cpp:29-53 in the
-// reference). Values are copied bit for bit; padding is zero.
+// reference). Values are copied bit for bit (u4 in the W4K64 layout: minus 8,
+// undone on the way back); padding is zero.
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
@@ -151,6 +153,69 @@ unpack_w4_kernel(const pack_params_t p, const w4_geom_t g) {
     }
 }
 
+// QMM_LAYOUT_MFMA_W4K64, one thread per packed dword (8 nibbles). u4 values are
+// stored as u - 8 (nibble ^ 8): the int8 GEMM reads every nibble as signed.
+__global__ void __launch_bounds__(256)
+pack_w4k_kernel(const pack_params_t p, const w4k_geom_t g) {
+    const int64_t dwords = p.batch * g.batch_bytes / 4;
+    const uint32_t flip = p.dt == dt_u4 ? 8u : 0u;
+    for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < dwords;
+            d += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t per_b = g.batch_bytes / 4;
+        const int64_t b = d / per_b, db = d % per_b;
+        const int dw = (int)(db % 4);
+        const int lane = (int)((db / 4) % 64);
+        const int64_t tile = db / 256;
+        const int64_t nb = tile / g.kt64, kt = tile % g.kt64;
+        const int64_t n = nb * 32 + (lane & 31);
+        const int64_t kbase
+                = kt * 64 + 32 * (dw / 2) + 16 * (lane >> 5) + 8 * (dw % 2);
+        uint32_t w = 0;
+        if (n < p.N) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int64_t k = kbase + j;
+                if (k >= p.K) continue;
+                const int64_t e = b * p.sb + k * p.sk + n * p.sn;
+                const uint32_t nib = (uint32_t)nibble_at(p.src, e) ^ flip;
+                const int pos = 2 * (j % 4) + j / 4;
+                w |= nib << (4 * pos);
+            }
+        }
+        ((uint32_t *)p.dst)[d] = w;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+unpack_w4k_kernel(const pack_params_t p, const w4k_geom_t g) {
+    const bool n_inner = p.sn == 1;
+    const int64_t total = p.batch * p.K * p.N / 2;
+    const int flip = p.dt == dt_u4 ? 8 : 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        uint8_t out = 0;
+        int64_t e0 = 0;
+        for (int h = 0; h < 2; h++) {
+            const int64_t l = 2 * i + h;
+            int64_t b, k, n;
+            if (n_inner) {
+                n = l % p.N;
+                k = (l / p.N) % p.K;
+                b = l / (p.N * p.K);
+            } else {
+                k = l % p.K;
+                n = (l / p.K) % p.N;
+                b = l / (p.N * p.K);
+            }
+            const int64_t e = b * p.sb + k * p.sk + n * p.sn;
+            if (h == 0) e0 = e;
+            const int64_t ni = b * g.batch_bytes * 2 + w4k_nibble_index(g, k, n);
+            out |= (uint8_t)((nibble_at(p.src, ni) ^ flip) << (4 * (int)(e & 1)));
+        }
+        p.dst[e0 >> 1] = out;
+    }
+}
+
 static unsigned grid_for(int64_t n) {
     int64_t b = (n + 255) / 256;
     if (b < 1) b = 1;
@@ -233,6 +298,27 @@ void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
     pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
             sn, dt, 0};
     hipLaunchKernelGGL(unpack_w4_kernel, dim3(grid_for(batch * K * N / 2)),
+            dim3(256), 0, stream, p, g);
+}
+
+void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4k_geom_t g = w4k_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(pack_w4k_kernel,
+            dim3(grid_for(batch * g.batch_bytes / 4)), dim3(256), 0, stream, p,
+            g);
+}
+
+void launch_unpack_w4k(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4k_geom_t g = w4k_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(unpack_w4k_kernel, dim3(grid_for(batch * K * N / 2)),
             dim3(256), 0, stream, p, g);
 }
 

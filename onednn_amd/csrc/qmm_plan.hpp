@@ -98,6 +98,32 @@ QMM_HD int64_t w4_nibble_index(const w4_geom_t &g, int64_t k, int64_t n) {
     return ((tile * 64 + lane) * 4 + s) * 8 + p;
 }
 
+// QMM_LAYOUT_MFMA_W4K64: nibble index of element (k, n) inside one batch slice.
+struct w4k_geom_t {
+    int64_t K, N, Kpad, Npad, kt64, nb32;
+    int64_t batch_bytes, total_bytes;
+};
+QMM_HD w4k_geom_t w4k_geom(int64_t batch, int64_t K, int64_t N) {
+    w4k_geom_t g;
+    g.K = K;
+    g.N = N;
+    g.Kpad = round_up(K, 64);
+    g.Npad = round_up(N, 32);
+    g.kt64 = g.Kpad / 64;
+    g.nb32 = g.Npad / 32;
+    g.batch_bytes = g.Kpad * g.Npad / 2;
+    g.total_bytes = batch * g.batch_bytes;
+    return g;
+}
+QMM_HD int64_t w4k_nibble_index(const w4k_geom_t &g, int64_t k, int64_t n) {
+    const int64_t tile = (n / 32) * g.kt64 + k / 64;
+    const int64_t kk = k % 64;
+    const int64_t i = kk / 32, h = (kk % 32) / 16, q = (kk % 16) / 8, j = kk % 8;
+    const int64_t lane = 32 * h + (n % 32);
+    const int64_t p = 2 * (j % 4) + j / 4;
+    return ((tile * 64 + lane) * 4 + 2 * i + q) * 8 + p;
+}
+
 // ---- MFMA GEMM (int8 / fp8) -----------------------------------------------
 struct gemm_params_t {
     const uint8_t *A; // src, rows K-contiguous
@@ -138,11 +164,48 @@ struct gemv_params_t {
     epilogue_t ep;
 };
 
+// ---- s8 activations x 4-bit weights, K-grouped scales on both sides ---------
+// The scale / zero-point buffers are rewritten per launch into the scratchpad,
+// transposed to [group][row or column], by w4a8_prep_kernel.
+struct w4a8_params_t {
+    const uint8_t *A; // s8 rows, K-contiguous
+    int64_t lda; // bytes
+    const uint8_t *B; // QMM_LAYOUT_MFMA_W4K64
+    const float *ssT; // [ng][Mpad] source scales
+    const int32_t *rsT; // [ng][Mpad] source row sums per group, or nullptr
+    const float *swT; // [ng][Npad] weights scales / 16
+    const int32_t *zwT; // [ng][Npad] -16 * (zero point - offset), or nullptr
+    int32_t M, N, K;
+    int32_t Mpad, Npad;
+    int32_t kt64, nb32;
+    int32_t tpg; // 64-k tiles per group
+    int32_t ng;
+    int32_t tiles_m, tiles_n;
+    int32_t pad_;
+    epilogue_t ep;
+};
+
+struct w4a8_prep_t {
+    const uint8_t *A;
+    int64_t lda;
+    const void *ss, *sw, *zw; // nullptr: default value
+    int32_t ss_dt, sw_dt, zw_dt;
+    int32_t w_off; // 8 for u4 weights (stored as u - 8)
+    int64_t ss_sm, ss_sk, sw_sk, sw_sn, zw_sk, zw_sn; // strides, elements
+    int32_t ss_g, sw_g, zw_g; // K extent of one entry
+    int32_t M, N, K, gk, ng, Mpad, Npad;
+    float *ssT;
+    int32_t *rsT;
+    float *swT;
+    int32_t *zwT;
+};
+
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
-    impl_gemv_w4 = 1, // decode: 4-bit weights, M small
-    impl_generic = 2,
-    impl_count = 3
+    impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales
+    impl_gemv_w4 = 2, // decode: 4-bit weights, 16-bit activations, M small
+    impl_generic = 3,
+    impl_count = 4
 };
 
 } // namespace qmm
