@@ -42,6 +42,11 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
     return src, wei, ss, ws
 
 
+# side measurements reported next to the headline configuration: key -> function
+EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
+          "attention_scores": "bench_c4", "int8_int4_grouped": "bench_w4a8"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -51,6 +56,8 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="mfma_b8 tile configuration (0 = heuristic)")
     ap.add_argument("--no-extras", action="store_true", help="skip the decode / fp8 side measurements")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default=None, choices=sorted(EXTRAS),
+                    help="run one of the side measurements alone and print its JSON (for profiling)")
     ap.add_argument("--cpu-rows", type=int, default=640, help="rows of config 2 timed on the CPU oracle")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device-to-device copy (reference point for the rocprofv3 "
@@ -83,6 +90,9 @@ def main():
     strm = dnnl.stream(eng)
     hs = C_stream(strm)
     _capi.lib().qmm_set_gemm_variant(args.variant)
+    if args.only:
+        print(json.dumps({args.only: globals()[EXTRAS[args.only]](A, memory, dt, tag, T, eng, strm, hs, hiprt)}))
+        return
 
     # ------------------------------------------------------------------ c2
     M, K, N = 4096, 4096, 14336
@@ -164,10 +174,8 @@ def main():
         out["parity_sample"] = {"rows": rows, "max_bf16_ulp": 1, "frac_off_by_one": round(frac, 6)}
 
     if not args.no_extras:
-        out["decode_gemv"] = bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt)
-        out["fp8_gemm"] = bench_fp8(A, memory, dt, tag, T, eng, strm, hs, hiprt)
-        out["int8_small"] = bench_c1(A, memory, dt, tag, T, eng, strm, hs, hiprt)
-        out["attention_scores"] = bench_c4(A, memory, dt, tag, T, eng, strm, hs, hiprt)
+        for name in EXTRAS:
+            out[name] = globals()[EXTRAS[name]](A, memory, dt, tag, T, eng, strm, hs, hiprt)
     print(json.dumps(out))
 
 
@@ -358,6 +366,66 @@ def bench_c4(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
     return {"ms_per_launch": round(ms, 4), "TOPs": round(2.0 * B * S * S * D / (ms * 1e-3) / 1e12, 1),
             "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str()}
+
+
+def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
+    """Dynamic quantization: s8 [M,4096] with f16 scales per row and 128 k, s4 [4096,14336] with f16 scales per
+    128 k and column, f16 dst (tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu:39,51,63,77). M = 2176 is
+    the prefill shape (MFMA-bound), M = 32 and 1 the decode shapes (bound by the 29 MB weights stream; 8 weight
+    sets are cycled so they do not sit in the last-level cache)."""
+    import oracle as O
+    K, N, G = 4096, 14336, 128
+    r = np.random.default_rng(6)
+    w = O.pack4(r.integers(-8, 8, (K, N)))
+    sw = O.from_f32(O.F16, r.uniform(0.002, 0.02, (K // G, N)).astype(np.float32))
+    plain = memory(memory.desc([K, N], dt.s4, T("ab")), eng).write(w)
+    res = {}
+    wsets = None
+    for M, sets, steps in ((2176, 1, 10), (32, 8, 40), (1, 8, 40)):
+        attr = A.primitive_attr()
+        attr.set_scales(A.DNNL_ARG_SRC, 3, [1, G], dt.f16)
+        attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.s8, T("ab")), memory.desc([K, N], dt.s4, tag.any),
+                                     memory.desc([M, N], dt.f16, T("ab")), attr=attr)
+        prim = A.matmul(pd)
+        if wsets is None:
+            first = memory(pd.weights_desc(), eng)
+            A.reorder(plain, first).execute(strm, plain, first)
+            strm.wait()
+            wsets = [first]
+            for _ in range(7):
+                m = memory(pd.weights_desc(), eng)
+                hiprt.memcpy_dtod(m.get_data_handle(), first.get_data_handle(), pd.weights_desc().get_size())
+                wsets.append(m)
+        m_src = memory(pd.src_desc(), eng).write(np.clip(np.rint(r.standard_normal((M, K)) * 40), -128, 127).astype(np.int8))
+        ss = O.from_f32(O.F16, r.uniform(0.005, 0.05, (M, K // G)).astype(np.float32))
+        m_ss = memory(memory.desc([ss.nbytes], dt.u8, T("a")), eng).write(ss)
+        m_sw = memory(memory.desc([sw.nbytes], dt.u8, T("a")), eng).write(sw)
+        m_dst = memory(pd.dst_desc(), eng)
+
+        def one(i):
+            prim.execute(strm, {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: wsets[i % sets], A.DNNL_ARG_DST: m_dst,
+                                A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: m_ss,
+                                A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: m_sw})
+
+        for i in range(8):
+            one(i)
+        strm.wait()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(hs)
+        for i in range(steps):
+            one(i)
+        e1.record(hs)
+        strm.wait()
+        ms = e1.elapsed_ms(e0) / steps
+        ops = 2.0 * M * K * N
+        nbytes = K * N // 2 + sw.nbytes + ss.nbytes + M * K + M * N * 2
+        res["M%d" % M] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / (ms * 1e-3) / 1e12, 1),
+                          "frac_of_int8_peak": round(ops / (ms * 1e-3) / 1e12 / PEAK_INT8, 4),
+                          "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                          "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4),
+                          "impl": pd.impl_info_str(), "includes": "scale pre-pass + GEMM"}
+    return res
 
 
 if __name__ == "__main__":

@@ -26,6 +26,8 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
+void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
+        hipStream_t stream);
 void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -468,6 +470,33 @@ w4a8_scratch_t w4a8_scratch(const qmm_matmul_desc_t &D,
     return s;
 }
 
+// rows <= 64: how the split-K streaming kernel cuts K
+struct w4a8_small_plan_t {
+    bool use;
+    int splits, gps, ldp;
+    size_t part_bytes;
+};
+w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
+    w4a8_small_plan_t s;
+    std::memset(&s, 0, sizeof(s));
+    s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0;
+    if (!s.use) return s;
+    const int64_t ng = P.ngroups_k;
+    const int64_t nblk = (P.N + 63) / 64;
+    // as many workgroups as the chip holds at once (3 per CU, 2 for 64 rows)
+    const int64_t slots = P.M > 32 ? 512 : 768;
+    int64_t want = slots / nblk;
+    if (want < 1) want = 1;
+    if (want > ng) want = ng;
+    int64_t gps = (ng + want - 1) / want;
+    if (gps > W4A8_SMALL_MAX_GPS) gps = W4A8_SMALL_MAX_GPS;
+    s.gps = (int)gps;
+    s.splits = (int)((ng + gps - 1) / gps);
+    s.ldp = (int)round_up(P.N, 4);
+    s.part_bytes = (size_t)s.splits * P.M * s.ldp * 4;
+    return s;
+}
+
 int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
     if (nd != 2) return QMM_UNIMPLEMENTED;
@@ -650,7 +679,11 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
                 ? round256(qmm_packed_size(
                         QMM_LAYOUT_MFMA_W4K64, desc->wei.dt, 1, K, N))
                 : 0;
-        return packed + w4a8_scratch(*desc, P).total;
+        const w4a8_small_plan_t sm = w4a8_small_plan(P, 0);
+        const size_t big = w4a8_scratch(*desc, P).total;
+        // the tile-configuration override of the tuning hook bypasses the
+        // small-row kernel, so leave room for either
+        return packed + (sm.use && sm.part_bytes > big ? sm.part_bytes : big);
     }
     if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     if (impl == impl_gemv_w4)
@@ -836,6 +869,25 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         q.swT = (float *)(arrays + sc.sw_off);
         q.rsT = sc.has_zp ? (int32_t *)(arrays + sc.rs_off) : nullptr;
         q.zwT = sc.has_zp ? (int32_t *)(arrays + sc.zw_off) : nullptr;
+        const w4a8_small_plan_t sm = w4a8_small_plan(P, g_w4a8_variant);
+        if (sm.use) {
+            w4a8_small_t h;
+            std::memset(&h, 0, sizeof(h));
+            h.q = q;
+            h.B = packed;
+            h.tpg = q.gk / 64;
+            h.kt64 = (int32_t)geom.kt64;
+            h.nb32 = (int32_t)geom.nb32;
+            h.gps = sm.gps;
+            h.splits = sm.splits;
+            h.ldp = sm.ldp;
+            h.part = (float *)arrays;
+            h.ep = g.ep;
+            launch_gemm_w4a8_small(h, sc.has_zp, stream);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return hip_fail(e, "kernel launch");
+            return QMM_OK;
+        }
         launch_w4a8_prep(q, stream);
         g.A = q.A;
         g.lda = q.lda;

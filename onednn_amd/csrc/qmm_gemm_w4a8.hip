@@ -392,6 +392,282 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
     }
 }
 
+// ---- rows <= 64: split-K streaming kernel ----
+// 64 columns x FM*32 rows per workgroup of two waves (32 columns each), a deep
+// ring (8 stages of 64 k) so that a workgroup keeps ~7 tiles in flight: at these
+// sizes the launch is a read of the weights and nothing else matters. The
+// scales / zero points of the workgroup's K slice are converted once into LDS;
+// row sums come from v_dot4 on the source fragments.
+constexpr int SM_STAGES = 8;
+
+template <int FM, bool HAS_ZP>
+__global__ void __launch_bounds__(128)
+w4a8_small_kernel(const w4a8_small_t p) {
+    constexpr int BM = FM * 32, BN = 64;
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK / 2;
+    constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    constexpr int A_W = A_BYTES / 1024, B_W = B_BYTES / 1024;
+    constexpr int PER_T = (A_W + B_W) / 2;
+    constexpr int MAXG = W4A8_SMALL_MAX_GPS;
+    constexpr int SS_OFF = SM_STAGES * STAGE_BYTES;
+    constexpr int SW_OFF = SS_OFF + MAXG * BM * 4;
+    constexpr int ZW_OFF = SW_OFF + MAXG * BN * 4;
+    constexpr int RS_OFF = ZW_OFF + MAXG * BN * 4; // [2 waves][BM] s32
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const w4a8_prep_t &q = p.q;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n0 = blockIdx.x * BN;
+    const int m0 = blockIdx.z * BM;
+    const int split = blockIdx.y;
+    const int g_begin = split * p.gps;
+    const int g_cnt = min(p.gps, q.ng - g_begin);
+    const int kt_begin = g_begin * p.tpg;
+    const int KT = g_cnt * p.tpg; // tiles of this workgroup
+
+    const uint8_t *t_ptr[PER_T];
+    int t_step[PER_T];
+    uint32_t t_lds[PER_T];
+#pragma unroll
+    for (int j = 0; j < PER_T; j++) {
+        const int x = wave * PER_T + j;
+        if (x < A_W) {
+            const int c = x * 64 + lane;
+            const int row = c >> 2, cp = c & 3;
+            const int gm = min(m0 + row, q.M - 1);
+            t_ptr[j] = q.A + (int64_t)gm * q.lda + (int64_t)kt_begin * BK
+                    + a_swz(row, cp) * 16;
+            t_step[j] = BK;
+            t_lds[j] = x * 1024;
+        } else {
+            const int y = x - A_W;
+            const int nb = min(n0 / 32 + y, p.nb32 - 1);
+            t_ptr[j] = p.B + ((int64_t)nb * p.kt64 + kt_begin) * 1024
+                    + lane * 16;
+            t_step[j] = 1024;
+            t_lds[j] = A_BYTES + y * 1024;
+        }
+    }
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    int is_kt = 0;
+    auto issue = [&]() {
+        const uint32_t st = lds_base + (is_kt % SM_STAGES) * STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < PER_T; j++)
+            load_to_lds16(t_ptr[j] + (int64_t)is_kt * t_step[j], st + t_lds[j]);
+        is_kt++;
+    };
+#pragma unroll 1
+    for (int s = 0; s < SM_STAGES - 1; s++)
+        if (s < KT) issue();
+
+    // scales and zero points of the slice -> LDS (f32 / s32, [group][row or
+    // column]); published by the first barrier of the loop
+    {
+        float *ssl = (float *)(lds + SS_OFF);
+        float *swl = (float *)(lds + SW_OFF);
+        int32_t *zwl = (int32_t *)(lds + ZW_OFF);
+        for (int i = tid; i < g_cnt * BM; i += 128) {
+            const int gl = i / BM, r = i % BM;
+            const int k0 = (g_begin + gl) * q.gk;
+            const int m = min(m0 + r, q.M - 1);
+            ssl[i] = q.ss ? load_float(q.ss_dt, q.ss,
+                             m * q.ss_sm + (k0 / q.ss_g) * q.ss_sk)
+                          : 1.f;
+        }
+        for (int i = tid; i < g_cnt * BN; i += 128) {
+            const int gl = i / BN, c = i % BN;
+            const int k0 = (g_begin + gl) * q.gk;
+            const int n = min(n0 + c, q.N - 1);
+            const float s = q.sw ? load_float(q.sw_dt, q.sw,
+                                    (k0 / q.sw_g) * q.sw_sk + n * q.sw_sn)
+                                 : 1.f;
+            swl[i] = s * 0.0625f;
+            if constexpr (HAS_ZP) {
+                const int z = q.zw ? load_int(q.zw_dt, q.zw,
+                                      (k0 / q.zw_g) * q.zw_sk + n * q.zw_sn)
+                                   : 0;
+                zwl[i] = -16 * (z - q.w_off);
+            }
+        }
+    }
+
+    v16i acc[FM];
+    v16f res[FM];
+    int rsum[FM];
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+        rsum[i] = 0;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            acc[i][r] = 0;
+            res[i][r] = 0.f;
+        }
+    }
+
+    auto tile_mma = [&](int kt, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
+        if (kt + SM_STAGES - 2 < KT)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((SM_STAGES - 2) * PER_T));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        if (kt + SM_STAGES - 1 < KT) issue();
+        const uint8_t *As = lds + (kt % SM_STAGES) * STAGE_BYTES;
+        const uint8_t *Bs = As + A_BYTES;
+        const uint4 braw = *(const uint4 *)(Bs + (wave * 64 + lane) * 16);
+#pragma unroll
+        for (int ki = 0; ki < 2; ki++) {
+            const uint32_t w0 = ki ? braw.z : braw.x;
+            const uint32_t w1 = ki ? braw.w : braw.y;
+            const v4i b = {(int)((w0 << 4) & 0xF0F0F0F0u), (int)(w0 & 0xF0F0F0F0u),
+                    (int)((w1 << 4) & 0xF0F0F0F0u), (int)(w1 & 0xF0F0F0F0u)};
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                const int row = i * 32 + (lane & 31);
+                const int cq = ki * 2 + (lane >> 5);
+                const uint4 v = *(const uint4 *)(As + row * BK
+                        + a_swz(row, cq) * 16);
+                const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                if constexpr (HAS_ZP) {
+                    int t = rsum[i];
+                    t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
+                    rsum[i] = t;
+                }
+                if (FIRST && ki == 0) {
+                    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                            0, 0};
+                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                            a, b, zero, 0, 0, 0);
+                } else {
+                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                            a, b, acc[i], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    const float *ssl = (const float *)(lds + SS_OFF);
+    const float *swl = (const float *)(lds + SW_OFF);
+    const int32_t *zwl = (const int32_t *)(lds + ZW_OFF);
+    int32_t *rsw = (int32_t *)(lds + RS_OFF) + wave * BM;
+    int kt = 0;
+    for (int gl = 0; gl < g_cnt; gl++) {
+        tile_mma(kt++, std::true_type {});
+        for (int t = 1; t < p.tpg; t++)
+            tile_mma(kt++, std::false_type {});
+        const float sw = swl[gl * BN + wave * 32 + (lane & 31)];
+        int zw = 0;
+        if constexpr (HAS_ZP) {
+            zw = zwl[gl * BN + wave * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                // both k halves of a row: lanes l and l ^ 32
+                const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
+                rsw[i * 32 + (lane & 31)] = tot;
+                rsum[i] = 0;
+            }
+        }
+        static_for<FM>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int row = i * 32 + 8 * c + 4 * (lane >> 5);
+                const float4 s4 = *(const float4 *)&ssl[gl * BM + row];
+                const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+                int rs[4] = {0, 0, 0, 0};
+                if constexpr (HAS_ZP) {
+                    const int4 r4 = *(const int4 *)&rsw[row];
+                    rs[0] = r4.x;
+                    rs[1] = r4.y;
+                    rs[2] = r4.z;
+                    rs[3] = r4.w;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int t = acc[i][4 * c + e];
+                    if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
+                    res[i][4 * c + e] = __builtin_fmaf(
+                            (float)t * ss[e], sw, res[i][4 * c + e]);
+                }
+            }
+        });
+    }
+
+    // slice result -> part[split][m][n]
+    const int n = n0 + wave * 32 + (lane & 31);
+    if (n < q.N) {
+        float *out = p.part + (int64_t)split * q.M * p.ldp + n;
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4;
+                if (m < q.M) out[(int64_t)m * p.ldp] = res[i][r];
+            }
+    }
+}
+
+// sum of the slices in slice order, then bias / post-ops / dst conversion:
+// one thread per four neighbouring columns of a row
+__global__ void __launch_bounds__(256)
+w4a8_reduce_kernel(const float *part, int splits, int M, int N, int ldp,
+        const epilogue_t ep) {
+    const int n4 = (N + 3) / 4;
+    const int64_t total = (int64_t)M * n4;
+    const float one4[4] = {1.f, 1.f, 1.f, 1.f};
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < splits; s++) {
+            const float4 t
+                    = *(const float4 *)&part[((int64_t)s * M + m) * ldp + n];
+            if (s == 0) {
+                v[0] = t.x;
+                v[1] = t.y;
+                v[2] = t.z;
+                v[3] = t.w;
+            } else {
+                v[0] += t.x;
+                v[1] += t.y;
+                v[2] += t.z;
+                v[3] += t.w;
+            }
+        }
+        const int nvalid = min(4, N - n);
+        if (ep.fast != EP_FAST_NONE)
+            epilogue_fast4(ep, v, false, 1.f, false, one4, 0, m, n, nvalid);
+        else
+            epilogue_apply_store4(ep, v, 0, m, n, nvalid);
+    }
+}
+
+template <int FM, bool HAS_ZP>
+static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
+    constexpr int BM = FM * 32;
+    constexpr size_t lds = (size_t)SM_STAGES * (BM * BK + 64 * BK / 2)
+            + (size_t)W4A8_SMALL_MAX_GPS * (BM * 4 + 64 * 4 + 64 * 4)
+            + 2 * BM * 4;
+    auto kern = w4a8_small_kernel<FM, HAS_ZP>;
+    static bool attr_done = false; // one per instantiation
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void *)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern,
+            dim3((p.q.N + 63) / 64, p.splits, (p.q.M + BM - 1) / BM), dim3(128),
+            lds, stream, p);
+}
+
 template <int BM, int BN, int WGM, int WGN, bool HAS_ZP>
 static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
     constexpr int STAGES = 3;
@@ -432,6 +708,29 @@ void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
     if (blocks > 65535) blocks = 65535;
     hipLaunchKernelGGL(w4a8::w4a8_prep_kernel, dim3((unsigned)blocks), dim3(256),
             0, stream, p);
+}
+
+void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
+        hipStream_t stream) {
+    if (p.q.M <= 0 || p.q.N <= 0) return;
+    const bool two = p.q.M > 32;
+    if (has_zp) {
+        if (two)
+            w4a8::launch_small_cfg<2, true>(p, stream);
+        else
+            w4a8::launch_small_cfg<1, true>(p, stream);
+    } else {
+        if (two)
+            w4a8::launch_small_cfg<2, false>(p, stream);
+        else
+            w4a8::launch_small_cfg<1, false>(p, stream);
+    }
+    const int64_t total = (int64_t)p.q.M * ((p.q.N + 3) / 4);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(w4a8::w4a8_reduce_kernel, dim3((unsigned)blocks),
+            dim3(256), 0, stream, (const float *)p.part, p.splits, p.q.M, p.q.N,
+            p.ldp, p.ep);
 }
 
 // variant: 0 = by problem size; 1: 128 x 128, 2: 64 x 128, 3: 32 x 64 tiles

@@ -200,6 +200,23 @@ struct w4a8_prep_t {
     int32_t *zwT;
 };
 
+// Rows <= 64 (decode): the K range is cut into `splits` slices of `gps` groups,
+// one workgroup per (64 columns, slice); slice results are summed in slice
+// order by w4a8_reduce_kernel, which also runs the epilogue. No pre-pass: the
+// workgroup converts the scales of its slice itself (fields of `q`; its
+// transposed-array pointers are unused).
+struct w4a8_small_t {
+    w4a8_prep_t q;
+    const uint8_t *B; // QMM_LAYOUT_MFMA_W4K64
+    int32_t tpg, kt64, nb32;
+    int32_t gps, splits;
+    int32_t ldp; // row pitch of the partial results, floats
+    float *part; // [splits][M][ldp]
+    epilogue_t ep;
+};
+constexpr int W4A8_SMALL_MAX_GPS = 16; // groups per slice (LDS)
+constexpr int W4A8_SMALL_MAX_M = 64;
+
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
     impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales

@@ -83,6 +83,9 @@ EXACT_CASES = {
     "u4_zp_u4_g192": dict(M=12, K=576, N=192, wei_dt=dt.u4, gs=192, gw=192, gz=192, zp_dt=dt.u4),
     "s4_ba_weights": dict(M=64, K=128, N=64, wei_layout="ba"),
     "m1": dict(M=1, K=512, N=160),
+    "m48_u4_zp": dict(M=48, K=512, N=200, wei_dt=dt.u4, gz=128),
+    "m64_many_groups": dict(M=64, K=2560, N=96, gs=64, gw=64, gz=64, zp_dt=dt.s8),
+    "m5_k4096": dict(M=5, K=4096, N=130, wei_dt=dt.u4),
     "edges": dict(M=129, K=320, N=162, gs=64, gw=64),
 }
 
@@ -123,6 +126,18 @@ def test_w4a8_arbitrary_scales(ctx, variant, dst_dt):
         assert_bf16_within_1ulp(got, want, "bf16", abs_slack=1e-5 * p.term_scale)
     else:  # f16: one ulp is 2^-10 relative
         assert_f32_close(g, w, rel=2.0 ** -10, scale=p.term_scale, what="f16")
+
+
+@pytest.mark.parametrize("M", [1, 24, 40])
+def test_w4a8_decode_rows_arbitrary_scales(ctx, M):
+    """Rows <= 64 take the split-K kernel: slices are summed in slice order,
+    which is not the oracle's group order, hence the f32 bar."""
+    eng, strm = ctx
+    say("mfma_w4a8 decode rows M=%d" % M)
+    p = dynamic_quant(M, 4096, 520, 15 + M, wei_dt=dt.u4, gz=128)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == W4A8
+    assert_f32_close(got, p.run_oracle(), rel=1e-5, scale=p.term_scale, what="decode rows")
 
 
 def test_w4a8_llm_post_ops(ctx):
