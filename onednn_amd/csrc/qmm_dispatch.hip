@@ -28,6 +28,7 @@ void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream);
+bool gemm_w4a8_small_takes(const w4a8_prep_t &q);
 void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -481,14 +482,21 @@ w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     std::memset(&s, 0, sizeof(s));
     s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0;
     if (!s.use) return s;
-    const int64_t ng = P.ngroups_k;
-    const int64_t nblk = (P.N + 63) / 64;
-    // as many workgroups as the chip holds at once (3 per CU, 2 for 64 rows)
-    const int64_t slots = P.M > 32 ? 512 : 768;
+    const int64_t ng = P.ngroups_k, tpg = P.group_k / 64;
+    const int64_t nblk = (P.N + 127) / 128;
+    // as many workgroups as the chip holds at once (2 per CU, 1 for 64 rows),
+    // but no more slices than keep the partial results (written and read once
+    // each) small next to the weights
+    const int64_t slots = P.M > 32 ? 256 : 512;
     int64_t want = slots / nblk;
+    const int64_t cap = P.K / (16 * P.M) > 2 ? P.K / (16 * P.M) : 2;
+    if (want > cap) want = cap;
     if (want < 1) want = 1;
     if (want > ng) want = ng;
     int64_t gps = (ng + want - 1) / want;
+    // a slice of at most one chunk of 16 tiles where the groups allow it
+    const int64_t one_chunk = 16 / tpg > 1 ? 16 / tpg : 1;
+    if (gps > one_chunk) gps = one_chunk;
     if (gps > W4A8_SMALL_MAX_GPS) gps = W4A8_SMALL_MAX_GPS;
     s.gps = (int)gps;
     s.splits = (int)((ng + gps - 1) / gps);
@@ -870,7 +878,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         q.rsT = sc.has_zp ? (int32_t *)(arrays + sc.rs_off) : nullptr;
         q.zwT = sc.has_zp ? (int32_t *)(arrays + sc.zw_off) : nullptr;
         const w4a8_small_plan_t sm = w4a8_small_plan(P, g_w4a8_variant);
-        if (sm.use) {
+        if (sm.use && gemm_w4a8_small_takes(q)) {
             w4a8_small_t h;
             std::memset(&h, 0, sizeof(h));
             h.q = q;

@@ -40,6 +40,7 @@ namespace w4a8 {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 template <int N, typename F>
 QMM_D void static_for(F &&f) {
@@ -70,6 +71,41 @@ constexpr int vmcnt_imm(int n) {
 
 constexpr int BK = 64;
 constexpr int X_BYTES = 1024; // one per-group array slice in LDS
+
+// Scale / zero-point fetch of the small-row kernel in two steps without any
+// control flow, so that a thread issues all its loads before it looks at the
+// first value. SC: bytes of a scale (2: f16 or bf16, 4: f32). ZPK: storage of a
+// zero point (1: s8 / u8, 2: s4 / u4, two per byte).
+template <int SC>
+QMM_D uint32_t scale_raw(const void *p, int64_t idx) {
+    if constexpr (SC == 4)
+        return ((const uint32_t *)p)[idx];
+    else
+        return ((const uint16_t *)p)[idx];
+}
+template <int SC>
+QMM_D float scale_value(int dt, uint32_t raw) {
+    if constexpr (SC == 4) {
+        return u2f(raw);
+    } else {
+        const float h = (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        const float b = u2f(raw << 16);
+        return dt == dt_f16 ? h : b;
+    }
+}
+template <int ZPK>
+QMM_D uint32_t zp_raw(const void *p, int64_t idx) {
+    return ((const uint8_t *)p)[ZPK == 2 ? (idx >> 1) : idx];
+}
+template <int ZPK>
+QMM_D int zp_value(int dt, uint32_t raw, int64_t idx) {
+    if constexpr (ZPK == 2) {
+        const int nib = (int)((raw >> (4 * (int)(idx & 1))) & 0xf);
+        return dt == dt_s4 ? ((nib ^ 8) - 8) : nib;
+    } else {
+        return dt == dt_s8 ? (int)(int8_t)raw : (int)raw;
+    }
+}
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, bool HAS_ZP>
 __global__ void __launch_bounds__(WGM *WGN * 64, 2)
@@ -393,27 +429,33 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
 }
 
 // ---- rows <= 64: split-K streaming kernel ----
-// 64 columns x FM*32 rows per workgroup of two waves (32 columns each), a deep
-// ring (8 stages of 64 k) so that a workgroup keeps ~7 tiles in flight: at these
-// sizes the launch is a read of the weights and nothing else matters. The
-// scales / zero points of the workgroup's K slice are converted once into LDS;
-// row sums come from v_dot4 on the source fragments.
-constexpr int SM_STAGES = 8;
+// At these sizes the launch is one read of the weights and nothing else
+// matters, so the kernel is built around memory-level parallelism: 128 columns
+// x FM*32 rows per workgroup of four waves, each wave owning 32 columns. The
+// packed layout already is the MFMA operand order per lane, so a wave loads
+// its weights fragments straight into registers, SM_CH tiles (1 KiB each) at
+// a time (the host cuts K so that a slice is one chunk where it can), all
+// requested first thing in the kernel; behind them the scales / zero points of
+// the slice (converted once into LDS) and the source rows of the chunk (staged
+// in LDS, shared by the four waves), so the whole workgroup costs one memory
+// round trip. Row sums come from v_dot4 on the source fragments. No pre-pass,
+// no direct-to-LDS loads.
+constexpr int SM_CH = 16; // 64-k tiles per chunk
 
-template <int FM, bool HAS_ZP>
-__global__ void __launch_bounds__(128)
+// HAS_ZP: zero points or u4 weights (row-sum path); ZPK: 0 = no zero-point
+// buffer (the constant u4 offset only), else its storage class.
+template <int FM, int SC, bool HAS_ZP, int ZPK>
+__global__ void __launch_bounds__(256)
 w4a8_small_kernel(const w4a8_small_t p) {
-    constexpr int BM = FM * 32, BN = 64;
-    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK / 2;
-    constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    constexpr int A_W = A_BYTES / 1024, B_W = B_BYTES / 1024;
-    constexpr int PER_T = (A_W + B_W) / 2;
+    constexpr int BM = FM * 32, BN = 128, NT = 256;
     constexpr int MAXG = W4A8_SMALL_MAX_GPS;
-    constexpr int SS_OFF = SM_STAGES * STAGE_BYTES;
+    constexpr int A_BYTES = SM_CH * BM * BK; // [tile][row][64 B], swizzled
+    constexpr int SS_OFF = A_BYTES;
     constexpr int SW_OFF = SS_OFF + MAXG * BM * 4;
     constexpr int ZW_OFF = SW_OFF + MAXG * BN * 4;
-    constexpr int RS_OFF = ZW_OFF + MAXG * BN * 4; // [2 waves][BM] s32
-    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    constexpr int RS_OFF = ZW_OFF + MAXG * BN * 4; // [4 waves][BM] s32
+    constexpr int A_PER = SM_CH * BM * 4 / NT; // 16-byte pieces per thread
+    constexpr int SS_PER = MAXG * BM / NT, SW_PER = MAXG * BN / NT;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const w4a8_prep_t &q = p.q;
@@ -425,76 +467,119 @@ w4a8_small_kernel(const w4a8_small_t p) {
     const int split = blockIdx.y;
     const int g_begin = split * p.gps;
     const int g_cnt = min(p.gps, q.ng - g_begin);
-    const int kt_begin = g_begin * p.tpg;
+    const int T0 = g_begin * p.tpg; // first 64-k tile of the slice
     const int KT = g_cnt * p.tpg; // tiles of this workgroup
 
-    const uint8_t *t_ptr[PER_T];
-    int t_step[PER_T];
-    uint32_t t_lds[PER_T];
+    // Request order = order of use: source rows, scales, then the weights tile
+    // by tile, so that every wait below leaves the younger requests in flight.
+    // source rows of a chunk: piece = 16 bytes, 64 pieces per row
+    uint4 av[A_PER];
+    auto load_rows = [&](int t0, int cnt) {
 #pragma unroll
-    for (int j = 0; j < PER_T; j++) {
-        const int x = wave * PER_T + j;
-        if (x < A_W) {
-            const int c = x * 64 + lane;
-            const int row = c >> 2, cp = c & 3;
-            const int gm = min(m0 + row, q.M - 1);
-            t_ptr[j] = q.A + (int64_t)gm * q.lda + (int64_t)kt_begin * BK
-                    + a_swz(row, cp) * 16;
-            t_step[j] = BK;
-            t_lds[j] = x * 1024;
-        } else {
-            const int y = x - A_W;
-            const int nb = min(n0 / 32 + y, p.nb32 - 1);
-            t_ptr[j] = p.B + ((int64_t)nb * p.kt64 + kt_begin) * 1024
-                    + lane * 16;
-            t_step[j] = 1024;
-            t_lds[j] = A_BYTES + y * 1024;
+        for (int j = 0; j < A_PER; j++) {
+            const int pc = tid + j * NT;
+            const int row = pc >> 6, c16 = pc & 63;
+            av[j] = make_uint4(0, 0, 0, 0);
+            if (m0 + row < q.M && (c16 >> 2) < cnt)
+                av[j] = *(const uint4 *)(q.A + (int64_t)(m0 + row) * q.lda
+                        + (int64_t)(T0 + t0) * BK + c16 * 16);
+        }
+    };
+    auto stage_rows = [&]() {
+#pragma unroll
+        for (int j = 0; j < A_PER; j++) {
+            const int pc = tid + j * NT;
+            const int row = pc >> 6, c16 = pc & 63;
+            const int tl = c16 >> 2, cp = c16 & 3;
+            *(uint4 *)(lds + (tl * BM + row) * BK + a_swz(row, cp) * 16) = av[j];
+        }
+    };
+    // this wave's 32-column block of the packed weights; tiles past the end of
+    // a chunk repeat its last one
+    const int nb = min(n0 / 32 + wave, p.nb32 - 1);
+    const v4u *bsrc = (const v4u *)(p.B + (int64_t)nb * p.kt64 * 1024) + lane;
+    v4u bq[SM_CH];
+    auto load_weights = [&](int t0, int cnt) {
+#pragma unroll
+        for (int j = 0; j < SM_CH; j++)
+            bq[j] = __builtin_nontemporal_load(
+                    bsrc + (int64_t)(T0 + t0 + min(j, cnt - 1)) * 64);
+    };
+
+    load_rows(0, min(SM_CH, KT));
+    // scales and zero points of the slice (f32 / s32 in LDS, [group][row or
+    // column]): all loads of a thread before the first conversion
+    uint32_t rs_[SS_PER], rw_[SW_PER], rz_[SW_PER];
+    int64_t iz_[SW_PER];
+    const bool has_ss = q.ss != nullptr, has_sw = q.sw != nullptr;
+#pragma unroll
+    for (int j = 0; j < SS_PER; j++)
+        rs_[j] = 0;
+#pragma unroll
+    for (int j = 0; j < SW_PER; j++) {
+        rw_[j] = rz_[j] = 0;
+        iz_[j] = 0;
+    }
+    if (has_ss) {
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++) {
+            const int i = tid + j * NT;
+            const int gl = min(i / BM, g_cnt - 1), r = i % BM;
+            const int k0 = (g_begin + gl) * q.gk;
+            const int m = min(m0 + r, q.M - 1);
+            rs_[j] = scale_raw<SC>(q.ss, m * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
         }
     }
-    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(lds_u8 *)lds);
-    int is_kt = 0;
-    auto issue = [&]() {
-        const uint32_t st = lds_base + (is_kt % SM_STAGES) * STAGE_BYTES;
+    if (has_sw) {
 #pragma unroll
-        for (int j = 0; j < PER_T; j++)
-            load_to_lds16(t_ptr[j] + (int64_t)is_kt * t_step[j], st + t_lds[j]);
-        is_kt++;
-    };
-#pragma unroll 1
-    for (int s = 0; s < SM_STAGES - 1; s++)
-        if (s < KT) issue();
+        for (int j = 0; j < SW_PER; j++) {
+            const int i = tid + j * NT;
+            const int gl = min(i / BN, g_cnt - 1), c = i % BN;
+            const int k0 = (g_begin + gl) * q.gk;
+            const int n = min(n0 + c, q.N - 1);
+            rw_[j] = scale_raw<SC>(q.sw, (k0 / q.sw_g) * q.sw_sk + n * q.sw_sn);
+        }
+    }
+    if constexpr (ZPK != 0) {
+#pragma unroll
+        for (int j = 0; j < SW_PER; j++) {
+            const int i = tid + j * NT;
+            const int gl = min(i / BN, g_cnt - 1), c = i % BN;
+            const int k0 = (g_begin + gl) * q.gk;
+            const int n = min(n0 + c, q.N - 1);
+            iz_[j] = (k0 / q.zw_g) * q.zw_sk + n * q.zw_sn;
+            rz_[j] = zp_raw<ZPK>(q.zw, iz_[j]);
+        }
+    }
+    load_weights(0, min(SM_CH, KT));
 
-    // scales and zero points of the slice -> LDS (f32 / s32, [group][row or
-    // column]); published by the first barrier of the loop
+    stage_rows();
     {
         float *ssl = (float *)(lds + SS_OFF);
         float *swl = (float *)(lds + SW_OFF);
         int32_t *zwl = (int32_t *)(lds + ZW_OFF);
-        for (int i = tid; i < g_cnt * BM; i += 128) {
-            const int gl = i / BM, r = i % BM;
-            const int k0 = (g_begin + gl) * q.gk;
-            const int m = min(m0 + r, q.M - 1);
-            ssl[i] = q.ss ? load_float(q.ss_dt, q.ss,
-                             m * q.ss_sm + (k0 / q.ss_g) * q.ss_sk)
-                          : 1.f;
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++) {
+            const int i = tid + j * NT;
+            const float v = scale_value<SC>(q.ss_dt, rs_[j]);
+            if (i < g_cnt * BM) ssl[i] = has_ss ? v : 1.f;
         }
-        for (int i = tid; i < g_cnt * BN; i += 128) {
-            const int gl = i / BN, c = i % BN;
-            const int k0 = (g_begin + gl) * q.gk;
-            const int n = min(n0 + c, q.N - 1);
-            const float s = q.sw ? load_float(q.sw_dt, q.sw,
-                                    (k0 / q.sw_g) * q.sw_sk + n * q.sw_sn)
-                                 : 1.f;
-            swl[i] = s * 0.0625f;
-            if constexpr (HAS_ZP) {
-                const int z = q.zw ? load_int(q.zw_dt, q.zw,
-                                      (k0 / q.zw_g) * q.zw_sk + n * q.zw_sn)
-                                   : 0;
-                zwl[i] = -16 * (z - q.w_off);
+#pragma unroll
+        for (int j = 0; j < SW_PER; j++) {
+            const int i = tid + j * NT;
+            const float v = scale_value<SC>(q.sw_dt, rw_[j]);
+            if (i < g_cnt * BN) {
+                swl[i] = (has_sw ? v : 1.f) * 0.0625f;
+                if constexpr (HAS_ZP) {
+                    int z = 0;
+                    if constexpr (ZPK != 0)
+                        z = zp_value<ZPK>(q.zw_dt, rz_[j], iz_[j]);
+                    zwl[i] = -16 * (z - q.w_off);
+                }
             }
         }
     }
+    __syncthreads();
 
     v16i acc[FM];
     v16f res[FM];
@@ -508,97 +593,108 @@ w4a8_small_kernel(const w4a8_small_t p) {
             res[i][r] = 0.f;
         }
     }
-
-    auto tile_mma = [&](int kt, auto first_tag) {
-        constexpr bool FIRST = decltype(first_tag)::value;
-        if (kt + SM_STAGES - 2 < KT)
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm((SM_STAGES - 2) * PER_T));
-        else
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-        __syncthreads();
-        if (kt + SM_STAGES - 1 < KT) issue();
-        const uint8_t *As = lds + (kt % SM_STAGES) * STAGE_BYTES;
-        const uint8_t *Bs = As + A_BYTES;
-        const uint4 braw = *(const uint4 *)(Bs + (wave * 64 + lane) * 16);
-#pragma unroll
-        for (int ki = 0; ki < 2; ki++) {
-            const uint32_t w0 = ki ? braw.z : braw.x;
-            const uint32_t w1 = ki ? braw.w : braw.y;
-            const v4i b = {(int)((w0 << 4) & 0xF0F0F0F0u), (int)(w0 & 0xF0F0F0F0u),
-                    (int)((w1 << 4) & 0xF0F0F0F0u), (int)(w1 & 0xF0F0F0F0u)};
-#pragma unroll
-            for (int i = 0; i < FM; i++) {
-                const int row = i * 32 + (lane & 31);
-                const int cq = ki * 2 + (lane >> 5);
-                const uint4 v = *(const uint4 *)(As + row * BK
-                        + a_swz(row, cq) * 16);
-                const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-                if constexpr (HAS_ZP) {
-                    int t = rsum[i];
-                    t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
-                    t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
-                    t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
-                    t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
-                    rsum[i] = t;
-                }
-                if (FIRST && ki == 0) {
-                    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
-                            0, 0};
-                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                            a, b, zero, 0, 0, 0);
-                } else {
-                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                            a, b, acc[i], 0, 0, 0);
-                }
-            }
-        }
-    };
-
     const float *ssl = (const float *)(lds + SS_OFF);
     const float *swl = (const float *)(lds + SW_OFF);
     const int32_t *zwl = (const int32_t *)(lds + ZW_OFF);
     int32_t *rsw = (int32_t *)(lds + RS_OFF) + wave * BM;
-    int kt = 0;
-    for (int gl = 0; gl < g_cnt; gl++) {
-        tile_mma(kt++, std::true_type {});
-        for (int t = 1; t < p.tpg; t++)
-            tile_mma(kt++, std::false_type {});
-        const float sw = swl[gl * BN + wave * 32 + (lane & 31)];
-        int zw = 0;
-        if constexpr (HAS_ZP) {
-            zw = zwl[gl * BN + wave * 32 + (lane & 31)];
+    int t_in_g = 0, gl = 0; // position of the next tile in its group; the group
+    const int mrows = min(BM, q.M - m0);
+
+    for (int t0 = 0; t0 < KT; t0 += SM_CH) {
+        const int cnt = min(SM_CH, KT - t0);
+        if (t0 > 0) {
+            load_rows(t0, cnt);
+            load_weights(t0, cnt);
+            __syncthreads(); // everybody is done with the previous chunk's rows
+            stage_rows();
+            __syncthreads();
+        }
 #pragma unroll
-            for (int i = 0; i < FM; i++) {
-                // both k halves of a row: lanes l and l ^ 32
-                const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
-                rsw[i * 32 + (lane & 31)] = tot;
-                rsum[i] = 0;
+        for (int j = 0; j < SM_CH; j++) {
+            if (j < cnt) {
+                const uint8_t *As = lds + j * BM * BK;
+                const bool first = t_in_g == 0; // the group's accumulators start at 0
+#pragma unroll
+                for (int ki = 0; ki < 2; ki++) {
+                    const uint32_t w0 = ki ? bq[j].z : bq[j].x;
+                    const uint32_t w1 = ki ? bq[j].w : bq[j].y;
+                    const v4i b = {(int)((w0 << 4) & 0xF0F0F0F0u),
+                            (int)(w0 & 0xF0F0F0F0u),
+                            (int)((w1 << 4) & 0xF0F0F0F0u),
+                            (int)(w1 & 0xF0F0F0F0u)};
+#pragma unroll
+                    for (int i = 0; i < FM; i++) {
+                        const int row = i * 32 + (lane & 31);
+                        const int cq = ki * 2 + (lane >> 5);
+                        const uint4 v = *(const uint4 *)(As + row * BK
+                                + a_swz(row, cq) * 16);
+                        const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        if constexpr (HAS_ZP) {
+                            int t = rsum[i];
+                            t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
+                            rsum[i] = t;
+                        }
+                        if (ki == 0 && first) {
+                            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                    0, 0, 0, 0};
+                            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    a, b, zero, 0, 0, 0);
+                        } else {
+                            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    a, b, acc[i], 0, 0, 0);
+                        }
+                    }
+                }
+                if (++t_in_g == p.tpg) {
+                    // group end: res += (float)(acc [- z * rowsum]) * ss * sw
+                    t_in_g = 0;
+                    const float sw = swl[gl * BN + wave * 32 + (lane & 31)];
+                    int zw = 0;
+                    if constexpr (HAS_ZP) {
+                        zw = zwl[gl * BN + wave * 32 + (lane & 31)];
+#pragma unroll
+                        for (int i = 0; i < FM; i++) {
+                            // both k halves of a row: lanes l and l ^ 32
+                            const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
+                            rsw[i * 32 + (lane & 31)] = tot;
+                            rsum[i] = 0;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < FM; i++) {
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            // registers 4c..4c+3 are rows 8c..8c+7 of the
+                            // fragment: skip those past the last row
+                            if (i * 32 + 8 * c >= mrows) continue;
+                            const int row = i * 32 + 8 * c + 4 * (lane >> 5);
+                            const float4 s4
+                                    = *(const float4 *)&ssl[gl * BM + row];
+                            const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+                            int rs[4] = {0, 0, 0, 0};
+                            if constexpr (HAS_ZP) {
+                                const int4 r4 = *(const int4 *)&rsw[row];
+                                rs[0] = r4.x;
+                                rs[1] = r4.y;
+                                rs[2] = r4.z;
+                                rs[3] = r4.w;
+                            }
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                int t = acc[i][4 * c + e];
+                                if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
+                                res[i][4 * c + e] = __builtin_fmaf(
+                                        (float)t * ss[e], sw, res[i][4 * c + e]);
+                            }
+                        }
+                    }
+                    gl++;
+                }
             }
         }
-        static_for<FM>([&](auto I) {
-            constexpr int i = decltype(I)::value;
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const int row = i * 32 + 8 * c + 4 * (lane >> 5);
-                const float4 s4 = *(const float4 *)&ssl[gl * BM + row];
-                const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
-                int rs[4] = {0, 0, 0, 0};
-                if constexpr (HAS_ZP) {
-                    const int4 r4 = *(const int4 *)&rsw[row];
-                    rs[0] = r4.x;
-                    rs[1] = r4.y;
-                    rs[2] = r4.z;
-                    rs[3] = r4.w;
-                }
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    int t = acc[i][4 * c + e];
-                    if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
-                    res[i][4 * c + e] = __builtin_fmaf(
-                            (float)t * ss[e], sw, res[i][4 * c + e]);
-                }
-            }
-        });
     }
 
     // slice result -> part[split][m][n]
@@ -650,13 +746,13 @@ w4a8_reduce_kernel(const float *part, int splits, int M, int N, int ldp,
     }
 }
 
-template <int FM, bool HAS_ZP>
+template <int FM, int SC, bool HAS_ZP, int ZPK>
 static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
     constexpr int BM = FM * 32;
-    constexpr size_t lds = (size_t)SM_STAGES * (BM * BK + 64 * BK / 2)
-            + (size_t)W4A8_SMALL_MAX_GPS * (BM * 4 + 64 * 4 + 64 * 4)
-            + 2 * BM * 4;
-    auto kern = w4a8_small_kernel<FM, HAS_ZP>;
+    constexpr size_t lds = (size_t)SM_CH * BM * BK
+            + (size_t)W4A8_SMALL_MAX_GPS * (BM * 4 + 128 * 4 + 128 * 4)
+            + 4 * BM * 4;
+    auto kern = w4a8_small_kernel<FM, SC, HAS_ZP, ZPK>;
     static bool attr_done = false; // one per instantiation
     if (!attr_done) {
         (void)hipFuncSetAttribute((const void *)kern,
@@ -664,8 +760,21 @@ static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
         attr_done = true;
     }
     hipLaunchKernelGGL(kern,
-            dim3((p.q.N + 63) / 64, p.splits, (p.q.M + BM - 1) / BM), dim3(128),
-            lds, stream, p);
+            dim3((p.q.N + 127) / 128, p.splits, (p.q.M + BM - 1) / BM),
+            dim3(256), lds, stream, p);
+}
+
+template <int FM, int SC>
+static void launch_small_zp(const w4a8_small_t &p, bool has_zp, int zpk,
+        hipStream_t stream) {
+    if (!has_zp)
+        launch_small_cfg<FM, SC, false, 0>(p, stream);
+    else if (zpk == 0)
+        launch_small_cfg<FM, SC, true, 0>(p, stream);
+    else if (zpk == 1)
+        launch_small_cfg<FM, SC, true, 1>(p, stream);
+    else
+        launch_small_cfg<FM, SC, true, 2>(p, stream);
 }
 
 template <int BM, int BN, int WGM, int WGN, bool HAS_ZP>
@@ -710,20 +819,35 @@ void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
             0, stream, p);
 }
 
+// Data types the small-row kernel reads directly: both scales of one size
+// (f16 / bf16, or f32) and zero points of one byte or less.
+bool gemm_w4a8_small_takes(const w4a8_prep_t &q) {
+    auto two = [](int dt) { return dt == dt_f16 || dt == dt_bf16; };
+    const int sdt = q.ss ? q.ss_dt : q.sw_dt, wdt = q.sw ? q.sw_dt : q.ss_dt;
+    if ((q.ss || q.sw) && !((two(sdt) && two(wdt)) || (sdt == dt_f32 && wdt == dt_f32)))
+        return false;
+    if (q.zw && q.zw_dt == dt_s32) return false;
+    return true;
+}
+
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream) {
     if (p.q.M <= 0 || p.q.N <= 0) return;
-    const bool two = p.q.M > 32;
-    if (has_zp) {
-        if (two)
-            w4a8::launch_small_cfg<2, true>(p, stream);
+    const w4a8_prep_t &q = p.q;
+    const bool two_frags = q.M > 32;
+    const int sdt = q.ss ? q.ss_dt : q.sw_dt;
+    const bool sc4 = (q.ss || q.sw) && sdt == dt_f32;
+    const int zpk = !q.zw ? 0 : ((q.zw_dt == dt_s4 || q.zw_dt == dt_u4) ? 2 : 1);
+    if (two_frags) {
+        if (sc4)
+            w4a8::launch_small_zp<2, 4>(p, has_zp, zpk, stream);
         else
-            w4a8::launch_small_cfg<1, true>(p, stream);
+            w4a8::launch_small_zp<2, 2>(p, has_zp, zpk, stream);
     } else {
-        if (two)
-            w4a8::launch_small_cfg<2, false>(p, stream);
+        if (sc4)
+            w4a8::launch_small_zp<1, 4>(p, has_zp, zpk, stream);
         else
-            w4a8::launch_small_cfg<1, false>(p, stream);
+            w4a8::launch_small_zp<1, 2>(p, has_zp, zpk, stream);
     }
     const int64_t total = (int64_t)p.q.M * ((p.q.N + 3) / 4);
     int64_t blocks = (total + 255) / 256;
