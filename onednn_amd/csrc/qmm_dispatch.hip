@@ -29,6 +29,8 @@ void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream);
 bool gemm_w4a8_small_takes(const w4a8_prep_t &q);
+void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
+        hipStream_t stream);
 void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -886,6 +888,24 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             h.tpg = q.gk / 64;
             h.kt64 = (int32_t)geom.kt64;
             h.nb32 = (int32_t)geom.nb32;
+            if (P.M <= 4) {
+                // single-token decode: the waves of a workgroup cut K between
+                // them, at most 16 groups and preferably 16 tiles per wave
+                int nwv = 4;
+                int64_t gpw = (q.ng + 3) / 4;
+                if (gpw * h.tpg > 16 || gpw > 16) {
+                    nwv = 8;
+                    gpw = (q.ng + 7) / 8;
+                }
+                if (gpw <= 16) {
+                    h.gps = (int32_t)gpw;
+                    h.ep = g.ep;
+                    launch_gemm_w4a8_tiny(h, sc.has_zp, nwv, stream);
+                    const hipError_t e = hipGetLastError();
+                    if (e != hipSuccess) return hip_fail(e, "kernel launch");
+                    return QMM_OK;
+                }
+            }
             h.gps = sm.gps;
             h.splits = sm.splits;
             h.ldp = sm.ldp;

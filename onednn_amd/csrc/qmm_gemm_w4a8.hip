@@ -127,7 +127,7 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     constexpr int PER_X = (NX + NW - 1) / NW;
     static_assert(A_W * 1024 == A_BYTES && B_W * 1024 == B_BYTES, "");
     static_assert(BM <= 256 && BN <= 256, "group arrays are 1 KiB of f32");
-    static_assert(STAGES == 3, "");
+    static_assert(STAGES >= 3 && STAGES <= 6, "");
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -711,6 +711,243 @@ w4a8_small_kernel(const w4a8_small_t p) {
     }
 }
 
+// ---- rows <= 4 (single-token decode): one launch, no partial results ----
+// A workgroup owns 32 columns; its NWV waves cut K between them (whole groups),
+// each wave exactly as a wave of the kernel above but with everything it
+// stages (its rows of the source, the scales of its groups) in a wave-private
+// piece of LDS, so there is no barrier before the end. The waves' results are
+// summed through LDS in wave order (= K order) by wave 0, which also runs the
+// epilogue. Accumulator registers 0..3 of lanes 0..31 are rows 0..3: the only
+// ones looked at.
+constexpr int TN_ROWS = 4;
+constexpr int TN_AROW = SM_CH * BK + 16; // staged row, padded against conflicts
+constexpr int TN_MAXG = 16; // groups per wave
+constexpr int TN_WAVE_BYTES = TN_ROWS * TN_AROW + TN_MAXG * 4 * 4
+        + TN_MAXG * 32 * 4 + TN_MAXG * 32 * 4;
+
+template <int NWV, int SC, bool HAS_ZP, int ZPK>
+__global__ void __launch_bounds__(NWV * 64)
+w4a8_tiny_kernel(const w4a8_small_t p) {
+    constexpr int SW_PER = TN_MAXG * 32 / 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const w4a8_prep_t &q = p.q;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * 32;
+    const int g_begin = wave * p.gps;
+    const int g_cnt = max(0, min(p.gps, q.ng - g_begin));
+    const int T0 = g_begin * p.tpg;
+    const int KT = g_cnt * p.tpg; // tiles of this wave
+    uint8_t *wA = lds + wave * TN_WAVE_BYTES;
+    float *wss = (float *)(wA + TN_ROWS * TN_AROW);
+    float *wsw = wss + TN_MAXG * 4;
+    int32_t *wzw = (int32_t *)(wsw + TN_MAXG * 32);
+    float *red = (float *)(lds + NWV * TN_WAVE_BYTES); // [NWV][4][32]
+
+    float res[4] = {0.f, 0.f, 0.f, 0.f};
+    if (KT > 0) {
+        // request order = order of use: rows, scales, weights tile by tile
+        uint4 av[TN_ROWS];
+        auto load_rows = [&](int t0, int cnt) {
+#pragma unroll
+            for (int r = 0; r < TN_ROWS; r++) {
+                av[r] = make_uint4(0, 0, 0, 0);
+                if (r < q.M && (lane >> 2) < cnt)
+                    av[r] = *(const uint4 *)(q.A + (int64_t)r * q.lda
+                            + (int64_t)(T0 + t0) * BK + lane * 16);
+            }
+        };
+        auto stage_rows = [&]() {
+#pragma unroll
+            for (int r = 0; r < TN_ROWS; r++)
+                *(uint4 *)(wA + r * TN_AROW + lane * 16) = av[r];
+        };
+        const int nb = min(n0 / 32, p.nb32 - 1);
+        const v4u *bsrc
+                = (const v4u *)(p.B + (int64_t)nb * p.kt64 * 1024) + lane;
+        v4u bq[SM_CH];
+        auto load_weights = [&](int t0, int cnt) {
+#pragma unroll
+            for (int j = 0; j < SM_CH; j++)
+                bq[j] = __builtin_nontemporal_load(
+                        bsrc + (int64_t)(T0 + t0 + min(j, cnt - 1)) * 64);
+        };
+
+        load_rows(0, min(SM_CH, KT));
+        const bool has_ss = q.ss != nullptr, has_sw = q.sw != nullptr;
+        uint32_t rs_ = 0, rw_[SW_PER], rz_[SW_PER];
+        int64_t iz_[SW_PER];
+#pragma unroll
+        for (int j = 0; j < SW_PER; j++) {
+            rw_[j] = rz_[j] = 0;
+            iz_[j] = 0;
+        }
+        if (has_ss) {
+            const int gl = min(lane >> 2, g_cnt - 1), r = min(lane & 3, q.M - 1);
+            const int k0 = (g_begin + gl) * q.gk;
+            rs_ = scale_raw<SC>(q.ss, r * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
+        }
+        if (has_sw) {
+#pragma unroll
+            for (int j = 0; j < SW_PER; j++) {
+                const int i = lane + j * 64;
+                const int gl = min(i >> 5, g_cnt - 1), c = i & 31;
+                const int k0 = (g_begin + gl) * q.gk;
+                const int n = min(n0 + c, q.N - 1);
+                rw_[j] = scale_raw<SC>(
+                        q.sw, (k0 / q.sw_g) * q.sw_sk + n * q.sw_sn);
+            }
+        }
+        if constexpr (ZPK != 0) {
+#pragma unroll
+            for (int j = 0; j < SW_PER; j++) {
+                const int i = lane + j * 64;
+                const int gl = min(i >> 5, g_cnt - 1), c = i & 31;
+                const int k0 = (g_begin + gl) * q.gk;
+                const int n = min(n0 + c, q.N - 1);
+                iz_[j] = (k0 / q.zw_g) * q.zw_sk + n * q.zw_sn;
+                rz_[j] = zp_raw<ZPK>(q.zw, iz_[j]);
+            }
+        }
+        load_weights(0, min(SM_CH, KT));
+
+        stage_rows();
+        {
+            const float v = scale_value<SC>(q.ss_dt, rs_);
+            wss[lane] = has_ss ? v : 1.f;
+        }
+#pragma unroll
+        for (int j = 0; j < SW_PER; j++) {
+            const int i = lane + j * 64;
+            const float v = scale_value<SC>(q.sw_dt, rw_[j]);
+            wsw[i] = (has_sw ? v : 1.f) * 0.0625f;
+            if constexpr (HAS_ZP) {
+                int z = 0;
+                if constexpr (ZPK != 0) z = zp_value<ZPK>(q.zw_dt, rz_[j], iz_[j]);
+                wzw[i] = -16 * (z - q.w_off);
+            }
+        }
+
+        v16i acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            acc[r] = 0;
+        int rsum = 0;
+        int t_in_g = 0, gl = 0;
+        const int arow = min(lane & 31, q.M - 1) * TN_AROW + (lane >> 5) * 16;
+        for (int t0 = 0; t0 < KT; t0 += SM_CH) {
+            const int cnt = min(SM_CH, KT - t0);
+            if (t0 > 0) {
+                load_rows(t0, cnt);
+                load_weights(t0, cnt);
+                stage_rows();
+            }
+#pragma unroll
+            for (int j = 0; j < SM_CH; j++) {
+                if (j < cnt) {
+                    const bool first = t_in_g == 0;
+#pragma unroll
+                    for (int ki = 0; ki < 2; ki++) {
+                        const uint32_t w0 = ki ? bq[j].z : bq[j].x;
+                        const uint32_t w1 = ki ? bq[j].w : bq[j].y;
+                        const v4i b = {(int)((w0 << 4) & 0xF0F0F0F0u),
+                                (int)(w0 & 0xF0F0F0F0u),
+                                (int)((w1 << 4) & 0xF0F0F0F0u),
+                                (int)(w1 & 0xF0F0F0F0u)};
+                        const uint4 v = *(const uint4 *)(wA + arow
+                                + (j * 4 + ki * 2) * 16);
+                        const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        if constexpr (HAS_ZP) {
+                            int t = rsum;
+                            t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
+                            rsum = t;
+                        }
+                        if (ki == 0 && first) {
+                            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                    0, 0, 0, 0};
+                            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    a, b, zero, 0, 0, 0);
+                        } else {
+                            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    a, b, acc, 0, 0, 0);
+                        }
+                    }
+                    if (++t_in_g == p.tpg) {
+                        t_in_g = 0;
+                        const float sw = wsw[gl * 32 + (lane & 31)];
+                        const float4 s4 = *(const float4 *)&wss[gl * 4];
+                        const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+                        int zw = 0, tot = 0;
+                        if constexpr (HAS_ZP) {
+                            zw = wzw[gl * 32 + (lane & 31)];
+                            // both k halves of a row: lanes l and l ^ 32;
+                            // row r of the source sits in lane r
+                            tot = rsum + __shfl_xor(rsum, 32);
+                            rsum = 0;
+                        }
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            int t = acc[r];
+                            if constexpr (HAS_ZP)
+                                t += __mul24(zw,
+                                        __builtin_amdgcn_readlane(tot, r));
+                            res[r] = __builtin_fmaf(
+                                    (float)t * ss[r], sw, res[r]);
+                        }
+                        gl++;
+                    }
+                }
+            }
+        }
+    }
+
+    if (lane < 32) {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            red[(wave * 4 + r) * 32 + lane] = res[r];
+    }
+    __syncthreads();
+    if (wave == 0 && lane < 32) {
+        const int n = n0 + lane;
+        for (int r = 0; r < q.M; r++) {
+            float v = red[r * 32 + lane];
+            for (int w = 1; w < NWV; w++)
+                v += red[(w * 4 + r) * 32 + lane];
+            if (n < q.N) epilogue_apply_store(p.ep, v, 0, r, n);
+        }
+    }
+}
+
+template <int NWV, int SC, bool HAS_ZP, int ZPK>
+static void launch_tiny_cfg(const w4a8_small_t &p, hipStream_t stream) {
+    constexpr size_t lds = (size_t)NWV * TN_WAVE_BYTES + NWV * 4 * 32 * 4;
+    auto kern = w4a8_tiny_kernel<NWV, SC, HAS_ZP, ZPK>;
+    static bool attr_done = false; // one per instantiation
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void *)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((p.q.N + 31) / 32), dim3(NWV * 64), lds,
+            stream, p);
+}
+
+template <int NWV, int SC>
+static void launch_tiny_zp(const w4a8_small_t &p, bool has_zp, int zpk,
+        hipStream_t stream) {
+    if (!has_zp)
+        launch_tiny_cfg<NWV, SC, false, 0>(p, stream);
+    else if (zpk == 0)
+        launch_tiny_cfg<NWV, SC, true, 0>(p, stream);
+    else if (zpk == 1)
+        launch_tiny_cfg<NWV, SC, true, 1>(p, stream);
+    else
+        launch_tiny_cfg<NWV, SC, true, 2>(p, stream);
+}
+
 // sum of the slices in slice order, then bias / post-ops / dst conversion:
 // one thread per four neighbouring columns of a row
 __global__ void __launch_bounds__(256)
@@ -779,7 +1016,9 @@ static void launch_small_zp(const w4a8_small_t &p, bool has_zp, int zpk,
 
 template <int BM, int BN, int WGM, int WGN, bool HAS_ZP>
 static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
-    constexpr int STAGES = 3;
+    // a tile is only 8 MFMAs per wave: five stages (four tiles in flight) are
+    // what it takes to cover the L2 / HBM latency; two workgroups still fit
+    constexpr int STAGES = 5;
     w4a8_params_t q = p;
     q.tiles_m = (p.M + BM - 1) / BM;
     q.tiles_n = (p.N + BN - 1) / BN;
@@ -828,6 +1067,28 @@ bool gemm_w4a8_small_takes(const w4a8_prep_t &q) {
         return false;
     if (q.zw && q.zw_dt == dt_s32) return false;
     return true;
+}
+
+// Single-token decode kernel: nwv waves per workgroup (4 or 8), p.gps groups
+// per wave; p.part / p.splits are unused.
+void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
+        hipStream_t stream) {
+    if (p.q.M <= 0 || p.q.N <= 0) return;
+    const w4a8_prep_t &q = p.q;
+    const int sdt = q.ss ? q.ss_dt : q.sw_dt;
+    const bool sc4 = (q.ss || q.sw) && sdt == dt_f32;
+    const int zpk = !q.zw ? 0 : ((q.zw_dt == dt_s4 || q.zw_dt == dt_u4) ? 2 : 1);
+    if (nwv == 8) {
+        if (sc4)
+            w4a8::launch_tiny_zp<8, 4>(p, has_zp, zpk, stream);
+        else
+            w4a8::launch_tiny_zp<8, 2>(p, has_zp, zpk, stream);
+    } else {
+        if (sc4)
+            w4a8::launch_tiny_zp<4, 4>(p, has_zp, zpk, stream);
+        else
+            w4a8::launch_tiny_zp<4, 2>(p, has_zp, zpk, stream);
+    }
 }
 
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,

@@ -86,6 +86,9 @@ EXACT_CASES = {
     "m48_u4_zp": dict(M=48, K=512, N=200, wei_dt=dt.u4, gz=128),
     "m64_many_groups": dict(M=64, K=2560, N=96, gs=64, gw=64, gz=64, zp_dt=dt.s8),
     "m5_k4096": dict(M=5, K=4096, N=130, wei_dt=dt.u4),
+    "m1_k4096_zp": dict(M=1, K=4096, N=200, wei_dt=dt.u4, gz=128),
+    "m3_k2048_g64": dict(M=3, K=2048, N=70, gs=64, gw=64, gz=64, zp_dt=dt.s4),
+    "m4_k8192": dict(M=4, K=8192, N=96),
     "edges": dict(M=129, K=320, N=162, gs=64, gw=64),
 }
 
@@ -128,7 +131,7 @@ def test_w4a8_arbitrary_scales(ctx, variant, dst_dt):
         assert_f32_close(g, w, rel=2.0 ** -10, scale=p.term_scale, what="f16")
 
 
-@pytest.mark.parametrize("M", [1, 24, 40])
+@pytest.mark.parametrize("M", [1, 3, 24, 40])
 def test_w4a8_decode_rows_arbitrary_scales(ctx, M):
     """Rows <= 64 take the split-K kernel: slices are summed in slice order,
     which is not the oracle's group order, hence the f32 bar."""
@@ -138,6 +141,16 @@ def test_w4a8_decode_rows_arbitrary_scales(ctx, M):
     got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
     assert pd.impl_info_str() == W4A8
     assert_f32_close(got, p.run_oracle(), rel=1e-5, scale=p.term_scale, what="decode rows")
+
+
+def test_w4a8_single_token_long_k(ctx):
+    """K = 14336: eight waves per workgroup, two chunks of tiles per wave."""
+    eng, strm = ctx
+    say("mfma_w4a8 M=2 K=14336")
+    p = dynamic_quant(2, 14336, 96, 31, wei_dt=dt.u4, gz=128, zp_dt=dt.u4, dst_dt=dt.f32)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == W4A8
+    assert_f32_close(got, p.run_oracle(), rel=1e-5, scale=p.term_scale, what="long K")
 
 
 def test_w4a8_llm_post_ops(ctx):
