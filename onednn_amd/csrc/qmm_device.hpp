@@ -340,7 +340,9 @@ struct epilogue_t {
     const int32_t *dst_zp; // s32; index dst_zp_sn * n
     int64_t dst_zp_sn;
     int32_t fast; // EP_FAST_* shape recognised by the host, 0: interpret
-    int32_t pad_;
+    // the shape additionally has a per-column bias, a dst scale / zero point
+    // or an f16 / s8 / u8 dst: only epilogue_full4<.., EXT> runs it straight
+    int32_t fast_ext;
     ep_postop_t po[EP_MAX_PO];
 };
 
@@ -391,67 +393,147 @@ QMM_D void epilogue_apply_store(const epilogue_t &ep, float acc, int64_t b,
     store_float(ep.dst.dt, d, (void *)ep.dst.ptr, dst_off);
 }
 
-// Four consecutive n at once (n % 4 == 0): the tiled GEMM hands its results
-// over row-wise so that a lane owns 4 neighbours of a dst row and 16 lanes
-// cover 64 columns; stores are 4-element vectors when the row is dense and
-// aligned. `nvalid` (1..4) masks the tail of a row.
-QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
-        int64_t b, int64_t m, int64_t n, int nvalid) {
-    if (ep.src_scale.ptr) {
-        const float s = ep_load(ep.src_scale, b, m, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            d[i] *= s;
+// Four elements per dispatch: the algorithm switch is taken once per row piece
+// instead of once per element (the kernels are otherwise busy jumping).
+#define QMM_ELT4(expr) \
+    { \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) { \
+            const float s = d[i]; \
+            d[i] = (expr)*scale; \
+        } \
+    } \
+    break;
+QMM_D void eltwise_fwd4(int alg, float (&d)[4], float alpha, float beta,
+        float scale) {
+    switch (alg) {
+        case alg_relu:
+        case alg_relu_dst: QMM_ELT4(s > 0 ? s : s * alpha)
+        case alg_swish: QMM_ELT4(s * logistic_f(alpha * s))
+        case alg_logistic:
+        case alg_logistic_dst: QMM_ELT4(logistic_f(s))
+        case alg_linear: QMM_ELT4(alpha * s + beta)
+        case alg_tanh:
+        case alg_tanh_dst: QMM_ELT4(tanhf(s))
+        case alg_gelu_tanh: QMM_ELT4(eltwise_fwd(alg_gelu_tanh, s, alpha, beta))
+        case alg_gelu_erf: QMM_ELT4(eltwise_fwd(alg_gelu_erf, s, alpha, beta))
+        case alg_clip: QMM_ELT4(eltwise_fwd(alg_clip, s, alpha, beta))
+        case alg_clip_v2:
+        case alg_clip_v2_dst: QMM_ELT4(eltwise_fwd(alg_clip_v2, s, alpha, beta))
+        case alg_hardswish: QMM_ELT4(s * hardsigmoid_f(s, alpha, beta))
+        case alg_hardsigmoid: QMM_ELT4(hardsigmoid_f(s, alpha, beta))
+        case alg_abs: QMM_ELT4(s > 0 ? s : -s)
+        case alg_square: QMM_ELT4(s * s)
+        case alg_exp:
+        case alg_exp_dst: QMM_ELT4(expf(s))
+        default: QMM_ELT4(eltwise_fwd(alg, s, alpha, beta))
     }
-    if (ep.wei_scale.ptr) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < nvalid) d[i] *= ep_load(ep.wei_scale, b, 0, n + i);
+}
+#undef QMM_ELT4
+#define QMM_BIN4(expr) \
+    { \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) { \
+            const float x = d[i], y = o[i]; \
+            d[i] = (expr); \
+        } \
+    } \
+    break;
+QMM_D void binary_op4(int alg, float (&d)[4], const float (&o)[4]) {
+    switch (alg) {
+        case alg_bin_add: QMM_BIN4(x + y)
+        case alg_bin_mul: QMM_BIN4(x * y)
+        case alg_bin_sub: QMM_BIN4(x - y)
+        case alg_bin_max: QMM_BIN4(x > y ? x : y)
+        case alg_bin_min: QMM_BIN4(x < y ? x : y)
+        case alg_bin_div: QMM_BIN4(x / y)
+        default: QMM_BIN4(binary_op(alg, x, y))
     }
-    if (ep.bias.ptr) {
+}
+#undef QMM_BIN4
+
+// ---- the same tail for four consecutive n at once (n % 4 == 0) -------------
+// The tiled kernels hand their results over row-wise: a lane owns 4 neighbouring
+// columns of every row it visits. What depends on the column only (weights
+// scales, a per-column bias, dst zero points, the inverted dst scale) is
+// fetched once per tile into ep_cols_t; row operands (binary / sum / prelu) are
+// read as 4-element vectors where the tensor is dense and aligned; f16 results
+// are converted by the hardware (round to nearest even, subnormals kept; NaNs
+// go through the bit-exact software conversion). The operation order is the
+// reference's, as in epilogue_apply_store().
+struct ep_cols_t {
+    float ws[4], bias[4], zp[4];
+    float inv_dst_scale;
+    int32_t has_ws, has_bias, bias_per_row, has_ds, has_zp;
+};
+
+QMM_D void epilogue_cols_load(const epilogue_t &ep, ep_cols_t &c, int64_t b,
+        int64_t n, int nvalid) {
+    c.has_ws = ep.wei_scale.ptr != nullptr;
+    c.has_bias = ep.bias.ptr != nullptr;
+    c.bias_per_row = c.has_bias && ep.bias.sm != 0;
+    c.has_ds = ep.dst_scale != nullptr;
+    c.has_zp = ep.dst_zp != nullptr;
+    c.inv_dst_scale
+            = c.has_ds ? 1.f / load_float(ep.dst_scale_dt, ep.dst_scale, 0) : 1.f;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < nvalid) d[i] += ep_load(ep.bias, b, m, n + i);
-    }
-    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n * ep.dst.sn;
-#pragma unroll 1
-    for (int pi = 0; pi < ep.npo; pi++) {
-        const ep_postop_t &e = ep.po[pi];
-        if (e.kind == pk_eltwise) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                d[i] = eltwise_fwd(e.alg, d[i], e.alpha, e.beta) * e.scale;
-        } else if (e.kind == pk_sum) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (i < nvalid) {
-                    const float old = load_float(
-                            e.t.dt, ep.dst.ptr, dst_off + i * ep.dst.sn);
-                    d[i] += e.scale * (old - (float)e.zero_point);
-                }
-        } else if (e.kind == pk_binary) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (i < nvalid)
-                    d[i] = binary_op(e.alg, d[i], ep_load(e.t, b, m, n + i));
-        } else if (e.kind == pk_prelu) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (i < nvalid && d[i] < 0)
-                    d[i] = ep_load(e.t, b, m, n + i) * d[i];
+    for (int i = 0; i < 4; i++) {
+        c.ws[i] = 1.f;
+        c.bias[i] = 0.f;
+        c.zp[i] = 0.f;
+        if (i < nvalid) {
+            if (c.has_ws) c.ws[i] = ep_load(ep.wei_scale, b, 0, n + i);
+            if (c.has_bias && !c.bias_per_row)
+                c.bias[i] = ep_load(ep.bias, b, 0, n + i);
+            if (c.has_zp) c.zp[i] = (float)ep.dst_zp[ep.dst_zp_sn * (n + i)];
         }
     }
-    if (ep.dst_scale) {
-        const float inv = 1.f / load_float(ep.dst_scale_dt, ep.dst_scale, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            d[i] *= inv;
+}
+
+QMM_D uint16_t f32_to_f16_hw(float x) {
+    return __builtin_bit_cast(uint16_t, (_Float16)x);
+}
+
+// four values of a (b, m, n..n+3) tensor operand
+QMM_D void ep_load4(const ep_tensor_t &t, int64_t b, int64_t m, int64_t n,
+        int nvalid, float (&o)[4]) {
+    const int64_t off = b * t.sb + m * t.sm + n * t.sn;
+    if (t.sn == 0) {
+        const float v = load_float(t.dt, t.ptr, off);
+        o[0] = o[1] = o[2] = o[3] = v;
+        return;
     }
-    if (ep.dst_zp) {
+    if (t.sn == 1 && nvalid == 4) {
+        if (t.dt == dt_f32) {
+            const float *q = (const float *)t.ptr + off;
+            if (((uintptr_t)q & 15) == 0) {
+                const float4 v = *(const float4 *)q;
+                o[0] = v.x;
+                o[1] = v.y;
+                o[2] = v.z;
+                o[3] = v.w;
+                return;
+            }
+        } else if (t.dt == dt_f16 || t.dt == dt_bf16) {
+            const uint16_t *q = (const uint16_t *)t.ptr + off;
+            if (((uintptr_t)q & 7) == 0) {
+                const uint2 v = *(const uint2 *)q;
+                const uint16_t h[4] = {(uint16_t)v.x, (uint16_t)(v.x >> 16),
+                        (uint16_t)v.y, (uint16_t)(v.y >> 16)};
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < nvalid) d[i] += (float)ep.dst_zp[ep.dst_zp_sn * (n + i)];
+                for (int i = 0; i < 4; i++)
+                    o[i] = t.dt == dt_f16
+                            ? (float)__builtin_bit_cast(_Float16, h[i])
+                            : bf16_to_f32(h[i]);
+                return;
+            }
+        }
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        o[i] = i < nvalid ? load_float(t.dt, t.ptr, off + i * t.sn) : 0.f;
+}
+
+QMM_D void epilogue_store4(const epilogue_t &ep, const float (&d)[4],
+        int64_t dst_off, int nvalid) {
     void *dst = (void *)ep.dst.ptr;
     const int dt = ep.dst.dt;
     if (nvalid == 4 && ep.dst.sn == 1) {
@@ -459,9 +541,20 @@ QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
             uint16_t *q = (uint16_t *)dst + dst_off;
             if (((uintptr_t)q & 7) == 0) {
                 uint16_t h[4];
+                if (dt == dt_bf16) {
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    h[i] = dt == dt_bf16 ? f32_to_bf16(d[i]) : f32_to_f16(d[i]);
+                    for (int i = 0; i < 4; i++)
+                        h[i] = f32_to_bf16(d[i]);
+                } else if (d[0] != d[0] || d[1] != d[1] || d[2] != d[2]
+                        || d[3] != d[3]) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        h[i] = f32_to_f16(d[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        h[i] = f32_to_f16_hw(d[i]);
+                }
                 *(uint2 *)q = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16),
                         (uint32_t)h[2] | ((uint32_t)h[3] << 16));
                 return;
@@ -490,6 +583,81 @@ QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
 #pragma unroll
     for (int i = 0; i < 4; i++)
         if (i < nvalid) store_float(dt, d[i], dst, dst_off + i * ep.dst.sn);
+}
+
+QMM_D void epilogue_post_op4(const epilogue_t &ep, const ep_postop_t &e,
+        float (&d)[4], int64_t b, int64_t m, int64_t n, int nvalid) {
+    if (e.kind == pk_eltwise) {
+        eltwise_fwd4(e.alg, d, e.alpha, e.beta, e.scale);
+    } else if (e.kind == pk_sum) {
+        ep_tensor_t t = ep.dst;
+        t.dt = e.t.dt;
+        float old[4];
+        ep_load4(t, b, m, n, nvalid, old);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] += e.scale * (old[i] - (float)e.zero_point);
+    } else if (e.kind == pk_binary) {
+        float y[4];
+        ep_load4(e.t, b, m, n, nvalid, y);
+        binary_op4(e.alg, d, y);
+    } else if (e.kind == pk_prelu) {
+        float w[4];
+        ep_load4(e.t, b, m, n, nvalid, w);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (d[i] < 0) d[i] = w[i] * d[i];
+    }
+}
+
+// d[i]: (float)acc of columns n..n+3 of row m; ss: the row's source scale
+QMM_D void epilogue_rows4(const epilogue_t &ep, const ep_cols_t &c,
+        float (&d)[4], bool has_ss, float ss, int64_t b, int64_t m, int64_t n,
+        int nvalid) {
+    // an absent scale is the factor 1.0f: x * 1.0f is x bit for bit, so the
+    // multiplications need no branch (has_ss only says where ss came from)
+    (void)has_ss;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        d[i] = d[i] * ss * c.ws[i];
+    if (c.has_bias) {
+        if (c.bias_per_row) {
+            float bv[4];
+            ep_load4(ep.bias, b, m, n, nvalid, bv);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] += bv[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] += c.bias[i];
+        }
+    }
+    const int64_t dst_off = b * ep.dst.sb + m * ep.dst.sm + n * ep.dst.sn;
+    // The first two post-ops are addressed with constant indices: what they
+    // read from the parameter block does not depend on the row, so a caller's
+    // row loop fetches it once instead of once per row.
+    if (ep.npo > 0) epilogue_post_op4(ep, ep.po[0], d, b, m, n, nvalid);
+    if (ep.npo > 1) epilogue_post_op4(ep, ep.po[1], d, b, m, n, nvalid);
+#pragma unroll 1
+    for (int pi = 2; pi < ep.npo; pi++)
+        epilogue_post_op4(ep, ep.po[pi], d, b, m, n, nvalid);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        d[i] *= c.inv_dst_scale; // 1.0f when there is no dst scale
+        d[i] = c.has_zp ? d[i] + c.zp[i] : d[i];
+    }
+    epilogue_store4(ep, d, dst_off, nvalid);
+}
+
+// one-off form: column operands fetched on the spot
+QMM_D void epilogue_apply_store4(const epilogue_t &ep, float (&d)[4],
+        int64_t b, int64_t m, int64_t n, int nvalid) {
+    ep_cols_t c;
+    epilogue_cols_load(ep, c, b, n, nvalid);
+    const bool has_ss = ep.src_scale.ptr != nullptr;
+    const float ss = has_ss ? ep_load(ep.src_scale, b, m, 0) : 1.f;
+    epilogue_rows4(ep, c, d, has_ss, ss, b, m, n, nvalid);
 }
 
 // Straight-line epilogue for the EP_FAST_* shapes: d[i] is (float)acc of four
@@ -588,9 +756,17 @@ QMM_D void epilogue_flush_denormals() {
     __builtin_amdgcn_s_setreg(1 | (4 << 6) | (1 << 11), 0);
 }
 
-template <int FAST, bool BF16>
-QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
-        const float (&ws4)[4], int64_t bz, int64_t m, int64_t en) {
+// Straight-line epilogue of the 256 x 256 kernels for full tiles: no control
+// flow at all, so that eight rows are in flight at a time. FAST is the post-op
+// shape, DSTK the dst type (EP_DST_*); EXT adds what ep.fast_ext announces: a
+// per-column bias, the dst scale and dst zero points, each applied through a
+// select or as the factor 1.0f so that an absent one changes no bit.
+enum : int { EP_DST_F32 = 0, EP_DST_BF16 = 1, EP_DST_F16 = 2, EP_DST_S8 = 3,
+    EP_DST_U8 = 4 };
+
+template <int FAST, int DSTK, bool EXT>
+QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
+        float (&d)[4], float ss, int64_t bz, int64_t m, int64_t en) {
     const float alpha = FAST == EP_FAST_RELU || FAST == EP_FAST_SWISH
             ? ep.po[0].alpha
             : 0.f;
@@ -599,7 +775,12 @@ QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
     // absent scales are 1.0 (exact)
 #pragma unroll
     for (int i = 0; i < 4; i++)
-        d[i] = d[i] * ss * ws4[i];
+        d[i] = d[i] * ss * c.ws[i];
+    if constexpr (EXT) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = c.has_bias ? d[i] + c.bias[i] : d[i];
+    }
     const int64_t dst_off = bz * ep.dst.sb + m * ep.dst.sm + en;
     if constexpr (FAST == EP_FAST_RELU) {
 #pragma unroll
@@ -619,23 +800,52 @@ QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
         d[2] += y.z;
         d[3] += y.w;
     } else if constexpr (FAST == EP_FAST_SUM) {
-        if constexpr (BF16) {
-            const uint2 o = *(const uint2 *)((const uint16_t *)ep.dst.ptr
+        static_assert(FAST != EP_FAST_SUM || DSTK <= EP_DST_F16, "");
+        float o[4];
+        if constexpr (DSTK == EP_DST_F32) {
+            const float4 v = *(const float4 *)((const float *)ep.dst.ptr
                     + dst_off);
-            d[0] += sum_scale * (u2f(o.x << 16) - 0.f);
-            d[1] += sum_scale * (u2f(o.x & 0xFFFF0000u) - 0.f);
-            d[2] += sum_scale * (u2f(o.y << 16) - 0.f);
-            d[3] += sum_scale * (u2f(o.y & 0xFFFF0000u) - 0.f);
+            o[0] = v.x;
+            o[1] = v.y;
+            o[2] = v.z;
+            o[3] = v.w;
         } else {
-            const float4 o = *(const float4 *)((const float *)ep.dst.ptr
+            const uint2 v = *(const uint2 *)((const uint16_t *)ep.dst.ptr
                     + dst_off);
-            d[0] += sum_scale * (o.x - 0.f);
-            d[1] += sum_scale * (o.y - 0.f);
-            d[2] += sum_scale * (o.z - 0.f);
-            d[3] += sum_scale * (o.w - 0.f);
+            if constexpr (DSTK == EP_DST_BF16) {
+                o[0] = u2f(v.x << 16);
+                o[1] = u2f(v.x & 0xFFFF0000u);
+                o[2] = u2f(v.y << 16);
+                o[3] = u2f(v.y & 0xFFFF0000u);
+            } else {
+                o[0] = (float)__builtin_bit_cast(_Float16, (uint16_t)v.x);
+                o[1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v.x >> 16));
+                o[2] = (float)__builtin_bit_cast(_Float16, (uint16_t)v.y);
+                o[3] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v.y >> 16));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] += sum_scale * (o[i] - 0.f);
+    }
+    if constexpr (EXT) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            d[i] *= c.inv_dst_scale;
+            d[i] = c.has_zp ? d[i] + c.zp[i] : d[i];
         }
     }
-    if constexpr (BF16) {
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    if constexpr (DSTK == EP_DST_BF16) {
+        if constexpr (EXT) {
+            // f32 subnormals convert to +-0 (src/common/bfloat16.cpp:22-56); the
+            // kernels that never take this branch get that from the FP mode
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] = __builtin_fabsf(d[i]) < 1.17549435e-38f
+                        ? __builtin_copysignf(0.f, d[i])
+                        : d[i];
+        }
         uint32_t h0, h1;
         asm("v_cvt_pk_bf16_f32 %0, %1, %2"
                 : "=v"(h0)
@@ -643,8 +853,26 @@ QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
         asm("v_cvt_pk_bf16_f32 %0, %1, %2"
                 : "=v"(h1)
                 : "v"(d[2]), "v"(d[3]));
-        typedef unsigned v2u __attribute__((ext_vector_type(2)));
         *(v2u *)((uint16_t *)ep.dst.ptr + dst_off) = v2u {h0, h1};
+    } else if constexpr (DSTK == EP_DST_F16) {
+        const uint32_t h0 = (uint32_t)f32_to_f16_hw(d[0])
+                | ((uint32_t)f32_to_f16_hw(d[1]) << 16);
+        const uint32_t h1 = (uint32_t)f32_to_f16_hw(d[2])
+                | ((uint32_t)f32_to_f16_hw(d[3]) << 16);
+        *(v2u *)((uint16_t *)ep.dst.ptr + dst_off) = v2u {h0, h1};
+    } else if constexpr (DSTK == EP_DST_S8 || DSTK == EP_DST_U8) {
+        const float lo = DSTK == EP_DST_S8 ? -128.f : 0.f;
+        const float hi = DSTK == EP_DST_S8 ? 127.f : 255.f;
+        uint32_t w = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float v = d[i];
+            v = v < lo ? lo : v;
+            v = v > hi ? hi : v;
+            const int r = (int)__builtin_rintf(v); // NaN -> 0, as the reference's low byte
+            w |= (uint32_t)(r & 0xff) << (8 * i);
+        }
+        *(uint32_t *)((uint8_t *)ep.dst.ptr + dst_off) = w;
     } else {
         typedef float v4fl __attribute__((ext_vector_type(4)));
         __builtin_nontemporal_store(v4fl {d[0], d[1], d[2], d[3]},
@@ -656,7 +884,7 @@ QMM_D void epilogue_full4(const epilogue_t &ep, float (&d)[4], float ss,
 // aligned for vector access
 QMM_D bool epilogue_full4_ok(const epilogue_t &ep) {
     bool ok = (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
-            && ((uintptr_t)ep.dst.ptr & 15) == 0;
+            && ((uintptr_t)ep.dst.ptr & 15) == 0 && ep.fast != EP_FAST_NONE;
     if (ep.fast == EP_FAST_ADD)
         ok = ok && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
                 && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;

@@ -317,10 +317,13 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
     }
     // straight-line shapes (see EP_FAST_* in qmm_device.hpp)
     ep.fast = EP_FAST_NONE;
+    ep.fast_ext = 0;
     const bool scales_f32 = (!ep.src_scale.ptr || ep.src_scale.dt == dt_f32)
             && (!ep.wei_scale.ptr || ep.wei_scale.dt == dt_f32);
-    if (scales_f32 && !ep.bias.ptr && !ep.dst_scale && !ep.dst_zp
-            && ep.dst.sn == 1 && (ep.dst.dt == dt_bf16 || ep.dst.dt == dt_f32)
+    const bool dst_base = ep.dst.dt == dt_bf16 || ep.dst.dt == dt_f32;
+    const bool dst_more = one_of(ep.dst.dt, {dt_f16, dt_s8, dt_u8});
+    const bool bias_ok = !ep.bias.ptr || ep.bias.sm == 0; // per column
+    if (scales_f32 && bias_ok && ep.dst.sn == 1 && (dst_base || dst_more)
             && ep.npo <= 1) {
         if (ep.npo == 0) {
             ep.fast = EP_FAST_PLAIN;
@@ -335,9 +338,12 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
                     && o.t.dt == dt_f32 && o.t.sn == 1)
                 ep.fast = EP_FAST_ADD;
             else if (o.kind == pk_sum && o.zero_point == 0
-                    && o.t.dt == ep.dst.dt)
+                    && o.t.dt == ep.dst.dt
+                    && one_of(ep.dst.dt, {dt_f32, dt_bf16, dt_f16}))
                 ep.fast = EP_FAST_SUM;
         }
+        if (ep.fast != EP_FAST_NONE)
+            ep.fast_ext = ep.bias.ptr || ep.dst_scale || ep.dst_zp || dst_more;
     }
     return true;
 }

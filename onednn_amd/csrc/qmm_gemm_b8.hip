@@ -318,14 +318,10 @@ gemm_b8_kernel(const gemm_params_t p) {
     const int envalid = min(4, p.N - en);
     const bool has_ss = p.ep.src_scale.ptr != nullptr;
     const bool has_ws = p.ep.wei_scale.ptr != nullptr;
-    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
-    if (p.ep.fast != EP_FAST_NONE && has_ws) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < envalid)
-                ws4[i] = ((const float *)p.ep.wei_scale.ptr)[bz * p.ep.wei_scale.sb
-                        + (int64_t)(en + i) * p.ep.wei_scale.sn];
-    }
+    // what depends on the lane's 4 columns only, fetched once
+    ep_cols_t cols;
+    epilogue_cols_load(p.ep, cols, bz, en, envalid > 0 ? envalid : 0);
+    const float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
 #pragma unroll
@@ -349,15 +345,13 @@ gemm_b8_kernel(const gemm_params_t p) {
             const int m = m0 + wm0 + i * 32 + row;
             if (m < p.M && en < p.N) {
                 float v[4] = {t.x, t.y, t.z, t.w};
-                if (p.ep.fast != EP_FAST_NONE) {
-                    float ss = 1.f;
-                    if (has_ss)
-                        ss = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
-                                + m * p.ep.src_scale.sm];
+                const float ss = has_ss ? ep_load(p.ep.src_scale, bz, m, 0) : 1.f;
+                if (p.ep.fast != EP_FAST_NONE && !p.ep.fast_ext)
                     epilogue_fast4(
                             p.ep, v, has_ss, ss, has_ws, ws4, bz, m, en, envalid);
-                } else
-                    epilogue_apply_store4(p.ep, v, bz, m, en, envalid);
+                else
+                    epilogue_rows4(
+                            p.ep, cols, v, has_ss, ss, bz, m, en, envalid);
             }
         }
     });

@@ -205,10 +205,11 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 
 // Epilogue of 64 staged rows when the wave's 128 x 128 tile lies fully inside
 // the matrix and the dst rows are vector-aligned: no per-lane conditions, so
-// the rows pipeline. FAST is the recognised epilogue shape, BF16 the dst type.
-template <int FAST, bool BF16, bool F8>
+// the rows pipeline. FAST is the recognised epilogue shape, DSTK the dst type,
+// EXT whether bias / dst scale / dst zero point take part (epilogue_full4).
+template <int FAST, int DSTK, bool EXT, bool F8>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
-        const float *ssl, int lane, const float (&ws4)[4],
+        const float *ssl, int lane, const ep_cols_t &cols,
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
     const int ecol = (lane & 31) * 4;
 #pragma unroll 8
@@ -229,7 +230,7 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
             d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
             d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
         }
-        epilogue_full4<FAST, BF16>(ep, d, ss, ws4, bz, m, en);
+        epilogue_full4<FAST, DSTK, EXT>(ep, cols, d, ss, bz, m, en);
     }
 }
 
@@ -258,32 +259,36 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     const bool has_ss = ep.src_scale.ptr != nullptr;
     const bool has_ws = ep.wei_scale.ptr != nullptr;
     const bool to_bf16 = ep.dst.dt == dt_bf16;
-    float ws4[4] = {1.f, 1.f, 1.f, 1.f};
+    const bool ext = ep.fast_ext != 0;
+    const int dstk = ep.dst.dt == dt_f32 ? EP_DST_F32
+            : ep.dst.dt == dt_bf16       ? EP_DST_BF16
+            : ep.dst.dt == dt_f16        ? EP_DST_F16
+            : ep.dst.dt == dt_s8         ? EP_DST_S8
+                                         : EP_DST_U8;
+    // what depends on the lane's 4 columns only: weights scales, a per-column
+    // bias, dst zero points, the zero-point compensation
+    ep_cols_t cols;
+    epilogue_cols_load(ep, cols, bz, en, envalid > 0 ? envalid : 0);
+    float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     int cs4[4] = {0, 0, 0, 0};
     {
         int comp = p.a_is_u8 ? 128 : 0;
         if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
 #pragma unroll
         for (int i = 0; i < 4; i++)
-            if (i < envalid) {
-                if (has_ws)
-                    ws4[i] = ((const float *)ep.wei_scale.ptr)[bz * ep.wei_scale.sb
-                            + (int64_t)(en + i) * ep.wei_scale.sn];
-                if (comp != 0 && p.colsum)
-                    cs4[i] = comp
-                            * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
-            }
+            if (i < envalid && comp != 0 && p.colsum)
+                cs4[i] = comp * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
     }
     // bf16 results: the reference conversion maps f32 subnormals to +-0
     // (src/common/bfloat16.cpp:22-56). With single-precision denormals flushed
     // for the rest of the wave's life, the last multiply of the chain (or the
     // packed conversion's input stage) produces that zero and
     // v_cvt_pk_bf16_f32 does the round-to-nearest-even.
-    if (to_bf16) epilogue_flush_denormals();
+    if (to_bf16 && !ext && ep.fast != EP_FAST_NONE) epilogue_flush_denormals();
     // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
     // operand's rows) aligned for vector access
     const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
-            && epilogue_full4_ok(ep);
+            && ep.fast != EP_FAST_NONE && epilogue_full4_ok(ep);
     static_for<2>([&](auto H) {
         constexpr int h = decltype(H)::value;
 #pragma unroll
@@ -301,13 +306,28 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
         if (full) {
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
+#define QX_EP_ROWS(F, D, X) \
+    ep_rows_full<F, D, X, F8>(ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en)
+#define QX_EP_DST(F) \
+    switch (dstk) { \
+        case EP_DST_F32: \
+            if (ext) QX_EP_ROWS(F, EP_DST_F32, true); \
+            else QX_EP_ROWS(F, EP_DST_F32, false); \
+            break; \
+        case EP_DST_BF16: \
+            if (ext) QX_EP_ROWS(F, EP_DST_BF16, true); \
+            else QX_EP_ROWS(F, EP_DST_BF16, false); \
+            break; \
+        case EP_DST_F16: QX_EP_ROWS(F, EP_DST_F16, true); break; \
+        case EP_DST_S8: \
+            if constexpr (F != EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_S8, true); \
+            break; \
+        default: \
+            if constexpr (F != EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_U8, true); \
+            break; \
+    }
 #define QX_EP_CASE(F) \
-    case F: \
-        if (to_bf16) \
-            ep_rows_full<F, true, F8>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
-        else \
-            ep_rows_full<F, false, F8>(ep, stg_r, ssh, lane, ws4, cs4, bz, m_first, en); \
-        break;
+    case F: QX_EP_DST(F) break;
             switch (ep.fast) {
                 QX_EP_CASE(EP_FAST_PLAIN)
                 QX_EP_CASE(EP_FAST_RELU)
@@ -316,9 +336,11 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
                 QX_EP_CASE(EP_FAST_SUM)
                 default: break;
             }
+#undef QX_EP_ROWS
+#undef QX_EP_DST
 #undef QX_EP_CASE
         } else {
-#pragma unroll 1
+#pragma unroll 2
             for (int it = 0; it < 32; it++) {
                 const int row = it * 2 + (lane >> 5);
                 const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
@@ -338,7 +360,10 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
                         v[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
                         v[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
                     }
-                    if (to_bf16 && envalid == 4)
+                    if (ep.fast == EP_FAST_NONE || ext)
+                        epilogue_rows4(
+                                ep, cols, v, has_ss, ss, bz, m, en, envalid);
+                    else if (to_bf16 && envalid == 4)
                         epilogue_fast4_bf16(
                                 ep, v, has_ss, ss, has_ws, ws4, bz, m, en);
                     else
@@ -459,8 +484,9 @@ gemm_b8x_kernel(const gemm_params_t p) {
     {
         float s = 1.f;
         if (p.ep.src_scale.ptr)
-            s = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
-                    + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm];
+            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
+                    bz * p.ep.src_scale.sb
+                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
         ((float *)(lds + SS_OFF))[tid] = s;
     }
 
@@ -693,8 +719,9 @@ gemm_f8x_kernel(const gemm_params_t p) {
     {
         float s = 1.f;
         if (p.ep.src_scale.ptr)
-            s = ((const float *)p.ep.src_scale.ptr)[bz * p.ep.src_scale.sb
-                    + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm];
+            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
+                    bz * p.ep.src_scale.sb
+                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
         ((float *)(lds + SS_OFF))[tid] = s;
     }
 
@@ -775,7 +802,7 @@ static bool short_k(const gemm_params_t &p) {
 }
 
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
-    if (p.ep.fast == EP_FAST_NONE || p.K % 64 != 0 || p.K < 64) return false;
+    if (p.K % 64 != 0 || p.K < 64) return false;
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
     if (p.a_is_u8 && !p.a_preflipped && !short_k(p)) return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;

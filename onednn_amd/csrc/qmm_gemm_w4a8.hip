@@ -356,6 +356,8 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     const int en = n0 + wn0 + ecol;
     const int envalid = min(4, p.N - en);
     const float one4[4] = {1.f, 1.f, 1.f, 1.f};
+    ep_cols_t cols;
+    epilogue_cols_load(p.ep, cols, 0, en, envalid > 0 ? envalid : 0);
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
 #pragma unroll
@@ -372,11 +374,12 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
             const int m = m0 + wm0 + i * 32 + row;
             if (m < p.M && en < p.N) {
                 float v[4] = {t.x, t.y, t.z, t.w};
-                if (p.ep.fast != EP_FAST_NONE)
+                if (p.ep.fast != EP_FAST_NONE && !p.ep.fast_ext)
                     epilogue_fast4(
                             p.ep, v, false, 1.f, false, one4, 0, m, en, envalid);
                 else
-                    epilogue_apply_store4(p.ep, v, 0, m, en, envalid);
+                    epilogue_rows4(
+                            p.ep, cols, v, false, 1.f, 0, m, en, envalid);
             }
         }
     });
@@ -976,7 +979,7 @@ w4a8_reduce_kernel(const float *part, int splits, int M, int N, int ldp,
             }
         }
         const int nvalid = min(4, N - n);
-        if (ep.fast != EP_FAST_NONE)
+        if (ep.fast != EP_FAST_NONE && !ep.fast_ext)
             epilogue_fast4(ep, v, false, 1.f, false, one4, 0, m, n, nvalid);
         else
             epilogue_apply_store4(ep, v, 0, m, n, nvalid);

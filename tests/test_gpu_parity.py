@@ -305,6 +305,55 @@ TILE256_CASES = {
 }
 
 
+# dst types, bias and dst quantization on the 256 x 256 kernel: straight-line
+# for full tiles (512-row cases), the row interpreter on edge tiles and for
+# post-op chains. The arithmetic is the reference's step for step, so integer
+# and f16 results without a transcendental are compared bit for bit.
+TILE256_EPILOGUE_CASES = {
+    "s8_bias_relu_dst_scale_zp": (lambda: int8_linear(512, 256, 512, 91, src_dt=dt.s8, dst_dt=dt.s8, src_zp=None, per_token=True,
+                                                      bias_dt=dt.f32, dst_scale=0.37, dst_zp=[3],
+                                                      post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]), True),
+    "u8_bias_bf16_dst_scale_edges": (lambda: int8_linear(300, 256, 260, 92, src_dt=dt.s8, dst_dt=dt.u8, src_zp=None,
+                                                         bias_dt=dt.bf16, dst_scale=0.21, dst_zp=[100]), True),
+    "s8_zp_per_n": (lambda: int8_linear(512, 320, 256, 93, src_dt=dt.s8, dst_dt=dt.s8, src_zp=2, dst_scale=0.5,
+                                        dst_zp=np.arange(256) % 7 - 3, dst_zp_per_n=True), True),
+    "f16_plain": (lambda: int8_linear(512, 256, 512, 94, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None, per_token=True), True),
+    "f16_bias_relu_edges": (lambda: int8_linear(260, 256, 300, 95, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None, bias_dt=dt.f16,
+                                                post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.25}]), True),
+    "f16_swish": (lambda: int8_linear(512, 256, 256, 96, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None, per_token=True,
+                                      post_ops=[{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]), False),
+    "bf16_bias_f32": (lambda: int8_linear(512, 256, 256, 97, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True,
+                                          bias_dt=dt.f32), True),
+    "f32_bias_dst_scale": (lambda: int8_linear(256, 256, 512, 98, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, bias_dt=dt.f32,
+                                               dst_scale=3.0), True),
+    "f32_gelu_then_linear_chain": (lambda: int8_linear(256, 256, 256, 99, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None,
+                                                       post_ops=[{"kind": "eltwise", "alg": A.eltwise_clip_v2, "alpha": -2.0, "beta": 3.0},
+                                                                 {"kind": "eltwise", "alg": A.eltwise_linear, "alpha": 0.5, "beta": 1.0},
+                                                                 {"kind": "eltwise", "alg": A.eltwise_abs}]), True),
+    "f16_sum": (lambda: int8_linear(512, 256, 256, 100, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None,
+                                    post_ops=[{"kind": "sum", "scale": 0.5}]), True),
+}
+
+
+@pytest.mark.parametrize("name", sorted(TILE256_EPILOGUE_CASES))
+def test_mfma_int8_tile256_epilogue_surface(ctx, tile256, name):
+    eng, strm = ctx
+    say("mfma_b8 256x256 kernel epilogue %s" % name)
+    build, exact = TILE256_EPILOGUE_CASES[name]
+    p = build()
+    init = None
+    if name == "f16_sum":
+        init = O.from_f32(O.F16, rnd(5).standard_normal(p.dst.dims).astype(np.float32)).reshape(p.dst.raw.shape)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True, dst_init=init)
+    assert pd.impl_info_str() == MFMA
+    want = p.run_oracle(dst_init=init)
+    if exact:
+        assert_bit_exact(got, want, name)
+    else:  # f16 after the device's exp2 / rcp: one f16 ulp
+        g, w = O.to_f32(dt.f16, got), O.to_f32(dt.f16, want)
+        assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-6, what=name)
+
+
 @pytest.mark.parametrize("name", sorted(TILE256_CASES))
 def test_mfma_int8_tile256_kernel(ctx, tile256, name):
     eng, strm = ctx
