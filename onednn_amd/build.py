@@ -37,7 +37,16 @@ UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
 # object so the instantiations compile in parallel
 GEMM_VARIANTS = [1, 2, 3]
 for v in GEMM_VARIANTS:
-    UNITS.append(("qmm_gemm_b8.hip", "_v%d" % v, ["-DQMM_GEMM_VARIANT=%d" % v]))
+    for k in (0, 1, 2):
+        UNITS.append(("qmm_gemm_b8.hip", "_v%d_k%d" % (v, k),
+                      ["-DQMM_GEMM_VARIANT=%d" % v, "-DQMM_GEMM_KIND=%d" % k]))
+# likewise the 256 x 256 kernels: int8, short-K int8, fp8
+for v in (1, 2, 3):
+    UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
+for v in (1, 2, 3, 4):
+    UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))
+# longest first, so that the pool finishes together
+UNITS.sort(key=lambda u: 0 if "w4a8" in u[0] else (1 if u[1] else 2))
 
 
 def _compile(unit):

@@ -356,7 +356,12 @@ enum : int {
     EP_FAST_RELU = 2, // eltwise relu(alpha)
     EP_FAST_SWISH = 3, // eltwise swish(alpha)
     EP_FAST_ADD = 4, // binary add with an f32 operand, dense along n
-    EP_FAST_SUM = 5 // sum with zero point 0 read in dst's own type
+    EP_FAST_SUM = 5, // sum with zero point 0 read in dst's own type
+    // shapes only the 256 x 256 kernels run straight-line (fast_ext is set):
+    EP_FAST_GELU_ERF = 6,
+    EP_FAST_GELU_TANH = 7,
+    EP_FAST_BIN32 = 8, // binary add / mul with a dense f32 operand
+    EP_FAST_BIN16 = 9 // binary add / mul with a dense f16 / bf16 operand
 };
 
 QMM_D float ep_load(const ep_tensor_t &t, int64_t b, int64_t m, int64_t n) {
@@ -463,6 +468,11 @@ struct ep_cols_t {
     float ws[4], bias[4], zp[4];
     float inv_dst_scale;
     int32_t has_ws, has_bias, bias_per_row, has_ds, has_zp;
+    // first post-op's binary operand (EP_FAST_BIN32 / BIN16), at this lane's
+    // columns of row 0
+    const void *bin_ptr;
+    int64_t bin_sm; // elements per row
+    int32_t bin_mul, bin_f16;
 };
 
 QMM_D void epilogue_cols_load(const epilogue_t &ep, ep_cols_t &c, int64_t b,
@@ -474,6 +484,18 @@ QMM_D void epilogue_cols_load(const epilogue_t &ep, ep_cols_t &c, int64_t b,
     c.has_zp = ep.dst_zp != nullptr;
     c.inv_dst_scale
             = c.has_ds ? 1.f / load_float(ep.dst_scale_dt, ep.dst_scale, 0) : 1.f;
+    c.bin_ptr = nullptr;
+    c.bin_sm = 0;
+    c.bin_mul = c.bin_f16 = 0;
+    if (ep.fast == EP_FAST_BIN32 || ep.fast == EP_FAST_BIN16) {
+        const int64_t off = b * ep.po[0].t.sb + n;
+        c.bin_ptr = ep.fast == EP_FAST_BIN32
+                ? (const void *)((const float *)ep.po[0].t.ptr + off)
+                : (const void *)((const uint16_t *)ep.po[0].t.ptr + off);
+        c.bin_sm = ep.po[0].t.sm;
+        c.bin_mul = ep.po[0].alg == alg_bin_mul;
+        c.bin_f16 = ep.po[0].t.dt == dt_f16;
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         c.ws[i] = 1.f;
@@ -761,8 +783,8 @@ QMM_D void epilogue_flush_denormals() {
 // shape, DSTK the dst type (EP_DST_*); EXT adds what ep.fast_ext announces: a
 // per-column bias, the dst scale and dst zero points, each applied through a
 // select or as the factor 1.0f so that an absent one changes no bit.
-enum : int { EP_DST_F32 = 0, EP_DST_BF16 = 1, EP_DST_F16 = 2, EP_DST_S8 = 3,
-    EP_DST_U8 = 4 };
+enum : int { EP_DST_F32 = 0, EP_DST_BF16 = 1, EP_DST_F16 = 2,
+    EP_DST_Q8 = 3 /* s8 or u8 */ };
 
 template <int FAST, int DSTK, bool EXT>
 QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
@@ -799,6 +821,38 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
         d[1] += y.y;
         d[2] += y.z;
         d[3] += y.w;
+    } else if constexpr (FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = eltwise_fwd(FAST == EP_FAST_GELU_ERF ? alg_gelu_erf
+                                                        : alg_gelu_tanh,
+                           d[i], ep.po[0].alpha, ep.po[0].beta)
+                    * ep.po[0].scale;
+    } else if constexpr (FAST == EP_FAST_BIN32 || FAST == EP_FAST_BIN16) {
+        const int64_t off = m * c.bin_sm;
+        const bool mul = c.bin_mul != 0;
+        float y[4];
+        if constexpr (FAST == EP_FAST_BIN32) {
+            const float4 v = *((const float4 *)((const float *)c.bin_ptr + off));
+            y[0] = v.x;
+            y[1] = v.y;
+            y[2] = v.z;
+            y[3] = v.w;
+        } else {
+            const uint2 v = *((const uint2 *)((const uint16_t *)c.bin_ptr + off));
+            const uint16_t h[4] = {(uint16_t)v.x, (uint16_t)(v.x >> 16),
+                    (uint16_t)v.y, (uint16_t)(v.y >> 16)};
+            const bool f16 = c.bin_f16 != 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float a = (float)__builtin_bit_cast(_Float16, h[i]);
+                const float b = u2f((uint32_t)h[i] << 16);
+                y[i] = f16 ? a : b;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = mul ? d[i] * y[i] : d[i] + y[i];
     } else if constexpr (FAST == EP_FAST_SUM) {
         static_assert(FAST != EP_FAST_SUM || DSTK <= EP_DST_F16, "");
         float o[4];
@@ -860,9 +914,9 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
         const uint32_t h1 = (uint32_t)f32_to_f16_hw(d[2])
                 | ((uint32_t)f32_to_f16_hw(d[3]) << 16);
         *(v2u *)((uint16_t *)ep.dst.ptr + dst_off) = v2u {h0, h1};
-    } else if constexpr (DSTK == EP_DST_S8 || DSTK == EP_DST_U8) {
-        const float lo = DSTK == EP_DST_S8 ? -128.f : 0.f;
-        const float hi = DSTK == EP_DST_S8 ? 127.f : 255.f;
+    } else if constexpr (DSTK == EP_DST_Q8) {
+        const float lo = ep.dst.dt == dt_s8 ? -128.f : 0.f;
+        const float hi = ep.dst.dt == dt_s8 ? 127.f : 255.f;
         uint32_t w = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -885,7 +939,8 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
 QMM_D bool epilogue_full4_ok(const epilogue_t &ep) {
     bool ok = (ep.dst.sm & 3) == 0 && (ep.dst.sb & 3) == 0
             && ((uintptr_t)ep.dst.ptr & 15) == 0 && ep.fast != EP_FAST_NONE;
-    if (ep.fast == EP_FAST_ADD)
+    if (ep.fast == EP_FAST_ADD || ep.fast == EP_FAST_BIN32
+            || ep.fast == EP_FAST_BIN16)
         ok = ok && (ep.po[0].t.sm & 3) == 0 && (ep.po[0].t.sb & 3) == 0
                 && ((uintptr_t)ep.po[0].t.ptr & 15) == 0;
     return ok;

@@ -341,9 +341,22 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
                     && o.t.dt == ep.dst.dt
                     && one_of(ep.dst.dt, {dt_f32, dt_bf16, dt_f16}))
                 ep.fast = EP_FAST_SUM;
+            else if (o.kind == pk_eltwise && o.alg == alg_gelu_erf)
+                ep.fast = EP_FAST_GELU_ERF;
+            else if (o.kind == pk_eltwise && o.alg == alg_gelu_tanh)
+                ep.fast = EP_FAST_GELU_TANH;
+            else if (o.kind == pk_binary
+                    && (o.alg == alg_bin_add || o.alg == alg_bin_mul)
+                    && o.t.sn == 1 && o.t.dt == dt_f32)
+                ep.fast = EP_FAST_BIN32;
+            else if (o.kind == pk_binary
+                    && (o.alg == alg_bin_add || o.alg == alg_bin_mul)
+                    && o.t.sn == 1 && one_of(o.t.dt, {dt_f16, dt_bf16}))
+                ep.fast = EP_FAST_BIN16;
         }
         if (ep.fast != EP_FAST_NONE)
-            ep.fast_ext = ep.bias.ptr || ep.dst_scale || ep.dst_zp || dst_more;
+            ep.fast_ext = ep.bias.ptr || ep.dst_scale || ep.dst_zp || dst_more
+                    || ep.fast > EP_FAST_SUM;
     }
     return true;
 }

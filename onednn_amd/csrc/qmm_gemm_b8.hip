@@ -321,6 +321,11 @@ gemm_b8_kernel(const gemm_params_t p) {
     // what depends on the lane's 4 columns only, fetched once
     ep_cols_t cols;
     epilogue_cols_load(p.ep, cols, bz, en, envalid > 0 ? envalid : 0);
+    // The row interpreter indexes the post-op list at run time: it reads the
+    // parameter block in the kernel argument segment (its only argument), so
+    // that the by-value copy `p` stays in registers.
+    const epilogue_t &epk
+            = ((const gemm_params_t *)__builtin_amdgcn_kernarg_segment_ptr())->ep;
     const float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
@@ -350,8 +355,7 @@ gemm_b8_kernel(const gemm_params_t p) {
                     epilogue_fast4(
                             p.ep, v, has_ss, ss, has_ws, ws4, bz, m, en, envalid);
                 else
-                    epilogue_rows4(
-                            p.ep, cols, v, has_ss, ss, bz, m, en, envalid);
+                    epilogue_rows4(epk, cols, v, has_ss, ss, bz, m, en, envalid);
             }
         }
     });
@@ -381,9 +385,9 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
             stream, q);
 }
 
-// One tile configuration per translation unit (QMM_GEMM_VARIANT), so the
-// instantiations build in parallel; the unit without the macro holds the
-// dispatcher.
+// One tile configuration and operand kind per translation unit
+// (QMM_GEMM_VARIANT, QMM_GEMM_KIND), so the instantiations build in parallel;
+// the unit without the macros holds the dispatcher.
 #if defined(QMM_GEMM_VARIANT)
 // BM, BN, BK, waves along M, waves along N, LDS stages
 #if QMM_GEMM_VARIANT == 1
@@ -395,19 +399,42 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
 #endif
 #define QMM_CAT_(a, b) a##b
 #define QMM_CAT(a, b) QMM_CAT_(a, b)
-void QMM_CAT(launch_gemm_b8_v, QMM_GEMM_VARIANT)(
-        const gemm_params_t &p, bool f8, hipStream_t stream) {
-    if (f8)
-        launch_cfg<QMM_CFG, true, false>(p, stream);
-    else if (p.a_is_u8)
-        launch_cfg<QMM_CFG, false, true>(p, stream);
-    else
-        launch_cfg<QMM_CFG, false, false>(p, stream);
+#define QMM_CAT3(a, b, c) QMM_CAT(QMM_CAT(a, b), c)
+// ... and one operand kind per unit (QMM_GEMM_KIND: 0 fp8, 1 u8 source, 2 s8)
+#if QMM_GEMM_KIND == 0
+void QMM_CAT3(launch_gemm_b8_v, QMM_GEMM_VARIANT, _f8)(
+        const gemm_params_t &p, hipStream_t stream) {
+    launch_cfg<QMM_CFG, true, false>(p, stream);
+}
+#elif QMM_GEMM_KIND == 1
+void QMM_CAT3(launch_gemm_b8_v, QMM_GEMM_VARIANT, _u8)(
+        const gemm_params_t &p, hipStream_t stream) {
+    launch_cfg<QMM_CFG, false, true>(p, stream);
 }
 #else
-void launch_gemm_b8_v1(const gemm_params_t &p, bool f8, hipStream_t stream);
-void launch_gemm_b8_v2(const gemm_params_t &p, bool f8, hipStream_t stream);
-void launch_gemm_b8_v3(const gemm_params_t &p, bool f8, hipStream_t stream);
+void QMM_CAT3(launch_gemm_b8_v, QMM_GEMM_VARIANT, _s8)(
+        const gemm_params_t &p, hipStream_t stream) {
+    launch_cfg<QMM_CFG, false, false>(p, stream);
+}
+#endif
+#else
+#define QMM_DECL_VARIANT(V) \
+    void launch_gemm_b8_v##V##_f8(const gemm_params_t &p, hipStream_t stream); \
+    void launch_gemm_b8_v##V##_u8(const gemm_params_t &p, hipStream_t stream); \
+    void launch_gemm_b8_v##V##_s8(const gemm_params_t &p, hipStream_t stream); \
+    static void launch_gemm_b8_v##V( \
+            const gemm_params_t &p, bool f8, hipStream_t stream) { \
+        if (f8) \
+            launch_gemm_b8_v##V##_f8(p, stream); \
+        else if (p.a_is_u8) \
+            launch_gemm_b8_v##V##_u8(p, stream); \
+        else \
+            launch_gemm_b8_v##V##_s8(p, stream); \
+    }
+QMM_DECL_VARIANT(1)
+QMM_DECL_VARIANT(2)
+QMM_DECL_VARIANT(3)
+#undef QMM_DECL_VARIANT
 // 256 x 256 tile kernel with the hand-ordered main loop (qmm_gemm_b8x.hip)
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8);
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream);

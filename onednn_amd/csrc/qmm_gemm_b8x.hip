@@ -212,7 +212,11 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const ep_cols_t &cols,
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
     const int ecol = (lane & 31) * 4;
-#pragma unroll 8
+    // rows in flight: fewer where a row is a long computation of its own
+    constexpr int UNR = FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH
+            ? 2
+            : (FAST > EP_FAST_SUM || EXT ? 4 : 8);
+#pragma unroll UNR
     for (int it = 0; it < 32; it++) {
         const int row = it * 2 + (lane >> 5);
         const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
@@ -235,7 +239,9 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
 }
 
 // Epilogue of one 256 x 256 block tile, shared by the int8 and fp8 kernels.
-template <bool F8, typename AccT>
+// LEAN: only the shapes up to EP_FAST_SUM with a float dst run straight-line
+// (fp8 and short-K launches; everything else they accept takes the row path)
+template <bool F8, bool LEAN, typename AccT>
 QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
         uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
         int wm0, int wn0, int bz) {
@@ -249,6 +255,12 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     // what it wrote itself: LDS executes a wave's instructions in order, no
     // barrier is involved.
     const epilogue_t &ep = p.ep;
+    // The row interpreter walks the post-op list with a run-time index: it
+    // reads the parameter block where it lies (the kernel argument segment,
+    // whose first and only argument is the gemm_params_t), so that the
+    // by-value copy `p` stays in registers.
+    const epilogue_t &epk
+            = ((const gemm_params_t *)__builtin_amdgcn_kernarg_segment_ptr())->ep;
     const uint32_t stg_w = lds_base + wave * STG_WAVE
             + (4 * (lane >> 5) * 128 + (lane & 31)) * 4;
     const int *const stg_r = (const int *)lds + wave * (STG_WAVE / 4);
@@ -263,8 +275,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     const int dstk = ep.dst.dt == dt_f32 ? EP_DST_F32
             : ep.dst.dt == dt_bf16       ? EP_DST_BF16
             : ep.dst.dt == dt_f16        ? EP_DST_F16
-            : ep.dst.dt == dt_s8         ? EP_DST_S8
-                                         : EP_DST_U8;
+                                         : EP_DST_Q8;
     // what depends on the lane's 4 columns only: weights scales, a per-column
     // bias, dst zero points, the zero-point compensation
     ep_cols_t cols;
@@ -288,7 +299,8 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
     // operand's rows) aligned for vector access
     const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
-            && ep.fast != EP_FAST_NONE && epilogue_full4_ok(ep);
+            && ep.fast != EP_FAST_NONE && epilogue_full4_ok(ep)
+            && (!LEAN || (ep.fast <= EP_FAST_SUM && dstk <= EP_DST_F16));
     static_for<2>([&](auto H) {
         constexpr int h = decltype(H)::value;
 #pragma unroll
@@ -312,28 +324,32 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     switch (dstk) { \
         case EP_DST_F32: \
             if (ext) QX_EP_ROWS(F, EP_DST_F32, true); \
-            else QX_EP_ROWS(F, EP_DST_F32, false); \
+            else if constexpr (F <= EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_F32, false); \
             break; \
         case EP_DST_BF16: \
             if (ext) QX_EP_ROWS(F, EP_DST_BF16, true); \
-            else QX_EP_ROWS(F, EP_DST_BF16, false); \
+            else if constexpr (F <= EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_BF16, false); \
             break; \
         case EP_DST_F16: QX_EP_ROWS(F, EP_DST_F16, true); break; \
-        case EP_DST_S8: \
-            if constexpr (F != EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_S8, true); \
-            break; \
         default: \
-            if constexpr (F != EP_FAST_SUM) QX_EP_ROWS(F, EP_DST_U8, true); \
+            if constexpr (!LEAN && F != EP_FAST_SUM) \
+                QX_EP_ROWS(F, EP_DST_Q8, true); \
             break; \
     }
 #define QX_EP_CASE(F) \
-    case F: QX_EP_DST(F) break;
+    case F: \
+        if constexpr (!LEAN || F <= EP_FAST_SUM) { QX_EP_DST(F) } \
+        break;
             switch (ep.fast) {
                 QX_EP_CASE(EP_FAST_PLAIN)
                 QX_EP_CASE(EP_FAST_RELU)
                 QX_EP_CASE(EP_FAST_SWISH)
                 QX_EP_CASE(EP_FAST_ADD)
                 QX_EP_CASE(EP_FAST_SUM)
+                QX_EP_CASE(EP_FAST_GELU_ERF)
+                QX_EP_CASE(EP_FAST_GELU_TANH)
+                QX_EP_CASE(EP_FAST_BIN32)
+                QX_EP_CASE(EP_FAST_BIN16)
                 default: break;
             }
 #undef QX_EP_ROWS
@@ -362,7 +378,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
                     }
                     if (ep.fast == EP_FAST_NONE || ext)
                         epilogue_rows4(
-                                ep, cols, v, has_ss, ss, bz, m, en, envalid);
+                                epk, cols, v, has_ss, ss, bz, m, en, envalid);
                     else if (to_bf16 && envalid == 4)
                         epilogue_fast4_bf16(
                                 ep, v, has_ss, ss, has_ws, ws4, bz, m, en);
@@ -578,7 +594,8 @@ gemm_b8x_kernel(const gemm_params_t p) {
         __syncthreads();
     }
 
-    tile_epilogue<false>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    tile_epilogue<false, SHORTK>(
+            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
 }
 
 // ---- fp8 (e4m3 x e4m3 -> f32) ----------------------------------------------
@@ -644,6 +661,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
     QF_MF(2, 0, CB); QF_MF(2, 1, CB); QF_MF(2, 2, CB); QF_MF(2, 3, CB); \
     QF_MF(3, 0, CB); QF_MF(3, 1, CB); QF_MF(3, 2, CB); QF_MF(3, 3, CB);
 
+#if defined(QMM_B8X_PART) && QMM_B8X_PART == 3
 __global__ void __launch_bounds__(b8x::NT, 1)
 gemm_f8x_kernel(const gemm_params_t p) {
     using namespace b8x;
@@ -765,8 +783,11 @@ gemm_f8x_kernel(const gemm_params_t p) {
     QF_LAST(1)
     __syncthreads();
 
-    tile_epilogue<true>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    tile_epilogue<true, true>(
+            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
 }
+
+#endif // fp8 kernel
 
 template <typename K>
 static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
@@ -794,9 +815,31 @@ static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
             stream, q);
 }
 
+// One kernel per translation unit (QMM_B8X_PART), so that they build in
+// parallel; the unit without the macro holds the dispatcher.
+#if defined(QMM_B8X_PART)
+#if QMM_B8X_PART == 1
+void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_b8x_kernel<false>, p, stream);
+}
+#elif QMM_B8X_PART == 2
+void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_b8x_kernel<true>, p, stream);
+}
+#elif QMM_B8X_PART == 3
+void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_f8x_kernel, p, stream);
+}
+#endif
+#else
+void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
+void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream);
+void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream);
+
 // Problems the kernels take: K a multiple of 64; s8 sources (u8 too when K is
-// at most 256), or fp8 sources with K a multiple of 128 and at least 6 k-steps; a straight-line epilogue, 32-bit addressable tiles, and enough
-// 256 x 256 tiles to occupy the chip.
+// at most 256, or rewritten as s8 by the caller), or fp8 sources with K a
+// multiple of 128 and at least 6 k-steps; 32-bit addressable tiles. Whether
+// there are enough 256 x 256 tiles to occupy the chip is the caller's call.
 static bool short_k(const gemm_params_t &p) {
     return p.K <= 4 * 64;
 }
@@ -812,11 +855,12 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
 
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     if (f8)
-        launch_b8x(gemm_f8x_kernel, p, stream);
+        launch_b8x_fp8(p, stream);
     else if (short_k(p))
-        launch_b8x(gemm_b8x_kernel<true>, p, stream);
+        launch_b8x_short_k(p, stream);
     else
-        launch_b8x(gemm_b8x_kernel<false>, p, stream);
+        launch_b8x_int8(p, stream);
 }
+#endif
 
 } // namespace qmm

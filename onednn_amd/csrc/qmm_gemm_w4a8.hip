@@ -358,6 +358,10 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     const float one4[4] = {1.f, 1.f, 1.f, 1.f};
     ep_cols_t cols;
     epilogue_cols_load(p.ep, cols, 0, en, envalid > 0 ? envalid : 0);
+    // the row interpreter reads the parameter block where it lies (the kernel
+    // argument segment): its run-time indexing must not drag `p` into memory
+    const epilogue_t &epk
+            = ((const w4a8_params_t *)__builtin_amdgcn_kernarg_segment_ptr())->ep;
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
 #pragma unroll
@@ -378,13 +382,13 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
                     epilogue_fast4(
                             p.ep, v, false, 1.f, false, one4, 0, m, en, envalid);
                 else
-                    epilogue_rows4(
-                            p.ep, cols, v, false, 1.f, 0, m, en, envalid);
+                    epilogue_rows4(epk, cols, v, false, 1.f, 0, m, en, envalid);
             }
         }
     });
 }
 
+#if !defined(QMM_W4A8_PART)
 // ---- pre-pass ----
 // One thread per (group, row) and per (group, column).
 __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
@@ -430,6 +434,8 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
         }
     }
 }
+
+#endif // pre-pass
 
 // ---- rows <= 64: split-K streaming kernel ----
 // At these sizes the launch is one read of the weights and nothing else
@@ -951,6 +957,7 @@ static void launch_tiny_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         launch_tiny_cfg<NWV, SC, true, 2>(p, stream);
 }
 
+#if defined(QMM_W4A8_PART) && QMM_W4A8_PART == 3
 // sum of the slices in slice order, then bias / post-ops / dst conversion:
 // one thread per four neighbouring columns of a row
 __global__ void __launch_bounds__(256)
@@ -985,6 +992,8 @@ w4a8_reduce_kernel(const float *part, int splits, int M, int N, int ldp,
             epilogue_apply_store4(ep, v, 0, m, n, nvalid);
     }
 }
+
+#endif // reduction
 
 template <int FM, int SC, bool HAS_ZP, int ZPK>
 static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
@@ -1053,56 +1062,25 @@ static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
 
 } // namespace w4a8
 
-void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
-    const int64_t total = (int64_t)p.ng * ((int64_t)p.M + p.N);
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 65535) blocks = 65535;
-    hipLaunchKernelGGL(w4a8::w4a8_prep_kernel, dim3((unsigned)blocks), dim3(256),
-            0, stream, p);
-}
-
-// Data types the small-row kernel reads directly: both scales of one size
-// (f16 / bf16, or f32) and zero points of one byte or less.
-bool gemm_w4a8_small_takes(const w4a8_prep_t &q) {
-    auto two = [](int dt) { return dt == dt_f16 || dt == dt_bf16; };
-    const int sdt = q.ss ? q.ss_dt : q.sw_dt, wdt = q.sw ? q.sw_dt : q.ss_dt;
-    if ((q.ss || q.sw) && !((two(sdt) && two(wdt)) || (sdt == dt_f32 && wdt == dt_f32)))
-        return false;
-    if (q.zw && q.zw_dt == dt_s32) return false;
-    return true;
-}
-
-// Single-token decode kernel: nwv waves per workgroup (4 or 8), p.gps groups
-// per wave; p.part / p.splits are unused.
-void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
+// The kernel families build in translation units of their own (QMM_W4A8_PART:
+// 1, 2 the tiled GEMM without / with zero points, 3 the split-K kernel and its
+// reduction, 4 the single-token kernel); the unit without the macro holds the
+// pre-pass and the dispatch.
+#if defined(QMM_W4A8_PART)
+#if QMM_W4A8_PART == 1
+void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
-    if (p.q.M <= 0 || p.q.N <= 0) return;
-    const w4a8_prep_t &q = p.q;
-    const int sdt = q.ss ? q.ss_dt : q.sw_dt;
-    const bool sc4 = (q.ss || q.sw) && sdt == dt_f32;
-    const int zpk = !q.zw ? 0 : ((q.zw_dt == dt_s4 || q.zw_dt == dt_u4) ? 2 : 1);
-    if (nwv == 8) {
-        if (sc4)
-            w4a8::launch_tiny_zp<8, 4>(p, has_zp, zpk, stream);
-        else
-            w4a8::launch_tiny_zp<8, 2>(p, has_zp, zpk, stream);
-    } else {
-        if (sc4)
-            w4a8::launch_tiny_zp<4, 4>(p, has_zp, zpk, stream);
-        else
-            w4a8::launch_tiny_zp<4, 2>(p, has_zp, zpk, stream);
-    }
+    w4a8::launch_zp<false>(p, variant, stream);
 }
-
-void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
+#elif QMM_W4A8_PART == 2
+void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
-    if (p.q.M <= 0 || p.q.N <= 0) return;
-    const w4a8_prep_t &q = p.q;
-    const bool two_frags = q.M > 32;
-    const int sdt = q.ss ? q.ss_dt : q.sw_dt;
-    const bool sc4 = (q.ss || q.sw) && sdt == dt_f32;
-    const int zpk = !q.zw ? 0 : ((q.zw_dt == dt_s4 || q.zw_dt == dt_u4) ? 2 : 1);
-    if (two_frags) {
+    w4a8::launch_zp<true>(p, variant, stream);
+}
+#elif QMM_W4A8_PART == 3
+void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, hipStream_t stream) {
+    if (p.q.M > 32) {
         if (sc4)
             w4a8::launch_small_zp<2, 4>(p, has_zp, zpk, stream);
         else
@@ -1120,6 +1098,75 @@ void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
             dim3(256), 0, stream, (const float *)p.part, p.splits, p.q.M, p.q.N,
             p.ldp, p.ep);
 }
+#elif QMM_W4A8_PART == 4
+void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream) {
+    if (nwv == 8) {
+        if (sc4)
+            w4a8::launch_tiny_zp<8, 4>(p, has_zp, zpk, stream);
+        else
+            w4a8::launch_tiny_zp<8, 2>(p, has_zp, zpk, stream);
+    } else {
+        if (sc4)
+            w4a8::launch_tiny_zp<4, 4>(p, has_zp, zpk, stream);
+        else
+            w4a8::launch_tiny_zp<4, 2>(p, has_zp, zpk, stream);
+    }
+}
+#endif
+#else
+void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
+        hipStream_t stream);
+void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
+        hipStream_t stream);
+void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, hipStream_t stream);
+void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream);
+
+void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
+    const int64_t total = (int64_t)p.ng * ((int64_t)p.M + p.N);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(w4a8::w4a8_prep_kernel, dim3((unsigned)blocks), dim3(256),
+            0, stream, p);
+}
+
+// Data types the small-row kernels read directly: both scales of one size
+// (f16 / bf16, or f32) and zero points of one byte or less.
+bool gemm_w4a8_small_takes(const w4a8_prep_t &q) {
+    auto two = [](int dt) { return dt == dt_f16 || dt == dt_bf16; };
+    const int sdt = q.ss ? q.ss_dt : q.sw_dt, wdt = q.sw ? q.sw_dt : q.ss_dt;
+    if ((q.ss || q.sw)
+            && !((two(sdt) && two(wdt)) || (sdt == dt_f32 && wdt == dt_f32)))
+        return false;
+    if (q.zw && q.zw_dt == dt_s32) return false;
+    return true;
+}
+
+static bool scales_are_f32(const w4a8_prep_t &q) {
+    const int sdt = q.ss ? q.ss_dt : q.sw_dt;
+    return (q.ss || q.sw) && sdt == dt_f32;
+}
+static int zp_storage(const w4a8_prep_t &q) {
+    return !q.zw ? 0 : ((q.zw_dt == dt_s4 || q.zw_dt == dt_u4) ? 2 : 1);
+}
+
+// Single-token decode kernel: nwv waves per workgroup (4 or 8), p.gps groups
+// per wave; p.part / p.splits are unused.
+void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
+        hipStream_t stream) {
+    if (p.q.M <= 0 || p.q.N <= 0) return;
+    launch_gemm_w4a8_tiny_part(
+            p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+}
+
+void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
+        hipStream_t stream) {
+    if (p.q.M <= 0 || p.q.N <= 0) return;
+    launch_gemm_w4a8_small_part(
+            p, has_zp, zp_storage(p.q), scales_are_f32(p.q), stream);
+}
 
 // variant: 0 = by problem size; 1: 128 x 128, 2: 64 x 128, 3: 32 x 64 tiles
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream) {
@@ -1131,9 +1178,10 @@ void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream) {
         if (variant == 3 && p.M > 64) variant = 2;
     }
     if (p.zwT)
-        w4a8::launch_zp<true>(p, variant, stream);
+        launch_gemm_w4a8_zp(p, variant, stream);
     else
-        w4a8::launch_zp<false>(p, variant, stream);
+        launch_gemm_w4a8_nozp(p, variant, stream);
 }
+#endif
 
 } // namespace qmm

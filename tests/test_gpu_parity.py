@@ -332,7 +332,25 @@ TILE256_EPILOGUE_CASES = {
                                                                  {"kind": "eltwise", "alg": A.eltwise_abs}]), True),
     "f16_sum": (lambda: int8_linear(512, 256, 256, 100, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None,
                                     post_ops=[{"kind": "sum", "scale": 0.5}]), True),
+    "s8_bias_gelu_erf_requant": (lambda: int8_linear(512, 256, 256, 101, src_dt=dt.s8, dst_dt=dt.s8, src_zp=None, per_token=True,
+                                                     bias_dt=dt.f32, dst_scale=0.05,
+                                                     post_ops=[{"kind": "eltwise", "alg": A.eltwise_gelu_erf}]), "s8"),
+    "bf16_gelu_tanh": (lambda: int8_linear(512, 256, 256, 102, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True,
+                                           post_ops=[{"kind": "eltwise", "alg": A.eltwise_gelu_tanh}]), "bf16"),
+    "f32_binary_mul_f32": (lambda: _with_binary(int8_linear(512, 256, 256, 103, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None),
+                                                A.binary_mul, dt.f32, 104), True),
+    "f16_binary_add_f16": (lambda: _with_binary(int8_linear(512, 256, 512, 105, src_dt=dt.s8, dst_dt=dt.f16, src_zp=None, per_token=True),
+                                                A.binary_add, dt.f16, 106), True),
+    "bf16_binary_mul_bf16_edges": (lambda: _with_binary(int8_linear(300, 256, 260, 107, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None),
+                                                        A.binary_mul, dt.bf16, 108), True),
 }
+
+
+def _with_binary(p, alg, code, seed):
+    M, N = p.dst.dims[-2:]
+    t = TensorSpec(code, [M, N], None, rnd(seed).uniform(-2, 2, (M, N)).astype(np.float32))
+    p.post_ops = [{"kind": "binary", "alg": alg, "src1": t}]
+    return p
 
 
 @pytest.mark.parametrize("name", sorted(TILE256_EPILOGUE_CASES))
@@ -347,8 +365,13 @@ def test_mfma_int8_tile256_epilogue_surface(ctx, tile256, name):
     got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True, dst_init=init)
     assert pd.impl_info_str() == MFMA
     want = p.run_oracle(dst_init=init)
-    if exact:
+    if exact is True:
         assert_bit_exact(got, want, name)
+    elif exact == "s8":  # device erff / tanhf against libm: the last bit may round the other way
+        diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+        assert diff.max() <= 1 and (diff > 0).mean() < 1e-3, (name, diff.max(), (diff > 0).mean())
+    elif exact == "bf16":
+        assert_bf16_within_1ulp(got, want, name, abs_slack=1e-30)
     else:  # f16 after the device's exp2 / rcp: one f16 ulp
         g, w = O.to_f32(dt.f16, got), O.to_f32(dt.f16, want)
         assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-6, what=name)
@@ -417,6 +440,23 @@ def test_mfma_fp8_tile256_kernel(ctx, tile256):
         else:
             assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
                              rel=1e-5, scale=a, what="fp8 f32")
+
+
+def test_mfma_fp8_tile256_f16_dst_bias_relu(ctx, tile256):
+    """fp8 through the straight-line epilogue with an f16 dst and a per-column bias."""
+    eng, strm = ctx
+    M, K, N = 512, 512, 256
+    say("mfma_b8 256x256 fp8 kernel, f16 dst + bias + relu")
+    p = fp8_gemm(M, K, N, 79, dst_dt=dt.f16, with_sum=False)
+    p.bias = TensorSpec(dt.f32, [1, N], None, rnd(80).standard_normal(N).astype(np.float32))
+    p.post_ops = [{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    want = p.run_oracle()
+    a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
+    g, w = O.to_f32(dt.f16, got).reshape(M, N), O.to_f32(dt.f16, want).reshape(M, N)
+    # f16 rounding (2^-11 relative) on top of the f32 bar for another summation order
+    assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-5 * a * 1024, what="fp8 f16")
 
 
 def test_mfma_int8_tile256_binary_add_and_sum(ctx, tile256):
