@@ -44,7 +44,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
-          "attention_scores": "bench_c4", "int8_int4_grouped": "bench_w4a8"}
+          "attention_scores": "bench_c4", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
 
 
 def main():
@@ -425,6 +425,35 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
                           "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                           "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4),
                           "impl": pd.impl_info_str(), "includes": "scale pre-pass + GEMM"}
+    return res
+
+
+def bench_quantize(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
+    """The reorder as a quantizer on the tensors of config 2: its weights f32 [4096,14336] -> s8 with per-column
+    scales (once per model), its activations bf16 [4096,4096] -> s8 with per-row scales (every step). A stream:
+    bytes read + written against HBM bandwidth."""
+    r = np.random.default_rng(8)
+    res = {}
+    for name, sdt, dims, mask, nsc in (("weights_f32_s8_per_column", dt.f32, [4096, 14336], 2, 14336),
+                                       ("activations_bf16_s8_per_row", dt.bf16, [4096, 4096], 1, 4096)):
+        attr = A.primitive_attr()
+        attr.set_scales_mask(A.DNNL_ARG_DST, mask)
+        s_md, d_md = memory.desc(dims, sdt, T("ab")), memory.desc(dims, dt.s8, T("ab"))
+        pd = A.reorder.primitive_desc(eng, s_md, eng, d_md, attr=attr)
+        prim = A.reorder(pd)
+        n = dims[0] * dims[1]
+        x = np.resize(r.standard_normal(1 << 20).astype(np.float32), n)
+        if sdt == dt.bf16:
+            import oracle as O
+            x = O.from_f32(O.BF16, x)
+        ex = {A.DNNL_ARG_FROM: memory(s_md, eng).write(x), A.DNNL_ARG_TO: memory(d_md, eng),
+              A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_DST: memory(memory.desc([nsc], dt.f32, T("a")), eng).write(
+                  r.uniform(0.01, 0.05, nsc).astype(np.float32))}
+        ms = _time(prim, strm, hs, hiprt, ex, steps)
+        nbytes = n * (4 if sdt == dt.f32 else 2) + n + nsc * 4
+        res[name] = {"us_per_launch": round(ms * 1e3, 2), "algorithmic_bytes": nbytes,
+                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str()}
     return res
 
 

@@ -156,6 +156,11 @@ typedef struct {
 } qmm_reorder_args_t;
 
 QMM_API int qmm_reorder_supports(const qmm_reorder_desc_t *desc);
+/* Name of the implementation qmm_reorder_launch() runs for `desc`:
+ * "hip:gfx950:prepack" (to / from a packed weights layout),
+ * "hip:gfx950:quantize" (row-wise element pass with scales / zero points) or
+ * "hip:gfx950:reorder" (any strides, one element per thread). */
+QMM_API const char *qmm_reorder_impl_name(const qmm_reorder_desc_t *desc);
 QMM_API int qmm_reorder_launch(const qmm_reorder_desc_t *desc,
         const qmm_reorder_args_t *args, void *hip_stream);
 

@@ -129,6 +129,7 @@ _SIGNATURES = {
     "qmm_last_error": (C.c_char_p, []),
     "qmm_matmul_impl_count": (_I, []),
     "qmm_matmul_impl_name": (C.c_char_p, [_I]),
+    "qmm_reorder_impl_name": (C.c_char_p, [_P]),
     "qmm_set_gemm_variant": (None, [_I]),
     "qmm_set_w4a8_variant": (None, [_I]),
 }

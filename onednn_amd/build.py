@@ -29,7 +29,8 @@ DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",
 
 # (source, object suffix, extra defines)
 UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
-         ("qmm_pack.hip", "", []), ("qmm_dispatch.hip", "", []),
+         ("qmm_pack.hip", "", []), ("qmm_quantize.hip", "", []),
+         ("qmm_dispatch.hip", "", []),
          ("qmm_gemm_b8.hip", "", []),
          ("qmm_gemm_b8x.hip", "", []), ("qmm_gemm_w4a8.hip", "", []),
          ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]

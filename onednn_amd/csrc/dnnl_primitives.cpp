@@ -765,10 +765,7 @@ dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *out,
     const int st = qmm_reorder_supports(&R);
     if (st != QMM_OK) return from_qmm(st);
     pd->impl = 0;
-    pd->impl_name = (R.src_layout != QMM_LAYOUT_PLAIN
-                            || R.dst_layout != QMM_LAYOUT_PLAIN)
-            ? "hip:gfx950:prepack"
-            : "hip:gfx950:reorder";
+    pd->impl_name = qmm_reorder_impl_name(&R);
     dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc {pd};
     if (!h) return dnnl_out_of_memory;
     *out = h;

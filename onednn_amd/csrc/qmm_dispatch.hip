@@ -24,6 +24,7 @@ void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream);
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
+void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
@@ -1067,6 +1068,96 @@ int qmm_reorder_supports(const qmm_reorder_desc_t *d) {
     return QMM_UNIMPLEMENTED;
 }
 
+// Row-wise quantizing pass (qmm_quantize.hip): both tensors plain, row-major
+// in the same dim order with stride 1 along the last dim, rows of a multiple
+// of 8 elements that start on the vector boundaries the kernel uses, a
+// floating-point source; scales / zero points over rows and columns of a 2-D
+// tensor (with or without groups), over the last dim only otherwise.
+static int elem_bits(int dt) {
+    switch (dt) {
+        case dt_f32:
+        case dt_s32: return 32;
+        case dt_bf16:
+        case dt_f16: return 16;
+        case dt_s4:
+        case dt_u4: return 4;
+        default: return 8;
+    }
+}
+static bool rows_quant(quant_rows_q_t &q, const qmm_quant_t &a, int nd,
+        const int64_t *dims) {
+    std::memset(&q, 0, sizeof(q));
+    q.gr = q.gc = 1;
+    q.dt = a.dt;
+    if (!a.set) return true;
+    const int last = 1 << (nd - 1), prev = nd >= 2 ? 1 << (nd - 2) : 0;
+    if (a.mask & ~(last | (nd == 2 ? prev : 0))) return false;
+    const int64_t g0 = a.has_groups && a.g0 > 0 ? a.g0 : 1;
+    const int64_t g1 = a.has_groups && a.g1 > 0 ? a.g1 : 1;
+    const int64_t C = dims[nd - 1];
+    if (nd >= 2 && (dims[nd - 2] % g0 || C % g1)) return false;
+    if (nd == 1 && a.has_groups) return false;
+    q.gr = g0;
+    q.gc = g1;
+    q.sc = (a.mask & last) ? 1 : 0;
+    q.sr = (a.mask & prev) && nd == 2 ? ((a.mask & last) ? C / g1 : 1) : 0;
+    q.ptr = (const void *)1; // set at launch
+    return true;
+}
+static bool reorder_rows_plan(const qmm_reorder_desc_t *d,
+        quant_rows_params_t &p) {
+    std::memset(&p, 0, sizeof(p));
+    const int nd = d->src.ndims;
+    if (d->src_layout != QMM_LAYOUT_PLAIN || d->dst_layout != QMM_LAYOUT_PLAIN)
+        return false;
+    if (!one_of(d->src.dt, {dt_f32, dt_bf16, dt_f16})) return false;
+    if (!one_of(d->dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s8, dt_u8, dt_s4,
+                dt_u4, dt_f8_e4m3, dt_f8_e5m2}))
+        return false;
+    const int64_t C = d->src.dims[nd - 1];
+    if (C % 8 != 0 || d->src.strides[nd - 1] != 1 || d->dst.strides[nd - 1] != 1)
+        return false;
+    int64_t rows = 1;
+    for (int i = 0; i < nd - 1; i++)
+        rows *= d->src.dims[i];
+    // leading dims nest densely over the row pitch, identically on both sides
+    const int64_t sp = nd >= 2 ? d->src.strides[nd - 2] : C;
+    const int64_t dp = nd >= 2 ? d->dst.strides[nd - 2] : C;
+    if (sp < C || dp < C) return false;
+    for (int i = nd - 3; i >= 0; i--) {
+        if (d->src.strides[i] != d->src.strides[i + 1] * d->src.dims[i + 1]
+                || d->dst.strides[i]
+                        != d->dst.strides[i + 1] * d->dst.dims[i + 1])
+            return false;
+    }
+    // 8 elements are one or two 16-byte loads and one 4..32-byte store
+    if ((sp * elem_bits(d->src.dt)) % 128 != 0) return false;
+    const int out_bits = 8 * elem_bits(d->dst.dt);
+    if ((dp * elem_bits(d->dst.dt)) % (out_bits > 128 ? 128 : out_bits) != 0)
+        return false;
+    if (!rows_quant(p.src_scale, d->src_scale, nd, d->src.dims)
+            || !rows_quant(p.dst_scale, d->dst_scale, nd, d->src.dims)
+            || !rows_quant(p.src_zp, d->src_zp, nd, d->src.dims))
+        return false;
+    if (d->dst_zp.set && d->dst_zp.mask != 0) return false;
+    p.rows = rows;
+    p.cols = C;
+    p.src_pitch = sp;
+    p.dst_pitch = dp;
+    p.src_dt = d->src.dt;
+    p.dst_dt = d->dst.dt;
+    return true;
+}
+
+const char *qmm_reorder_impl_name(const qmm_reorder_desc_t *d) {
+    if (!d) return "";
+    if (d->src_layout != QMM_LAYOUT_PLAIN || d->dst_layout != QMM_LAYOUT_PLAIN)
+        return "hip:gfx950:prepack";
+    quant_rows_params_t p;
+    return reorder_rows_plan(d, p) ? "hip:gfx950:quantize"
+                                   : "hip:gfx950:reorder";
+}
+
 int qmm_reorder_launch(const qmm_reorder_desc_t *d,
         const qmm_reorder_args_t *args, void *hip_stream) {
     const int st = qmm_reorder_supports(d);
@@ -1080,7 +1171,28 @@ int qmm_reorder_launch(const qmm_reorder_desc_t *d,
         nelems *= d->src.dims[i];
     if (nelems == 0) return QMM_OK;
 
-    if (d->src_layout == QMM_LAYOUT_PLAIN && d->dst_layout == QMM_LAYOUT_PLAIN) {
+    quant_rows_params_t qr;
+    // tensors and scale buffers on the vector boundaries the kernel assumes
+    const bool vec_ok = (((uintptr_t)args->src | (uintptr_t)args->dst
+                                 | (uintptr_t)args->src_scale
+                                 | (uintptr_t)args->dst_scale)
+                                & 15)
+            == 0;
+    if (vec_ok && reorder_rows_plan(d, qr)) {
+        if ((d->src_scale.set && !args->src_scale)
+                || (d->dst_scale.set && !args->dst_scale)
+                || (d->src_zp.set && !args->src_zp)
+                || (d->dst_zp.set && !args->dst_zp))
+            return fail(QMM_INVALID_ARGUMENTS, "reorder attribute buffer missing");
+        qr.src = args->src;
+        qr.dst = args->dst;
+        qr.src_scale.ptr = d->src_scale.set ? args->src_scale : nullptr;
+        qr.dst_scale.ptr = d->dst_scale.set ? args->dst_scale : nullptr;
+        qr.src_zp.ptr = d->src_zp.set ? args->src_zp : nullptr;
+        qr.dst_zp = d->dst_zp.set ? (const int32_t *)args->dst_zp : nullptr;
+        launch_quantize_rows(qr, stream);
+    } else if (d->src_layout == QMM_LAYOUT_PLAIN
+            && d->dst_layout == QMM_LAYOUT_PLAIN) {
         generic_reorder_params_t P;
         std::memset(&P, 0, sizeof(P));
         P.desc = *d;

@@ -217,6 +217,25 @@ struct w4a8_small_t {
 constexpr int W4A8_SMALL_MAX_GPS = 16; // groups per slice (LDS)
 constexpr int W4A8_SMALL_MAX_M = 64;
 
+// ---- reorder as a quantizer over rows (qmm_quantize.hip) --------------------
+struct quant_rows_q_t {
+    const void *ptr; // nullptr: default value
+    int64_t sr, sc; // strides of the buffer over (row / gr, col / gc)
+    int64_t gr, gc;
+    int32_t dt;
+    int32_t pad_;
+};
+struct quant_rows_params_t {
+    const void *src;
+    void *dst;
+    int64_t rows, cols; // cols % 8 == 0
+    int64_t src_pitch, dst_pitch; // elements
+    int32_t src_dt, dst_dt;
+    int32_t rows_per_thread, pad_; // set by the launcher
+    quant_rows_q_t src_scale, dst_scale, src_zp;
+    const int32_t *dst_zp; // single value or nullptr
+};
+
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
     impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales

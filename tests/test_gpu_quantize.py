@@ -1,0 +1,134 @@
+"""GPU parity of the row-wise quantizing reorder (hip:gfx950:quantize) against
+the CPU oracle's reorder, bit for bit: the kernel performs the reference's
+operations in the reference's order (src/cpu/reorder/simple_reorder.hpp:2500-2640)."""
+import sys
+
+import numpy as np
+import pytest
+
+import onednn_amd as dnnl
+import oracle as O
+from onednn_amd import memory
+from qmm_harness import T, TensorSpec, assert_bit_exact, dt
+
+pytestmark = pytest.mark.gpu
+
+QUANTIZE, REORDER = "hip:gfx950:quantize", "hip:gfx950:reorder"
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    eng = dnnl.engine(dnnl.engine.kind.gpu, 0)
+    return eng, dnnl.stream(eng)
+
+
+def _raw(code, values):
+    v = np.asarray(values).reshape(-1)
+    if code in (dt.s32, dt.s8, dt.u8):
+        return v.astype(O.STORAGE[code])
+    return O.from_f32(code, v.astype(np.float32))
+
+
+def run_case(eng, strm, src_dt, dst_dt, dims, seed, src_scale=None, dst_scale=None, src_zp=None, dst_zp=None,
+             layout=None, dst_layout=None, expect=QUANTIZE, amp=3.0):
+    """Each of *_scale / src_zp: (mask, dt, groups or None, values); dst_zp: int."""
+    r = np.random.default_rng(seed)
+    x = (r.standard_normal(dims) * amp).astype(np.float32)
+    src = TensorSpec(src_dt, list(dims), layout, x)
+    dst = TensorSpec(dst_dt, list(dims), dst_layout or layout)
+    attr = dnnl.primitive_attr()
+    quants, args = {}, {}
+    for name, arg, q, zp in (("src_scale", dnnl.DNNL_ARG_SRC, src_scale, False), ("dst_scale", dnnl.DNNL_ARG_DST, dst_scale, False),
+                             ("src_zp", dnnl.DNNL_ARG_SRC, src_zp, True)):
+        if q is None:
+            continue
+        mask, code, groups, values = q
+        raw = _raw(code, values)
+        if zp:
+            attr.set_zero_points(arg, mask, list(groups or []), code)
+            key = dnnl.DNNL_ARG_ATTR_ZERO_POINTS | arg
+        else:
+            attr.set_scales(arg, mask, list(groups or []), code)
+            key = dnnl.DNNL_ARG_ATTR_SCALES | arg
+        quants[name] = O.Quant(mask, code, raw, groups)
+        args[key] = memory(memory.desc([raw.nbytes], dt.u8, T("a")), eng).write(raw)
+    if dst_zp is not None:
+        attr.set_zero_points_mask(dnnl.DNNL_ARG_DST, 0)
+        raw = np.array([dst_zp], np.int32)
+        quants["dst_zp"] = O.Quant(0, dt.s32, raw)
+        args[dnnl.DNNL_ARG_ATTR_ZERO_POINTS | dnnl.DNNL_ARG_DST] = memory(memory.desc([1], dt.s32, T("a")), eng).write(raw)
+    pd = dnnl.reorder.primitive_desc(eng, src.md(), eng, dst.md(), attr=attr)
+    assert pd.impl_info_str() == expect, pd.impl_info_str()
+    s_mem = memory(src.md(), eng).write(src.raw)
+    d_mem = memory(dst.md(), eng).write(dst.raw)
+    args[dnnl.DNNL_ARG_FROM], args[dnnl.DNNL_ARG_TO] = s_mem, d_mem
+    dnnl.reorder(pd).execute(strm, args)
+    strm.wait()
+    want = dst.raw.copy()
+    O.reorder(src.oracle(), dst.oracle(want), **quants)
+    assert_bit_exact(d_mem.read(dst.raw.dtype), want, "%s -> %s %s" % (src_dt, dst_dt, dims))
+
+
+def test_weights_f32_to_s8_per_column(ctx):
+    eng, strm = ctx
+    say("quantize f32 -> s8, per-column scales")
+    N = 200
+    run_case(eng, strm, dt.f32, dt.s8, (96, N), 1, dst_scale=(2, dt.f32, None, np.random.default_rng(2).uniform(0.01, 0.1, N)))
+
+
+def test_activations_bf16_to_s8_per_row_and_to_u8_with_zero_point(ctx):
+    eng, strm = ctx
+    say("quantize bf16 -> s8 per-row scales; f16 -> u8 with dst zero point")
+    M = 70
+    run_case(eng, strm, dt.bf16, dt.s8, (M, 256), 3, dst_scale=(1, dt.f32, None, np.random.default_rng(4).uniform(0.02, 0.05, M)))
+    run_case(eng, strm, dt.f16, dt.u8, (M, 64), 5, dst_scale=(0, dt.f32, None, [0.04]), dst_zp=128)
+
+
+def test_grouped_source_scales(ctx):
+    """Groups are a source-side attribute in the reference (src/common/reorder.cpp:121-143)."""
+    eng, strm = ctx
+    say("f32 -> s8 with f16 source scales per row and 128 columns; per 64 rows and column")
+    M, K, G = 33, 512, 128
+    sc = np.random.default_rng(6).uniform(2.0, 6.0, (M, K // G))
+    run_case(eng, strm, dt.f32, dt.s8, (M, K), 7, src_scale=(3, dt.f16, (1, G), sc))
+    sc = np.random.default_rng(60).uniform(2.0, 6.0, (256 // 64, 48))
+    run_case(eng, strm, dt.bf16, dt.s8, (256, 48), 70, src_scale=(3, dt.f32, (64, 1), sc), dst_scale=(0, dt.f32, None, [0.5]))
+
+
+def test_weights_to_int4(ctx):
+    eng, strm = ctx
+    say("quantize f32 -> u4 / s4, per-column scales, dst zero point")
+    K, N = 256, 48
+    sc = np.random.default_rng(8).uniform(0.3, 0.6, N)
+    run_case(eng, strm, dt.f32, dt.u4, (K, N), 9, dst_scale=(2, dt.f32, None, sc), dst_zp=8)
+    run_case(eng, strm, dt.bf16, dt.s4, (K, N), 10, dst_scale=(2, dt.bf16, None, sc))
+
+
+def test_to_fp8_and_float_types_with_both_scales(ctx):
+    eng, strm = ctx
+    say("f32 -> f8_e4m3 / f8_e5m2 / bf16 / f16 / f32 with src and dst scales")
+    # (zero points go with integral types only: src/common/reorder.cpp:98-106)
+    for code in (dt.f8_e4m3, dt.f8_e5m2, dt.bf16, dt.f16, dt.f32):
+        run_case(eng, strm, dt.f32, code, (40, 72), 11 + code, src_scale=(0, dt.f32, None, [0.37]),
+                 dst_scale=(2, dt.f32, None, np.random.default_rng(12).uniform(0.5, 2, 72)))
+
+
+def test_three_dims_last_dim_scales(ctx):
+    eng, strm = ctx
+    say("quantize f16 [3, 20, 64] -> s8, scales over the last dim")
+    run_case(eng, strm, dt.f16, dt.s8, (3, 20, 64), 13, dst_scale=(4, dt.f32, None, np.random.default_rng(14).uniform(0.02, 0.05, 64)))
+
+
+def test_other_shapes_stay_with_the_general_reorder(ctx):
+    eng, strm = ctx
+    say("transposing / ragged reorders take the per-element kernel")
+    N = 24
+    sc = (2, dt.f32, None, np.random.default_rng(15).uniform(0.01, 0.1, N))
+    run_case(eng, strm, dt.f32, dt.s8, (64, N), 16, dst_scale=sc, layout="ab", dst_layout="ba", expect=REORDER)
+    run_case(eng, strm, dt.f32, dt.s8, (64, 20), 17, dst_scale=(0, dt.f32, None, [0.05]), expect=REORDER)
+    run_case(eng, strm, dt.f32, dt.s8, (3, 8, 16), 18, dst_scale=(1, dt.f32, None, [0.05, 0.07, 0.09]), expect=REORDER)
