@@ -180,6 +180,16 @@ dnnl_status_t DNNL_API dnnl_matmul_primitive_desc_create(
         const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
         const_dnnl_primitive_attr_t attr);
 
+/* ---- inner product (forward): dnnl.h:2462-2469. Lowered onto the matmul
+ * implementations: src [MB, IC, spatial...] is read as [MB, K], weights
+ * [OC, IC, spatial...] as the transposed [K, OC]. ---- */
+dnnl_status_t DNNL_API dnnl_inner_product_forward_primitive_desc_create(
+        dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine,
+        dnnl_prop_kind_t prop_kind, const_dnnl_memory_desc_t src_desc,
+        const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
+        const_dnnl_primitive_attr_t attr);
+
 #ifdef __cplusplus
 }
 #endif

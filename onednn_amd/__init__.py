@@ -498,6 +498,26 @@ class matmul(_primitive):
             super().__init__(h, eng)
 
 
+class prop_kind:
+    forward_training, forward_inference = 64, 96
+    forward = forward_training
+
+
+class inner_product_forward(_primitive):
+    """dnnl::inner_product_forward: src [MB, IC, spatial...] x weights
+    [OC, IC, spatial...] -> dst [MB, OC], run by the matmul implementations."""
+
+    class primitive_desc(_primitive_desc):
+        def __init__(self, eng, aprop_kind, src_md, weights_md, dst_md,
+                     bias_md=None, attr=None):
+            h = C.c_void_p()
+            _capi.call("dnnl_inner_product_forward_primitive_desc_create",
+                       C.byref(h), eng._h, aprop_kind, src_md._h, weights_md._h,
+                       bias_md._h if bias_md is not None else None, dst_md._h,
+                       attr._h if attr is not None else None)
+            super().__init__(h, eng)
+
+
 class reorder(_primitive):
     class primitive_desc(_primitive_desc):
         def __init__(self, src_engine, src_md, dst_engine, dst_md, attr=None):

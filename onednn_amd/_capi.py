@@ -122,6 +122,7 @@ _SIGNATURES = {
     "dnnl_memory_destroy": (None, [_P]),
     "dnnl_reorder_primitive_desc_create": (None, [_PP, _P, _P, _P, _P, _P]),
     "dnnl_matmul_primitive_desc_create": (None, [_PP, _P, _P, _P, _P, _P, _P]),
+    "dnnl_inner_product_forward_primitive_desc_create": (None, [_PP, _P, _I, _P, _P, _P, _P, _P]),
     # HIP interop and the kernel-level ABI (include/qmm_hip.h)
     "dnnl_hip_interop_stream_create": (None, [_PP, _P, _P]),
     "dnnl_hip_interop_stream_get_stream": (None, [_P, _PP]),

@@ -106,7 +106,8 @@ bool md_equal(const dnnl_memory_desc &a, const dnnl_memory_desc &b) {
     }
     if (a.format_kind == dnnl_format_kind_opaque)
         return a.packed_layout == b.packed_layout
-                && a.packed_bytes == b.packed_bytes;
+                && a.packed_bytes == b.packed_bytes
+                && a.packed_transposed == b.packed_transposed;
     return true;
 }
 

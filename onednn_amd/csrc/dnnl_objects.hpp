@@ -28,6 +28,9 @@ struct dnnl_memory_desc {
     int64_t offset0 = 0;
     int packed_layout = QMM_LAYOUT_PLAIN; // format_kind == opaque
     size_t packed_bytes = 0;
+    // opaque weights of an inner product: dims are [OC, IC, spatial...], the
+    // packed image is that of the matmul weights [K = IC * spatial, N = OC]
+    bool packed_transposed = false;
 
     bool is_zero() const { return ndims == 0; }
     bool is_any() const { return format_kind == dnnl_format_kind_any; }
@@ -164,6 +167,11 @@ struct pd_impl_t {
     dnnl_memory_desc scratchpad;
     int impl = -1; // index into the implementation list
     std::string impl_name;
+    // inner product lowered to matmul: src / wei / bias / dst above are the
+    // matmul view ([MB, K] x [K, OC]); these are what the user sees
+    bool ip = false;
+    dnnl_memory_desc ip_src, ip_wei, ip_bias, ip_dst;
+    dnnl_memory_desc ip_wei_user; // weights as passed (may be format any)
     qmm_matmul_desc_t mm; // kernel-level description (matmul)
     qmm_reorder_desc_t ro; // kernel-level description (reorder)
     size_t scratch_bytes = 0;

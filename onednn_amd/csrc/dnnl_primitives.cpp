@@ -540,6 +540,33 @@ std::string dims_str(const dnnl_memory_desc &md) {
     return s;
 }
 
+// inner product: the weights descriptor the user sees after an implementation
+// resolved format any -- the matmul's packed layout under the inner product's
+// dims, or the plain tensor that is the matmul's row-major [K, OC] (IC-major
+// for the inner product: stride 1 along OC)
+void ip_refresh_weights_md(pd_impl_t &pd) {
+    if (!pd.ip) return;
+    const dnnl_memory_desc &user = pd.ip_wei_user;
+    if (pd.wei.is_packed()) {
+        dnnl_memory_desc r = pd.wei;
+        r.ndims = user.ndims;
+        for (int d = 0; d < user.ndims; d++)
+            r.dims[d] = user.dims[d];
+        r.packed_transposed = true;
+        pd.ip_wei = r;
+    } else if (user.is_any()) {
+        dnnl_dims_t strides;
+        const int nd = user.ndims;
+        strides[0] = 1;
+        strides[nd - 1] = user.dims[0];
+        for (int d = nd - 2; d >= 1; d--)
+            strides[d] = strides[d + 1] * user.dims[d + 1];
+        md_init_plain(pd.ip_wei, nd, user.dims, user.data_type, strides);
+    } else {
+        pd.ip_wei = user;
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -576,12 +603,145 @@ dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *out,
     return dnnl_success;
 }
 
+// ======================= inner product (forward) ===========================
+// src/common/inner_product.cpp:33-110 for the shape rules. The primitive is
+// the matmul [MB, K] x [K, OC] with K = IC * spatial: a source whose trailing
+// dims nest densely is that matrix as it lies in memory, and OC-major weights
+// [OC, IC, spatial...] are the K x OC matrix with strides (1, pitch) -- no
+// data moves. The descriptors the user sees (queries, format any) keep the
+// inner product's dims; opaque weights are marked as transposed so that the
+// prepacking reorder reads the user's [OC, IC, ...] tensor the same way.
+static bool trailing_dims_nest(const dnnl_memory_desc &md) {
+    if (!md.is_plain() || md.strides[md.ndims - 1] != 1) return false;
+    for (int d = md.ndims - 2; d >= 1; d--)
+        if (md.strides[d] != md.strides[d + 1] * md.dims[d + 1]) return false;
+    return true;
+}
+
+dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(
+        dnnl_primitive_desc_t *out, dnnl_engine_t engine,
+        dnnl_prop_kind_t prop_kind, const_dnnl_memory_desc_t src_desc,
+        const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
+        const_dnnl_primitive_attr_t attr) {
+    if (!out || !engine || !src_desc || !weights_desc || !dst_desc)
+        return dnnl_invalid_arguments;
+    if (prop_kind != dnnl_forward_training && prop_kind != dnnl_forward_inference)
+        return dnnl_invalid_arguments;
+    if (bias_desc && bias_desc->ndims == 0) bias_desc = nullptr;
+    const int nd = src_desc->ndims;
+    if (nd < 2 || nd > 5 || weights_desc->ndims != nd || dst_desc->ndims != 2)
+        return dnnl_invalid_arguments;
+    if (src_desc->has_runtime_dims() || weights_desc->has_runtime_dims()
+            || dst_desc->has_runtime_dims())
+        return dnnl_unimplemented;
+    const int64_t MB = src_desc->dims[0], OC = weights_desc->dims[0];
+    int64_t K = 1;
+    for (int d = 1; d < nd; d++) {
+        if (src_desc->dims[d] != weights_desc->dims[d])
+            return dnnl_invalid_arguments;
+        K *= src_desc->dims[d];
+    }
+    if (dst_desc->dims[0] != MB || dst_desc->dims[1] != OC)
+        return dnnl_invalid_arguments;
+    if (bias_desc && (bias_desc->ndims != 1 || bias_desc->dims[0] != OC))
+        return dnnl_invalid_arguments;
+    if (engine->kind != dnnl_gpu) return dnnl_unimplemented;
+
+    // the user-visible descriptors, format any resolved to row-major
+    auto pd = std::make_shared<pd_impl_t>();
+    pd->ip = true;
+    pd->ip_src = *src_desc;
+    pd->ip_wei = pd->ip_wei_user = *weights_desc;
+    pd->ip_dst = *dst_desc;
+    if (bias_desc) pd->ip_bias = *bias_desc;
+    for (dnnl_memory_desc *md : {&pd->ip_src, &pd->ip_dst, &pd->ip_bias}) {
+        if (md->ndims && md->is_any()) {
+            dnnl_memory_desc r;
+            md_init_plain(r, md->ndims, md->dims, md->data_type, nullptr);
+            *md = r;
+        }
+    }
+    if (!trailing_dims_nest(pd->ip_src) || !pd->ip_dst.is_plain()
+            || (pd->ip_bias.ndims && !pd->ip_bias.is_plain()))
+        return dnnl_unimplemented;
+
+    // the matmul view
+    dnnl_memory_desc m_src, m_wei, m_bias;
+    {
+        const dnnl_dims_t dims = {MB, K}, strides = {pd->ip_src.strides[0], 1};
+        md_init_plain(m_src, 2, dims, pd->ip_src.data_type, strides);
+    }
+    const dnnl_dims_t wdims = {K, OC};
+    if (pd->ip_wei.is_any()) {
+        md_init_plain(m_wei, 2, wdims, pd->ip_wei.data_type, nullptr);
+        m_wei.format_kind = dnnl_format_kind_any;
+    } else if (pd->ip_wei.is_packed()) {
+        if (!pd->ip_wei.packed_transposed) return dnnl_unimplemented;
+        m_wei = pd->ip_wei;
+        m_wei.ndims = 2;
+        m_wei.dims[0] = K;
+        m_wei.dims[1] = OC;
+        m_wei.packed_transposed = false;
+    } else if (trailing_dims_nest(pd->ip_wei)) { // OC-major
+        const dnnl_dims_t strides = {1, pd->ip_wei.strides[0]};
+        md_init_plain(m_wei, 2, wdims, pd->ip_wei.data_type, strides);
+    } else if (nd == 2 && pd->ip_wei.is_plain() && pd->ip_wei.strides[0] == 1) {
+        const dnnl_dims_t strides = {pd->ip_wei.strides[1], 1}; // IC-major
+        md_init_plain(m_wei, 2, wdims, pd->ip_wei.data_type, strides);
+    } else {
+        return dnnl_unimplemented;
+    }
+    if (pd->ip_bias.ndims) {
+        const dnnl_dims_t dims = {1, OC}, strides = {OC * pd->ip_bias.strides[0],
+                                                  pd->ip_bias.strides[0]};
+        md_init_plain(m_bias, 2, dims, pd->ip_bias.data_type, strides);
+    }
+
+    // attributes: the weights' OC dim is dim 0 here and dim 1 of the matmul
+    static const dnnl_primitive_attr default_attr;
+    dnnl_primitive_attr a = attr ? *attr : default_attr;
+    {
+        auto it = a.scales.find(DNNL_ARG_WEIGHTS);
+        if (it != a.scales.end() && !it->second.is_default()) {
+            if (it->second.mask == 1)
+                it->second.mask = 2;
+            else if (it->second.mask != 0 || it->second.group_ndims != 0)
+                return dnnl_unimplemented;
+        }
+        if (!a.zp(DNNL_ARG_SRC).is_default() || !a.zp(DNNL_ARG_WEIGHTS).is_default()
+                || !a.zp(DNNL_ARG_DST).is_default())
+            return dnnl_unimplemented; // src/common/inner_product.cpp:99-103
+    }
+    dnnl_status_t st = matmul_shape_check(
+            &m_src, &m_wei, pd->ip_bias.ndims ? &m_bias : nullptr, &pd->ip_dst);
+    if (st != dnnl_success) return st;
+    st = matmul_attr_check(m_src, m_wei, pd->ip_dst, engine, a);
+    if (st != dnnl_success) return st;
+
+    pd->kind = dnnl_matmul;
+    pd->engine = engine;
+    pd->attr = a;
+    pd->user_src = m_src;
+    pd->user_wei = m_wei;
+    if (pd->ip_bias.ndims) pd->user_bias = m_bias;
+    pd->user_dst = pd->ip_dst;
+    st = walk_matmul_impls(*pd, 0);
+    if (st != dnnl_success) return st;
+    ip_refresh_weights_md(*pd);
+    dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc {pd};
+    if (!h) return dnnl_out_of_memory;
+    *out = h;
+    return dnnl_success;
+}
+
 dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd) {
     if (!pd || !pd->p) return dnnl_invalid_arguments;
     if (pd->p->kind != dnnl_matmul) return dnnl_last_impl_reached;
     auto next = std::make_shared<pd_impl_t>(*pd->p);
     const dnnl_status_t st = walk_matmul_impls(*next, pd->p->impl + 1);
     if (st != dnnl_success) return dnnl_last_impl_reached;
+    ip_refresh_weights_md(*next);
     pd->p = next;
     return dnnl_success;
 }
@@ -609,12 +769,17 @@ const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(
         const_dnnl_primitive_desc_t pd, dnnl_query_t what, int index) {
     if (!pd) return nullptr;
     const pd_impl_t &p = *pd->p;
+    // an inner product shows its own descriptors, not the matmul view
+    const dnnl_memory_desc &q_src = p.ip ? p.ip_src : p.src;
+    const dnnl_memory_desc &q_wei = p.ip ? p.ip_wei : p.wei;
+    const dnnl_memory_desc &q_bias = p.ip ? p.ip_bias : p.bias;
+    const dnnl_memory_desc &q_dst = p.ip ? p.ip_dst : p.dst;
     switch (what) {
-        case dnnl_query_src_md: return index == 0 ? &p.src : &g_zero_md;
+        case dnnl_query_src_md: return index == 0 ? &q_src : &g_zero_md;
         case dnnl_query_weights_md:
             if (p.kind != dnnl_matmul) return &g_zero_md;
-            return index == 0 ? &p.wei : index == 1 ? &p.bias : &g_zero_md;
-        case dnnl_query_dst_md: return index == 0 ? &p.dst : &g_zero_md;
+            return index == 0 ? &q_wei : index == 1 ? &q_bias : &g_zero_md;
+        case dnnl_query_dst_md: return index == 0 ? &q_dst : &g_zero_md;
         case dnnl_query_scratchpad_md:
             return index == 0 ? &p.scratchpad : &g_zero_md;
         case dnnl_query_diff_src_md:
@@ -623,10 +788,10 @@ const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(
         case dnnl_query_workspace_md: return &g_zero_md;
         case dnnl_query_exec_arg_md: {
             if (p.kind == dnnl_matmul) {
-                if (index == DNNL_ARG_SRC) return &p.src;
-                if (index == DNNL_ARG_WEIGHTS) return &p.wei;
-                if (index == DNNL_ARG_BIAS) return &p.bias;
-                if (index == DNNL_ARG_DST) return &p.dst;
+                if (index == DNNL_ARG_SRC) return &q_src;
+                if (index == DNNL_ARG_WEIGHTS) return &q_wei;
+                if (index == DNNL_ARG_BIAS) return &q_bias;
+                if (index == DNNL_ARG_DST) return &q_dst;
             } else {
                 if (index == DNNL_ARG_FROM) return &p.src;
                 if (index == DNNL_ARG_TO) return &p.dst;
@@ -657,7 +822,7 @@ dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t pd,
             *(dnnl_engine_t *)result = p.engine;
             break;
         case dnnl_query_primitive_kind:
-            *(dnnl_primitive_kind_t *)result = p.kind;
+            *(dnnl_primitive_kind_t *)result = p.ip ? dnnl_inner_product : p.kind;
             break;
         case dnnl_query_num_of_inputs_s32: *(int *)result = n_inputs(p); break;
         case dnnl_query_num_of_outputs_s32: *(int *)result = 1; break;
@@ -758,6 +923,31 @@ dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *out,
     if (!(src_md->is_plain() || src_md->is_packed())
             || !(dst_md->is_plain() || dst_md->is_packed()))
         return dnnl_unimplemented;
+    // Packed weights of an inner product carry dims [OC, IC, spatial...] over
+    // the image of the matmul weights [K, OC]: hand the kernels that matrix.
+    // The plain side's dims 1.. must nest (then K has one stride).
+    const dnnl_memory_desc *tp = src_md->is_packed() && src_md->packed_transposed
+            ? src_md
+            : (dst_md->is_packed() && dst_md->packed_transposed ? dst_md
+                                                                : nullptr);
+    if (tp) {
+        const dnnl_memory_desc *pl = tp == src_md ? dst_md : src_md;
+        const int nd = pl->ndims;
+        if (!pl->is_plain() || nd < 2) return dnnl_unimplemented;
+        int64_t K = 1;
+        for (int d = 1; d < nd; d++)
+            K *= pl->dims[d];
+        for (int d = nd - 2; d >= 1; d--)
+            if (pl->strides[d] != pl->strides[d + 1] * pl->dims[d + 1])
+                return dnnl_unimplemented;
+        for (qmm_tensor_t *t : {&R.src, &R.dst}) {
+            t->ndims = 2;
+            t->dims[0] = K;
+            t->dims[1] = pl->dims[0];
+            t->strides[0] = pl->strides[nd - 1];
+            t->strides[1] = pl->strides[0];
+        }
+    }
     fill_quant(R.src_scale, a.scale(DNNL_ARG_SRC), dnnl_f32);
     fill_quant(R.dst_scale, a.scale(DNNL_ARG_DST), dnnl_f32);
     fill_quant(R.src_zp, a.zp(DNNL_ARG_SRC), dnnl_s32);

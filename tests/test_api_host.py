@@ -374,3 +374,25 @@ def test_memory_without_device_fails_loudly(eng):
     expect(status.runtime_error, lambda: dnnl.stream(eng))
     pd = dnnl.matmul.primitive_desc(eng, md, md, md)
     expect(status.runtime_error, lambda: dnnl.matmul(pd))
+
+
+def test_inner_product_descriptor_is_lowered_to_matmul(eng):
+    src = memory.desc([8, 16, 2, 2], dt.s8, T("abcd"))
+    wei = memory.desc([32, 16, 2, 2], dt.s8, tag.any)
+    dst = memory.desc([8, 32], dt.f32, T("ab"))
+    pd = dnnl.inner_product_forward.primitive_desc(eng, dnnl.prop_kind.forward_inference, src, wei, dst)
+    assert pd.impl_info_str() == "hip:gfx950:mfma_b8"
+    assert pd.src_desc().get_dims() == [8, 16, 2, 2]
+    w = pd.weights_desc()
+    assert w.get_dims() == [32, 16, 2, 2] and w.get_format_kind() == memory.format_kind.opaque
+    # the prepacking reorder takes the user's OC-major tensor
+    r = dnnl.reorder.primitive_desc(eng, memory.desc([32, 16, 2, 2], dt.s8, T("abcd")), eng, w)
+    assert r.impl_info_str() == "hip:gfx950:prepack"
+    # shape errors and unsupported attributes
+    expect(status.invalid_arguments, lambda: dnnl.inner_product_forward.primitive_desc(
+        eng, dnnl.prop_kind.forward_inference, src, memory.desc([32, 8, 2, 2], dt.s8, tag.any), dst))
+    attr = dnnl.primitive_attr()
+    attr.set_zero_points_mask(dnnl.DNNL_ARG_SRC, 0)
+    expect(status.unimplemented, lambda: dnnl.inner_product_forward.primitive_desc(
+        eng, dnnl.prop_kind.forward_inference, src, wei, dst, attr=attr))
+
