@@ -179,6 +179,29 @@ def test_generic_grouped_dynamic_quant_and_chain(ctx):
     assert_bit_exact(got, p.run_oracle(), "grouped chain")
 
 
+@pytest.mark.parametrize("mask,big", [(1, False), (2, False), (4, False), (6, False), (7, False), (3, False),
+                                      (4, True), (6, True), (7, True)])
+def test_prelu_weights_layout_batched(ctx, mask, big):
+    """prelu weights of a 3-D dst lie in acb order (the N axis outside the M
+    axis), src/cpu/primitive_attr_postops.cpp:190-225; `big` takes the MFMA
+    kernels' row interpreter instead of the generic kernel."""
+    eng, strm = ctx
+    say("prelu mask %d big %d" % (mask, big))
+    r = rnd(300 + mask)
+    B, M, K, N = (2, 128, 64, 192) if big else (3, 5, 32, 7)
+    wd = [B if mask & 1 else 1, N if mask & 4 else 1, M if mask & 2 else 1]  # a, c, b
+    p = Problem(TensorSpec(dt.s8, [B, M, K], None, r.integers(-20, 21, (B, M, K))),
+                TensorSpec(dt.s8, [B, K, N], None, r.integers(-20, 21, (B, K, N))),
+                TensorSpec(dt.f32, [B, M, N]),
+                post_ops=[{"kind": "prelu", "mask": mask, "weights": 2.0 ** r.integers(-3, 3, wd)}])
+    got, pd = p.run_gpu(eng, strm, return_pd=True)
+    if big:
+        assert pd.impl_info_str() == MFMA, pd.impl_info_str()
+    assert_bit_exact(got, p.run_oracle(), "prelu")
+    if not big:
+        assert_bit_exact(p.run_gpu(eng, strm, impl=GENERIC), p.run_oracle(), "prelu generic")
+
+
 @pytest.mark.parametrize("act,wei,zp", [(dt.bf16, dt.u4, dt.u4), (dt.f16, dt.s4, dt.s8), (dt.bf16, dt.s8, None)])
 def test_generic_float_paths_bit_exact(ctx, act, wei, zp):
     """Sequential f32 accumulation in k order, as the reference's float path."""

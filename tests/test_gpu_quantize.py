@@ -35,10 +35,10 @@ def _raw(code, values):
 
 
 def run_case(eng, strm, src_dt, dst_dt, dims, seed, src_scale=None, dst_scale=None, src_zp=None, dst_zp=None,
-             layout=None, dst_layout=None, expect=QUANTIZE, amp=3.0):
+             layout=None, dst_layout=None, expect=QUANTIZE, amp=3.0, src_values=None):
     """Each of *_scale / src_zp: (mask, dt, groups or None, values); dst_zp: int."""
     r = np.random.default_rng(seed)
-    x = (r.standard_normal(dims) * amp).astype(np.float32)
+    x = (r.standard_normal(dims) * amp).astype(np.float32) if src_values is None else src_values
     src = TensorSpec(src_dt, list(dims), layout, x)
     dst = TensorSpec(dst_dt, list(dims), dst_layout or layout)
     attr = dnnl.primitive_attr()
@@ -132,3 +132,26 @@ def test_other_shapes_stay_with_the_general_reorder(ctx):
     run_case(eng, strm, dt.f32, dt.s8, (64, N), 16, dst_scale=sc, layout="ab", dst_layout="ba", expect=REORDER)
     run_case(eng, strm, dt.f32, dt.s8, (64, 20), 17, dst_scale=(0, dt.f32, None, [0.05]), expect=REORDER)
     run_case(eng, strm, dt.f32, dt.s8, (3, 8, 16), 18, dst_scale=(1, dt.f32, None, [0.05, 0.07, 0.09]), expect=REORDER)
+
+
+def test_dequantize_int4_and_int8_weights_with_grouped_scales_and_zero_points(ctx):
+    """The decompression direction (src/cpu/reorder/simple_reorder.hpp:2240-2400,
+    :2560-2640): dst = scale[k / g, n] * (w[k, n] - zp[k / g, n]), scale and zero
+    point each with its own groups and type."""
+    eng, strm = ctx
+    say("u4 / s4 / s8 -> f32 / bf16 / f16 with grouped source scales and zero points")
+    K, N = 256, 48
+    r = np.random.default_rng(80)
+    w = r.integers(0, 16, (K, N))
+    for out in (dt.f32, dt.bf16, dt.f16):
+        run_case(eng, strm, dt.u4, out, (K, N), 81, expect=REORDER, src_values=w,
+                 src_scale=(3, dt.f16, (64, 1), r.uniform(0.01, 0.1, (K // 64, N))),
+                 src_zp=(3, dt.u4, (64, 1), r.integers(5, 11, (K // 64, N))))
+    run_case(eng, strm, dt.s4, dt.f32, (K, N), 82, expect=REORDER, src_values=r.integers(-8, 8, (K, N)),
+             src_scale=(3, dt.bf16, (32, 1), r.uniform(0.01, 0.1, (K // 32, N))),
+             src_zp=(3, dt.s8, (128, 1), r.integers(-3, 4, (K // 128, N))))
+    run_case(eng, strm, dt.s8, dt.f32, (K, N), 83, expect=REORDER, src_values=r.integers(-128, 128, (K, N)),
+             src_scale=(2, dt.f32, None, r.uniform(0.01, 0.1, N)), src_zp=(0, dt.s32, None, [3]))
+    # groups along the last dim (activations quantized per row and 64 columns)
+    run_case(eng, strm, dt.s8, dt.bf16, (40, K), 84, expect=REORDER, src_values=r.integers(-128, 128, (40, K)),
+             src_scale=(3, dt.f32, (1, 64), r.uniform(0.01, 0.1, (40, K // 64))))

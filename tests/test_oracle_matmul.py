@@ -269,6 +269,27 @@ def test_post_op_chain_order_bias_and_prelu():
     assert np.array_equal(dst, v.astype(np.float32))
 
 
+@pytest.mark.parametrize("mask", [0, 1, 2, 4, 3, 5, 6, 7])
+def test_prelu_weights_layout_3d(mask):
+    # src/cpu/primitive_attr_postops.cpp:190-225: the weights tensor has dst's
+    # dims where the mask bit is set and 1 elsewhere, in the layout acb for a
+    # 3-D dst (the N axis is the *outer* of the two matrix axes), ab for 2-D.
+    rng = np.random.default_rng(40 + mask)
+    B, M, K, N = 3, 4, 16, 5
+    src = rng.integers(-8, 9, (B, M, K)).astype(np.int8)
+    wei = rng.integers(-8, 9, (B, K, N)).astype(np.int8)
+    wd = [B if mask & 1 else 1, M if mask & 2 else 1, N if mask & 4 else 1]
+    # physical order a, c, b
+    phys = (2.0 ** rng.integers(-3, 3, (wd[0], wd[2], wd[1]))).astype(np.float32)
+    dst = np.zeros((B, M, N), np.float32)
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.F32, dst),
+             post_ops=[{"kind": "prelu", "mask": mask, "weights": phys.reshape(-1)}])
+    acc = np.einsum("bmk,bkn->bmn", src.astype(np.int64), wei.astype(np.int64)).astype(np.float32)
+    logical = np.broadcast_to(phys.transpose(0, 2, 1), (B, M, N))
+    want = np.where(acc >= 0, acc, acc * logical)
+    assert np.array_equal(dst, want)
+
+
 def test_zero_dim_is_a_no_op():
     dst = np.full((0, 4), 7, np.float32)
     O.matmul(T(O.S8, np.zeros((0, 8), np.int8)), T(O.S8, np.zeros((8, 4), np.int8)), T(O.F32, dst, dims=(0, 4)))
