@@ -26,6 +26,7 @@ DNNL_ARG_ATTR_SCALES = 4096
 DNNL_ARG_ATTR_ZERO_POINTS = 8192
 DNNL_ARG_ATTR_MULTIPLE_POST_OP_BASE = 32768
 DNNL_RUNTIME_DIM_VAL = -(2 ** 63)
+DNNL_RUNTIME_SIZE_VAL = 2 ** 63  # (size_t)DNNL_RUNTIME_DIM_VAL
 DNNL_MEMORY_ALLOCATE = C.c_void_p(2 ** 64 - 1)
 DNNL_MEMORY_NONE = None
 

@@ -9,6 +9,7 @@
 #include <cstring>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -175,6 +176,20 @@ struct pd_impl_t {
     qmm_matmul_desc_t mm; // kernel-level description (matmul)
     qmm_reorder_desc_t ro; // kernel-level description (reorder)
     size_t scratch_bytes = 0;
+    // matmul whose descriptors hold DNNL_RUNTIME_DIM_VAL: no implementation is
+    // chosen until execute sees the memory objects' own descriptors
+    bool runtime = false;
+};
+
+// One resolved shape of a runtime-dims matmul: the concrete descriptor, its
+// plan and a library-owned scratchpad. Owned by the primitive's cache.
+struct rt_entry_t {
+    dnnl_memory_desc src, wei, bias, dst;
+    std::shared_ptr<pd_impl_t> pd;
+    qmm_plan_t *plan = nullptr;
+    void *scratch = nullptr;
+    uint64_t stamp = 0;
+    ~rt_entry_t();
 };
 
 struct dnnl_primitive_desc {
@@ -186,6 +201,10 @@ struct dnnl_primitive {
     dnnl_primitive_desc pd_handle; // what dnnl_primitive_get_primitive_desc returns
     qmm_plan_t *plan = nullptr;
     void *lib_scratch = nullptr; // library-managed scratchpad
+    // runtime dims: the shapes seen so far, least recently used evicted
+    std::mutex rt_mutex;
+    std::vector<std::shared_ptr<rt_entry_t>> rt;
+    uint64_t rt_clock = 0;
 };
 
 // helpers shared between translation units

@@ -567,7 +567,104 @@ void ip_refresh_weights_md(pd_impl_t &pd) {
     }
 }
 
+// ---- runtime dims -----------------------------------------------------------
+// The descriptors of the memory objects passed to execute stand in for the
+// primitive descriptor's wherever that holds DNNL_RUNTIME_DIM_VAL (as
+// ctx.memory_mdw does in the reference, src/common/primitive_exec_types.cpp);
+// the concrete problem then goes through the ordinary implementation list.
+// Each primitive remembers the last few shapes it has run.
+constexpr size_t RT_CACHE_ENTRIES = 16;
+
+bool rt_md_matches(const dnnl_memory_desc &want, const dnnl_memory_desc &got) {
+    if (got.ndims != want.ndims || got.data_type != want.data_type) return false;
+    if (!got.is_plain() || got.has_runtime_dims()) return false;
+    for (int d = 0; d < want.ndims; d++) {
+        if (want.dims[d] != DNNL_RUNTIME_DIM_VAL && want.dims[d] != got.dims[d])
+            return false;
+        if (want.strides[d] != DNNL_RUNTIME_DIM_VAL
+                && want.strides[d] != got.strides[d])
+            return false;
+    }
+    return true;
+}
+
+dnnl_status_t resolve_runtime_matmul(dnnl_primitive *prim,
+        const std::map<int, dnnl_memory_t> &args,
+        std::shared_ptr<rt_entry_t> &out) {
+    const pd_impl_t &pd = *prim->pd;
+    auto md_of = [&](int arg) -> const dnnl_memory_desc * {
+        auto it = args.find(arg);
+        return it == args.end() ? nullptr : &it->second->md;
+    };
+    const dnnl_memory_desc *src = md_of(DNNL_ARG_SRC), *wei = md_of(DNNL_ARG_WEIGHTS),
+                           *dst = md_of(DNNL_ARG_DST), *bias = md_of(DNNL_ARG_BIAS);
+    if (!src || !wei || !dst) return dnnl_invalid_arguments;
+    const bool with_bias = pd.bias.ndims != 0;
+    if (with_bias && !bias) return dnnl_invalid_arguments;
+    if (!rt_md_matches(pd.src, *src) || !rt_md_matches(pd.wei, *wei)
+            || !rt_md_matches(pd.dst, *dst)
+            || (with_bias && !rt_md_matches(pd.bias, *bias)))
+        return dnnl_invalid_arguments;
+    if (src->has_zero_dim() || wei->has_zero_dim() || dst->has_zero_dim()) {
+        out.reset();
+        return matmul_shape_check(src, wei, with_bias ? bias : nullptr, dst);
+    }
+
+    std::lock_guard<std::mutex> lock(prim->rt_mutex);
+    for (auto &e : prim->rt)
+        if (md_equal(e->src, *src) && md_equal(e->wei, *wei)
+                && md_equal(e->dst, *dst)
+                && (!with_bias || md_equal(e->bias, *bias))) {
+            e->stamp = ++prim->rt_clock;
+            out = e;
+            return dnnl_success;
+        }
+
+    dnnl_status_t st
+            = matmul_shape_check(src, wei, with_bias ? bias : nullptr, dst);
+    if (st != dnnl_success) return st;
+    st = matmul_attr_check(*src, *wei, *dst, pd.engine, pd.attr);
+    if (st != dnnl_success) return st;
+    auto e = std::make_shared<rt_entry_t>();
+    e->src = *src;
+    e->wei = *wei;
+    e->dst = *dst;
+    if (with_bias) e->bias = *bias;
+    e->pd = std::make_shared<pd_impl_t>(pd);
+    pd_impl_t &c = *e->pd;
+    c.runtime = false;
+    c.user_src = *src;
+    c.user_wei = *wei;
+    c.user_dst = *dst;
+    c.user_bias = with_bias ? *bias : dnnl_memory_desc();
+    // the scratchpad of a shape is not known to the user beforehand
+    c.attr.scratchpad_mode = dnnl_scratchpad_mode_library;
+    st = walk_matmul_impls(c, 0);
+    if (st != dnnl_success) return st;
+    const int qs = qmm_matmul_plan_create(&e->plan, c.impl, &c.mm);
+    if (qs != QMM_OK) return from_qmm(qs);
+    if (c.scratch_bytes && hipMalloc(&e->scratch, c.scratch_bytes) != hipSuccess)
+        return dnnl_out_of_memory;
+    e->stamp = ++prim->rt_clock;
+    if (prim->rt.size() >= RT_CACHE_ENTRIES) {
+        size_t oldest = 0;
+        for (size_t i = 1; i < prim->rt.size(); i++)
+            if (prim->rt[i]->stamp < prim->rt[oldest]->stamp) oldest = i;
+        prim->rt.erase(prim->rt.begin() + oldest);
+    }
+    prim->rt.push_back(e);
+    out = e;
+    return dnnl_success;
+}
+
 } // namespace
+
+// An evicted or destroyed shape: hipFree waits for the kernels that still use
+// the scratchpad.
+rt_entry_t::~rt_entry_t() {
+    if (plan) qmm_matmul_plan_destroy(plan);
+    if (scratch) (void)hipFree(scratch);
+}
 
 extern "C" {
 
@@ -595,8 +692,32 @@ dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *out,
     if (bias_desc) pd->user_bias = *bias_desc;
     pd->user_dst = *dst_desc;
     if (engine->kind != dnnl_gpu) return dnnl_unimplemented; // empty list
-    st = walk_matmul_impls(*pd, 0);
-    if (st != dnnl_success) return st;
+    bool runtime = false;
+    for (const dnnl_memory_desc *md :
+            {&pd->user_src, &pd->user_wei, &pd->user_bias, &pd->user_dst})
+        runtime = runtime || (md->ndims && md->has_runtime_dims());
+    if (runtime) {
+        // format any cannot be resolved without the dims
+        // (src/common/matmul_pd.hpp:266-277); everything that depends on the
+        // dims is decided per shape at execution
+        for (const dnnl_memory_desc *md :
+                {&pd->user_src, &pd->user_wei, &pd->user_bias, &pd->user_dst})
+            if (md->ndims && !md->is_plain()) return dnnl_unimplemented;
+        pd->runtime = true;
+        pd->src = pd->user_src;
+        pd->wei = pd->user_wei;
+        pd->bias = pd->user_bias;
+        pd->dst = pd->user_dst;
+        for (auto &e : pd->attr.post_ops.entries)
+            if (e.kind == dnnl_binary) {
+                if (!e.user_src1_desc.is_plain()) return dnnl_unimplemented;
+                e.src1_desc = e.user_src1_desc;
+            }
+        pd->impl_name = "hip:gfx950:runtime_dims";
+    } else {
+        st = walk_matmul_impls(*pd, 0);
+        if (st != dnnl_success) return st;
+    }
     dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc {pd};
     if (!h) return dnnl_out_of_memory;
     *out = h;
@@ -737,7 +858,8 @@ dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(
 
 dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd) {
     if (!pd || !pd->p) return dnnl_invalid_arguments;
-    if (pd->p->kind != dnnl_matmul) return dnnl_last_impl_reached;
+    if (pd->p->kind != dnnl_matmul || pd->p->runtime)
+        return dnnl_last_impl_reached;
     auto next = std::make_shared<pd_impl_t>(*pd->p);
     const dnnl_status_t st = walk_matmul_impls(*next, pd->p->impl + 1);
     if (st != dnnl_success) return dnnl_last_impl_reached;
@@ -970,7 +1092,7 @@ dnnl_status_t dnnl_primitive_create(
     if (!p) return dnnl_out_of_memory;
     p->pd = pd->p;
     p->pd_handle.p = pd->p;
-    if (p->pd->kind == dnnl_matmul) {
+    if (p->pd->kind == dnnl_matmul && !p->pd->runtime) {
         const dnnl_engine *eng = p->pd->engine;
         if (eng->device < 0 || hipSetDevice(eng->device) != hipSuccess) {
             delete p;
@@ -1013,8 +1135,8 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         dnnl_stream_t stream, int nargs, const dnnl_exec_arg_t *c_args) {
     if (!primitive || !stream) return dnnl_invalid_arguments;
     if (nargs > 0 && !c_args) return dnnl_invalid_arguments;
-    const pd_impl_t &pd = *primitive->pd;
-    if (stream->engine != pd.engine) return dnnl_invalid_arguments;
+    const pd_impl_t &upd = *primitive->pd;
+    if (stream->engine != upd.engine) return dnnl_invalid_arguments;
 
     std::map<int, dnnl_memory_t> args;
     int n_in = 0, extra_in = 0, n_out = 0, extra_out = 0;
@@ -1023,7 +1145,7 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         dnnl_memory_t mem = c_args[i].memory;
         if (!mem) continue; // dummy arguments are allowed
         if (args.count(arg)) return dnnl_invalid_arguments;
-        switch (arg_usage(pd, arg)) {
+        switch (arg_usage(upd, arg)) {
             case usage_t::input:
                 args[arg] = mem;
                 n_in++;
@@ -1038,15 +1160,32 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
             case usage_t::unused: break;
         }
     }
-    if (n_in != n_inputs(pd) + extra_in) return dnnl_invalid_arguments;
+    if (n_in != n_inputs(upd) + extra_in) return dnnl_invalid_arguments;
     if (n_out != 1 + extra_out) return dnnl_invalid_arguments;
 
     auto handle = [&](int arg) -> void * {
         auto it = args.find(arg);
         return it == args.end() ? nullptr : it->second->handle;
     };
-    if (pd.engine->device < 0 || hipSetDevice(pd.engine->device) != hipSuccess)
+    if (upd.engine->device < 0
+            || hipSetDevice(upd.engine->device) != hipSuccess)
         return dnnl_runtime_error;
+
+    // a runtime-dims matmul becomes a concrete one here, per shape
+    const pd_impl_t *concrete = &upd;
+    qmm_plan_t *plan = primitive->plan;
+    void *lib_scratch = primitive->lib_scratch;
+    std::shared_ptr<rt_entry_t> rt_hold;
+    if (upd.kind == dnnl_matmul && upd.runtime) {
+        const dnnl_status_t rs = resolve_runtime_matmul(
+                const_cast<dnnl_primitive *>(primitive), args, rt_hold);
+        if (rs != dnnl_success) return rs;
+        if (!rt_hold) return dnnl_success; // a zero dim: nothing to compute
+        concrete = rt_hold->pd.get();
+        plan = rt_hold->plan;
+        lib_scratch = rt_hold->scratch;
+    }
+    const pd_impl_t &pd = *concrete;
 
     const int verbose = dnnl_amd_verbose_level();
     std::chrono::steady_clock::time_point t0;
@@ -1087,8 +1226,8 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
                         DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_WEIGHTS);
         }
         A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
-                                        : primitive->lib_scratch;
-        st = qmm_matmul_launch(primitive->plan, &A, stream->hip_stream);
+                                        : lib_scratch;
+        st = qmm_matmul_launch(plan, &A, stream->hip_stream);
     } else {
         if (pd.src.has_zero_dim()) return dnnl_success;
         qmm_reorder_args_t A;

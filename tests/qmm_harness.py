@@ -196,10 +196,27 @@ class Problem:
                     raise RuntimeError("implementation %s does not take this problem" % impl)
         return pd
 
+    def runtime_primitive_desc(self, eng, runtime):
+        """`runtime`: {"src" / "wei" / "dst" / "bias": dim indices that become
+        DNNL_RUNTIME_DIM_VAL}; layouts must be tags."""
+        def md(spec, name):
+            dims = list(spec.dims)
+            for i in runtime.get(name, ()):
+                dims[i] = dnnl.DNNL_RUNTIME_DIM_VAL
+            return memory.desc(dims, spec.dt, T(spec.layout))
+        return dnnl.matmul.primitive_desc(
+            eng, md(self.src, "src"), md(self.wei, "wei"), md(self.dst, "dst"),
+            bias_md=md(self.bias, "bias") if self.bias is not None else None, attr=self.attr())
+
     def run_gpu(self, eng, strm, weights_any=False, impl=None, dst_init=None,
-                scratchpad_user=False, return_pd=False):
-        pd = self.primitive_desc(eng, weights_any, impl, scratchpad_user)
-        prim = dnnl.matmul(pd)
+                scratchpad_user=False, return_pd=False, prim=None):
+        """`prim`: a primitive made from runtime_primitive_desc (its memory
+        objects then carry this problem's own descriptors)."""
+        if prim is not None:
+            pd = _ConcreteDescs(self)
+        else:
+            pd = self.primitive_desc(eng, weights_any, impl, scratchpad_user)
+            prim = dnnl.matmul(pd)
         args = {}
         args[dnnl.DNNL_ARG_SRC] = memory(pd.src_desc(), eng).write(self.src.raw)
         wmd = pd.weights_desc()
@@ -238,6 +255,29 @@ class Problem:
         strm.wait()
         out = dst_mem.read(self.dst.raw.dtype)
         return (out, pd) if return_pd else out
+
+
+class _ConcreteDescs:
+    """Stands in for a primitive descriptor when the primitive was created with
+    runtime dims: the descriptors are the problem's own."""
+
+    def __init__(self, p):
+        self.p = p
+
+    def src_desc(self):
+        return self.p.src.md()
+
+    def weights_desc(self):
+        return self.p.wei.md()
+
+    def dst_desc(self):
+        return self.p.dst.md()
+
+    def bias_desc(self):
+        return self.p.bias.md()
+
+    def scratchpad_desc(self):
+        return memory.desc()
 
 
 # ---------------------------------------------------------------------------

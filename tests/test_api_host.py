@@ -396,3 +396,31 @@ def test_inner_product_descriptor_is_lowered_to_matmul(eng):
     expect(status.unimplemented, lambda: dnnl.inner_product_forward.primitive_desc(
         eng, dnnl.prop_kind.forward_inference, src, wei, dst, attr=attr))
 
+
+
+def test_runtime_dims_descriptor(eng):
+    """Descriptors holding DNNL_RUNTIME_DIM_VAL: the dims stay open until
+    execute; format any cannot be resolved without them
+    (src/common/matmul_pd.hpp:266-277) and the batch dims are runtime together
+    or not at all (src/common/matmul.cpp:375-386)."""
+    R = dnnl.DNNL_RUNTIME_DIM_VAL
+    src = memory.desc([R, 256], dt.s8, T("ab"))
+    wei = memory.desc([256, 128], dt.s8, T("ab"))
+    dst = memory.desc([R, 128], dt.f32, T("ab"))
+    assert src.get_strides() == [256, 1]
+    assert src.get_size() == dnnl.DNNL_RUNTIME_SIZE_VAL
+    pd = dnnl.matmul.primitive_desc(eng, src, wei, dst)
+    assert pd.impl_info_str() == "hip:gfx950:runtime_dims"
+    assert pd.src_desc().get_dims() == [R, 256]
+    assert pd.dst_desc() == dst
+    assert pd.scratchpad_desc().is_zero()
+    assert not pd.next_impl()
+    expect(status.unimplemented, lambda: dnnl.matmul.primitive_desc(
+        eng, src, memory.desc([256, 128], dt.s8, tag.any), dst))
+    expect(status.invalid_arguments, lambda: dnnl.matmul.primitive_desc(
+        eng, memory.desc([R, 8, 256], dt.s8, T("abc")), memory.desc([4, 256, 128], dt.s8, T("abc")),
+        memory.desc([R, 8, 128], dt.f32, T("abc"))))
+    # fully open
+    pd = dnnl.matmul.primitive_desc(eng, memory.desc([R, R], dt.s8, T("ab")), memory.desc([R, R], dt.s8, T("ab")),
+                                    memory.desc([R, R], dt.f32, T("ab")))
+    assert pd.impl_info_str() == "hip:gfx950:runtime_dims"
