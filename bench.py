@@ -147,7 +147,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TFLOP/s",
                      "frac": round(kern_tops / PEAK_INT8, 4),
                      "traffic": TRAFFIC_C2_BYTES if args.variant == 0 else None,
-                     "kernel": "gemm_b8x_kernel (int8, 256x256 tile)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
+                     "kernel": "gemm_b8y_kernel (int8, 256x256 tile, 16x16x64 MFMA)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }
 

@@ -133,6 +133,7 @@ _SIGNATURES = {
     "qmm_reorder_impl_name": (C.c_char_p, [_P]),
     "qmm_set_gemm_variant": (None, [_I]),
     "qmm_set_w4a8_variant": (None, [_I]),
+    "qmm_set_b8x_variant": (None, [_I]),
 }
 
 _lib = None
@@ -153,6 +154,7 @@ def lib():
             f.restype = _I if res is None else res
         L.qmm_set_gemm_variant.restype = None
         L.qmm_set_w4a8_variant.restype = None
+        L.qmm_set_b8x_variant.restype = None
         _lib = L
     return _lib
 

@@ -50,6 +50,7 @@ void launch_pack_w4(const void *src, void *dst, int dt, int64_t batch,
 void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
+void set_gemm_b8x_variant(int v);
 } // namespace qmm
 
 using namespace qmm;
@@ -1003,6 +1004,10 @@ QMM_API void qmm_set_gemm_variant(int v) {
 // same for mfma_w4a8 (0: by problem size, 1..3: tile configuration)
 QMM_API void qmm_set_w4a8_variant(int v) {
     g_w4a8_variant = v;
+}
+// the 256 x 256 int8 kernel's MFMA shape (0: 32 x 32 x 32, 1: 16 x 16 x 64)
+QMM_API void qmm_set_b8x_variant(int v) {
+    qmm::set_gemm_b8x_variant(v);
 }
 
 // ---------------------------------------------------------------------------

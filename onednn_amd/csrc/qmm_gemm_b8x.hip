@@ -45,9 +45,14 @@ constexpr int STAGES = 4;
 constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
 constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
 constexpr uint32_t RING = STAGES * STAGE_BYTES; // 128 KiB, power of two
-constexpr int SS_OFF = RING; // 256 per-row source scales (f32)
 constexpr int STG_WAVE = 64 * 128 * 4; // epilogue staging of one wave (in the ring)
-constexpr int LDS_TOTAL = RING + 1024;
+// The kernels on 16 x 16 MFMAs stage with a row pitch of 132 words: a lane
+// group of 16 holds rows 4 apart, which a pitch of 128 would put on the same
+// banks.
+constexpr int STG_PITCH16 = 132;
+constexpr int STG_WAVE16 = 64 * STG_PITCH16 * 4;
+constexpr int SS_OFF = 4 * STG_WAVE16; // 256 per-row source scales (f32)
+constexpr int LDS_TOTAL = SS_OFF + 1024;
 
 template <int N, typename F>
 QMM_D void static_for(F &&f) {
@@ -60,6 +65,12 @@ QMM_D void static_for(F &&f) {
 // chunk swizzle of the row-major A tile (4 chunks of 16 bytes per row)
 QMM_D int a_swz(int row, int q) {
     return q ^ ((row >> 2) & 3);
+}
+// the same for fragments of 16 rows x 4 chunks (lane = row % 16 + 16 * chunk):
+// measured free of bank conflicts (SQ_LDS_BANK_CONFLICT), which the swizzle
+// above is not for that access shape
+QMM_D int a_swz16(int row, int q) {
+    return q ^ ((row >> 1) & 3);
 }
 
 } // namespace b8x
@@ -207,7 +218,7 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 // the matrix and the dst rows are vector-aligned: no per-lane conditions, so
 // the rows pipeline. FAST is the recognised epilogue shape, DSTK the dst type,
 // EXT whether bias / dst scale / dst zero point take part (epilogue_full4).
-template <int FAST, int DSTK, bool EXT, bool F8>
+template <int FAST, int DSTK, bool EXT, bool F8, int PITCH>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const ep_cols_t &cols,
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
@@ -219,7 +230,7 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
 #pragma unroll UNR
     for (int it = 0; it < 32; it++) {
         const int row = it * 2 + (lane >> 5);
-        const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
+        const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
         const float ss = ssl[row];
         const int64_t m = m_first + row;
         float d[4];
@@ -241,11 +252,16 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
 // Epilogue of one 256 x 256 block tile, shared by the int8 and fp8 kernels.
 // LEAN: only the shapes up to EP_FAST_SUM with a float dst run straight-line
 // (fp8 and short-K launches; everything else they accept takes the row path)
-template <bool F8, bool LEAN, typename AccT>
-QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
+template <bool F8, bool LEAN, typename AccT, int NFRAG>
+QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
         uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
         int wm0, int wn0, int bz) {
     using namespace b8x;
+    // NFRAG 4: 32 x 32 fragments (layout below); NFRAG 8: 16 x 16 fragments,
+    // register r of lane l is row 4*(l/16) + r, column l%16
+    constexpr bool MI16 = NFRAG == 8;
+    constexpr int PITCH = MI16 ? STG_PITCH16 : 128;
+    constexpr int STGW = MI16 ? STG_WAVE16 : STG_WAVE;
     // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
     // column l%32 of its 32x32 fragment. The wave tile goes through LDS in two
     // halves of 64 rows x 128 columns (the ring is free now, every wave takes a
@@ -261,9 +277,11 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
     // by-value copy `p` stays in registers.
     const epilogue_t &epk
             = ((const gemm_params_t *)__builtin_amdgcn_kernarg_segment_ptr())->ep;
-    const uint32_t stg_w = lds_base + wave * STG_WAVE
-            + (4 * (lane >> 5) * 128 + (lane & 31)) * 4;
-    const int *const stg_r = (const int *)lds + wave * (STG_WAVE / 4);
+    const uint32_t stg_w = lds_base + wave * STGW
+            + (MI16 ? 4 * (lane >> 4) * PITCH + (lane & 15)
+                    : 4 * (lane >> 5) * 128 + (lane & 31))
+                    * 4;
+    const int *const stg_r = (const int *)lds + wave * (STGW / 4);
     const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
     const int ecol = (lane & 31) * 4;
     const int en = n0 + wn0 + ecol;
@@ -303,23 +321,37 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
             && (!LEAN || (ep.fast <= EP_FAST_SUM && dstk <= EP_DST_F16));
     static_for<2>([&](auto H) {
         constexpr int h = decltype(H)::value;
+        if constexpr (MI16) {
 #pragma unroll
-        for (int i2 = 0; i2 < 2; i2++)
+            for (int i2 = 0; i2 < 4; i2++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+                for (int j = 0; j < 8; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
-                                 "a"(acc[2 * h + i2][j][r]),
-                                 "n"(((i2 * 32 + 8 * (r / 4) + (r % 4)) * 128
-                                             + j * 32)
-                                         * 4)
-                                 : "memory");
+                    for (int r = 0; r < 4; r++)
+                        asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
+                                     "a"(acc[4 * h + i2][j][r]),
+                                     "n"(((i2 * 16 + r) * PITCH + j * 16) * 4)
+                                     : "memory");
+        } else {
+#pragma unroll
+            for (int i2 = 0; i2 < 2; i2++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
+                                     "a"(acc[2 * h + i2][j][r]),
+                                     "n"(((i2 * 32 + 8 * (r / 4) + (r % 4)) * 128
+                                                 + j * 32)
+                                             * 4)
+                                     : "memory");
+        }
         if (full) {
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
 #define QX_EP_ROWS(F, D, X) \
-    ep_rows_full<F, D, X, F8>(ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en)
+    ep_rows_full<F, D, X, F8, PITCH>( \
+            ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en)
 #define QX_EP_DST(F) \
     switch (dstk) { \
         case EP_DST_F32: \
@@ -359,7 +391,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[4][4],
 #pragma unroll 2
             for (int it = 0; it < 32; it++) {
                 const int row = it * 2 + (lane >> 5);
-                const int4 t = *(const int4 *)&stg_r[row * 128 + ecol];
+                const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
                 const int lrow = h * 64 + row;
                 const int m = m0 + wm0 + lrow;
                 const float ss = ssl[lrow];
@@ -598,11 +630,200 @@ gemm_b8x_kernel(const gemm_params_t p) {
             p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
 }
 
+
+// ---- int8 on 16 x 16 x 64 MFMAs ---------------------------------------------
+// Same block tile, LDS ring, direct loads and epilogue as gemm_b8x_kernel, but
+// the wave's 128 x 128 tile is 8 x 8 fragments of v_mfma_i32_16x16x64_i8: one
+// instruction contracts a whole 64-k tile (16 cycles), so each accumulator is
+// read and written half as often per multiply-accumulate as with the
+// 32 x 32 x 32 shape. On MI355X that is what the sustained clock responds to:
+// a loop of nothing but MFMAs on random int8 data holds 3.9 POP/s with this
+// shape and 2.9-3.2 POP/s with 32 x 32 x 32 (both 4.6-4.8 POP/s on zeros).
+// An operand fragment is one 16-byte read: lane l holds row (column) l % 16,
+// k 16 * (l / 16) .. + 15 -- chunk l / 16 of the row in the swizzled A tile, and
+// for B the chunk of the packed tile that holds that column and k range.
+// A k-step multiplies the fragments read during the previous k-step (64 MFMAs),
+// reads the next tile's 16 fragments into the other register buffer and
+// requests the tile two further on (8 direct loads), one barrier per k-step.
+#define QY_MF(i, j, cb) \
+    { \
+        QX_SB(); \
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8( \
+                fa[cb][i], fb[cb][j], acc[i][j], 0, 0, 0); \
+        QX_SB(); \
+    }
+#define QY_RA(nb, i) \
+    { \
+        fa[nb][i] = *(const v4i *)(ldsn + a_rel + (i)*1024); \
+        QX_SB(); \
+    }
+#define QY_RB(nb, j) \
+    { \
+        fb[nb][j] = *(const v4i *)(ldsn + b_rel + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        QX_SB(); \
+    }
+// row i of the fragment grid: 8 MFMAs, with up to four other instructions
+// (X0..X3) after the 1st, 3rd, 5th and 7th
+#define QY_ROW(i, CB, X0, X1, X2, X3) \
+    QY_MF(i, 0, CB); X0; QY_MF(i, 1, CB); QY_MF(i, 2, CB); X1; \
+    QY_MF(i, 3, CB); QY_MF(i, 4, CB); X2; QY_MF(i, 5, CB); \
+    QY_MF(i, 6, CB); X3; QY_MF(i, 7, CB);
+#define QY_STEP(CB, NB, DA0, DA1, DA2, DA3, DA4, DB0, DB1, DB2, DB3, DB4) \
+    QY_ROW(0, CB, QY_RA(NB, 0), QY_RB(NB, 0), QY_RB(NB, 1), QY_RB(NB, 2)) \
+    QY_ROW(1, CB, QY_RB(NB, 3), QY_RB(NB, 4), QY_RB(NB, 5), QY_RB(NB, 6)) \
+    QY_ROW(2, CB, QY_RB(NB, 7), QY_RA(NB, 1), DA0, DA1) \
+    QY_ROW(3, CB, QY_RA(NB, 2), DA2, DA3, DA4) \
+    QY_ROW(4, CB, QY_RA(NB, 3), QY_RA(NB, 4), DB0, DB1) \
+    QY_ROW(5, CB, QY_RA(NB, 5), DB2, DB3, DB4) \
+    QY_ROW(6, CB, QY_RA(NB, 6), QY_RA(NB, 7), , ) \
+    QY_ROW(7, CB, , , , )
+#define QY_STEP_D(CB, NB) \
+    QY_STEP(CB, NB, QX_D0(a_vo, sa, dA), QX_D1(a_vo, sa, dA), \
+            QX_D2(a_vo, sa, dA), QX_D3(a_vo, sa, dA), QX_D4(a_vo, sa, dA), \
+            QX_D0(b_vo, sb, dB), QX_D1(b_vo, sb, dB), QX_D2(b_vo, sb, dB), \
+            QX_D3(b_vo, sb, dB), QX_D4(b_vo, sb, dB))
+#define QY_STEP_ND(CB, NB) QY_STEP(CB, NB, , , , , , , , , , )
+#define QY_LAST(CB) \
+    QY_ROW(0, CB, , , , ) QY_ROW(1, CB, , , , ) QY_ROW(2, CB, , , , ) \
+    QY_ROW(3, CB, , , , ) QY_ROW(4, CB, , , , ) QY_ROW(5, CB, , , , ) \
+    QY_ROW(6, CB, , , , ) QY_ROW(7, CB, , , , )
+
+#if defined(QMM_B8X_PART) && QMM_B8X_PART == 4
+__global__ void __launch_bounds__(b8x::NT, 1)
+gemm_b8y_kernel(const gemm_params_t p) {
+    using namespace b8x;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        lt = xcd * per + slot;
+        if (slot >= per || lt >= ntiles) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const int KT = p.K / BK; // host guarantees K % 128 == 0 and KT >= 6
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+
+    uint32_t a_vo[4], b_vo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tid + j * NT;
+        const int row = c >> 2, cp = c & 3;
+        const int gm = min(m0 + row, p.M - 1) - m0;
+        a_vo[j] = (uint32_t)gm * (uint32_t)p.lda + a_swz16(row, cp) * 16;
+        const int nbl = c >> 7, rem = c & 127;
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1) - n0 / 32;
+        b_vo[j] = (uint32_t)nb * (uint32_t)p.kb32 * 1024u + rem * 16;
+    }
+    auto sgpr_ptr = [](const uint8_t *q) {
+        const uint64_t v = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi
+                = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+    };
+    const uint8_t *sa = sgpr_ptr(
+            p.A + (int64_t)bz * p.a_sb + (int64_t)m0 * p.lda);
+    const uint8_t *sb = sgpr_ptr(p.B + (int64_t)bz * p.b_sb
+            + (int64_t)(n0 / 32) * p.kb32 * 1024);
+    uint32_t dA = lds_base + wave * 1024;
+    uint32_t dB = dA + A_BYTES;
+
+    // fragment offsets inside a stage: lane group g = lane / 16 takes k chunk g
+    const int g = lane >> 4;
+    const int arow = wm0 + (lane & 15);
+    const int a_rel = arow * BK + a_swz16(arow, g) * 16;
+    const int b_rel = A_BYTES + (wn0 >> 5) * 2048 + (g >> 1) * 1024
+            + ((g & 1) * 32 + (lane & 15)) * 16;
+
+    v4i acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                acc[i][j][r] = 0;
+    v4i fa[2][8], fb[2][8];
+
+    {
+        float s = 1.f;
+        if (p.ep.src_scale.ptr)
+            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
+                    bz * p.ep.src_scale.sb
+                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
+        ((float *)(lds + SS_OFF))[tid] = s;
+    }
+
+    // ---- prologue: tiles 0..3 requested (the whole ring); tile 0's
+    // fragments read ----
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_WV(24);
+    __syncthreads();
+    uint32_t st = 0; // ring offset of the tile whose fragments are read next
+    {
+        const uint8_t *ldsn = lds;
+        QX_SB();
+        QY_RA(0, 0); QY_RB(0, 0); QY_RB(0, 1); QY_RB(0, 2); QY_RB(0, 3);
+        QY_RB(0, 4); QY_RB(0, 5); QY_RB(0, 6); QY_RB(0, 7); QY_RA(0, 1);
+        QY_RA(0, 2); QY_RA(0, 3); QY_RA(0, 4); QY_RA(0, 5); QY_RA(0, 6);
+        QY_RA(0, 7);
+    }
+    // k-step kt: multiplies tile kt-1 (buffer (kt-1)&1), reads tile kt's
+    // fragments, requests tile kt+3 into the stage tile kt-1 was read from
+    // during the previous k-step
+#define QY_KSTEP(WAITV, BODY) \
+    { \
+        st = (st + STAGE_BYTES) & (RING - 1); \
+        const uint8_t *ldsn = lds + st; \
+        QX_WV(WAITV); \
+        __builtin_amdgcn_s_barrier(); \
+        QX_SB(); \
+        BODY \
+    }
+    for (int kt = 1; kt <= KT - 5; kt += 2) {
+        QY_KSTEP(16, QY_STEP_D(0, 1) QX_ADV_A(); QX_ADV_B();)
+        QY_KSTEP(16, QY_STEP_D(1, 0) QX_ADV_A(); QX_ADV_B();)
+    }
+    QY_KSTEP(16, QY_STEP_ND(0, 1)) // kt = KT-3
+    QY_KSTEP(8, QY_STEP_ND(1, 0)) // kt = KT-2
+    QY_KSTEP(0, QY_STEP_ND(0, 1)) // kt = KT-1
+    QY_LAST(1)
+    __syncthreads();
+
+    tile_epilogue<false, false>(
+            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+}
+#endif // int8, 16 x 16 x 64
+
 // ---- fp8 (e4m3 x e4m3 -> f32) ----------------------------------------------
 // Same tile, ring and epilogue. v_mfma_f32_32x32x64_f8f6f4 consumes a whole
 // 64-k tile per instruction (64 cycles), so a k-step is one group of 16 MFMAs
 // on the fragments read during the previous k-step; the 16 fragment reads of
-// the next tile and the 8 direct loads two tiles further on are spread between
+// the next tile and the 8 direct loads three tiles further on are spread between
 // them. The fragment reads are ordinary LDS loads here (the compiler counts
 // their waits itself; it does not see the direct loads, so it adds no vmcnt);
 // the scheduling barriers keep everything where it is written. An operand is
@@ -743,14 +964,17 @@ gemm_f8x_kernel(const gemm_params_t p) {
         ((float *)(lds + SS_OFF))[tid] = s;
     }
 
-    // ---- prologue: tiles 0, 1, 2 requested; tile 0's fragments read ----
+    // ---- prologue: tiles 0..3 requested (the whole ring); tile 0's
+    // fragments read ----
     QX_FETCH(a_vo, sa, dA); QX_ADV_A();
     QX_FETCH(b_vo, sb, dB); QX_ADV_B();
     QX_FETCH(a_vo, sa, dA); QX_ADV_A();
     QX_FETCH(b_vo, sb, dB); QX_ADV_B();
     QX_FETCH(a_vo, sa, dA); QX_ADV_A();
     QX_FETCH(b_vo, sb, dB); QX_ADV_B();
-    QX_WV(16);
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_WV(24);
     __syncthreads();
     uint32_t st = 0; // ring offset of the tile whose fragments are read next
     {
@@ -763,7 +987,8 @@ gemm_f8x_kernel(const gemm_params_t p) {
         QF_RA(0, 0, 3); QF_RA(0, 1, 3);
     }
     // k-step kt: multiplies tile kt-1 (buffer (kt-1)&1), reads tile kt's
-    // fragments, requests tile kt+2
+    // fragments, requests tile kt+3 into the stage tile kt-1 was read from
+    // during the previous k-step
 #define QF_KSTEP(WAITV, BODY) \
     { \
         st = (st + STAGE_BYTES) & (RING - 1); \
@@ -773,12 +998,12 @@ gemm_f8x_kernel(const gemm_params_t p) {
         QX_SB(); \
         BODY \
     }
-    for (int kt = 1; kt <= KT - 4; kt += 2) {
-        QF_KSTEP(8, QF_STEP_D(0, 1) QX_ADV_A(); QX_ADV_B();)
-        QF_KSTEP(8, QF_STEP_D(1, 0) QX_ADV_A(); QX_ADV_B();)
+    for (int kt = 1; kt <= KT - 5; kt += 2) {
+        QF_KSTEP(16, QF_STEP_D(0, 1) QX_ADV_A(); QX_ADV_B();)
+        QF_KSTEP(16, QF_STEP_D(1, 0) QX_ADV_A(); QX_ADV_B();)
     }
-    QF_KSTEP(8, QF_STEP_D(0, 1)) // kt = KT-3: requests tile KT-1
-    QF_KSTEP(0, QF_STEP_ND(1, 0)) // kt = KT-2
+    QF_KSTEP(16, QF_STEP_ND(0, 1)) // kt = KT-3
+    QF_KSTEP(8, QF_STEP_ND(1, 0)) // kt = KT-2
     QF_KSTEP(0, QF_STEP_ND(0, 1)) // kt = KT-1
     QF_LAST(1)
     __syncthreads();
@@ -830,8 +1055,13 @@ void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream) {
 void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_f8x_kernel, p, stream);
 }
+#elif QMM_B8X_PART == 4
+void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_b8y_kernel, p, stream);
+}
 #endif
 #else
+void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream);
@@ -853,11 +1083,20 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
+// 0: the 32 x 32 x 32 loop, 1: the 16 x 16 x 64 loop (an even number of
+// k-steps, at least 6)
+static int g_b8x_variant = 1;
+void set_gemm_b8x_variant(int v) {
+    g_b8x_variant = v;
+}
+
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     if (f8)
         launch_b8x_fp8(p, stream);
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
+    else if (g_b8x_variant == 1 && p.K % 128 == 0 && p.K >= 6 * 64)
+        launch_b8x_int8_mi16(p, stream);
     else
         launch_b8x_int8(p, stream);
 }
