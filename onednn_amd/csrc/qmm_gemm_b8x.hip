@@ -8,11 +8,12 @@
 // (32 cycles of matrix-core time) is followed by at most two cheap
 // instructions, the LDS fragment reads for the next 16 MFMAs and the
 // global -> LDS loads two tiles ahead are spread between the MFMAs, and the
-// waits are counted (lgkmcnt / vmcnt) instead of full. Measured on MI355X the
-// loop then runs at the MFMA issue rate (65.5 k of 74 k cycles per tile); what
-// remains is the clock the chip sustains while matrix cores and the L2 -> LDS
-// stream are both busy, and the 256 x 256 tile is what minimises that stream
-// per MFMA (32 KiB per 128 MFMAs and CU).
+// waits are counted (lgkmcnt / vmcnt) instead of full. Measured on MI355X
+// (per-dispatch counters) a k-step still takes about 1.5 times its MFMA
+// cycles: what the loop waits for is the L2 -> LDS operand stream, and the
+// 256 x 256 tile is what minimises that stream per MFMA (32 KiB per 128 MFMAs
+// and CU). gemm_b8y_kernel below is the same design on 16 x 16 x 64 MFMAs and
+// is preferred where its K constraints hold.
 //
 // Pipeline (k-step = 64 k, two MFMA sub-steps of 32 k):
 //   LDS ring of 4 stages x (A 256x64 + B 256x64 bytes). Loop iteration kt first
