@@ -419,6 +419,49 @@ def test_mfma_int8_tile256_kernel(ctx, tile256, name):
                          rel=1e-5, scale=np.abs(want.view(np.float32).reshape(-1, N)) + 1e-30, what=name)
 
 
+MI16_CASES = {
+    # K a multiple of 128 with at least 6 k-steps takes the loop on v_mfma_i32_16x16x64_i8
+    "k384_edges_f32": lambda: int8_linear(300, 384, 502, 111, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None),
+    "k640_edges_zp_bias_s32": lambda: int8_linear(260, 640, 250, 112, src_dt=dt.s8, dst_dt=dt.s32, src_zp=3,
+                                                  src_scale=None, bias_dt=dt.s32),
+    "k1024_batched_per_token_bf16": lambda: int8_linear(256, 1024, 300, 113, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None,
+                                                        per_token=True, batch=(3,)),
+    "k512_s8_requant_relu": lambda: int8_linear(512, 512, 256, 114, src_dt=dt.s8, dst_dt=dt.s8, src_zp=None, per_token=True,
+                                                bias_dt=dt.f32, dst_scale=0.25, dst_zp=[-3],
+                                                post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}]),
+    "k768_chain_rows": lambda: int8_linear(130, 768, 260, 115, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None,
+                                           post_ops=[{"kind": "eltwise", "alg": A.eltwise_linear, "alpha": 2.0, "beta": 1.0},
+                                                     {"kind": "eltwise", "alg": A.eltwise_clip_v2, "alpha": -50.0, "beta": 60.0}]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(MI16_CASES))
+def test_mfma_int8_tile256_mi16_loop(ctx, tile256, name):
+    """Bit-exact against the oracle, and the same bits from the 32 x 32 x 32 loop."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    say("mfma_b8 256x256 kernel, 16x16x64 loop, %s" % name)
+    p = MI16_CASES[name]()
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    assert_bit_exact(got, p.run_oracle(), name)
+    _capi.lib().qmm_set_b8x_variant(0)
+    try:
+        other = p.run_gpu(eng, strm, weights_any=True)
+    finally:
+        _capi.lib().qmm_set_b8x_variant(1)
+    assert_bit_exact(other, got, name + " (32x32x32 loop)")
+
+
+def test_mfma_int8_large_u8_source_prepass_mi16(ctx):
+    eng, strm = ctx
+    say("mfma_b8 u8 source 4096x384x3072, 16x16x64 loop")
+    p = int8_linear(4096, 384, 3072, 116, src_zp=121)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    assert_bit_exact(got, p.run_oracle(), "u8 prepass, K 384")
+
+
 def test_mfma_int8_large_u8_source_prepass(ctx):
     """192 tiles of 256 x 256 with a u8 source: rewritten as s8 by a pre-pass into the
     scratchpad, then the 256 x 256 kernel with the +128 * colsum correction."""
