@@ -689,7 +689,11 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QY_ROW(3, CB, , , , ) QY_ROW(4, CB, , , , ) QY_ROW(5, CB, , , , ) \
     QY_ROW(6, CB, , , , ) QY_ROW(7, CB, , , , )
 
-#if defined(QMM_B8X_PART) && QMM_B8X_PART == 4
+#if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5)
+// ODD: an odd number of k-steps (the register buffers alternate per k-step, so
+// the two parities end on different buffers; one instantiation each keeps the
+// tail single and the accumulators out of scratch)
+template <bool ODD>
 __global__ void __launch_bounds__(b8x::NT, 1)
 gemm_b8y_kernel(const gemm_params_t p) {
     using namespace b8x;
@@ -717,7 +721,7 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int bz = blockIdx.y;
 
-    const int KT = p.K / BK; // host guarantees K % 128 == 0 and KT >= 6
+    const int KT = p.K / BK; // host guarantees K % 64 == 0, KT >= 5 and KT % 2 == ODD
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(lds_u8 *)lds);
 
@@ -805,14 +809,24 @@ gemm_b8y_kernel(const gemm_params_t p) {
         QX_SB(); \
         BODY \
     }
-    for (int kt = 1; kt <= KT - 5; kt += 2) {
+    // requesting steps kt = 1 .. KT-4, in pairs; an odd KT leaves one more
+    constexpr int PAIRED_END = ODD ? 6 : 5;
+    for (int kt = 1; kt <= KT - PAIRED_END; kt += 2) {
         QY_KSTEP(16, QY_STEP_D(0, 1) QX_ADV_A(); QX_ADV_B();)
         QY_KSTEP(16, QY_STEP_D(1, 0) QX_ADV_A(); QX_ADV_B();)
     }
-    QY_KSTEP(16, QY_STEP_ND(0, 1)) // kt = KT-3
-    QY_KSTEP(8, QY_STEP_ND(1, 0)) // kt = KT-2
-    QY_KSTEP(0, QY_STEP_ND(0, 1)) // kt = KT-1
-    QY_LAST(1)
+    if constexpr (ODD) {
+        QY_KSTEP(16, QY_STEP_D(0, 1)) // kt = KT-4: requests tile KT-1
+        QY_KSTEP(16, QY_STEP_ND(1, 0)) // kt = KT-3
+        QY_KSTEP(8, QY_STEP_ND(0, 1)) // kt = KT-2
+        QY_KSTEP(0, QY_STEP_ND(1, 0)) // kt = KT-1
+        QY_LAST(0)
+    } else {
+        QY_KSTEP(16, QY_STEP_ND(0, 1)) // kt = KT-3
+        QY_KSTEP(8, QY_STEP_ND(1, 0)) // kt = KT-2
+        QY_KSTEP(0, QY_STEP_ND(0, 1)) // kt = KT-1
+        QY_LAST(1)
+    }
     __syncthreads();
 
     tile_epilogue<false, false>(
@@ -1058,11 +1072,16 @@ void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream) {
 }
 #elif QMM_B8X_PART == 4
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_b8y_kernel, p, stream);
+    launch_b8x(gemm_b8y_kernel<false>, p, stream);
+}
+#elif QMM_B8X_PART == 5
+void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_b8y_kernel<true>, p, stream);
 }
 #endif
 #else
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream);
+void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream);
@@ -1084,8 +1103,7 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
-// 0: the 32 x 32 x 32 loop, 1: the 16 x 16 x 64 loop (an even number of
-// k-steps, at least 6)
+// 0: the 32 x 32 x 32 loop, 1: the 16 x 16 x 64 loop (at least 5 k-steps)
 static int g_b8x_variant = 1;
 void set_gemm_b8x_variant(int v) {
     g_b8x_variant = v;
@@ -1096,8 +1114,12 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
         launch_b8x_fp8(p, stream);
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
-    else if (g_b8x_variant == 1 && p.K % 128 == 0 && p.K >= 6 * 64)
-        launch_b8x_int8_mi16(p, stream);
+    else if (g_b8x_variant == 1 && p.K >= 5 * 64) {
+        if ((p.K / 64) & 1)
+            launch_b8x_int8_mi16_odd(p, stream);
+        else
+            launch_b8x_int8_mi16(p, stream);
+    }
     else
         launch_b8x_int8(p, stream);
 }

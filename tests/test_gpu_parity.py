@@ -420,7 +420,12 @@ def test_mfma_int8_tile256_kernel(ctx, tile256, name):
 
 
 MI16_CASES = {
-    # K a multiple of 128 with at least 6 k-steps takes the loop on v_mfma_i32_16x16x64_i8
+    # at least 5 k-steps of 64 take the loop on v_mfma_i32_16x16x64_i8 (one instantiation per parity of the count)
+    "k320_odd_min_f32": lambda: int8_linear(260, 320, 300, 117, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None),
+    "k448_odd_edges_per_token_bf16": lambda: int8_linear(300, 448, 502, 118, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None,
+                                                         per_token=True),
+    "k704_odd_batched_s32": lambda: int8_linear(256, 704, 256, 119, src_dt=dt.s8, dst_dt=dt.s32, src_zp=2, src_scale=None,
+                                                batch=(2,)),
     "k384_edges_f32": lambda: int8_linear(300, 384, 502, 111, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None),
     "k640_edges_zp_bias_s32": lambda: int8_linear(260, 640, 250, 112, src_dt=dt.s8, dst_dt=dt.s32, src_zp=3,
                                                   src_scale=None, bias_dt=dt.s32),
