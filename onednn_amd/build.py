@@ -42,8 +42,8 @@ for v in GEMM_VARIANTS:
         UNITS.append(("qmm_gemm_b8.hip", "_v%d_k%d" % (v, k),
                       ["-DQMM_GEMM_VARIANT=%d" % v, "-DQMM_GEMM_KIND=%d" % k]))
 # likewise the 256 x 256 kernels: int8, short-K int8, fp8, int8 on 16 x 16 MFMAs
-# (even and odd numbers of k-steps)
-for v in (1, 2, 3, 4, 5):
+# (even and odd numbers of k-steps), fp8 on 16 x 16 MFMAs
+for v in (1, 2, 3, 4, 5, 6):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
 for v in (1, 2, 3, 4):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))

@@ -847,6 +847,7 @@ gemm_b8y_kernel(const gemm_params_t p) {
 // both operands.
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 #define QF_MF(i, j, cb) \
     { \
@@ -1029,6 +1030,290 @@ gemm_f8x_kernel(const gemm_params_t p) {
 
 #endif // fp8 kernel
 
+// ---- fp8 on 16 x 16 x 128 MFMAs (opt-in: qmm_set_b8x_variant(2)) -------------
+// v_mfma_f32_16x16x128_f8f6f4 contracts 128 k per instruction, i.e. two stages
+// of the ring: a k-step is 128 k, 64 MFMAs of 32 cycles, and the ring holds two
+// k-steps. Lane l of an operand holds row (column) l % 16 and 32 bytes of k:
+// lane group g = l / 16 takes, from stage g / 2 of the pair, the 16-byte chunks
+// g % 2 and g % 2 + 2 of the row -- two ds_read_b128 per fragment, measured free
+// of bank conflicts with the 16-row swizzle; the B chunks of the packed tile that
+// hold the same k are one 256-byte run per lane group.
+// The fragments of a k-step are single-buffered (8 + 8 fragments of 8 registers)
+// and the MFMAs walk the 8 x 8 fragment grid in growing squares, so that
+// fragment n of either operand is first needed at MFMA n * n: fragments 4..7 are
+// read during the first quarter of their own k-step, fragments 0..3 of the next
+// k-step right after this k-step's barrier, into a second register set.
+// One barrier per k-step, after MFMA 40: every wave has read what it needs from
+// this k-step's pair of stages, which then receives the k-step after next (16
+// direct loads per wave), and the next pair has landed for everyone.
+// Measured (8192^3, MI355X): correct, and it holds 1.96-1.99 GHz where the
+// 32 x 32 x 64 loop holds 1.5-1.7 GHz, but it needs about 18 % more cycles
+// (800-850 k against 690-720 k per launch; the same on all-zero operands,
+// whatever the placement of reads, requests and barriers), so the two run
+// equally fast (2.3 PFLOP/s) and the 32 x 32 x 64 loop stays the default.
+#define QZ_S(i, PS) ((i) < 4 ? (PS) : 0)
+// The MFMA is inline assembly with the accumulator constrained to an AGPR:
+// with the builtin, the register allocator kept part of the accumulators in
+// VGPRs on some paths and moved them at every loop seam (60 v_accvgpr_read per
+// two k-steps, each waiting for its MFMA). Operand waits are still the
+// compiler's (it sees the loads that feed the "v" operands); the accumulator of
+// one MFMA is next touched 64 MFMAs later.
+#define QZ_MF(i, j, PS) \
+    { \
+        QX_SB(); \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" \
+                     : "+a"(acc[i][j]) \
+                     : "v"(fa[QZ_S(i, PS)][i]), "v"(fb[QZ_S(j, PS)][j])); \
+        QX_SB(); \
+    }
+#define QZ_RA(S, i, base) \
+    { \
+        const v4i lo_ = *(const v4i *)((base) + a_lo + (i)*1024); \
+        const v4i hi_ = *(const v4i *)((base) + a_hi + (i)*1024); \
+        fa[S][i] = __builtin_shufflevector(lo_, hi_, 0, 1, 2, 3, 4, 5, 6, 7); \
+        QX_SB(); \
+    }
+#define QZ_RB(S, j, base) \
+    { \
+        const v4i lo_ = *(const v4i *)((base) + b_lo + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        const v4i hi_ = *(const v4i *)((base) + b_lo + 1024 + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        fb[S][j] = __builtin_shufflevector(lo_, hi_, 0, 1, 2, 3, 4, 5, 6, 7); \
+        QX_SB(); \
+    }
+// DMA(x): x when this k-step requests the one after next, PRE(x): x when a
+// next k-step exists; QZ_BAR_A / QZ_BAR_B as described above
+#define QZ_STEP_BODY(PS, NS, DMA, PRE, QZ_BAR_A, QZ_BAR_B) \
+    QZ_MF(0, 0, PS); QZ_RA(0, 4, ldsc); \
+    QZ_MF(0, 1, PS); \
+    QZ_MF(1, 1, PS); QZ_RB(0, 4, ldsc); \
+    QZ_MF(1, 0, PS); \
+    QZ_MF(0, 2, PS); QZ_RA(0, 5, ldsc); \
+    QZ_MF(1, 2, PS); \
+    QZ_MF(2, 2, PS); QZ_RB(0, 5, ldsc); \
+    QZ_MF(2, 1, PS); \
+    QZ_MF(2, 0, PS); QZ_RA(0, 6, ldsc); \
+    QZ_MF(0, 3, PS); \
+    QZ_MF(1, 3, PS); QZ_RB(0, 6, ldsc); \
+    QZ_MF(2, 3, PS); \
+    QZ_MF(3, 3, PS); QZ_RA(0, 7, ldsc); \
+    QZ_MF(3, 2, PS); \
+    QZ_MF(3, 1, PS); QZ_RB(0, 7, ldsc); \
+    QZ_MF(3, 0, PS); \
+    QZ_MF(0, 4, PS); \
+    QZ_MF(1, 4, PS); \
+    QZ_MF(2, 4, PS); \
+    QZ_MF(3, 4, PS); \
+    QZ_MF(4, 4, PS); \
+    QZ_MF(4, 3, PS); \
+    QZ_MF(4, 2, PS); \
+    QZ_MF(4, 1, PS); \
+    QZ_MF(4, 0, PS); \
+    QZ_MF(0, 5, PS); \
+    QZ_MF(1, 5, PS); \
+    QZ_MF(2, 5, PS); \
+    QZ_MF(3, 5, PS); \
+    QZ_MF(4, 5, PS); \
+    QZ_MF(5, 5, PS); \
+    QZ_MF(5, 4, PS); \
+    QZ_MF(5, 3, PS); \
+    QZ_MF(5, 2, PS); \
+    QZ_MF(5, 1, PS); \
+    QZ_MF(5, 0, PS); \
+    QZ_MF(0, 6, PS); \
+    QZ_MF(1, 6, PS); \
+    QZ_MF(2, 6, PS); \
+    QZ_MF(3, 6, PS); \
+    QZ_MF(4, 6, PS); QZ_BAR_A; QZ_BAR_B; \
+    QZ_MF(5, 6, PS); PRE(QZ_RA(NS, 0, ldsn)); \
+    QZ_MF(6, 6, PS); PRE(QZ_RB(NS, 0, ldsn)); \
+    QZ_MF(6, 5, PS); PRE(QZ_RA(NS, 1, ldsn)); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(6, 4, PS); PRE(QZ_RB(NS, 1, ldsn)); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(6, 3, PS); PRE(QZ_RA(NS, 2, ldsn)); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(6, 2, PS); PRE(QZ_RB(NS, 2, ldsn)); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(6, 1, PS); PRE(QZ_RA(NS, 3, ldsn)); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(6, 0, PS); PRE(QZ_RB(NS, 3, ldsn)); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(0, 7, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(1, 7, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(2, 7, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(3, 7, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(4, 7, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(5, 7, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(6, 7, PS); DMA(QX_D2(b_vo, sb, dB)); \
+    QZ_MF(7, 7, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(7, 6, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(7, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(7, 4, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(7, 3, PS); DMA(QX_D2(b_vo, sb, dB)); \
+    QZ_MF(7, 2, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(7, 1, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(7, 0, PS);
+// advance to the next 64-k tile, staying on the last one once it is reached
+#define QZ_ADV_A() \
+    { \
+        const int go = adv_a > 0; \
+        sa += go ? BK : 0; \
+        adv_a -= go; \
+        dA = ((dA - lds_base + STAGE_BYTES) & (RING - 1)) + lds_base; \
+    }
+#define QZ_ADV_B() \
+    { \
+        const int go = adv_b > 0; \
+        sb += go ? 2048 : 0; \
+        adv_b -= go; \
+        dB = ((dB - lds_base + STAGE_BYTES) & (RING - 1)) + lds_base; \
+    }
+#define QZ_ON(x) x
+#define QZ_OFF(x)
+#define QZ_BARRIER_A \
+    { \
+        QX_WL(0); \
+        __builtin_amdgcn_s_barrier(); \
+        QX_SB(); \
+    }
+#define QZ_BARRIER_B(WAITV) \
+    { \
+        QX_WV(WAITV); \
+        __builtin_amdgcn_s_barrier(); \
+        QX_SB(); \
+    }
+#define QZ_NONE \
+    { }
+
+#if defined(QMM_B8X_PART) && QMM_B8X_PART == 6
+__global__ void __launch_bounds__(b8x::NT, 1)
+gemm_f8y_kernel(const gemm_params_t p) {
+    using namespace b8x;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        lt = xcd * per + slot;
+        if (slot >= per || lt >= ntiles) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const int KS = p.K / 128; // host guarantees K % 256 == 0 and KS >= 4
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+
+    uint32_t a_vo[4], b_vo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tid + j * NT;
+        const int row = c >> 2, cp = c & 3;
+        const int gm = min(m0 + row, p.M - 1) - m0;
+        a_vo[j] = (uint32_t)gm * (uint32_t)p.lda + a_swz16(row, cp) * 16;
+        const int nbl = c >> 7, rem = c & 127;
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1) - n0 / 32;
+        b_vo[j] = (uint32_t)nb * (uint32_t)p.kb32 * 1024u + rem * 16;
+    }
+    auto sgpr_ptr = [](const uint8_t *q) {
+        const uint64_t v = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi
+                = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+    };
+    const uint8_t *sa = sgpr_ptr(
+            p.A + (int64_t)bz * p.a_sb + (int64_t)m0 * p.lda);
+    const uint8_t *sb = sgpr_ptr(p.B + (int64_t)bz * p.b_sb
+            + (int64_t)(n0 / 32) * p.kb32 * 1024);
+    uint32_t dA = lds_base + wave * 1024;
+    uint32_t dB = dA + A_BYTES;
+    // tile advances left after the four of the prologue
+    int adv_a = p.K / BK - 5, adv_b = p.K / BK - 5;
+
+    // fragment offsets inside a pair of stages
+    const int g = lane >> 4;
+    const int arow = wm0 + (lane & 15);
+    const int a_lo = (g >> 1) * STAGE_BYTES + arow * BK
+            + a_swz16(arow, g & 1) * 16;
+    const int a_hi = (g >> 1) * STAGE_BYTES + arow * BK
+            + a_swz16(arow, (g & 1) + 2) * 16;
+    const int b_lo = (g >> 1) * STAGE_BYTES + A_BYTES + (wn0 >> 5) * 2048
+            + (g & 1) * 512 + (lane & 15) * 16;
+    const uint8_t *const pair0 = lds, *const pair1 = lds + 2 * STAGE_BYTES;
+
+    v4f acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                acc[i][j][r] = 0.f;
+    v8i fa[2][8], fb[2][8]; // [set][fragment]; set 1 only for fragments 0..3
+
+    {
+        float s = 1.f;
+        if (p.ep.src_scale.ptr)
+            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
+                    bz * p.ep.src_scale.sb
+                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
+        ((float *)(lds + SS_OFF))[tid] = s;
+    }
+
+    // ---- prologue: k-steps 0 and 1 requested (the whole ring); the first
+    // fragments of k-step 0 read ----
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QX_ADV_A();
+    QX_FETCH(b_vo, sb, dB); QX_ADV_B();
+    QX_WV(16);
+    __syncthreads();
+    QX_SB();
+    QZ_RA(0, 0, pair0); QZ_RB(0, 0, pair0); QZ_RA(0, 1, pair0);
+    QZ_RB(0, 1, pair0); QZ_RA(0, 2, pair0); QZ_RB(0, 2, pair0);
+    QZ_RA(0, 3, pair0); QZ_RB(0, 3, pair0);
+
+    // k-step t works on pair t % 2 with fragment set t % 2 for fragments 0..2
+#define QZ_STEP_FULL(PS, NS, CUR, NXT) \
+    { \
+        const uint8_t *const ldsc = CUR, *const ldsn = NXT; \
+        QZ_STEP_BODY(PS, NS, QZ_ON, QZ_ON, QX_WL(0), QZ_BARRIER_B(0)) \
+    }
+    // One code path for every k-step, so that each accumulator keeps its
+    // register from the first MFMA to the epilogue (at the seam between a loop
+    // and separate tail copies the register allocator permutes them, and it
+    // cannot know that the inline-assembly MFMAs are still writing): the last
+    // two k-steps request again what the ring already holds -- the source
+    // pointers stop advancing at the last tile -- into stages nobody reads any
+    // more, and read "next" fragments that are never used.
+    for (int t = 0; t < KS; t += 2) {
+        QZ_STEP_FULL(0, 1, pair0, pair1)
+        QZ_STEP_FULL(1, 0, pair1, pair0)
+    }
+    // the last MFMAs are still writing (16 passes), and the surplus requests
+    // must have landed before the ring is reused as staging
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    QX_WV(0);
+    __syncthreads();
+
+    tile_epilogue<true, true>(
+            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+}
+#endif // fp8, 16 x 16 x 128
+
+
 template <typename K>
 static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
     using namespace b8x;
@@ -1078,8 +1363,13 @@ void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_b8y_kernel<true>, p, stream);
 }
+#elif QMM_B8X_PART == 6
+void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream) {
+    launch_b8x(gemm_f8y_kernel, p, stream);
+}
 #endif
 #else
+void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
@@ -1103,18 +1393,23 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
-// 0: the 32 x 32 x 32 loop, 1: the 16 x 16 x 64 loop (at least 5 k-steps)
+// int8: 0: the 32 x 32 x 32 loop, 1 or 2: the 16 x 16 x 64 loop (at least 5
+// k-steps). fp8: 2: the 16 x 16 x 128 loop (K a multiple of 256, at least 512),
+// which is correct but, as measured, no faster than the 32 x 32 x 64 loop: it
+// holds a higher clock for about 18 % more cycles.
 static int g_b8x_variant = 1;
 void set_gemm_b8x_variant(int v) {
     g_b8x_variant = v;
 }
 
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
-    if (f8)
+    if (f8 && g_b8x_variant == 2 && p.K % 256 == 0 && p.K >= 4 * 128)
+        launch_b8x_fp8_mi16(p, stream);
+    else if (f8)
         launch_b8x_fp8(p, stream);
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
-    else if (g_b8x_variant == 1 && p.K >= 5 * 64) {
+    else if (g_b8x_variant >= 1 && p.K >= 5 * 64) {
         if ((p.K / 64) & 1)
             launch_b8x_int8_mi16_odd(p, stream);
         else
