@@ -1042,15 +1042,18 @@ gemm_f8x_kernel(const gemm_params_t p) {
 // and the MFMAs walk the 8 x 8 fragment grid in growing squares, so that
 // fragment n of either operand is first needed at MFMA n * n: fragments 4..7 are
 // read during the first quarter of their own k-step, fragments 0..3 of the next
-// k-step right after this k-step's barrier, into a second register set.
-// One barrier per k-step, after MFMA 40: every wave has read what it needs from
+// k-step during the last quarter of this one, into a second register set; one
+// memory instruction per MFMA slot throughout.
+// Two barriers per k-step: after MFMA 17 every wave has read what it needs from
 // this k-step's pair of stages, which then receives the k-step after next (16
-// direct loads per wave), and the next pair has landed for everyone.
+// direct loads per wave); after MFMA 45 the next pair has landed for everyone
+// and its first fragments are read.
 // Measured (8192^3, MI355X): correct, and it holds 1.96-1.99 GHz where the
 // 32 x 32 x 64 loop holds 1.5-1.7 GHz, but it needs about 18 % more cycles
-// (800-850 k against 690-720 k per launch; the same on all-zero operands,
-// whatever the placement of reads, requests and barriers), so the two run
-// equally fast (2.3 PFLOP/s) and the 32 x 32 x 64 loop stays the default.
+// (800-850 k against 690-720 k per launch; on all-zero operands 0.59 us
+// against 0.52 us per 64 k, whatever the placement of reads, requests and
+// barriers), so the two run equally fast (2.3 PFLOP/s) and the 32 x 32 x 64
+// loop stays the default.
 #define QZ_S(i, PS) ((i) < 4 ? (PS) : 0)
 // The MFMA is inline assembly with the accumulator constrained to an AGPR:
 // with the builtin, the register allocator kept part of the accumulators in
@@ -1063,89 +1066,102 @@ gemm_f8x_kernel(const gemm_params_t p) {
         QX_SB(); \
         asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" \
                      : "+a"(acc[i][j]) \
-                     : "v"(fa[QZ_S(i, PS)][i]), "v"(fb[QZ_S(j, PS)][j])); \
+                     : "v"(__builtin_shufflevector(fal[QZ_S(i, PS)][i], \
+                               fah[QZ_S(i, PS)][i], 0, 1, 2, 3, 4, 5, 6, 7)), \
+                     "v"(__builtin_shufflevector(fbl[QZ_S(j, PS)][j], \
+                             fbh[QZ_S(j, PS)][j], 0, 1, 2, 3, 4, 5, 6, 7))); \
         QX_SB(); \
     }
-#define QZ_RA(S, i, base) \
+// one ds_read_b128 each: with 32-cycle MFMAs a single memory instruction
+// between two MFMAs is hidden, two are not
+#define QZ_RA_LO(S, i, base) \
     { \
-        const v4i lo_ = *(const v4i *)((base) + a_lo + (i)*1024); \
-        const v4i hi_ = *(const v4i *)((base) + a_hi + (i)*1024); \
-        fa[S][i] = __builtin_shufflevector(lo_, hi_, 0, 1, 2, 3, 4, 5, 6, 7); \
+        fal[S][i] = *(const v4i *)((base) + a_lo + (i)*1024); \
         QX_SB(); \
     }
-#define QZ_RB(S, j, base) \
+#define QZ_RA_HI(S, i, base) \
     { \
-        const v4i lo_ = *(const v4i *)((base) + b_lo + ((j) >> 1) * 2048 + ((j)&1) * 256); \
-        const v4i hi_ = *(const v4i *)((base) + b_lo + 1024 + ((j) >> 1) * 2048 + ((j)&1) * 256); \
-        fb[S][j] = __builtin_shufflevector(lo_, hi_, 0, 1, 2, 3, 4, 5, 6, 7); \
+        fah[S][i] = *(const v4i *)((base) + a_hi + (i)*1024); \
         QX_SB(); \
     }
+#define QZ_RB_LO(S, j, base) \
+    { \
+        fbl[S][j] = *(const v4i *)((base) + b_lo + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        QX_SB(); \
+    }
+#define QZ_RB_HI(S, j, base) \
+    { \
+        fbh[S][j] = *(const v4i *)((base) + b_lo + 1024 + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        QX_SB(); \
+    }
+#define QZ_RA(S, i, base) QZ_RA_LO(S, i, base) QZ_RA_HI(S, i, base)
+#define QZ_RB(S, j, base) QZ_RB_LO(S, j, base) QZ_RB_HI(S, j, base)
 // DMA(x): x when this k-step requests the one after next, PRE(x): x when a
 // next k-step exists; QZ_BAR_A / QZ_BAR_B as described above
 #define QZ_STEP_BODY(PS, NS, DMA, PRE, QZ_BAR_A, QZ_BAR_B) \
-    QZ_MF(0, 0, PS); QZ_RA(0, 4, ldsc); \
-    QZ_MF(0, 1, PS); \
-    QZ_MF(1, 1, PS); QZ_RB(0, 4, ldsc); \
-    QZ_MF(1, 0, PS); \
-    QZ_MF(0, 2, PS); QZ_RA(0, 5, ldsc); \
-    QZ_MF(1, 2, PS); \
-    QZ_MF(2, 2, PS); QZ_RB(0, 5, ldsc); \
-    QZ_MF(2, 1, PS); \
-    QZ_MF(2, 0, PS); QZ_RA(0, 6, ldsc); \
-    QZ_MF(0, 3, PS); \
-    QZ_MF(1, 3, PS); QZ_RB(0, 6, ldsc); \
-    QZ_MF(2, 3, PS); \
-    QZ_MF(3, 3, PS); QZ_RA(0, 7, ldsc); \
-    QZ_MF(3, 2, PS); \
-    QZ_MF(3, 1, PS); QZ_RB(0, 7, ldsc); \
-    QZ_MF(3, 0, PS); \
+    QZ_MF(0, 0, PS); QZ_RA_LO(0, 4, ldsc); \
+    QZ_MF(0, 1, PS); QZ_RA_HI(0, 4, ldsc); \
+    QZ_MF(1, 1, PS); QZ_RB_LO(0, 4, ldsc); \
+    QZ_MF(1, 0, PS); QZ_RB_HI(0, 4, ldsc); \
+    QZ_MF(0, 2, PS); QZ_RA_LO(0, 5, ldsc); \
+    QZ_MF(1, 2, PS); QZ_RA_HI(0, 5, ldsc); \
+    QZ_MF(2, 2, PS); QZ_RB_LO(0, 5, ldsc); \
+    QZ_MF(2, 1, PS); QZ_RB_HI(0, 5, ldsc); \
+    QZ_MF(2, 0, PS); QZ_RA_LO(0, 6, ldsc); \
+    QZ_MF(0, 3, PS); QZ_RA_HI(0, 6, ldsc); \
+    QZ_MF(1, 3, PS); QZ_RB_LO(0, 6, ldsc); \
+    QZ_MF(2, 3, PS); QZ_RB_HI(0, 6, ldsc); \
+    QZ_MF(3, 3, PS); QZ_RA_LO(0, 7, ldsc); \
+    QZ_MF(3, 2, PS); QZ_RA_HI(0, 7, ldsc); \
+    QZ_MF(3, 1, PS); QZ_RB_LO(0, 7, ldsc); \
+    QZ_MF(3, 0, PS); QZ_RB_HI(0, 7, ldsc); \
     QZ_MF(0, 4, PS); \
-    QZ_MF(1, 4, PS); \
-    QZ_MF(2, 4, PS); \
-    QZ_MF(3, 4, PS); \
-    QZ_MF(4, 4, PS); \
-    QZ_MF(4, 3, PS); \
-    QZ_MF(4, 2, PS); \
-    QZ_MF(4, 1, PS); \
-    QZ_MF(4, 0, PS); \
-    QZ_MF(0, 5, PS); \
-    QZ_MF(1, 5, PS); \
-    QZ_MF(2, 5, PS); \
-    QZ_MF(3, 5, PS); \
-    QZ_MF(4, 5, PS); \
-    QZ_MF(5, 5, PS); \
-    QZ_MF(5, 4, PS); \
-    QZ_MF(5, 3, PS); \
-    QZ_MF(5, 2, PS); \
-    QZ_MF(5, 1, PS); \
-    QZ_MF(5, 0, PS); \
-    QZ_MF(0, 6, PS); \
-    QZ_MF(1, 6, PS); \
+    QZ_MF(1, 4, PS); QZ_BAR_A; \
+    QZ_MF(2, 4, PS); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(3, 4, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(4, 4, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(4, 3, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(4, 2, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(4, 1, PS); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(4, 0, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(0, 5, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(1, 5, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(2, 5, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(3, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(4, 5, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(5, 5, PS); DMA(QX_D2(b_vo, sb, dB)); \
+    QZ_MF(5, 4, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(5, 3, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(5, 2, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(5, 1, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(5, 0, PS); DMA(QX_D2(b_vo, sb, dB)); \
+    QZ_MF(0, 6, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(1, 6, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
     QZ_MF(2, 6, PS); \
     QZ_MF(3, 6, PS); \
-    QZ_MF(4, 6, PS); QZ_BAR_A; QZ_BAR_B; \
-    QZ_MF(5, 6, PS); PRE(QZ_RA(NS, 0, ldsn)); \
-    QZ_MF(6, 6, PS); PRE(QZ_RB(NS, 0, ldsn)); \
-    QZ_MF(6, 5, PS); PRE(QZ_RA(NS, 1, ldsn)); DMA(QX_D0(a_vo, sa, dA)); \
-    QZ_MF(6, 4, PS); PRE(QZ_RB(NS, 1, ldsn)); DMA(QX_D1(a_vo, sa, dA)); \
-    QZ_MF(6, 3, PS); PRE(QZ_RA(NS, 2, ldsn)); DMA(QX_D2(a_vo, sa, dA)); \
-    QZ_MF(6, 2, PS); PRE(QZ_RB(NS, 2, ldsn)); DMA(QX_D3(a_vo, sa, dA)); \
-    QZ_MF(6, 1, PS); PRE(QZ_RA(NS, 3, ldsn)); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
-    QZ_MF(6, 0, PS); PRE(QZ_RB(NS, 3, ldsn)); DMA(QX_D0(a_vo, sa, dA)); \
-    QZ_MF(0, 7, PS); DMA(QX_D1(a_vo, sa, dA)); \
-    QZ_MF(1, 7, PS); DMA(QX_D2(a_vo, sa, dA)); \
-    QZ_MF(2, 7, PS); DMA(QX_D3(a_vo, sa, dA)); \
-    QZ_MF(3, 7, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
-    QZ_MF(4, 7, PS); DMA(QX_D0(b_vo, sb, dB)); \
-    QZ_MF(5, 7, PS); DMA(QX_D1(b_vo, sb, dB)); \
-    QZ_MF(6, 7, PS); DMA(QX_D2(b_vo, sb, dB)); \
-    QZ_MF(7, 7, PS); DMA(QX_D3(b_vo, sb, dB)); \
-    QZ_MF(7, 6, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
-    QZ_MF(7, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
-    QZ_MF(7, 4, PS); DMA(QX_D1(b_vo, sb, dB)); \
-    QZ_MF(7, 3, PS); DMA(QX_D2(b_vo, sb, dB)); \
-    QZ_MF(7, 2, PS); DMA(QX_D3(b_vo, sb, dB)); \
-    QZ_MF(7, 1, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(4, 6, PS); \
+    QZ_MF(5, 6, PS); \
+    QZ_MF(6, 6, PS); \
+    QZ_MF(6, 5, PS); \
+    QZ_MF(6, 4, PS); \
+    QZ_MF(6, 3, PS); QZ_BAR_B; \
+    QZ_MF(6, 2, PS); PRE(QZ_RA_LO(NS, 0, ldsn)); \
+    QZ_MF(6, 1, PS); PRE(QZ_RA_HI(NS, 0, ldsn)); \
+    QZ_MF(6, 0, PS); PRE(QZ_RB_LO(NS, 0, ldsn)); \
+    QZ_MF(0, 7, PS); PRE(QZ_RB_HI(NS, 0, ldsn)); \
+    QZ_MF(1, 7, PS); PRE(QZ_RA_LO(NS, 1, ldsn)); \
+    QZ_MF(2, 7, PS); PRE(QZ_RA_HI(NS, 1, ldsn)); \
+    QZ_MF(3, 7, PS); PRE(QZ_RB_LO(NS, 1, ldsn)); \
+    QZ_MF(4, 7, PS); PRE(QZ_RB_HI(NS, 1, ldsn)); \
+    QZ_MF(5, 7, PS); PRE(QZ_RA_LO(NS, 2, ldsn)); \
+    QZ_MF(6, 7, PS); PRE(QZ_RA_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 7, PS); PRE(QZ_RB_LO(NS, 2, ldsn)); \
+    QZ_MF(7, 6, PS); PRE(QZ_RB_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 5, PS); PRE(QZ_RA_LO(NS, 3, ldsn)); \
+    QZ_MF(7, 4, PS); PRE(QZ_RA_HI(NS, 3, ldsn)); \
+    QZ_MF(7, 3, PS); PRE(QZ_RB_LO(NS, 3, ldsn)); \
+    QZ_MF(7, 2, PS); PRE(QZ_RB_HI(NS, 3, ldsn)); \
+    QZ_MF(7, 1, PS); \
     QZ_MF(7, 0, PS);
 // advance to the next 64-k tile, staying on the last one once it is reached
 #define QZ_ADV_A() \
@@ -1257,7 +1273,9 @@ gemm_f8y_kernel(const gemm_params_t p) {
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 acc[i][j][r] = 0.f;
-    v8i fa[2][8], fb[2][8]; // [set][fragment]; set 1 only for fragments 0..3
+    // [set][fragment], low and high 16 bytes of each lane's 32; set 1 only for
+    // fragments 0..3
+    v4i fal[2][8], fah[2][8], fbl[2][8], fbh[2][8];
 
     {
         float s = 1.f;
@@ -1289,7 +1307,7 @@ gemm_f8y_kernel(const gemm_params_t p) {
 #define QZ_STEP_FULL(PS, NS, CUR, NXT) \
     { \
         const uint8_t *const ldsc = CUR, *const ldsn = NXT; \
-        QZ_STEP_BODY(PS, NS, QZ_ON, QZ_ON, QX_WL(0), QZ_BARRIER_B(0)) \
+        QZ_STEP_BODY(PS, NS, QZ_ON, QZ_ON, QZ_BARRIER_A, QZ_BARRIER_B(16)) \
     }
     // One code path for every k-step, so that each accumulator keeps its
     // register from the first MFMA to the epilogue (at the seam between a loop
