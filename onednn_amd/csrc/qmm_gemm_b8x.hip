@@ -1180,9 +1180,10 @@ gemm_f8x_kernel(const gemm_params_t p) {
     }
 #define QZ_ON(x) x
 #define QZ_OFF(x)
+// every wave has issued its reads of this pair of stages: the requests that
+// follow land hundreds of cycles later, LDS serves a wave's reads in order
 #define QZ_BARRIER_A \
     { \
-        QX_WL(0); \
         __builtin_amdgcn_s_barrier(); \
         QX_SB(); \
     }
