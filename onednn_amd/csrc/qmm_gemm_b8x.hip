@@ -669,15 +669,18 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QY_MF(i, 0, CB); X0; QY_MF(i, 1, CB); QY_MF(i, 2, CB); X1; \
     QY_MF(i, 3, CB); QY_MF(i, 4, CB); X2; QY_MF(i, 5, CB); \
     QY_MF(i, 6, CB); X3; QY_MF(i, 7, CB);
+// the 16 fragment reads and the direct loads (with their M0 writes) are spread
+// evenly over the 64 MFMAs: requests issued in a cluster run into the rate the
+// L2 -> LDS path accepts them at
 #define QY_STEP(CB, NB, DA0, DA1, DA2, DA3, DA4, DB0, DB1, DB2, DB3, DB4) \
-    QY_ROW(0, CB, QY_RA(NB, 0), QY_RB(NB, 0), QY_RB(NB, 1), QY_RB(NB, 2)) \
-    QY_ROW(1, CB, QY_RB(NB, 3), QY_RB(NB, 4), QY_RB(NB, 5), QY_RB(NB, 6)) \
-    QY_ROW(2, CB, QY_RB(NB, 7), QY_RA(NB, 1), DA0, DA1) \
-    QY_ROW(3, CB, QY_RA(NB, 2), DA2, DA3, DA4) \
-    QY_ROW(4, CB, QY_RA(NB, 3), QY_RA(NB, 4), DB0, DB1) \
-    QY_ROW(5, CB, QY_RA(NB, 5), DB2, DB3, DB4) \
-    QY_ROW(6, CB, QY_RA(NB, 6), QY_RA(NB, 7), , ) \
-    QY_ROW(7, CB, , , , )
+    QY_ROW(0, CB, QY_RA(NB, 0), QY_RB(NB, 0), DA0, QY_RB(NB, 1)) \
+    QY_ROW(1, CB, QY_RB(NB, 2), DA1, QY_RB(NB, 3), QY_RB(NB, 4)) \
+    QY_ROW(2, CB, DA2, QY_RB(NB, 5), QY_RB(NB, 6), DA3) \
+    QY_ROW(3, CB, QY_RB(NB, 7), QY_RA(NB, 1), DA4, QY_RA(NB, 2)) \
+    QY_ROW(4, CB, QY_RA(NB, 3), DB0, QY_RA(NB, 4), QY_RA(NB, 5)) \
+    QY_ROW(5, CB, DB1, QY_RA(NB, 6), QY_RA(NB, 7), DB2) \
+    QY_ROW(6, CB, , , DB3, ) \
+    QY_ROW(7, CB, , DB4, , )
 #define QY_STEP_D(CB, NB) \
     QY_STEP(CB, NB, QX_D0(a_vo, sa, dA), QX_D1(a_vo, sa, dA), \
             QX_D2(a_vo, sa, dA), QX_D3(a_vo, sa, dA), QX_D4(a_vo, sa, dA), \
@@ -872,20 +875,25 @@ typedef float v4f __attribute__((ext_vector_type(4)));
     }
 // one k-step: 16 MFMAs on buffer CB, the next tile's fragments into buffer NB
 // (order a0 b0 b1 b2 b3 a1 a2 a3, both halves each); D*: direct loads or empty
+// one fragment read after every MFMA; the direct loads (with their M0 writes)
+// spread evenly over the k-step
 #define QF_STEP(CB, NB, DA0, DA1, DA2, DA3, DA4, DB0, DB1, DB2, DB3, DB4) \
-    QF_MF(0, 0, CB); QF_RA(NB, 0, 0); QF_RA(NB, 1, 0); \
-    QF_MF(0, 1, CB); QF_RB(NB, 0, 0); QF_RB(NB, 1, 0); \
-    QF_MF(0, 2, CB); QF_RB(NB, 0, 1); QF_RB(NB, 1, 1); \
-    QF_MF(0, 3, CB); QF_RB(NB, 0, 2); QF_RB(NB, 1, 2); \
-    DA0; QF_MF(1, 0, CB); DA1; QF_RB(NB, 0, 3); \
-    QF_MF(1, 1, CB); DA2; QF_RB(NB, 1, 3); \
-    QF_MF(1, 2, CB); DA3; QF_RA(NB, 0, 1); \
-    QF_MF(1, 3, CB); DA4; QF_RA(NB, 1, 1); \
-    DB0; QF_MF(2, 0, CB); DB1; QF_RA(NB, 0, 2); \
-    QF_MF(2, 1, CB); DB2; QF_RA(NB, 1, 2); \
-    QF_MF(2, 2, CB); DB3; QF_RA(NB, 0, 3); \
-    QF_MF(2, 3, CB); DB4; QF_RA(NB, 1, 3); \
-    QF_MF(3, 0, CB); QF_MF(3, 1, CB); QF_MF(3, 2, CB); QF_MF(3, 3, CB);
+    QF_MF(0, 0, CB); QF_RA(NB, 0, 0); \
+    QF_MF(0, 1, CB); QF_RA(NB, 1, 0); DA0; \
+    QF_MF(0, 2, CB); QF_RB(NB, 0, 0); DA1; \
+    QF_MF(0, 3, CB); QF_RB(NB, 1, 0); \
+    QF_MF(1, 0, CB); QF_RB(NB, 0, 1); DA2; \
+    QF_MF(1, 1, CB); QF_RB(NB, 1, 1); DA3; \
+    QF_MF(1, 2, CB); QF_RB(NB, 0, 2); \
+    QF_MF(1, 3, CB); QF_RB(NB, 1, 2); DA4; \
+    QF_MF(2, 0, CB); QF_RB(NB, 0, 3); DB0; \
+    QF_MF(2, 1, CB); QF_RB(NB, 1, 3); \
+    QF_MF(2, 2, CB); QF_RA(NB, 0, 1); DB1; \
+    QF_MF(2, 3, CB); QF_RA(NB, 1, 1); DB2; \
+    QF_MF(3, 0, CB); QF_RA(NB, 0, 2); \
+    QF_MF(3, 1, CB); QF_RA(NB, 1, 2); DB3; \
+    QF_MF(3, 2, CB); QF_RA(NB, 0, 3); DB4; \
+    QF_MF(3, 3, CB); QF_RA(NB, 1, 3);
 #define QF_STEP_D(CB, NB) \
     QF_STEP(CB, NB, QX_D0(a_vo, sa, dA), QX_D1(a_vo, sa, dA), \
             QX_D2(a_vo, sa, dA), QX_D3(a_vo, sa, dA), QX_D4(a_vo, sa, dA), \
@@ -1030,7 +1038,7 @@ gemm_f8x_kernel(const gemm_params_t p) {
 
 #endif // fp8 kernel
 
-// ---- fp8 on 16 x 16 x 128 MFMAs (opt-in: qmm_set_b8x_variant(2)) -------------
+// ---- fp8 on 16 x 16 x 128 MFMAs -------------------------------------------------
 // v_mfma_f32_16x16x128_f8f6f4 contracts 128 k per instruction, i.e. two stages
 // of the ring: a k-step is 128 k, 64 MFMAs of 32 cycles, and the ring holds two
 // k-steps. Lane l of an operand holds row (column) l % 16 and 32 bytes of k:
@@ -1048,12 +1056,12 @@ gemm_f8x_kernel(const gemm_params_t p) {
 // this k-step's pair of stages, which then receives the k-step after next (16
 // direct loads per wave); after MFMA 45 the next pair has landed for everyone
 // and its first fragments are read.
-// Measured (8192^3, MI355X): correct, and it holds 1.96-1.99 GHz where the
-// 32 x 32 x 64 loop holds 1.5-1.7 GHz, but it needs about 18 % more cycles
-// (800-850 k against 690-720 k per launch; on all-zero operands 0.59 us
-// against 0.52 us per 64 k, whatever the placement of reads, requests and
-// barriers), so the two run equally fast (2.3 PFLOP/s) and the 32 x 32 x 64
-// loop stays the default.
+// The 16 direct loads of a k-step are spread over MFMAs 9..47, one every other
+// MFMA: issued back to back (20 consecutive slots) they cost 18 % of the
+// kernel's cycles, wherever in the k-step the cluster sat -- the L2 -> LDS path
+// takes requests at a limited rate, and the stream has to be even.
+// Measured (8192^3, MI355X): 2.50-2.59 PFLOP/s against 2.38-2.46 for the
+// 32 x 32 x 64 loop in the same session, at 1.96-1.99 GHz against 1.5-1.7 GHz.
 #define QZ_S(i, PS) ((i) < 4 ? (PS) : 0)
 // The MFMA is inline assembly with the accumulator constrained to an AGPR:
 // with the builtin, the register allocator kept part of the accumulators in
@@ -1099,70 +1107,70 @@ gemm_f8x_kernel(const gemm_params_t p) {
 // DMA(x): x when this k-step requests the one after next, PRE(x): x when a
 // next k-step exists; QZ_BAR_A / QZ_BAR_B as described above
 #define QZ_STEP_BODY(PS, NS, DMA, PRE, QZ_BAR_A, QZ_BAR_B) \
-    QZ_MF(0, 0, PS); QZ_RA_LO(0, 4, ldsc); \
-    QZ_MF(0, 1, PS); QZ_RA_HI(0, 4, ldsc); \
-    QZ_MF(1, 1, PS); QZ_RB_LO(0, 4, ldsc); \
-    QZ_MF(1, 0, PS); QZ_RB_HI(0, 4, ldsc); \
-    QZ_MF(0, 2, PS); QZ_RA_LO(0, 5, ldsc); \
-    QZ_MF(1, 2, PS); QZ_RA_HI(0, 5, ldsc); \
-    QZ_MF(2, 2, PS); QZ_RB_LO(0, 5, ldsc); \
-    QZ_MF(2, 1, PS); QZ_RB_HI(0, 5, ldsc); \
-    QZ_MF(2, 0, PS); QZ_RA_LO(0, 6, ldsc); \
-    QZ_MF(0, 3, PS); QZ_RA_HI(0, 6, ldsc); \
-    QZ_MF(1, 3, PS); QZ_RB_LO(0, 6, ldsc); \
-    QZ_MF(2, 3, PS); QZ_RB_HI(0, 6, ldsc); \
-    QZ_MF(3, 3, PS); QZ_RA_LO(0, 7, ldsc); \
-    QZ_MF(3, 2, PS); QZ_RA_HI(0, 7, ldsc); \
-    QZ_MF(3, 1, PS); QZ_RB_LO(0, 7, ldsc); \
-    QZ_MF(3, 0, PS); QZ_RB_HI(0, 7, ldsc); \
+    QZ_MF(0, 0, PS); QZ_RA_LO(0, 4, ldsc); QZ_RA_HI(0, 4, ldsc); \
+    QZ_MF(0, 1, PS); QZ_RB_LO(0, 4, ldsc); QZ_RB_HI(0, 4, ldsc); \
+    QZ_MF(1, 1, PS); QZ_RA_LO(0, 5, ldsc); QZ_RA_HI(0, 5, ldsc); \
+    QZ_MF(1, 0, PS); QZ_RB_LO(0, 5, ldsc); QZ_RB_HI(0, 5, ldsc); \
+    QZ_MF(0, 2, PS); QZ_RA_LO(0, 6, ldsc); QZ_RA_HI(0, 6, ldsc); \
+    QZ_MF(1, 2, PS); QZ_RB_LO(0, 6, ldsc); QZ_RB_HI(0, 6, ldsc); \
+    QZ_MF(2, 2, PS); QZ_RA_LO(0, 7, ldsc); QZ_RA_HI(0, 7, ldsc); \
+    QZ_MF(2, 1, PS); QZ_RB_LO(0, 7, ldsc); QZ_RB_HI(0, 7, ldsc); \
+    QZ_MF(2, 0, PS); QZ_BAR_A; \
+    QZ_MF(0, 3, PS); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(1, 3, PS); \
+    QZ_MF(2, 3, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(3, 3, PS); \
+    QZ_MF(3, 2, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(3, 1, PS); \
+    QZ_MF(3, 0, PS); DMA(QX_D3(a_vo, sa, dA)); \
     QZ_MF(0, 4, PS); \
-    QZ_MF(1, 4, PS); QZ_BAR_A; \
-    QZ_MF(2, 4, PS); DMA(QX_D0(a_vo, sa, dA)); \
-    QZ_MF(3, 4, PS); DMA(QX_D1(a_vo, sa, dA)); \
-    QZ_MF(4, 4, PS); DMA(QX_D2(a_vo, sa, dA)); \
-    QZ_MF(4, 3, PS); DMA(QX_D3(a_vo, sa, dA)); \
-    QZ_MF(4, 2, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
-    QZ_MF(4, 1, PS); DMA(QX_D0(a_vo, sa, dA)); \
-    QZ_MF(4, 0, PS); DMA(QX_D1(a_vo, sa, dA)); \
-    QZ_MF(0, 5, PS); DMA(QX_D2(a_vo, sa, dA)); \
-    QZ_MF(1, 5, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(1, 4, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(2, 4, PS); \
+    QZ_MF(3, 4, PS); DMA(QX_D0(a_vo, sa, dA)); \
+    QZ_MF(4, 4, PS); \
+    QZ_MF(4, 3, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(4, 2, PS); \
+    QZ_MF(4, 1, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(4, 0, PS); \
+    QZ_MF(0, 5, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(1, 5, PS); \
     QZ_MF(2, 5, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
-    QZ_MF(3, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
-    QZ_MF(4, 5, PS); DMA(QX_D1(b_vo, sb, dB)); \
-    QZ_MF(5, 5, PS); DMA(QX_D2(b_vo, sb, dB)); \
-    QZ_MF(5, 4, PS); DMA(QX_D3(b_vo, sb, dB)); \
-    QZ_MF(5, 3, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
-    QZ_MF(5, 2, PS); DMA(QX_D0(b_vo, sb, dB)); \
-    QZ_MF(5, 1, PS); DMA(QX_D1(b_vo, sb, dB)); \
-    QZ_MF(5, 0, PS); DMA(QX_D2(b_vo, sb, dB)); \
-    QZ_MF(0, 6, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(3, 5, PS); \
+    QZ_MF(4, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(5, 5, PS); \
+    QZ_MF(5, 4, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(5, 3, PS); \
+    QZ_MF(5, 2, PS); DMA(QX_D2(b_vo, sb, dB)); \
+    QZ_MF(5, 1, PS); \
+    QZ_MF(5, 0, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(0, 6, PS); \
     QZ_MF(1, 6, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
     QZ_MF(2, 6, PS); \
-    QZ_MF(3, 6, PS); \
+    QZ_MF(3, 6, PS); DMA(QX_D0(b_vo, sb, dB)); \
     QZ_MF(4, 6, PS); \
-    QZ_MF(5, 6, PS); \
+    QZ_MF(5, 6, PS); DMA(QX_D1(b_vo, sb, dB)); \
     QZ_MF(6, 6, PS); \
-    QZ_MF(6, 5, PS); \
+    QZ_MF(6, 5, PS); DMA(QX_D2(b_vo, sb, dB)); \
     QZ_MF(6, 4, PS); \
-    QZ_MF(6, 3, PS); QZ_BAR_B; \
-    QZ_MF(6, 2, PS); PRE(QZ_RA_LO(NS, 0, ldsn)); \
-    QZ_MF(6, 1, PS); PRE(QZ_RA_HI(NS, 0, ldsn)); \
-    QZ_MF(6, 0, PS); PRE(QZ_RB_LO(NS, 0, ldsn)); \
-    QZ_MF(0, 7, PS); PRE(QZ_RB_HI(NS, 0, ldsn)); \
-    QZ_MF(1, 7, PS); PRE(QZ_RA_LO(NS, 1, ldsn)); \
-    QZ_MF(2, 7, PS); PRE(QZ_RA_HI(NS, 1, ldsn)); \
-    QZ_MF(3, 7, PS); PRE(QZ_RB_LO(NS, 1, ldsn)); \
-    QZ_MF(4, 7, PS); PRE(QZ_RB_HI(NS, 1, ldsn)); \
-    QZ_MF(5, 7, PS); PRE(QZ_RA_LO(NS, 2, ldsn)); \
-    QZ_MF(6, 7, PS); PRE(QZ_RA_HI(NS, 2, ldsn)); \
-    QZ_MF(7, 7, PS); PRE(QZ_RB_LO(NS, 2, ldsn)); \
-    QZ_MF(7, 6, PS); PRE(QZ_RB_HI(NS, 2, ldsn)); \
-    QZ_MF(7, 5, PS); PRE(QZ_RA_LO(NS, 3, ldsn)); \
-    QZ_MF(7, 4, PS); PRE(QZ_RA_HI(NS, 3, ldsn)); \
-    QZ_MF(7, 3, PS); PRE(QZ_RB_LO(NS, 3, ldsn)); \
-    QZ_MF(7, 2, PS); PRE(QZ_RB_HI(NS, 3, ldsn)); \
-    QZ_MF(7, 1, PS); \
-    QZ_MF(7, 0, PS);
+    QZ_MF(6, 3, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(6, 2, PS); \
+    QZ_MF(6, 1, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(6, 0, PS); \
+    QZ_MF(0, 7, PS); QZ_BAR_B; \
+    QZ_MF(1, 7, PS); PRE(QZ_RA_LO(NS, 0, ldsn)); PRE(QZ_RA_HI(NS, 0, ldsn)); \
+    QZ_MF(2, 7, PS); PRE(QZ_RB_LO(NS, 0, ldsn)); PRE(QZ_RB_HI(NS, 0, ldsn)); \
+    QZ_MF(3, 7, PS); PRE(QZ_RA_LO(NS, 1, ldsn)); \
+    QZ_MF(4, 7, PS); PRE(QZ_RA_HI(NS, 1, ldsn)); \
+    QZ_MF(5, 7, PS); PRE(QZ_RB_LO(NS, 1, ldsn)); \
+    QZ_MF(6, 7, PS); PRE(QZ_RB_HI(NS, 1, ldsn)); \
+    QZ_MF(7, 7, PS); PRE(QZ_RA_LO(NS, 2, ldsn)); \
+    QZ_MF(7, 6, PS); PRE(QZ_RA_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 5, PS); PRE(QZ_RB_LO(NS, 2, ldsn)); \
+    QZ_MF(7, 4, PS); PRE(QZ_RB_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 3, PS); PRE(QZ_RA_LO(NS, 3, ldsn)); \
+    QZ_MF(7, 2, PS); PRE(QZ_RA_HI(NS, 3, ldsn)); \
+    QZ_MF(7, 1, PS); PRE(QZ_RB_LO(NS, 3, ldsn)); \
+    QZ_MF(7, 0, PS); PRE(QZ_RB_HI(NS, 3, ldsn));
 // advance to the next 64-k tile, staying on the last one once it is reached
 #define QZ_ADV_A() \
     { \
@@ -1412,17 +1420,15 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
-// int8: 0: the 32 x 32 x 32 loop, 1 or 2: the 16 x 16 x 64 loop (at least 5
-// k-steps). fp8: 2: the 16 x 16 x 128 loop (K a multiple of 256, at least 512),
-// which is correct but, as measured, no faster than the 32 x 32 x 64 loop: it
-// holds a higher clock for about 18 % more cycles.
+// 0: the loops on 32 x 32 MFMAs; 1: int8 on 16 x 16 x 64 (at least 5 k-steps)
+// and fp8 on 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply
 static int g_b8x_variant = 1;
 void set_gemm_b8x_variant(int v) {
     g_b8x_variant = v;
 }
 
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
-    if (f8 && g_b8x_variant == 2 && p.K % 256 == 0 && p.K >= 4 * 128)
+    if (f8 && g_b8x_variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)
         launch_b8x_fp8(p, stream);

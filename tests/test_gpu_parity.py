@@ -514,26 +514,29 @@ def test_mfma_fp8_tile256_kernel(ctx, tile256):
 
 
 def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
-    """The fp8 loop on v_mfma_f32_16x16x128_f8f6f4 (opt-in): same bar as the default loop."""
+    """The fp8 loop on v_mfma_f32_16x16x128_f8f6f4 (K a multiple of 256) and, on the same
+    problems, the 32 x 32 x 64 loop it replaced."""
     from onednn_amd import _capi
     eng, strm = ctx
-    _capi.lib().qmm_set_b8x_variant(2)
-    try:
-        for (M, K, N, dd, with_sum) in ((256, 512, 256, dt.bf16, True), (300, 768, 260, dt.f32, False),
-                                        (128, 1024, 512, dt.bf16, False), (512, 2048, 256, dt.f32, False)):
-            say("mfma_b8 256x256 fp8 kernel, 16x16x128 loop, %dx%dx%d" % (M, K, N))
-            p = fp8_gemm(M, K, N, 178, dst_dt=dd, with_sum=with_sum)
-            got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
-            assert pd.impl_info_str() == MFMA
-            want = p.run_oracle()
-            a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
-            if dd == dt.bf16:
-                assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
-            else:
-                assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
-                                 rel=1e-5, scale=a, what="fp8 f32")
-    finally:
-        _capi.lib().qmm_set_b8x_variant(1)
+    shapes = ((256, 512, 256, dt.bf16, True), (300, 768, 260, dt.f32, False),
+              (128, 1024, 512, dt.bf16, False), (512, 2048, 256, dt.f32, False))
+    for variant in (1, 0):
+        _capi.lib().qmm_set_b8x_variant(variant)
+        try:
+            for (M, K, N, dd, with_sum) in shapes:
+                say("mfma_b8 256x256 fp8 kernel, variant %d, %dx%dx%d" % (variant, M, K, N))
+                p = fp8_gemm(M, K, N, 178, dst_dt=dd, with_sum=with_sum)
+                got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+                assert pd.impl_info_str() == MFMA
+                want = p.run_oracle()
+                a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
+                if dd == dt.bf16:
+                    assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
+                else:
+                    assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
+                                     rel=1e-5, scale=a, what="fp8 f32")
+        finally:
+            _capi.lib().qmm_set_b8x_variant(1)
 
 
 def test_mfma_fp8_tile256_f16_dst_bias_relu(ctx, tile256):
