@@ -1056,8 +1056,9 @@ gemm_f8x_kernel(const gemm_params_t p) {
 // this k-step's pair of stages, which then receives the k-step after next (16
 // direct loads per wave); after MFMA 45 the next pair has landed for everyone
 // and its first fragments are read.
-// The 16 direct loads of a k-step are spread over MFMAs 9..47, one every other
-// MFMA: issued back to back (20 consecutive slots) they cost 18 % of the
+// The 16 direct loads of a k-step are spread over MFMAs 9..62, about one in
+// three (the second barrier's vmcnt counts the 12 issued before it): issued
+// back to back (20 consecutive slots) they cost 18 % of the
 // kernel's cycles, wherever in the k-step the cluster sat -- the L2 -> LDS path
 // takes requests at a limited rate, and the stream has to be even.
 // Measured (8192^3, MI355X): 2.50-2.59 PFLOP/s against 2.38-2.46 for the
@@ -1118,58 +1119,58 @@ gemm_f8x_kernel(const gemm_params_t p) {
     QZ_MF(2, 0, PS); QZ_BAR_A; \
     QZ_MF(0, 3, PS); DMA(QX_D0(a_vo, sa, dA)); \
     QZ_MF(1, 3, PS); \
-    QZ_MF(2, 3, PS); DMA(QX_D1(a_vo, sa, dA)); \
-    QZ_MF(3, 3, PS); \
-    QZ_MF(3, 2, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(2, 3, PS); \
+    QZ_MF(3, 3, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(3, 2, PS); \
     QZ_MF(3, 1, PS); \
-    QZ_MF(3, 0, PS); DMA(QX_D3(a_vo, sa, dA)); \
+    QZ_MF(3, 0, PS); DMA(QX_D2(a_vo, sa, dA)); \
     QZ_MF(0, 4, PS); \
-    QZ_MF(1, 4, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(1, 4, PS); DMA(QX_D3(a_vo, sa, dA)); \
     QZ_MF(2, 4, PS); \
-    QZ_MF(3, 4, PS); DMA(QX_D0(a_vo, sa, dA)); \
-    QZ_MF(4, 4, PS); \
-    QZ_MF(4, 3, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(3, 4, PS); \
+    QZ_MF(4, 4, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(4, 3, PS); \
     QZ_MF(4, 2, PS); \
-    QZ_MF(4, 1, PS); DMA(QX_D2(a_vo, sa, dA)); \
+    QZ_MF(4, 1, PS); DMA(QX_D0(a_vo, sa, dA)); \
     QZ_MF(4, 0, PS); \
-    QZ_MF(0, 5, PS); DMA(QX_D3(a_vo, sa, dA)); \
-    QZ_MF(1, 5, PS); \
-    QZ_MF(2, 5, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(0, 5, PS); \
+    QZ_MF(1, 5, PS); DMA(QX_D1(a_vo, sa, dA)); \
+    QZ_MF(2, 5, PS); \
     QZ_MF(3, 5, PS); \
-    QZ_MF(4, 5, PS); DMA(QX_D0(b_vo, sb, dB)); \
+    QZ_MF(4, 5, PS); DMA(QX_D2(a_vo, sa, dA)); \
     QZ_MF(5, 5, PS); \
-    QZ_MF(5, 4, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(5, 4, PS); DMA(QX_D3(a_vo, sa, dA)); \
     QZ_MF(5, 3, PS); \
-    QZ_MF(5, 2, PS); DMA(QX_D2(b_vo, sb, dB)); \
-    QZ_MF(5, 1, PS); \
-    QZ_MF(5, 0, PS); DMA(QX_D3(b_vo, sb, dB)); \
+    QZ_MF(5, 2, PS); \
+    QZ_MF(5, 1, PS); DMA(QX_D4(a_vo, sa, dA)); DMA(QZ_ADV_A()); \
+    QZ_MF(5, 0, PS); \
     QZ_MF(0, 6, PS); \
-    QZ_MF(1, 6, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
+    QZ_MF(1, 6, PS); DMA(QX_D0(b_vo, sb, dB)); \
     QZ_MF(2, 6, PS); \
-    QZ_MF(3, 6, PS); DMA(QX_D0(b_vo, sb, dB)); \
-    QZ_MF(4, 6, PS); \
-    QZ_MF(5, 6, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(3, 6, PS); \
+    QZ_MF(4, 6, PS); DMA(QX_D1(b_vo, sb, dB)); \
+    QZ_MF(5, 6, PS); \
     QZ_MF(6, 6, PS); \
     QZ_MF(6, 5, PS); DMA(QX_D2(b_vo, sb, dB)); \
     QZ_MF(6, 4, PS); \
     QZ_MF(6, 3, PS); DMA(QX_D3(b_vo, sb, dB)); \
     QZ_MF(6, 2, PS); \
-    QZ_MF(6, 1, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
-    QZ_MF(6, 0, PS); \
+    QZ_MF(6, 1, PS); \
+    QZ_MF(6, 0, PS); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
     QZ_MF(0, 7, PS); QZ_BAR_B; \
     QZ_MF(1, 7, PS); PRE(QZ_RA_LO(NS, 0, ldsn)); PRE(QZ_RA_HI(NS, 0, ldsn)); \
-    QZ_MF(2, 7, PS); PRE(QZ_RB_LO(NS, 0, ldsn)); PRE(QZ_RB_HI(NS, 0, ldsn)); \
+    QZ_MF(2, 7, PS); PRE(QZ_RB_LO(NS, 0, ldsn)); PRE(QZ_RB_HI(NS, 0, ldsn)); DMA(QX_D0(b_vo, sb, dB)); \
     QZ_MF(3, 7, PS); PRE(QZ_RA_LO(NS, 1, ldsn)); \
     QZ_MF(4, 7, PS); PRE(QZ_RA_HI(NS, 1, ldsn)); \
-    QZ_MF(5, 7, PS); PRE(QZ_RB_LO(NS, 1, ldsn)); \
+    QZ_MF(5, 7, PS); PRE(QZ_RB_LO(NS, 1, ldsn)); DMA(QX_D1(b_vo, sb, dB)); \
     QZ_MF(6, 7, PS); PRE(QZ_RB_HI(NS, 1, ldsn)); \
     QZ_MF(7, 7, PS); PRE(QZ_RA_LO(NS, 2, ldsn)); \
-    QZ_MF(7, 6, PS); PRE(QZ_RA_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 6, PS); PRE(QZ_RA_HI(NS, 2, ldsn)); DMA(QX_D2(b_vo, sb, dB)); \
     QZ_MF(7, 5, PS); PRE(QZ_RB_LO(NS, 2, ldsn)); \
-    QZ_MF(7, 4, PS); PRE(QZ_RB_HI(NS, 2, ldsn)); \
+    QZ_MF(7, 4, PS); PRE(QZ_RB_HI(NS, 2, ldsn)); DMA(QX_D3(b_vo, sb, dB)); \
     QZ_MF(7, 3, PS); PRE(QZ_RA_LO(NS, 3, ldsn)); \
     QZ_MF(7, 2, PS); PRE(QZ_RA_HI(NS, 3, ldsn)); \
-    QZ_MF(7, 1, PS); PRE(QZ_RB_LO(NS, 3, ldsn)); \
+    QZ_MF(7, 1, PS); PRE(QZ_RB_LO(NS, 3, ldsn)); DMA(QX_D4(b_vo, sb, dB)); DMA(QZ_ADV_B()); \
     QZ_MF(7, 0, PS); PRE(QZ_RB_HI(NS, 3, ldsn));
 // advance to the next 64-k tile, staying on the last one once it is reached
 #define QZ_ADV_A() \
@@ -1316,7 +1317,7 @@ gemm_f8y_kernel(const gemm_params_t p) {
 #define QZ_STEP_FULL(PS, NS, CUR, NXT) \
     { \
         const uint8_t *const ldsc = CUR, *const ldsn = NXT; \
-        QZ_STEP_BODY(PS, NS, QZ_ON, QZ_ON, QZ_BARRIER_A, QZ_BARRIER_B(16)) \
+        QZ_STEP_BODY(PS, NS, QZ_ON, QZ_ON, QZ_BARRIER_A, QZ_BARRIER_B(12)) \
     }
     // One code path for every k-step, so that each accumulator keeps its
     // register from the first MFMA to the epilogue (at the seam between a loop
