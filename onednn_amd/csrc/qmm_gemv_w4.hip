@@ -46,6 +46,14 @@ QMM_D v4f mfma16(const v4u &a, const v4u &b, const v4f &c) {
                 0, 0);
 }
 
+// lane i of every row of 16 lanes takes the value of lane i + S of that row
+// (zero past the row's end)
+template <int S>
+QMM_D uint32_t row_shl(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(
+            0, (int)v, 0x100 + S, 0xf, 0xf, true);
+}
+
 // weights are read exactly once: keep them from displacing reusable lines
 QMM_D uint4 ld_stream(const uint8_t *ptr) {
     const v4u v = __builtin_nontemporal_load((const v4u *)ptr);
@@ -57,7 +65,7 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
 // (out-of-range tiles re-read the last valid one, absent buffers are replaced
 // by the weights pointer), so the number of loads in flight is known at
 // compile time and no wait has to drain the whole queue.
-template <bool F16, bool FAST>
+template <bool F16, int FAST>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -181,11 +189,19 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 #pragma unroll
             for (int u = 0; u < UNR; u++) {
                 const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+                if constexpr (FAST == 2) {
+                    // a single activation row: lane (r, c) fetches what lane
+                    // (0, c) multiplies in step r % 4, one load per tile
+                    const int k = min(
+                            tc * 128 + (r & 3) * 32 + c * 8, p.K - 8);
+                    av[u][0] = *(const uint4 *)(p.A + (int64_t)m_base * p.lda + k);
+                } else {
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++) {
-                    // chunks past the row's end re-read its last one
-                    const int k = min(tc * 128 + s4 * 32 + c * 8, p.K - 8);
-                    av[u][s4] = *(const uint4 *)(Arow + k);
+                    for (int s4 = 0; s4 < 4; s4++) {
+                        // chunks past the row's end re-read its last one
+                        const int k = min(tc * 128 + s4 * 32 + c * 8, p.K - 8);
+                        av[u][s4] = *(const uint4 *)(Arow + k);
+                    }
                 }
                 const int gsc = p.gs_shift < 0 ? 0 : tc >> p.gs_shift;
                 scp[u] = scn[(int64_t)gsc * sN];
@@ -198,10 +214,15 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 #pragma unroll
                 for (int u = 0; u < UNR; u++) {
                     const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+                    if constexpr (FAST == 2) {
+                        if (tc * 128 + (r & 3) * 32 + c * 8 >= p.K)
+                            av[u][0] = make_uint4(0, 0, 0, 0);
+                    } else {
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; s4++)
-                        if (tc * 128 + s4 * 32 + c * 8 >= p.K)
-                            av[u][s4] = make_uint4(0, 0, 0, 0);
+                        for (int s4 = 0; s4 < 4; s4++)
+                            if (tc * 128 + s4 * 32 + c * 8 >= p.K)
+                                av[u][s4] = make_uint4(0, 0, 0, 0);
+                    }
                 }
             }
             // the four tiles are independent accumulation chains: a tile past
@@ -226,8 +247,27 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
                     b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
                     b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
                     b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
-                    const v4u a = {av[u][s4].x, av[u][s4].y, av[u][s4].z,
-                            av[u][s4].w};
+                    v4u a;
+                    if constexpr (FAST == 2) {
+                        // row 0 of the operand takes step s4's chunk from lane
+                        // (s4, c); the other rows hold other steps' chunks and
+                        // produce rows of the result that are never stored
+                        const uint4 v = av[u][0];
+                        if (s4 == 0)
+                            a = v4u {v.x, v.y, v.z, v.w};
+                        else if (s4 == 1)
+                            a = v4u {row_shl<1>(v.x), row_shl<1>(v.y),
+                                    row_shl<1>(v.z), row_shl<1>(v.w)};
+                        else if (s4 == 2)
+                            a = v4u {row_shl<2>(v.x), row_shl<2>(v.y),
+                                    row_shl<2>(v.z), row_shl<2>(v.w)};
+                        else
+                            a = v4u {row_shl<3>(v.x), row_shl<3>(v.y),
+                                    row_shl<3>(v.z), row_shl<3>(v.w)};
+                    } else {
+                        a = v4u {av[u][s4].x, av[u][s4].y, av[u][s4].z,
+                                av[u][s4].w};
+                    }
                     Pu[u] = mfma16<F16>(a, b, Pu[u]);
                     Su[u] = mfma16<F16>(a, ones, Su[u]);
                 }
@@ -440,8 +480,8 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
             && (p.gz > 0 ? shift_of(p.gz, q.gz_shift)
                          : ((q.gz_shift = -1), true));
     auto launch = [&](auto kern) {
-        // (the four kernels share this lambda's type: one call each)
-        static const void *done[4] = {};
+        // (the six kernels share this lambda's type: one call each)
+        static const void *done[6] = {};
         bool seen = false;
         for (const void *d : done)
             seen = seen || d == (const void *)kern;
@@ -459,16 +499,21 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
                 MR, KC);
     };
     if (fast) lds = red; // that variant keeps its activations in registers
+    // a single row: one activation load per tile instead of four (FAST == 2)
     if (p.act_f16) {
-        if (fast)
-            launch(gemv_w4_kernel<true, true>);
+        if (fast && p.M == 1)
+            launch(gemv_w4_kernel<true, 2>);
+        else if (fast)
+            launch(gemv_w4_kernel<true, 1>);
         else
-            launch(gemv_w4_kernel<true, false>);
+            launch(gemv_w4_kernel<true, 0>);
     } else {
-        if (fast)
-            launch(gemv_w4_kernel<false, true>);
+        if (fast && p.M == 1)
+            launch(gemv_w4_kernel<false, 2>);
+        else if (fast)
+            launch(gemv_w4_kernel<false, 1>);
         else
-            launch(gemv_w4_kernel<false, false>);
+            launch(gemv_w4_kernel<false, 0>);
     }
 }
 
