@@ -786,9 +786,51 @@ QMM_D void epilogue_flush_denormals() {
 enum : int { EP_DST_F32 = 0, EP_DST_BF16 = 1, EP_DST_F16 = 2,
     EP_DST_Q8 = 3 /* s8 or u8 */ };
 
-template <int FAST, int DSTK, bool EXT>
+// The post-ops that read a second tensor (binary operand, old dst of a sum)
+// fetch 8 or 16 bytes per lane and row. The loads cannot be left to the
+// compiler's scheduling: it has to assume that the dst store of one row
+// aliases the operand load of the next, which leaves one row's load in flight
+// at a time. ep_operand_load issues the load on its own, so that a caller can
+// request a batch of rows before the first store, and hands the result to
+// epilogue_full4<.., PRE = true>.
+template <int FAST>
+constexpr bool ep_reads_operand() {
+    return FAST == EP_FAST_ADD || FAST == EP_FAST_SUM || FAST == EP_FAST_BIN32
+            || FAST == EP_FAST_BIN16;
+}
+
+template <int FAST, int DSTK>
+QMM_D uint4 ep_operand_load(const epilogue_t &ep, const ep_cols_t &c,
+        int64_t bz, int64_t m, int64_t en) {
+    if constexpr (FAST == EP_FAST_ADD) {
+        return *(const uint4 *)((const float *)ep.po[0].t.ptr
+                + bz * ep.po[0].t.sb + m * ep.po[0].t.sm + en);
+    } else if constexpr (FAST == EP_FAST_BIN32) {
+        return *(const uint4 *)((const float *)c.bin_ptr + m * c.bin_sm);
+    } else if constexpr (FAST == EP_FAST_BIN16) {
+        const uint2 v
+                = *(const uint2 *)((const uint16_t *)c.bin_ptr + m * c.bin_sm);
+        return make_uint4(v.x, v.y, 0, 0);
+    } else if constexpr (FAST == EP_FAST_SUM) {
+        const int64_t dst_off = bz * ep.dst.sb + m * ep.dst.sm + en;
+        if constexpr (DSTK == EP_DST_F32) {
+            return *(const uint4 *)((const float *)ep.dst.ptr + dst_off);
+        } else {
+            const uint2 v
+                    = *(const uint2 *)((const uint16_t *)ep.dst.ptr + dst_off);
+            return make_uint4(v.x, v.y, 0, 0);
+        }
+    } else {
+        return make_uint4(0, 0, 0, 0);
+    }
+}
+
+template <int FAST, int DSTK, bool EXT, bool PRE = false>
 QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
-        float (&d)[4], float ss, int64_t bz, int64_t m, int64_t en) {
+        float (&d)[4], float ss, int64_t bz, int64_t m, int64_t en,
+        uint4 pre = make_uint4(0, 0, 0, 0)) {
+    if constexpr (!PRE && ep_reads_operand<FAST>())
+        pre = ep_operand_load<FAST, DSTK>(ep, c, bz, m, en);
     const float alpha = FAST == EP_FAST_RELU || FAST == EP_FAST_SWISH
             ? ep.po[0].alpha
             : 0.f;
@@ -815,12 +857,10 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
             d[i] = d[i] * __builtin_amdgcn_rcpf(1.0f + e);
         }
     } else if constexpr (FAST == EP_FAST_ADD) {
-        const float4 y = *(const float4 *)((const float *)ep.po[0].t.ptr
-                + bz * ep.po[0].t.sb + m * ep.po[0].t.sm + en);
-        d[0] += y.x;
-        d[1] += y.y;
-        d[2] += y.z;
-        d[3] += y.w;
+        d[0] += u2f(pre.x);
+        d[1] += u2f(pre.y);
+        d[2] += u2f(pre.z);
+        d[3] += u2f(pre.w);
     } else if constexpr (FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -829,17 +869,15 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
                            d[i], ep.po[0].alpha, ep.po[0].beta)
                     * ep.po[0].scale;
     } else if constexpr (FAST == EP_FAST_BIN32 || FAST == EP_FAST_BIN16) {
-        const int64_t off = m * c.bin_sm;
         const bool mul = c.bin_mul != 0;
         float y[4];
         if constexpr (FAST == EP_FAST_BIN32) {
-            const float4 v = *((const float4 *)((const float *)c.bin_ptr + off));
-            y[0] = v.x;
-            y[1] = v.y;
-            y[2] = v.z;
-            y[3] = v.w;
+            y[0] = u2f(pre.x);
+            y[1] = u2f(pre.y);
+            y[2] = u2f(pre.z);
+            y[3] = u2f(pre.w);
         } else {
-            const uint2 v = *((const uint2 *)((const uint16_t *)c.bin_ptr + off));
+            const uint2 v = make_uint2(pre.x, pre.y);
             const uint16_t h[4] = {(uint16_t)v.x, (uint16_t)(v.x >> 16),
                     (uint16_t)v.y, (uint16_t)(v.y >> 16)};
             const bool f16 = c.bin_f16 != 0;
@@ -857,15 +895,12 @@ QMM_D void epilogue_full4(const epilogue_t &ep, const ep_cols_t &c,
         static_assert(FAST != EP_FAST_SUM || DSTK <= EP_DST_F16, "");
         float o[4];
         if constexpr (DSTK == EP_DST_F32) {
-            const float4 v = *(const float4 *)((const float *)ep.dst.ptr
-                    + dst_off);
-            o[0] = v.x;
-            o[1] = v.y;
-            o[2] = v.z;
-            o[3] = v.w;
+            o[0] = u2f(pre.x);
+            o[1] = u2f(pre.y);
+            o[2] = u2f(pre.z);
+            o[3] = u2f(pre.w);
         } else {
-            const uint2 v = *(const uint2 *)((const uint16_t *)ep.dst.ptr
-                    + dst_off);
+            const uint2 v = make_uint2(pre.x, pre.y);
             if constexpr (DSTK == EP_DST_BF16) {
                 o[0] = u2f(v.x << 16);
                 o[1] = u2f(v.x & 0xFFFF0000u);

@@ -219,7 +219,10 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 // the matrix and the dst rows are vector-aligned: no per-lane conditions, so
 // the rows pipeline. FAST is the recognised epilogue shape, DSTK the dst type,
 // EXT whether bias / dst scale / dst zero point take part (epilogue_full4).
-template <int FAST, int DSTK, bool EXT, bool F8, int PITCH>
+// BATCHED: operands of the post-ops that read a second tensor are requested a
+// batch of rows ahead (the kernels with the LEAN epilogue only: the others'
+// register allocation does not survive it).
+template <int FAST, int DSTK, bool EXT, bool F8, int PITCH, bool BATCHED>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const ep_cols_t &cols,
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
@@ -228,6 +231,39 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
     constexpr int UNR = FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH
             ? 2
             : (FAST > EP_FAST_SUM || EXT ? 4 : 8);
+    if constexpr (BATCHED && ep_reads_operand<FAST>()) {
+        // a batch of rows' operands requested before the first of their stores
+        constexpr int BATCH = 16;
+#pragma unroll 1
+        for (int it0 = 0; it0 < 32; it0 += BATCH) {
+            uint4 pre[BATCH];
+#pragma unroll
+            for (int k = 0; k < BATCH; k++)
+                pre[k] = ep_operand_load<FAST, DSTK>(ep, cols, bz,
+                        m_first + (it0 + k) * 2 + (lane >> 5), en);
+#pragma unroll
+            for (int k = 0; k < BATCH; k++) {
+                const int row = (it0 + k) * 2 + (lane >> 5);
+                const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
+                const float ss = ssl[row];
+                float d[4];
+                if constexpr (F8) {
+                    d[0] = u2f((uint32_t)t.x);
+                    d[1] = u2f((uint32_t)t.y);
+                    d[2] = u2f((uint32_t)t.z);
+                    d[3] = u2f((uint32_t)t.w);
+                } else {
+                    d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
+                    d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
+                    d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
+                    d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+                }
+                epilogue_full4<FAST, DSTK, EXT, true>(
+                        ep, cols, d, ss, bz, m_first + row, en, pre[k]);
+            }
+        }
+        return;
+    }
 #pragma unroll UNR
     for (int it = 0; it < 32; it++) {
         const int row = it * 2 + (lane >> 5);
@@ -351,7 +387,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
 #define QX_EP_ROWS(F, D, X) \
-    ep_rows_full<F, D, X, F8, PITCH>( \
+    ep_rows_full<F, D, X, F8, PITCH, LEAN>( \
             ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en)
 #define QX_EP_DST(F) \
     switch (dstk) { \
