@@ -556,6 +556,29 @@ def test_mfma_fp8_tile256_f16_dst_bias_relu(ctx, tile256):
     assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-5 * a * 1024, what="fp8 f16")
 
 
+@pytest.mark.parametrize("dd", [dt.f32, dt.f16, dt.bf16])
+def test_mfma_fp8_tile256_sum_operand_batches(ctx, tile256, dd):
+    """The sum post-op of the fp8 kernels reads the old dst 16 rows ahead of its stores: every dst type it takes,
+    several row batches per wave tile (512 rows: two tile rows), with a scale other than one."""
+    eng, strm = ctx
+    M, K, N = 512, 768, 512
+    say("mfma_b8 256x256 fp8 kernel, sum post-op, dst %s" % dd)
+    p = fp8_gemm(M, K, N, 81, dst_dt=dd, with_sum=True)
+    p.post_ops = [{"kind": "sum", "scale": 0.75}]
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    want = p.run_oracle()
+    a = np.abs(p.src.logical().astype(np.float64)) @ np.abs(p.wei.logical().astype(np.float64)) * 0.125
+    if dd == dt.bf16:
+        assert_bf16_within_1ulp(got, want, "fp8 sum bf16", abs_slack=1e-5 * a)
+    elif dd == dt.f32:
+        assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
+                         rel=1e-5, scale=a, what="fp8 sum f32")
+    else:
+        g, w = O.to_f32(dt.f16, got).reshape(M, N), O.to_f32(dt.f16, want).reshape(M, N)
+        assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-5 * a * 1024, what="fp8 sum f16")
+
+
 def test_mfma_int8_tile256_binary_add_and_sum(ctx, tile256):
     eng, strm = ctx
     r = rnd(77)
