@@ -65,7 +65,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the path shards "
-              "along N without any exchange, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "along N with each GPU holding its own column slice and no exchange step); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     if args.calibrate_copy:
