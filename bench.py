@@ -50,8 +50,8 @@ EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c2", choices=["c2"])
     ap.add_argument("--variant", type=int, default=0, help="mfma_b8 tile configuration (0 = heuristic)")
     ap.add_argument("--no-extras", action="store_true", help="skip the decode / fp8 side measurements")

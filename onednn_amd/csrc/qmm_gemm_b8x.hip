@@ -219,9 +219,11 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 // the matrix and the dst rows are vector-aligned: no per-lane conditions, so
 // the rows pipeline. FAST is the recognised epilogue shape, DSTK the dst type,
 // EXT whether bias / dst scale / dst zero point take part (epilogue_full4).
-// BATCHED: operands of the post-ops that read a second tensor are requested a
-// batch of rows ahead (the kernels with the LEAN epilogue only: the others'
-// register allocation does not survive it).
+// Operands of the post-ops that read a second tensor are requested a batch of
+// rows ahead of the stores: 16 rows in the kernels with the LEAN epilogue
+// (BATCHED), 4 in the others, whose register allocation does not survive more
+// (with 8 the compiler spills 2 KB per lane and moves scalar operands of the
+// direct loads into vector registers).
 template <int FAST, int DSTK, bool EXT, bool F8, int PITCH, bool BATCHED>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const ep_cols_t &cols,
@@ -231,9 +233,9 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
     constexpr int UNR = FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH
             ? 2
             : (FAST > EP_FAST_SUM || EXT ? 4 : 8);
-    if constexpr (BATCHED && ep_reads_operand<FAST>()) {
+    if constexpr (ep_reads_operand<FAST>()) {
         // a batch of rows' operands requested before the first of their stores
-        constexpr int BATCH = 16;
+        constexpr int BATCH = BATCHED ? 16 : 4;
 #pragma unroll 1
         for (int it0 = 0; it0 < 32; it0 += BATCH) {
             uint4 pre[BATCH];
