@@ -72,7 +72,12 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     // lds: activations [KC/8 chunks][MR rows][16 bytes]; later reused for the
     // cross-wave reduction [GEMV_WAVES][64 lanes][4 floats]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nb = blockIdx.x;
+    // consecutive workgroups run on the 8 XCDs in turn: give each XCD a
+    // contiguous range of column blocks, so that a scale / zero-point line
+    // (64 and more neighbouring columns) is fetched into one L2 only
+    const int nb = (gridDim.x & 7) == 0
+            ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3))
+            : (int)blockIdx.x;
     const int m_base = p.m0 + blockIdx.y * 16;
     const int rows = min(16, p.M - m_base);
     const int c = lane >> 4; // k chunk of the lane
