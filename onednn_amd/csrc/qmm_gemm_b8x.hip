@@ -34,6 +34,11 @@
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
+// rows of a staged tile in flight in the straight-line epilogue
+#ifndef QMM_EP_UNR
+#define QMM_EP_UNR 8
+#endif
+
 namespace qmm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -53,7 +58,14 @@ constexpr int STG_WAVE = 64 * 128 * 4; // epilogue staging of one wave (in the r
 constexpr int STG_PITCH16 = 132;
 constexpr int STG_WAVE16 = 64 * STG_PITCH16 * 4;
 constexpr int SS_OFF = 4 * STG_WAVE16; // 256 per-row source scales (f32)
-constexpr int LDS_TOTAL = SS_OFF + 1024;
+// what the epilogue of the kernels on 16 x 16 MFMAs needs per column of the
+// block tile, staged before the main loop: weights scale (f32), source
+// zero-point compensation (s32), per-column bias (f32), dst zero point (f32)
+constexpr int WS_OFF = SS_OFF + 1024;
+constexpr int CS_OFF = WS_OFF + 1024;
+constexpr int BI_OFF = CS_OFF + 1024;
+constexpr int ZP_OFF = BI_OFF + 1024;
+constexpr int LDS_TOTAL = ZP_OFF + 1024;
 
 template <int N, typename F>
 QMM_D void static_for(F &&f) {
@@ -232,7 +244,20 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
     // rows in flight: fewer where a row is a long computation of its own
     constexpr int UNR = FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH
             ? 2
-            : (FAST > EP_FAST_SUM || EXT ? 4 : 8);
+            : (FAST > EP_FAST_SUM || EXT ? 4 : QMM_EP_UNR);
+    auto to_f32 = [&](const int4 &t, float (&d)[4]) {
+        if constexpr (F8) { // f32 accumulators, staged as bits
+            d[0] = u2f((uint32_t)t.x);
+            d[1] = u2f((uint32_t)t.y);
+            d[2] = u2f((uint32_t)t.z);
+            d[3] = u2f((uint32_t)t.w);
+        } else {
+            d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
+            d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
+            d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
+            d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
+        }
+    };
     if constexpr (ep_reads_operand<FAST>()) {
         // a batch of rows' operands requested before the first of their stores
         constexpr int BATCH = BATCHED ? 16 : 4;
@@ -249,17 +274,7 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
                 const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
                 const float ss = ssl[row];
                 float d[4];
-                if constexpr (F8) {
-                    d[0] = u2f((uint32_t)t.x);
-                    d[1] = u2f((uint32_t)t.y);
-                    d[2] = u2f((uint32_t)t.z);
-                    d[3] = u2f((uint32_t)t.w);
-                } else {
-                    d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
-                    d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
-                    d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
-                    d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
-                }
+                to_f32(t, d);
                 epilogue_full4<FAST, DSTK, EXT, true>(
                         ep, cols, d, ss, bz, m_first + row, en, pre[k]);
             }
@@ -271,44 +286,69 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const int row = it * 2 + (lane >> 5);
         const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
         const float ss = ssl[row];
-        const int64_t m = m_first + row;
         float d[4];
-        if constexpr (F8) { // f32 accumulators, staged as bits
-            d[0] = u2f((uint32_t)t.x);
-            d[1] = u2f((uint32_t)t.y);
-            d[2] = u2f((uint32_t)t.z);
-            d[3] = u2f((uint32_t)t.w);
-        } else {
-            d[0] = (float)(int32_t)((uint32_t)t.x + (uint32_t)cs4[0]);
-            d[1] = (float)(int32_t)((uint32_t)t.y + (uint32_t)cs4[1]);
-            d[2] = (float)(int32_t)((uint32_t)t.z + (uint32_t)cs4[2]);
-            d[3] = (float)(int32_t)((uint32_t)t.w + (uint32_t)cs4[3]);
-        }
-        epilogue_full4<FAST, DSTK, EXT>(ep, cols, d, ss, bz, m, en);
+        to_f32(t, d);
+        epilogue_full4<FAST, DSTK, EXT>(ep, cols, d, ss, bz, m_first + row, en);
     }
 }
 
-// Epilogue of one 256 x 256 block tile, shared by the int8 and fp8 kernels.
+// Column operands of the epilogue of one block tile, and its per-row source
+// scales, written to LDS by the first 256 threads before the main loop (the
+// loads' latency passes under the prologue): absent ones as 1.0 / 0, columns
+// past N likewise.
+QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
+        int m0, int n0, int bz) {
+    using namespace b8x;
+    const epilogue_t &ep = p.ep;
+    float ss = 1.f, ws = 1.f, bi = 0.f, zp = 0.f;
+    int cs = 0;
+    if (ep.src_scale.ptr)
+        ss = load_float(ep.src_scale.dt, ep.src_scale.ptr,
+                bz * ep.src_scale.sb
+                        + (int64_t)min(m0 + tid, p.M - 1) * ep.src_scale.sm);
+    const int n = n0 + tid;
+    if (n < p.N) {
+        if (ep.wei_scale.ptr) ws = ep_load(ep.wei_scale, bz, 0, n);
+        if (ep.bias.ptr && ep.bias.sm == 0) bi = ep_load(ep.bias, bz, 0, n);
+        if (ep.dst_zp) zp = (float)ep.dst_zp[ep.dst_zp_sn * n];
+        int comp = p.a_is_u8 ? 128 : 0;
+        if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+        if (comp != 0 && p.colsum)
+            cs = comp * p.colsum[(int64_t)bz * p.colsum_sb + n];
+    }
+    ((float *)(lds + SS_OFF))[tid] = ss;
+    ((float *)(lds + WS_OFF))[tid] = ws;
+    ((int *)(lds + CS_OFF))[tid] = cs;
+    ((float *)(lds + BI_OFF))[tid] = bi;
+    ((float *)(lds + ZP_OFF))[tid] = zp;
+}
+
+// Epilogue of one block tile, shared by the int8 and fp8 kernels.
 // LEAN: only the shapes up to EP_FAST_SUM with a float dst run straight-line
 // (fp8 and short-K launches; everything else they accept takes the row path)
-template <bool F8, bool LEAN, typename AccT, int NFRAG>
-QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
+// The accumulators are NFI x NFJ fragments per wave: 4 x 4 of 32 x 32, or
+// 8 x NFJ of 16 x 16 (a wave tile of 128 x 16 NFJ).
+template <bool F8, bool LEAN, typename AccT, int NFI, int NFJ>
+QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
         uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
         int wm0, int wn0, int bz) {
     using namespace b8x;
-    // NFRAG 4: 32 x 32 fragments (layout below); NFRAG 8: 16 x 16 fragments,
-    // register r of lane l is row 4*(l/16) + r, column l%16
-    constexpr bool MI16 = NFRAG == 8;
+    constexpr bool MI16 = NFI == 8;
+    constexpr int WN = MI16 ? 16 * NFJ : 128; // columns of the wave tile
     constexpr int PITCH = MI16 ? STG_PITCH16 : 128;
     constexpr int STGW = MI16 ? STG_WAVE16 : STG_WAVE;
-    // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
-    // column l%32 of its 32x32 fragment. The wave tile goes through LDS in two
-    // halves of 64 rows x 128 columns (the ring is free now, every wave takes a
-    // quarter of it), straight from the accumulator registers, and comes back
-    // row-wise, 4 neighbouring columns per lane, so that the arithmetic exists
-    // once per half and every store is a dense vector. A wave reads back only
-    // what it wrote itself: LDS executes a wave's instructions in order, no
-    // barrier is involved.
+    // 32 x 32 fragments: accumulator register r of lane l is row
+    // 8*(r/4) + 4*(l/32) + r%4, column l%32; written to LDS register by
+    // register. 16 x 16 fragments are computed transposed (the kernels pass the
+    // weights as the MFMA's first operand): register r of lane l is row l%16,
+    // column 4*(l/16) + r, so a lane's four registers are neighbouring columns
+    // of one row and go to LDS as one 16-byte write.
+    // The wave tile goes through LDS in two halves of 64 rows (the ring is
+    // free now, every wave takes a quarter of it), straight from the
+    // accumulator registers, and comes back row-wise, 4 neighbouring columns
+    // per lane, so that the arithmetic exists once per half and every store is
+    // a dense vector. A wave reads back only what it wrote itself: LDS
+    // executes a wave's instructions in order, no barrier is involved.
     const epilogue_t &ep = p.ep;
     // The row interpreter walks the post-op list with a run-time index: it
     // reads the parameter block where it lies (the kernel argument segment,
@@ -317,14 +357,15 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
     const epilogue_t &epk
             = ((const gemm_params_t *)__builtin_amdgcn_kernarg_segment_ptr())->ep;
     const uint32_t stg_w = lds_base + wave * STGW
-            + (MI16 ? 4 * (lane >> 4) * PITCH + (lane & 15)
+            + (MI16 ? (lane & 15) * PITCH + 4 * (lane >> 4)
                     : 4 * (lane >> 5) * 128 + (lane & 31))
                     * 4;
     const int *const stg_r = (const int *)lds + wave * (STGW / 4);
     const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
     const int ecol = (lane & 31) * 4;
+    const bool lane_on = ecol < WN; // lanes past a 112-column wave tile idle
     const int en = n0 + wn0 + ecol;
-    const int envalid = min(4, p.N - en);
+    const int envalid = lane_on ? min(4, p.N - en) : 0;
     const bool has_ss = ep.src_scale.ptr != nullptr;
     const bool has_ws = ep.wei_scale.ptr != nullptr;
     const bool to_bf16 = ep.dst.dt == dt_bf16;
@@ -336,10 +377,21 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
     // what depends on the lane's 4 columns only: weights scales, a per-column
     // bias, dst zero points, the zero-point compensation
     ep_cols_t cols;
-    epilogue_cols_load(ep, cols, bz, en, envalid > 0 ? envalid : 0);
-    float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     int cs4[4] = {0, 0, 0, 0};
-    {
+    if constexpr (MI16) {
+        // staged by tile_operands_stage()
+        epilogue_cols_load(ep, cols, bz, en, 0);
+        const int cw = lane_on ? wn0 + ecol : 0;
+        const float4 w4 = *(const float4 *)(lds + WS_OFF + cw * 4);
+        const int4 c4 = *(const int4 *)(lds + CS_OFF + cw * 4);
+        const float4 b4 = *(const float4 *)(lds + BI_OFF + cw * 4);
+        const float4 z4 = *(const float4 *)(lds + ZP_OFF + cw * 4);
+        cols.ws[0] = w4.x, cols.ws[1] = w4.y, cols.ws[2] = w4.z, cols.ws[3] = w4.w;
+        cols.bias[0] = b4.x, cols.bias[1] = b4.y, cols.bias[2] = b4.z, cols.bias[3] = b4.w;
+        cols.zp[0] = z4.x, cols.zp[1] = z4.y, cols.zp[2] = z4.z, cols.zp[3] = z4.w;
+        cs4[0] = c4.x, cs4[1] = c4.y, cs4[2] = c4.z, cs4[3] = c4.w;
+    } else {
+        epilogue_cols_load(ep, cols, bz, en, envalid > 0 ? envalid : 0);
         int comp = p.a_is_u8 ? 128 : 0;
         if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
 #pragma unroll
@@ -347,6 +399,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
             if (i < envalid && comp != 0 && p.colsum)
                 cs4[i] = comp * p.colsum[(int64_t)bz * p.colsum_sb + en + i];
     }
+    float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     // bf16 results: the reference conversion maps f32 subnormals to +-0
     // (src/common/bfloat16.cpp:22-56). With single-precision denormals flushed
     // for the rest of the wave's life, the last multiply of the chain (or the
@@ -355,7 +408,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
     if (to_bf16 && !ext && ep.fast != EP_FAST_NONE) epilogue_flush_denormals();
     // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
     // operand's rows) aligned for vector access
-    const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + 128 <= p.N
+    const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + WN <= p.N
             && ep.fast != EP_FAST_NONE && epilogue_full4_ok(ep)
             && (!LEAN || (ep.fast <= EP_FAST_SUM && dstk <= EP_DST_F16));
     static_for<2>([&](auto H) {
@@ -364,13 +417,11 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
 #pragma unroll
             for (int i2 = 0; i2 < 4; i2++)
 #pragma unroll
-                for (int j = 0; j < 8; j++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(stg_w),
-                                     "a"(acc[4 * h + i2][j][r]),
-                                     "n"(((i2 * 16 + r) * PITCH + j * 16) * 4)
-                                     : "memory");
+                for (int j = 0; j < NFJ; j++)
+                    asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(stg_w),
+                                 "a"(acc[4 * h + i2][j]),
+                                 "n"((i2 * 16 * PITCH + j * 16) * 4)
+                                 : "memory");
         } else {
 #pragma unroll
             for (int i2 = 0; i2 < 2; i2++)
@@ -389,8 +440,11 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFRAG][NFRAG],
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
 #define QX_EP_ROWS(F, D, X) \
-    ep_rows_full<F, D, X, F8, PITCH, LEAN>( \
-            ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en)
+    do { \
+        if (lane_on) \
+            ep_rows_full<F, D, X, F8, PITCH, LEAN>( \
+                    ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en); \
+    } while (0)
 #define QX_EP_DST(F) \
     switch (dstk) { \
         case EP_DST_F32: \
@@ -684,11 +738,15 @@ gemm_b8x_kernel(const gemm_params_t p) {
 // A k-step multiplies the fragments read during the previous k-step (64 MFMAs),
 // reads the next tile's 16 fragments into the other register buffer and
 // requests the tile two further on (8 direct loads), one barrier per k-step.
+// The weights fragment is the MFMA's first operand: the accumulator comes out
+// transposed (register r of lane l is row l % 16, column 4 * (l / 16) + r of
+// the fragment), four neighbouring columns of one row per lane, which is what
+// the epilogue stores.
 #define QY_MF(i, j, cb) \
     { \
         QX_SB(); \
         acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8( \
-                fa[cb][i], fb[cb][j], acc[i][j], 0, 0, 0); \
+                fb[cb][j], fa[cb][i], acc[i][j], 0, 0, 0); \
         QX_SB(); \
     }
 #define QY_RA(nb, i) \
@@ -733,17 +791,20 @@ gemm_b8x_kernel(const gemm_params_t p) {
 #if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5)
 // ODD: an odd number of k-steps (the register buffers alternate per k-step, so
 // the two parities end on different buffers; one instantiation each keeps the
-// tail single and the accumulators out of scratch)
+// tail single and the accumulators out of scratch). A 224-column block tile
+// (wave tiles of 128 x 112, four equal rounds of workgroups on a 4096 x 14336
+// dst instead of three and a half) was measured at 0.6 % and is not kept.
 template <bool ODD>
 __global__ void __launch_bounds__(b8x::NT, 1)
 gemm_b8y_kernel(const gemm_params_t p) {
     using namespace b8x;
+    constexpr int NFJ = 8, BNY = BN;
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * (16 * NFJ);
 
     const int ntiles = p.tiles_m * p.tiles_n;
     int lt;
@@ -759,7 +820,7 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int gsz = min(p.tiles_m - first_m, GROUP_M);
     const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
     const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * BNY;
     const int bz = blockIdx.y;
 
     const int KT = p.K / BK; // host guarantees K % 64 == 0, KT >= 5 and KT % 2 == ODD
@@ -798,24 +859,17 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int b_rel = A_BYTES + (wn0 >> 5) * 2048 + (g >> 1) * 1024
             + ((g & 1) * 32 + (lane & 15)) * 16;
 
-    v4i acc[8][8];
+    v4i acc[8][NFJ];
 #pragma unroll
     for (int i = 0; i < 8; i++)
 #pragma unroll
-        for (int j = 0; j < 8; j++)
+        for (int j = 0; j < NFJ; j++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
                 acc[i][j][r] = 0;
-    v4i fa[2][8], fb[2][8];
+    v4i fa[2][8], fb[2][NFJ];
 
-    {
-        float s = 1.f;
-        if (p.ep.src_scale.ptr)
-            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
-                    bz * p.ep.src_scale.sb
-                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
-        ((float *)(lds + SS_OFF))[tid] = s;
-    }
+    tile_operands_stage(p, lds, tid, m0, n0, bz);
 
     // ---- prologue: tiles 0..3 requested (the whole ring); tile 0's
     // fragments read ----
@@ -1102,7 +1156,8 @@ gemm_f8x_kernel(const gemm_params_t p) {
 // Measured (8192^3, MI355X): 2.50-2.59 PFLOP/s against 2.38-2.46 for the
 // 32 x 32 x 64 loop in the same session, at 1.96-1.99 GHz against 1.5-1.7 GHz.
 #define QZ_S(i, PS) ((i) < 4 ? (PS) : 0)
-// The MFMA is inline assembly with the accumulator constrained to an AGPR:
+// The weights fragment is the first operand (transposed accumulator, see
+// QY_MF). The MFMA is inline assembly with the accumulator constrained to an AGPR:
 // with the builtin, the register allocator kept part of the accumulators in
 // VGPRs on some paths and moved them at every loop seam (60 v_accvgpr_read per
 // two k-steps, each waiting for its MFMA). Operand waits are still the
@@ -1111,7 +1166,7 @@ gemm_f8x_kernel(const gemm_params_t p) {
 #define QZ_MF(i, j, PS) \
     { \
         QX_SB(); \
-        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %2, %1, %0" \
                      : "+a"(acc[i][j]) \
                      : "v"(__builtin_shufflevector(fal[QZ_S(i, PS)][i], \
                                fah[QZ_S(i, PS)][i], 0, 1, 2, 3, 4, 5, 6, 7)), \
@@ -1325,14 +1380,7 @@ gemm_f8y_kernel(const gemm_params_t p) {
     // fragments 0..3
     v4i fal[2][8], fah[2][8], fbl[2][8], fbh[2][8];
 
-    {
-        float s = 1.f;
-        if (p.ep.src_scale.ptr)
-            s = load_float(p.ep.src_scale.dt, p.ep.src_scale.ptr,
-                    bz * p.ep.src_scale.sb
-                            + (int64_t)min(m0 + tid, p.M - 1) * p.ep.src_scale.sm);
-        ((float *)(lds + SS_OFF))[tid] = s;
-    }
+    tile_operands_stage(p, lds, tid, m0, n0, bz);
 
     // ---- prologue: k-steps 0 and 1 requested (the whole ring); the first
     // fragments of k-step 0 read ----
@@ -1389,7 +1437,7 @@ static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ((ntiles + 7) / 8) * 8;
     // one attribute call per kernel (the kernels share this function's type)
-    static const void *done[8] = {};
+    static const void *done[12] = {};
     bool seen = false;
     for (const void *d : done)
         seen = seen || d == (const void *)kern;
