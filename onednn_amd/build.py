@@ -28,7 +28,10 @@ DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 # (source, object suffix, extra defines)
-UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", []),
+# the decode kernel takes its address-forming arguments preloaded into scalar
+# registers at wave launch (leading kernel arguments, at most 14 dwords)
+PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
+UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", PRELOAD),
          ("qmm_pack.hip", "", []), ("qmm_quantize.hip", "", []),
          ("qmm_dispatch.hip", "", []),
          ("qmm_gemm_b8.hip", "", []),

@@ -60,14 +60,36 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-// FAST: one 16-bit scale and at most one byte-sized (4- or 8-bit) zero point
-// per column and 128-k tile. Every load of that variant is unconditional
-// (out-of-range tiles re-read the last valid one, absent buffers are replaced
-// by the weights pointer), so the number of loads in flight is known at
-// compile time and no wait has to drain the whole queue.
-template <bool F16, int FAST>
+// Cross-wave reduction of the partial sums and the epilogue, shared by the two
+// kernels: every wave leaves its 4 values per lane in LDS, wave 0 adds them in
+// wave order and stores.
+QMM_D void gemv_reduce_store(const gemv_params_t &p, float *red, const v4f &out,
+        int wave, int lane, int m_base, int rows, int n) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        red[(wave * 64 + lane) * 4 + j] = out[j];
+    __syncthreads();
+    if (wave == 0) {
+        const int c = lane >> 4;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float v = 0.f;
+            for (int w = 0; w < GEMV_WAVES; w++)
+                v += red[(w * 64 + lane) * 4 + j];
+            // MFMA output: register j of lane l is row 4*(l/16)+j, column l%16
+            const int m = m_base + 4 * c + j;
+            if (m < p.M && n < p.N && 4 * c + j < rows)
+                epilogue_apply_store(p.ep, v, 0, m, n);
+        }
+    }
+}
+
+// General kernel: any group sizes and scale / zero-point types the
+// implementation accepts; activations staged in LDS, K walked in a loop.
+template <bool F16>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
+    constexpr int FAST = 0;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // lds: activations [KC/8 chunks][MR rows][16 bytes]; later reused for the
     // cross-wave reduction [GEMV_WAVES][64 lanes][4 floats]
@@ -162,150 +184,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     const uint8_t *const fast_zp = p.zps ? (const uint8_t *)p.zps : p.B;
     const bool zp4 = p.zp_dt == dt_s4 || p.zp_dt == dt_u4;
 
-    if constexpr (FAST) {
-        // Waves are independent until the final reduction: each one fetches
-        // its weight tiles, their scales / zero points AND its activation
-        // fragments (lane (r, c) holds row r, k = 32 s + 8 c .. + 7 of a tile)
-        // straight into registers, every load unconditional (clamped
-        // addresses), all issued before the first use. No LDS staging, no
-        // barrier before the arithmetic. Tile and group indices are wave
-        // uniform (scalar arithmetic, shifts instead of divisions). Rows past
-        // M compute on a repeated row and are never stored; only k past K has
-        // to be zeroed (the padded weights decode to the magic offset, not 0).
-        const int uw = __builtin_amdgcn_readfirstlane(wave);
-        const int tiles = Kpad / 128;
-        const int rr = min(r, rows - 1);
-        const uint16_t *__restrict__ Arow
-                = p.A + (int64_t)(m_base + rr) * p.lda;
-        const int nn = min(n, p.N - 1);
-        const uint16_t *const scn = fast_sc + (p.scale_per_n ? nn : 0);
-        const int zcol = p.zp_per_n ? nn : 0;
-        const bool sc_f16 = p.scale_dt == dt_f16;
-        const bool k_tail = (p.K & 127) != 0;
-        constexpr int UNR = 4;
-        for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
-            uint4 wt[UNR], av[UNR][4];
-            uint32_t scp[UNR], zpp[UNR];
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
-                wt[u] = ld_stream(Bt + (int64_t)tc * 1024);
-            }
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
-                if constexpr (FAST == 2) {
-                    // a single activation row: lane (r, c) fetches what lane
-                    // (0, c) multiplies in step r % 4, one load per tile
-                    const int k = min(
-                            tc * 128 + (r & 3) * 32 + c * 8, p.K - 8);
-                    av[u][0] = *(const uint4 *)(p.A + (int64_t)m_base * p.lda + k);
-                } else {
-#pragma unroll
-                    for (int s4 = 0; s4 < 4; s4++) {
-                        // chunks past the row's end re-read its last one
-                        const int k = min(tc * 128 + s4 * 32 + c * 8, p.K - 8);
-                        av[u][s4] = *(const uint4 *)(Arow + k);
-                    }
-                }
-                const int gsc = p.gs_shift < 0 ? 0 : tc >> p.gs_shift;
-                scp[u] = scn[(int64_t)gsc * sN];
-                const int gzp = p.gz_shift < 0 ? 0 : tc >> p.gz_shift;
-                const int64_t zi = p.zps ? (int64_t)gzp * zN + zcol : 0;
-                zpp[u] = fast_zp[zp4 ? zi >> 1 : zi];
-            }
-            if (k_tail && tb + UNR * GEMV_WAVES >= tiles) {
-                // zero the activations past K (last tile of the matrix)
-#pragma unroll
-                for (int u = 0; u < UNR; u++) {
-                    const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
-                    if constexpr (FAST == 2) {
-                        if (tc * 128 + (r & 3) * 32 + c * 8 >= p.K)
-                            av[u][0] = make_uint4(0, 0, 0, 0);
-                    } else {
-#pragma unroll
-                        for (int s4 = 0; s4 < 4; s4++)
-                            if (tc * 128 + s4 * 32 + c * 8 >= p.K)
-                                av[u][s4] = make_uint4(0, 0, 0, 0);
-                    }
-                }
-            }
-            // the four tiles are independent accumulation chains: a tile past
-            // the end is a repeat of the last one and is folded with scale 0
-            v4f Pu[UNR], Su[UNR];
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                Pu[u] = v4f {0.f, 0.f, 0.f, 0.f};
-                Su[u] = v4f {0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int s4 = 0; s4 < 4; s4++) {
-#pragma unroll
-                for (int u = 0; u < UNR; u++) {
-                    const uint32_t d = (s4 == 0 ? wt[u].x
-                                    : s4 == 1   ? wt[u].y
-                                    : s4 == 2   ? wt[u].z
-                                                : wt[u].w)
-                            ^ sflip;
-                    v4u b;
-                    b.x = (d & 0x000F000Fu) | MAGIC;
-                    b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
-                    b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
-                    b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
-                    v4u a;
-                    if constexpr (FAST == 2) {
-                        // row 0 of the operand takes step s4's chunk from lane
-                        // (s4, c); the other rows hold other steps' chunks and
-                        // produce rows of the result that are never stored
-                        const uint4 v = av[u][0];
-                        if (s4 == 0)
-                            a = v4u {v.x, v.y, v.z, v.w};
-                        else if (s4 == 1)
-                            a = v4u {row_shl<1>(v.x), row_shl<1>(v.y),
-                                    row_shl<1>(v.z), row_shl<1>(v.w)};
-                        else if (s4 == 2)
-                            a = v4u {row_shl<2>(v.x), row_shl<2>(v.y),
-                                    row_shl<2>(v.z), row_shl<2>(v.w)};
-                        else
-                            a = v4u {row_shl<3>(v.x), row_shl<3>(v.y),
-                                    row_shl<3>(v.z), row_shl<3>(v.w)};
-                    } else {
-                        a = v4u {av[u][s4].x, av[u][s4].y, av[u][s4].z,
-                                av[u][s4].w};
-                    }
-                    Pu[u] = mfma16<F16>(a, b, Pu[u]);
-                    Su[u] = mfma16<F16>(a, ones, Su[u]);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int t = tb + uw + u * GEMV_WAVES;
-                const int tc = min(t, tiles - 1);
-                // one scale and one zero point per column and tile
-                float sc = sc_f16
-                        ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
-                        : u2f(scp[u] << 16);
-                if (t >= tiles) sc = 0.f;
-                float zp = 0.f;
-                if (p.zps) {
-                    const int gzp = p.gz_shift < 0 ? 0 : tc >> p.gz_shift;
-                    const int64_t zi = (int64_t)gzp * zN + zcol;
-                    const uint32_t raw = zpp[u];
-                    if (zp4) {
-                        const int nib = (zi & 1) ? (raw >> 4) & 0xf : raw & 0xf;
-                        zp = (float)(p.zp_dt == dt_s4 ? s4_value(nib) : nib);
-                    } else {
-                        zp = p.zp_dt == dt_s8 ? (float)(int8_t)raw
-                                              : (float)(uint8_t)raw;
-                    }
-                }
-                const float off = OFFSET + soff + zp;
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    out[j] = __builtin_fmaf(sc, Pu[u][j] - off * Su[u][j], out[j]);
-            }
-        }
-    } else {
+    {
         for (int kc0 = 0; kc0 < Kpad; kc0 += KC) {
             const int kc_len = min(KC, Kpad - kc0);
             const int tiles = kc_len / 128;
@@ -419,24 +298,201 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
     }
 
     // ---- reduce the waves' partial sums and finish ----
-    if constexpr (!FAST) __syncthreads(); // the staged activations are dead
-    float *red = (float *)lds;
+    __syncthreads(); // the staged activations are dead
+    gemv_reduce_store(p, (float *)lds, out, wave, lane, m_base, rows, n);
+}
+
+// Fast kernel: one 16-bit scale and at most one byte-sized (4- or 8-bit) zero
+// point per column and 128-k tile, group widths 128 << s (or all of K). Every
+// load is unconditional (out-of-range tiles re-read the last valid one, an
+// absent zero-point buffer is replaced by the weights pointer), so the number
+// of loads in flight is known at compile time and no wait drains the whole
+// queue. ONE_ROW: a single activation row, one activation load per tile.
+//
+// A launch of this kernel lives a few microseconds, and the first of them
+// passes before its first load is issued. Part of that was the kernel waiting
+// for its own arguments: the parameter block arrived through three dependent
+// rounds of scalar loads before the first weights address existed. Everything
+// the load addresses depend on is therefore passed as 14 leading scalar
+// arguments, which the hardware preloads into registers while the wave is
+// launched (the build enables this for this file); the rest of the parameter
+// block is only needed for the epilogue and is fetched under the weights'
+// latency.
+//   shifts: gs_shift | gz_shift << 8 (as bytes; 0xff: one group over all of K)
+//   flags_m: bit 0 scale per column, 1 zero point per column, 2 zero points
+//     4-bit, 3 zero points signed, 4 scales f16 (else bf16), 5 weights signed,
+//     6 zero points present; bits 8..: M
+template <bool F16, bool ONE_ROW>
+__global__ void __launch_bounds__(GEMV_WAVES * 64)
+gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
+        const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
+        const uint8_t *__restrict__ pZP, const int kg128, const int N,
+        const int K, const int lda, const int shifts, const int flags_m,
+        const gemv_params_t p) {
+    __shared__ __attribute__((aligned(16))) float red[GEMV_WAVES * 64 * 4];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int uw = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // consecutive workgroups run on the 8 XCDs in turn: give each XCD a
+    // contiguous range of column blocks, so that a scale / zero-point line
+    // (64 and more neighbouring columns) is fetched into one L2 only
+    const int nb16 = (N + 15) >> 4;
+    const int bx = blockIdx.x;
+    const int nb = (nb16 & 7) == 0 ? (bx & 7) * (nb16 >> 3) + (bx >> 3) : bx;
+    const int M = flags_m >> 8;
+    const int m_base = blockIdx.y * 16;
+    const int rows = min(16, M - m_base);
+    const int c = lane >> 4; // k chunk of the lane
+    const int r = lane & 15; // activation row (A operand) / column (B operand)
+    const int n = nb * 16 + r;
+    const int gs_shift = (int8_t)(shifts & 0xff), gz_shift = (int8_t)(shifts >> 8);
+    const bool scale_per_n = flags_m & 1, zp_per_n = flags_m & 2;
+    const bool zp4 = flags_m & 4, zp_signed = flags_m & 8, sc_f16 = flags_m & 16;
+    const bool wei_signed = flags_m & 32, has_zp = flags_m & 64;
+
+    constexpr uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    constexpr float OFFSET = F16 ? 1024.f : 128.f;
+    constexpr uint32_t ONE2 = F16 ? 0x3C003C00u : 0x3F803F80u;
+    const v4u ones = {ONE2, ONE2, ONE2, ONE2};
+    const uint32_t sflip = wei_signed ? 0x88888888u : 0u;
+    const float soff = wei_signed ? 8.f : 0.f;
+
+    v4f out = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t *__restrict__ Bt = pB + ((int64_t)nb * kg128) * 1024 + lane * 16;
+    const int64_t sN = scale_per_n ? N : 0, zN = zp_per_n ? N : 0;
+
+    // Waves are independent until the final reduction: each one fetches its
+    // weight tiles, their scales / zero points AND its activation fragments
+    // (lane (r, c) holds row r, k = 32 s + 8 c .. + 7 of a tile) straight into
+    // registers, every load unconditional (clamped addresses), all issued
+    // before the first use. No LDS staging, no barrier before the arithmetic.
+    // Tile and group indices are wave uniform (scalar arithmetic, shifts
+    // instead of divisions). Rows past M compute on a repeated row and are
+    // never stored; only k past K has to be zeroed (the padded weights decode
+    // to the magic offset, not 0).
+    const int tiles = kg128;
+    const int rr = min(r, rows - 1);
+    const uint16_t *__restrict__ Arow = pA + (int64_t)(m_base + rr) * lda;
+    const int nn = min(n, N - 1);
+    const uint16_t *const scn = pSC + (scale_per_n ? nn : 0);
+    const int zcol = zp_per_n ? nn : 0;
+    const bool k_tail = (K & 127) != 0;
+    constexpr int UNR = 4;
+    constexpr int NA = ONE_ROW ? 1 : 4; // activation loads per tile
+    for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
+        // Loads are issued tile by tile (weights, activations, scale, zero
+        // point) and consumed in the same order below: results return in
+        // issue order, so tile u is unpacked and multiplied while tiles
+        // u + 1 .. are still arriving. (Requesting all activations first and
+        // the scales last, so that only the weights order the arithmetic, was
+        // measured slower: the first weights request leaves later.)
+        uint4 wt[UNR], av[UNR][NA];
+        uint32_t scp[UNR], zpp[UNR];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-        red[(wave * 64 + lane) * 4 + j] = out[j];
-    __syncthreads();
-    if (wave == 0) {
+        for (int u = 0; u < UNR; u++) {
+            const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+            wt[u] = ld_stream(Bt + (int64_t)tc * 1024);
+            if constexpr (ONE_ROW) {
+                // a single activation row: lane (r, c) fetches what lane
+                // (0, c) multiplies in step r % 4, one load per tile
+                const int k = min(tc * 128 + (r & 3) * 32 + c * 8, K - 8);
+                av[u][0] = *(const uint4 *)(pA + (int64_t)m_base * lda + k);
+            } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float v = 0.f;
-            for (int w = 0; w < GEMV_WAVES; w++)
-                v += red[(w * 64 + lane) * 4 + j];
-            // MFMA output: register j of lane l is row 4*(l/16)+j, column l%16
-            const int m = m_base + 4 * c + j;
-            if (m < p.M && n < p.N && 4 * c + j < rows)
-                epilogue_apply_store(p.ep, v, 0, m, n);
+                for (int s4 = 0; s4 < 4; s4++) {
+                    // chunks past the row's end re-read its last one
+                    const int k = min(tc * 128 + s4 * 32 + c * 8, K - 8);
+                    av[u][s4] = *(const uint4 *)(Arow + k);
+                }
+            }
+            const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
+            scp[u] = scn[(int64_t)gsc * sN];
+            const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+            const int64_t zi = has_zp ? (int64_t)gzp * zN + zcol : 0;
+            zpp[u] = pZP[zp4 ? zi >> 1 : zi];
+        }
+        if (k_tail && tb + UNR * GEMV_WAVES >= tiles) {
+            // zero the activations past K (last tile of the matrix)
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+                if constexpr (ONE_ROW) {
+                    if (tc * 128 + (r & 3) * 32 + c * 8 >= K)
+                        av[u][0] = make_uint4(0, 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++)
+                        if (tc * 128 + s4 * 32 + c * 8 >= K)
+                            av[u][s4] = make_uint4(0, 0, 0, 0);
+                }
+            }
+        }
+        // the four tiles are independent accumulation chains: a tile past
+        // the end is a repeat of the last one and is folded with scale 0
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            v4f Pu = {0.f, 0.f, 0.f, 0.f}, Su = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+                const uint32_t d = (s4 == 0 ? wt[u].x
+                                : s4 == 1   ? wt[u].y
+                                : s4 == 2   ? wt[u].z
+                                            : wt[u].w)
+                        ^ sflip;
+                v4u b;
+                b.x = (d & 0x000F000Fu) | MAGIC;
+                b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
+                b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
+                b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
+                v4u a;
+                if constexpr (ONE_ROW) {
+                    // row 0 of the operand takes step s4's chunk from lane
+                    // (s4, c); the other rows hold other steps' chunks and
+                    // produce rows of the result that are never stored
+                    const uint4 v = av[u][0];
+                    if (s4 == 0)
+                        a = v4u {v.x, v.y, v.z, v.w};
+                    else if (s4 == 1)
+                        a = v4u {row_shl<1>(v.x), row_shl<1>(v.y),
+                                row_shl<1>(v.z), row_shl<1>(v.w)};
+                    else if (s4 == 2)
+                        a = v4u {row_shl<2>(v.x), row_shl<2>(v.y),
+                                row_shl<2>(v.z), row_shl<2>(v.w)};
+                    else
+                        a = v4u {row_shl<3>(v.x), row_shl<3>(v.y),
+                                row_shl<3>(v.z), row_shl<3>(v.w)};
+                } else {
+                    a = v4u {av[u][s4].x, av[u][s4].y, av[u][s4].z,
+                            av[u][s4].w};
+                }
+                Pu = mfma16<F16>(a, b, Pu);
+                Su = mfma16<F16>(a, ones, Su);
+            }
+            const int t = tb + uw + u * GEMV_WAVES;
+            const int tc = min(t, tiles - 1);
+            // one scale and one zero point per column and tile
+            float sc = sc_f16
+                    ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
+                    : u2f(scp[u] << 16);
+            if (t >= tiles) sc = 0.f;
+            float zp = 0.f;
+            if (has_zp) {
+                const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+                const int64_t zi = (int64_t)gzp * zN + zcol;
+                const uint32_t raw = zpp[u];
+                if (zp4) {
+                    const int nib = (zi & 1) ? (raw >> 4) & 0xf : raw & 0xf;
+                    zp = (float)(zp_signed ? s4_value(nib) : nib);
+                } else {
+                    zp = zp_signed ? (float)(int8_t)raw : (float)(uint8_t)raw;
+                }
+            }
+            const float off = OFFSET + soff + zp;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                out[j] = __builtin_fmaf(sc, Pu[j] - off * Su[j], out[j]);
         }
     }
+    gemv_reduce_store(p, red, out, uw, lane, m_base, rows, n);
 }
 
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
@@ -484,9 +540,32 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
             && (!p.zps || p.zp_dt != dt_s32) && shift_of(p.gs, q.gs_shift)
             && (p.gz > 0 ? shift_of(p.gz, q.gz_shift)
                          : ((q.gz_shift = -1), true));
+    if (fast && p.m0 == 0 && p.lda < ((int64_t)1 << 31)) {
+        const int flags_m = (p.scale_per_n ? 1 : 0) | (p.zp_per_n ? 2 : 0)
+                | (p.zp_dt == dt_s4 || p.zp_dt == dt_u4 ? 4 : 0)
+                | (p.zp_dt == dt_s4 || p.zp_dt == dt_s8 ? 8 : 0)
+                | (p.scale_dt == dt_f16 ? 16 : 0) | (p.wei_signed ? 32 : 0)
+                | (p.zps ? 64 : 0) | (p.M << 8);
+        const int shifts = (q.gs_shift & 0xff) | ((q.gz_shift & 0xff) << 8);
+        // an absent zero-point buffer is never dereferenced past its first
+        // byte: the weights stand in for it
+        const uint8_t *zp = p.zps ? (const uint8_t *)p.zps : p.B;
+        auto go = [&](auto kern) {
+            hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), 0, stream, p.B,
+                    p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
+                    (int)p.lda, shifts, flags_m, q);
+        };
+        if (p.act_f16)
+            p.M == 1 ? go(gemv_w4_fast_kernel<true, true>)
+                     : go(gemv_w4_fast_kernel<true, false>);
+        else
+            p.M == 1 ? go(gemv_w4_fast_kernel<false, true>)
+                     : go(gemv_w4_fast_kernel<false, false>);
+        return;
+    }
     auto launch = [&](auto kern) {
-        // (the six kernels share this lambda's type: one call each)
-        static const void *done[6] = {};
+        // (the two kernels share this lambda's type: one call each)
+        static const void *done[2] = {};
         bool seen = false;
         for (const void *d : done)
             seen = seen || d == (const void *)kern;
@@ -503,23 +582,10 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, q,
                 MR, KC);
     };
-    if (fast) lds = red; // that variant keeps its activations in registers
-    // a single row: one activation load per tile instead of four (FAST == 2)
-    if (p.act_f16) {
-        if (fast && p.M == 1)
-            launch(gemv_w4_kernel<true, 2>);
-        else if (fast)
-            launch(gemv_w4_kernel<true, 1>);
-        else
-            launch(gemv_w4_kernel<true, 0>);
-    } else {
-        if (fast && p.M == 1)
-            launch(gemv_w4_kernel<false, 2>);
-        else if (fast)
-            launch(gemv_w4_kernel<false, 1>);
-        else
-            launch(gemv_w4_kernel<false, 0>);
-    }
+    if (p.act_f16)
+        launch(gemv_w4_kernel<true>);
+    else
+        launch(gemv_w4_kernel<false>);
 }
 
 } // namespace qmm
