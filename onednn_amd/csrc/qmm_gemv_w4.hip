@@ -62,24 +62,37 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
 
 // Cross-wave reduction of the partial sums and the epilogue, shared by the two
 // kernels: every wave leaves its 4 values per lane in LDS, wave 0 adds them in
-// wave order and stores.
+// wave order and stores. ONE_ROW: only row 0 (register 0 of lanes 0..15) is
+// live. `plain` (wave-uniform): nothing follows the accumulation (no scales,
+// bias, post-ops, dst scale or zero point) and dst is dense along n, so the
+// value is converted and stored without the post-op interpreter; `dst` and
+// `dst_sm` are then the dst pointer and row pitch, read by the caller long
+// before (the parameter block is cold, its first touch costs a trip to memory).
+template <bool ONE_ROW>
 QMM_D void gemv_reduce_store(const gemv_params_t &p, float *red, const v4f &out,
-        int wave, int lane, int m_base, int rows, int n) {
+        int wave, int lane, int m_base, int rows, int n, bool plain = false,
+        void *dst = nullptr, int64_t dst_sm = 0, int dst_dt = 0) {
+    constexpr int NJ = ONE_ROW ? 1 : 4;
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-        red[(wave * 64 + lane) * 4 + j] = out[j];
+    for (int j = 0; j < NJ; j++)
+        red[(wave * 64 + lane) * NJ + j] = out[j];
     __syncthreads();
     if (wave == 0) {
         const int c = lane >> 4;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NJ; j++) {
             float v = 0.f;
+#pragma unroll
             for (int w = 0; w < GEMV_WAVES; w++)
-                v += red[(w * 64 + lane) * 4 + j];
+                v += red[(w * 64 + lane) * NJ + j];
             // MFMA output: register j of lane l is row 4*(l/16)+j, column l%16
             const int m = m_base + 4 * c + j;
-            if (m < p.M && n < p.N && 4 * c + j < rows)
-                epilogue_apply_store(p.ep, v, 0, m, n);
+            if (m < p.M && n < p.N && 4 * c + j < rows) {
+                if (plain)
+                    store_float(dst_dt, v, dst, m * dst_sm + n);
+                else
+                    epilogue_apply_store(p.ep, v, 0, m, n);
+            }
         }
     }
 }
@@ -299,7 +312,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 
     // ---- reduce the waves' partial sums and finish ----
     __syncthreads(); // the staged activations are dead
-    gemv_reduce_store(p, (float *)lds, out, wave, lane, m_base, rows, n);
+    gemv_reduce_store<false>(p, (float *)lds, out, wave, lane, m_base, rows, n);
 }
 
 // Fast kernel: one 16-bit scale and at most one byte-sized (4- or 8-bit) zero
@@ -321,8 +334,9 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 //   shifts: gs_shift | gz_shift << 8 (as bytes; 0xff: one group over all of K)
 //   flags_m: bit 0 scale per column, 1 zero point per column, 2 zero points
 //     4-bit, 3 zero points signed, 4 scales f16 (else bf16), 5 weights signed,
-//     6 zero points present; bits 8..: M
-template <bool F16, bool ONE_ROW>
+//     6 zero points present, 7 plain store (see gemv_reduce_store);
+//     bits 8..: M
+template <bool F16, bool ONE_ROW, bool WSIGNED>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
@@ -338,7 +352,7 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     const int nb16 = (N + 15) >> 4;
     const int bx = blockIdx.x;
     const int nb = (nb16 & 7) == 0 ? (bx & 7) * (nb16 >> 3) + (bx >> 3) : bx;
-    const int M = flags_m >> 8;
+    const int M = (uint32_t)flags_m >> 8;
     const int m_base = blockIdx.y * 16;
     const int rows = min(16, M - m_base);
     const int c = lane >> 4; // k chunk of the lane
@@ -347,14 +361,20 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     const int gs_shift = (int8_t)(shifts & 0xff), gz_shift = (int8_t)(shifts >> 8);
     const bool scale_per_n = flags_m & 1, zp_per_n = flags_m & 2;
     const bool zp4 = flags_m & 4, zp_signed = flags_m & 8, sc_f16 = flags_m & 16;
-    const bool wei_signed = flags_m & 32, has_zp = flags_m & 64;
+    const bool has_zp = flags_m & 64;
 
-    constexpr uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
     constexpr float OFFSET = F16 ? 1024.f : 128.f;
     constexpr uint32_t ONE2 = F16 ? 0x3C003C00u : 0x3F803F80u;
     const v4u ones = {ONE2, ONE2, ONE2, ONE2};
-    const uint32_t sflip = wei_signed ? 0x88888888u : 0u;
-    const float soff = wei_signed ? 8.f : 0.f;
+    constexpr uint32_t sflip = WSIGNED ? 0x88888888u : 0u;
+    constexpr float soff = WSIGNED ? 8.f : 0.f;
+    // the exponent pattern lives in a vector register and the nibble mask in a
+    // scalar one: (d >> 4 i) & mask | magic is then a shift and one
+    // v_and_or_b32 (an instruction takes one scalar or literal operand only)
+    uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    asm volatile("" : "+v"(MAGIC));
+    uint32_t NIB = 0x000F000Fu;
+    asm volatile("" : "+s"(NIB));
 
     v4f out = {0.f, 0.f, 0.f, 0.f};
     const uint8_t *__restrict__ Bt = pB + ((int64_t)nb * kg128) * 1024 + lane * 16;
@@ -378,6 +398,9 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     const bool k_tail = (K & 127) != 0;
     constexpr int UNR = 4;
     constexpr int NA = ONE_ROW ? 1 : 4; // activation loads per tile
+    void *dst_ptr = nullptr;
+    int64_t dst_sm = 0;
+    int dst_dt = 0;
     for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
         // Loads are issued tile by tile (weights, activations, scale, zero
         // point) and consumed in the same order below: results return in
@@ -426,6 +449,14 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                 }
             }
         }
+        // what the final store needs from the (cold) parameter block is
+        // requested here, behind the loads and ahead of the arithmetic
+        if (tb == 0) {
+            dst_ptr = (void *)p.ep.dst.ptr;
+            dst_sm = p.ep.dst.sm;
+            dst_dt = p.ep.dst.dt;
+            asm volatile("" ::"s"(dst_ptr), "s"(dst_sm), "s"(dst_dt));
+        }
         // the four tiles are independent accumulation chains: a tile past
         // the end is a repeat of the last one and is folded with scale 0
 #pragma unroll
@@ -439,10 +470,10 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                                             : wt[u].w)
                         ^ sflip;
                 v4u b;
-                b.x = (d & 0x000F000Fu) | MAGIC;
-                b.y = ((d >> 4) & 0x000F000Fu) | MAGIC;
-                b.z = ((d >> 8) & 0x000F000Fu) | MAGIC;
-                b.w = ((d >> 12) & 0x000F000Fu) | MAGIC;
+                b.x = (d & NIB) | MAGIC;
+                b.y = ((d >> 4) & NIB) | MAGIC;
+                b.z = ((d >> 8) & NIB) | MAGIC;
+                b.w = ((d >> 12) & NIB) | MAGIC;
                 v4u a;
                 if constexpr (ONE_ROW) {
                     // row 0 of the operand takes step s4's chunk from lane
@@ -474,25 +505,23 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                     ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
                     : u2f(scp[u] << 16);
             if (t >= tiles) sc = 0.f;
-            float zp = 0.f;
-            if (has_zp) {
-                const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
-                const int64_t zi = (int64_t)gzp * zN + zcol;
-                const uint32_t raw = zpp[u];
-                if (zp4) {
-                    const int nib = (zi & 1) ? (raw >> 4) & 0xf : raw & 0xf;
-                    zp = (float)(zp_signed ? s4_value(nib) : nib);
-                } else {
-                    zp = zp_signed ? (float)(int8_t)raw : (float)(uint8_t)raw;
-                }
-            }
+            // zero point: byte or nibble, signed or not, by shifts and selects
+            // (wave-uniform branches here cost more than the arithmetic)
+            const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+            const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol) & 1) : 0;
+            const int zbits = zp4 ? 4 : 8;
+            const uint32_t zraw = (zpp[u] >> (4 * odd)) & ((1u << zbits) - 1u);
+            const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
+            const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
             const float off = OFFSET + soff + zp;
+            // a single row: only register 0 (row 0) is stored
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int j = 0; j < (ONE_ROW ? 1 : 4); j++)
                 out[j] = __builtin_fmaf(sc, Pu[j] - off * Su[j], out[j]);
         }
     }
-    gemv_reduce_store(p, red, out, uw, lane, m_base, rows, n);
+    gemv_reduce_store<ONE_ROW>(p, red, out, uw, lane, m_base, rows, n,
+            (flags_m & 128) != 0, dst_ptr, dst_sm, dst_dt);
 }
 
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
@@ -540,12 +569,16 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
             && (!p.zps || p.zp_dt != dt_s32) && shift_of(p.gs, q.gs_shift)
             && (p.gz > 0 ? shift_of(p.gz, q.gz_shift)
                          : ((q.gz_shift = -1), true));
-    if (fast && p.m0 == 0 && p.lda < ((int64_t)1 << 31)) {
+    if (fast && p.m0 == 0 && p.lda < ((int64_t)1 << 31) && p.M < (1 << 23)) {
+        // nothing between the accumulation and a dense dst row
+        const bool plain = !p.ep.src_scale.ptr && !p.ep.wei_scale.ptr
+                && !p.ep.bias.ptr && p.ep.npo == 0 && !p.ep.dst_scale
+                && !p.ep.dst_zp && p.ep.dst.sn == 1;
         const int flags_m = (p.scale_per_n ? 1 : 0) | (p.zp_per_n ? 2 : 0)
                 | (p.zp_dt == dt_s4 || p.zp_dt == dt_u4 ? 4 : 0)
                 | (p.zp_dt == dt_s4 || p.zp_dt == dt_s8 ? 8 : 0)
                 | (p.scale_dt == dt_f16 ? 16 : 0) | (p.wei_signed ? 32 : 0)
-                | (p.zps ? 64 : 0) | (p.M << 8);
+                | (p.zps ? 64 : 0) | (plain ? 128 : 0) | (p.M << 8);
         const int shifts = (q.gs_shift & 0xff) | ((q.gz_shift & 0xff) << 8);
         // an absent zero-point buffer is never dereferenced past its first
         // byte: the weights stand in for it
@@ -555,12 +588,18 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
                     (int)p.lda, shifts, flags_m, q);
         };
-        if (p.act_f16)
-            p.M == 1 ? go(gemv_w4_fast_kernel<true, true>)
-                     : go(gemv_w4_fast_kernel<true, false>);
-        else
-            p.M == 1 ? go(gemv_w4_fast_kernel<false, true>)
-                     : go(gemv_w4_fast_kernel<false, false>);
+        const int which = (p.act_f16 ? 4 : 0) | (p.M == 1 ? 2 : 0)
+                | (p.wei_signed ? 1 : 0);
+        switch (which) {
+            case 0: go(gemv_w4_fast_kernel<false, false, false>); break;
+            case 1: go(gemv_w4_fast_kernel<false, false, true>); break;
+            case 2: go(gemv_w4_fast_kernel<false, true, false>); break;
+            case 3: go(gemv_w4_fast_kernel<false, true, true>); break;
+            case 4: go(gemv_w4_fast_kernel<true, false, false>); break;
+            case 5: go(gemv_w4_fast_kernel<true, false, true>); break;
+            case 6: go(gemv_w4_fast_kernel<true, true, false>); break;
+            default: go(gemv_w4_fast_kernel<true, true, true>); break;
+        }
         return;
     }
     auto launch = [&](auto kern) {
