@@ -136,6 +136,23 @@ QMM_API void qmm_matmul_plan_destroy(qmm_plan_t *plan);
 QMM_API int qmm_matmul_launch(const qmm_plan_t *plan,
         const qmm_matmul_args_t *args, void *hip_stream);
 
+/* qmm_matmul_launch() for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc). No counterpart in the reference: there the scratchpad is always
+ * a memory object the user or the library allocates. args->scratch is ignored;
+ * the kernels' scratch (weights packed on the fly, the s8 copy of a u8 source,
+ * per-group scale arrays) is a buffer of QMM_STATIC_SCRATCH_BYTES that the
+ * library holds on every GPU it runs on from load to process end. The call
+ * allocates nothing and fails with QMM_INVALID_ARGUMENTS (qmm_last_error()
+ * says why) when qmm_matmul_scratch_size() exceeds that size. All calls on one
+ * GPU share the buffer: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls on one stream do not. Every kernel writes
+ * the part of the buffer it later reads, so nothing has to be cleared between
+ * calls. */
+#define QMM_STATIC_SCRATCH_BYTES (32u << 20)
+QMM_API int qmm_matmul_launch_static_scratch(const qmm_plan_t *plan,
+        const qmm_matmul_args_t *args, void *hip_stream);
+
 /* ---- packed weights layouts ---- */
 /* Bytes a weights tensor [batch..., K, N] of type dt occupies in `layout`. */
 QMM_API size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N);

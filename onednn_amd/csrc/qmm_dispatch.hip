@@ -766,6 +766,52 @@ static bool aligned16(const void *p) {
     return ((uintptr_t)p & 15) == 0;
 }
 
+// ---- scratch for callers that cannot allocate ------------------------------
+// One array per GPU, resident from the moment the library's code is loaded on
+// that GPU until the process ends. Host code never uses the array's name as an
+// address: that name is a host-side stand-in, the device address is asked for
+// once per device (with that device current) and kept.
+static __device__ __align__(256) unsigned char scratch[QMM_STATIC_SCRATCH_BYTES];
+
+static void *static_scratch_ptr() {
+    constexpr int MAX_DEV = 64;
+    static std::mutex mu;
+    static void *ptr[MAX_DEV] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+        g_last_error = "no current HIP device for the static scratch";
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void *q = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !q) {
+            g_last_error = std::string("hipGetSymbolAddress(scratch): ")
+                    + hipGetErrorString(e);
+            return nullptr;
+        }
+        ptr[dev] = q;
+    }
+    return ptr[dev];
+}
+
+int qmm_matmul_launch_static_scratch(const qmm_plan_t *plan,
+        const qmm_matmul_args_t *args, void *hip_stream) {
+    if (!plan || !args) return QMM_INVALID_ARGUMENTS;
+    if (plan->scratch_bytes > (size_t)QMM_STATIC_SCRATCH_BYTES)
+        return fail(QMM_INVALID_ARGUMENTS,
+                "the problem needs more scratch than the static buffer holds "
+                "(QMM_STATIC_SCRATCH_BYTES)");
+    qmm_matmul_args_t a = *args;
+    a.scratch = nullptr;
+    if (plan->scratch_bytes) {
+        a.scratch = static_scratch_ptr();
+        if (!a.scratch) return QMM_RUNTIME_ERROR;
+    }
+    return qmm_matmul_launch(plan, &a, hip_stream);
+}
+
 int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         void *hip_stream) {
     if (!plan || !args) return QMM_INVALID_ARGUMENTS;
