@@ -291,20 +291,41 @@ def assert_bit_exact(got, want, what=""):
                                 want.reshape(-1)[bad[0]]))
 
 
-def assert_f32_close(got, want, rel=1e-5, scale=None, what=""):
+# Where a tolerance is widened (`scale` / `abs_slack` below), the share of elements
+# that needed the wider bound is measured, printed and capped: a regression that
+# pushes a large part of the outputs into the slack must not pass.
+SLACK_FRAC_MAX = 0.02
+
+
+def _report_slack(what, frac, ceiling):
+    if frac > 0:
+        print("[slack] %s: %.4f %% of the elements needed the widened bound (ceiling %.2f %%)"
+              % (what, 100 * frac, 100 * ceiling), flush=True)
+    assert frac <= ceiling, "%s: %.3f %% of the elements needed the widened bound (ceiling %.2f %%)" % (
+        what, 100 * frac, 100 * ceiling)
+
+
+def assert_f32_close(got, want, rel=1e-5, scale=None, what="", max_slack_frac=SLACK_FRAC_MAX):
     """|got - want| <= rel * max(|want|, scale): `scale` is the magnitude of the
     terms of the sum (a result that cancels to ~0 cannot be compared relative to
-    itself)."""
+    itself). Returns the fraction of elements that were outside rel * |want| and
+    only passed through `scale`; that fraction may not exceed max_slack_frac."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
     ref = np.abs(want) if scale is None else np.maximum(np.abs(want), scale)
     err = np.abs(got - want)
-    ok = (err <= rel * ref) | (got == want) | (np.isnan(got) & np.isnan(want))
+    same = (got == want) | (np.isnan(got) & np.isnan(want))
+    ok = (err <= rel * ref) | same
     if not ok.all():
         i = np.argmax(err / np.maximum(ref, 1e-300))
         raise AssertionError("%s: max rel err %.3g at %d (got %r want %r)"
                              % (what, (err / np.maximum(ref, 1e-300)).reshape(-1)[i], i,
                                 got.reshape(-1)[i], want.reshape(-1)[i]))
+    strict = (err <= rel * np.abs(want)) | same
+    frac = float(1.0 - strict.mean()) if strict.size else 0.0
+    if scale is not None:
+        _report_slack(what, frac, max_slack_frac)
+    return frac
 
 
 def bf16_ulp_distance(a_raw, b_raw):
@@ -315,19 +336,23 @@ def bf16_ulp_distance(a_raw, b_raw):
     return np.abs(key(np.asarray(a_raw)) - key(np.asarray(b_raw)))
 
 
-def assert_bf16_within_1ulp(got_raw, want_raw, what="", abs_slack=None):
+def assert_bf16_within_1ulp(got_raw, want_raw, what="", abs_slack=None, max_slack_frac=SLACK_FRAC_MAX):
     """bf16 results at most one representable value apart. `abs_slack` (array or
     scalar) additionally accepts |got - want| <= abs_slack: a kernel that sums
     in another order than the reference carries the f32 bar (1e-5 of the
     magnitude of the summed terms) into results that cancel towards zero, where
-    one bf16 ulp is arbitrarily small."""
-    d = bf16_ulp_distance(got_raw, want_raw)
+    one bf16 ulp is arbitrarily small. The fraction of elements more than one
+    representable value apart that only passed through abs_slack may not exceed
+    max_slack_frac. Returns the fraction of elements that differ at all."""
+    d = bf16_ulp_distance(got_raw, want_raw).reshape(-1)
     if abs_slack is not None:
         g = O.to_f32(O.BF16, np.asarray(got_raw)).astype(np.float64).reshape(-1)
         w = O.to_f32(O.BF16, np.asarray(want_raw)).astype(np.float64).reshape(-1)
         slack = np.asarray(abs_slack, np.float64).reshape(-1)
         ok = np.abs(g - w) <= (slack if slack.size == g.size else slack[0])
-        d = np.where(ok, np.minimum(d.reshape(-1), 1), d.reshape(-1))
+        needed = float(((d > 1) & ok).mean()) if d.size else 0.0
+        d = np.where(ok, np.minimum(d, 1), d)
+        _report_slack(what, needed, max_slack_frac)
     if d.max(initial=0) > 1:
         i = int(np.argmax(d))
         raise AssertionError("%s: bf16 distance %d at %d (got 0x%04x want 0x%04x)"

@@ -1,0 +1,141 @@
+"""How far the s32 accumulation over all of K (what every kernel here and the
+reference's optimized kernels do) is from what v3.8's ref_int8:any executes
+when no K groups are given: quant_entry_t::get_group() returns 1 there
+(src/common/primitive_attr_quant.hpp:83-90), so ref_matmul_int8.cpp:139-219
+closes a "group" after every k and sums (float)(s * w) * src_scale * wei_scale
+in f32, one k at a time (the oracle's KGROUP_LITERAL mode). The two agree bit
+for bit while every partial sum is exactly representable and differ by f32
+summation error otherwise. These tests measure that difference on the benchmark
+configurations and cap it:
+  * integer dst: never more than one unit apart, and rarely;
+  * f32 dst: the share of elements further than rel 1e-5 of |want| apart is
+    small, and every element is within 1e-5 of the magnitude of the summed
+    terms.
+The measured shares are printed ([literal] lines)."""
+import sys
+
+import numpy as np
+import pytest
+
+import onednn_amd as dnnl
+import oracle as O
+from onednn_amd import memory
+from qmm_harness import T, dt, tag
+import test_gpu_parity as cases
+
+pytestmark = pytest.mark.gpu
+A = dnnl
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    eng = dnnl.engine(dnnl.engine.kind.gpu, 0)
+    return eng, dnnl.stream(eng)
+
+
+def f32_shares(got, want, term):
+    """(share beyond rel 1e-5 of |want|, max error in units of 1e-5 * term scale)"""
+    got, want = got.astype(np.float64).reshape(-1), want.astype(np.float64).reshape(-1)
+    term = np.asarray(term, np.float64).reshape(-1)
+    err = np.abs(got - want)
+    beyond = float((err > 1e-5 * np.abs(want)).mean())
+    worst = float((err / (1e-5 * term)).max())
+    return beyond, worst
+
+
+def test_config1_f32_against_literal(ctx):
+    """Config 1 whole: u8 - 128 in [-128, 127], K = 1024: |acc| <= 2^24, every s32 sum exact in f32."""
+    eng, strm = ctx
+    say("config 1 (256x1024x1024, u8 zp 128, f32 dst) vs the literal per-k f32 reference")
+    p = cases.int8_linear(256, 1024, 1024, 41)
+    got = p.run_gpu(eng, strm, weights_any=True).view(np.float32)
+    want = p.run_oracle(k_group_mode=O.KGROUP_LITERAL).view(np.float32)
+    beyond, worst = f32_shares(got, want, cases.term_scale(p))
+    print("[literal] config 1 f32: %.4f %% of the elements beyond rel 1e-5 of |want|; worst error %.3f x 1e-5 of the term scale"
+          % (100 * beyond, worst), flush=True)
+    assert worst <= 1.0
+    assert beyond <= 0.05
+
+
+def test_config4_f32_against_literal(ctx):
+    """Config 4 (sampled heads and rows, K = 128: partial sums stay below 2^24)."""
+    eng, strm = ctx
+    say("config 4 rows (K=128, per-tensor scales, f32 dst + mask) vs the literal reference")
+    B, S, D = 2, 2048, 128
+    r = np.random.default_rng(4)
+    q = np.clip(np.rint(r.standard_normal((B, 64, D)) * 40), -127, 127).astype(np.int8)
+    k = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127).astype(np.int8)
+    attr = A.primitive_attr()
+    attr.set_scales_mask(A.DNNL_ARG_SRC, 0)
+    attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 0)
+    kt_md = memory.desc([B, D, S], dt.s8, T("acb"))
+    pd = A.matmul.primitive_desc(eng, memory.desc([B, 64, D], dt.s8, T("abc")), kt_md,
+                                 memory.desc([B, 64, S], dt.f32, T("abc")), attr=attr)
+    m_dst = memory(pd.dst_desc(), eng)
+    A.matmul(pd).execute(strm, {
+        A.DNNL_ARG_SRC: memory(pd.src_desc(), eng).write(q), A.DNNL_ARG_WEIGHTS: memory(kt_md, eng).write(k),
+        A.DNNL_ARG_DST: m_dst,
+        A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: memory(memory.desc([1], dt.f32, T("a")), eng).write(np.array([0.01], np.float32)),
+        A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: memory(memory.desc([1], dt.f32, T("a")), eng).write(np.array([0.012], np.float32))})
+    strm.wait()
+    got = m_dst.read(np.float32, (B, 64, S))
+    want = np.zeros((B, 64, S), np.float32)
+    O.matmul(O.Tensor(O.S8, [B, 64, D], q), O.Tensor(O.S8, [B, D, S], k, (D * S, 1, D)), O.Tensor(O.F32, [B, 64, S], want),
+             scales={O.Q_SRC: O.Quant(0, O.F32, np.array([0.01], np.float32)),
+                     O.Q_WEI: O.Quant(0, O.F32, np.array([0.012], np.float32))},
+             k_group_mode=O.KGROUP_LITERAL)
+    term = np.einsum("bmd,bnd->bmn", np.abs(q.astype(np.float64)), np.abs(k.astype(np.float64))) * 0.01 * 0.012
+    beyond, worst = f32_shares(got, want, term)
+    print("[literal] config 4 f32: %.4f %% of the elements beyond rel 1e-5 of |want|; worst error %.3f x 1e-5 of the term scale"
+          % (100 * beyond, worst), flush=True)
+    assert worst <= 1.0
+    assert beyond <= 0.10  # scores cancel towards 0: relative to |want| alone many tiny results are "far"
+
+
+def test_config2_slice_bf16_against_literal(ctx):
+    """A slice of config 2 (K = 4096, per-token and per-column scales, bf16 dst,
+    no post-op: the accumulation is what is compared)."""
+    eng, strm = ctx
+    say("config 2 slice (384x4096x512, per-token scales, bf16 dst) vs the literal reference")
+    p = cases.int8_linear(384, 4096, 512, 47, src_dt=dt.s8, dst_dt=dt.bf16, src_zp=None, per_token=True)
+    got = p.run_gpu(eng, strm, weights_any=True)
+    want = p.run_oracle(k_group_mode=O.KGROUP_LITERAL)
+    from qmm_harness import bf16_ulp_distance
+    d = bf16_ulp_distance(got, want).reshape(-1)
+    share = float((d > 0).mean())
+    far = d > 1
+    # further than one bf16 value only where the sum cancels: there the f32 bar
+    # relative to the summed terms holds
+    err = np.abs(O.to_f32(O.BF16, got).astype(np.float64) - O.to_f32(O.BF16, want).astype(np.float64)).reshape(-1)
+    term = cases.term_scale(p).reshape(-1)
+    print("[literal] config 2 slice bf16: %.4f %% of the elements differ, %.4f %% by more than one bf16 value "
+          "(max distance %d, all of them within %.3f x 1e-5 of the term scale)"
+          % (100 * share, 100 * float(far.mean()), int(d.max()),
+             float((err[far] / (1e-5 * term[far])).max()) if far.any() else 0.0), flush=True)
+    assert (err[far] <= 1e-5 * term[far]).all()
+    assert float(far.mean()) <= 0.001
+    assert share <= 0.02
+
+
+@pytest.mark.parametrize("name", ["u8_zp_7_s8_dst", "s8_u8_dst_relu"])
+def test_integer_dst_against_literal(ctx, name):
+    """s8 / u8 dst (dst scale, zero point, bias, relu): at most one unit from the
+    literal reference, on a small share of the elements."""
+    eng, strm = ctx
+    say("integer dst %s vs the literal reference" % name)
+    p = cases.MFMA_CASES[name][0]()
+    got = p.run_gpu(eng, strm, weights_any=True)
+    want = p.run_oracle(k_group_mode=O.KGROUP_LITERAL)
+    is_s8 = p.dst.dt == dt.s8
+    g = got.view(np.int8 if is_s8 else np.uint8).astype(np.int32)
+    w = want.view(np.int8 if is_s8 else np.uint8).astype(np.int32)
+    diff = np.abs(g - w)
+    share = float((diff > 0).mean())
+    print("[literal] %s: %.4f %% of the elements differ, max |diff| %d" % (name, 100 * share, int(diff.max())), flush=True)
+    assert diff.max() <= 1
+    assert share <= 0.01

@@ -233,6 +233,13 @@ def test_generic_fp8_and_f32(ctx):
     assert_bit_exact(p.run_gpu(eng, strm), p.run_oracle(), "f32")
 
 
+# f32 results of the fp8 kernels: the MFMA's summation tree against the reference's
+# sequential k loop. Both are f32 sums of exact products; they differ in the low
+# bits of most results (more than 1e-5 of the result for about 60 % of them at
+# K = 1024, the reference's own sequential rounding being the larger part), and
+# every result stays within 1e-5 of the magnitude of the summed terms.
+FP8_F32_SLACK = 0.80
+
 # ---------------------------------------------------------------------------
 # MFMA int8 GEMM: exact s32 accumulation + reference-ordered epilogue
 MFMA_CASES = {
@@ -288,7 +295,7 @@ def test_mfma_int8_against_literal_v38_reference(ctx):
     p = int8_linear(64, 1024, 128, 52)
     got = p.run_gpu(eng, strm, weights_any=True).view(np.float32).reshape(64, 128)
     want = p.run_oracle(k_group_mode=O.KGROUP_LITERAL).view(np.float32).reshape(64, 128)
-    assert_f32_close(got, want, rel=1e-5, scale=term_scale(p), what="literal")
+    assert_f32_close(got, want, rel=1e-5, scale=term_scale(p), what="literal", max_slack_frac=0.05)  # measured 1.9 %
 
 
 # ---------------------------------------------------------------------------
@@ -510,7 +517,7 @@ def test_mfma_fp8_tile256_kernel(ctx, tile256):
             assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
         else:
             assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
-                             rel=1e-5, scale=a, what="fp8 f32")
+                             rel=1e-5, scale=a, what="fp8 f32", max_slack_frac=FP8_F32_SLACK)
 
 
 def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
@@ -534,7 +541,7 @@ def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
                     assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
                 else:
                     assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
-                                     rel=1e-5, scale=a, what="fp8 f32")
+                                     rel=1e-5, scale=a, what="fp8 f32", max_slack_frac=FP8_F32_SLACK)
         finally:
             _capi.lib().qmm_set_b8x_variant(1)
 
@@ -573,7 +580,7 @@ def test_mfma_fp8_tile256_sum_operand_batches(ctx, tile256, dd):
         assert_bf16_within_1ulp(got, want, "fp8 sum bf16", abs_slack=1e-5 * a)
     elif dd == dt.f32:
         assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
-                         rel=1e-5, scale=a, what="fp8 sum f32")
+                         rel=1e-5, scale=a, what="fp8 sum f32", max_slack_frac=FP8_F32_SLACK)
     else:
         g, w = O.to_f32(dt.f16, got).reshape(M, N), O.to_f32(dt.f16, want).reshape(M, N)
         assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 1e-5 * a * 1024, what="fp8 sum f16")
@@ -633,7 +640,7 @@ def test_mfma_fp8(ctx):
                 assert_bf16_within_1ulp(got, want, "fp8 bf16", abs_slack=1e-5 * a)
             else:
                 assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
-                                 rel=1e-5, scale=a, what="fp8 f32")
+                                 rel=1e-5, scale=a, what="fp8 f32", max_slack_frac=FP8_F32_SLACK)
 
 
 # ---------------------------------------------------------------------------
