@@ -181,6 +181,19 @@ QMM_API const char *qmm_reorder_impl_name(const qmm_reorder_desc_t *desc);
 QMM_API int qmm_reorder_launch(const qmm_reorder_desc_t *desc,
         const qmm_reorder_args_t *args, void *hip_stream);
 
+/* ---- tuning / test hooks ----
+ * Process-wide kernel-selection overrides for A/B measurements and for tests
+ * that must reach a particular kernel at sizes the oracle finishes quickly.
+ * Atomic; a launch reads each once. Production code leaves them alone.
+ *   gemm variant: 0 by problem size (default); 1..3 a tile configuration of
+ *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible
+ *   w4a8 variant: 0 by problem size (default); 1..3 a tile configuration
+ *   b8x variant: MFMA shape of the 256 x 256 kernels: 1 = 16 x 16 (default),
+ *     0 = 32 x 32 */
+QMM_API void qmm_set_gemm_variant(int v);
+QMM_API void qmm_set_w4a8_variant(int v);
+QMM_API void qmm_set_b8x_variant(int v);
+
 /* ---- device queries used by the engine ---- */
 QMM_API int qmm_device_count(void);
 QMM_API const char *qmm_last_error(void);

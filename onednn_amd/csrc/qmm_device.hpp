@@ -239,71 +239,126 @@ QMM_D float hardsigmoid_f(float s, float alpha, float beta) {
     return v <= 0.f ? 0.f : v >= 1.f ? 1.f : v;
 }
 
-QMM_D float eltwise_fwd(int alg, float s, float alpha, float beta) {
+// One definition per algorithm (eltwise_one / binary_one); the scalar and the
+// four-element dispatchers below are generated from the same lists, so they
+// cannot drift apart. The *_use_dst_for_bwd aliases compute their base
+// algorithm's forward formula.
+template <int ALG>
+QMM_D float eltwise_one(float s, float alpha, float beta) {
+    if constexpr (ALG == alg_relu) {
+        return s > 0 ? s : s * alpha;
+    } else if constexpr (ALG == alg_tanh) {
+        return tanhf(s);
+    } else if constexpr (ALG == alg_elu) {
+        return s > 0 ? s : alpha * expm1f(s);
+    } else if constexpr (ALG == alg_square) {
+        return s * s;
+    } else if constexpr (ALG == alg_abs) {
+        return s > 0 ? s : -s;
+    } else if constexpr (ALG == alg_sqrt) {
+        return sqrtf(s);
+    } else if constexpr (ALG == alg_linear) {
+        return alpha * s + beta;
+    } else if constexpr (ALG == alg_soft_relu) {
+        return soft_relu_f(s, alpha);
+    } else if constexpr (ALG == alg_hardsigmoid) {
+        return hardsigmoid_f(s, alpha, beta);
+    } else if constexpr (ALG == alg_logistic) {
+        return logistic_f(s);
+    } else if constexpr (ALG == alg_exp) {
+        return expf(s);
+    } else if constexpr (ALG == alg_gelu_tanh) {
+        const float sqrt_2_over_pi = 0.79788458347320556640625f;
+        const float fitting_const = 0.044715f;
+        const float v = tanhf(sqrt_2_over_pi * s * (1 + fitting_const * s * s));
+        return (float)(0.5 * s * (1. + v));
+    } else if constexpr (ALG == alg_swish) {
+        return s * logistic_f(alpha * s);
+    } else if constexpr (ALG == alg_log) {
+        return logf(s);
+    } else if constexpr (ALG == alg_clip) {
+        s = s > alpha ? s : alpha;
+        return s > beta ? beta : s;
+    } else if constexpr (ALG == alg_clip_v2) {
+        s = s > alpha ? s : alpha;
+        return s < beta ? s : beta;
+    } else if constexpr (ALG == alg_pow) {
+        return alpha * powf(s, beta);
+    } else if constexpr (ALG == alg_gelu_erf) {
+        const float sqrt_2_over_2 = 0.707106769084930419921875f;
+        const float v = s * sqrt_2_over_2;
+        return 0.5f * s * (1.f + erff(v));
+    } else if constexpr (ALG == alg_round) {
+        return __builtin_rintf(s);
+    } else if constexpr (ALG == alg_mish) {
+        return s * tanhf(soft_relu_f(s, 1.f));
+    } else {
+        static_assert(ALG == alg_hardswish, "unknown eltwise algorithm");
+        return s * hardsigmoid_f(s, alpha, beta);
+    }
+}
+// X(algorithm, rows of a four-element group computed by inlined copies): the
+// long library routines keep one copy in a loop
+#define QMM_ELTWISE_LIST(X) \
+    X(alg_relu, 4) X(alg_tanh, 1) X(alg_elu, 1) X(alg_square, 4) X(alg_abs, 4) \
+    X(alg_sqrt, 4) X(alg_linear, 4) X(alg_soft_relu, 1) X(alg_hardsigmoid, 4) \
+    X(alg_logistic, 4) X(alg_exp, 4) X(alg_gelu_tanh, 1) X(alg_swish, 4) \
+    X(alg_log, 1) X(alg_clip, 4) X(alg_clip_v2, 4) X(alg_pow, 1) \
+    X(alg_gelu_erf, 1) X(alg_round, 4) X(alg_mish, 1) X(alg_hardswish, 4)
+
+QMM_D int eltwise_base_alg(int alg) {
     switch (alg) {
-        case alg_relu:
-        case alg_relu_dst: return s > 0 ? s : s * alpha;
-        case alg_tanh:
-        case alg_tanh_dst: return tanhf(s);
-        case alg_elu:
-        case alg_elu_dst: return s > 0 ? s : alpha * expm1f(s);
-        case alg_square: return s * s;
-        case alg_abs: return s > 0 ? s : -s;
-        case alg_sqrt:
-        case alg_sqrt_dst: return sqrtf(s);
-        case alg_linear: return alpha * s + beta;
-        case alg_soft_relu: return soft_relu_f(s, alpha);
-        case alg_hardsigmoid: return hardsigmoid_f(s, alpha, beta);
-        case alg_logistic:
-        case alg_logistic_dst: return logistic_f(s);
-        case alg_exp:
-        case alg_exp_dst: return expf(s);
-        case alg_gelu_tanh: {
-            const float sqrt_2_over_pi = 0.79788458347320556640625f;
-            const float fitting_const = 0.044715f;
-            const float v = tanhf(
-                    sqrt_2_over_pi * s * (1 + fitting_const * s * s));
-            return (float)(0.5 * s * (1. + v));
-        }
-        case alg_swish: return s * logistic_f(alpha * s);
-        case alg_log: return logf(s);
-        case alg_clip: {
-            s = s > alpha ? s : alpha;
-            return s > beta ? beta : s;
-        }
-        case alg_clip_v2:
-        case alg_clip_v2_dst: {
-            s = s > alpha ? s : alpha;
-            return s < beta ? s : beta;
-        }
-        case alg_pow: return alpha * powf(s, beta);
-        case alg_gelu_erf: {
-            const float sqrt_2_over_2 = 0.707106769084930419921875f;
-            const float v = s * sqrt_2_over_2;
-            return 0.5f * s * (1.f + erff(v));
-        }
-        case alg_round: return __builtin_rintf(s);
-        case alg_mish: return s * tanhf(soft_relu_f(s, 1.f));
-        case alg_hardswish: return s * hardsigmoid_f(s, alpha, beta);
+        case alg_relu_dst: return alg_relu;
+        case alg_tanh_dst: return alg_tanh;
+        case alg_elu_dst: return alg_elu;
+        case alg_sqrt_dst: return alg_sqrt;
+        case alg_logistic_dst: return alg_logistic;
+        case alg_exp_dst: return alg_exp;
+        case alg_clip_v2_dst: return alg_clip_v2;
+        default: return alg;
+    }
+}
+
+QMM_D float eltwise_fwd(int alg, float s, float alpha, float beta) {
+    switch (eltwise_base_alg(alg)) {
+#define QMM_X(A, U) \
+    case A: return eltwise_one<A>(s, alpha, beta);
+        QMM_ELTWISE_LIST(QMM_X)
+#undef QMM_X
         default: return u2f(0x7fc00000u);
     }
 }
 
 // src/cpu/primitive_attr_postops.cpp:29-46
+template <int ALG>
+QMM_D float binary_one(float x, float y) {
+    if constexpr (ALG == alg_bin_add) return x + y;
+    else if constexpr (ALG == alg_bin_div) return x / y;
+    else if constexpr (ALG == alg_bin_max) return x > y ? x : y;
+    else if constexpr (ALG == alg_bin_min) return x < y ? x : y;
+    else if constexpr (ALG == alg_bin_mul) return x * y;
+    else if constexpr (ALG == alg_bin_sub) return x - y;
+    else if constexpr (ALG == alg_bin_ge) return x >= y;
+    else if constexpr (ALG == alg_bin_gt) return x > y;
+    else if constexpr (ALG == alg_bin_le) return x <= y;
+    else if constexpr (ALG == alg_bin_lt) return x < y;
+    else if constexpr (ALG == alg_bin_eq) return x == y;
+    else {
+        static_assert(ALG == alg_bin_ne, "unknown binary algorithm");
+        return x != y;
+    }
+}
+#define QMM_BINARY_LIST(X) \
+    X(alg_bin_add) X(alg_bin_mul) X(alg_bin_max) X(alg_bin_min) X(alg_bin_div) \
+    X(alg_bin_sub) X(alg_bin_ge) X(alg_bin_gt) X(alg_bin_le) X(alg_bin_lt) \
+    X(alg_bin_eq) X(alg_bin_ne)
+
 QMM_D float binary_op(int alg, float x, float y) {
     switch (alg) {
-        case alg_bin_add: return x + y;
-        case alg_bin_div: return x / y;
-        case alg_bin_max: return x > y ? x : y;
-        case alg_bin_min: return x < y ? x : y;
-        case alg_bin_mul: return x * y;
-        case alg_bin_sub: return x - y;
-        case alg_bin_ge: return x >= y;
-        case alg_bin_gt: return x > y;
-        case alg_bin_le: return x <= y;
-        case alg_bin_lt: return x < y;
-        case alg_bin_eq: return x == y;
-        case alg_bin_ne: return x != y;
+#define QMM_X(A) \
+    case A: return binary_one<A>(x, y);
+        QMM_BINARY_LIST(QMM_X)
+#undef QMM_X
         default: return u2f(0x7fc00000u);
     }
 }
@@ -400,60 +455,40 @@ QMM_D void epilogue_apply_store(const epilogue_t &ep, float acc, int64_t b,
 
 // Four elements per dispatch: the algorithm switch is taken once per row piece
 // instead of once per element (the kernels are otherwise busy jumping).
-#define QMM_ELT4(expr) \
-    { \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) { \
-            const float s = d[i]; \
-            d[i] = (expr)*scale; \
-        } \
-    } \
-    break;
+#define QMM_PRAGMA(x) _Pragma(#x)
 QMM_D void eltwise_fwd4(int alg, float (&d)[4], float alpha, float beta,
         float scale) {
-    switch (alg) {
-        case alg_relu:
-        case alg_relu_dst: QMM_ELT4(s > 0 ? s : s * alpha)
-        case alg_swish: QMM_ELT4(s * logistic_f(alpha * s))
-        case alg_logistic:
-        case alg_logistic_dst: QMM_ELT4(logistic_f(s))
-        case alg_linear: QMM_ELT4(alpha * s + beta)
-        case alg_tanh:
-        case alg_tanh_dst: QMM_ELT4(tanhf(s))
-        case alg_gelu_tanh: QMM_ELT4(eltwise_fwd(alg_gelu_tanh, s, alpha, beta))
-        case alg_gelu_erf: QMM_ELT4(eltwise_fwd(alg_gelu_erf, s, alpha, beta))
-        case alg_clip: QMM_ELT4(eltwise_fwd(alg_clip, s, alpha, beta))
-        case alg_clip_v2:
-        case alg_clip_v2_dst: QMM_ELT4(eltwise_fwd(alg_clip_v2, s, alpha, beta))
-        case alg_hardswish: QMM_ELT4(s * hardsigmoid_f(s, alpha, beta))
-        case alg_hardsigmoid: QMM_ELT4(hardsigmoid_f(s, alpha, beta))
-        case alg_abs: QMM_ELT4(s > 0 ? s : -s)
-        case alg_square: QMM_ELT4(s * s)
-        case alg_exp:
-        case alg_exp_dst: QMM_ELT4(expf(s))
-        default: QMM_ELT4(eltwise_fwd(alg, s, alpha, beta))
+    switch (eltwise_base_alg(alg)) {
+#define QMM_X(A, U) \
+    case A: \
+        QMM_PRAGMA(unroll U) for (int i = 0; i < 4; i++) d[i] \
+                = eltwise_one<A>(d[i], alpha, beta) * scale; \
+        break;
+        QMM_ELTWISE_LIST(QMM_X)
+#undef QMM_X
+        default:
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] = u2f(0x7fc00000u);
+            break;
     }
 }
-#undef QMM_ELT4
-#define QMM_BIN4(expr) \
-    { \
-        _Pragma("unroll") for (int i = 0; i < 4; i++) { \
-            const float x = d[i], y = o[i]; \
-            d[i] = (expr); \
-        } \
-    } \
-    break;
 QMM_D void binary_op4(int alg, float (&d)[4], const float (&o)[4]) {
     switch (alg) {
-        case alg_bin_add: QMM_BIN4(x + y)
-        case alg_bin_mul: QMM_BIN4(x * y)
-        case alg_bin_sub: QMM_BIN4(x - y)
-        case alg_bin_max: QMM_BIN4(x > y ? x : y)
-        case alg_bin_min: QMM_BIN4(x < y ? x : y)
-        case alg_bin_div: QMM_BIN4(x / y)
-        default: QMM_BIN4(binary_op(alg, x, y))
+#define QMM_X(A) \
+    case A: \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) d[i] \
+                = binary_one<A>(d[i], o[i]); \
+        break;
+        QMM_BINARY_LIST(QMM_X)
+#undef QMM_X
+        default:
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                d[i] = u2f(0x7fc00000u);
+            break;
     }
 }
-#undef QMM_BIN4
 
 // ---- the same tail for four consecutive n at once (n % 4 == 0) -------------
 // The tiled kernels hand their results over row-wise: a lane owns 4 neighbouring

@@ -5,6 +5,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -463,8 +464,16 @@ int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
         if (P.q_wei_scale.g1 != 1) return QMM_UNIMPLEMENTED; // N groups
     }
     if (wz.set) {
-        if (!one_of(wz.dt, {dt_s32, dt_s8, dt_u8, dt_s4, dt_u4}))
+        // The kernels keep 16 * sum s * (w - z) of a group in s32 (the weights
+        // enter the MFMA as 16 w') and apply the zero point through the
+        // group's source row sum with a 24-bit multiply. That sum is bounded by
+        // 16 * 128 * max|w - z| * gk: within s32 for 4-bit zero points at every
+        // group size taken here (|w - z| <= 23, gk <= 32768), for 8-bit ones
+        // (|w - z| <= 255) up to gk = 3968; s32 zero points have no bound.
+        // The rest goes to the generic implementation.
+        if (!one_of(wz.dt, {dt_s8, dt_u8, dt_s4, dt_u4}))
             return QMM_UNIMPLEMENTED;
+        if (one_of(wz.dt, {dt_s8, dt_u8}) && gk > 3968) return QMM_UNIMPLEMENTED;
         if (P.q_wei_zp.g1 != 1) return QMM_UNIMPLEMENTED;
     }
     epilogue_t ep;
@@ -609,8 +618,8 @@ int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
 const char *impl_names[impl_count] = {"hip:gfx950:mfma_b8",
         "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:generic"};
 
-int g_gemm_variant = 0;
-int g_w4a8_variant = 0;
+std::atomic<int> g_gemm_variant {0};
+std::atomic<int> g_w4a8_variant {0};
 
 } // namespace
 
@@ -837,6 +846,11 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
     if (plan->scratch_bytes && !args->scratch)
         return fail(QMM_INVALID_ARGUMENTS, "scratch buffer is missing");
 
+    // one read per launch: a launch never sees two values of a tuning hook
+    const int gemm_variant = g_gemm_variant.load(std::memory_order_relaxed);
+    const int w4a8_variant = g_w4a8_variant.load(std::memory_order_relaxed);
+    (void)gemm_variant;
+    (void)w4a8_variant;
     int impl = plan->impl;
     if (impl != impl_generic && !aligned16(args->src)) {
         if (!plan->dev)
@@ -891,13 +905,13 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             h.lda = P.K;
             h.a_sb = P.M * P.K;
             h.a_preflipped = 1;
-            if (gemm_b8_uses_tile256(h, f8, g_gemm_variant)) {
+            if (gemm_b8_uses_tile256(h, f8, gemm_variant)) {
                 launch_flip_u8(g.A, copy, P.batch, P.M, P.K, g.lda, g.a_sb,
                         stream);
                 g = h;
             }
         }
-        launch_gemm_b8(g, f8, g_gemm_variant, stream);
+        launch_gemm_b8(g, f8, gemm_variant, stream);
     } else if (impl == impl_gemm_w4a8) {
         w4a8_params_t g;
         std::memset(&g, 0, sizeof(g));
@@ -946,7 +960,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         q.swT = (float *)(arrays + sc.sw_off);
         q.rsT = sc.has_zp ? (int32_t *)(arrays + sc.rs_off) : nullptr;
         q.zwT = sc.has_zp ? (int32_t *)(arrays + sc.zw_off) : nullptr;
-        const w4a8_small_plan_t sm = w4a8_small_plan(P, g_w4a8_variant);
+        const w4a8_small_plan_t sm = w4a8_small_plan(P, w4a8_variant);
         if (sm.use && gemm_w4a8_small_takes(q)) {
             w4a8_small_t h;
             std::memset(&h, 0, sizeof(h));
@@ -1000,7 +1014,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.nb32 = (int32_t)geom.nb32;
         g.tpg = q.gk / 64;
         g.ng = q.ng;
-        launch_gemm_w4a8(g, g_w4a8_variant, stream);
+        launch_gemm_w4a8(g, w4a8_variant, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;
         std::memset(&g, 0, sizeof(g));
@@ -1043,7 +1057,10 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
     return QMM_OK;
 }
 
-// tuning hook used by the benchmark sweep: tile configuration of mfma_b8
+// Tuning / test hooks (declared in qmm_hip.h): process-wide, atomic, read once
+// per launch. The default of each (0, 0, 1) is what the implementations are
+// tuned and documented for.
+// tile configuration of mfma_b8
 QMM_API void qmm_set_gemm_variant(int v) {
     g_gemm_variant = v;
 }

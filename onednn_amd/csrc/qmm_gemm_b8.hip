@@ -375,12 +375,7 @@ static void launch_cfg(const gemm_params_t &p, hipStream_t stream) {
             = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
     constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
     auto kern = gemm_b8_kernel<BM, BN, BK, WGM, WGN, STAGES, F8, U8A>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void *)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_done = true;
-    }
+    ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(WGM * WGN * 64), lds,
             stream, q);
 }

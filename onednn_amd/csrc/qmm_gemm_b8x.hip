@@ -29,6 +29,7 @@
 // arithmetic as src/cpu/matmul/ref_matmul_int8.cpp:195-259); only epilogues of
 // the straight-line kinds (EP_FAST_*) are handled here, everything else stays
 // with the general kernel.
+#include <atomic>
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -1436,20 +1437,7 @@ static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ((ntiles + 7) / 8) * 8;
-    // one attribute call per kernel (the kernels share this function's type)
-    static const void *done[12] = {};
-    bool seen = false;
-    for (const void *d : done)
-        seen = seen || d == (const void *)kern;
-    if (!seen) {
-        (void)hipFuncSetAttribute((const void *)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-        for (const void *&d : done)
-            if (!d) {
-                d = (const void *)kern;
-                break;
-            }
-    }
+    ensure_dynamic_lds((const void *)kern, LDS_TOTAL);
     hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(NT), LDS_TOTAL,
             stream, q);
 }
@@ -1509,19 +1497,20 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
 
 // 0: the loops on 32 x 32 MFMAs; 1: int8 on 16 x 16 x 64 (at least 5 k-steps)
 // and fp8 on 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply
-static int g_b8x_variant = 1;
+static std::atomic<int> g_b8x_variant {1};
 void set_gemm_b8x_variant(int v) {
     g_b8x_variant = v;
 }
 
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
-    if (f8 && g_b8x_variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
+    const int variant = g_b8x_variant.load(std::memory_order_relaxed);
+    if (f8 && variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)
         launch_b8x_fp8(p, stream);
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
-    else if (g_b8x_variant >= 1 && p.K >= 5 * 64) {
+    else if (variant >= 1 && p.K >= 5 * 64) {
         if ((p.K / 64) & 1)
             launch_b8x_int8_mi16_odd(p, stream);
         else

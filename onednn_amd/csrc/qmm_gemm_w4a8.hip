@@ -934,12 +934,7 @@ template <int NWV, int SC, bool HAS_ZP, int ZPK>
 static void launch_tiny_cfg(const w4a8_small_t &p, hipStream_t stream) {
     constexpr size_t lds = (size_t)NWV * TN_WAVE_BYTES + NWV * 4 * 32 * 4;
     auto kern = w4a8_tiny_kernel<NWV, SC, HAS_ZP, ZPK>;
-    static bool attr_done = false; // one per instantiation
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void *)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_done = true;
-    }
+    ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3((p.q.N + 31) / 32), dim3(NWV * 64), lds,
             stream, p);
 }
@@ -1002,12 +997,7 @@ static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
             + (size_t)W4A8_SMALL_MAX_GPS * (BM * 4 + 128 * 4 + 128 * 4)
             + 4 * BM * 4;
     auto kern = w4a8_small_kernel<FM, SC, HAS_ZP, ZPK>;
-    static bool attr_done = false; // one per instantiation
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void *)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_done = true;
-    }
+    ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern,
             dim3((p.q.N + 127) / 128, p.splits, (p.q.M + BM - 1) / BM),
             dim3(256), lds, stream, p);
@@ -1042,12 +1032,7 @@ static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
             = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
     constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
     auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, HAS_ZP>;
-    static bool attr_done = false; // one per instantiation
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void *)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_done = true;
-    }
+    ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3(grid_x), dim3(WGM * WGN * 64), lds, stream, q);
 }
 

@@ -603,21 +603,7 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         return;
     }
     auto launch = [&](auto kern) {
-        // (the two kernels share this lambda's type: one call each)
-        static const void *done[2] = {};
-        bool seen = false;
-        for (const void *d : done)
-            seen = seen || d == (const void *)kern;
-        if (!seen) {
-            (void)hipFuncSetAttribute((const void *)kern,
-                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                    GEMV_LDS_BUDGET);
-            for (const void *&d : done)
-                if (!d) {
-                    d = (const void *)kern;
-                    break;
-                }
-        }
+        ensure_dynamic_lds((const void *)kern, GEMV_LDS_BUDGET);
         hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, q,
                 MR, KC);
     };

@@ -5,10 +5,26 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "qmm_device.hpp"
 #include "qmm_hip.h"
 
 namespace qmm {
+
+// Raises a kernel's dynamic LDS limit once per kernel; safe to call from
+// several host threads that launch concurrently.
+inline void ensure_dynamic_lds(const void *kern, int bytes) {
+    static std::mutex mu;
+    static const void *seen[96];
+    static int n = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < n; i++)
+        if (seen[i] == kern) return;
+    (void)hipFuncSetAttribute(
+            kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (n < 96) seen[n++] = kern;
+}
 
 // A scales / zero-points buffer as the generic kernels index it: dense
 // row-major over the masked dims, last two dims divided by the groups

@@ -217,3 +217,50 @@ def test_w4a8_prepack_round_trip(ctx):
         dnnl.reorder(packed, back).execute(strm, packed, back)
         strm.wait()
         assert np.array_equal(t.logical(back.read(t.raw.dtype)), t.logical()), (code, dims, layout)
+
+
+def _extreme_zero_point(K, gk, zp_value=255):
+    """Saturated activations against the largest u8 zero point: the group sum
+    16 * sum s * (w - z) reaches 16 * 127 * 255 * gk."""
+    M, N = 8, 64
+    r = np.random.default_rng(77)
+    s = np.full((M, K), 127)
+    s[1::2] = -128
+    w = r.integers(0, 16, (K, N))
+    src = TensorSpec(dt.s8, [M, K], None, s)
+    wei = TensorSpec(dt.u4, [K, N], "ab", w)
+    dst = TensorSpec(dt.f32, [M, N])
+    scales = {"src": (3, dt.f32, (1, gk), np.full((M, K // gk), 2.0 ** -20)),
+              "wei": (3, dt.f32, (gk, 1), np.full((K // gk, N), 2.0 ** -8))}
+    zps = {"wei": (3, dt.u8, (gk, 1), np.full((K // gk, N), zp_value))}
+    return Problem(src, wei, dst, scales=scales, zps=zps)
+
+
+def test_w4a8_largest_8bit_zero_point_stays_in_s32(ctx):
+    """u8 zero point 255 with saturated activations: the largest group the
+    MFMA implementation takes with 8-bit zero points (3968) is exact; a group of
+    4096 would leave s32 in its 16 x scaled sums and goes to the generic
+    implementation, which is exact as well."""
+    eng, strm = ctx
+    say("mfma_w4a8 u8 zp=255, gk=3968 (MFMA) and gk=4096 (generic)")
+    p = _extreme_zero_point(3968, 3968)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == W4A8
+    assert_bit_exact(got, p.run_oracle(), "gk 3968")
+    # closed form: one group, (float)s32 rounds to nearest even, the scales are powers of two
+    acc = p.src.logical().astype(np.int64) @ (p.wei.logical().astype(np.int64) - 255)
+    assert 2 ** 30 < np.abs(acc).max() * 16 < 2 ** 31  # the 16 x scaled sum is within 5 % of the s32 range
+    assert np.array_equal(got.view(np.float32).reshape(8, 64), acc.astype(np.float32) * np.float32(2.0 ** -28))
+    p = _extreme_zero_point(4096, 4096)
+    got, pd = p.run_gpu(eng, strm, return_pd=True)
+    assert pd.impl_info_str() == GENERIC
+    assert_bit_exact(got, p.run_oracle(), "gk 4096")
+
+
+def test_w4a8_s32_zero_points_go_to_generic(ctx):
+    eng, strm = ctx
+    say("mfma_w4a8 refuses s32 zero points")
+    p = dynamic_quant(16, 256, 64, 5, wei_dt=dt.u4, gz=128, zp_dt=dt.s32, exact=True)
+    got, pd = p.run_gpu(eng, strm, return_pd=True)
+    assert pd.impl_info_str() == GENERIC
+    assert_bit_exact(got, p.run_oracle(), "s32 zp")
