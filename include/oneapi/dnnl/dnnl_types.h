@@ -83,7 +83,9 @@ typedef enum {
     dnnl_abcdefghji = 49,
     dnnl_abcdefghikj = 50,
     dnnl_abcdefghijlk = 51,
-    dnnl_format_tag_last,
+    /* one past the last tag of oneDNN v3.8's full list (its blocked tags are not
+     * part of this subset): the same value as there */
+    dnnl_format_tag_last = 847,
     dnnl_x = dnnl_a,
     dnnl_nc = dnnl_ab,
     dnnl_cn = dnnl_ba,

@@ -12,6 +12,7 @@
 #include <new>
 
 #include "dnnl_objects.hpp"
+#include "oneapi/dnnl/dnnl_debug.h"
 
 namespace host {
 
@@ -926,4 +927,252 @@ dnnl_status_t dnnl_post_ops_get_params_prelu(
     return dnnl_success;
 }
 
+} // extern "C"
+
+// ---- enumerator names (include/oneapi/dnnl/dnnl_debug.h) --------------------
+// One switch per enumeration of the public headers: the enumerator's name
+// without its dnnl_ prefix, as the reference's generated
+// src/common/dnnl_debug_autogenerated.cpp returns it.
+extern "C" {
+const char *dnnl_status2str(dnnl_status_t v) {
+    switch ((int)v) {
+        case dnnl_success: return "success";
+        case dnnl_out_of_memory: return "out_of_memory";
+        case dnnl_invalid_arguments: return "invalid_arguments";
+        case dnnl_unimplemented: return "unimplemented";
+        case dnnl_last_impl_reached: return "last_impl_reached";
+        case dnnl_runtime_error: return "runtime_error";
+        case dnnl_not_required: return "not_required";
+        case dnnl_invalid_graph: return "invalid_graph";
+        case dnnl_invalid_graph_op: return "invalid_graph_op";
+        case dnnl_invalid_shape: return "invalid_shape";
+        case dnnl_invalid_data_type: return "invalid_data_type";
+        default: return "unknown status";
+    }
+}
+const char *dnnl_dt2str(dnnl_data_type_t v) {
+    switch ((int)v) {
+        case dnnl_data_type_undef: return "undef";
+        case dnnl_f16: return "f16";
+        case dnnl_bf16: return "bf16";
+        case dnnl_f32: return "f32";
+        case dnnl_s32: return "s32";
+        case dnnl_s8: return "s8";
+        case dnnl_u8: return "u8";
+        case dnnl_f64: return "f64";
+        case dnnl_boolean: return "boolean";
+        case dnnl_f8_e5m2: return "f8_e5m2";
+        case dnnl_f8_e4m3: return "f8_e4m3";
+        case dnnl_s4: return "s4";
+        case dnnl_u4: return "u4";
+        case dnnl_e8m0: return "e8m0";
+        case dnnl_f4_e2m1: return "f4_e2m1";
+        case dnnl_f4_e3m0: return "f4_e3m0";
+        default: return "unknown dt";
+    }
+}
+const char *dnnl_fpmath_mode2str(dnnl_fpmath_mode_t v) {
+    switch ((int)v) {
+        case dnnl_fpmath_mode_strict: return "strict";
+        case dnnl_fpmath_mode_bf16: return "bf16";
+        case dnnl_fpmath_mode_f16: return "f16";
+        case dnnl_fpmath_mode_any: return "any";
+        case dnnl_fpmath_mode_tf32: return "tf32";
+        default: return "unknown fpmath_mode";
+    }
+}
+const char *dnnl_accumulation_mode2str(dnnl_accumulation_mode_t v) {
+    switch ((int)v) {
+        case dnnl_accumulation_mode_strict: return "strict";
+        case dnnl_accumulation_mode_relaxed: return "relaxed";
+        case dnnl_accumulation_mode_any: return "any";
+        case dnnl_accumulation_mode_s32: return "s32";
+        case dnnl_accumulation_mode_f32: return "f32";
+        case dnnl_accumulation_mode_f16: return "f16";
+        default: return "unknown accumulation_mode";
+    }
+}
+const char *dnnl_engine_kind2str(dnnl_engine_kind_t v) {
+    switch ((int)v) {
+        case dnnl_any_engine: return "any";
+        case dnnl_cpu: return "cpu";
+        case dnnl_gpu: return "gpu";
+        default: return "unknown engine_kind";
+    }
+}
+const char *dnnl_fmt_tag2str(dnnl_format_tag_t v) {
+    switch ((int)v) {
+        case dnnl_format_tag_undef: return "undef";
+        case dnnl_format_tag_any: return "any";
+        case dnnl_a: return "a";
+        case dnnl_ab: return "ab";
+        case dnnl_abc: return "abc";
+        case dnnl_abcd: return "abcd";
+        case dnnl_abcde: return "abcde";
+        case dnnl_abcdef: return "abcdef";
+        case dnnl_abcdefg: return "abcdefg";
+        case dnnl_abcdefgh: return "abcdefgh";
+        case dnnl_abcdefghi: return "abcdefghi";
+        case dnnl_abcdefghij: return "abcdefghij";
+        case dnnl_abcdefghijk: return "abcdefghijk";
+        case dnnl_abcdefghijkl: return "abcdefghijkl";
+        case dnnl_ba: return "ba";
+        case dnnl_acb: return "acb";
+        case dnnl_bac: return "bac";
+        case dnnl_bca: return "bca";
+        case dnnl_cab: return "cab";
+        case dnnl_cba: return "cba";
+        case dnnl_abdc: return "abdc";
+        case dnnl_acbd: return "acbd";
+        case dnnl_acdb: return "acdb";
+        case dnnl_adbc: return "adbc";
+        case dnnl_adcb: return "adcb";
+        case dnnl_bacd: return "bacd";
+        case dnnl_bcda: return "bcda";
+        case dnnl_cdab: return "cdab";
+        case dnnl_cdba: return "cdba";
+        case dnnl_dcab: return "dcab";
+        case dnnl_abced: return "abced";
+        case dnnl_abdec: return "abdec";
+        case dnnl_acbde: return "acbde";
+        case dnnl_acdeb: return "acdeb";
+        case dnnl_adecb: return "adecb";
+        case dnnl_bacde: return "bacde";
+        case dnnl_bcdea: return "bcdea";
+        case dnnl_cdeab: return "cdeab";
+        case dnnl_cdeba: return "cdeba";
+        case dnnl_decab: return "decab";
+        case dnnl_abcdfe: return "abcdfe";
+        case dnnl_abdefc: return "abdefc";
+        case dnnl_abdfce: return "abdfce";
+        case dnnl_acbdef: return "acbdef";
+        case dnnl_adefcb: return "adefcb";
+        case dnnl_defcab: return "defcab";
+        case dnnl_abcdegf: return "abcdegf";
+        case dnnl_abcdefhg: return "abcdefhg";
+        case dnnl_abcdefgih: return "abcdefgih";
+        case dnnl_abcdefghji: return "abcdefghji";
+        case dnnl_abcdefghikj: return "abcdefghikj";
+        case dnnl_abcdefghijlk: return "abcdefghijlk";
+        default: return "unknown fmt_tag";
+    }
+}
+const char *dnnl_prop_kind2str(dnnl_prop_kind_t v) {
+    switch ((int)v) {
+        case dnnl_prop_kind_undef: return "undef";
+        case dnnl_forward_training: return "forward_training";
+        case dnnl_forward_inference: return "forward_inference";
+        default: return "unknown prop_kind";
+    }
+}
+const char *dnnl_prim_kind2str(dnnl_primitive_kind_t v) {
+    switch ((int)v) {
+        case dnnl_undefined_primitive: return "undef";
+        case dnnl_reorder: return "reorder";
+        case dnnl_shuffle: return "shuffle";
+        case dnnl_concat: return "concat";
+        case dnnl_sum: return "sum";
+        case dnnl_convolution: return "convolution";
+        case dnnl_deconvolution: return "deconvolution";
+        case dnnl_eltwise: return "eltwise";
+        case dnnl_lrn: return "lrn";
+        case dnnl_batch_normalization: return "batch_normalization";
+        case dnnl_inner_product: return "inner_product";
+        case dnnl_rnn: return "rnn";
+        case dnnl_gemm: return "gemm";
+        case dnnl_binary: return "binary";
+        case dnnl_matmul: return "matmul";
+        case dnnl_resampling: return "resampling";
+        case dnnl_pooling: return "pooling";
+        case dnnl_reduction: return "reduction";
+        case dnnl_prelu: return "prelu";
+        case dnnl_softmax: return "softmax";
+        case dnnl_layer_normalization: return "layer_normalization";
+        case dnnl_group_normalization: return "group_normalization";
+        default: return "unknown prim_kind";
+    }
+}
+const char *dnnl_alg_kind2str(dnnl_alg_kind_t v) {
+    switch ((int)v) {
+        case dnnl_alg_kind_undef: return "undef";
+        case dnnl_eltwise_relu: return "eltwise_relu";
+        case dnnl_eltwise_tanh: return "eltwise_tanh";
+        case dnnl_eltwise_elu: return "eltwise_elu";
+        case dnnl_eltwise_square: return "eltwise_square";
+        case dnnl_eltwise_abs: return "eltwise_abs";
+        case dnnl_eltwise_sqrt: return "eltwise_sqrt";
+        case dnnl_eltwise_linear: return "eltwise_linear";
+        case dnnl_eltwise_soft_relu: return "eltwise_soft_relu";
+        case dnnl_eltwise_hardsigmoid: return "eltwise_hardsigmoid";
+        case dnnl_eltwise_logistic: return "eltwise_logistic";
+        case dnnl_eltwise_exp: return "eltwise_exp";
+        case dnnl_eltwise_gelu_tanh: return "eltwise_gelu_tanh";
+        case dnnl_eltwise_swish: return "eltwise_swish";
+        case dnnl_eltwise_log: return "eltwise_log";
+        case dnnl_eltwise_clip: return "eltwise_clip";
+        case dnnl_eltwise_clip_v2: return "eltwise_clip_v2";
+        case dnnl_eltwise_pow: return "eltwise_pow";
+        case dnnl_eltwise_gelu_erf: return "eltwise_gelu_erf";
+        case dnnl_eltwise_round: return "eltwise_round";
+        case dnnl_eltwise_mish: return "eltwise_mish";
+        case dnnl_eltwise_hardswish: return "eltwise_hardswish";
+        case dnnl_eltwise_relu_use_dst_for_bwd: return "eltwise_relu_use_dst_for_bwd";
+        case dnnl_eltwise_tanh_use_dst_for_bwd: return "eltwise_tanh_use_dst_for_bwd";
+        case dnnl_eltwise_elu_use_dst_for_bwd: return "eltwise_elu_use_dst_for_bwd";
+        case dnnl_eltwise_sqrt_use_dst_for_bwd: return "eltwise_sqrt_use_dst_for_bwd";
+        case dnnl_eltwise_logistic_use_dst_for_bwd: return "eltwise_logistic_use_dst_for_bwd";
+        case dnnl_eltwise_exp_use_dst_for_bwd: return "eltwise_exp_use_dst_for_bwd";
+        case dnnl_eltwise_clip_v2_use_dst_for_bwd: return "eltwise_clip_v2_use_dst_for_bwd";
+        case dnnl_binary_add: return "binary_add";
+        case dnnl_binary_mul: return "binary_mul";
+        case dnnl_binary_max: return "binary_max";
+        case dnnl_binary_min: return "binary_min";
+        case dnnl_binary_div: return "binary_div";
+        case dnnl_binary_sub: return "binary_sub";
+        case dnnl_binary_ge: return "binary_ge";
+        case dnnl_binary_gt: return "binary_gt";
+        case dnnl_binary_le: return "binary_le";
+        case dnnl_binary_lt: return "binary_lt";
+        case dnnl_binary_eq: return "binary_eq";
+        case dnnl_binary_ne: return "binary_ne";
+        case dnnl_binary_select: return "binary_select";
+        default: return "unknown alg_kind";
+    }
+}
+const char *dnnl_scratchpad_mode2str(dnnl_scratchpad_mode_t v) {
+    switch ((int)v) {
+        case dnnl_scratchpad_mode_library: return "library";
+        case dnnl_scratchpad_mode_user: return "user";
+        default: return "unknown scratchpad_mode";
+    }
+}
+const char *dnnl_rounding_mode2str(dnnl_rounding_mode_t v) {
+    switch ((int)v) {
+        case dnnl_rounding_mode_environment: return "environment";
+        case dnnl_rounding_mode_stochastic: return "stochastic";
+        default: return "unknown rounding_mode";
+    }
+}
+const char *dnnl_fmt_kind2str(dnnl_format_kind_t v) {
+    switch ((int)v) {
+        case dnnl_format_kind_undef: return "undef";
+        case dnnl_format_kind_any: return "any";
+        case dnnl_blocked: return "blocked";
+        case dnnl_format_kind_opaque: return "opaque";
+        default: return "unknown fmt_kind";
+    }
+}
+const char *dnnl_runtime2str(unsigned v) {
+    switch (v) {
+        case DNNL_RUNTIME_NONE: return "none";
+        case DNNL_RUNTIME_SEQ: return "sequential";
+        case DNNL_RUNTIME_OMP: return "OpenMP";
+        case DNNL_RUNTIME_TBB: return "TBB";
+        case DNNL_RUNTIME_THREADPOOL: return "threadpool";
+        case DNNL_RUNTIME_OCL: return "OpenCL";
+        case DNNL_RUNTIME_SYCL: return "DPC++";
+        case DNNL_RUNTIME_HIP: return "HIP";
+        default: return "unknown";
+    }
+}
 } // extern "C"
