@@ -577,6 +577,9 @@ constexpr size_t RT_CACHE_ENTRIES = 16;
 
 bool rt_md_matches(const dnnl_memory_desc &want, const dnnl_memory_desc &got) {
     if (got.ndims != want.ndims || got.data_type != want.data_type) return false;
+    // prepacked weights (all dims known): the very descriptor the primitive
+    // descriptor reports
+    if (!want.is_plain()) return md_equal(want, got);
     if (!got.is_plain() || got.has_runtime_dims()) return false;
     for (int d = 0; d < want.ndims; d++) {
         if (want.dims[d] != DNNL_RUNTIME_DIM_VAL && want.dims[d] != got.dims[d])
@@ -697,17 +700,49 @@ dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *out,
             {&pd->user_src, &pd->user_wei, &pd->user_bias, &pd->user_dst})
         runtime = runtime || (md->ndims && md->has_runtime_dims());
     if (runtime) {
-        // format any cannot be resolved without the dims
-        // (src/common/matmul_pd.hpp:266-277); everything that depends on the
-        // dims is decided per shape at execution
+        // format any cannot be resolved on a descriptor that has runtime dims
+        // itself (src/common/matmul_pd.hpp:266-277); everything that depends
+        // on the dims is decided per shape at execution
         for (const dnnl_memory_desc *md :
-                {&pd->user_src, &pd->user_wei, &pd->user_bias, &pd->user_dst})
+                {&pd->user_src, &pd->user_bias, &pd->user_dst})
             if (md->ndims && !md->is_plain()) return dnnl_unimplemented;
         pd->runtime = true;
         pd->src = pd->user_src;
         pd->wei = pd->user_wei;
         pd->bias = pd->user_bias;
         pd->dst = pd->user_dst;
+        if (!pd->user_wei.is_plain()) {
+            // Weights whose own dims are all known may still be `any` or
+            // prepacked (the usual case: a linear layer with a run-time batch,
+            // examples/tutorials/matmul/inference_int8_matmul.cpp:104-125).
+            // The packed layout depends on K, N, the types and the attributes
+            // only: it is resolved here on a stand-in problem in which every
+            // runtime dim has a nominal value.
+            if (pd->user_wei.has_runtime_dims()) return dnnl_unimplemented;
+            if (!pd->user_wei.is_any() && !pd->user_wei.is_packed())
+                return dnnl_unimplemented;
+            pd_impl_t nominal = *pd;
+            nominal.runtime = false;
+            for (dnnl_memory_desc *md :
+                    {&nominal.user_src, &nominal.user_bias, &nominal.user_dst}) {
+                if (!md->ndims || !md->has_runtime_dims()) continue;
+                bool rt_strides = false;
+                for (int d = 0; d < md->ndims; d++) {
+                    if (md->dims[d] == DNNL_RUNTIME_DIM_VAL)
+                        md->dims[d] = d < md->ndims - 2 ? 4 : 256;
+                    rt_strides = rt_strides
+                            || md->strides[d] == DNNL_RUNTIME_DIM_VAL;
+                }
+                if (rt_strides) {
+                    dnnl_memory_desc r;
+                    md_init_plain(r, md->ndims, md->dims, md->data_type, nullptr);
+                    *md = r;
+                }
+            }
+            st = walk_matmul_impls(nominal, 0);
+            if (st != dnnl_success) return st;
+            pd->wei = nominal.wei;
+        }
         for (auto &e : pd->attr.post_ops.entries)
             if (e.kind == dnnl_binary) {
                 if (!e.user_src1_desc.is_plain()) return dnnl_unimplemented;

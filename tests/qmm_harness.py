@@ -196,24 +196,28 @@ class Problem:
                     raise RuntimeError("implementation %s does not take this problem" % impl)
         return pd
 
-    def runtime_primitive_desc(self, eng, runtime):
+    def runtime_primitive_desc(self, eng, runtime, weights_any=False):
         """`runtime`: {"src" / "wei" / "dst" / "bias": dim indices that become
-        DNNL_RUNTIME_DIM_VAL}; layouts must be tags."""
+        DNNL_RUNTIME_DIM_VAL}; layouts must be tags. weights_any: the weights
+        (all of their dims known) are given as format_tag::any."""
         def md(spec, name):
             dims = list(spec.dims)
             for i in runtime.get(name, ()):
                 dims[i] = dnnl.DNNL_RUNTIME_DIM_VAL
+            if name == "wei" and weights_any:
+                return memory.desc(dims, spec.dt, tag.any)
             return memory.desc(dims, spec.dt, T(spec.layout))
         return dnnl.matmul.primitive_desc(
             eng, md(self.src, "src"), md(self.wei, "wei"), md(self.dst, "dst"),
             bias_md=md(self.bias, "bias") if self.bias is not None else None, attr=self.attr())
 
     def run_gpu(self, eng, strm, weights_any=False, impl=None, dst_init=None,
-                scratchpad_user=False, return_pd=False, prim=None):
+                scratchpad_user=False, return_pd=False, prim=None, prim_wei_md=None):
         """`prim`: a primitive made from runtime_primitive_desc (its memory
-        objects then carry this problem's own descriptors)."""
+        objects then carry this problem's own descriptors; prim_wei_md: the
+        prepacked weights descriptor that primitive descriptor reports)."""
         if prim is not None:
-            pd = _ConcreteDescs(self)
+            pd = _ConcreteDescs(self, prim_wei_md)
         else:
             pd = self.primitive_desc(eng, weights_any, impl, scratchpad_user)
             prim = dnnl.matmul(pd)
@@ -261,14 +265,15 @@ class _ConcreteDescs:
     """Stands in for a primitive descriptor when the primitive was created with
     runtime dims: the descriptors are the problem's own."""
 
-    def __init__(self, p):
+    def __init__(self, p, wei_md=None):
         self.p = p
+        self.wei_md = wei_md
 
     def src_desc(self):
         return self.p.src.md()
 
     def weights_desc(self):
-        return self.p.wei.md()
+        return self.wei_md if self.wei_md is not None else self.p.wei.md()
 
     def dst_desc(self):
         return self.p.dst.md()

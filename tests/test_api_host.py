@@ -415,8 +415,14 @@ def test_runtime_dims_descriptor(eng):
     assert pd.dst_desc() == dst
     assert pd.scratchpad_desc().is_zero()
     assert not pd.next_impl()
+    # format any: refused on a descriptor that has runtime dims itself, resolved on
+    # weights whose own dims are known (src/common/matmul_pd.hpp:266-277,
+    # examples/tutorials/matmul/inference_int8_matmul.cpp:104-125)
     expect(status.unimplemented, lambda: dnnl.matmul.primitive_desc(
-        eng, src, memory.desc([256, 128], dt.s8, tag.any), dst))
+        eng, memory.desc([R, 256], dt.s8, tag.any), wei, dst))
+    pd_any = dnnl.matmul.primitive_desc(eng, src, memory.desc([256, 128], dt.s8, tag.any), dst)
+    assert pd_any.impl_info_str() == "hip:gfx950:runtime_dims"
+    assert pd_any.weights_desc().get_format_kind() == memory.format_kind.opaque
     expect(status.invalid_arguments, lambda: dnnl.matmul.primitive_desc(
         eng, memory.desc([R, 8, 256], dt.s8, T("abc")), memory.desc([4, 256, 128], dt.s8, T("abc")),
         memory.desc([R, 8, 128], dt.f32, T("abc"))))

@@ -32,6 +32,23 @@ def test_runtime_m_one_primitive_many_batch_sizes(ctx):
         assert_bit_exact(p.run_gpu(eng, strm, prim=prim), p.run_oracle(), "M=%d" % M)
 
 
+def test_runtime_m_with_prepacked_weights(ctx):
+    """The reference's int8 inference tutorial
+    (examples/tutorials/matmul/inference_int8_matmul.cpp:104-125): M open, weights
+    format_tag::any, u8 source and dst with run-time zero points and scales, relu."""
+    eng, strm = ctx
+    K, N = 256, 384
+    mk = lambda M, seed: cases.int8_linear(M, K, N, seed, dst_dt=dt.u8, src_zp=7, dst_scale=0.25, dst_zp=[3],
+                                           post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0}])
+    pd = mk(8, 1).runtime_primitive_desc(eng, {"src": [0], "dst": [0]}, weights_any=True)
+    assert pd.weights_desc().get_format_kind() == memory.format_kind.opaque
+    prim = dnnl.matmul(pd)
+    for i, M in enumerate([5, 300, 64, 1024, 1]):
+        cases.say("runtime M = %d, prepacked weights" % M)
+        p = mk(M, 150 + i)
+        assert_bit_exact(p.run_gpu(eng, strm, prim=prim, prim_wei_md=pd.weights_desc()), p.run_oracle(), "M=%d" % M)
+
+
 def test_runtime_everything_and_post_ops(ctx):
     eng, strm = ctx
     po = [{"kind": "eltwise", "alg": A.eltwise_swish, "alpha": 1.0}]
