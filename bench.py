@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default=None, choices=sorted(EXTRAS),
                     help="run one of the side measurements alone and print its JSON (for profiling)")
+    ap.add_argument("--clock-warmup-s", type=float, default=2.0,
+                    help="seconds of untimed launches of the same primitive before the timed steps (after --warmup)")
     ap.add_argument("--cpu-rows", type=int, default=640, help="rows of config 2 timed on the CPU oracle")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device-to-device copy (reference point for the rocprofv3 "
@@ -69,13 +71,13 @@ def main():
         sys.exit(2)
 
     if args.calibrate_copy:
-        import torch
+        from onednn_amd import hiprt as H
         n = 1 << 30
-        a = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
-        b = torch.empty_like(a)
+        a, b = H.malloc(n), H.malloc(n)
+        H.memset(a, 0x5A, n)
         for _ in range(3):
-            b.copy_(a)
-        torch.cuda.synchronize()
+            H.memcpy_dtod(b, a, n)
+        H.device_synchronize()
         print(json.dumps({"calibrate_copy_bytes": n, "launches": 3}))
         return
 
@@ -121,6 +123,15 @@ def main():
     for _ in range(args.warmup):
         prim.execute(strm, exec_args)
     strm.wait()
+    # The card idles at a low clock and takes on the order of a second of
+    # sustained load to settle at its working point; a handful of 0.2 ms
+    # launches does not get there. Run the same launch for a fixed wall time,
+    # whatever --warmup says, so the timed steps see the settled clock.
+    t_end = time.perf_counter() + args.clock_warmup_s
+    while time.perf_counter() < t_end:
+        for _ in range(50):
+            prim.execute(strm, exec_args)
+        strm.wait()
     hiprt.device_synchronize()
     e0, e1 = hiprt.Event(), hiprt.Event()
     t0 = time.perf_counter()
@@ -143,8 +154,10 @@ def main():
         "dtype": "s8", "data": "synthetic",
         "config": {"workload": "config 2: W8A8 linear, s8[4096,4096] x s8[4096,14336] -> bf16, per-token src scales, "
                                "per-N weights scales, swish; weights prepacked via format_tag any",
-                   "impl": pd.impl_info_str(), "tile_variant": args.variant},
-        "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TFLOP/s",
+                   "impl": pd.impl_info_str(), "tile_variant": args.variant,
+                   "clock_warmup": "%g s of untimed launches of the same primitive after the --warmup steps, "
+                                   "so the timed steps run at the settled clock" % args.clock_warmup_s},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TOP/s",
                      "frac": round(kern_tops / PEAK_INT8, 4),
                      "traffic": TRAFFIC_C2_BYTES if args.variant == 0 else None,
                      "kernel": "gemm_b8y_kernel (int8, 256x256 tile, 16x16x64 MFMA)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
@@ -158,14 +171,23 @@ def main():
         sel = np.linspace(0, M - 1, rows).astype(np.int64)
         s_sub = np.ascontiguousarray(src[sel])
         d_sub = np.zeros((rows, N), np.uint16)
-        ncores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        host = host_cpu()
+        ncores = min(host["usable_cpus"], int(os.environ.get("OMP_NUM_THREADS", "16")))
         t = time.perf_counter()
         O.matmul(O.Tensor(O.S8, [rows, K], s_sub), O.Tensor(O.S8, [K, N], wei), O.Tensor(O.BF16, [rows, N], d_sub),
                  scales={O.Q_SRC: O.Quant(3, O.F32, np.ascontiguousarray(ss[sel]), (1, K)), O.Q_WEI: O.Quant(2, O.F32, ws)},
                  post_ops=[{"kind": "eltwise", "alg": A.algorithm.eltwise_swish, "alpha": 1.0}], nthreads=ncores)
         cpu_s = time.perf_counter() - t
         out["cpu_baseline"] = {"value": round(2.0 * rows * K * N / cpu_s / 1e12, 5), "unit": "TOP/s", "cores": ncores,
-                               "kind": "port",
+                               "kind": "port", "host": host,
+                               # what the reference's own CPU implementation reached where it could be built and run:
+                               # a different, smaller host than the one timed here, quoted for scale only
+                               "reference_brgemm_elsewhere": {
+                                   "where": "survey container, 8 vCPU, isa avx10_1_512_amx (brg_matmul:avx10_1_512_amx), benchdnn",
+                                   "config2_TOPs": 11.3, "config1_TOPs": 17.7, "config4_TOPs": 1.9,
+                                   "decode_common_zp_M1_ms": 20.1,
+                                   "note": "config 2 there ran with one common src scale: the reference's brgemm has no "
+                                           "per-token src scales, and its scalar fallback was not timed"},
                                "sample": "%d of the 4096 rows of config 2 (evenly spaced), full K and N, "
                                          "scalar C oracle with OpenMP, %.1f s" % (rows, cpu_s)}
         # the same rows double as a parity check of the timed kernel's output
@@ -177,6 +199,28 @@ def main():
         for name in EXTRAS:
             out[name] = globals()[EXTRAS[name]](A, memory, dt, tag, T, eng, strm, hs, hiprt)
     print(json.dumps(out))
+
+
+def host_cpu():
+    """Model name, usable CPU count and the widest matmul-relevant ISA of the host."""
+    model, flags = "unknown", set()
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name") and model == "unknown":
+                    model = line.split(":", 1)[1].strip()
+                elif line.startswith("flags") and not flags:
+                    flags = set(line.split(":", 1)[1].split())
+    except OSError:
+        pass
+    isa = next((name for name, flag in (("amx_int8", "amx_int8"), ("avx512_vnni", "avx512_vnni"), ("avx512", "avx512f"),
+                                        ("avx_vnni", "avx_vnni"), ("avx2", "avx2")) if flag in flags), "baseline")
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"model": model, "logical_cpus": os.cpu_count(), "usable_cpus": usable, "widest_isa": isa,
+            "note": "the oracle is scalar C with OpenMP: it uses none of the vector ISAs named here"}
 
 
 def C_stream(strm):
@@ -244,9 +288,39 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20):
         strm.wait()
         us = e1.elapsed_ms(e0) * 1e3 / (reps * sets)
         nbytes = K * N // 2 + sc.nbytes + zp.nbytes + M * K * 2 + M * N * 2
+        floor = None
+        if M == 1:
+            # the same bytes, the same weight sets and the same graph harness, read by a kernel that
+            # does nothing else (qmm_stream_read): what the launch gaps and a cold 8.7 MB read cost alone
+            from onednn_amd import _capi
+            sink = memory(memory.desc([8192], dt.u8, T("a")), eng)
+            L = _capi.lib()
+
+            def rd(i):
+                rc = L.qmm_stream_read(wsets[i].get_data_handle(), nb, ssets[i].get_data_handle(), sc.nbytes,
+                                       zsets[i].get_data_handle(), zp.nbytes, sink.get_data_handle(), hs)
+                assert rc == 0, rc
+
+            for i in range(sets):
+                rd(i)
+            strm.wait()
+            g2 = hiprt.Graph(hs, lambda: [rd(i) for i in range(sets)])
+            g2.launch()
+            strm.wait()
+            f0, f1 = hiprt.Event(), hiprt.Event()
+            f0.record(hs)
+            for _ in range(reps):
+                g2.launch()
+            f1.record(hs)
+            strm.wait()
+            floor = round(f1.elapsed_ms(f0) * 1e3 / (reps * sets), 3)
         res["M%d" % M] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
                           "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
                           "impl": pd.impl_info_str(), "weight_sets": sets, "timing": "hip graph of %d launches x %d" % (sets, reps)}
+        if floor is not None:
+            res["M1"]["read_floor_us"] = floor
+            res["M1"]["read_floor_kernel"] = ("qmm_stream_read: 256 workgroups x 512 lanes, 16-byte loads of the same "
+                                              "weights + scales + zero points, same graph of %d launches x %d" % (sets, reps))
     return res
 
 

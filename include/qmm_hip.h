@@ -194,6 +194,17 @@ QMM_API void qmm_set_gemm_variant(int v);
 QMM_API void qmm_set_w4a8_variant(int v);
 QMM_API void qmm_set_b8x_variant(int v);
 
+/* ---- measurement aid ----
+ * Launches a kernel that only reads: up to three byte ranges (16-byte aligned,
+ * lengths rounded down to 16), pulled with 16-byte vector loads by
+ * QMM_STREAM_READ_GROUPS workgroups of 512 lanes (the decode kernel's launch
+ * shape), one word stored per wave into `sink` (QMM_STREAM_READ_GROUPS * 32
+ * bytes). No counterpart in the reference; benchmarks use it to put a
+ * read-only floor next to the decode kernel's time. */
+#define QMM_STREAM_READ_GROUPS 256
+QMM_API int qmm_stream_read(const void *p0, size_t n0, const void *p1,
+        size_t n1, const void *p2, size_t n2, void *sink, void *stream);
+
 /* ---- device queries used by the engine ---- */
 QMM_API int qmm_device_count(void);
 QMM_API const char *qmm_last_error(void);

@@ -134,6 +134,7 @@ _SIGNATURES = {
     "qmm_set_gemm_variant": (None, [_I]),
     "qmm_set_w4a8_variant": (None, [_I]),
     "qmm_set_b8x_variant": (None, [_I]),
+    "qmm_stream_read": (_I, [_P, C.c_size_t, _P, C.c_size_t, _P, C.c_size_t, _P, _P]),
 }
 
 _lib = None

@@ -42,6 +42,20 @@ class Event:
             self.h = None
 
 
+def malloc(nbytes):
+    p = C.c_void_p()
+    check(rt().hipMalloc(C.byref(p), C.c_size_t(nbytes)), "hipMalloc")
+    return p.value
+
+
+def free(ptr):
+    check(rt().hipFree(C.c_void_p(ptr)), "hipFree")
+
+
+def memset(ptr, byte, nbytes):
+    check(rt().hipMemset(C.c_void_p(ptr), C.c_int(byte), C.c_size_t(nbytes)), "hipMemset")
+
+
 def memcpy_dtod(dst, src, nbytes):
     check(rt().hipMemcpy(C.c_void_p(dst), C.c_void_p(src), C.c_size_t(nbytes), 3), "hipMemcpy")
 
