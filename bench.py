@@ -192,7 +192,9 @@ def main():
                                          "scalar C oracle with OpenMP, %.1f s" % (rows, cpu_s)}
         # the same rows double as a parity check of the timed kernel's output
         got = m_dst.read(np.uint16, (M, N))[sel]
-        frac = assert_bf16_within_1ulp(got, d_sub, "bench parity sample", abs_slack=1e-30)  # x*rcp(1+e^-x) is 0 where libm keeps 1e-37
+        import contextlib
+        with contextlib.redirect_stdout(sys.stderr):  # stdout carries the one JSON line only
+            frac = assert_bf16_within_1ulp(got, d_sub, "bench parity sample", abs_slack=1e-30)  # x*rcp(1+e^-x) is 0 where libm keeps 1e-37
         out["parity_sample"] = {"rows": rows, "max_bf16_ulp": 1, "frac_off_by_one": round(frac, 6)}
 
     if not args.no_extras:

@@ -608,7 +608,11 @@ int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
                 && (D.scales[QMM_WEI].mask & ~(1 << (D.dst.ndims - 1))))
             return QMM_UNIMPLEMENTED;
     }
-    if (D.scales[QMM_DST].set && D.scales[QMM_DST].mask != 0)
+    if (D.scales[QMM_DST].set
+            && ((D.scales[QMM_DST].mask & ~(3 << (D.dst.ndims - 2)))
+                    || (D.scales[QMM_DST].has_groups
+                            && (D.scales[QMM_DST].g0 != 1
+                                    || D.scales[QMM_DST].g1 != 1))))
         return QMM_UNIMPLEMENTED;
     if (D.zps[QMM_DST].set && D.zps[QMM_DST].dt != dt_s32)
         return QMM_UNIMPLEMENTED;

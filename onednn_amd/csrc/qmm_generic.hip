@@ -156,8 +156,24 @@ matmul_generic_kernel(const generic_params_t *__restrict__ Pp,
                     : 0.f;
             d = generic_post_ops(P, A, d, dst_val, didx);
         }
-        if (D.scales[QMM_DST].set)
-            d *= 1.f / load_float(D.scales[QMM_DST].dt, A.scales[QMM_DST], 0);
+        if (D.scales[QMM_DST].set) {
+            // one value: times its reciprocal (src/cpu/matmul/ref_matmul.cpp:
+            // 208); masked over M and / or N (GPU engines only,
+            // src/common/matmul.cpp:150-154): divided by the element's entry
+            // of a dense [M or 1][N or 1] buffer
+            // (src/gpu/intel/ocl/ref_matmul.cl:239-245)
+            const int mask = D.scales[QMM_DST].mask;
+            if (mask == 0) {
+                d *= 1.f
+                        / load_float(D.scales[QMM_DST].dt, A.scales[QMM_DST], 0);
+            } else {
+                const bool per_m = (mask >> (nd - 2)) & 1;
+                const bool per_n = (mask >> (nd - 1)) & 1;
+                const int64_t i = (per_m ? didx[nd - 2] * (per_n ? P.N : 1) : 0)
+                        + (per_n ? n : 0);
+                d /= load_float(D.scales[QMM_DST].dt, A.scales[QMM_DST], i);
+            }
+        }
         if (D.zps[QMM_DST].set)
             d += (float)((const int32_t *)A.zps[QMM_DST])[P.dst_zp_mult * n];
         store_float(D.dst.dt, d, A.dst, dst_off);

@@ -14,39 +14,56 @@ struct read_seg_t {
     uint32_t n16[3]; // 16-byte words
 };
 
+__device__ inline void fold(uint4 &acc, const uint4 &v, bool keep) {
+    const uint32_t m = keep ? 0xFFFFFFFFu : 0u;
+    acc.x ^= v.x & m;
+    acc.y ^= v.y & m;
+    acc.z ^= v.z & m;
+    acc.w ^= v.w & m;
+}
+
+// Each workgroup reads one contiguous slab of every range, as the decode
+// kernel reads the weights, scales and zero points of its columns. The first
+// four loads of range 0 and the first load of ranges 1 and 2 are issued
+// back to back before any is consumed (indices past a slab's end are clamped
+// and their data dropped, so that no load waits on a branch); what a slab
+// holds beyond that is read by the loops that follow.
 __global__ __launch_bounds__(512) void stream_read_kernel(
         read_seg_t s, uint32_t *sink) {
-    const uint32_t t = blockIdx.x * 512u + threadIdx.x;
-    const uint32_t stride = gridDim.x * 512u;
-    uint4 acc = {0, 0, 0, 0};
+    uint32_t lo[3], hi[3];
 #pragma unroll
     for (int g = 0; g < 3; g++) {
-        const uint4 *p = s.p[g];
         const uint32_t n = s.n16[g];
-        uint32_t i = t;
-        // four loads in flight per lane
-        for (; i + 3 * stride < n; i += 4 * stride) {
-            const uint4 a = p[i];
-            const uint4 b = p[i + stride];
-            const uint4 c = p[i + 2 * stride];
-            const uint4 d = p[i + 3 * stride];
-            acc.x ^= a.x ^ b.x ^ c.x ^ d.x;
-            acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
-            acc.z ^= a.z ^ b.z ^ c.z ^ d.z;
-            acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
-        }
-        for (; i < n; i += stride) {
-            const uint4 a = p[i];
-            acc.x ^= a.x;
-            acc.y ^= a.y;
-            acc.z ^= a.z;
-            acc.w ^= a.w;
-        }
+        const uint32_t slab = (n + gridDim.x - 1) / gridDim.x;
+        lo[g] = blockIdx.x * slab < n ? blockIdx.x * slab : n;
+        hi[g] = lo[g] + slab < n ? lo[g] + slab : n;
     }
+    const uint32_t t = threadIdx.x;
+    uint4 v0[4], v1, v2;
+    const bool any0 = hi[0] > lo[0], any1 = hi[1] > lo[1], any2 = hi[2] > lo[2];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const uint32_t j = lo[0] + t + u * 512;
+        if (any0) v0[u] = s.p[0][j < hi[0] ? j : hi[0] - 1];
+    }
+    if (any1) v1 = s.p[1][lo[1] + t < hi[1] ? lo[1] + t : hi[1] - 1];
+    if (any2) v2 = s.p[2][lo[2] + t < hi[2] ? lo[2] + t : hi[2] - 1];
+    uint4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (any0) fold(acc, v0[u], lo[0] + t + u * 512 < hi[0]);
+    if (any1) fold(acc, v1, lo[1] + t < hi[1]);
+    if (any2) fold(acc, v2, lo[2] + t < hi[2]);
+    for (uint32_t i = lo[0] + t + 4 * 512; i < hi[0]; i += 512)
+        fold(acc, s.p[0][i], true);
+    for (uint32_t i = lo[1] + t + 512; i < hi[1]; i += 512)
+        fold(acc, s.p[1][i], true);
+    for (uint32_t i = lo[2] + t + 512; i < hi[2]; i += 512)
+        fold(acc, s.p[2][i], true);
     uint32_t v = acc.x ^ acc.y ^ acc.z ^ acc.w;
 #pragma unroll
     for (int o = 32; o; o >>= 1) v ^= __shfl_xor(v, o);
-    if ((threadIdx.x & 63) == 0) sink[t >> 6] = v;
+    if ((t & 63) == 0) sink[(blockIdx.x * 512u + t) >> 6] = v;
 }
 
 } // namespace

@@ -543,6 +543,21 @@ static int sum_dt_of(const orc_matmul_t *p) {
 /* A single-element scale is pre-converted to f32 (and inverted for dst); a
  * multi-element buffer is read element-wise in its own type:
  * src/cpu/cpu_primitive.hpp:32-62 */
+/* Destination scales. One value: multiply by its reciprocal
+ * (src/cpu/matmul/ref_matmul.cpp:208-209, ref_matmul_int8.cpp:237-238). A mask
+ * over M and / or N is accepted for GPU engines only
+ * (src/common/matmul.cpp:150-154); the reference's GPU implementation of it
+ * divides by the element's entry (src/gpu/intel/ocl/ref_matmul.cl:239-245,
+ * mask N); the buffer is dense row-major over the masked dims. */
+static float apply_dst_scale(const orc_quant_t *ds, float inv0, float d,
+        int64_t m, int64_t n, int64_t N, int nd) {
+    if (!ds->set) return d;
+    if (ds->mask == 0) return d * inv0;
+    const int per_m = (ds->mask >> (nd - 2)) & 1, per_n = (ds->mask >> (nd - 1)) & 1;
+    const int64_t i = (per_m ? m * (per_n ? N : 1) : 0) + (per_n ? n : 0);
+    return d / orc_load_float(ds->dt, ds->ptr, i);
+}
+
 static float single_scale(const orc_quant_t *a, int invert) {
     if (!a->set) return 1.f;
     float s = orc_load_float(a->dt, a->ptr, 0);
@@ -694,7 +709,7 @@ static void matmul_int8(const orc_matmul_t *p, const mm_ctx_t *c,
             if (non_default) {
                 float dst_val = orc_load_float(sum_dt, p->dst.ptr, dst_off);
                 d = apply_post_ops(p, d, dst_val, l_offset);
-                if (ds->set) d *= dst_scale_inv;
+                d = apply_dst_scale(ds, dst_scale_inv, d, m, n, c->N, nd);
                 if (dz->set)
                     d += (float)orc_load_int(
                             ORC_S32, dz->ptr, dst_zp_mult * n);
@@ -773,7 +788,7 @@ static void matmul_float(const orc_matmul_t *p, const mm_ctx_t *c) {
                 float dst_val = orc_load_float(sum_dt, p->dst.ptr, dst_off);
                 d = apply_post_ops(p, d, dst_val, l_offset);
             }
-            if (ds->set) d *= dst_scale_inv;
+            d = apply_dst_scale(ds, dst_scale_inv, d, m, n, c->N, nd);
             orc_store_float(p->dst.dt, d, p->dst.ptr, dst_off);
         }
     }
