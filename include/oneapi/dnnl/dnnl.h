@@ -69,6 +69,20 @@ dnnl_status_t DNNL_API dnnl_primitive_attr_get_deterministic(
         const_dnnl_primitive_attr_t attr, int *value);
 dnnl_status_t DNNL_API dnnl_primitive_attr_set_deterministic(
         dnnl_primitive_attr_t attr, int value);
+/* Dropout and stochastic rounding: the setters and getters store and return
+ * the values as the reference does (src/common/primitive_attr.cpp:430-442,
+ * 564-575); no implementation on this path computes either, so a matmul
+ * primitive descriptor created with a non-default value of one of them
+ * returns dnnl_unimplemented. */
+dnnl_status_t DNNL_API dnnl_primitive_attr_get_dropout(
+        const_dnnl_primitive_attr_t attr,
+        const_dnnl_memory_desc_t *dropout_desc);
+dnnl_status_t DNNL_API dnnl_primitive_attr_set_dropout(
+        dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t dropout_desc);
+dnnl_status_t DNNL_API dnnl_primitive_attr_get_rounding(
+        dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t *mode);
+dnnl_status_t DNNL_API dnnl_primitive_attr_set_rounding(
+        dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t mode);
 dnnl_status_t DNNL_API dnnl_primitive_attr_get_accumulation_mode(
         const_dnnl_primitive_attr_t attr, dnnl_accumulation_mode_t *mode);
 dnnl_status_t DNNL_API dnnl_primitive_attr_set_accumulation_mode(

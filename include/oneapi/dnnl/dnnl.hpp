@@ -78,6 +78,13 @@ enum class scratchpad_mode {
     library = dnnl_scratchpad_mode_library,
     user = dnnl_scratchpad_mode_user,
 };
+enum class rounding_mode {
+    environment = dnnl_rounding_mode_environment,
+    stochastic = dnnl_rounding_mode_stochastic,
+};
+inline dnnl_rounding_mode_t convert_to_c(rounding_mode mode) {
+    return static_cast<dnnl_rounding_mode_t>(mode);
+}
 enum class fpmath_mode {
     strict = dnnl_fpmath_mode_strict,
     bf16 = dnnl_fpmath_mode_bf16,
@@ -543,6 +550,31 @@ struct primitive_attr : public handle<dnnl_primitive_attr_t> {
         error::wrap_c_api(
                 dnnl_primitive_attr_set_scratchpad_mode(get(), convert_to_c(mode)),
                 "could not set scratchpad mode primitive attribute");
+    }
+    void get_dropout(memory::desc &mask_desc) const {
+        const_dnnl_memory_desc_t cdesc;
+        error::wrap_c_api(dnnl_primitive_attr_get_dropout(get(), &cdesc),
+                "could not get parameters of a dropout attribute");
+        dnnl_memory_desc_t cloned;
+        error::wrap_c_api(dnnl_memory_desc_clone(&cloned, cdesc),
+                "could not clone a memory descriptor");
+        mask_desc = memory::desc(cloned);
+    }
+    void set_dropout(const memory::desc &mask_desc) {
+        error::wrap_c_api(
+                dnnl_primitive_attr_set_dropout(get(), mask_desc.get()),
+                "could not set dropout primitive attribute");
+    }
+    rounding_mode get_rounding_mode(int arg) const {
+        dnnl_rounding_mode_t result;
+        error::wrap_c_api(dnnl_primitive_attr_get_rounding(get(), arg, &result),
+                "could not get rounding mode primitive attribute");
+        return rounding_mode(result);
+    }
+    void set_rounding_mode(int arg, rounding_mode mode) {
+        error::wrap_c_api(dnnl_primitive_attr_set_rounding(
+                                  get(), arg, convert_to_c(mode)),
+                "could not set rounding mode primitive attribute");
     }
     void set_scales_mask(int arg, int mask) {
         error::wrap_c_api(dnnl_primitive_attr_set_scales_mask(get(), arg, mask),

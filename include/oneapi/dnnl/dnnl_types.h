@@ -234,6 +234,14 @@ static const int DNNL_RUNTIME_S32_VAL_REP = INT32_MIN;
 #define DNNL_ARG_WEIGHTS DNNL_ARG_WEIGHTS_0
 #define DNNL_ARG_BIAS 41
 #define DNNL_ARG_SCRATCHPAD 80
+#define DNNL_ARG_DIFF_SRC_0 129
+#define DNNL_ARG_DIFF_SRC DNNL_ARG_DIFF_SRC_0
+#define DNNL_ARG_DIFF_WEIGHTS_0 161
+#define DNNL_ARG_DIFF_WEIGHTS DNNL_ARG_DIFF_WEIGHTS_0
+#define DNNL_ARG_ATTR_ROUNDING_SEED 508
+#define DNNL_ARG_ATTR_DROPOUT_MASK 509
+#define DNNL_ARG_ATTR_DROPOUT_PROBABILITY 510
+#define DNNL_ARG_ATTR_DROPOUT_SEED 511
 #define DNNL_ARG_ATTR_SCALES 4096
 #define DNNL_ARG_ATTR_ZERO_POINTS 8192
 #define DNNL_ARG_ATTR_MULTIPLE_POST_OP_BASE 32768

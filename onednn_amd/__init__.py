@@ -380,6 +380,25 @@ class primitive_attr:
                    C.byref(m), C.byref(a))
         return m.value, bool(a.value)
 
+    def set_rounding_mode(self, arg, mode):
+        _capi.call("dnnl_primitive_attr_set_rounding", self._h, arg, mode)
+
+    def get_rounding_mode(self, arg):
+        m = C.c_int()
+        _capi.call("dnnl_primitive_attr_get_rounding", self._h, arg, C.byref(m))
+        return m.value
+
+    def set_dropout(self, mask_desc):
+        _capi.call("dnnl_primitive_attr_set_dropout", self._h, mask_desc._h)
+
+    def get_dropout_ndims(self):
+        """ndims of the stored dropout mask descriptor (0: no dropout)."""
+        p = C.c_void_p()
+        _capi.call("dnnl_primitive_attr_get_dropout", self._h, C.byref(p))
+        n = C.c_int()
+        _capi.call("dnnl_memory_desc_query", p, query.ndims_s32, C.byref(n))
+        return n.value
+
     def set_scratchpad_mode(self, mode):
         _capi.call("dnnl_primitive_attr_set_scratchpad_mode", self._h, mode)
 

@@ -75,6 +75,10 @@ _SIGNATURES = {
     "dnnl_primitive_attr_get_fpmath_mode_v2":
         (None, [_P, C.POINTER(_I), C.POINTER(_I)]),
     "dnnl_primitive_attr_set_fpmath_mode_v2": (None, [_P, _I, _I]),
+    "dnnl_primitive_attr_get_dropout": (None, [_P, _PP]),
+    "dnnl_primitive_attr_set_dropout": (None, [_P, _P]),
+    "dnnl_primitive_attr_get_rounding": (None, [_P, _I, C.POINTER(_I)]),
+    "dnnl_primitive_attr_set_rounding": (None, [_P, _I, _I]),
     "dnnl_primitive_attr_get_deterministic": (None, [_P, C.POINTER(_I)]),
     "dnnl_primitive_attr_set_deterministic": (None, [_P, _I]),
     "dnnl_primitive_attr_get_accumulation_mode": (None, [_P, C.POINTER(_I)]),

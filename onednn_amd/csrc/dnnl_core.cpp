@@ -668,6 +668,40 @@ dnnl_status_t dnnl_primitive_attr_set_fpmath_mode_v2(
     attr->fpmath_apply_to_int = apply_to_int != 0;
     return dnnl_success;
 }
+// src/common/primitive_attr.cpp:430-442, primitive_attr.hpp:351-356
+dnnl_status_t dnnl_primitive_attr_get_dropout(const_dnnl_primitive_attr_t attr,
+        const_dnnl_memory_desc_t *dropout_desc) {
+    if (!attr) return dnnl_invalid_arguments;
+    if (dropout_desc) *dropout_desc = &attr->dropout_desc;
+    return dnnl_success;
+}
+dnnl_status_t dnnl_primitive_attr_set_dropout(
+        dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t dropout_desc) {
+    if (!attr || !dropout_desc) return dnnl_invalid_arguments;
+    attr->dropout_desc = *dropout_desc;
+    return dnnl_success;
+}
+// src/common/primitive_attr.cpp:564-575, primitive_attr.hpp:207-238: only
+// dst and the gradients may take a non-default mode; the default is not stored
+dnnl_status_t dnnl_primitive_attr_get_rounding(
+        dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t *mode) {
+    if (!attr || !mode) return dnnl_invalid_arguments;
+    auto it = attr->rounding.find(arg);
+    *mode = it == attr->rounding.end() ? dnnl_rounding_mode_environment
+                                       : it->second;
+    return dnnl_success;
+}
+dnnl_status_t dnnl_primitive_attr_set_rounding(
+        dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t mode) {
+    if (!attr) return dnnl_invalid_arguments;
+    if (mode != dnnl_rounding_mode_environment) {
+        if (arg != DNNL_ARG_DST && arg != DNNL_ARG_DIFF_SRC
+                && arg != DNNL_ARG_DIFF_WEIGHTS)
+            return dnnl_invalid_arguments;
+        attr->rounding[arg] = mode;
+    }
+    return dnnl_success;
+}
 dnnl_status_t dnnl_primitive_attr_get_deterministic(
         const_dnnl_primitive_attr_t attr, int *value) {
     if (!attr || !value) return dnnl_invalid_arguments;

@@ -114,6 +114,8 @@ struct dnnl_primitive_attr {
     dnnl_accumulation_mode_t acc_mode = dnnl_accumulation_mode_strict;
     dnnl_scratchpad_mode_t scratchpad_mode = dnnl_scratchpad_mode_library;
     bool deterministic = false;
+    dnnl_memory_desc dropout_desc; // zero descriptor: no dropout
+    std::map<int, dnnl_rounding_mode_t> rounding; // non-default entries only
     dnnl_post_ops post_ops;
 
     const quant_entry_t &scale(int arg) const { return get(scales, arg); }

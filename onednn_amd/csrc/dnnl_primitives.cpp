@@ -109,6 +109,11 @@ dnnl_status_t matmul_attr_check(const dnnl_memory_desc &src,
     const bool wei_is_fp8 = is_f8(wei_dt);
     const dnnl_status_t U = dnnl_unimplemented;
 
+    // Dropout and stochastic rounding pass the reference's common check
+    // (src/common/matmul.cpp:52-79) and are computed by its ref_matmul only
+    // (src/cpu/matmul/ref_matmul.cpp:186,214-228); no implementation here.
+    if (!attr.dropout_desc.is_zero() || !attr.rounding.empty()) return U;
+
     // Which attribute kinds may be non-default at all (the skip mask of
     // src/common/matmul.cpp:52-79; the "groups" and "data type" mask bits
     // include the plain zero-points / scales bit).

@@ -129,6 +129,28 @@ def test_attr_and_post_ops_setters():
     expect(status.out_of_memory, lambda: po2.append_prelu(1))
 
 
+def test_dropout_and_rounding_mode_are_stored_and_refused_by_matmul(eng):
+    """The setters behave as the reference's (src/common/primitive_attr.cpp:430-442, 564-575; primitive_attr.hpp:
+    207-238: a non-default rounding mode only for dst and the gradients); no implementation on this path computes
+    dropout or stochastic rounding, so the matmul descriptor is unimplemented with either."""
+    env, sto = 0, 1  # dnnl_rounding_mode_environment / _stochastic
+    a_md = memory.desc([16, 64], dt.bf16, T("ab"))
+    b_md = memory.desc([64, 32], dt.bf16, T("ab"))
+    c_md = memory.desc([16, 32], dt.bf16, T("ab"))
+    attr = dnnl.primitive_attr()
+    assert attr.get_rounding_mode(dnnl.DNNL_ARG_DST) == env and attr.get_dropout_ndims() == 0
+    expect(status.invalid_arguments, lambda: attr.set_rounding_mode(dnnl.DNNL_ARG_SRC, sto))
+    attr.set_rounding_mode(dnnl.DNNL_ARG_SRC, env)  # the default is accepted for any argument
+    expect(status.success, lambda: dnnl.matmul.primitive_desc(eng, a_md, b_md, c_md, attr=attr))
+    attr.set_rounding_mode(dnnl.DNNL_ARG_DST, sto)
+    assert attr.get_rounding_mode(dnnl.DNNL_ARG_DST) == sto
+    expect(status.unimplemented, lambda: dnnl.matmul.primitive_desc(eng, a_md, b_md, c_md, attr=attr))
+    attr2 = dnnl.primitive_attr()
+    attr2.set_dropout(memory.desc([16, 32], dt.u8, T("ab")))
+    assert attr2.get_dropout_ndims() == 2
+    expect(status.unimplemented, lambda: dnnl.matmul.primitive_desc(eng, a_md, b_md, c_md, attr=attr2))
+
+
 def _scales(arg=None, mask=0, data_type=dt.f32, groups=()):
     attr = dnnl.primitive_attr()
     for a in ([arg] if arg is not None else [dnnl.DNNL_ARG_SRC, dnnl.DNNL_ARG_WEIGHTS, dnnl.DNNL_ARG_DST]):

@@ -313,3 +313,48 @@ def test_reorder_quantize_and_transpose():
     out4 = np.zeros(K * N // 2, np.uint8)
     O.reorder(T(O.S8, v), O.Tensor(O.U4, (K, N), out4))
     assert np.array_equal(out4, O.pack4(v))
+
+
+def test_reorder_every_quantization_entry_against_numpy_float32():
+    """d = src_scale * (in - src_zp); d = d * (1 / dst_scale) + dst_zp; saturating round-to-nearest-even store
+    (src/cpu/reorder/simple_reorder.hpp:2500-2640), with scales that are not powers of two, so that every float32
+    rounding step counts. numpy float32 arithmetic performs the same single IEEE operations step by step; a dropped
+    step, a division where the reference multiplies by the reciprocal, a swapped scale or a wrong group index changes
+    bits here."""
+    rng = np.random.default_rng(18)
+    R, Ccols, G = 24, 64, 32
+    # s8 source with per-row-and-column-group scales and zero points (groups along the last dim)
+    src = rng.integers(-128, 128, (R, Ccols)).astype(np.int8)
+    ss = rng.uniform(0.01, 0.3, (R, Ccols // G)).astype(np.float32)
+    sz = rng.integers(-5, 6, (R, Ccols // G)).astype(np.int32)
+    ds = np.array([0.037], np.float32)
+    dz = np.array([3], np.int32)
+    for dst_code, lo, hi, store in ((O.S8, -128, 127, np.int8), (O.U8, 0, 255, np.uint8)):
+        out = np.zeros((R, Ccols), store)
+        O.reorder(T(O.S8, src), T(dst_code, out), src_scale=O.Quant(3, O.F32, ss, (1, G)),
+                  src_zp=O.Quant(3, O.S32, sz, (1, G)), dst_scale=O.Quant(0, O.F32, ds), dst_zp=O.Quant(0, O.S32, dz))
+        s_full = np.repeat(ss, G, axis=1)
+        z_full = np.repeat(sz, G, axis=1).astype(np.float32)
+        d = s_full * (src.astype(np.float32) - z_full)                # one multiply, one subtract, both float32
+        d = d * (np.float32(1.0) / ds[0]) + np.float32(dz[0])         # reciprocal first, then multiply, then add
+        want = np.clip(np.rint(d), lo, hi).astype(store)
+        assert np.array_equal(out, want)
+    # the same entries into an f32 destination: every bit of the float32 chain is visible, and the variant that
+    # divides by the destination scale instead of multiplying by its reciprocal differs on this data
+    outf = np.zeros((R, Ccols), np.float32)
+    O.reorder(T(O.S8, src), T(O.F32, outf), src_scale=O.Quant(3, O.F32, ss, (1, G)),
+              src_zp=O.Quant(3, O.S32, sz, (1, G)), dst_scale=O.Quant(0, O.F32, ds))
+    base = s_full * (src.astype(np.float32) - z_full)
+    assert np.array_equal(outf.view(np.uint32), (base * (np.float32(1.0) / ds[0])).view(np.uint32))
+    assert not np.array_equal(outf.view(np.uint32), (base / ds[0]).view(np.uint32))
+    # f32 -> bf16 / f16 with a per-column destination scale: numpy / torch conversions as the independent rounding
+    import torch
+    x = (rng.standard_normal((R, Ccols)) * 5).astype(np.float32)
+    dsc = rng.uniform(0.3, 3.0, Ccols).astype(np.float32)
+    scaled = x * (np.float32(1.0) / dsc)[None, :]
+    out16 = np.zeros((R, Ccols), np.uint16)
+    O.reorder(T(O.F32, x), T(O.F16, out16), dst_scale=O.Quant(2, O.F32, dsc))
+    assert np.array_equal(out16, scaled.astype(np.float16).view(np.uint16))
+    outb = np.zeros((R, Ccols), np.uint16)
+    O.reorder(T(O.F32, x), T(O.BF16, outb), dst_scale=O.Quant(2, O.F32, dsc))
+    assert np.array_equal(outb, torch.from_numpy(scaled).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16))
