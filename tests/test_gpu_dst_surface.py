@@ -195,3 +195,26 @@ def test_masked_dst_scale_over_batch_m_or_m_and_n_is_refused(ctx):
     with pytest.raises(dnnl.error) as e:
         p.primitive_desc(eng)
     assert e.value.status == dnnl.status.unimplemented
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("route", ROUTES)
+@pytest.mark.parametrize("dst_dt", [dt.s8, dt.u8], ids=str)
+def test_swish_into_quantized_dst(ctx, route, dst_dt):
+    """swish followed by a dst scale, a dst zero point and the saturating integer store. A transcendental
+    sits in front of the rounding (hardware exp2 / reciprocal in the straight-line epilogue, device libm elsewhere,
+    host libm in the oracle), so a value within float rounding of a .5 boundary may land on the neighbouring
+    integer: never further, and for few elements."""
+    say("swish -> %s with dst scale and zero point via %s" % (dst_dt, route))
+    M, K, N = (512, 256, 512) if route == "tile256" else (300, 128, 130)
+    p = cases.int8_linear(M, K, N, 57, src_dt=dt.s8, dst_dt=dst_dt, src_zp=None, src_scale=0.01,
+                          post_ops=[{"kind": "eltwise", "alg": dnnl.algorithm.eltwise_swish, "alpha": 1.0}],
+                          dst_scale=0.05, dst_zp=[7])
+    got = _run(ctx, route, p).astype(np.int32)
+    want = p.run_oracle().astype(np.int32)
+    d = np.abs(got - want)
+    frac = float((d != 0).mean())
+    print("[swish q8] %s %s: %.4f %% of the elements one step off, max distance %d; distinct values %d"
+          % (route, dst_dt, 100 * frac, d.max(), len(np.unique(want))))
+    assert len(np.unique(want)) > 50  # the case exercises the range, not a saturated constant
+    assert d.max() <= 1 and frac < 2e-3, (int(d.max()), frac)
