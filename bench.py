@@ -233,20 +233,19 @@ def C_stream(strm):
     return p.value
 
 
-def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20):
+def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, K=4096, N=4096, rows=(1, 16)):
     """Config 3: bf16 x u4 GEMV, G=128 f16 scales + u4 zero points. The 8.7 MB
     of one weights set would sit in the last-level cache, so `sets` distinct
     copies are cycled; the launches are replayed from a HIP graph so that the
     host does not pace them."""
     import oracle as O
-    K = N = 4096
     G = 128
     r = np.random.default_rng(3)
     res = {}
     w = O.pack4(r.integers(0, 16, (K, N)))
     sc = O.from_f32(O.F16, r.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
     zp = O.pack4(r.integers(6, 10, (K // G, N)))
-    for M in (1, 16):
+    for M in rows:
         attr = A.primitive_attr()
         attr.set_fpmath_mode(A.fpmath_mode.bf16, True)
         attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
