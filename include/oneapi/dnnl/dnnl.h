@@ -69,6 +69,14 @@ dnnl_status_t DNNL_API dnnl_primitive_attr_get_deterministic(
         const_dnnl_primitive_attr_t attr, int *value);
 dnnl_status_t DNNL_API dnnl_primitive_attr_set_deterministic(
         dnnl_primitive_attr_t attr, int value);
+/* Softmax forward (include/oneapi/dnnl/dnnl.h:1960-1964 of the reference):
+ * the step between the score and the value matmul of an attention block. */
+dnnl_status_t DNNL_API dnnl_softmax_forward_primitive_desc_create(
+        dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine,
+        dnnl_prop_kind_t prop_kind, dnnl_alg_kind_t alg_kind,
+        const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t dst_desc,
+        int softmax_axis, const_dnnl_primitive_attr_t attr);
+
 /* Dropout and stochastic rounding: the setters and getters store and return
  * the values as the reference does (src/common/primitive_attr.cpp:430-442,
  * 564-575); no implementation on this path computes either, so a matmul

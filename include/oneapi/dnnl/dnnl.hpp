@@ -133,6 +133,8 @@ enum class algorithm {
     binary_lt = dnnl_binary_lt,
     binary_eq = dnnl_binary_eq,
     binary_ne = dnnl_binary_ne,
+    softmax_accurate = dnnl_softmax_accurate,
+    softmax_log = dnnl_softmax_log,
 };
 enum class query {
     undef = dnnl_query_undef,
@@ -803,6 +805,47 @@ struct inner_product_forward : public primitive {
     inner_product_forward() = default;
     explicit inner_product_forward(const primitive_desc &pd)
         : primitive(pd.get()) {}
+};
+
+// Softmax forward (reference include/oneapi/dnnl/dnnl.hpp softmax_forward):
+// the step between the score and the value matmul of an attention block.
+struct softmax_forward : public primitive {
+    struct primitive_desc : public primitive_desc_base {
+        using primitive_desc_base::primitive_desc_base;
+        primitive_desc() = default;
+        primitive_desc(const engine &aengine, prop_kind aprop_kind,
+                algorithm aalgorithm, const memory::desc &src_desc,
+                const memory::desc &dst_desc, int axis,
+                const primitive_attr &attr = primitive_attr(),
+                bool allow_empty = false) {
+            dnnl_primitive_desc_t pd = nullptr;
+            const dnnl_status_t st = dnnl_softmax_forward_primitive_desc_create(
+                    &pd, aengine.get(), convert_to_c(aprop_kind),
+                    convert_to_c(aalgorithm), src_desc.get(), dst_desc.get(),
+                    axis, attr.get());
+            if (!allow_empty)
+                error::wrap_c_api(st,
+                        "could not create a primitive descriptor for a softmax "
+                        "forward propagation primitive");
+            reset(pd);
+        }
+        algorithm get_algorithm() const {
+            dnnl_alg_kind_t a = dnnl_alg_kind_undef;
+            error::wrap_c_api(dnnl_primitive_desc_query(
+                                      get(), dnnl_query_alg_kind, 0, &a),
+                    "could not query the algorithm");
+            return (algorithm)a;
+        }
+        int get_axis() const {
+            int a = -1;
+            error::wrap_c_api(dnnl_primitive_desc_query(
+                                      get(), dnnl_query_axis_s32, 0, &a),
+                    "could not query the axis");
+            return a;
+        }
+    };
+    softmax_forward() = default;
+    explicit softmax_forward(const primitive_desc &pd) : primitive(pd.get()) {}
 };
 
 } // namespace dnnl

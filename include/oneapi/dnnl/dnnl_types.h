@@ -180,6 +180,8 @@ typedef enum {
     dnnl_binary_eq = 0x1fffa,
     dnnl_binary_ne = 0x1fffb,
     dnnl_binary_select = 0x1fffc,
+    dnnl_softmax_accurate = 0x30000,
+    dnnl_softmax_log,
 } dnnl_alg_kind_t;
 
 typedef enum {

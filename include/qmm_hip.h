@@ -181,6 +181,29 @@ QMM_API const char *qmm_reorder_impl_name(const qmm_reorder_desc_t *desc);
 QMM_API int qmm_reorder_launch(const qmm_reorder_desc_t *desc,
         const qmm_reorder_args_t *args, void *hip_stream);
 
+/* ---- softmax (forward) ----
+ * The step between the two matmuls of an attention block. Stands in for
+ * ref_softmax_fwd_t::execute (src/cpu/ref_softmax.cpp:40-312). Plain strided
+ * tensors of equal dims; alg is dnnl_softmax_accurate or dnnl_softmax_log;
+ * scales are single values (mask 0). */
+typedef struct {
+    qmm_tensor_t src, dst;
+    int32_t axis;
+    int32_t alg;
+    qmm_quant_t src_scale, dst_scale;
+} qmm_softmax_desc_t;
+
+typedef struct {
+    const void *src;
+    void *dst;
+    const void *src_scale, *dst_scale;
+} qmm_softmax_args_t;
+
+QMM_API int qmm_softmax_supports(const qmm_softmax_desc_t *desc);
+QMM_API const char *qmm_softmax_impl_name(const qmm_softmax_desc_t *desc);
+QMM_API int qmm_softmax_launch(const qmm_softmax_desc_t *desc,
+        const qmm_softmax_args_t *args, void *hip_stream);
+
 /* ---- tuning / test hooks ----
  * Process-wide kernel-selection overrides for A/B measurements and for tests
  * that must reach a particular kernel at sizes the oracle finishes quickly.

@@ -54,6 +54,7 @@ class algorithm:
     (binary_add, binary_mul, binary_max, binary_min, binary_div, binary_sub,
      binary_ge, binary_gt, binary_le, binary_lt, binary_eq, binary_ne,
      binary_select) = range(0x1FFF0, 0x1FFF0 + 13)
+    softmax_accurate, softmax_log = 0x30000, 0x30001
 
 
 class fpmath_mode:
@@ -558,6 +559,22 @@ class reorder(_primitive):
         if dst is None:
             return super().execute(strm, src)
         return super().execute(strm, {DNNL_ARG_FROM: src, DNNL_ARG_TO: dst})
+
+
+class softmax_forward(_primitive):
+    """dnnl::softmax_forward over one axis (softmax_accurate / softmax_log)."""
+
+    class primitive_desc(_primitive_desc):
+        def __init__(self, eng, aprop_kind, aalgorithm, src_md, dst_md, axis, attr=None):
+            h = C.c_void_p()
+            _capi.call("dnnl_softmax_forward_primitive_desc_create", C.byref(h), eng._h, aprop_kind, aalgorithm,
+                       src_md._h, dst_md._h, axis, attr._h if attr is not None else None)
+            super().__init__(h, eng)
+
+    def execute(self, strm, src, dst=None):
+        if dst is None:
+            return super().execute(strm, src)
+        return super().execute(strm, {DNNL_ARG_SRC: src, DNNL_ARG_DST: dst})
 
 
 def version():

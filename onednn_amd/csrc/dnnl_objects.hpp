@@ -177,6 +177,8 @@ struct pd_impl_t {
     dnnl_memory_desc ip_wei_user; // weights as passed (may be format any)
     qmm_matmul_desc_t mm; // kernel-level description (matmul)
     qmm_reorder_desc_t ro; // kernel-level description (reorder)
+    qmm_softmax_desc_t sm; // kernel-level description (softmax)
+    dnnl_prop_kind_t prop_kind = dnnl_forward_inference;
     size_t scratch_bytes = 0;
     // matmul whose descriptors hold DNNL_RUNTIME_DIM_VAL: no implementation is
     // chosen until execute sees the memory objects' own descriptors

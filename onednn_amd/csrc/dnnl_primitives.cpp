@@ -481,7 +481,7 @@ dnnl_status_t walk_matmul_impls(pd_impl_t &pd, int first) {
 }
 
 int n_inputs(const pd_impl_t &pd) {
-    if (pd.kind == dnnl_reorder) return 1;
+    if (pd.kind == dnnl_reorder || pd.kind == dnnl_softmax) return 1;
     int n = 2 + (pd.bias.ndims != 0);
     for (auto &e : pd.attr.post_ops.entries)
         n += e.kind == dnnl_binary || e.kind == dnnl_prelu;
@@ -495,6 +495,9 @@ usage_t arg_usage(const pd_impl_t &pd, int arg) {
         if (arg == DNNL_ARG_SRC || arg == DNNL_ARG_WEIGHTS) return usage_t::input;
         if (arg == DNNL_ARG_BIAS)
             return pd.bias.ndims ? usage_t::input : usage_t::unused;
+        if (arg == DNNL_ARG_DST) return usage_t::output;
+    } else if (pd.kind == dnnl_softmax) {
+        if (arg == DNNL_ARG_SRC) return usage_t::input;
         if (arg == DNNL_ARG_DST) return usage_t::output;
     } else {
         if (arg == DNNL_ARG_FROM) return usage_t::input;
@@ -954,6 +957,9 @@ const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(
                 if (index == DNNL_ARG_WEIGHTS) return &q_wei;
                 if (index == DNNL_ARG_BIAS) return &q_bias;
                 if (index == DNNL_ARG_DST) return &q_dst;
+            } else if (p.kind == dnnl_softmax) {
+                if (index == DNNL_ARG_SRC) return &p.src;
+                if (index == DNNL_ARG_DST) return &p.dst;
             } else {
                 if (index == DNNL_ARG_FROM) return &p.src;
                 if (index == DNNL_ARG_TO) return &p.dst;
@@ -998,7 +1004,15 @@ dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t pd,
                     : 0;
             break;
         case dnnl_query_prop_kind:
-            *(dnnl_prop_kind_t *)result = dnnl_forward_inference;
+            *(dnnl_prop_kind_t *)result = p.prop_kind;
+            break;
+        case dnnl_query_alg_kind:
+            if (p.kind != dnnl_softmax) return dnnl_unimplemented;
+            *(dnnl_alg_kind_t *)result = (dnnl_alg_kind_t)p.sm.alg;
+            break;
+        case dnnl_query_axis_s32:
+            if (p.kind != dnnl_softmax) return dnnl_unimplemented;
+            *(int *)result = p.sm.axis;
             break;
         case dnnl_query_time_estimate_f64: *(double *)result = 0; break;
         default: {
@@ -1120,6 +1134,88 @@ dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *out,
     pd->impl_name = qmm_reorder_impl_name(&R);
     dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc {pd};
     if (!h) return dnnl_out_of_memory;
+    *out = h;
+    return dnnl_success;
+}
+
+// ======================= softmax primitive descriptor ========================
+// src/common/softmax.cpp:42-182 (descriptor and attribute checks),
+// src/cpu/ref_softmax.hpp:44-70 (what the reference implementation takes)
+dnnl_status_t dnnl_softmax_forward_primitive_desc_create(
+        dnnl_primitive_desc_t *out, dnnl_engine_t engine,
+        dnnl_prop_kind_t prop_kind, dnnl_alg_kind_t alg_kind,
+        const_dnnl_memory_desc_t src_md, const_dnnl_memory_desc_t dst_md,
+        int softmax_axis, const_dnnl_primitive_attr_t attr) {
+    if (!out || !engine || !src_md || !dst_md) return dnnl_invalid_arguments;
+    if (prop_kind != dnnl_forward_training && prop_kind != dnnl_forward_inference)
+        return dnnl_invalid_arguments;
+    if (alg_kind != dnnl_softmax_accurate && alg_kind != dnnl_softmax_log)
+        return dnnl_invalid_arguments;
+    if (softmax_axis < 0 || softmax_axis >= dst_md->ndims)
+        return dnnl_invalid_arguments;
+    if (src_md->is_any()) return dnnl_invalid_arguments;
+    if (src_md->has_runtime_dims() || dst_md->has_runtime_dims())
+        return dnnl_unimplemented;
+    if (src_md->ndims != dst_md->ndims) return dnnl_invalid_arguments;
+    for (int d = 0; d < src_md->ndims; d++)
+        if (src_md->dims[d] != dst_md->dims[d]) return dnnl_invalid_arguments;
+    if (engine->kind != dnnl_gpu) return dnnl_unimplemented;
+    if (!src_md->is_plain() || !(dst_md->is_plain() || dst_md->is_any()))
+        return dnnl_unimplemented;
+
+    static const dnnl_primitive_attr default_attr;
+    const dnnl_primitive_attr &a = attr ? *attr : default_attr;
+    // attributes: post-ops in general and, for int8 src or dst, scales
+    // (softmax.cpp:96-140); no post-op is implemented here
+    if (!a.post_ops.entries.empty()) return dnnl_unimplemented;
+    if (!a.has_default_zps()) return dnnl_unimplemented;
+    if (!a.dropout_desc.is_zero() || !a.rounding.empty()) return dnnl_unimplemented;
+    const bool int8 = is_int8(src_md->data_type) || is_int8(dst_md->data_type);
+    if (!a.has_default_scales()) {
+        if (!int8) return dnnl_unimplemented;
+        for (auto &kv : a.scales) {
+            if (kv.second.is_default()) continue;
+            if (kv.first != DNNL_ARG_SRC && kv.first != DNNL_ARG_DST)
+                return dnnl_unimplemented;
+            if (kv.second.mask != 0 || kv.second.has_groups())
+                return dnnl_unimplemented;
+        }
+    }
+    // the reference keeps the exponentials in f32 unless the accumulation
+    // mode is relaxed (ref_softmax.hpp:80-92); only the f32 form exists here
+    if (a.acc_mode != dnnl_accumulation_mode_strict
+            && src_md->data_type == dst_md->data_type
+            && src_md->data_type != dnnl_f32 && !is_int8(dst_md->data_type))
+        return dnnl_unimplemented;
+
+    auto pd = std::make_shared<pd_impl_t>();
+    pd->kind = dnnl_softmax;
+    pd->engine = engine;
+    pd->attr = a;
+    pd->prop_kind = prop_kind;
+    pd->user_src = pd->src = *src_md;
+    pd->user_dst = *dst_md;
+    pd->dst = *dst_md;
+    if (dst_md->is_any()) {
+        // softmax_pd.hpp set_default_formats: dst takes the layout of src
+        if (!md_init_plain(pd->dst, src_md->ndims, src_md->dims,
+                    dst_md->data_type, src_md->strides))
+            return dnnl_invalid_arguments;
+    }
+    qmm_softmax_desc_t &S = pd->sm;
+    std::memset(&S, 0, sizeof(S));
+    md_to_tensor(S.src, pd->src);
+    md_to_tensor(S.dst, pd->dst);
+    S.axis = softmax_axis;
+    S.alg = (int32_t)alg_kind;
+    fill_quant(S.src_scale, a.scale(DNNL_ARG_SRC), dnnl_f32);
+    fill_quant(S.dst_scale, a.scale(DNNL_ARG_DST), dnnl_f32);
+    if (qmm_softmax_supports(&S) != QMM_OK) return dnnl_unimplemented;
+    pd->impl = 0;
+    pd->impl_name = qmm_softmax_impl_name(&S);
+    dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc();
+    if (!h) return dnnl_out_of_memory;
+    h->p = pd;
     *out = h;
     return dnnl_success;
 }
@@ -1268,6 +1364,15 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
                                         : lib_scratch;
         st = qmm_matmul_launch(plan, &A, stream->hip_stream);
+    } else if (pd.kind == dnnl_softmax) {
+        if (pd.src.has_zero_dim()) return dnnl_success;
+        qmm_softmax_args_t A;
+        std::memset(&A, 0, sizeof(A));
+        A.src = handle(DNNL_ARG_SRC);
+        A.dst = handle(DNNL_ARG_DST);
+        A.src_scale = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_SRC);
+        A.dst_scale = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_DST);
+        st = qmm_softmax_launch(&pd.sm, &A, stream->hip_stream);
     } else {
         if (pd.src.has_zero_dim()) return dnnl_success;
         qmm_reorder_args_t A;
@@ -1291,7 +1396,13 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         const double ms = std::chrono::duration<double, std::milli>(
                 std::chrono::steady_clock::now() - t0)
                                   .count();
-        if (pd.kind == dnnl_matmul)
+        if (pd.kind == dnnl_softmax)
+            std::printf("onednn_verbose,v1,primitive,exec,gpu,softmax,%s,"
+                        "forward_inference,src:%s dst:%s,,axis:%d,%s,%g\n",
+                    pd.impl_name.c_str(), dt_name(pd.src.data_type),
+                    dt_name(pd.dst.data_type), pd.sm.axis,
+                    dims_str(pd.src).c_str(), ms);
+        else if (pd.kind == dnnl_matmul)
             std::printf("onednn_verbose,v1,primitive,exec,gpu,matmul,%s,"
                         "undef,src:%s wei:%s dst:%s,,,%s:%s,%g\n",
                     pd.impl_name.c_str(), dt_name(pd.src.data_type),

@@ -72,6 +72,11 @@ class _Reorder(C.Structure):
                 ("dst_scale", _Quant), ("src_zp", _Quant), ("dst_zp", _Quant)]
 
 
+class _Softmax(C.Structure):
+    _fields_ = [("src", _Tensor), ("dst", _Tensor), ("axis", C.c_int32), ("log_softmax", C.c_int32),
+                ("src_scale", _Quant), ("dst_scale", _Quant)]
+
+
 _lib = None
 
 
@@ -279,4 +284,18 @@ def reorder(src, dst, src_scale=None, dst_scale=None, src_zp=None,
     rc = lib().orc_reorder(C.byref(p))
     if rc != 0:
         raise RuntimeError("oracle reorder failed (%d)" % rc)
+    return dst.data
+
+
+def softmax(src, dst, axis, log=False, src_scale=None, dst_scale=None):
+    """Reference softmax forward over `axis` (src/cpu/ref_softmax.cpp); scales are single-value Quant entries."""
+    p = _Softmax()
+    p.src, p.dst = src.c(), dst.c()
+    p.axis, p.log_softmax = axis, 1 if log else 0
+    for name, q in (("src_scale", src_scale), ("dst_scale", dst_scale)):
+        if q is not None:
+            setattr(p, name, q.c())
+    rc = lib().orc_softmax(C.byref(p))
+    if rc != 0:
+        raise RuntimeError("oracle softmax failed (%d)" % rc)
     return dst.data

@@ -11,6 +11,7 @@
  */
 #include "qmm_oracle.h"
 
+#include <float.h>
 #include <limits.h>
 #include <math.h>
 #include <string.h>
@@ -876,6 +877,101 @@ int orc_reorder(const orc_reorder_t *p) {
                          : (uint8_t)((*b & 0xf0) | nib);
         } else
             orc_store_float(p->dst.dt, d, p->dst.ptr, o);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* softmax forward: src/cpu/ref_softmax.cpp. The reference has two loops and
+ * picks by layout (ref_softmax.hpp:137-139): "dense" when the axis is the
+ * innermost dim and src and dst are one dense layout AND one data type
+ * (memory descriptors compare equal) -- exp(s - max) * (1 / sum),
+ * ref_softmax.cpp:40-193 -- and "generic" otherwise -- exp(s - max) / sum,
+ * :196-312. Both keep the exponentials in f32 (the default accumulation mode,
+ * ref_softmax.hpp:80-92), multiply by the source scale, then by the inverted
+ * destination scale (cpu_primitive.hpp:48-56), and convert. */
+static int softmax_is_dense(const orc_softmax_t *p) {
+    const int nd = p->src.ndims;
+    if (p->src.dt != p->dst.dt) return 0;
+    if (p->src.strides[p->axis] != 1) return 0;
+    for (int d = 0; d < nd; d++)
+        if (p->src.strides[d] != p->dst.strides[d]) return 0;
+    /* dense: the dims other than the axis, sorted by stride, nest without gaps
+     * over rows of `channels` elements */
+    int order[ORC_MAX_NDIMS], n = 0;
+    for (int d = 0; d < nd; d++)
+        if (d != p->axis) order[n++] = d;
+    for (int i = 0; i < n; i++)
+        for (int j = i + 1; j < n; j++)
+            if (p->src.strides[order[j]] < p->src.strides[order[i]]) {
+                int t = order[i];
+                order[i] = order[j];
+                order[j] = t;
+            }
+    int64_t expect = p->src.dims[p->axis];
+    for (int i = 0; i < n; i++) {
+        const int k = order[i];
+        if (p->src.dims[k] == 1) continue;
+        if (p->src.strides[k] != expect) return 0;
+        expect *= p->src.dims[k];
+    }
+    return 1;
+}
+
+int orc_softmax(const orc_softmax_t *p) {
+    const int nd = p->src.ndims;
+    if (nd < 1 || nd > ORC_MAX_NDIMS || p->dst.ndims != nd) return 2;
+    if (p->axis < 0 || p->axis >= nd) return 2;
+    if (has_zero_dim(&p->src)) return 0;
+    const int64_t C = p->src.dims[p->axis];
+    const int64_t cs = p->src.strides[p->axis], cd = p->dst.strides[p->axis];
+    int64_t odims[ORC_MAX_NDIMS], rows = 1;
+    int omap[ORC_MAX_NDIMS], no = 0;
+    for (int d = 0; d < nd; d++)
+        if (d != p->axis) {
+            odims[no] = p->src.dims[d];
+            omap[no++] = d;
+            rows *= p->src.dims[d];
+        }
+    const int dense = softmax_is_dense(p);
+    const float ss = single_scale(&p->src_scale, 0);
+    const float ds = single_scale(&p->dst_scale, 1);
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; row++) {
+        int64_t so = 0, dof = 0, r = row;
+        for (int i = no - 1; i >= 0; i--) {
+            const int64_t ix = r % odims[i];
+            r /= odims[i];
+            so += ix * p->src.strides[omap[i]];
+            dof += ix * p->dst.strides[omap[i]];
+        }
+        float mx = -FLT_MAX;
+        for (int64_t c = 0; c < C; c++) {
+            const float s = orc_load_float(p->src.dt, p->src.ptr, so + c * cs);
+            mx = s > mx ? s : mx;
+        }
+        float denom = 0.f;
+        for (int64_t c = 0; c < C; c++)
+            denom += expf(orc_load_float(p->src.dt, p->src.ptr, so + c * cs) - mx);
+        float scal;
+        if (p->log_softmax)
+            scal = logf(denom);
+        else if (dense)
+            scal = denom ? 1.f / denom : 1.f;
+        else
+            scal = denom;
+        for (int64_t c = 0; c < C; c++) {
+            float d = orc_load_float(p->src.dt, p->src.ptr, so + c * cs) - mx;
+            if (p->log_softmax)
+                d = d - scal;
+            else if (dense)
+                d = expf(d) * scal;
+            else
+                d = expf(d) / scal;
+            d *= ss;
+            d *= ds;
+            orc_store_float(p->dst.dt, d, p->dst.ptr, dof + c * cd);
+        }
     }
     return 0;
 }

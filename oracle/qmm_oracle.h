@@ -104,6 +104,16 @@ typedef struct {
 } orc_reorder_t;
 int orc_reorder(const orc_reorder_t *p);
 
+/* Reference softmax forward over one axis of a plain strided tensor
+ * (src/cpu/ref_softmax.cpp:40-312); scales are single values. */
+typedef struct {
+    orc_tensor_t src, dst;
+    int32_t axis;
+    int32_t log_softmax; /* 0: softmax_accurate, 1: softmax_log */
+    orc_quant_t src_scale, dst_scale;
+} orc_softmax_t;
+int orc_softmax(const orc_softmax_t *p);
+
 /* scalar conversions */
 uint16_t orc_f32_to_bf16(float f);
 float orc_bf16_to_f32(uint16_t r);
