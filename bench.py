@@ -44,7 +44,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
-          "attention_scores": "bench_c4", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
+          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
 
 
 def main():
@@ -441,6 +441,79 @@ def bench_c4(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
     return {"ms_per_launch": round(ms, 4), "TOPs": round(2.0 * B * S * S * D / (ms * 1e-3) / 1e12, 1),
             "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str()}
+
+
+def bench_attention_chain(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=10):
+    """The attention block around config 4 as a chain of primitives: s8 Q x s8 K^T -> f32 scores + causal mask
+    (config 4 itself), softmax over the keys -> u8 probabilities (dst scale 1/255), u8 P x s8 V -> bf16. The
+    537 MB f32 scores and the 134 MB u8 probabilities cross HBM between the stages: that traffic, not the 68.7 GOP,
+    sets the time."""
+    B, S, D = 32, 2048, 128
+    r = np.random.default_rng(4)
+    f = A.prop_kind.forward_inference
+    one = lambda v: memory(memory.desc([1], dt.f32, T("a")), eng).write(np.array([v], np.float32))
+    q = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127).astype(np.int8)
+    k = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127).astype(np.int8)
+    v = np.clip(np.rint(r.standard_normal((B, S, D)) * 40), -127, 127).astype(np.int8)
+    mask = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], -1e4, 0).astype(np.float32)[None]
+    a1 = A.primitive_attr()
+    a1.set_scales_mask(A.DNNL_ARG_SRC, 0)
+    a1.set_scales_mask(A.DNNL_ARG_WEIGHTS, 0)
+    po = A.post_ops()
+    mask_md = memory.desc([1, S, S], dt.f32, T("abc"))
+    po.append_binary(A.algorithm.binary_add, mask_md)
+    a1.set_post_ops(po)
+    s_md = memory.desc([B, S, S], dt.f32, T("abc"))
+    p_md = memory.desc([B, S, S], dt.u8, T("abc"))
+    o_md = memory.desc([B, S, D], dt.bf16, T("abc"))
+    kt_md = memory.desc([B, D, S], dt.s8, T("acb"))  # the K cache [heads, keys, d] viewed as K^T
+    pd1 = A.matmul.primitive_desc(eng, memory.desc([B, S, D], dt.s8, T("abc")), kt_md, s_md, attr=a1)
+    a2 = A.primitive_attr()
+    a2.set_scales_mask(A.DNNL_ARG_DST, 0)
+    pd2 = A.softmax_forward.primitive_desc(eng, f, A.algorithm.softmax_accurate, s_md, p_md, 2, a2)
+    a3 = A.primitive_attr()
+    a3.set_scales_mask(A.DNNL_ARG_SRC, 0)
+    a3.set_scales_mask(A.DNNL_ARG_WEIGHTS, 0)
+    v_md = memory.desc([B, S, D], dt.s8, T("abc"))
+    pd3 = A.matmul.primitive_desc(eng, p_md, v_md, o_md, attr=a3)
+    p1, p2, p3 = A.matmul(pd1), A.softmax_forward(pd2), A.matmul(pd3)
+    score, prob, out = memory(s_md, eng), memory(p_md, eng), memory(o_md, eng)
+    ex1 = {A.DNNL_ARG_SRC: memory(pd1.src_desc(), eng).write(q), A.DNNL_ARG_WEIGHTS: memory(kt_md, eng).write(k),
+           A.DNNL_ARG_DST: score, A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: one(0.01),
+           A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: one(0.012),
+           A.DNNL_ARG_ATTR_MULTIPLE_POST_OP(0) | A.DNNL_ARG_SRC_1: memory(mask_md, eng).write(mask)}
+    ex2 = {A.DNNL_ARG_SRC: score, A.DNNL_ARG_DST: prob, A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_DST: one(1.0 / 255.0)}
+    ex3 = {A.DNNL_ARG_SRC: prob, A.DNNL_ARG_WEIGHTS: memory(v_md, eng).write(v), A.DNNL_ARG_DST: out,
+           A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: one(1.0 / 255.0), A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: one(0.02)}
+    stages = ((p1, ex1), (p2, ex2), (p3, ex3))
+
+    def run():
+        for prim, ex in stages:
+            prim.execute(strm, ex)
+
+    for _ in range(3):
+        run()
+    strm.wait()
+    ev = [hiprt.Event() for _ in range(4)]
+    per = [0.0, 0.0, 0.0]
+    for _ in range(steps):
+        ev[0].record(hs)
+        for i, (prim, ex) in enumerate(stages):
+            prim.execute(strm, ex)
+            ev[i + 1].record(hs)
+        strm.wait()
+        for i in range(3):
+            per[i] += ev[i + 1].elapsed_ms(ev[i]) / steps
+    total = sum(per)
+    ops = 2 * 2.0 * B * S * S * D
+    moved = (2 * B * S * D + 4 * B * S * S + 4 * S * S) + (4 * B * S * S + B * S * S) + (B * S * S + B * S * D + 2 * B * S * D)
+    fused = 3 * B * S * D + 2 * B * S * D  # what one fused kernel would have to move: Q, K, V in, bf16 out
+    return {"ms_per_block": round(total, 4), "stages_ms": {"scores": round(per[0], 4), "softmax": round(per[1], 4),
+                                                           "values": round(per[2], 4)},
+            "TOPs": round(ops / (total * 1e-3) / 1e12, 1), "bytes_moved": moved,
+            "GBps": round(moved / (total * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(moved / (total * 1e-3) / 1e9 / PEAK_HBM, 4),
+            "bytes_if_fused": fused,
+            "impl": [pd1.impl_info_str(), pd2.impl_info_str(), pd3.impl_info_str()]}
 
 
 def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):

@@ -49,6 +49,22 @@ QMM_D float wave_sum(float v) {
     return v;
 }
 
+// exp(d) for d <= 0 on the hardware's 2^x: the argument d * log2(e) is formed
+// in two parts (the rounded product and its exact remainder plus the part of
+// log2(e) a float does not hold), the 2^x of the first is corrected by the
+// second, so the error does not grow with |d| (a bare 2^(d * log2e) is off by
+// |d| * 2^-24 relative). About 2 ulp; results below the normal range are 0.
+QMM_D float exp_nonpos(float d) {
+    constexpr float L2E = 1.44269502162933349609375f; // (float)log2(e)
+    constexpr float L2E_LO = 1.925963033500011e-08f; // log2(e) - (float)log2(e)
+    constexpr float LN2 = 0.693147182464599609375f;
+    const float hi = d * L2E;
+    float lo = __builtin_fmaf(d, L2E, -hi);
+    lo = __builtin_fmaf(d, L2E_LO, lo);
+    const float e = __builtin_amdgcn_exp2f(hi);
+    return __builtin_fmaf(e, lo * LN2, e);
+}
+
 QMM_D void row_offsets(const softmax_params_t &p, int64_t row, int64_t &so,
         int64_t &dof) {
     so = 0;
@@ -106,14 +122,20 @@ softmax_rows_kernel(const softmax_params_t p) {
     float v[MAXV][4];
     float mx = -3.402823466e+38f;
     if (in_regs) {
+        // every load of the row is issued before the first value is used:
+        // groups past the row's end re-read its last group and are ignored
 #pragma unroll
         for (int g = 0; g < MAXV; g++) {
-            const int64_t q = lane + 64 * g;
-            if (q < C4) {
-                load4<SDT>(srow, q * 4, v[g]);
+            if (64 * g < C4) { // wave uniform
+                const int64_t q = lane + 64 * g;
+                load4<SDT>(srow, (q < C4 ? q : C4 - 1) * 4, v[g]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < MAXV; g++) {
+            if (lane + 64 * g < C4)
                 mx = fmaxf(mx, fmaxf(fmaxf(v[g][0], v[g][1]),
                                        fmaxf(v[g][2], v[g][3])));
-            }
         }
     } else {
         for (int64_t q = lane; q < C4; q += 64) {
@@ -134,7 +156,7 @@ softmax_rows_kernel(const softmax_params_t p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float d = v[g][i] - mx;
-                    const float e = expf(d);
+                    const float e = exp_nonpos(d);
                     sum += e;
                     v[g][i] = p.log_softmax ? d : e;
                 }
@@ -145,11 +167,11 @@ softmax_rows_kernel(const softmax_params_t p) {
             float t[4];
             load4<SDT>(srow, q * 4, t);
 #pragma unroll
-            for (int i = 0; i < 4; i++) sum += expf(t[i] - mx);
+            for (int i = 0; i < 4; i++) sum += exp_nonpos(t[i] - mx);
         }
     }
     for (int64_t c = C4 * 4 + lane; c < C; c += 64)
-        sum += expf(load_float(SDT, srow, c) - mx);
+        sum += exp_nonpos(load_float(SDT, srow, c) - mx);
     sum = wave_sum(sum);
 
     // src/cpu/ref_softmax.cpp:160-182 (src and dst of one type and layout: the
@@ -177,12 +199,22 @@ softmax_rows_kernel(const softmax_params_t p) {
             uint16_t h[4];
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                h[i] = ddt == dt_bf16 ? f32_to_bf16(o[i]) : f32_to_f16(o[i]);
+                h[i] = ddt == dt_bf16
+                        ? f32_to_bf16(o[i])
+                        // the hardware conversion: round to nearest even,
+                        // subnormals kept, as src/common/float16.hpp:52-127
+                        : __builtin_bit_cast(uint16_t, (_Float16)o[i]);
             *(uint2 *)((uint16_t *)p.dst + dof + idx) = make_uint2(
                     h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
         } else {
+            // saturate, round to nearest even, four bytes in one store
+            // (src/cpu/ref_io_helper.hpp store_float_value -> saturate_and_round)
+            const float lo = ddt == dt_s8 ? -128.f : 0.f, hi = ddt == dt_s8 ? 127.f : 255.f;
+            uint32_t w = 0;
 #pragma unroll
-            for (int i = 0; i < 4; i++) store_float(ddt, o[i], p.dst, dof + idx + i);
+            for (int i = 0; i < 4; i++)
+                w |= ((uint32_t)round_sat(o[i], lo, hi) & 0xffu) << (8 * i);
+            *(uint32_t *)((uint8_t *)p.dst + dof + idx) = w;
         }
     };
     if (in_regs) {
@@ -203,14 +235,14 @@ softmax_rows_kernel(const softmax_params_t p) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const float d = t[i] - mx;
-                o[i] = finish(p.log_softmax ? d : expf(d));
+                o[i] = finish(p.log_softmax ? d : exp_nonpos(d));
             }
             store4(q * 4, o);
         }
     }
     for (int64_t c = C4 * 4 + lane; c < C; c += 64) {
         const float d = load_float(SDT, srow, c) - mx;
-        store_float(ddt, finish(p.log_softmax ? d : expf(d)), p.dst, dof + c);
+        store_float(ddt, finish(p.log_softmax ? d : exp_nonpos(d)), p.dst, dof + c);
     }
 }
 
