@@ -229,6 +229,8 @@ static const int DNNL_RUNTIME_S32_VAL_REP = INT32_MIN;
 #define DNNL_ARG_FROM DNNL_ARG_SRC_0
 #define DNNL_ARG_SRC_1 2
 #define DNNL_ARG_SRC_2 3
+#define DNNL_ARG_SCALE 51
+#define DNNL_ARG_SHIFT 52
 #define DNNL_ARG_DST_0 17
 #define DNNL_ARG_DST DNNL_ARG_DST_0
 #define DNNL_ARG_TO DNNL_ARG_DST_0

@@ -204,6 +204,36 @@ QMM_API const char *qmm_softmax_impl_name(const qmm_softmax_desc_t *desc);
 QMM_API int qmm_softmax_launch(const qmm_softmax_desc_t *desc,
         const qmm_softmax_args_t *args, void *hip_stream);
 
+/* ---- scaled dot-product attention ----
+ * dst = softmax(scale * Q x K + mask) x V in one kernel. Stands in for the
+ * reference's internal sdpa primitive (src/common/sdpa_types.hpp:38-80,
+ * sdpa_utils.hpp:116-180; execute arguments src/gpu/intel/ocl/micro_sdpa.cpp:
+ * 674-690). q [.., Q, D], k [.., D, S] (the transposed view of a [S, D]
+ * cache), v [.., S, D], dst [.., Q, D]; mask: ndims 0 when absent, else dims
+ * equal to the scores' [.., Q, S] or 1; scale_dt 0 when there is no scale
+ * tensor; k / v may be s8 / u8 with one scale and zero point per key. */
+typedef struct {
+    qmm_tensor_t q, k, v, dst, mask;
+    int32_t scale_dt;
+    int32_t invert_scale; /* multiply by 1 / scale */
+    int32_t causal; /* key index > query index is masked out */
+    int32_t reserved;
+    int64_t kv_head_number;
+    qmm_quant_t k_scale, k_zp, v_scale, v_zp;
+} qmm_sdpa_desc_t;
+
+typedef struct {
+    const void *q, *k, *v;
+    void *dst;
+    const void *mask, *scale;
+    const void *k_scale, *k_zp, *v_scale, *v_zp;
+} qmm_sdpa_args_t;
+
+QMM_API int qmm_sdpa_supports(const qmm_sdpa_desc_t *desc);
+QMM_API const char *qmm_sdpa_impl_name(const qmm_sdpa_desc_t *desc);
+QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
+        const qmm_sdpa_args_t *args, void *hip_stream);
+
 /* ---- tuning / test hooks ----
  * Process-wide kernel-selection overrides for A/B measurements and for tests
  * that must reach a particular kernel at sizes the oracle finishes quickly.

@@ -577,6 +577,26 @@ class softmax_forward(_primitive):
         return super().execute(strm, {DNNL_ARG_SRC: src, DNNL_ARG_DST: dst})
 
 
+DNNL_ARG_QUERIES, DNNL_ARG_KEYS, DNNL_ARG_VALUES = 1, 2, 3
+DNNL_ARG_SCALE, DNNL_ARG_ATTN_MASK = 51, 52
+
+
+class sdpa(_primitive):
+    """The reference's internal scaled dot-product attention primitive (tests/gtests/internals/sdpa_internal.hpp):
+    dst = softmax(scale * Q x K + mask) x V. kq_attr / vs_attr carry the scales and zero points of a quantized
+    key / value cache as DNNL_ARG_WEIGHTS entries."""
+
+    class primitive_desc(_primitive_desc):
+        def __init__(self, eng, query_md, key_md, value_md, mask_md, scale_dt, dst_md, invert_scale=False,
+                     kv_head_number=0, causal_mask=False, attr=None, kq_attr=None, vs_attr=None):
+            h = C.c_void_p()
+            opt = lambda a: a._h if a is not None else None
+            _capi.call("sdpa_primitive_desc_create", C.byref(h), eng._h, query_md._h, key_md._h, value_md._h,
+                       dst_md._h, opt(mask_md), scale_dt, bool(invert_scale), kv_head_number, bool(causal_mask),
+                       opt(attr), opt(kq_attr), opt(vs_attr))
+            super().__init__(h, eng)
+
+
 def version():
     v = _capi.lib().dnnl_version().contents
     return v.major, v.minor, v.patch

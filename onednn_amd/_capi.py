@@ -76,6 +76,7 @@ _SIGNATURES = {
         (None, [_P, C.POINTER(_I), C.POINTER(_I)]),
     "dnnl_primitive_attr_set_fpmath_mode_v2": (None, [_P, _I, _I]),
     "dnnl_softmax_forward_primitive_desc_create": (None, [_PP, _P, _I, _I, _P, _P, _I, _P]),
+    "sdpa_primitive_desc_create": (None, [_PP, _P, _P, _P, _P, _P, _P, _I, C.c_bool, C.c_int64, C.c_bool, _P, _P, _P]),
     "dnnl_primitive_attr_get_dropout": (None, [_P, _PP]),
     "dnnl_primitive_attr_set_dropout": (None, [_P, _P]),
     "dnnl_primitive_attr_get_rounding": (None, [_P, _I, C.POINTER(_I)]),

@@ -33,7 +33,7 @@ DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off",
 PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
 UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", PRELOAD),
          ("qmm_pack.hip", "", []), ("qmm_quantize.hip", "", []),
-         ("qmm_dispatch.hip", "", []), ("qmm_measure.hip", "", PRELOAD), ("qmm_softmax.hip", "", []),
+         ("qmm_dispatch.hip", "", []), ("qmm_measure.hip", "", PRELOAD), ("qmm_softmax.hip", "", []), ("qmm_sdpa.hip", "", []),
          ("qmm_gemm_b8.hip", "", []),
          ("qmm_gemm_b8x.hip", "", []), ("qmm_gemm_w4a8.hip", "", []),
          ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]

@@ -178,6 +178,8 @@ struct pd_impl_t {
     qmm_matmul_desc_t mm; // kernel-level description (matmul)
     qmm_reorder_desc_t ro; // kernel-level description (reorder)
     qmm_softmax_desc_t sm; // kernel-level description (softmax)
+    qmm_sdpa_desc_t sd; // kernel-level description (sdpa)
+    dnnl_memory_desc sdpa_k, sdpa_v, sdpa_mask; // src = queries
     dnnl_prop_kind_t prop_kind = dnnl_forward_inference;
     size_t scratch_bytes = 0;
     // matmul whose descriptors hold DNNL_RUNTIME_DIM_VAL: no implementation is

@@ -20,6 +20,7 @@
 #include <new>
 
 #include "dnnl_objects.hpp"
+#include "sdpa_internal.h"
 
 using namespace host;
 
@@ -480,8 +481,12 @@ dnnl_status_t walk_matmul_impls(pd_impl_t &pd, int first) {
     return first == 0 ? dnnl_unimplemented : dnnl_last_impl_reached;
 }
 
+const dnnl_primitive_kind_t kind_sdpa = DNNL_PRIMITIVE_KIND_SDPA;
+
 int n_inputs(const pd_impl_t &pd) {
     if (pd.kind == dnnl_reorder || pd.kind == dnnl_softmax) return 1;
+    if (pd.kind == kind_sdpa)
+        return 3 + (pd.sdpa_mask.ndims != 0) + (pd.sd.scale_dt != 0);
     int n = 2 + (pd.bias.ndims != 0);
     for (auto &e : pd.attr.post_ops.entries)
         n += e.kind == dnnl_binary || e.kind == dnnl_prelu;
@@ -499,6 +504,26 @@ usage_t arg_usage(const pd_impl_t &pd, int arg) {
     } else if (pd.kind == dnnl_softmax) {
         if (arg == DNNL_ARG_SRC) return usage_t::input;
         if (arg == DNNL_ARG_DST) return usage_t::output;
+    } else if (pd.kind == kind_sdpa) {
+        // src/gpu/intel/ocl/micro_sdpa.cpp:674-690
+        if (arg == DNNL_ARG_QUERIES || arg == DNNL_ARG_KEYS
+                || arg == DNNL_ARG_VALUES)
+            return usage_t::input;
+        if (arg == DNNL_ARG_DST) return usage_t::output;
+        if (arg == DNNL_ARG_SCALE)
+            return pd.sd.scale_dt ? usage_t::input : usage_t::unused;
+        if (arg == DNNL_ARG_ATTN_MASK)
+            return pd.sdpa_mask.ndims ? usage_t::input : usage_t::unused;
+        const struct {
+            int arg;
+            int set;
+        } q[4] = {{DNNL_ARG_ATTR_SCALES | DNNL_ARG_KEYS, pd.sd.k_scale.set},
+                {DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_KEYS, pd.sd.k_zp.set},
+                {DNNL_ARG_ATTR_SCALES | DNNL_ARG_VALUES, pd.sd.v_scale.set},
+                {DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_VALUES, pd.sd.v_zp.set}};
+        for (auto &e : q)
+            if (arg == e.arg) return e.set ? usage_t::input : usage_t::unused;
+        return usage_t::unused;
     } else {
         if (arg == DNNL_ARG_FROM) return usage_t::input;
         if (arg == DNNL_ARG_TO) return usage_t::output;
@@ -960,6 +985,13 @@ const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(
             } else if (p.kind == dnnl_softmax) {
                 if (index == DNNL_ARG_SRC) return &p.src;
                 if (index == DNNL_ARG_DST) return &p.dst;
+            } else if (p.kind == kind_sdpa) {
+                if (index == DNNL_ARG_QUERIES) return &p.src;
+                if (index == DNNL_ARG_KEYS) return &p.sdpa_k;
+                if (index == DNNL_ARG_VALUES) return &p.sdpa_v;
+                if (index == DNNL_ARG_ATTN_MASK) return &p.sdpa_mask;
+                if (index == DNNL_ARG_DST) return &p.dst;
+                return &g_zero_md;
             } else {
                 if (index == DNNL_ARG_FROM) return &p.src;
                 if (index == DNNL_ARG_TO) return &p.dst;
@@ -1220,6 +1252,85 @@ dnnl_status_t dnnl_softmax_forward_primitive_desc_create(
     return dnnl_success;
 }
 
+// ======================= sdpa primitive descriptor ===========================
+// src/common/sdpa_test_iface.cpp:27-44, sdpa_utils.hpp:51-180
+dnnl_status_t sdpa_primitive_desc_create(dnnl_primitive_desc_t *out,
+        dnnl_engine_t engine, const_dnnl_memory_desc_t q_md,
+        const_dnnl_memory_desc_t k_md, const_dnnl_memory_desc_t v_md,
+        const_dnnl_memory_desc_t dst_md, const_dnnl_memory_desc_t mask_md,
+        dnnl_data_type_t scale_dt, bool invert_scale, dnnl_dim_t kv_head_number,
+        bool causal_mask, const_dnnl_primitive_attr_t attr,
+        const_dnnl_primitive_attr_t kq_attr,
+        const_dnnl_primitive_attr_t vs_attr) {
+    if (!out || !engine || !q_md || !k_md || !v_md || !dst_md)
+        return dnnl_invalid_arguments;
+    // sdpa_attr_check: scales f16 / f32, zero points u4 / s4 / u8 / s8 / s32,
+    // nothing else on the primitive's own attributes
+    for (const_dnnl_primitive_attr_t a : {kq_attr, vs_attr}) {
+        if (!a) continue;
+        const quant_entry_t &sc = a->scale(DNNL_ARG_WEIGHTS);
+        const quant_entry_t &zp = a->zp(DNNL_ARG_WEIGHTS);
+        if (!sc.is_default() && sc.dt != dnnl_f16 && sc.dt != dnnl_f32)
+            return dnnl_invalid_arguments;
+        if (!zp.is_default() && zp.dt != dnnl_s4 && zp.dt != dnnl_u4
+                && zp.dt != dnnl_u8 && zp.dt != dnnl_s8 && zp.dt != dnnl_s32)
+            return dnnl_invalid_arguments;
+    }
+    if (attr
+            && (!attr->has_default_scales() || !attr->has_default_zps()
+                    || !attr->post_ops.entries.empty()
+                    || attr->fpmath_mode != dnnl_fpmath_mode_strict
+                    || !attr->dropout_desc.is_zero() || !attr->rounding.empty()))
+        return dnnl_unimplemented;
+    // create_sdpa_pd: shapes
+    const int nd = dst_md->ndims;
+    if (q_md->ndims != nd || k_md->ndims != nd || v_md->ndims != nd || nd < 2)
+        return dnnl_invalid_arguments;
+    const int r = nd - 2, c = nd - 1;
+    if (q_md->dims[c] != k_md->dims[r] || k_md->dims[c] != v_md->dims[r]
+            || dst_md->dims[r] != q_md->dims[r] || dst_md->dims[c] != v_md->dims[c])
+        return dnnl_invalid_arguments;
+    if (engine->kind != dnnl_gpu) return dnnl_unimplemented;
+    for (const_dnnl_memory_desc_t md : {q_md, k_md, v_md, dst_md})
+        if (!md->is_plain() || md->has_runtime_dims()) return dnnl_unimplemented;
+    if (mask_md && (!mask_md->is_plain() || mask_md->has_runtime_dims()))
+        return dnnl_unimplemented;
+
+    auto pd = std::make_shared<pd_impl_t>();
+    pd->kind = kind_sdpa;
+    pd->engine = engine;
+    if (attr) pd->attr = *attr;
+    pd->user_src = pd->src = *q_md;
+    pd->sdpa_k = *k_md;
+    pd->sdpa_v = *v_md;
+    pd->user_dst = pd->dst = *dst_md;
+    if (mask_md) pd->sdpa_mask = *mask_md;
+    qmm_sdpa_desc_t &S = pd->sd;
+    std::memset(&S, 0, sizeof(S));
+    md_to_tensor(S.q, pd->src);
+    md_to_tensor(S.k, pd->sdpa_k);
+    md_to_tensor(S.v, pd->sdpa_v);
+    md_to_tensor(S.dst, pd->dst);
+    if (mask_md) md_to_tensor(S.mask, pd->sdpa_mask);
+    S.scale_dt = scale_dt;
+    S.invert_scale = invert_scale;
+    S.causal = causal_mask;
+    S.kv_head_number = kv_head_number;
+    static const quant_entry_t none;
+    fill_quant(S.k_scale, kq_attr ? kq_attr->scale(DNNL_ARG_WEIGHTS) : none, dnnl_f32);
+    fill_quant(S.k_zp, kq_attr ? kq_attr->zp(DNNL_ARG_WEIGHTS) : none, dnnl_s32);
+    fill_quant(S.v_scale, vs_attr ? vs_attr->scale(DNNL_ARG_WEIGHTS) : none, dnnl_f32);
+    fill_quant(S.v_zp, vs_attr ? vs_attr->zp(DNNL_ARG_WEIGHTS) : none, dnnl_s32);
+    if (qmm_sdpa_supports(&S) != QMM_OK) return dnnl_unimplemented;
+    pd->impl = 0;
+    pd->impl_name = qmm_sdpa_impl_name(&S);
+    dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc();
+    if (!h) return dnnl_out_of_memory;
+    h->p = pd;
+    *out = h;
+    return dnnl_success;
+}
+
 // ======================= primitives ========================================
 dnnl_status_t dnnl_primitive_create(
         dnnl_primitive_t *primitive, const_dnnl_primitive_desc_t pd) {
@@ -1364,6 +1475,21 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
                                         : lib_scratch;
         st = qmm_matmul_launch(plan, &A, stream->hip_stream);
+    } else if (pd.kind == kind_sdpa) {
+        if (pd.dst.has_zero_dim()) return dnnl_success;
+        qmm_sdpa_args_t A;
+        std::memset(&A, 0, sizeof(A));
+        A.q = handle(DNNL_ARG_QUERIES);
+        A.k = handle(DNNL_ARG_KEYS);
+        A.v = handle(DNNL_ARG_VALUES);
+        A.dst = handle(DNNL_ARG_DST);
+        A.mask = handle(DNNL_ARG_ATTN_MASK);
+        A.scale = handle(DNNL_ARG_SCALE);
+        A.k_scale = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_KEYS);
+        A.k_zp = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_KEYS);
+        A.v_scale = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_VALUES);
+        A.v_zp = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_VALUES);
+        st = qmm_sdpa_launch(&pd.sd, &A, stream->hip_stream);
     } else if (pd.kind == dnnl_softmax) {
         if (pd.src.has_zero_dim()) return dnnl_success;
         qmm_softmax_args_t A;
@@ -1396,7 +1522,13 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         const double ms = std::chrono::duration<double, std::milli>(
                 std::chrono::steady_clock::now() - t0)
                                   .count();
-        if (pd.kind == dnnl_softmax)
+        if (pd.kind == kind_sdpa)
+            std::printf("onednn_verbose,v1,primitive,exec,gpu,sdpa,%s,undef,"
+                        "q:%s k:%s dst:%s,,,%s:%s,%g\n",
+                    pd.impl_name.c_str(), dt_name(pd.src.data_type),
+                    dt_name(pd.sdpa_k.data_type), dt_name(pd.dst.data_type),
+                    dims_str(pd.src).c_str(), dims_str(pd.sdpa_k).c_str(), ms);
+        else if (pd.kind == dnnl_softmax)
             std::printf("onednn_verbose,v1,primitive,exec,gpu,softmax,%s,"
                         "forward_inference,src:%s dst:%s,,axis:%d,%s,%g\n",
                     pd.impl_name.c_str(), dt_name(pd.src.data_type),

@@ -1,0 +1,484 @@
+// hip:gfx950:sdpa_f16 -- scaled dot-product attention in one kernel:
+//   dst = softmax(scale * Q x K + mask) x V
+// (the reference's internal sdpa primitive: src/common/sdpa_types.hpp:38-80,
+// semantics src/gpu/intel/ocl/ref_sdpa.cl:21-78; its test's gold path is the
+// matmul -> softmax -> matmul chain, tests/gtests/internals/test_sdpa.cpp:893-
+// 1043). Q, K, V, dst are f16; K and V may instead be an s8 / u8 cache with one
+// scale (and zero point) per key, dequantized to f16 as the chain's reorder
+// does: f16(scale * (x - zero_point)).
+//
+// The scores never leave the CU. A workgroup owns 128 queries of one head (four
+// waves of 32) and walks the keys 32 at a time:
+//   * the K tile [32 keys][D] and the V tile, transposed to [Dv][32 keys], are
+//     staged in LDS once per workgroup;
+//   * S^T = K x Q^T on v_mfma_f32_16x16x32_f16 with the K rows as the first
+//     operand: a lane then holds, for ONE query (lane % 16), eight of the 32
+//     keys, so the row maximum and sum are per-lane values plus two cross-lane
+//     steps, and the eight probabilities, packed to f16, ARE the second
+//     operand of O^T += V^T x P^T -- no shuffle between the two products. The
+//     32 keys enter that product in the order the lanes hold them (k index
+//     8c + i <-> key 4c + i for i < 4, key 16 + 4c + i - 4 otherwise); the V
+//     tile is written to LDS in the same order;
+//   * online softmax in the base-2 domain: running maximum m and sum l per
+//     query, the output accumulators rescaled by 2^(m_old - m_new).
+// HBM traffic is Q, K, V in and dst out; the chain moves the f32 scores and
+// the probabilities through HBM in between (34 x more bytes at 2048 keys).
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "qmm_device.hpp"
+#include "qmm_hip.h"
+
+namespace qmm {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+constexpr int SDPA_WAVES = 4;
+constexpr int SDPA_QB = 2; // 16-query blocks per wave
+constexpr int SDPA_QW = 16 * SDPA_QB; // queries per wave
+constexpr int SDPA_QT = SDPA_QW * SDPA_WAVES; // queries per workgroup
+constexpr int SDPA_KT = 32; // keys per tile
+constexpr int VT_PITCH = 80; // bytes per V^T row (32 keys x 2 + pad)
+
+struct sdpa_strides_t {
+    int64_t b0, b1, row; // two outer dims, then the row dim (elements)
+};
+
+struct sdpa_params_t {
+    const uint16_t *Q;
+    const void *K, *V;
+    uint16_t *dst;
+    const void *mask; // nullptr: none
+    const void *scale; // nullptr: 1
+    const void *k_scale, *k_zp, *v_scale, *v_zp; // per (kv batch, key)
+    sdpa_strides_t q, k, v, o, m;
+    int64_t m_col; // mask stride over keys (0 or 1)
+    int32_t B0, B1; // outer dims of Q / dst
+    int32_t kv_div0, kv_div1; // q batch index / div = kv batch index
+    int64_t qz_b0, qz_b1; // scale / zero-point index = kb0 * qz_b0 + kb1 * qz_b1 + key
+    int32_t Qn, S;
+    int32_t scale_dt, mask_dt, invert_scale, causal;
+    int32_t kv_dt; // dt_f16, dt_s8, dt_u8
+    int32_t ks_dt, kz_dt, vs_dt, vz_dt;
+    int32_t pad_;
+};
+
+QMM_D float wave_bcast_max16(float v) {
+    // lanes that differ only in their 16-lane group hold parts of one query
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+// position of key k (0..31) of a tile in the order the P^T operand holds it
+QMM_D int key_pos(int k) {
+    return k < 16 ? 8 * (k >> 2) + (k & 3) : 8 * ((k - 16) >> 2) + 4 + (k & 3);
+}
+
+template <int DC>
+__global__ void __launch_bounds__(SDPA_WAVES * 64)
+sdpa_f16_kernel(const sdpa_params_t p) {
+    constexpr int D = 32 * DC;
+    constexpr int DVB = D / 16;
+    constexpr int K_PITCH = D * 2 + 16; // bytes
+    __shared__ __attribute__((aligned(16))) uint8_t lds_k[SDPA_KT * K_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_v[D * VT_PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, c = lane >> 4;
+    const int b1 = blockIdx.y % p.B1, b0 = blockIdx.y / p.B1;
+    const int kb0 = b0 / p.kv_div0, kb1 = b1 / p.kv_div1;
+    const int q_wg = blockIdx.x * SDPA_QT;
+    const int q_wave = q_wg + wave * SDPA_QW;
+
+    const uint16_t *Qb = p.Q + b0 * p.q.b0 + b1 * p.q.b1;
+    const uint8_t *Kb8 = (const uint8_t *)p.K;
+    const uint8_t *Vb8 = (const uint8_t *)p.V;
+    const int64_t k_base = kb0 * p.k.b0 + kb1 * p.k.b1;
+    const int64_t v_base = kb0 * p.v.b0 + kb1 * p.v.b1;
+    const int64_t qz_base = kb0 * p.qz_b0 + kb1 * p.qz_b1; // scales / zps
+    const bool quant = p.kv_dt != dt_f16;
+
+    // ---- the wave's query fragments: lane (r, c) holds Q[q][32 dc + 8 c ..]
+    v8h qf[SDPA_QB][DC];
+#pragma unroll
+    for (int qb = 0; qb < SDPA_QB; qb++) {
+        const int q = min(q_wave + qb * 16 + r, p.Qn - 1);
+#pragma unroll
+        for (int dc = 0; dc < DC; dc++)
+            qf[qb][dc] = *(const v8h *)(Qb + q * p.q.row + dc * 32 + c * 8);
+    }
+    float sc = 1.f;
+    if (p.scale) {
+        sc = load_float(p.scale_dt, p.scale, 0);
+        if (p.invert_scale) sc = 1.f / sc;
+    }
+    constexpr float L2E = 1.44269504088896340736f;
+    const float sc2 = sc * L2E;
+
+    v4f oacc[SDPA_QB][DVB];
+#pragma unroll
+    for (int qb = 0; qb < SDPA_QB; qb++)
+#pragma unroll
+        for (int d = 0; d < DVB; d++) oacc[qb][d] = v4f {0.f, 0.f, 0.f, 0.f};
+    float m_run[SDPA_QB], l_run[SDPA_QB];
+#pragma unroll
+    for (int qb = 0; qb < SDPA_QB; qb++) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
+    }
+
+    int n_tiles = (p.S + SDPA_KT - 1) / SDPA_KT;
+    if (p.causal) {
+        const int last_q = min(q_wg + SDPA_QT, p.Qn) - 1;
+        n_tiles = min(n_tiles, last_q / SDPA_KT + 1);
+    }
+    const uint8_t *mask_b = nullptr;
+    if (p.mask) {
+        const size_t msz = p.mask_dt == dt_f32 ? 4 : 2;
+        mask_b = (const uint8_t *)p.mask + (b0 * p.m.b0 + b1 * p.m.b1) * msz;
+    }
+
+    for (int kt = 0; kt < n_tiles; kt++) {
+        const int key0 = kt * SDPA_KT;
+        __syncthreads(); // the previous tile has been consumed
+        // ---- stage K [32][D] and V^T [D][32 positions] as f16
+        for (int i = tid; i < SDPA_KT * (D / 8); i += SDPA_WAVES * 64) {
+            const int kk = i / (D / 8), ch = i % (D / 8);
+            const int key = key0 + kk;
+            uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+            if (key < p.S) {
+                if (!quant) {
+                    kv = *(const uint4 *)((const uint16_t *)Kb8 + k_base
+                            + key * p.k.row + ch * 8);
+                    vv = *(const uint4 *)((const uint16_t *)Vb8 + v_base
+                            + key * p.v.row + ch * 8);
+                } else {
+                    // the cache's reorder: f16(scale * (x - zero_point))
+                    const uint2 kq = *(const uint2 *)(Kb8 + k_base
+                            + key * p.k.row + ch * 8);
+                    const uint2 vq = *(const uint2 *)(Vb8 + v_base
+                            + key * p.v.row + ch * 8);
+                    const float ks = p.k_scale
+                            ? load_float(p.ks_dt, p.k_scale, qz_base + key)
+                            : 1.f;
+                    const float vs = p.v_scale
+                            ? load_float(p.vs_dt, p.v_scale, qz_base + key)
+                            : 1.f;
+                    const float kz = p.k_zp
+                            ? (float)load_int(p.kz_dt, p.k_zp, qz_base + key)
+                            : 0.f;
+                    const float vz = p.v_zp
+                            ? (float)load_int(p.vz_dt, p.v_zp, qz_base + key)
+                            : 0.f;
+                    const uint32_t kw[2] = {kq.x, kq.y}, vw[2] = {vq.x, vq.y};
+                    uint16_t kh[8], vh[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const uint32_t kb = (kw[j >> 2] >> (8 * (j & 3))) & 0xff;
+                        const uint32_t vb = (vw[j >> 2] >> (8 * (j & 3))) & 0xff;
+                        const float kf = p.kv_dt == dt_s8 ? (float)(int8_t)kb
+                                                          : (float)kb;
+                        const float vf = p.kv_dt == dt_s8 ? (float)(int8_t)vb
+                                                          : (float)vb;
+                        kh[j] = __builtin_bit_cast(
+                                uint16_t, (_Float16)(ks * (kf - kz)));
+                        vh[j] = __builtin_bit_cast(
+                                uint16_t, (_Float16)(vs * (vf - vz)));
+                    }
+                    kv = make_uint4(kh[0] | (kh[1] << 16), kh[2] | (kh[3] << 16),
+                            kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
+                    vv = make_uint4(vh[0] | (vh[1] << 16), vh[2] | (vh[3] << 16),
+                            vh[4] | (vh[5] << 16), vh[6] | (vh[7] << 16));
+                }
+            }
+            *(uint4 *)(lds_k + kk * K_PITCH + ch * 16) = kv;
+            const int pos = key_pos(kk);
+            const uint32_t vw4[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                *(uint16_t *)(lds_v + (ch * 8 + j) * VT_PITCH + pos * 2)
+                        = (uint16_t)(vw4[j >> 1] >> (16 * (j & 1)));
+        }
+        __syncthreads();
+
+        // ---- S^T = K x Q^T: st[qb][kb] register i = key 16 kb + 4 c + i
+        v4f st[SDPA_QB][2];
+#pragma unroll
+        for (int qb = 0; qb < SDPA_QB; qb++)
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) st[qb][kb] = v4f {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int dc = 0; dc < DC; dc++) {
+                const v8h a = *(const v8h *)(lds_k + (kb * 16 + r) * K_PITCH
+                        + dc * 64 + c * 16);
+#pragma unroll
+                for (int qb = 0; qb < SDPA_QB; qb++)
+                    st[qb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            a, qf[qb][dc], st[qb][kb], 0, 0, 0);
+            }
+
+        // ---- scale, mask, online softmax (base 2), probabilities to f16
+        v8h pb[SDPA_QB];
+#pragma unroll
+        for (int qb = 0; qb < SDPA_QB; qb++) {
+            const int q = q_wave + qb * 16 + r;
+            float sv[8];
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = key0 + kb * 16 + 4 * c + i;
+                    float s = st[qb][kb][i] * sc2;
+                    if (mask_b && q < p.Qn && key < p.S) {
+                        const int64_t mo = (int64_t)q * p.m.row + key * p.m_col;
+                        s += L2E * load_float(p.mask_dt, mask_b, mo);
+                    }
+                    if (key >= p.S || (p.causal && key > q)) s = -INFINITY;
+                    sv[kb * 4 + i] = s;
+                }
+            float mt = sv[0];
+#pragma unroll
+            for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
+            mt = wave_bcast_max16(mt);
+            const float m_new = fmaxf(m_run[qb], mt);
+            // nothing but masked keys so far: keep everything at zero
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+            m_run[qb] = m_new;
+            float ls = 0.f;
+            _Float16 ph[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float pv = __builtin_amdgcn_exp2f(sv[i] - m_use);
+                ls += pv;
+                ph[i] = (_Float16)pv;
+            }
+            l_run[qb] = l_run[qb] * alpha + ls;
+            pb[qb] = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
+#pragma unroll
+            for (int d = 0; d < DVB; d++) oacc[qb][d] *= alpha;
+        }
+
+        // ---- O^T += V^T x P^T
+#pragma unroll
+        for (int d = 0; d < DVB; d++) {
+            const v8h a = *(const v8h *)(lds_v + (d * 16 + r) * VT_PITCH + c * 16);
+#pragma unroll
+            for (int qb = 0; qb < SDPA_QB; qb++)
+                oacc[qb][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        a, pb[qb], oacc[qb][d], 0, 0, 0);
+        }
+    }
+
+    // ---- normalise and store: register i of oacc[qb][d] is dst[q][16 d + 4 c + i]
+    uint16_t *Ob = p.dst + b0 * p.o.b0 + b1 * p.o.b1;
+#pragma unroll
+    for (int qb = 0; qb < SDPA_QB; qb++) {
+        float l = l_run[qb];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        const int q = q_wave + qb * 16 + r;
+        if (q >= p.Qn) continue;
+#pragma unroll
+        for (int d = 0; d < DVB; d++) {
+            uint16_t h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                h[i] = __builtin_bit_cast(uint16_t, (_Float16)(oacc[qb][d][i] / l));
+            *(uint2 *)(Ob + (int64_t)q * p.o.row + d * 16 + 4 * c) = make_uint2(
+                    h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------
+bool outer_strides(const qmm_tensor_t &t, sdpa_strides_t &s) {
+    const int nd = t.ndims;
+    if (nd < 2 || nd > 4) return false;
+    s.row = t.strides[nd - 2];
+    s.b1 = nd >= 3 ? t.strides[nd - 3] : 0;
+    s.b0 = nd >= 4 ? t.strides[nd - 4] : 0;
+    return true;
+}
+
+int64_t outer_dim(const qmm_tensor_t &t, int which) { // 0: outermost of two
+    const int nd = t.ndims;
+    if (which == 1) return nd >= 3 ? t.dims[nd - 3] : 1;
+    return nd >= 4 ? t.dims[nd - 4] : 1;
+}
+
+bool quant_ok(const qmm_quant_t &q, bool scale) {
+    if (!q.set) return true;
+    if (scale) return q.dt == dt_f16 || q.dt == dt_f32;
+    return q.dt == dt_s8 || q.dt == dt_u8 || q.dt == dt_s32;
+}
+
+bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
+    const int nd = d.q.ndims;
+    if (nd < 2 || nd > 4) return false;
+    if (d.k.ndims != nd || d.v.ndims != nd || d.dst.ndims != nd) return false;
+    if (d.q.dt != dt_f16 || d.dst.dt != dt_f16) return false;
+    if (d.k.dt != d.v.dt) return false;
+    if (d.k.dt != dt_f16 && d.k.dt != dt_s8 && d.k.dt != dt_u8) return false;
+    const int64_t Qn = d.q.dims[nd - 2], D = d.q.dims[nd - 1];
+    const int64_t S = d.k.dims[nd - 1];
+    if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
+    if (d.v.dims[nd - 1] != D) return false; // head size of V = head size of Q
+    if (d.dst.dims[nd - 2] != Qn || d.dst.dims[nd - 1] != D) return false;
+    if (D != 64 && D != 128) return false;
+    if (Qn < 1 || S < 1 || Qn > (1 << 30) || S > (1 << 30)) return false;
+    // innermost-contiguous rows: Q [q][d], K as the transposed view of a
+    // [keys][d] cache, V [keys][d], dst [q][d]
+    if (d.q.strides[nd - 1] != 1 || d.k.strides[nd - 2] != 1
+            || d.v.strides[nd - 1] != 1 || d.dst.strides[nd - 1] != 1)
+        return false;
+    // 16-byte (f16) or 8-byte (8-bit) vector loads of 8 elements
+    const int64_t al = 8;
+    if (d.q.strides[nd - 2] % al || d.k.strides[nd - 1] % al
+            || d.v.strides[nd - 2] % al || d.dst.strides[nd - 2] % 4)
+        return false;
+    sdpa_params_t p;
+    ::memset(&p, 0, sizeof(p));
+    p.B0 = (int32_t)outer_dim(d.q, 0);
+    p.B1 = (int32_t)outer_dim(d.q, 1);
+    if (outer_dim(d.dst, 0) != p.B0 || outer_dim(d.dst, 1) != p.B1) return false;
+    // K / V batch dims: equal, or dividing the query's (grouped heads)
+    const int64_t k0 = outer_dim(d.k, 0), k1 = outer_dim(d.k, 1);
+    if (outer_dim(d.v, 0) != k0 || outer_dim(d.v, 1) != k1) return false;
+    if (k0 < 1 || k1 < 1 || p.B0 % k0 || p.B1 % k1) return false;
+    if (d.kv_head_number > 0 && nd >= 3 && d.kv_head_number != k1) return false;
+    p.kv_div0 = (int32_t)(p.B0 / k0);
+    p.kv_div1 = (int32_t)(p.B1 / k1);
+    for (int i = 0; i < nd - 2; i++) {
+        if (d.q.strides[i] % al || d.k.strides[i] % al || d.v.strides[i] % al
+                || d.dst.strides[i] % 4)
+            return false;
+    }
+    outer_strides(d.q, p.q);
+    outer_strides(d.k, p.k);
+    p.k.row = d.k.strides[nd - 1]; // one key to the next
+    outer_strides(d.v, p.v);
+    outer_strides(d.dst, p.o);
+    if (d.mask.ndims) {
+        if (d.mask.ndims != nd) return false;
+        if (d.mask.dt != dt_f16 && d.mask.dt != dt_f32) return false;
+        // each dim equal to the scores' or 1 (broadcast)
+        const int64_t want[4] = {p.B0, p.B1, Qn, S};
+        int64_t ms[4] = {0, 0, 0, 0};
+        for (int i = 0; i < nd; i++) {
+            const int64_t w = want[4 - nd + i];
+            if (d.mask.dims[i] != w && d.mask.dims[i] != 1) return false;
+            ms[4 - nd + i] = d.mask.dims[i] == 1 ? 0 : d.mask.strides[i];
+        }
+        p.m.b0 = ms[0];
+        p.m.b1 = ms[1];
+        p.m.row = ms[2];
+        p.m_col = ms[3];
+        p.mask_dt = d.mask.dt;
+    }
+    if (d.scale_dt != dt_undef && d.scale_dt != dt_f16 && d.scale_dt != dt_f32)
+        return false;
+    // quantized cache: one scale / zero point per (batch, key), i.e. a mask
+    // over the batch dims and the key dim with the head-size dim in one group
+    const bool quant = d.k.dt != dt_f16;
+    for (const qmm_quant_t *q : {&d.k_scale, &d.k_zp, &d.v_scale, &d.v_zp})
+        if (q->set && !quant) return false;
+    if (!quant_ok(d.k_scale, true) || !quant_ok(d.v_scale, true)
+            || !quant_ok(d.k_zp, false) || !quant_ok(d.v_zp, false))
+        return false;
+    if (quant) {
+        // the last two dims both masked, the head-size dim in one group (K is
+        // [.., D, S]: dim nd-2; V is [.., S, D]: dim nd-1); the batch dims
+        // masked or not, alike in every entry
+        const int last2 = 3 << (nd - 2);
+        int batch_bits = -1;
+        for (const qmm_quant_t *q : {&d.k_scale, &d.k_zp, &d.v_scale, &d.v_zp}) {
+            if (!q->set) continue;
+            if ((q->mask & last2) != last2 || (q->mask >> nd)) return false;
+            const int bb = q->mask & ~last2;
+            if (batch_bits >= 0 && bb != batch_bits) return false;
+            batch_bits = bb;
+        }
+        for (const qmm_quant_t *q : {&d.k_scale, &d.k_zp})
+            if (q->set && (q->g0 != D || q->g1 != 1)) return false;
+        for (const qmm_quant_t *q : {&d.v_scale, &d.v_zp})
+            if (q->set && (q->g0 != 1 || q->g1 != D)) return false;
+        if (batch_bits < 0) batch_bits = 0;
+        const bool m1 = nd >= 3 && ((batch_bits >> (nd - 3)) & 1);
+        const bool m0 = nd >= 4 && ((batch_bits >> (nd - 4)) & 1);
+        p.qz_b1 = m1 ? S : 0;
+        p.qz_b0 = m0 ? (m1 ? k1 * S : S) : 0;
+    }
+    p.Qn = (int32_t)Qn;
+    p.S = (int32_t)S;
+    p.scale_dt = d.scale_dt;
+    p.invert_scale = d.invert_scale;
+    p.causal = d.causal;
+    p.kv_dt = d.k.dt;
+    p.ks_dt = d.k_scale.dt;
+    p.kz_dt = d.k_zp.dt;
+    p.vs_dt = d.v_scale.dt;
+    p.vz_dt = d.v_zp.dt;
+    if (out) *out = p;
+    return true;
+}
+
+} // namespace
+} // namespace qmm
+
+using namespace qmm;
+
+extern "C" {
+
+int qmm_sdpa_supports(const qmm_sdpa_desc_t *desc) {
+    if (!desc) return QMM_INVALID_ARGUMENTS;
+    return supported(*desc, nullptr) ? QMM_OK : QMM_UNIMPLEMENTED;
+}
+
+const char *qmm_sdpa_impl_name(const qmm_sdpa_desc_t *desc) {
+    return desc && supported(*desc, nullptr) ? "hip:gfx950:sdpa_f16" : "";
+}
+
+int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
+        void *hip_stream) {
+    if (!desc || !args) return QMM_INVALID_ARGUMENTS;
+    sdpa_params_t p;
+    if (!supported(*desc, &p)) return QMM_UNIMPLEMENTED;
+    if (!args->q || !args->k || !args->v || !args->dst)
+        return QMM_INVALID_ARGUMENTS;
+    if ((desc->mask.ndims && !args->mask)
+            || (desc->scale_dt != dt_undef && !args->scale)
+            || (desc->k_scale.set && !args->k_scale)
+            || (desc->k_zp.set && !args->k_zp)
+            || (desc->v_scale.set && !args->v_scale)
+            || (desc->v_zp.set && !args->v_zp))
+        return QMM_INVALID_ARGUMENTS;
+    for (const void *ptr : {args->q, args->k, args->v, (const void *)args->dst})
+        if ((uintptr_t)ptr & 15) return QMM_INVALID_ARGUMENTS;
+    p.Q = (const uint16_t *)args->q;
+    p.K = args->k;
+    p.V = args->v;
+    p.dst = (uint16_t *)args->dst;
+    p.mask = desc->mask.ndims ? args->mask : nullptr;
+    p.scale = desc->scale_dt != dt_undef ? args->scale : nullptr;
+    p.k_scale = desc->k_scale.set ? args->k_scale : nullptr;
+    p.k_zp = desc->k_zp.set ? args->k_zp : nullptr;
+    p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
+    p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
+    const dim3 grid((unsigned)((p.Qn + SDPA_QT - 1) / SDPA_QT),
+            (unsigned)(p.B0 * p.B1));
+    if (desc->q.dims[desc->q.ndims - 1] == 128)
+        hipLaunchKernelGGL(sdpa_f16_kernel<4>, grid, dim3(SDPA_WAVES * 64), 0,
+                (hipStream_t)hip_stream, p);
+    else
+        hipLaunchKernelGGL(sdpa_f16_kernel<2>, grid, dim3(SDPA_WAVES * 64), 0,
+                (hipStream_t)hip_stream, p);
+    return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
+}
+
+} // extern "C"

@@ -58,6 +58,10 @@ QMM_D float exp_nonpos(float d) {
     constexpr float L2E = 1.44269502162933349609375f; // (float)log2(e)
     constexpr float L2E_LO = 1.925963033500011e-08f; // log2(e) - (float)log2(e)
     constexpr float LN2 = 0.693147182464599609375f;
+    // below -150 the result is 0 in f32 either way; the clamp keeps -inf (a
+    // masked position) out of the remainder arithmetic, where it would turn
+    // into inf - inf
+    d = fmaxf(d, -150.f);
     const float hi = d * L2E;
     float lo = __builtin_fmaf(d, L2E, -hi);
     lo = __builtin_fmaf(d, L2E_LO, lo);

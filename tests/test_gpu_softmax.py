@@ -149,6 +149,18 @@ def test_quantized_probabilities(ctx, dst_dt):
     compare(dt.f32, got, want, "s8 source", channels=512)
 
 
+def test_minus_infinity_mask(ctx):
+    """Masked scores given as -inf (what the reference's SDPA test fills its causal mask with): exactly 0, the rest
+    of the row unaffected."""
+    r = np.random.default_rng(12)
+    x = (r.standard_normal((9, 300)) * 2).astype(np.float32)
+    x[:, 1::3] = -np.inf
+    got, want, impl = run_both(ctx, x, dt.f32, dt.f32, 1)
+    assert impl == ROWS and not np.isnan(got).any()
+    assert np.all(got[:, 1::3] == 0)
+    compare(dt.f32, got, want, "-inf mask", channels=300)
+
+
 def test_creation_rules(ctx):
     """src/common/softmax.cpp:42-140: axis range, algorithm, equal dims; scales only with an int8 side; post-ops
     are not implemented here."""
