@@ -44,7 +44,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
-          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
+          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
 
 
 def main():
@@ -514,6 +514,50 @@ def bench_attention_chain(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=10)
             "GBps": round(moved / (total * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(moved / (total * 1e-3) / 1e9 / PEAK_HBM, 4),
             "bytes_if_fused": fused,
             "impl": [pd1.impl_info_str(), pd2.impl_info_str(), pd3.impl_info_str()]}
+
+
+def bench_attention_fused(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
+    """The same attention block (32 heads, 2048 queries and keys, head size 128, causal) in one kernel: f16 Q and
+    dst, K / V either f16 or an s8 cache with per-key f16 scales and zero points. 2 x 2 x 32 x 2048 x 2048 x 128 =
+    68.7 GFLOP nominal (the causal half is skipped); bytes: Q, K, V in and dst out."""
+    import oracle as O
+    B, S, D = 32, 2048, 128
+    r = np.random.default_rng(4)
+    h16 = lambda x: O.from_f32(O.F16, np.ascontiguousarray(x, np.float32))
+    res = {}
+    q_md = memory.desc([1, B, S, D], dt.f16, T("abcd"))
+    o_md = memory.desc([1, B, S, D], dt.f16, T("abcd"))
+    q = memory(q_md, eng).write(h16(r.standard_normal((B, S, D))))
+    out = memory(o_md, eng)
+    scale = memory(memory.desc([1], dt.f16, T("a")), eng).write(h16(np.array([1.0 / np.sqrt(D)])))
+    for name, code in (("f16_cache", dt.f16), ("s8_cache", dt.s8)):
+        kt_md = memory.desc([1, B, D, S], code, T("abdc"))
+        v_md = memory.desc([1, B, S, D], code, T("abcd"))
+        ex = {A.DNNL_ARG_QUERIES: q, A.DNNL_ARG_DST: out, A.DNNL_ARG_SCALE: scale}
+        kq = vs = None
+        if code == dt.f16:
+            ex[A.DNNL_ARG_KEYS] = memory(kt_md, eng).write(h16(r.standard_normal((B, S, D))))
+            ex[A.DNNL_ARG_VALUES] = memory(v_md, eng).write(h16(r.standard_normal((B, S, D))))
+            nbytes = 4 * B * S * D * 2
+        else:
+            ex[A.DNNL_ARG_KEYS] = memory(kt_md, eng).write(r.integers(-128, 128, (B, S, D), dtype=np.int8))
+            ex[A.DNNL_ARG_VALUES] = memory(v_md, eng).write(r.integers(-128, 128, (B, S, D), dtype=np.int8))
+            kq, vs = A.primitive_attr(), A.primitive_attr()
+            for a, groups, which in ((kq, [D, 1], A.DNNL_ARG_KEYS), (vs, [1, D], A.DNNL_ARG_VALUES)):
+                a.set_scales(A.DNNL_ARG_WEIGHTS, 0b1110, groups, dt.f16)
+                a.set_zero_points(A.DNNL_ARG_WEIGHTS, 0b1110, groups, dt.s8)
+                sc = h16(r.uniform(0.005, 0.02, (B, S)))
+                zp = r.integers(-6, 7, (B, S), dtype=np.int8)
+                ex[A.DNNL_ARG_ATTR_SCALES | which] = memory(memory.desc([sc.nbytes], dt.u8, T("a")), eng).write(sc)
+                ex[A.DNNL_ARG_ATTR_ZERO_POINTS | which] = memory(memory.desc([zp.nbytes], dt.u8, T("a")), eng).write(zp)
+            nbytes = 2 * B * S * D * 2 + 2 * B * S * D + 2 * B * S * 3
+        pd = A.sdpa.primitive_desc(eng, q_md, kt_md, v_md, None, dt.f16, o_md, False, B, True, None, kq, vs)
+        ms = _time(A.sdpa(pd), strm, hs, hiprt, ex, steps)
+        flops = 2 * 2.0 * B * S * S * D
+        res[name] = {"ms_per_block": round(ms, 4), "TFLOPs_nominal": round(flops / (ms * 1e-3) / 1e12, 1),
+                     "TFLOPs_causal_half": round(flops / 2 / (ms * 1e-3) / 1e12, 1), "algorithmic_bytes": nbytes,
+                     "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "impl": pd.impl_info_str()}
+    return res
 
 
 def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):

@@ -9,16 +9,17 @@
 //
 // The scores never leave the CU. A workgroup owns 128 queries of one head (four
 // waves of 32) and walks the keys 32 at a time:
-//   * the K tile [32 keys][D] and the V tile, transposed to [Dv][32 keys], are
-//     staged in LDS once per workgroup;
+//   * the K tile and the V tile [32 keys][D] are staged in LDS once per
+//     workgroup (requested one tile ahead, so a step does not wait for memory);
 //   * S^T = K x Q^T on v_mfma_f32_16x16x32_f16 with the K rows as the first
 //     operand: a lane then holds, for ONE query (lane % 16), eight of the 32
 //     keys, so the row maximum and sum are per-lane values plus two cross-lane
 //     steps, and the eight probabilities, packed to f16, ARE the second
 //     operand of O^T += V^T x P^T -- no shuffle between the two products. The
 //     32 keys enter that product in the order the lanes hold them (k index
-//     8c + i <-> key 4c + i for i < 4, key 16 + 4c + i - 4 otherwise); the V
-//     tile is written to LDS in the same order;
+//     8c + i <-> key 4c + i for i < 4, key 16 + 4c + i - 4 otherwise); V^T in
+//     that order comes out of the row-major tile through the transposing LDS
+//     read (ds_read_b64_tr_b16);
 //   * online softmax in the base-2 domain: running maximum m and sum l per
 //     query, the output accumulators rescaled by 2^(m_old - m_new).
 // HBM traffic is Q, K, V in and dst out; the chain moves the f32 scores and
@@ -40,7 +41,10 @@ constexpr int SDPA_QB = 2; // 16-query blocks per wave
 constexpr int SDPA_QW = 16 * SDPA_QB; // queries per wave
 constexpr int SDPA_QT = SDPA_QW * SDPA_WAVES; // queries per workgroup
 constexpr int SDPA_KT = 32; // keys per tile
-constexpr int VT_PITCH = 80; // bytes per V^T row (32 keys x 2 + pad)
+#ifndef SDPA_MIN_BLOCKS
+#define SDPA_MIN_BLOCKS 2
+#endif
+typedef short v4s __attribute__((ext_vector_type(4)));
 
 struct sdpa_strides_t {
     int64_t b0, b1, row; // two outer dims, then the row dim (elements)
@@ -72,25 +76,32 @@ QMM_D float wave_bcast_max16(float v) {
     return v;
 }
 
-// position of key k (0..31) of a tile in the order the P^T operand holds it
-QMM_D int key_pos(int k) {
-    return k < 16 ? 8 * (k >> 2) + (k & 3) : 8 * ((k - 16) >> 2) + 4 + (k & 3);
-}
-
 template <int DC>
-__global__ void __launch_bounds__(SDPA_WAVES * 64)
+__global__ void __launch_bounds__(SDPA_WAVES * 64, SDPA_MIN_BLOCKS)
 sdpa_f16_kernel(const sdpa_params_t p) {
     constexpr int D = 32 * DC;
     constexpr int DVB = D / 16;
     constexpr int K_PITCH = D * 2 + 16; // bytes
     __shared__ __attribute__((aligned(16))) uint8_t lds_k[SDPA_KT * K_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_v[D * VT_PITCH];
+    // V rows 32 bytes further apart than K rows: eight consecutive rows then
+    // start on eight different groups of 8 banks, which is what the 8-byte
+    // transposing reads below touch per row
+    constexpr int V_PITCH = D * 2 + 32;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_v[SDPA_KT * V_PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4;
     const int b1 = blockIdx.y % p.B1, b0 = blockIdx.y / p.B1;
     const int kb0 = b0 / p.kv_div0, kb1 = b1 / p.kv_div1;
-    const int q_wg = blockIdx.x * SDPA_QT;
+    // Under a causal mask the last query tiles walk the most keys. The first
+    // half of the grid takes the query tiles last to first (long walks start
+    // early), the second half first to last, so that workgroups half a grid
+    // apart -- which share a CU when the whole grid is resident -- add up to
+    // the same number of key tiles everywhere.
+    const bool mirrored = 2 * (blockIdx.y * gridDim.x + blockIdx.x)
+            >= gridDim.x * gridDim.y;
+    const int q_wg = (int)(mirrored ? blockIdx.x : gridDim.x - 1 - blockIdx.x)
+            * SDPA_QT;
     const int q_wave = q_wg + wave * SDPA_QW;
 
     const uint16_t *Qb = p.Q + b0 * p.q.b0 + b1 * p.q.b1;
@@ -141,68 +152,89 @@ sdpa_f16_kernel(const sdpa_params_t p) {
         mask_b = (const uint8_t *)p.mask + (b0 * p.m.b0 + b1 * p.m.b1) * msz;
     }
 
+    // ---- staging: a thread carries NS (key, 8-element chunk) pieces of a
+    // tile from global memory to LDS. The pieces of tile kt + 1 are requested
+    // before tile kt is multiplied and written to LDS after it, so a
+    // workgroup's walk over the keys (up to S / 32 dependent steps) does not
+    // pay a trip to memory per step.
+    constexpr int NS = SDPA_KT * (D / 8) / (SDPA_WAVES * 64);
+    uint4 pk[NS], pv[NS]; // f16: 8 values each; 8-bit: x, y hold 8 values
+    float pks[NS], pvs[NS], pkz[NS], pvz[NS];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int n = 0; n < NS; n++) {
+            const int i = tid + n * SDPA_WAVES * 64;
+            const int kk = i / (D / 8), ch = i % (D / 8);
+            const int key = min(kt * SDPA_KT + kk, p.S - 1); // clamped: zeroed below
+            if (!quant) {
+                pk[n] = *(const uint4 *)((const uint16_t *)Kb8 + k_base
+                        + key * p.k.row + ch * 8);
+                pv[n] = *(const uint4 *)((const uint16_t *)Vb8 + v_base
+                        + key * p.v.row + ch * 8);
+            } else {
+                const uint2 kq = *(const uint2 *)(Kb8 + k_base + key * p.k.row
+                        + ch * 8);
+                const uint2 vq = *(const uint2 *)(Vb8 + v_base + key * p.v.row
+                        + ch * 8);
+                pk[n] = make_uint4(kq.x, kq.y, 0, 0);
+                pv[n] = make_uint4(vq.x, vq.y, 0, 0);
+                pks[n] = p.k_scale ? load_float(p.ks_dt, p.k_scale, qz_base + key)
+                                   : 1.f;
+                pvs[n] = p.v_scale ? load_float(p.vs_dt, p.v_scale, qz_base + key)
+                                   : 1.f;
+                pkz[n] = p.k_zp
+                        ? (float)load_int(p.kz_dt, p.k_zp, qz_base + key)
+                        : 0.f;
+                pvz[n] = p.v_zp
+                        ? (float)load_int(p.vz_dt, p.v_zp, qz_base + key)
+                        : 0.f;
+            }
+        }
+    };
+    auto commit = [&](int kt) {
+#pragma unroll
+        for (int n = 0; n < NS; n++) {
+            const int i = tid + n * SDPA_WAVES * 64;
+            const int kk = i / (D / 8), ch = i % (D / 8);
+            uint4 kv = pk[n], vv = pv[n];
+            if (quant) {
+                // the cache's reorder: f16(scale * (x - zero_point))
+                const uint32_t kw[2] = {pk[n].x, pk[n].y};
+                const uint32_t vw[2] = {pv[n].x, pv[n].y};
+                uint32_t kh[8], vh[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const uint32_t kb = (kw[j >> 2] >> (8 * (j & 3))) & 0xff;
+                    const uint32_t vb = (vw[j >> 2] >> (8 * (j & 3))) & 0xff;
+                    const float kf = p.kv_dt == dt_s8 ? (float)(int8_t)kb : (float)kb;
+                    const float vf = p.kv_dt == dt_s8 ? (float)(int8_t)vb : (float)vb;
+                    kh[j] = __builtin_bit_cast(
+                            uint16_t, (_Float16)(pks[n] * (kf - pkz[n])));
+                    vh[j] = __builtin_bit_cast(
+                            uint16_t, (_Float16)(pvs[n] * (vf - pvz[n])));
+                }
+                kv = make_uint4(kh[0] | (kh[1] << 16), kh[2] | (kh[3] << 16),
+                        kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
+                vv = make_uint4(vh[0] | (vh[1] << 16), vh[2] | (vh[3] << 16),
+                        vh[4] | (vh[5] << 16), vh[6] | (vh[7] << 16));
+            }
+            if (kt * SDPA_KT + kk >= p.S) {
+                // keys past the end: zero, so that probability 0 x V stays 0
+                kv = make_uint4(0, 0, 0, 0);
+                vv = make_uint4(0, 0, 0, 0);
+            }
+            *(uint4 *)(lds_k + kk * K_PITCH + ch * 16) = kv;
+            *(uint4 *)(lds_v + kk * V_PITCH + ch * 16) = vv;
+        }
+    };
+
+    if (n_tiles > 0) fetch(0);
     for (int kt = 0; kt < n_tiles; kt++) {
         const int key0 = kt * SDPA_KT;
         __syncthreads(); // the previous tile has been consumed
-        // ---- stage K [32][D] and V^T [D][32 positions] as f16
-        for (int i = tid; i < SDPA_KT * (D / 8); i += SDPA_WAVES * 64) {
-            const int kk = i / (D / 8), ch = i % (D / 8);
-            const int key = key0 + kk;
-            uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-            if (key < p.S) {
-                if (!quant) {
-                    kv = *(const uint4 *)((const uint16_t *)Kb8 + k_base
-                            + key * p.k.row + ch * 8);
-                    vv = *(const uint4 *)((const uint16_t *)Vb8 + v_base
-                            + key * p.v.row + ch * 8);
-                } else {
-                    // the cache's reorder: f16(scale * (x - zero_point))
-                    const uint2 kq = *(const uint2 *)(Kb8 + k_base
-                            + key * p.k.row + ch * 8);
-                    const uint2 vq = *(const uint2 *)(Vb8 + v_base
-                            + key * p.v.row + ch * 8);
-                    const float ks = p.k_scale
-                            ? load_float(p.ks_dt, p.k_scale, qz_base + key)
-                            : 1.f;
-                    const float vs = p.v_scale
-                            ? load_float(p.vs_dt, p.v_scale, qz_base + key)
-                            : 1.f;
-                    const float kz = p.k_zp
-                            ? (float)load_int(p.kz_dt, p.k_zp, qz_base + key)
-                            : 0.f;
-                    const float vz = p.v_zp
-                            ? (float)load_int(p.vz_dt, p.v_zp, qz_base + key)
-                            : 0.f;
-                    const uint32_t kw[2] = {kq.x, kq.y}, vw[2] = {vq.x, vq.y};
-                    uint16_t kh[8], vh[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        const uint32_t kb = (kw[j >> 2] >> (8 * (j & 3))) & 0xff;
-                        const uint32_t vb = (vw[j >> 2] >> (8 * (j & 3))) & 0xff;
-                        const float kf = p.kv_dt == dt_s8 ? (float)(int8_t)kb
-                                                          : (float)kb;
-                        const float vf = p.kv_dt == dt_s8 ? (float)(int8_t)vb
-                                                          : (float)vb;
-                        kh[j] = __builtin_bit_cast(
-                                uint16_t, (_Float16)(ks * (kf - kz)));
-                        vh[j] = __builtin_bit_cast(
-                                uint16_t, (_Float16)(vs * (vf - vz)));
-                    }
-                    kv = make_uint4(kh[0] | (kh[1] << 16), kh[2] | (kh[3] << 16),
-                            kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
-                    vv = make_uint4(vh[0] | (vh[1] << 16), vh[2] | (vh[3] << 16),
-                            vh[4] | (vh[5] << 16), vh[6] | (vh[7] << 16));
-                }
-            }
-            *(uint4 *)(lds_k + kk * K_PITCH + ch * 16) = kv;
-            const int pos = key_pos(kk);
-            const uint32_t vw4[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-                *(uint16_t *)(lds_v + (ch * 8 + j) * VT_PITCH + pos * 2)
-                        = (uint16_t)(vw4[j >> 1] >> (16 * (j & 1)));
-        }
+        commit(kt);
         __syncthreads();
+        if (kt + 1 < n_tiles) fetch(kt + 1);
 
         // ---- S^T = K x Q^T: st[qb][kb] register i = key 16 kb + 4 c + i
         v4f st[SDPA_QB][2];
@@ -222,8 +254,13 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                             a, qf[qb][dc], st[qb][kb], 0, 0, 0);
             }
 
-        // ---- scale, mask, online softmax (base 2), probabilities to f16
+        // ---- scale, mask, online softmax (base 2), probabilities to f16.
+        // Wave-uniform: does this tile need the per-key checks at all?
+        const bool edge = key0 + SDPA_KT > p.S
+                || (p.causal && key0 + SDPA_KT - 1 > q_wave);
         v8h pb[SDPA_QB];
+        bool rescale = false;
+        float alpha_q[SDPA_QB];
 #pragma unroll
         for (int qb = 0; qb < SDPA_QB; qb++) {
             const int q = q_wave + qb * 16 + r;
@@ -231,16 +268,31 @@ sdpa_f16_kernel(const sdpa_params_t p) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int key = key0 + kb * 16 + 4 * c + i;
-                    float s = st[qb][kb][i] * sc2;
-                    if (mask_b && q < p.Qn && key < p.S) {
-                        const int64_t mo = (int64_t)q * p.m.row + key * p.m_col;
-                        s += L2E * load_float(p.mask_dt, mask_b, mo);
+                for (int i = 0; i < 4; i++)
+                    sv[kb * 4 + i] = st[qb][kb][i] * sc2;
+            if (mask_b) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = key0 + kb * 16 + 4 * c + i;
+                        if (q < p.Qn && key < p.S) {
+                            const int64_t mo = (int64_t)q * p.m.row + key * p.m_col;
+                            sv[kb * 4 + i]
+                                    += L2E * load_float(p.mask_dt, mask_b, mo);
+                        }
                     }
-                    if (key >= p.S || (p.causal && key > q)) s = -INFINITY;
-                    sv[kb * 4 + i] = s;
-                }
+            }
+            if (edge) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = key0 + kb * 16 + 4 * c + i;
+                        if (key >= p.S || (p.causal && key > q))
+                            sv[kb * 4 + i] = -INFINITY;
+                    }
+            }
             float mt = sv[0];
 #pragma unroll
             for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
@@ -249,25 +301,46 @@ sdpa_f16_kernel(const sdpa_params_t p) {
             // nothing but masked keys so far: keep everything at zero
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+            rescale |= m_new != m_run[qb];
+            alpha_q[qb] = alpha;
             m_run[qb] = m_new;
             float ls = 0.f;
             _Float16 ph[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const float pv = __builtin_amdgcn_exp2f(sv[i] - m_use);
-                ls += pv;
-                ph[i] = (_Float16)pv;
+                const float pv1 = __builtin_amdgcn_exp2f(sv[i] - m_use);
+                ls += pv1;
+                ph[i] = (_Float16)pv1;
             }
             l_run[qb] = l_run[qb] * alpha + ls;
             pb[qb] = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
+        }
+        // the accumulators only move when some query's maximum did
+        if (__builtin_amdgcn_ballot_w64(rescale)) {
 #pragma unroll
-            for (int d = 0; d < DVB; d++) oacc[qb][d] *= alpha;
+            for (int qb = 0; qb < SDPA_QB; qb++)
+#pragma unroll
+                for (int d = 0; d < DVB; d++) oacc[qb][d] *= alpha_q[qb];
         }
 
-        // ---- O^T += V^T x P^T
+        // ---- O^T += V^T x P^T. The first operand is V^T [16 d][32 keys] from
+        // the row-major tile: ds_read_b64_tr_b16 hands lane i of a 16-lane
+        // group element (i & 3) of the 8-byte chunk that lane (i >> 2) + 4 t
+        // of the group addressed, t = 0..3. With lane j addressing row
+        // (key) 4 c + (j >> 2), columns d0 + 4 (j & 3) .. + 3, lane r receives
+        // V[4 c + t][d0 + r]: its column of V for four keys. Two reads (keys
+        // 4 c .. and 16 + 4 c ..) make the eight keys of its k slots.
 #pragma unroll
         for (int d = 0; d < DVB; d++) {
-            const v8h a = *(const v8h *)(lds_v + (d * 16 + r) * VT_PITCH + c * 16);
+            const uint8_t *va = lds_v + (4 * c + (r >> 2)) * V_PITCH
+                    + (d * 16 + 4 * (r & 3)) * 2;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)va);
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)(va + 16 * V_PITCH));
+            typedef short v8s __attribute__((ext_vector_type(8)));
+            const v8h a = __builtin_bit_cast(v8h,
+                    v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
 #pragma unroll
             for (int qb = 0; qb < SDPA_QB; qb++)
                 oacc[qb][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
