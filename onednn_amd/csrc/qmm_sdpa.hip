@@ -66,42 +66,69 @@ struct sdpa_params_t {
     int32_t scale_dt, mask_dt, invert_scale, causal;
     int32_t kv_dt; // dt_f16, dt_s8, dt_u8
     int32_t ks_dt, kz_dt, vs_dt, vz_dt;
-    int32_t pad_;
+    int32_t pair_halves; // the grid fits the chip at once: see the kernel
 };
 
-QMM_D float wave_bcast_max16(float v) {
-    // lanes that differ only in their 16-lane group hold parts of one query
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+// Lanes that differ only in their 16-lane row hold parts of one query. The two
+// exchange steps (row r <-> r ^ 1, half <-> other half) as vector-ALU lane
+// swaps: v_permlane16_swap returns (rows 0 0 2 2, rows 1 1 3 3) of its two
+// inputs' rows, v_permlane32_swap (lower lower, upper upper) halves; with both
+// inputs the same value the two results are the partners of a butterfly.
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+QMM_D float rows_max(float v) {
+    unsigned u = f2u(v);
+    const v2u a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    u = f2u(fmaxf(u2f(a.x), u2f(a.y)));
+    const v2u b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(u2f(b.x), u2f(b.y));
+}
+QMM_D float rows_sum(float v) {
+    unsigned u = f2u(v);
+    const v2u a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    u = f2u(u2f(a.x) + u2f(a.y));
+    const v2u b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return u2f(b.x) + u2f(b.y);
 }
 
-template <int DC>
+// the cache's scales are f16 or f32, its zero points s8, u8 or s32
+QMM_D float ld_scale(int dt, const void *p, int64_t i) {
+    return dt == dt_f16 ? (float)((const _Float16 *)p)[i] : ((const float *)p)[i];
+}
+QMM_D float ld_zp(int dt, const void *p, int64_t i) {
+    return dt == dt_s8  ? (float)((const int8_t *)p)[i]
+            : dt == dt_u8 ? (float)((const uint8_t *)p)[i]
+                          : (float)((const int32_t *)p)[i];
+}
+
+// QUANT: K / V are an 8-bit cache; MASKED: an explicit mask tensor is added
+template <int DC, bool QUANT, bool MASKED>
 __global__ void __launch_bounds__(SDPA_WAVES * 64, SDPA_MIN_BLOCKS)
 sdpa_f16_kernel(const sdpa_params_t p) {
     constexpr int D = 32 * DC;
     constexpr int DVB = D / 16;
     constexpr int K_PITCH = D * 2 + 16; // bytes
-    __shared__ __attribute__((aligned(16))) uint8_t lds_k[SDPA_KT * K_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_k2[2][SDPA_KT * K_PITCH];
     // V rows 32 bytes further apart than K rows: eight consecutive rows then
     // start on eight different groups of 8 banks, which is what the 8-byte
     // transposing reads below touch per row
     constexpr int V_PITCH = D * 2 + 32;
-    __shared__ __attribute__((aligned(16))) uint8_t lds_v[SDPA_KT * V_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_v2[2][SDPA_KT * V_PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, c = lane >> 4;
-    const int b1 = blockIdx.y % p.B1, b0 = blockIdx.y / p.B1;
+    const int b1 = blockIdx.x % p.B1, b0 = blockIdx.x / p.B1;
     const int kb0 = b0 / p.kv_div0, kb1 = b1 / p.kv_div1;
-    // Under a causal mask the last query tiles walk the most keys. The first
-    // half of the grid takes the query tiles last to first (long walks start
-    // early), the second half first to last, so that workgroups half a grid
-    // apart -- which share a CU when the whole grid is resident -- add up to
-    // the same number of key tiles everywhere.
-    const bool mirrored = 2 * (blockIdx.y * gridDim.x + blockIdx.x)
-            >= gridDim.x * gridDim.y;
-    const int q_wg = (int)(mirrored ? blockIdx.x : gridDim.x - 1 - blockIdx.x)
-            * SDPA_QT;
+    // Under a causal mask the last query tiles walk the most keys. Workgroups
+    // are dispatched heads first, query tiles from the last to the first, so
+    // the long walks start early and the short ones fill the gaps. When the
+    // whole grid is resident at once (two workgroups per CU) nothing is left
+    // to fill gaps with: then the second half of the grid runs first to last
+    // instead, so that workgroups half a grid apart, which share a CU, add up
+    // to the same number of key tiles everywhere.
+    int rank = blockIdx.y;
+    const int nq = gridDim.y;
+    if (p.pair_halves && rank >= nq / 2) rank = nq / 2 + (nq - 1 - rank);
+    const int q_wg = (nq - 1 - rank) * SDPA_QT;
     const int q_wave = q_wg + wave * SDPA_QW;
 
     const uint16_t *Qb = p.Q + b0 * p.q.b0 + b1 * p.q.b1;
@@ -110,7 +137,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
     const int64_t k_base = kb0 * p.k.b0 + kb1 * p.k.b1;
     const int64_t v_base = kb0 * p.v.b0 + kb1 * p.v.b1;
     const int64_t qz_base = kb0 * p.qz_b0 + kb1 * p.qz_b1; // scales / zps
-    const bool quant = p.kv_dt != dt_f16;
+    constexpr bool quant = QUANT;
 
     // ---- the wave's query fragments: lane (r, c) holds Q[q][32 dc + 8 c ..]
     v8h qf[SDPA_QB][DC];
@@ -147,7 +174,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
         n_tiles = min(n_tiles, last_q / SDPA_KT + 1);
     }
     const uint8_t *mask_b = nullptr;
-    if (p.mask) {
+    if (MASKED) {
         const size_t msz = p.mask_dt == dt_f32 ? 4 : 2;
         mask_b = (const uint8_t *)p.mask + (b0 * p.m.b0 + b1 * p.m.b1) * msz;
     }
@@ -157,13 +184,14 @@ sdpa_f16_kernel(const sdpa_params_t p) {
     // before tile kt is multiplied and written to LDS after it, so a
     // workgroup's walk over the keys (up to S / 32 dependent steps) does not
     // pay a trip to memory per step.
-    constexpr int NS = SDPA_KT * (D / 8) / (SDPA_WAVES * 64);
+    constexpr int PIECES = SDPA_KT * (D / 8);
+    constexpr int NS = (PIECES + SDPA_WAVES * 64 - 1) / (SDPA_WAVES * 64);
     uint4 pk[NS], pv[NS]; // f16: 8 values each; 8-bit: x, y hold 8 values
     float pks[NS], pvs[NS], pkz[NS], pvz[NS];
     auto fetch = [&](int kt) {
 #pragma unroll
         for (int n = 0; n < NS; n++) {
-            const int i = tid + n * SDPA_WAVES * 64;
+            const int i = min(tid + n * SDPA_WAVES * 64, PIECES - 1);
             const int kk = i / (D / 8), ch = i % (D / 8);
             const int key = min(kt * SDPA_KT + kk, p.S - 1); // clamped: zeroed below
             if (!quant) {
@@ -178,40 +206,44 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                         + ch * 8);
                 pk[n] = make_uint4(kq.x, kq.y, 0, 0);
                 pv[n] = make_uint4(vq.x, vq.y, 0, 0);
-                pks[n] = p.k_scale ? load_float(p.ks_dt, p.k_scale, qz_base + key)
+                pks[n] = p.k_scale ? ld_scale(p.ks_dt, p.k_scale, qz_base + key)
                                    : 1.f;
-                pvs[n] = p.v_scale ? load_float(p.vs_dt, p.v_scale, qz_base + key)
+                pvs[n] = p.v_scale ? ld_scale(p.vs_dt, p.v_scale, qz_base + key)
                                    : 1.f;
-                pkz[n] = p.k_zp
-                        ? (float)load_int(p.kz_dt, p.k_zp, qz_base + key)
-                        : 0.f;
-                pvz[n] = p.v_zp
-                        ? (float)load_int(p.vz_dt, p.v_zp, qz_base + key)
-                        : 0.f;
+                pkz[n] = p.k_zp ? ld_zp(p.kz_dt, p.k_zp, qz_base + key) : 0.f;
+                pvz[n] = p.v_zp ? ld_zp(p.vz_dt, p.v_zp, qz_base + key) : 0.f;
             }
         }
     };
     auto commit = [&](int kt) {
+        uint8_t *lds_k = lds_k2[kt & 1], *lds_v = lds_v2[kt & 1];
 #pragma unroll
         for (int n = 0; n < NS; n++) {
             const int i = tid + n * SDPA_WAVES * 64;
+            if (i >= PIECES) break; // fewer pieces than threads
             const int kk = i / (D / 8), ch = i % (D / 8);
             uint4 kv = pk[n], vv = pv[n];
             if (quant) {
                 // the cache's reorder: f16(scale * (x - zero_point))
-                const uint32_t kw[2] = {pk[n].x, pk[n].y};
-                const uint32_t vw[2] = {pv[n].x, pv[n].y};
+                // s8 bytes are read as u8 after flipping the sign bit (x + 128),
+                // and the 128 joins the zero point: (x + 128) - (zp + 128) is
+                // the same exact difference, and unsigned bytes convert in one
+                // instruction each
+                const bool sgn = p.kv_dt == dt_s8;
+                const uint32_t flip = sgn ? 0x80808080u : 0u;
+                const float kzb = pkz[n] + (sgn ? 128.f : 0.f);
+                const float vzb = pvz[n] + (sgn ? 128.f : 0.f);
+                const uint32_t kw[2] = {pk[n].x ^ flip, pk[n].y ^ flip};
+                const uint32_t vw[2] = {pv[n].x ^ flip, pv[n].y ^ flip};
                 uint32_t kh[8], vh[8];
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    const uint32_t kb = (kw[j >> 2] >> (8 * (j & 3))) & 0xff;
-                    const uint32_t vb = (vw[j >> 2] >> (8 * (j & 3))) & 0xff;
-                    const float kf = p.kv_dt == dt_s8 ? (float)(int8_t)kb : (float)kb;
-                    const float vf = p.kv_dt == dt_s8 ? (float)(int8_t)vb : (float)vb;
+                    const float kf = (float)((kw[j >> 2] >> (8 * (j & 3))) & 0xff);
+                    const float vf = (float)((vw[j >> 2] >> (8 * (j & 3))) & 0xff);
                     kh[j] = __builtin_bit_cast(
-                            uint16_t, (_Float16)(pks[n] * (kf - pkz[n])));
+                            uint16_t, (_Float16)(pks[n] * (kf - kzb)));
                     vh[j] = __builtin_bit_cast(
-                            uint16_t, (_Float16)(pvs[n] * (vf - pvz[n])));
+                            uint16_t, (_Float16)(pvs[n] * (vf - vzb)));
                 }
                 kv = make_uint4(kh[0] | (kh[1] << 16), kh[2] | (kh[3] << 16),
                         kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
@@ -228,13 +260,18 @@ sdpa_f16_kernel(const sdpa_params_t p) {
         }
     };
 
-    if (n_tiles > 0) fetch(0);
+    // Two LDS buffers: while tile kt is multiplied out of one, tile kt + 1
+    // (requested an iteration earlier) is written into the other between the
+    // two products, and tile kt + 2 is requested. One barrier per tile.
+    if (n_tiles > 0) {
+        fetch(0);
+        commit(0);
+        if (n_tiles > 1) fetch(1);
+    }
+    __syncthreads();
     for (int kt = 0; kt < n_tiles; kt++) {
         const int key0 = kt * SDPA_KT;
-        __syncthreads(); // the previous tile has been consumed
-        commit(kt);
-        __syncthreads();
-        if (kt + 1 < n_tiles) fetch(kt + 1);
+        const uint8_t *lds_k = lds_k2[kt & 1], *lds_v = lds_v2[kt & 1];
 
         // ---- S^T = K x Q^T: st[qb][kb] register i = key 16 kb + 4 c + i
         v4f st[SDPA_QB][2];
@@ -270,18 +307,23 @@ sdpa_f16_kernel(const sdpa_params_t p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     sv[kb * 4 + i] = st[qb][kb][i] * sc2;
-            if (mask_b) {
+            if (MASKED) {
+                // every load unconditional: positions past the ends re-read the
+                // last row / key (they are overwritten or never stored)
+                const int64_t mrow = (int64_t)min(q, p.Qn - 1) * p.m.row;
+                float mv[8];
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const int key = key0 + kb * 16 + 4 * c + i;
-                        if (q < p.Qn && key < p.S) {
-                            const int64_t mo = (int64_t)q * p.m.row + key * p.m_col;
-                            sv[kb * 4 + i]
-                                    += L2E * load_float(p.mask_dt, mask_b, mo);
-                        }
+                        const int key = min(key0 + kb * 16 + 4 * c + i, p.S - 1);
+                        const int64_t mo = mrow + key * p.m_col;
+                        mv[kb * 4 + i] = p.mask_dt == dt_f32
+                                ? ((const float *)mask_b)[mo]
+                                : (float)((const _Float16 *)mask_b)[mo];
                     }
+#pragma unroll
+                for (int i = 0; i < 8; i++) sv[i] += L2E * mv[i];
             }
             if (edge) {
 #pragma unroll
@@ -296,7 +338,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
             float mt = sv[0];
 #pragma unroll
             for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
-            mt = wave_bcast_max16(mt);
+            mt = rows_max(mt);
             const float m_new = fmaxf(m_run[qb], mt);
             // nothing but masked keys so far: keep everything at zero
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -323,6 +365,11 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                 for (int d = 0; d < DVB; d++) oacc[qb][d] *= alpha_q[qb];
         }
 
+        if (kt + 1 < n_tiles) {
+            commit(kt + 1); // the other buffer: last read before the previous barrier
+            if (kt + 2 < n_tiles) fetch(kt + 2);
+        }
+
         // ---- O^T += V^T x P^T. The first operand is V^T [16 d][32 keys] from
         // the row-major tile: ds_read_b64_tr_b16 hands lane i of a 16-lane
         // group element (i & 3) of the 8-byte chunk that lane (i >> 2) + 4 t
@@ -346,15 +393,14 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                 oacc[qb][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                         a, pb[qb], oacc[qb][d], 0, 0, 0);
         }
+        __syncthreads();
     }
 
     // ---- normalise and store: register i of oacc[qb][d] is dst[q][16 d + 4 c + i]
     uint16_t *Ob = p.dst + b0 * p.o.b0 + b1 * p.o.b1;
 #pragma unroll
     for (int qb = 0; qb < SDPA_QB; qb++) {
-        float l = l_run[qb];
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
+        const float l = rows_sum(l_run[qb]);
         const int q = q_wave + qb * 16 + r;
         if (q >= p.Qn) continue;
 #pragma unroll
@@ -543,14 +589,30 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.k_zp = desc->k_zp.set ? args->k_zp : nullptr;
     p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
-    const dim3 grid((unsigned)((p.Qn + SDPA_QT - 1) / SDPA_QT),
-            (unsigned)(p.B0 * p.B1));
-    if (desc->q.dims[desc->q.ndims - 1] == 128)
-        hipLaunchKernelGGL(sdpa_f16_kernel<4>, grid, dim3(SDPA_WAVES * 64), 0,
+    const dim3 grid((unsigned)(p.B0 * p.B1),
+            (unsigned)((p.Qn + SDPA_QT - 1) / SDPA_QT));
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess)
+        (void)hipDeviceGetAttribute(
+                &cus, hipDeviceAttributeMultiprocessorCount, dev);
+    p.pair_halves = p.causal && grid.y % 2 == 0
+            && (int64_t)grid.x * grid.y <= (int64_t)SDPA_MIN_BLOCKS * cus;
+    const bool d128 = desc->q.dims[desc->q.ndims - 1] == 128;
+    const bool qn = p.kv_dt != dt_f16, mk = p.mask != nullptr;
+    auto go = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);
-    else
-        hipLaunchKernelGGL(sdpa_f16_kernel<2>, grid, dim3(SDPA_WAVES * 64), 0,
-                (hipStream_t)hip_stream, p);
+    };
+    switch ((d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
+        case 0: go(sdpa_f16_kernel<2, false, false>); break;
+        case 1: go(sdpa_f16_kernel<2, false, true>); break;
+        case 2: go(sdpa_f16_kernel<2, true, false>); break;
+        case 3: go(sdpa_f16_kernel<2, true, true>); break;
+        case 4: go(sdpa_f16_kernel<4, false, false>); break;
+        case 5: go(sdpa_f16_kernel<4, false, true>); break;
+        case 6: go(sdpa_f16_kernel<4, true, false>); break;
+        default: go(sdpa_f16_kernel<4, true, true>); break;
+    }
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }
 
