@@ -44,7 +44,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
-          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
+          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
 
 
 def main():
@@ -557,6 +557,48 @@ def bench_attention_fused(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20,
         res[name] = {"ms_per_block": round(ms, 4), "TFLOPs_nominal": round(flops / (ms * 1e-3) / 1e12, 1),
                      "TFLOPs_computed": round(flops / (2 if causal else 1) / (ms * 1e-3) / 1e12, 1), "algorithmic_bytes": nbytes,
                      "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "impl": pd.impl_info_str()}
+    return res
+
+
+def bench_attention_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=50):
+    """One query per head against a long K / V cache (32 heads, head size 128): the decode step of the same block.
+    The keys are cut into ranges (one workgroup each), partial results merged by a second small kernel. Bytes: the
+    cache once (+ per-key scales and zero points for the 8-bit cache)."""
+    import oracle as O
+    H, D = 32, 128
+    r = np.random.default_rng(8)
+    h16 = lambda x: O.from_f32(O.F16, np.ascontiguousarray(x, np.float32))
+    res = {}
+    q_md = memory.desc([1, H, 1, D], dt.f16, T("abcd"))
+    for S in (8192, 32768):
+        for name, code in (("f16_cache", dt.f16), ("s8_cache", dt.s8)):
+            kt_md = memory.desc([1, H, D, S], code, T("abdc"))
+            v_md = memory.desc([1, H, S, D], code, T("abcd"))
+            ex = {A.DNNL_ARG_QUERIES: memory(q_md, eng).write(h16(r.standard_normal((H, 1, D)))),
+                  A.DNNL_ARG_DST: memory(q_md, eng)}
+            kq = vs = None
+            if code == dt.f16:
+                ex[A.DNNL_ARG_KEYS] = memory(kt_md, eng).write(h16(r.standard_normal((H, S, D))))
+                ex[A.DNNL_ARG_VALUES] = memory(v_md, eng).write(h16(r.standard_normal((H, S, D))))
+                nbytes = 2 * H * S * D * 2
+            else:
+                ex[A.DNNL_ARG_KEYS] = memory(kt_md, eng).write(r.integers(-128, 128, (H, S, D), dtype=np.int8))
+                ex[A.DNNL_ARG_VALUES] = memory(v_md, eng).write(r.integers(-128, 128, (H, S, D), dtype=np.int8))
+                kq, vs = A.primitive_attr(), A.primitive_attr()
+                for a, groups, which in ((kq, [D, 1], A.DNNL_ARG_KEYS), (vs, [1, D], A.DNNL_ARG_VALUES)):
+                    a.set_scales(A.DNNL_ARG_WEIGHTS, 0b1110, groups, dt.f16)
+                    a.set_zero_points(A.DNNL_ARG_WEIGHTS, 0b1110, groups, dt.s8)
+                    sc = h16(r.uniform(0.005, 0.02, (H, S)))
+                    zp = r.integers(-6, 7, (H, S), dtype=np.int8)
+                    ex[A.DNNL_ARG_ATTR_SCALES | which] = memory(memory.desc([sc.nbytes], dt.u8, T("a")), eng).write(sc)
+                    ex[A.DNNL_ARG_ATTR_ZERO_POINTS | which] = memory(memory.desc([zp.nbytes], dt.u8, T("a")), eng).write(zp)
+                nbytes = 2 * H * S * D + 2 * H * S * 3
+            pd = A.sdpa.primitive_desc(eng, q_md, kt_md, v_md, None, dt.undef, q_md, False, H, False, None, kq, vs)
+            ms = _time(A.sdpa(pd), strm, hs, hiprt, ex, steps, warm=5)
+            res["keys%d_%s" % (S, name)] = {"us_per_step": round(ms * 1e3, 2), "algorithmic_bytes": nbytes,
+                                             "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                             "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4),
+                                             "impl": pd.impl_info_str()}
     return res
 
 

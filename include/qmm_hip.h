@@ -227,10 +227,14 @@ typedef struct {
     void *dst;
     const void *mask, *scale;
     const void *k_scale, *k_zp, *v_scale, *v_zp;
+    void *scratch; /* qmm_sdpa_scratch_size() bytes, or NULL when 0 */
 } qmm_sdpa_args_t;
 
 QMM_API int qmm_sdpa_supports(const qmm_sdpa_desc_t *desc);
 QMM_API const char *qmm_sdpa_impl_name(const qmm_sdpa_desc_t *desc);
+/* Bytes of scratch a launch needs: non-zero only for at most 16 queries with
+ * enough keys to be cut into several ranges (partial results per range). */
+QMM_API size_t qmm_sdpa_scratch_size(const qmm_sdpa_desc_t *desc);
 QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
         const qmm_sdpa_args_t *args, void *hip_stream);
 

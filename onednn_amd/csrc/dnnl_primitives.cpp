@@ -523,6 +523,8 @@ usage_t arg_usage(const pd_impl_t &pd, int arg) {
                 {DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_VALUES, pd.sd.v_zp.set}};
         for (auto &e : q)
             if (arg == e.arg) return e.set ? usage_t::input : usage_t::unused;
+        if (arg == DNNL_ARG_SCRATCHPAD)
+            return pd.scratchpad.ndims ? usage_t::output : usage_t::unused;
         return usage_t::unused;
     } else {
         if (arg == DNNL_ARG_FROM) return usage_t::input;
@@ -1324,6 +1326,12 @@ dnnl_status_t sdpa_primitive_desc_create(dnnl_primitive_desc_t *out,
     if (qmm_sdpa_supports(&S) != QMM_OK) return dnnl_unimplemented;
     pd->impl = 0;
     pd->impl_name = qmm_sdpa_impl_name(&S);
+    pd->scratch_bytes = qmm_sdpa_scratch_size(&S);
+    if (pd->scratch_bytes
+            && pd->attr.scratchpad_mode == dnnl_scratchpad_mode_user) {
+        dnnl_dims_t dims = {(int64_t)pd->scratch_bytes};
+        md_init_plain(pd->scratchpad, 1, dims, dnnl_u8, nullptr);
+    }
     dnnl_primitive_desc *h = new (std::nothrow) dnnl_primitive_desc();
     if (!h) return dnnl_out_of_memory;
     h->p = pd;
@@ -1357,6 +1365,16 @@ dnnl_status_t dnnl_primitive_create(
                 delete p;
                 return dnnl_out_of_memory;
             }
+        }
+    }
+    if (p->pd->kind == kind_sdpa && p->pd->scratch_bytes
+            && p->pd->attr.scratchpad_mode == dnnl_scratchpad_mode_library) {
+        const dnnl_engine *eng = p->pd->engine;
+        if (eng->device < 0 || hipSetDevice(eng->device) != hipSuccess
+                || hipMalloc(&p->lib_scratch, p->pd->scratch_bytes)
+                        != hipSuccess) {
+            delete p;
+            return eng->device < 0 ? dnnl_runtime_error : dnnl_out_of_memory;
         }
     }
     *primitive = p;
@@ -1489,6 +1507,8 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         A.k_zp = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_KEYS);
         A.v_scale = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_VALUES);
         A.v_zp = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_VALUES);
+        A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
+                                        : lib_scratch;
         st = qmm_sdpa_launch(&pd.sd, &A, stream->hip_stream);
     } else if (pd.kind == dnnl_softmax) {
         if (pd.src.has_zero_dim()) return dnnl_success;

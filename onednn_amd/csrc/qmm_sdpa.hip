@@ -27,6 +27,8 @@
 #include <hip/hip_runtime.h>
 #include <string.h>
 
+#include <algorithm>
+
 #include "qmm_device.hpp"
 #include "qmm_hip.h"
 
@@ -67,6 +69,10 @@ struct sdpa_params_t {
     int32_t kv_dt; // dt_f16, dt_s8, dt_u8
     int32_t ks_dt, kz_dt, vs_dt, vz_dt;
     int32_t pair_halves; // the grid fits the chip at once: see the kernel
+    // few queries (decode): the keys are cut into nsplit ranges of tps tiles
+    int32_t nsplit, tps;
+    int32_t fastq, pad2_; // f16 scales and 8-bit zero points: f16 dequantisation
+    float *part; // [head][split][16 queries][D + 2]: O (unnormalised), m, l
 };
 
 // Lanes that differ only in their 16-lane row hold parts of one query. The two
@@ -98,6 +104,30 @@ QMM_D float ld_zp(int dt, const void *p, int64_t i) {
     return dt == dt_s8  ? (float)((const int8_t *)p)[i]
             : dt == dt_u8 ? (float)((const uint8_t *)p)[i]
                           : (float)((const int32_t *)p)[i];
+}
+
+// Eight cache bytes -> eight f16 values scale * (x - zero_point), in f16
+// arithmetic: byte b behind the exponent pattern 0x64 is the f16 number
+// 1024 + b, (1024 + b) - (1024 + z) is exact (integers up to 2048 are f16
+// numbers), and an f16 scale times that small integer has at most 20
+// significant bits, so rounding the f16 product is the same single rounding as
+// f16(f32 product): the values of the reference's dequantizing reorder, at 1.5
+// instructions per element. `raw`: bytes with the sign bit already flipped for
+// s8; zb: zero point (+ 128 for s8), within [0, 1023].
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+QMM_D uint4 dequant8_f16(uint32_t w0, uint32_t w1, float s1, float zb) {
+    const h2 off = h2 {(_Float16)(1024.f + zb), (_Float16)(1024.f + zb)};
+    const h2 sc = h2 {(_Float16)s1, (_Float16)s1};
+    const uint32_t w[2] = {w0, w1};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t m = __builtin_amdgcn_perm(
+                0x64646464u, w[j >> 1], (j & 1) ? 0x04030402u : 0x04010400u);
+        const h2 v = (__builtin_bit_cast(h2, m) - off) * sc;
+        o[j] = __builtin_bit_cast(uint32_t, v);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // QUANT: K / V are an 8-bit cache; MASKED: an explicit mask tensor is added
@@ -235,6 +265,10 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                 const float vzb = pvz[n] + (sgn ? 128.f : 0.f);
                 const uint32_t kw[2] = {pk[n].x ^ flip, pk[n].y ^ flip};
                 const uint32_t vw[2] = {pv[n].x ^ flip, pv[n].y ^ flip};
+                if (p.fastq) {
+                    kv = dequant8_f16(kw[0], kw[1], pks[n], kzb);
+                    vv = dequant8_f16(vw[0], vw[1], pvs[n], vzb);
+                } else {
                 uint32_t kh[8], vh[8];
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -249,6 +283,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                         kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
                 vv = make_uint4(vh[0] | (vh[1] << 16), vh[2] | (vh[3] << 16),
                         vh[4] | (vh[5] << 16), vh[6] | (vh[7] << 16));
+                }
             }
             if (kt * SDPA_KT + kk >= p.S) {
                 // keys past the end: zero, so that probability 0 x V stays 0
@@ -415,6 +450,357 @@ sdpa_f16_kernel(const sdpa_params_t p) {
     }
 }
 
+
+// ---- few queries (at most 16 per head: the decode step) ----------------------
+// One workgroup per (head, key range); its four waves take the range's key
+// tiles in turn, each with its own running maximum, sum and accumulators and
+// its own piece of LDS (the V tile it transposes): no barrier until the end,
+// where wave 0 merges the four states. A launch is then heads x splits
+// workgroups streaming K and V once, instead of one workgroup per head walking
+// all keys. With more than one split the merged state goes to the scratchpad
+// (unnormalised accumulators, maximum, sum per query) and sdpa_combine_kernel
+// finishes.
+template <int DC, bool QUANT, bool MASKED>
+__global__ void __launch_bounds__(SDPA_WAVES * 64)
+sdpa_decode_kernel(const sdpa_params_t p) {
+    constexpr int D = 32 * DC;
+    constexpr int DVB = D / 16;
+    constexpr int V_PITCH = D * 2 + 32;
+    constexpr int ST = D + 2; // floats of one query's state
+    __shared__ __attribute__((aligned(16))) uint8_t lds_v4[SDPA_WAVES][SDPA_KT * V_PITCH];
+    __shared__ float lds_st[SDPA_WAVES][16 * ST];
+    // a tile's 32 key scales and zero points of K and of V, per wave
+    __shared__ float lds_q[SDPA_WAVES][4 * SDPA_KT];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, c = lane >> 4;
+    const int head = blockIdx.x, split = blockIdx.y;
+    const int b1 = head % p.B1, b0 = head / p.B1;
+    const int kb0 = b0 / p.kv_div0, kb1 = b1 / p.kv_div1;
+    const uint16_t *Qb = p.Q + b0 * p.q.b0 + b1 * p.q.b1;
+    const uint8_t *Kb8 = (const uint8_t *)p.K, *Vb8 = (const uint8_t *)p.V;
+    const int64_t k_base = kb0 * p.k.b0 + kb1 * p.k.b1;
+    const int64_t v_base = kb0 * p.v.b0 + kb1 * p.v.b1;
+    const int64_t qz_base = kb0 * p.qz_b0 + kb1 * p.qz_b1;
+    uint8_t *lds_v = lds_v4[wave];
+
+    const int q = r; // the single 16-query block; rows past Qn repeat the last
+    v8h qf[DC];
+#pragma unroll
+    for (int dc = 0; dc < DC; dc++)
+        qf[dc] = *(const v8h *)(Qb + (int64_t)min(q, p.Qn - 1) * p.q.row + dc * 32
+                + c * 8);
+    float sc = 1.f;
+    if (p.scale) {
+        sc = load_float(p.scale_dt, p.scale, 0);
+        if (p.invert_scale) sc = 1.f / sc;
+    }
+    constexpr float L2E = 1.44269504088896340736f;
+    const float sc2 = sc * L2E;
+    const uint8_t *mask_b = nullptr;
+    if (MASKED) {
+        const size_t msz = p.mask_dt == dt_f32 ? 4 : 2;
+        mask_b = (const uint8_t *)p.mask + (b0 * p.m.b0 + b1 * p.m.b1) * msz;
+    }
+
+    v4f oacc[DVB];
+#pragma unroll
+    for (int d = 0; d < DVB; d++) oacc[d] = v4f {0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    int n_tiles = (p.S + SDPA_KT - 1) / SDPA_KT;
+    if (p.causal) n_tiles = min(n_tiles, (p.Qn - 1) / SDPA_KT + 1);
+    const int t_begin = split * p.tps, t_end = min(n_tiles, t_begin + p.tps);
+
+    // K fragments straight from memory in operand order (lane (r, c): key
+    // 16 kb + r, 8 values at 32 dc + 8 c); V rows through the wave's LDS piece
+    uint4 kr[2][DC], vr[D / 16];
+    float qsz[2]; // lanes 0..31: K scale, zero point of key lane; 32..63: V's
+    float *qz = lds_q[wave];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const int key = min(kt * SDPA_KT + kb * 16 + r, p.S - 1);
+#pragma unroll
+            for (int dc = 0; dc < DC; dc++) {
+                if (!QUANT) {
+                    kr[kb][dc] = *(const uint4 *)((const uint16_t *)Kb8 + k_base
+                            + key * p.k.row + dc * 32 + c * 8);
+                } else {
+                    const uint2 w = *(const uint2 *)(Kb8 + k_base + key * p.k.row
+                            + dc * 32 + c * 8);
+                    kr[kb][dc] = make_uint4(w.x, w.y, 0, 0);
+                }
+            }
+        }
+        if (QUANT) {
+            // one scale and one zero point per lane: the tile's 32 keys, K's in
+            // the lower half of the wave, V's in the upper
+            const int key = min(kt * SDPA_KT + (lane & 31), p.S - 1);
+            const bool up = lane >= 32;
+            const void *sp = up ? p.v_scale : p.k_scale;
+            const void *zp = up ? p.v_zp : p.k_zp;
+            qsz[0] = sp ? ld_scale(up ? p.vs_dt : p.ks_dt, sp, qz_base + key) : 1.f;
+            qsz[1] = zp ? ld_zp(up ? p.vz_dt : p.kz_dt, zp, qz_base + key) : 0.f;
+        }
+        // V: lane l carries chunk (l % (D / 8)) of key (l / (D / 8)) + 64 / (D / 8) * n
+#pragma unroll
+        for (int n = 0; n < D / 16; n++) {
+            const int i = lane + 64 * n;
+            const int kk = i / (D / 8), ch = i % (D / 8);
+            const int key = min(kt * SDPA_KT + kk, p.S - 1);
+            if (!QUANT) {
+                vr[n] = *(const uint4 *)((const uint16_t *)Vb8 + v_base
+                        + key * p.v.row + ch * 8);
+            } else {
+                const uint2 w = *(const uint2 *)(Vb8 + v_base + key * p.v.row
+                        + ch * 8);
+                vr[n] = make_uint4(w.x, w.y, 0, 0);
+            }
+        }
+    };
+    auto dequant8 = [&](const uint4 &raw, float s1, float z1) {
+        const bool sgn = p.kv_dt == dt_s8;
+        const uint32_t flip = sgn ? 0x80808080u : 0u;
+        const float zb = z1 + (sgn ? 128.f : 0.f);
+        const uint32_t w[2] = {raw.x ^ flip, raw.y ^ flip};
+        if (p.fastq) return dequant8_f16(w[0], w[1], s1, zb);
+        uint32_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float f = (float)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
+            h[j] = __builtin_bit_cast(uint16_t, (_Float16)(s1 * (f - zb)));
+        }
+        return make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+    };
+
+    int kt = t_begin + wave;
+    if (kt < t_end) fetch(kt);
+    for (; kt < t_end; kt += SDPA_WAVES) {
+        const int key0 = kt * SDPA_KT;
+        // this tile's operands out of the request registers
+        if (QUANT) {
+            // [K scale | V scale | K zero point | V zero point] x 32 keys
+            qz[lane] = qsz[0];
+            qz[64 + lane] = qsz[1];
+        }
+        v8h ka[2][DC];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int dc = 0; dc < DC; dc++) {
+                uint4 w = QUANT ? dequant8(kr[kb][dc], qz[kb * 16 + r],
+                                          qz[64 + kb * 16 + r])
+                                : kr[kb][dc];
+                if (key0 + kb * 16 + r >= p.S) w = make_uint4(0, 0, 0, 0);
+                ka[kb][dc] = __builtin_bit_cast(v8h, w);
+            }
+#pragma unroll
+        for (int n = 0; n < D / 16; n++) {
+            const int i = lane + 64 * n;
+            const int kk = i / (D / 8), ch = i % (D / 8);
+            uint4 w = QUANT ? dequant8(vr[n], qz[32 + kk], qz[96 + kk]) : vr[n];
+            if (key0 + kk >= p.S) w = make_uint4(0, 0, 0, 0);
+            *(uint4 *)(lds_v + kk * V_PITCH + ch * 16) = w;
+        }
+        if (kt + SDPA_WAVES < t_end) fetch(kt + SDPA_WAVES);
+
+        v4f st[2] = {v4f {0.f, 0.f, 0.f, 0.f}, v4f {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int dc = 0; dc < DC; dc++)
+                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        ka[kb][dc], qf[dc], st[kb], 0, 0, 0);
+        float sv[8];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) sv[kb * 4 + i] = st[kb][i] * sc2;
+        if (MASKED) {
+            const int64_t mrow = (int64_t)min(q, p.Qn - 1) * p.m.row;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = min(key0 + kb * 16 + 4 * c + i, p.S - 1);
+                    const int64_t mo = mrow + key * p.m_col;
+                    sv[kb * 4 + i] += L2E
+                            * (p.mask_dt == dt_f32
+                                            ? ((const float *)mask_b)[mo]
+                                            : (float)((const _Float16 *)mask_b)[mo]);
+                }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int key = key0 + kb * 16 + 4 * c + i;
+                if (key >= p.S || (p.causal && key > q)) sv[kb * 4 + i] = -INFINITY;
+            }
+        float mt = sv[0];
+#pragma unroll
+        for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
+        mt = rows_max(mt);
+        const float m_new = fmaxf(m_run, mt);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        m_run = m_new;
+        float ls = 0.f;
+        _Float16 ph[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float pv1 = __builtin_amdgcn_exp2f(sv[i] - m_use);
+            ls += pv1;
+            ph[i] = (_Float16)pv1;
+        }
+        l_run = l_run * alpha + ls;
+        const v8h pb = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
+#pragma unroll
+        for (int d = 0; d < DVB; d++) {
+            oacc[d] *= alpha;
+            const uint8_t *va = lds_v + (4 * c + (r >> 2)) * V_PITCH
+                    + (d * 16 + 4 * (r & 3)) * 2;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)va);
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)(va + 16 * V_PITCH));
+            typedef short v8s __attribute__((ext_vector_type(8)));
+            const v8h a = __builtin_bit_cast(v8h,
+                    v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+            oacc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, oacc[d], 0, 0, 0);
+        }
+    }
+
+    // ---- merge the four waves' states: query r, accumulator rows d = 16 dv + 4 c + i
+    const float l_wave = rows_sum(l_run);
+    float *mine = lds_st[wave] + r * ST;
+#pragma unroll
+    for (int d = 0; d < DVB; d++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) mine[d * 16 + 4 * c + i] = oacc[d][i];
+    if (c == 0) {
+        mine[D] = m_run;
+        mine[D + 1] = l_wave;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < SDPA_WAVES; w++) m_all = fmaxf(m_all, lds_st[w][r * ST + D]);
+    const float m_use = m_all == -INFINITY ? 0.f : m_all;
+    float l_all = 0.f, wgt[SDPA_WAVES];
+#pragma unroll
+    for (int w = 0; w < SDPA_WAVES; w++) {
+        wgt[w] = __builtin_amdgcn_exp2f(lds_st[w][r * ST + D] - m_use);
+        l_all += wgt[w] * lds_st[w][r * ST + D + 1];
+    }
+    if (q >= p.Qn) return;
+    if (p.nsplit == 1) {
+        uint16_t *Ob = p.dst + b0 * p.o.b0 + b1 * p.o.b1 + (int64_t)q * p.o.row;
+#pragma unroll
+        for (int d = 0; d < DVB; d++) {
+            uint16_t h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float o = 0.f;
+#pragma unroll
+                for (int w = 0; w < SDPA_WAVES; w++)
+                    o += wgt[w] * lds_st[w][r * ST + d * 16 + 4 * c + i];
+                h[i] = __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
+            }
+            *(uint2 *)(Ob + d * 16 + 4 * c) = make_uint2(
+                    h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+        }
+    } else {
+        float *out = p.part + (((int64_t)head * p.nsplit + split) * 16 + q) * ST;
+#pragma unroll
+        for (int d = 0; d < DVB; d++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float o = 0.f;
+#pragma unroll
+                for (int w = 0; w < SDPA_WAVES; w++)
+                    o += wgt[w] * lds_st[w][r * ST + d * 16 + 4 * c + i];
+                out[d * 16 + 4 * c + i] = o;
+            }
+        if (c == 0) {
+            out[D] = m_all;
+            out[D + 1] = l_all;
+        }
+    }
+}
+
+// the splits' states of one (head, query) -> dst. The weights of the splits
+// are formed once in LDS; a thread then owns one d and adds the splits'
+// accumulators with independent loads.
+constexpr int SDPA_MAX_SPLIT = 256;
+__global__ void __launch_bounds__(128)
+sdpa_combine_kernel(const sdpa_params_t p, const int D) {
+    __shared__ float w_s[SDPA_MAX_SPLIT];
+    __shared__ float red[2];
+    const int head = blockIdx.x, q = blockIdx.y, t = threadIdx.x;
+    const int b1 = head % p.B1, b0 = head / p.B1;
+    const int ST = D + 2;
+    const float *st = p.part + ((int64_t)head * p.nsplit * 16 + q) * ST;
+    // every thread finds the maximum itself (at most 256 values from L2)
+    float m_all = -INFINITY;
+    for (int s1 = t; s1 < p.nsplit; s1 += 128)
+        m_all = fmaxf(m_all, st[(int64_t)s1 * 16 * ST + D]);
+#pragma unroll
+    for (int o = 32; o; o >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, o));
+    if ((t & 63) == 0) red[t >> 6] = m_all;
+    __syncthreads();
+    m_all = fmaxf(red[0], red[1]);
+    const float m_use = m_all == -INFINITY ? 0.f : m_all;
+    float l_part = 0.f;
+    for (int s1 = t; s1 < p.nsplit; s1 += 128) {
+        const float *e = st + (int64_t)s1 * 16 * ST;
+        const float w = __builtin_amdgcn_exp2f(e[D] - m_use);
+        w_s[s1] = w;
+        l_part += w * e[D + 1];
+    }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) l_part += __shfl_xor(l_part, o);
+    __syncthreads(); // red[] has been read by everyone
+    if ((t & 63) == 0) red[t >> 6] = l_part;
+    __syncthreads();
+    const float l_all = red[0] + red[1];
+    if (t < D) {
+        float o = 0.f;
+#pragma unroll 8
+        for (int s1 = 0; s1 < p.nsplit; s1++)
+            o += w_s[s1] * st[(int64_t)s1 * 16 * ST + t];
+        p.dst[b0 * p.o.b0 + b1 * p.o.b1 + (int64_t)q * p.o.row + t]
+                = __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
+    }
+}
+
+// how a decode-sized problem is cut over the keys
+struct sdpa_split_t {
+    int nsplit, tps;
+};
+sdpa_split_t decode_split(int64_t heads, int64_t S, int64_t Qn, bool causal) {
+    int64_t tiles = (S + SDPA_KT - 1) / SDPA_KT;
+    if (causal) tiles = std::min<int64_t>(tiles, (Qn - 1) / SDPA_KT + 1);
+    // enough workgroups to fill the chip twice, at least one tile per wave
+    int64_t want = std::max<int64_t>(1, 512 / std::max<int64_t>(1, heads));
+    int64_t tps = std::max<int64_t>(SDPA_WAVES, (tiles + want - 1) / want);
+    tps = (tps + SDPA_WAVES - 1) / SDPA_WAVES * SDPA_WAVES;
+    sdpa_split_t r;
+    r.tps = (int)tps;
+    r.nsplit = (int)std::max<int64_t>(1, (tiles + tps - 1) / tps);
+    if (r.nsplit > SDPA_MAX_SPLIT) {
+        tps = (tiles + SDPA_MAX_SPLIT - 1) / SDPA_MAX_SPLIT;
+        tps = (tps + SDPA_WAVES - 1) / SDPA_WAVES * SDPA_WAVES;
+        r.tps = (int)tps;
+        r.nsplit = (int)((tiles + tps - 1) / tps);
+    }
+    return r;
+}
+
 // ---- host side ---------------------------------------------------------------
 bool outer_strides(const qmm_tensor_t &t, sdpa_strides_t &s) {
     const int nd = t.ndims;
@@ -539,6 +925,10 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     p.invert_scale = d.invert_scale;
     p.causal = d.causal;
     p.kv_dt = d.k.dt;
+    p.fastq = quant && (!d.k_scale.set || d.k_scale.dt == dt_f16)
+            && (!d.v_scale.set || d.v_scale.dt == dt_f16)
+            && (!d.k_zp.set || d.k_zp.dt == dt_s8 || d.k_zp.dt == dt_u8)
+            && (!d.v_zp.set || d.v_zp.dt == dt_s8 || d.v_zp.dt == dt_u8);
     p.ks_dt = d.k_scale.dt;
     p.kz_dt = d.k_zp.dt;
     p.vs_dt = d.v_scale.dt;
@@ -561,6 +951,16 @@ int qmm_sdpa_supports(const qmm_sdpa_desc_t *desc) {
 
 const char *qmm_sdpa_impl_name(const qmm_sdpa_desc_t *desc) {
     return desc && supported(*desc, nullptr) ? "hip:gfx950:sdpa_f16" : "";
+}
+
+size_t qmm_sdpa_scratch_size(const qmm_sdpa_desc_t *desc) {
+    sdpa_params_t p;
+    if (!desc || !supported(*desc, &p) || p.Qn > 16) return 0;
+    const sdpa_split_t sp
+            = decode_split((int64_t)p.B0 * p.B1, p.S, p.Qn, p.causal != 0);
+    if (sp.nsplit <= 1) return 0;
+    const int64_t D = desc->q.dims[desc->q.ndims - 1];
+    return (size_t)p.B0 * p.B1 * sp.nsplit * 16 * (D + 2) * sizeof(float);
 }
 
 int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
@@ -589,6 +989,36 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.k_zp = desc->k_zp.set ? args->k_zp : nullptr;
     p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
+    const bool d128 = desc->q.dims[desc->q.ndims - 1] == 128;
+    const bool qn = p.kv_dt != dt_f16, mk = p.mask != nullptr;
+    if (p.Qn <= 16) {
+        const sdpa_split_t sp
+                = decode_split((int64_t)p.B0 * p.B1, p.S, p.Qn, p.causal != 0);
+        p.nsplit = sp.nsplit;
+        p.tps = sp.tps;
+        p.part = (float *)args->scratch;
+        if (p.nsplit > 1 && !p.part) return QMM_INVALID_ARGUMENTS;
+        const dim3 dgrid((unsigned)(p.B0 * p.B1), (unsigned)p.nsplit);
+        auto god = [&](auto kern) {
+            hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
+                    (hipStream_t)hip_stream, p);
+        };
+        switch ((d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
+            case 0: god(sdpa_decode_kernel<2, false, false>); break;
+            case 1: god(sdpa_decode_kernel<2, false, true>); break;
+            case 2: god(sdpa_decode_kernel<2, true, false>); break;
+            case 3: god(sdpa_decode_kernel<2, true, true>); break;
+            case 4: god(sdpa_decode_kernel<4, false, false>); break;
+            case 5: god(sdpa_decode_kernel<4, false, true>); break;
+            case 6: god(sdpa_decode_kernel<4, true, false>); break;
+            default: god(sdpa_decode_kernel<4, true, true>); break;
+        }
+        if (p.nsplit > 1)
+            hipLaunchKernelGGL(sdpa_combine_kernel,
+                    dim3((unsigned)(p.B0 * p.B1), (unsigned)p.Qn), dim3(128), 0,
+                    (hipStream_t)hip_stream, p, d128 ? 128 : 64);
+        return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
+    }
     const dim3 grid((unsigned)(p.B0 * p.B1),
             (unsigned)((p.Qn + SDPA_QT - 1) / SDPA_QT));
     int dev = 0, cus = 256;
@@ -597,8 +1027,6 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
                 &cus, hipDeviceAttributeMultiprocessorCount, dev);
     p.pair_halves = p.causal && grid.y % 2 == 0
             && (int64_t)grid.x * grid.y <= (int64_t)SDPA_MIN_BLOCKS * cus;
-    const bool d128 = desc->q.dims[desc->q.ndims - 1] == 128;
-    const bool qn = p.kv_dt != dt_f16, mk = p.mask != nullptr;
     auto go = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);

@@ -178,6 +178,74 @@ def test_quantized_cache(ctx, kv_dt, with_zp, Qn):
     assert bad <= total * 0.0006
 
 
+@pytest.mark.parametrize("Qn,S,D,heads,kvh,mkind,quant", [
+    (1, 4096, 128, 8, 0, "none", False), (1, 2049, 128, 32, 8, "none", True), (5, 1500, 64, 4, 0, "2d", False),
+    (16, 3000, 128, 6, 2, "causal", False), (2, 640, 64, 40, 0, "1d", True), (1, 96, 128, 2, 0, "none", False),
+], ids=str)
+def test_few_queries_split_over_the_keys(ctx, Qn, S, D, heads, kvh, mkind, quant):
+    """At most 16 queries per head (the decode step): the keys are cut into ranges, one workgroup each, the ranges'
+    running maxima, sums and accumulators merged afterwards (in the scratchpad when there are several ranges)."""
+    say("sdpa decode Qn=%d S=%d D=%d heads=%d kv=%d mask=%s quant=%s" % (Qn, S, D, heads, kvh, mkind, quant))
+    r = np.random.default_rng(Qn * 7 + S)
+    kh = kvh or heads
+    q = f16(r.standard_normal((1, heads, Qn, D)))
+    scale = 1.0 / np.sqrt(D)
+    mask = None
+    if mkind == "2d":
+        mask = (r.standard_normal((1, 1, Qn, S)) * 2).astype(np.float32)
+        mask[..., 3::7] = -np.inf
+    elif mkind == "1d":
+        mask = (r.standard_normal((1, 1, 1, S)) * 2).astype(np.float32)
+    if quant:
+        kq = r.integers(-128, 128, (1, kh, S, D)).astype(np.int8)
+        vq = r.integers(-128, 128, (1, kh, S, D)).astype(np.int8)
+        ksc, vsc = f16(r.uniform(0.005, 0.02, (kh, S))), f16(r.uniform(0.005, 0.02, (kh, S)))
+        kzp, vzp = r.integers(-6, 7, (kh, S)).astype(np.int8), r.integers(-6, 7, (kh, S)).astype(np.int8)
+        got = run_sdpa(ctx, q, kq, vq, scale=scale, mask=mask, causal=(mkind == "causal"), kv_heads=kvh, kv_dt=dt.s8,
+                       k_q=(0b1110, (D, 1), dt.f16, ksc, dt.s8, kzp), v_q=(0b1110, (1, D), dt.f16, vsc, dt.s8, vzp))
+        kd, vd = np.zeros((1, kh, S, D), np.uint16), np.zeros((1, kh, S, D), np.uint16)
+        for raw, sc, zp, outd in ((kq, ksc, kzp, kd), (vq, vsc, vzp, vd)):
+            O.reorder(O.Tensor(dt.s8, [1, kh, S, D], raw), O.Tensor(dt.f16, [1, kh, S, D], outd),
+                      src_scale=O.Quant(0b1110, dt.f16, sc, (1, D)), src_zp=O.Quant(0b1110, dt.s8, zp, (1, D)))
+        k64, v64 = f16_to_f64(kd), f16_to_f64(vd)
+    else:
+        k, v = f16(r.standard_normal((1, kh, S, D))), f16(r.standard_normal((1, kh, S, D)))
+        got = run_sdpa(ctx, q, k, v, scale=scale, mask=mask, causal=(mkind == "causal"), kv_heads=kvh)
+        k64, v64 = f16_to_f64(k), f16_to_f64(v)
+    s_eff = float(f16_to_f64(f16(np.array([scale])))[0])
+    gold = attention64(f16_to_f64(q), np.swapaxes(k64, -1, -2), v64, s_eff,
+                       None if mask is None else mask.astype(np.float64), mkind == "causal", heads // kh)
+    bad, total, worst = reference_rule(f16_to_f64(got), gold)
+    print("[sdpa decode] %d of %d outside the threshold, max diff %.2e" % (bad, total, worst))
+    assert bad <= total * 0.0006
+
+
+def test_few_queries_with_a_user_scratchpad(ctx):
+    """The ranges' partial results live in the primitive's scratchpad: library-owned by default, the user's in
+    scratchpad_mode::user (filled with NaN patterns here, to show that nothing of it is read before it is written)."""
+    eng, strm = ctx
+    H, S, D = 16, 4096, 128
+    r = np.random.default_rng(5)
+    q, k, v = f16(r.standard_normal((1, H, 1, D))), f16(r.standard_normal((1, H, S, D))), f16(r.standard_normal((1, H, S, D)))
+    attr = dnnl.primitive_attr()
+    attr.set_scratchpad_mode(dnnl.scratchpad_mode.user)
+    q_md = memory.desc([1, H, 1, D], dt.f16, T("abcd"))
+    kt_md = memory.desc([1, H, D, S], dt.f16, T("abdc"))
+    v_md = memory.desc([1, H, S, D], dt.f16, T("abcd"))
+    pd = dnnl.sdpa.primitive_desc(eng, q_md, kt_md, v_md, None, dt.undef, q_md, False, 0, False, attr)
+    smd = pd.scratchpad_desc()
+    assert smd.get_size() > 0
+    scratch = memory(smd, eng).write(np.full(smd.get_size(), 0xFF, np.uint8))
+    out = memory(q_md, eng)
+    dnnl.sdpa(pd).execute(strm, {dnnl.DNNL_ARG_QUERIES: memory(q_md, eng).write(q), dnnl.DNNL_ARG_KEYS: memory(kt_md, eng).write(k),
+                                 dnnl.DNNL_ARG_VALUES: memory(v_md, eng).write(v), dnnl.DNNL_ARG_DST: out,
+                                 dnnl.DNNL_ARG_SCRATCHPAD: scratch})
+    strm.wait()
+    gold = attention64(f16_to_f64(q), np.swapaxes(f16_to_f64(k), -1, -2), f16_to_f64(v), 1.0, None, False, 1)
+    bad, total, worst = reference_rule(f16_to_f64(out.read(np.uint16, (1, H, 1, D))), gold)
+    assert bad <= total * 0.0006, (bad, worst)
+
+
 def test_fused_kernel_against_the_primitive_chain_on_the_device(ctx):
     """Same operands through matmul -> softmax -> matmul (generic kernels, f32 scores in memory) and through the
     fused kernel: the two device results agree under the reference test's rule."""
