@@ -28,6 +28,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 
 #include "qmm_device.hpp"
 #include "qmm_hip.h"
@@ -336,6 +337,32 @@ sdpa_f16_kernel(const sdpa_params_t p) {
 #pragma unroll
         for (int qb = 0; qb < SDPA_QB; qb++) {
             const int q = q_wave + qb * 16 + r;
+            if (!MASKED && !edge && sc2 > 0.f) {
+                // interior tile, nothing added to the scores: the maximum is
+                // taken on the raw products and the scale rides in the
+                // exponent's multiply-add (one instruction per score less)
+                float mr = fmaxf(fmaxf(st[qb][0][0], st[qb][0][1]),
+                        fmaxf(st[qb][0][2], st[qb][0][3]));
+                mr = fmaxf(mr, fmaxf(fmaxf(st[qb][1][0], st[qb][1][1]),
+                                       fmaxf(st[qb][1][2], st[qb][1][3])));
+                const float m_new = fmaxf(m_run[qb], rows_max(mr) * sc2);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+                rescale |= m_new != m_run[qb];
+                alpha_q[qb] = alpha;
+                m_run[qb] = m_new;
+                float ls = 0.f;
+                _Float16 ph[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float pv1 = __builtin_amdgcn_exp2f(
+                            __builtin_fmaf(st[qb][i >> 2][i & 3], sc2, -m_new));
+                    ls += pv1;
+                    ph[i] = (_Float16)pv1;
+                }
+                l_run[qb] = l_run[qb] * alpha + ls;
+                pb[qb] = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
+                continue;
+            }
             float sv[8];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
@@ -1021,10 +1048,18 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     }
     const dim3 grid((unsigned)(p.B0 * p.B1),
             (unsigned)((p.Qn + SDPA_QT - 1) / SDPA_QT));
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess)
-        (void)hipDeviceGetAttribute(
-                &cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (grid.y > 65535) return QMM_UNIMPLEMENTED;
+    // compute units of the device (asked once; every MI355X has the same)
+    static std::atomic<int> cu_count {0};
+    int cus = cu_count.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        int dev = 0;
+        cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess)
+            (void)hipDeviceGetAttribute(
+                    &cus, hipDeviceAttributeMultiprocessorCount, dev);
+        cu_count.store(cus, std::memory_order_relaxed);
+    }
     p.pair_halves = p.causal && grid.y % 2 == 0
             && (int64_t)grid.x * grid.y <= (int64_t)SDPA_MIN_BLOCKS * cus;
     auto go = [&](auto kern) {
