@@ -143,6 +143,21 @@ static int host_checks() {
             src_md, ip_wei, ip_bias, dst_md);
     CHECK(ipd.get_kind() == primitive::kind::inner_product);
     CHECK(ipd.bias_desc() == ip_bias);
+
+    // softmax forward descriptor: axis, algorithm, destination layout from any
+    memory::desc sm_src({4, 6, 32}, dt::f32, tag::abc);
+    softmax_forward::primitive_desc spd(eng, prop_kind::forward_inference,
+            algorithm::softmax_accurate, sm_src,
+            memory::desc({4, 6, 32}, dt::f16, tag::any), 2);
+    CHECK(spd.get_axis() == 2);
+    CHECK(spd.get_algorithm() == algorithm::softmax_accurate);
+    CHECK(spd.dst_desc() == memory::desc({4, 6, 32}, dt::f16, tag::abc));
+    thrown = false;
+    try {
+        softmax_forward::primitive_desc bad(eng, prop_kind::forward_inference,
+                algorithm::softmax_accurate, sm_src, sm_src, 3);
+    } catch (const error &e) { thrown = e.status == dnnl_invalid_arguments; }
+    CHECK(thrown);
     std::printf("host ok\n");
     return 0;
 }
@@ -247,6 +262,21 @@ static int gpu_checks() {
                         (long)m, (long)n, got32[m * N + n], want);
                 return 1;
             }
+        }
+    // softmax over rows of equal values: every probability is exactly 1 / 64
+    memory::desc sm_md({8, 64}, dt::f32, tag::ab);
+    softmax_forward::primitive_desc spd(eng, prop_kind::forward_inference,
+            algorithm::softmax_accurate, sm_md, sm_md, 1);
+    memory sm_src(sm_md, eng), sm_dst(sm_md, eng);
+    std::vector<float> ones(8 * 64, 3.25f);
+    upload(sm_src, ones);
+    softmax_forward(spd).execute(
+            strm, {{DNNL_ARG_SRC, sm_src}, {DNNL_ARG_DST, sm_dst}});
+    strm.wait();
+    for (float v : download<float>(sm_dst, 8 * 64))
+        if (v != 1.f / 64.f) {
+            std::printf("softmax mismatch: %g\n", v);
+            return 1;
         }
     std::printf("gpu ok\n");
     return 0;
