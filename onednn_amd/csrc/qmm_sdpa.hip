@@ -3,8 +3,9 @@
 // (the reference's internal sdpa primitive: src/common/sdpa_types.hpp:38-80,
 // semantics src/gpu/intel/ocl/ref_sdpa.cl:21-78; its test's gold path is the
 // matmul -> softmax -> matmul chain, tests/gtests/internals/test_sdpa.cpp:893-
-// 1043). Q, K, V, dst are f16; K and V may instead be an s8 / u8 cache with one
-// scale (and zero point) per key, dequantized to f16 as the chain's reorder
+// 1043). Q, K, V, dst are f16 or bf16 (the kernels' BF flag; the text below
+// says f16 for both); with f16, K and V may instead be an s8 / u8 cache with
+// one scale (and zero point) per key, dequantized to f16 as the chain's reorder
 // does: f16(scale * (x - zero_point)).
 //
 // The scores never leave the CU. A workgroup owns 128 queries of one head (four
@@ -48,6 +49,25 @@ constexpr int SDPA_KT = 32; // keys per tile
 #define SDPA_MIN_BLOCKS 2
 #endif
 typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+
+// BF: the 16-bit type of Q, K, V and dst is bf16 (else f16). Operands travel
+// as raw 16-byte vectors; only the MFMA and the conversions know the type.
+template <bool BF>
+QMM_D v4f mma16(const v8h &a, const v8h &b, const v4f &c) {
+    if constexpr (BF)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(v8b, a), __builtin_bit_cast(v8b, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+template <bool BF>
+QMM_D _Float16 cvt16(float v) { // the bits of v in the 16-bit type, carried as _Float16
+    if constexpr (BF)
+        return __builtin_bit_cast(_Float16, (__bf16)v); // v_cvt_pk_bf16_f32
+    else
+        return (_Float16)v;
+}
 
 struct sdpa_strides_t {
     int64_t b0, b1, row; // two outer dims, then the row dim (elements)
@@ -67,12 +87,12 @@ struct sdpa_params_t {
     int64_t qz_b0, qz_b1; // scale / zero-point index = kb0 * qz_b0 + kb1 * qz_b1 + key
     int32_t Qn, S;
     int32_t scale_dt, mask_dt, invert_scale, causal;
-    int32_t kv_dt; // dt_f16, dt_s8, dt_u8
+    int32_t kv_dt; // the queries' type, or dt_s8 / dt_u8
     int32_t ks_dt, kz_dt, vs_dt, vz_dt;
     int32_t pair_halves; // the grid fits the chip at once: see the kernel
     // few queries (decode): the keys are cut into nsplit ranges of tps tiles
     int32_t nsplit, tps;
-    int32_t fastq, pad2_; // f16 scales and 8-bit zero points: f16 dequantisation
+    int32_t fastq, bf; // f16 scales and 8-bit zero points: f16 dequantisation
     float *part; // [head][split][16 queries][D + 2]: O (unnormalised), m, l
 };
 
@@ -95,6 +115,14 @@ QMM_D float rows_sum(float v) {
     u = f2u(u2f(a.x) + u2f(a.y));
     const v2u b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return u2f(b.x) + u2f(b.y);
+}
+
+// the mask is f32 or one of the 16-bit types
+QMM_D float ld_mask(int dt, const void *p, int64_t i) {
+    if (dt == dt_f32) return ((const float *)p)[i];
+    const uint16_t h = ((const uint16_t *)p)[i];
+    return dt == dt_bf16 ? __uint_as_float((uint32_t)h << 16)
+                         : (float)__builtin_bit_cast(_Float16, h);
 }
 
 // the cache's scales are f16 or f32, its zero points s8, u8 or s32
@@ -132,7 +160,7 @@ QMM_D uint4 dequant8_f16(uint32_t w0, uint32_t w1, float s1, float zb) {
 }
 
 // QUANT: K / V are an 8-bit cache; MASKED: an explicit mask tensor is added
-template <int DC, bool QUANT, bool MASKED>
+template <int DC, bool QUANT, bool MASKED, bool BF>
 __global__ void __launch_bounds__(SDPA_WAVES * 64, SDPA_MIN_BLOCKS)
 sdpa_f16_kernel(const sdpa_params_t p) {
     constexpr int D = 32 * DC;
@@ -323,8 +351,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                         + dc * 64 + c * 16);
 #pragma unroll
                 for (int qb = 0; qb < SDPA_QB; qb++)
-                    st[qb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            a, qf[qb][dc], st[qb][kb], 0, 0, 0);
+                    st[qb][kb] = mma16<BF>(a, qf[qb][dc], st[qb][kb]);
             }
 
         // ---- scale, mask, online softmax (base 2), probabilities to f16.
@@ -357,7 +384,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                     const float pv1 = __builtin_amdgcn_exp2f(
                             __builtin_fmaf(st[qb][i >> 2][i & 3], sc2, -m_new));
                     ls += pv1;
-                    ph[i] = (_Float16)pv1;
+                    ph[i] = cvt16<BF>(pv1);
                 }
                 l_run[qb] = l_run[qb] * alpha + ls;
                 pb[qb] = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
@@ -380,9 +407,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                     for (int i = 0; i < 4; i++) {
                         const int key = min(key0 + kb * 16 + 4 * c + i, p.S - 1);
                         const int64_t mo = mrow + key * p.m_col;
-                        mv[kb * 4 + i] = p.mask_dt == dt_f32
-                                ? ((const float *)mask_b)[mo]
-                                : (float)((const _Float16 *)mask_b)[mo];
+                        mv[kb * 4 + i] = ld_mask(p.mask_dt, mask_b, mo);
                     }
 #pragma unroll
                 for (int i = 0; i < 8; i++) sv[i] += L2E * mv[i];
@@ -414,7 +439,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
             for (int i = 0; i < 8; i++) {
                 const float pv1 = __builtin_amdgcn_exp2f(sv[i] - m_use);
                 ls += pv1;
-                ph[i] = (_Float16)pv1;
+                ph[i] = cvt16<BF>(pv1);
             }
             l_run[qb] = l_run[qb] * alpha + ls;
             pb[qb] = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
@@ -452,8 +477,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                     v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
 #pragma unroll
             for (int qb = 0; qb < SDPA_QB; qb++)
-                oacc[qb][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        a, pb[qb], oacc[qb][d], 0, 0, 0);
+                oacc[qb][d] = mma16<BF>(a, pb[qb], oacc[qb][d]);
         }
         __syncthreads();
     }
@@ -470,7 +494,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
             uint16_t h[4];
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                h[i] = __builtin_bit_cast(uint16_t, (_Float16)(oacc[qb][d][i] / l));
+                h[i] = __builtin_bit_cast(uint16_t, cvt16<BF>(oacc[qb][d][i] / l));
             *(uint2 *)(Ob + (int64_t)q * p.o.row + d * 16 + 4 * c) = make_uint2(
                     h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
         }
@@ -487,7 +511,7 @@ sdpa_f16_kernel(const sdpa_params_t p) {
 // all keys. With more than one split the merged state goes to the scratchpad
 // (unnormalised accumulators, maximum, sum per query) and sdpa_combine_kernel
 // finishes.
-template <int DC, bool QUANT, bool MASKED>
+template <int DC, bool QUANT, bool MASKED, bool BF>
 __global__ void __launch_bounds__(SDPA_WAVES * 64)
 sdpa_decode_kernel(const sdpa_params_t p) {
     constexpr int D = 32 * DC;
@@ -639,8 +663,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int dc = 0; dc < DC; dc++)
-                st[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        ka[kb][dc], qf[dc], st[kb], 0, 0, 0);
+                st[kb] = mma16<BF>(ka[kb][dc], qf[dc], st[kb]);
         float sv[8];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
@@ -654,10 +677,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
                 for (int i = 0; i < 4; i++) {
                     const int key = min(key0 + kb * 16 + 4 * c + i, p.S - 1);
                     const int64_t mo = mrow + key * p.m_col;
-                    sv[kb * 4 + i] += L2E
-                            * (p.mask_dt == dt_f32
-                                            ? ((const float *)mask_b)[mo]
-                                            : (float)((const _Float16 *)mask_b)[mo]);
+                    sv[kb * 4 + i] += L2E * ld_mask(p.mask_dt, mask_b, mo);
                 }
         }
 #pragma unroll
@@ -681,7 +701,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
         for (int i = 0; i < 8; i++) {
             const float pv1 = __builtin_amdgcn_exp2f(sv[i] - m_use);
             ls += pv1;
-            ph[i] = (_Float16)pv1;
+            ph[i] = cvt16<BF>(pv1);
         }
         l_run = l_run * alpha + ls;
         const v8h pb = v8h {ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]};
@@ -697,7 +717,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
             typedef short v8s __attribute__((ext_vector_type(8)));
             const v8h a = __builtin_bit_cast(v8h,
                     v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
-            oacc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, oacc[d], 0, 0, 0);
+            oacc[d] = mma16<BF>(a, pb, oacc[d]);
         }
     }
 
@@ -736,7 +756,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
 #pragma unroll
                 for (int w = 0; w < SDPA_WAVES; w++)
                     o += wgt[w] * lds_st[w][r * ST + d * 16 + 4 * c + i];
-                h[i] = __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
+                h[i] = __builtin_bit_cast(uint16_t, cvt16<BF>(o / l_all));
             }
             *(uint2 *)(Ob + d * 16 + 4 * c) = make_uint2(
                     h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
@@ -801,7 +821,8 @@ sdpa_combine_kernel(const sdpa_params_t p, const int D) {
         for (int s1 = 0; s1 < p.nsplit; s1++)
             o += w_s[s1] * st[(int64_t)s1 * 16 * ST + t];
         p.dst[b0 * p.o.b0 + b1 * p.o.b1 + (int64_t)q * p.o.row + t]
-                = __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
+                = p.bf ? f32_to_bf16(o / l_all)
+                       : __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
     }
 }
 
@@ -854,9 +875,12 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     const int nd = d.q.ndims;
     if (nd < 2 || nd > 4) return false;
     if (d.k.ndims != nd || d.v.ndims != nd || d.dst.ndims != nd) return false;
-    if (d.q.dt != dt_f16 || d.dst.dt != dt_f16) return false;
+    if ((d.q.dt != dt_f16 && d.q.dt != dt_bf16) || d.dst.dt != d.q.dt) return false;
     if (d.k.dt != d.v.dt) return false;
-    if (d.k.dt != dt_f16 && d.k.dt != dt_s8 && d.k.dt != dt_u8) return false;
+    // K / V in the queries' type, or (f16 only) an 8-bit cache
+    if (d.k.dt != d.q.dt
+            && !(d.q.dt == dt_f16 && (d.k.dt == dt_s8 || d.k.dt == dt_u8)))
+        return false;
     const int64_t Qn = d.q.dims[nd - 2], D = d.q.dims[nd - 1];
     const int64_t S = d.k.dims[nd - 1];
     if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
@@ -898,7 +922,8 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     outer_strides(d.dst, p.o);
     if (d.mask.ndims) {
         if (d.mask.ndims != nd) return false;
-        if (d.mask.dt != dt_f16 && d.mask.dt != dt_f32) return false;
+        if (d.mask.dt != dt_f16 && d.mask.dt != dt_bf16 && d.mask.dt != dt_f32)
+            return false;
         // each dim equal to the scores' or 1 (broadcast)
         const int64_t want[4] = {p.B0, p.B1, Qn, S};
         int64_t ms[4] = {0, 0, 0, 0};
@@ -913,11 +938,12 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
         p.m_col = ms[3];
         p.mask_dt = d.mask.dt;
     }
-    if (d.scale_dt != dt_undef && d.scale_dt != dt_f16 && d.scale_dt != dt_f32)
+    if (d.scale_dt != dt_undef && d.scale_dt != dt_f16 && d.scale_dt != dt_bf16
+            && d.scale_dt != dt_f32)
         return false;
     // quantized cache: one scale / zero point per (batch, key), i.e. a mask
     // over the batch dims and the key dim with the head-size dim in one group
-    const bool quant = d.k.dt != dt_f16;
+    const bool quant = d.k.dt != d.q.dt;
     for (const qmm_quant_t *q : {&d.k_scale, &d.k_zp, &d.v_scale, &d.v_zp})
         if (q->set && !quant) return false;
     if (!quant_ok(d.k_scale, true) || !quant_ok(d.v_scale, true)
@@ -952,6 +978,7 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     p.invert_scale = d.invert_scale;
     p.causal = d.causal;
     p.kv_dt = d.k.dt;
+    p.bf = d.q.dt == dt_bf16;
     p.fastq = quant && (!d.k_scale.set || d.k_scale.dt == dt_f16)
             && (!d.v_scale.set || d.v_scale.dt == dt_f16)
             && (!d.k_zp.set || d.k_zp.dt == dt_s8 || d.k_zp.dt == dt_u8)
@@ -977,7 +1004,8 @@ int qmm_sdpa_supports(const qmm_sdpa_desc_t *desc) {
 }
 
 const char *qmm_sdpa_impl_name(const qmm_sdpa_desc_t *desc) {
-    return desc && supported(*desc, nullptr) ? "hip:gfx950:sdpa_f16" : "";
+    if (!desc || !supported(*desc, nullptr)) return "";
+    return desc->q.dt == dt_bf16 ? "hip:gfx950:sdpa_bf16" : "hip:gfx950:sdpa_f16";
 }
 
 size_t qmm_sdpa_scratch_size(const qmm_sdpa_desc_t *desc) {
@@ -1017,7 +1045,8 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
     const bool d128 = desc->q.dims[desc->q.ndims - 1] == 128;
-    const bool qn = p.kv_dt != dt_f16, mk = p.mask != nullptr;
+    const bool qn = p.kv_dt != desc->q.dt, mk = p.mask != nullptr;
+    const bool bf = p.bf != 0; // never together with qn
     if (p.Qn <= 16) {
         const sdpa_split_t sp
                 = decode_split((int64_t)p.B0 * p.B1, p.S, p.Qn, p.causal != 0);
@@ -1030,15 +1059,20 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
             hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
                     (hipStream_t)hip_stream, p);
         };
-        switch ((d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
-            case 0: god(sdpa_decode_kernel<2, false, false>); break;
-            case 1: god(sdpa_decode_kernel<2, false, true>); break;
-            case 2: god(sdpa_decode_kernel<2, true, false>); break;
-            case 3: god(sdpa_decode_kernel<2, true, true>); break;
-            case 4: god(sdpa_decode_kernel<4, false, false>); break;
-            case 5: god(sdpa_decode_kernel<4, false, true>); break;
-            case 6: god(sdpa_decode_kernel<4, true, false>); break;
-            default: god(sdpa_decode_kernel<4, true, true>); break;
+        switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
+            case 0: god(sdpa_decode_kernel<2, false, false, false>); break;
+            case 1: god(sdpa_decode_kernel<2, false, true, false>); break;
+            case 2: god(sdpa_decode_kernel<2, true, false, false>); break;
+            case 3: god(sdpa_decode_kernel<2, true, true, false>); break;
+            case 4: god(sdpa_decode_kernel<4, false, false, false>); break;
+            case 5: god(sdpa_decode_kernel<4, false, true, false>); break;
+            case 6: god(sdpa_decode_kernel<4, true, false, false>); break;
+            case 7: god(sdpa_decode_kernel<4, true, true, false>); break;
+            case 8: god(sdpa_decode_kernel<2, false, false, true>); break;
+            case 9: god(sdpa_decode_kernel<2, false, true, true>); break;
+            case 12: god(sdpa_decode_kernel<4, false, false, true>); break;
+            case 13: god(sdpa_decode_kernel<4, false, true, true>); break;
+            default: return QMM_UNIMPLEMENTED;
         }
         if (p.nsplit > 1)
             hipLaunchKernelGGL(sdpa_combine_kernel,
@@ -1066,15 +1100,20 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);
     };
-    switch ((d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
-        case 0: go(sdpa_f16_kernel<2, false, false>); break;
-        case 1: go(sdpa_f16_kernel<2, false, true>); break;
-        case 2: go(sdpa_f16_kernel<2, true, false>); break;
-        case 3: go(sdpa_f16_kernel<2, true, true>); break;
-        case 4: go(sdpa_f16_kernel<4, false, false>); break;
-        case 5: go(sdpa_f16_kernel<4, false, true>); break;
-        case 6: go(sdpa_f16_kernel<4, true, false>); break;
-        default: go(sdpa_f16_kernel<4, true, true>); break;
+    switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
+        case 0: go(sdpa_f16_kernel<2, false, false, false>); break;
+        case 1: go(sdpa_f16_kernel<2, false, true, false>); break;
+        case 2: go(sdpa_f16_kernel<2, true, false, false>); break;
+        case 3: go(sdpa_f16_kernel<2, true, true, false>); break;
+        case 4: go(sdpa_f16_kernel<4, false, false, false>); break;
+        case 5: go(sdpa_f16_kernel<4, false, true, false>); break;
+        case 6: go(sdpa_f16_kernel<4, true, false, false>); break;
+        case 7: go(sdpa_f16_kernel<4, true, true, false>); break;
+        case 8: go(sdpa_f16_kernel<2, false, false, true>); break;
+        case 9: go(sdpa_f16_kernel<2, false, true, true>); break;
+        case 12: go(sdpa_f16_kernel<4, false, false, true>); break;
+        case 13: go(sdpa_f16_kernel<4, false, true, true>); break;
+        default: return QMM_UNIMPLEMENTED;
     }
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }

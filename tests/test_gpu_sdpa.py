@@ -1,8 +1,8 @@
-"""The fused attention kernel (hip:gfx950:sdpa_f16) behind the reference's internal sdpa entry point, against
+"""The fused attention kernel (hip:gfx950:sdpa_f16 / sdpa_bf16) behind the reference's internal sdpa entry point, against
 float64 attention on the operands the kernel sees (for a quantized cache: the f16 values the chain's dequantizing
 reorder produces, taken from the oracle), with the comparison rule of the reference's own SDPA test
-(tests/gtests/internals/test_sdpa.cpp:1043-1106: abs 0.001466 up to |gold| = 1, relative above; at most 0.06 % of the
-elements outside), and against the primitive chain of that test run on the device."""
+(tests/gtests/internals/test_sdpa.cpp:1043-1106: abs 0.001466 (f16; 0.0079 for bf16) up to |gold| = 1, relative
+above; at most 0.06 % of the elements outside), and against the primitive chain of that test run on the device."""
 import sys
 
 import numpy as np
@@ -28,12 +28,12 @@ def ctx():
     return eng, dnnl.stream(eng)
 
 
-def f16(x):
-    return O.from_f32(dt.f16, np.ascontiguousarray(x, np.float32)).reshape(np.shape(x))
+def f16(x, code=dt.f16):
+    return O.from_f32(code, np.ascontiguousarray(x, np.float32)).reshape(np.shape(x))
 
 
-def f16_to_f64(raw):
-    return O.to_f32(dt.f16, np.ascontiguousarray(raw)).reshape(raw.shape).astype(np.float64)
+def f16_to_f64(raw, code=dt.f16):
+    return O.to_f32(code, np.ascontiguousarray(raw)).reshape(raw.shape).astype(np.float64)
 
 
 def reference_rule(test, gold, thr=0.001466):
@@ -60,27 +60,28 @@ def attention64(q, kt, v, scale, mask, causal, kv_rep):
 
 
 def run_sdpa(ctx, q, k_store, v, *, scale=None, invert=False, mask=None, mask_dt=dt.f32, causal=False, kv_heads=0,
-             kv_dt=dt.f16, k_q=None, v_q=None):
-    """q [.., Q, D] f16 raw; k_store [.., S, D] (the cache as stored: keys major), passed as its transposed view;
+             kv_dt=None, k_q=None, v_q=None, qdt=dt.f16):
+    """q [.., Q, D] raw 16-bit values of type qdt; k_store [.., S, D] (the cache as stored: keys major), passed as its transposed view;
     v [.., S, D]. k_q / v_q: (mask, groups, scale_dt, scales, zp_dt, zps) for a quantized cache."""
     eng, strm = ctx
     nd = q.ndim
     letters = "abcd"[:nd]
-    q_md = memory.desc(list(q.shape), dt.f16, T(letters))
+    kv_dt = qdt if kv_dt is None else kv_dt
+    q_md = memory.desc(list(q.shape), qdt, T(letters))
     kdims = list(k_store.shape[:-2]) + [k_store.shape[-1], k_store.shape[-2]]
     kt_md = memory.desc(kdims, kv_dt, T(letters[:-2] + letters[-1] + letters[-2]))  # D contiguous: the transposed view
     v_md = memory.desc(list(v.shape), kv_dt, T(letters))
-    o_md = memory.desc(list(q.shape), dt.f16, T(letters))
+    o_md = memory.desc(list(q.shape), qdt, T(letters))
     args = {dnnl.DNNL_ARG_QUERIES: memory(q_md, eng).write(q), dnnl.DNNL_ARG_KEYS: memory(kt_md, eng).write(k_store),
             dnnl.DNNL_ARG_VALUES: memory(v_md, eng).write(v)}
     m_md = None
     if mask is not None:
         m_md = memory.desc(list(mask.shape), mask_dt, T(letters))
-        args[dnnl.DNNL_ARG_ATTN_MASK] = memory(m_md, eng).write(mask if mask_dt == dt.f32 else f16(mask))
+        args[dnnl.DNNL_ARG_ATTN_MASK] = memory(m_md, eng).write(mask if mask_dt == dt.f32 else f16(mask, mask_dt))
     scale_dt = dt.undef
     if scale is not None:
-        scale_dt = dt.f16
-        args[dnnl.DNNL_ARG_SCALE] = memory(memory.desc([1], dt.f16, T("a")), eng).write(f16(np.array([scale])))
+        scale_dt = qdt
+        args[dnnl.DNNL_ARG_SCALE] = memory(memory.desc([1], qdt, T("a")), eng).write(f16(np.array([scale]), qdt))
     attrs = []
     for which, qq in ((dnnl.DNNL_ARG_KEYS, k_q), (dnnl.DNNL_ARG_VALUES, v_q)):
         a = None
@@ -95,7 +96,7 @@ def run_sdpa(ctx, q, k_store, v, *, scale=None, invert=False, mask=None, mask_dt
         attrs.append(a)
     pd = dnnl.sdpa.primitive_desc(eng, q_md, kt_md, v_md, m_md, scale_dt, o_md, invert, kv_heads, causal,
                                   None, attrs[0], attrs[1])
-    assert pd.impl_info_str() == "hip:gfx950:sdpa_f16"
+    assert pd.impl_info_str() == ("hip:gfx950:sdpa_bf16" if qdt == dt.bf16 else "hip:gfx950:sdpa_f16")
     out = memory(o_md, eng)
     args[dnnl.DNNL_ARG_DST] = out
     dnnl.sdpa(pd).execute(strm, args)
@@ -115,15 +116,16 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("qdt", [dt.f16, dt.bf16], ids=["f16", "bf16"])
 @pytest.mark.parametrize("case", CASES, ids=str)
-def test_f16_attention(ctx, case):
+def test_f16_attention(ctx, case, qdt):
     bdims, kvh, Qn, S, D, mkind, smode = case
-    say("sdpa f16 %r" % (case,))
+    say("sdpa %s %r" % (qdt, case))
     r = np.random.default_rng(Qn + S + D)
     kb = tuple(bdims[:-1]) + ((kvh,) if kvh else tuple(bdims[-1:])) if bdims else ()
-    q = f16(r.standard_normal(bdims + (Qn, D)))
-    k = f16(r.standard_normal(kb + (S, D)))
-    v = f16(r.standard_normal(kb + (S, D)))
+    q = f16(r.standard_normal(bdims + (Qn, D)), qdt)
+    k = f16(r.standard_normal(kb + (S, D)), qdt)
+    v = f16(r.standard_normal(kb + (S, D)), qdt)
     scale = None if smode == "none" else (1.0 / np.sqrt(D) if smode == "mul" else np.sqrt(D))
     mask = None
     nb = len(bdims)
@@ -134,14 +136,14 @@ def test_f16_attention(ctx, case):
     elif mkind == "1d":
         mask = (r.standard_normal((1,) * nb + (1, S)) * 2).astype(np.float32)
     got = run_sdpa(ctx, q, k, v, scale=scale, invert=(smode == "div"), mask=mask,
-                   mask_dt=dt.f16 if mkind == "1d" else dt.f32, causal=(mkind == "causal"), kv_heads=kvh)
-    s_eff = 1.0 if scale is None else float(f16_to_f64(f16(np.array([scale])))[0])
+                   mask_dt=qdt if mkind == "1d" else dt.f32, causal=(mkind == "causal"), kv_heads=kvh, qdt=qdt)
+    s_eff = 1.0 if scale is None else float(f16_to_f64(f16(np.array([scale]), qdt), qdt)[0])
     if smode == "div":
         s_eff = 1.0 / s_eff
-    m_eff = None if mask is None else (mask.astype(np.float64) if mkind != "1d" else f16_to_f64(f16(mask)))
-    gold = attention64(f16_to_f64(q), np.swapaxes(f16_to_f64(k), -1, -2), f16_to_f64(v), s_eff, m_eff,
+    m_eff = None if mask is None else (mask.astype(np.float64) if mkind != "1d" else f16_to_f64(f16(mask, qdt), qdt))
+    gold = attention64(f16_to_f64(q, qdt), np.swapaxes(f16_to_f64(k, qdt), -1, -2), f16_to_f64(v, qdt), s_eff, m_eff,
                        mkind == "causal", (bdims[-1] // kvh) if kvh else 1)
-    bad, total, worst = reference_rule(f16_to_f64(got), gold)
+    bad, total, worst = reference_rule(f16_to_f64(got, qdt), gold, 0.001466 if qdt == dt.f16 else 0.0079)
     print("[sdpa] %d of %d outside the reference test's threshold, max diff %.2e" % (bad, total, worst))
     assert bad <= total * 0.0006
 
@@ -181,6 +183,7 @@ def test_quantized_cache(ctx, kv_dt, with_zp, Qn):
 @pytest.mark.parametrize("Qn,S,D,heads,kvh,mkind,quant", [
     (1, 4096, 128, 8, 0, "none", False), (1, 2049, 128, 32, 8, "none", True), (5, 1500, 64, 4, 0, "2d", False),
     (16, 3000, 128, 6, 2, "causal", False), (2, 640, 64, 40, 0, "1d", True), (1, 96, 128, 2, 0, "none", False),
+    (1, 5000, 128, 8, 2, "none", "bf16"), (7, 1111, 64, 3, 0, "2d", "bf16"),
 ], ids=str)
 def test_few_queries_split_over_the_keys(ctx, Qn, S, D, heads, kvh, mkind, quant):
     """At most 16 queries per head (the decode step): the keys are cut into ranges, one workgroup each, the ranges'
@@ -188,7 +191,9 @@ def test_few_queries_split_over_the_keys(ctx, Qn, S, D, heads, kvh, mkind, quant
     say("sdpa decode Qn=%d S=%d D=%d heads=%d kv=%d mask=%s quant=%s" % (Qn, S, D, heads, kvh, mkind, quant))
     r = np.random.default_rng(Qn * 7 + S)
     kh = kvh or heads
-    q = f16(r.standard_normal((1, heads, Qn, D)))
+    qdt = dt.bf16 if quant == "bf16" else dt.f16
+    quant = quant is True
+    q = f16(r.standard_normal((1, heads, Qn, D)), qdt)
     scale = 1.0 / np.sqrt(D)
     mask = None
     if mkind == "2d":
@@ -209,13 +214,13 @@ def test_few_queries_split_over_the_keys(ctx, Qn, S, D, heads, kvh, mkind, quant
                       src_scale=O.Quant(0b1110, dt.f16, sc, (1, D)), src_zp=O.Quant(0b1110, dt.s8, zp, (1, D)))
         k64, v64 = f16_to_f64(kd), f16_to_f64(vd)
     else:
-        k, v = f16(r.standard_normal((1, kh, S, D))), f16(r.standard_normal((1, kh, S, D)))
-        got = run_sdpa(ctx, q, k, v, scale=scale, mask=mask, causal=(mkind == "causal"), kv_heads=kvh)
-        k64, v64 = f16_to_f64(k), f16_to_f64(v)
-    s_eff = float(f16_to_f64(f16(np.array([scale])))[0])
-    gold = attention64(f16_to_f64(q), np.swapaxes(k64, -1, -2), v64, s_eff,
+        k, v = f16(r.standard_normal((1, kh, S, D)), qdt), f16(r.standard_normal((1, kh, S, D)), qdt)
+        got = run_sdpa(ctx, q, k, v, scale=scale, mask=mask, causal=(mkind == "causal"), kv_heads=kvh, qdt=qdt)
+        k64, v64 = f16_to_f64(k, qdt), f16_to_f64(v, qdt)
+    s_eff = float(f16_to_f64(f16(np.array([scale]), qdt), qdt)[0])
+    gold = attention64(f16_to_f64(q, qdt), np.swapaxes(k64, -1, -2), v64, s_eff,
                        None if mask is None else mask.astype(np.float64), mkind == "causal", heads // kh)
-    bad, total, worst = reference_rule(f16_to_f64(got), gold)
+    bad, total, worst = reference_rule(f16_to_f64(got, qdt), gold, 0.001466 if qdt == dt.f16 else 0.0079)
     print("[sdpa decode] %d of %d outside the threshold, max diff %.2e" % (bad, total, worst))
     assert bad <= total * 0.0006
 
@@ -299,7 +304,9 @@ def test_what_the_kernel_does_not_take_is_unimplemented(ctx):
     make()
     for bad in (dict(q=md([1, 2, 16, 96]), k=md([1, 2, 96, 32], t="abdc"), v=md([1, 2, 32, 96]), o=md([1, 2, 16, 96])),  # head size
                 dict(k=md([1, 2, 64, 32])),                                    # keys contiguous instead of head size
-                dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16))):  # bf16
+                dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16)),  # bf16 queries on f16 keys
+                dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16),  # bf16 on an 8-bit cache
+                     k=md([1, 2, 64, 32], dt.s8, t="abdc"), v=md([1, 2, 32, 64], dt.s8))):
         with pytest.raises(dnnl.error) as e:
             make(**bad)
         assert e.value.status == dnnl.status.unimplemented
