@@ -1196,6 +1196,11 @@ static bool reorder_rows_plan(const qmm_reorder_desc_t *d,
     const int64_t sp = nd >= 2 ? d->src.strides[nd - 2] : C;
     const int64_t dp = nd >= 2 ? d->dst.strides[nd - 2] : C;
     if (sp < C || dp < C) return false;
+    // 32-bit index arithmetic, and a grid of at most 2^31 workgroups of 128
+    // or more 8-column chunks
+    if (rows >= (int64_t(1) << 31) || C >= (int64_t(1) << 31)
+            || rows * C >= (int64_t(1) << 40))
+        return false;
     for (int i = nd - 3; i >= 0; i--) {
         if (d->src.strides[i] != d->src.strides[i + 1] * d->src.dims[i + 1]
                 || d->dst.strides[i]

@@ -247,9 +247,10 @@ struct quant_rows_params_t {
     int64_t rows, cols; // cols % 8 == 0
     int64_t src_pitch, dst_pitch; // elements
     int32_t src_dt, dst_dt;
-    int32_t rows_per_thread, pad_; // set by the launcher
+    int32_t rows_per_thread, tpr_log2; // set by the launcher
     quant_rows_q_t src_scale, dst_scale, src_zp;
     const int32_t *dst_zp; // single value or nullptr
+    int32_t col_groups, pad_; // set by the launcher
 };
 
 enum impl_id_t : int {

@@ -16,8 +16,13 @@ namespace qmm {
 
 // scales / zero points as a function of (row, col): element
 // (row / gr) * sr + (col / gc) * sc of the buffer
+// (rows and columns are below 2^31, host-checked: 32-bit divisions, and none
+// where the group is 1 or the stride 0)
 QMM_D int64_t qr_off(const quant_rows_q_t &q, int64_t row, int64_t col) {
-    return (row / q.gr) * q.sr + (col / q.gc) * q.sc;
+    const uint32_t r = (uint32_t)row, c = (uint32_t)col;
+    const uint32_t rg = q.gr == 1 || q.sr == 0 ? r : r / (uint32_t)q.gr;
+    const uint32_t cg = q.gc == 1 || q.sc == 0 ? c : c / (uint32_t)q.gc;
+    return (int64_t)rg * q.sr + (int64_t)cg * q.sc;
 }
 
 // Rows per thread: 8 where an operand depends on the column only (it is
@@ -55,10 +60,19 @@ QMM_D void qr_fetch_scale(const quant_rows_q_t &q, int64_t row, int64_t col,
 template <int RPT>
 __global__ void __launch_bounds__(256)
 quantize_rows_kernel(const quant_rows_params_t p) {
-    const int64_t c8 = p.cols / 8;
+    // A workgroup covers 256 >> tpr_log2 row blocks (of RPT rows) with
+    // 1 << tpr_log2 threads each, for one group of 1 << tpr_log2 chunks of 8
+    // columns; neighbouring workgroups are neighbours along a row. One 32-bit
+    // division per workgroup in the index arithmetic.
+    const uint32_t c8 = (uint32_t)(p.cols / 8);
     constexpr int rpt = RPT;
-    const int64_t row_blocks = (p.rows + rpt - 1) / rpt;
-    const int64_t total = row_blocks * c8;
+    const uint32_t tpr = 1u << p.tpr_log2;
+    const uint32_t rw = blockIdx.x / (uint32_t)p.col_groups;
+    const uint32_t cg = blockIdx.x - rw * (uint32_t)p.col_groups;
+    const int64_t row0 = ((int64_t)rw * (256u >> p.tpr_log2)
+                                 + (threadIdx.x >> p.tpr_log2))
+            * rpt;
+    if (row0 >= p.rows) return;
     const bool f32_in = p.src_dt == dt_f32;
     // a buffer that does not change within 8 columns is read once per row
     const bool ss_one = !p.src_scale.ptr || p.src_scale.sc == 0
@@ -72,9 +86,9 @@ quantize_rows_kernel(const quant_rows_params_t p) {
     const bool ds_col = p.dst_scale.ptr && p.dst_scale.sr == 0;
     const bool sz_col = p.src_zp.ptr && p.src_zp.sr == 0;
     const float dst_zp = p.dst_zp ? (float)p.dst_zp[0] : 0.f;
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
-            t += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t row0 = (t / c8) * rpt, col = (t % c8) * 8;
+    const uint32_t cb = cg * tpr + (threadIdx.x & (tpr - 1));
+    if (cb < c8) {
+        const int64_t col = (int64_t)cb * 8;
         float ss[8], ds[8], szf[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -86,7 +100,8 @@ quantize_rows_kernel(const quant_rows_params_t p) {
         if (ds_col) qr_fetch_scale(p.dst_scale, 0, col, ds_one, true, ds);
         if (sz_col) qr_fetch_scale(p.src_zp, 0, col, sz_one, false, szf);
         const int nrows = (int)min((int64_t)rpt, p.rows - row0);
-#pragma unroll(RPT > 1 ? 2 : 1)
+        constexpr int UN = RPT > 1 ? 2 : 1;
+#pragma unroll UN
         for (int rr = 0; rr < nrows; rr++) {
             const int64_t row = row0 + rr;
             float in[8];
@@ -178,23 +193,239 @@ quantize_rows_kernel(const quant_rows_params_t p) {
     }
 }
 
+// The quantizer that runs every step (a linear layer's activations): f32 /
+// bf16 / f16 rows -> s8 / u8 with nothing but one f32 dst scale for the tensor
+// or per row, and a dst zero point. The arithmetic of the kernel above with
+// its defaults taken out (1 * x and x - 0 are x): d = in * (1 / scale) + zp,
+// each step rounded. A thread converts Q8_CHUNKS chunks of 8 columns,
+// 1 << tpr_log2 chunks apart, all requested before the first is used; a
+// workgroup covers 256 >> tpr_log2 rows of one group of Q8_CHUNKS << tpr_log2
+// chunks.
+constexpr int Q8_CHUNKS = 4;
+template <int SRC, bool PER_ROW> // SRC: 0 f32, 1 bf16, 2 f16
+__global__ void __launch_bounds__(256)
+quantize8_kernel(const quant_rows_params_t p) {
+    const uint32_t c8 = (uint32_t)(p.cols / 8);
+    const uint32_t tpr = 1u << p.tpr_log2;
+    const uint32_t rw = blockIdx.x / (uint32_t)p.col_groups;
+    const uint32_t cg = blockIdx.x - rw * (uint32_t)p.col_groups;
+    const int64_t row = (int64_t)rw * (256u >> p.tpr_log2)
+            + (threadIdx.x >> p.tpr_log2);
+    if (row >= p.rows) return;
+    constexpr int U = Q8_CHUNKS;
+    const uint32_t cb0 = cg * U * tpr + (threadIdx.x & (tpr - 1));
+    if (cb0 >= c8) return;
+    uint32_t cb[U]; // chunks past the row's end read the first again
+#pragma unroll
+    for (int u = 0; u < U; u++) cb[u] = cb0 + u * tpr < c8 ? cb0 + u * tpr : cb0;
+    uint4 raw[U][2];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if constexpr (SRC == 0) {
+            const uint4 *s = (const uint4 *)((const float *)p.src
+                    + row * p.src_pitch + (int64_t)cb[u] * 8);
+            raw[u][0] = s[0];
+            raw[u][1] = s[1];
+        } else {
+            raw[u][0] = *(const uint4 *)((const uint16_t *)p.src
+                    + row * p.src_pitch + (int64_t)cb[u] * 8);
+        }
+    }
+    float inv = 1.f;
+    if (p.dst_scale.ptr)
+        inv = 1.f / ((const float *)p.dst_scale.ptr)[PER_ROW ? row : 0];
+    const float dst_zp = p.dst_zp ? (float)p.dst_zp[0] : 0.f;
+    const bool sgn = p.dst_dt == dt_s8;
+    const float lo = sgn ? -128.f : 0.f, hi = sgn ? 127.f : 255.f;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (u > 0 && cb0 + u * tpr >= c8) break;
+        float in[8];
+        if constexpr (SRC == 0) {
+            const uint32_t w[8] = {raw[u][0].x, raw[u][0].y, raw[u][0].z,
+                    raw[u][0].w, raw[u][1].x, raw[u][1].y, raw[u][1].z,
+                    raw[u][1].w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) in[i] = u2f(w[i]);
+        } else {
+            const uint32_t w[4]
+                    = {raw[u][0].x, raw[u][0].y, raw[u][0].z, raw[u][0].w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if constexpr (SRC == 2)
+                    in[i] = (float)__builtin_bit_cast(_Float16,
+                            (uint16_t)(w[i / 2] >> (16 * (i % 2))));
+                else
+                    in[i] = u2f(i % 2 ? (w[i / 2] & 0xFFFF0000u)
+                                      : (w[i / 2] << 16));
+            }
+        }
+        uint32_t o[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            o[i / 4] |= (uint32_t)(round_sat(in[i] * inv + dst_zp, lo, hi) & 0xff)
+                    << (8 * (i % 4));
+        *(uint2 *)((uint8_t *)p.dst + row * p.dst_pitch + (int64_t)cb[u] * 8)
+                = make_uint2(o[0], o[1]);
+    }
+}
+
+// The same with one f32 dst scale per column (a layer's weights): a thread
+// owns one chunk of 8 columns, inverts its 8 scales once and converts 8 rows,
+// all of them requested before the first is used.
+template <int SRC>
+__global__ void __launch_bounds__(256)
+quantize8_cols_kernel(const quant_rows_params_t p) {
+    constexpr int R = QR_ROWS, V = SRC == 0 ? 2 : 1;
+    const uint32_t c8 = (uint32_t)(p.cols / 8);
+    const uint32_t tpr = 1u << p.tpr_log2;
+    const uint32_t rw = blockIdx.x / (uint32_t)p.col_groups;
+    const uint32_t cg = blockIdx.x - rw * (uint32_t)p.col_groups;
+    const int64_t row0 = ((int64_t)rw * (256u >> p.tpr_log2)
+                                 + (threadIdx.x >> p.tpr_log2))
+            * R;
+    const uint32_t cb = cg * tpr + (threadIdx.x & (tpr - 1));
+    if (row0 >= p.rows || cb >= c8) return;
+    const int64_t col = (int64_t)cb * 8;
+    uint4 raw[R][V];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        // rows past the end read the last row again and are not stored
+        const int64_t row = min(row0 + r, p.rows - 1);
+        const uint4 *s = (const uint4 *)((const char *)p.src
+                + (row * p.src_pitch + col) * (SRC == 0 ? 4 : 2));
+#pragma unroll
+        for (int v = 0; v < V; v++) raw[r][v] = s[v];
+    }
+    const float4 *sp = (const float4 *)((const float *)p.dst_scale.ptr + col);
+    const float4 sa = sp[0], sb = sp[1];
+    const float inv[8] = {1.f / sa.x, 1.f / sa.y, 1.f / sa.z, 1.f / sa.w,
+            1.f / sb.x, 1.f / sb.y, 1.f / sb.z, 1.f / sb.w};
+    const float dst_zp = p.dst_zp ? (float)p.dst_zp[0] : 0.f;
+    const bool sgn = p.dst_dt == dt_s8;
+    const float lo = sgn ? -128.f : 0.f, hi = sgn ? 127.f : 255.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (row0 + r >= p.rows) break;
+        float in[8];
+        if constexpr (SRC == 0) {
+            const uint32_t w[8] = {raw[r][0].x, raw[r][0].y, raw[r][0].z,
+                    raw[r][0].w, raw[r][V - 1].x, raw[r][V - 1].y,
+                    raw[r][V - 1].z, raw[r][V - 1].w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) in[i] = u2f(w[i]);
+        } else {
+            const uint32_t w[4]
+                    = {raw[r][0].x, raw[r][0].y, raw[r][0].z, raw[r][0].w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                if constexpr (SRC == 2)
+                    in[i] = (float)__builtin_bit_cast(_Float16,
+                            (uint16_t)(w[i / 2] >> (16 * (i % 2))));
+                else
+                    in[i] = u2f(i % 2 ? (w[i / 2] & 0xFFFF0000u)
+                                      : (w[i / 2] << 16));
+            }
+        }
+        uint32_t o[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            o[i / 4] |= (uint32_t)(round_sat(in[i] * inv[i] + dst_zp, lo, hi)
+                                & 0xff)
+                    << (8 * (i % 4));
+        *(uint2 *)((uint8_t *)p.dst + (row0 + r) * p.dst_pitch + col)
+                = make_uint2(o[0], o[1]);
+    }
+}
+
+// whether the 8-bit kernels cover the plan; how the dst scale runs (0: one
+// or none, 1: per row, 2: per column)
+static bool quantize8_takes(const quant_rows_params_t &p, int &mode) {
+    if (p.dst_dt != dt_s8 && p.dst_dt != dt_u8) return false;
+    if (p.src_scale.ptr || p.src_zp.ptr) return false;
+    mode = 0;
+    const quant_rows_q_t &q = p.dst_scale;
+    if (!q.ptr) return true;
+    if (q.dt != dt_f32) return false;
+    if (q.sr == 0 && q.sc == 0) return true;
+    if (q.sc == 0 && q.sr == 1 && q.gr == 1) mode = 1;
+    if (q.sr == 0 && q.sc == 1 && q.gc == 1) mode = 2;
+    return mode != 0;
+}
+
 void launch_quantize_rows(const quant_rows_params_t &p0, hipStream_t stream) {
     quant_rows_params_t p = p0;
+    int mode = 0;
+    if (quantize8_takes(p, mode)) {
+        const int64_t c8 = p.cols / 8, c16 = (c8 + Q8_CHUNKS - 1) / Q8_CHUNKS;
+        if (p.rows <= 0 || c8 <= 0) return;
+        if (mode == 2) {
+            p.tpr_log2 = 0;
+            while (p.tpr_log2 < 8 && (int64_t(1) << p.tpr_log2) < c8)
+                p.tpr_log2++;
+            const int64_t tpr = int64_t(1) << p.tpr_log2;
+            const int64_t rows_wg = (256 >> p.tpr_log2) * QR_ROWS;
+            p.col_groups = (int32_t)((c8 + tpr - 1) / tpr);
+            const dim3 grid((unsigned)(((p.rows + rows_wg - 1) / rows_wg)
+                    * p.col_groups));
+            auto go = [&](auto kern) {
+                hipLaunchKernelGGL(kern, grid, dim3(256), 0, stream, p);
+            };
+            if (p.src_dt == dt_f32)
+                go(quantize8_cols_kernel<0>);
+            else if (p.src_dt == dt_bf16)
+                go(quantize8_cols_kernel<1>);
+            else
+                go(quantize8_cols_kernel<2>);
+            return;
+        }
+        const bool per_row = mode == 1;
+        p.tpr_log2 = 0;
+        while (p.tpr_log2 < 8 && (int64_t(1) << p.tpr_log2) < c16)
+            p.tpr_log2++;
+        const int64_t per_wg = 256 >> p.tpr_log2, span = int64_t(Q8_CHUNKS) << p.tpr_log2;
+        p.col_groups = (int32_t)((c8 + span - 1) / span);
+        // below 2^31: the plan bounds rows * cols
+        const dim3 grid((unsigned)(((p.rows + per_wg - 1) / per_wg) * p.col_groups));
+        auto go = [&](auto kern) {
+            hipLaunchKernelGGL(kern, grid, dim3(256), 0, stream, p);
+        };
+        switch ((p.src_dt == dt_f32 ? 0 : p.src_dt == dt_bf16 ? 2 : 4)
+                | (per_row ? 1 : 0)) {
+            case 0: go(quantize8_kernel<0, false>); break;
+            case 1: go(quantize8_kernel<0, true>); break;
+            case 2: go(quantize8_kernel<1, false>); break;
+            case 3: go(quantize8_kernel<1, true>); break;
+            case 4: go(quantize8_kernel<2, false>); break;
+            default: go(quantize8_kernel<2, true>); break;
+        }
+        return;
+    }
     const bool col_only = (p.src_scale.ptr && p.src_scale.sr == 0
                                   && p.src_scale.sc != 0)
             || (p.dst_scale.ptr && p.dst_scale.sr == 0 && p.dst_scale.sc != 0);
     p.rows_per_thread = col_only ? QR_ROWS : 1;
-    const int64_t total = ((p.rows + p.rows_per_thread - 1) / p.rows_per_thread)
-            * (p.cols / 8);
-    if (total <= 0) return;
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 262144) blocks = 262144;
+    const int64_t row_blocks
+            = (p.rows + p.rows_per_thread - 1) / p.rows_per_thread;
+    const int64_t c8 = p.cols / 8;
+    if (row_blocks <= 0 || c8 <= 0) return;
+    // threads per row block: the power of two at or above the chunks of a row,
+    // 256 at most
+    p.tpr_log2 = 0;
+    while (p.tpr_log2 < 8 && (int64_t(1) << p.tpr_log2) < c8)
+        p.tpr_log2++;
+    const int64_t per_wg = 256 >> p.tpr_log2;
+    const int64_t tpr = int64_t(1) << p.tpr_log2;
+    p.col_groups = (int32_t)((c8 + tpr - 1) / tpr);
+    // below 2^31: the plan bounds rows * cols
+    const dim3 grid(
+            (unsigned)(((row_blocks + per_wg - 1) / per_wg) * p.col_groups));
     if (col_only)
-        hipLaunchKernelGGL(quantize_rows_kernel<QR_ROWS>, dim3((unsigned)blocks),
-                dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(quantize_rows_kernel<QR_ROWS>, grid, dim3(256), 0,
+                stream, p);
     else
-        hipLaunchKernelGGL(quantize_rows_kernel<1>, dim3((unsigned)blocks),
-                dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(
+                quantize_rows_kernel<1>, grid, dim3(256), 0, stream, p);
 }
 
 } // namespace qmm

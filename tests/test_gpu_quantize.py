@@ -89,6 +89,35 @@ def test_activations_bf16_to_s8_per_row_and_to_u8_with_zero_point(ctx):
     run_case(eng, strm, dt.f16, dt.u8, (M, 64), 5, dst_scale=(0, dt.f32, None, [0.04]), dst_zp=128)
 
 
+@pytest.mark.parametrize("src_dt", [dt.f32, dt.bf16, dt.f16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("dims,scale,zp,dst_dt", [
+    ((1, 8), "row", None, dt.s8), ((5, 24), "one", 3, dt.u8), ((300, 40), "row", None, dt.u8),
+    ((37, 4104), "row", -7, dt.s8), ((129, 4096), "none", None, dt.s8), ((2, 9, 520), "one", None, dt.s8),
+    ((1000, 16), "row", 100, dt.u8), ((3, 12296), "row", None, dt.s8),
+    ((97, 200), "col", None, dt.s8), ((13, 4104), "col", -3, dt.s8), ((3, 21, 64), "col", 9, dt.u8),
+    ((2050, 8), "col", None, dt.u8),
+], ids=str)
+def test_activation_quantizer_shapes(ctx, src_dt, dims, scale, zp, dst_dt):
+    """The specialised 8-bit kernels (one dst scale for the tensor, per row or per column, dst zero point): rows and
+    columns that do not fill their workgroups, a thread's second chunk past the row's end, row blocks past the last
+    row, values that saturate, a NaN."""
+    eng, strm = ctx
+    say("activation quantizer %s -> %s %s scale=%s zp=%s" % (src_dt, dst_dt, dims, scale, zp))
+    r = np.random.default_rng(sum(dims) + src_dt)
+    x = (r.standard_normal(dims) * 40).astype(np.float32)
+    x.reshape(-1)[::97] *= 50  # saturating values
+    x.reshape(-1)[5 % x.size] = np.nan
+    rows = int(np.prod(dims[:-1]))
+    ds = None
+    if scale == "row" and len(dims) == 2:
+        ds = (1, dt.f32, None, r.uniform(0.2, 0.9, rows))
+    elif scale == "col":
+        ds = (1 << (len(dims) - 1), dt.f32, None, r.uniform(0.2, 0.9, dims[-1]))
+    elif scale != "none":
+        ds = (0, dt.f32, None, [0.37])
+    run_case(eng, strm, src_dt, dst_dt, dims, 0, dst_scale=ds, dst_zp=zp, src_values=x)
+
+
 def test_grouped_source_scales(ctx):
     """Groups are a source-side attribute in the reference (src/common/reorder.cpp:121-143)."""
     eng, strm = ctx
