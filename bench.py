@@ -233,7 +233,7 @@ def C_stream(strm):
     return p.value
 
 
-def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, K=4096, N=4096, rows=(1, 16)):
+def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, K=4096, N=4096, rows=(1, 4, 8, 16)):
     """Config 3: bf16 x u4 GEMV, G=128 f16 scales + u4 zero points. The 8.7 MB
     of one weights set would sit in the last-level cache, so `sets` distinct
     copies are cycled; the launches are replayed from a HIP graph so that the

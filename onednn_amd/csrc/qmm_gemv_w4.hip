@@ -62,20 +62,23 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
 
 // Cross-wave reduction of the partial sums and the epilogue, shared by the two
 // kernels: every wave leaves its 4 values per lane in LDS, wave 0 adds them in
-// wave order and stores. ONE_ROW: only row 0 (register 0 of lanes 0..15) is
-// live. `plain` (wave-uniform): nothing follows the accumulation (no scales,
+// wave order and stores. Register j of lane l is row 4 * (l / 16) + j of the
+// MFMA result. ROWS = 16: every row is an activation row; ROWS = 8: the even
+// rows (registers 0 and 2) are activation rows 0..7; ROWS = 4 and 1: rows 0,
+// 4, 8, 12 (register 0) are activation rows 0..3. `plain` (wave-uniform): nothing follows the accumulation (no scales,
 // bias, post-ops, dst scale or zero point) and dst is dense along n, so the
 // value is converted and stored without the post-op interpreter; `dst` and
 // `dst_sm` are then the dst pointer and row pitch, read by the caller long
 // before (the parameter block is cold, its first touch costs a trip to memory).
-template <bool ONE_ROW>
+template <int ROWS>
 QMM_D void gemv_reduce_store(const gemv_params_t &p, float *red, const v4f &out,
         int wave, int lane, int m_base, int rows, int n, bool plain = false,
         void *dst = nullptr, int64_t dst_sm = 0, int dst_dt = 0) {
-    constexpr int NJ = ONE_ROW ? 1 : 4;
+    constexpr int SPL = ROWS == 16 ? 1 : ROWS == 8 ? 2 : 4; // MFMA rows per activation row
+    constexpr int NJ = 4 / SPL;
 #pragma unroll
     for (int j = 0; j < NJ; j++)
-        red[(wave * 64 + lane) * NJ + j] = out[j];
+        red[(wave * 64 + lane) * NJ + j] = out[j * SPL];
     __syncthreads();
     if (wave == 0) {
         const int c = lane >> 4;
@@ -86,8 +89,9 @@ QMM_D void gemv_reduce_store(const gemv_params_t &p, float *red, const v4f &out,
             for (int w = 0; w < GEMV_WAVES; w++)
                 v += red[(w * 64 + lane) * NJ + j];
             // MFMA output: register j of lane l is row 4*(l/16)+j, column l%16
-            const int m = m_base + 4 * c + j;
-            if (m < p.M && n < p.N && 4 * c + j < rows) {
+            const int row = (4 * c + j * SPL) / SPL;
+            const int m = m_base + row;
+            if (m < p.M && n < p.N && row < rows) {
                 if (plain)
                     store_float(dst_dt, v, dst, m * dst_sm + n);
                 else
@@ -312,7 +316,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 
     // ---- reduce the waves' partial sums and finish ----
     __syncthreads(); // the staged activations are dead
-    gemv_reduce_store<false>(p, (float *)lds, out, wave, lane, m_base, rows, n);
+    gemv_reduce_store<16>(p, (float *)lds, out, wave, lane, m_base, rows, n);
 }
 
 // Fast kernel: one 16-bit scale and at most one byte-sized (4- or 8-bit) zero
@@ -320,7 +324,13 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 // load is unconditional (out-of-range tiles re-read the last valid one, an
 // absent zero-point buffer is replaced by the weights pointer), so the number
 // of loads in flight is known at compile time and no wait drains the whole
-// queue. ONE_ROW: a single activation row, one activation load per tile.
+// queue. ROWS: 16 activation rows per workgroup (four activation loads per
+// lane and tile, one per MFMA step), at most 8 with two loads, or at most 4 /
+// exactly 1 with ONE load per lane and tile. With SPL = 4, 2, 1 steps per
+// load, load h of lane (r, c) fetches, for activation row r / SPL, the chunk
+// that MFMA step h SPL + r % SPL multiplies; in step s the operand row SPL j
+// takes it from lane SPL j + s % SPL (a shift within the 16 lanes), so every
+// SPL-th row of the MFMA is an activation row and the others are never stored.
 //
 // A launch of this kernel lives a few microseconds, and the first of them
 // passes before its first load is issued. Part of that was the kernel waiting
@@ -336,7 +346,7 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 //     4-bit, 3 zero points signed, 4 scales f16 (else bf16), 5 weights signed,
 //     6 zero points present, 7 plain store (see gemv_reduce_store);
 //     bits 8..: M
-template <bool F16, bool ONE_ROW, bool WSIGNED>
+template <bool F16, int ROWS, bool WSIGNED>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
@@ -390,17 +400,20 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     // never stored; only k past K has to be zeroed (the padded weights decode
     // to the magic offset, not 0).
     const int tiles = kg128;
-    const int rr = min(r, rows - 1);
+    constexpr int SPL = ROWS == 16 ? 1 : ROWS == 8 ? 2 : 4; // steps per load
+    constexpr int NA = 4 / SPL; // activation loads per tile
+    const int rr = ROWS == 1 ? 0 : min(r / SPL, rows - 1);
     const uint16_t *__restrict__ Arow = pA + (int64_t)(m_base + rr) * lda;
     const int nn = min(n, N - 1);
     const uint16_t *const scn = pSC + (scale_per_n ? nn : 0);
     const int zcol = zp_per_n ? nn : 0;
     const bool k_tail = (K & 127) != 0;
     constexpr int UNR = 4;
-    constexpr int NA = ONE_ROW ? 1 : 4; // activation loads per tile
     void *dst_ptr = nullptr;
     int64_t dst_sm = 0;
     int dst_dt = 0;
+    // steps past the end repeat the last tile and are folded with scale 0
+    auto tile_of = [&](int t) { return min(t, tiles - 1); };
     for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
         // Loads are issued tile by tile (weights, activations, scale, zero
         // point) and consumed in the same order below: results return in
@@ -412,20 +425,15 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         uint32_t scp[UNR], zpp[UNR];
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
-            const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
+            const int tc = tile_of(tb + uw + u * GEMV_WAVES);
             wt[u] = ld_stream(Bt + (int64_t)tc * 1024);
-            if constexpr (ONE_ROW) {
-                // a single activation row: lane (r, c) fetches what lane
-                // (0, c) multiplies in step r % 4, one load per tile
-                const int k = min(tc * 128 + (r & 3) * 32 + c * 8, K - 8);
-                av[u][0] = *(const uint4 *)(pA + (int64_t)m_base * lda + k);
-            } else {
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++) {
-                    // chunks past the row's end re-read its last one
-                    const int k = min(tc * 128 + s4 * 32 + c * 8, K - 8);
-                    av[u][s4] = *(const uint4 *)(Arow + k);
-                }
+            for (int h = 0; h < NA; h++) {
+                // chunks past the row's end re-read its last one, rows past M
+                // the last row
+                const int k = min(
+                        tc * 128 + (h * SPL + r % SPL) * 32 + c * 8, K - 8);
+                av[u][h] = *(const uint4 *)(Arow + k);
             }
             const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
             scp[u] = scn[(int64_t)gsc * sN];
@@ -437,16 +445,11 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             // zero the activations past K (last tile of the matrix)
 #pragma unroll
             for (int u = 0; u < UNR; u++) {
-                const int tc = min(tb + uw + u * GEMV_WAVES, tiles - 1);
-                if constexpr (ONE_ROW) {
-                    if (tc * 128 + (r & 3) * 32 + c * 8 >= K)
-                        av[u][0] = make_uint4(0, 0, 0, 0);
-                } else {
+                const int tc = tile_of(tb + uw + u * GEMV_WAVES);
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; s4++)
-                        if (tc * 128 + s4 * 32 + c * 8 >= K)
-                            av[u][s4] = make_uint4(0, 0, 0, 0);
-                }
+                for (int h = 0; h < NA; h++)
+                    if (tc * 128 + (h * SPL + r % SPL) * 32 + c * 8 >= K)
+                        av[u][h] = make_uint4(0, 0, 0, 0);
             }
         }
         // what the final store needs from the (cold) parameter block is
@@ -475,31 +478,27 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                 b.z = ((d >> 8) & NIB) | MAGIC;
                 b.w = ((d >> 12) & NIB) | MAGIC;
                 v4u a;
-                if constexpr (ONE_ROW) {
-                    // row 0 of the operand takes step s4's chunk from lane
-                    // (s4, c); the other rows hold other steps' chunks and
-                    // produce rows of the result that are never stored
-                    const uint4 v = av[u][0];
-                    if (s4 == 0)
+                {
+                    // operand row SPL j takes step s4's chunk from lane
+                    // (SPL j + s4 % SPL, c) of load s4 / SPL
+                    const uint4 v = av[u][s4 / SPL];
+                    if (s4 % SPL == 0)
                         a = v4u {v.x, v.y, v.z, v.w};
-                    else if (s4 == 1)
+                    else if (s4 % SPL == 1)
                         a = v4u {row_shl<1>(v.x), row_shl<1>(v.y),
                                 row_shl<1>(v.z), row_shl<1>(v.w)};
-                    else if (s4 == 2)
+                    else if (s4 % SPL == 2)
                         a = v4u {row_shl<2>(v.x), row_shl<2>(v.y),
                                 row_shl<2>(v.z), row_shl<2>(v.w)};
                     else
                         a = v4u {row_shl<3>(v.x), row_shl<3>(v.y),
                                 row_shl<3>(v.z), row_shl<3>(v.w)};
-                } else {
-                    a = v4u {av[u][s4].x, av[u][s4].y, av[u][s4].z,
-                            av[u][s4].w};
                 }
                 Pu = mfma16<F16>(a, b, Pu);
                 Su = mfma16<F16>(a, ones, Su);
             }
             const int t = tb + uw + u * GEMV_WAVES;
-            const int tc = min(t, tiles - 1);
+            const int tc = tile_of(t);
             // one scale and one zero point per column and tile
             float sc = sc_f16
                     ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[u])
@@ -516,11 +515,11 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             const float off = OFFSET + soff + zp;
             // a single row: only register 0 (row 0) is stored
 #pragma unroll
-            for (int j = 0; j < (ONE_ROW ? 1 : 4); j++)
+            for (int j = 0; j < 4; j += SPL)
                 out[j] = __builtin_fmaf(sc, Pu[j] - off * Su[j], out[j]);
         }
     }
-    gemv_reduce_store<ONE_ROW>(p, red, out, uw, lane, m_base, rows, n,
+    gemv_reduce_store<ROWS>(p, red, out, uw, lane, m_base, rows, n,
             (flags_m & 128) != 0, dst_ptr, dst_sm, dst_dt);
 }
 
@@ -588,17 +587,29 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
                     (int)p.lda, shifts, flags_m, q);
         };
-        const int which = (p.act_f16 ? 4 : 0) | (p.M == 1 ? 2 : 0)
-                | (p.wei_signed ? 1 : 0);
+        const int which = (p.act_f16 ? 8 : 0)
+                + (p.M == 1               ? 2
+                                : p.M <= 4 ? 4
+                                : p.M <= 8 ? 6
+                                           : 0)
+                + (p.wei_signed ? 1 : 0);
         switch (which) {
-            case 0: go(gemv_w4_fast_kernel<false, false, false>); break;
-            case 1: go(gemv_w4_fast_kernel<false, false, true>); break;
-            case 2: go(gemv_w4_fast_kernel<false, true, false>); break;
-            case 3: go(gemv_w4_fast_kernel<false, true, true>); break;
-            case 4: go(gemv_w4_fast_kernel<true, false, false>); break;
-            case 5: go(gemv_w4_fast_kernel<true, false, true>); break;
-            case 6: go(gemv_w4_fast_kernel<true, true, false>); break;
-            default: go(gemv_w4_fast_kernel<true, true, true>); break;
+            case 0: go(gemv_w4_fast_kernel<false, 16, false>); break;
+            case 1: go(gemv_w4_fast_kernel<false, 16, true>); break;
+            case 2: go(gemv_w4_fast_kernel<false, 1, false>); break;
+            case 3: go(gemv_w4_fast_kernel<false, 1, true>); break;
+            case 4: go(gemv_w4_fast_kernel<false, 4, false>); break;
+            case 5: go(gemv_w4_fast_kernel<false, 4, true>); break;
+            case 6: go(gemv_w4_fast_kernel<false, 8, false>); break;
+            case 7: go(gemv_w4_fast_kernel<false, 8, true>); break;
+            case 8: go(gemv_w4_fast_kernel<true, 16, false>); break;
+            case 9: go(gemv_w4_fast_kernel<true, 16, true>); break;
+            case 10: go(gemv_w4_fast_kernel<true, 1, false>); break;
+            case 11: go(gemv_w4_fast_kernel<true, 1, true>); break;
+            case 12: go(gemv_w4_fast_kernel<true, 4, false>); break;
+            case 13: go(gemv_w4_fast_kernel<true, 4, true>); break;
+            case 14: go(gemv_w4_fast_kernel<true, 8, false>); break;
+            default: go(gemv_w4_fast_kernel<true, 8, true>); break;
         }
         return;
     }

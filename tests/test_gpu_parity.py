@@ -645,7 +645,7 @@ def test_mfma_fp8(ctx):
 
 # ---------------------------------------------------------------------------
 # decode: 4-bit weights
-@pytest.mark.parametrize("M", [1, 2, 16, 19])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8, 9, 16, 19])
 @pytest.mark.parametrize("weights_any", [True, False])
 def test_decode_w4_config3(ctx, M, weights_any):
     eng, strm = ctx
