@@ -615,11 +615,15 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
     plain = memory(memory.desc([K, N], dt.s4, T("ab")), eng).write(w)
     res = {}
     wsets = None
-    for M, sets, steps in ((2176, 1, 10), (32, 8, 40), (1, 8, 40)):
+    # the last entry: asymmetric activations (u8 with a u8 zero point per row and 128 k)
+    for M, sets, steps, szp in ((2176, 1, 10, False), (32, 8, 40, False), (1, 8, 40, False), (2176, 1, 10, True)):
         attr = A.primitive_attr()
         attr.set_scales(A.DNNL_ARG_SRC, 3, [1, G], dt.f16)
         attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
-        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.s8, T("ab")), memory.desc([K, N], dt.s4, tag.any),
+        if szp:
+            attr.set_zero_points(A.DNNL_ARG_SRC, 3, [1, G], dt.u8)
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.u8 if szp else dt.s8, T("ab")),
+                                     memory.desc([K, N], dt.s4, tag.any),
                                      memory.desc([M, N], dt.f16, T("ab")), attr=attr)
         prim = A.matmul(pd)
         if wsets is None:
@@ -631,16 +635,21 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
                 m = memory(pd.weights_desc(), eng)
                 hiprt.memcpy_dtod(m.get_data_handle(), first.get_data_handle(), pd.weights_desc().get_size())
                 wsets.append(m)
-        m_src = memory(pd.src_desc(), eng).write(np.clip(np.rint(r.standard_normal((M, K)) * 40), -128, 127).astype(np.int8))
+        a8 = np.clip(np.rint(r.standard_normal((M, K)) * 40), -128, 127)
+        m_src = memory(pd.src_desc(), eng).write((a8 + 128).astype(np.uint8) if szp else a8.astype(np.int8))
+        m_sz = memory(memory.desc([M * (K // G)], dt.u8, T("a")), eng).write(
+            r.integers(100, 156, M * (K // G)).astype(np.uint8))
         ss = O.from_f32(O.F16, r.uniform(0.005, 0.05, (M, K // G)).astype(np.float32))
         m_ss = memory(memory.desc([ss.nbytes], dt.u8, T("a")), eng).write(ss)
         m_sw = memory(memory.desc([sw.nbytes], dt.u8, T("a")), eng).write(sw)
         m_dst = memory(pd.dst_desc(), eng)
 
         def one(i):
-            prim.execute(strm, {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: wsets[i % sets], A.DNNL_ARG_DST: m_dst,
-                                A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: m_ss,
-                                A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: m_sw})
+            ex = {A.DNNL_ARG_SRC: m_src, A.DNNL_ARG_WEIGHTS: wsets[i % sets], A.DNNL_ARG_DST: m_dst,
+                  A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: m_ss, A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: m_sw}
+            if szp:
+                ex[A.DNNL_ARG_ATTR_ZERO_POINTS | A.DNNL_ARG_SRC] = m_sz
+            prim.execute(strm, ex)
 
         for i in range(8):
             one(i)
@@ -654,11 +663,12 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
         ms = e1.elapsed_ms(e0) / steps
         ops = 2.0 * M * K * N
         nbytes = K * N // 2 + sw.nbytes + ss.nbytes + M * K + M * N * 2
-        res["M%d" % M] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / (ms * 1e-3) / 1e12, 1),
+        res["M%d%s" % (M, "_u8_src_zero_points" if szp else "")] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / (ms * 1e-3) / 1e12, 1),
                           "frac_of_int8_peak": round(ops / (ms * 1e-3) / 1e12 / PEAK_INT8, 4),
                           "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                           "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4),
-                          "impl": pd.impl_info_str(), "includes": "scale pre-pass + GEMM"}
+                          "impl": pd.impl_info_str(),
+                          "includes": "scale pre-pass%s + GEMM" % (" with weights column sums" if szp else "")}
     return res
 
 

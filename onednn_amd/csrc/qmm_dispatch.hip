@@ -434,10 +434,17 @@ int64_t k_extent(const qmm_quant_t &a, int which, int kbit, int64_t K) {
     return (a.mask & kbit) ? (int64_t)1 : K;
 }
 
+// mfma_w4a8 with source zero points or a u8 source: the tiled kernel's third
+// mode (weights column sums per group from a pre-pass), at every M
+bool w4a8_src_zp_mode(const qmm_matmul_desc_t &D) {
+    return D.zps[QMM_SRC].set || D.src.dt == dt_u8;
+}
+
 int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
     if (nd != 2) return QMM_UNIMPLEMENTED;
-    if (D.src.dt != dt_s8 || !is_int4(D.wei.dt)) return QMM_UNIMPLEMENTED;
+    if ((D.src.dt != dt_s8 && D.src.dt != dt_u8) || !is_int4(D.wei.dt))
+        return QMM_UNIMPLEMENTED;
     if (!one_of(D.dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s32, dt_s8, dt_u8}))
         return QMM_UNIMPLEMENTED;
     if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
@@ -452,10 +459,20 @@ int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int64_t gk = P.group_k;
     if (P.K % 64 != 0 || gk % 64 != 0 || gk > 32768) return QMM_UNIMPLEMENTED;
     const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
-    const qmm_quant_t &wz = D.zps[QMM_WEI];
-    if (D.zps[QMM_SRC].set) return QMM_UNIMPLEMENTED;
+    const qmm_quant_t &wz = D.zps[QMM_WEI], &sz = D.zps[QMM_SRC];
     if (k_extent(ss, 1, 2, P.K) % gk || k_extent(ws, 0, 1, P.K) % gk
-            || k_extent(wz, 0, 1, P.K) % gk)
+            || k_extent(wz, 0, 1, P.K) % gk || k_extent(sz, 1, 2, P.K) % gk)
+        return QMM_UNIMPLEMENTED;
+    // Source zero points, or a u8 source (read as s8 = u8 - 128 with the zero
+    // point moved along): the group's s32 sum is 16 * sum (s - z_s)(w - z_w),
+    // |s - z_s| <= 383 with 8-bit source zero points, so the bound of the
+    // weights zero-point comment below tightens to gk <= 8192 (4-bit or no
+    // weights zero points) / 1024 (8-bit ones); s32 source zero points have
+    // no bound and stay with the generic implementation.
+    const bool src_zp_mode = w4a8_src_zp_mode(D);
+    if (sz.set && !one_of(sz.dt, {dt_s8, dt_u8})) return QMM_UNIMPLEMENTED;
+    if (src_zp_mode
+            && gk > (wz.set && one_of(wz.dt, {dt_s8, dt_u8}) ? 1024 : 8192))
         return QMM_UNIMPLEMENTED;
     if (ss.set && !one_of(ss.dt, {dt_f32, dt_f16, dt_bf16}))
         return QMM_UNIMPLEMENTED;
@@ -484,8 +501,8 @@ int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
 // scratchpad of mfma_w4a8 behind the packed weights: the per-group arrays
 struct w4a8_scratch_t {
     int64_t Mpad, Npad, ng;
-    bool has_zp;
-    size_t ss_off, rs_off, sw_off, zw_off, total;
+    bool has_zp, src_zp;
+    size_t ss_off, rs_off, sw_off, zw_off, zs_off, c2_off, total;
 };
 w4a8_scratch_t w4a8_scratch(const qmm_matmul_desc_t &D,
         const generic_params_t &P) {
@@ -493,13 +510,16 @@ w4a8_scratch_t w4a8_scratch(const qmm_matmul_desc_t &D,
     s.Mpad = round_up(P.M, 256) + 256;
     s.Npad = round_up(P.N, 256) + 256;
     s.ng = P.ngroups_k;
-    s.has_zp = D.zps[QMM_WEI].set || D.wei.dt == dt_u4;
+    s.src_zp = w4a8_src_zp_mode(D);
+    s.has_zp = D.zps[QMM_WEI].set || D.wei.dt == dt_u4 || s.src_zp;
     const size_t rows = (size_t)s.ng * s.Mpad * 4, cols = (size_t)s.ng * s.Npad * 4;
     s.ss_off = 0;
     s.sw_off = rows;
     s.rs_off = rows + cols;
     s.zw_off = s.rs_off + (s.has_zp ? rows : 0);
-    s.total = s.zw_off + (s.has_zp ? cols : 0);
+    s.zs_off = s.zw_off + (s.has_zp ? cols : 0);
+    s.c2_off = s.zs_off + (s.src_zp ? rows : 0);
+    s.total = s.c2_off + (s.src_zp ? cols : 0);
     return s;
 }
 
@@ -512,7 +532,8 @@ struct w4a8_small_plan_t {
 w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     w4a8_small_plan_t s;
     std::memset(&s, 0, sizeof(s));
-    s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0;
+    s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0
+            && !w4a8_src_zp_mode(P.desc);
     if (!s.use) return s;
     const int64_t ng = P.ngroups_k, tpg = P.group_k / 64;
     const int64_t nblk = (P.N + 127) / 128;
@@ -964,6 +985,19 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         q.swT = (float *)(arrays + sc.sw_off);
         q.rsT = sc.has_zp ? (int32_t *)(arrays + sc.rs_off) : nullptr;
         q.zwT = sc.has_zp ? (int32_t *)(arrays + sc.zw_off) : nullptr;
+        if (sc.src_zp) {
+            const qmm_quant_t &sz = D.zps[QMM_SRC];
+            q.zs = sz.set ? args->zps[QMM_SRC] : nullptr;
+            q.zs_dt = sz.dt;
+            q.zs_sm = P.q_src_zp.strides[0];
+            q.zs_sk = P.q_src_zp.strides[1];
+            q.zs_g = (int32_t)k_extent(sz, 1, 2, P.K);
+            q.a_flip = D.src.dt == dt_u8 ? 0x80808080u : 0u;
+            q.kt64 = (int32_t)geom.kt64;
+            q.B = packed;
+            q.zsT = (int32_t *)(arrays + sc.zs_off);
+            q.c2T = (int32_t *)(arrays + sc.c2_off);
+        }
         const w4a8_small_plan_t sm = w4a8_small_plan(P, w4a8_variant);
         if (sm.use && gemm_w4a8_small_takes(q)) {
             w4a8_small_t h;
@@ -1009,6 +1043,9 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.rsT = q.rsT;
         g.swT = q.swT;
         g.zwT = q.zwT;
+        g.zsT = q.zsT;
+        g.c2T = q.c2T;
+        g.a_flip = q.a_flip;
         g.M = q.M;
         g.N = q.N;
         g.K = q.K;

@@ -18,6 +18,11 @@
 //   * zero points and the u4 offset leave the dot product through the row sums
 //     of the source: sum(s * (w - z)) = sum(s * w') - (z - off) * sum(s), all in
 //     s32 (off = 8 for u4, 0 for s4);
+//   * source zero points and u8 sources (read as s' = s - 128 by flipping the
+//     top bit of each byte, zero point z_s' = z_s - 128) add the mirror term
+//     through the column sums of the stored nibbles per group:
+//     16 sum((s' - z_s')(w' - z_w')) = 16 sum(s' w') - 16 z_w' sum(s')
+//         - z_s' * 16 (sum(w') - group * z_w');
 //   * a pre-pass (w4a8_prep_kernel) rewrites the scale and zero-point buffers of
 //     the launch, whatever their data types and strides, as f32 / s32 arrays
 //     [group][row] and [group][column] in the scratchpad and computes the row
@@ -107,15 +112,21 @@ QMM_D int zp_value(int dt, uint32_t raw, int64_t idx) {
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool HAS_ZP>
+// ZPM: 0 no zero points and s4 weights; 1 weights zero points or u4 weights
+// (the group's source row sums take part); 2 also source zero points or a u8
+// source (the group's weights column sums take part, and the source bytes
+// are shifted to s8 by flipping their top bit).
+template <int BM, int BN, int WGM, int WGN, int STAGES, int ZPM>
 __global__ void __launch_bounds__(WGM *WGN * 64, 2)
 gemm_w4a8_kernel(const w4a8_params_t p) {
+    constexpr bool HAS_ZP = ZPM >= 1, SRC_ZP = ZPM == 2;
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int FM = WM / 32, FN = WN / 32;
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK / 2;
     constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    constexpr int NX = HAS_ZP ? 4 : 2; // per-group arrays: ss, sw [, rs, zw]
+    // per-group arrays: ss, sw [, rs, zw [, zs, c2]]
+    constexpr int NX = SRC_ZP ? 6 : HAS_ZP ? 4 : 2;
     constexpr int XSLOT = NX * X_BYTES;
     constexpr int X_OFF = STAGES * STAGE_BYTES;
     // wave-wide 1 KiB loads per tile / per group, spread over the waves; a
@@ -189,11 +200,14 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
 #pragma unroll
     for (int j = 0; j < PER_X; j++) {
         const int x = (wave * PER_X + j) % NX;
-        const bool row_side = (x & 1) == 0; // 0: ss, 1: sw, 2: rs, 3: zw
+        // 0: ss, 1: sw, 2: rs, 3: zw, 4: zs, 5: c2
+        const bool row_side = (x & 1) == 0;
         const void *base = x == 0 ? (const void *)p.ssT
                 : x == 1          ? (const void *)p.swT
                 : x == 2          ? (const void *)p.rsT
-                                  : (const void *)p.zwT;
+                : x == 3          ? (const void *)p.zwT
+                : x == 4          ? (const void *)p.zsT
+                                  : (const void *)p.c2T;
         x_ptr[j] = (const uint8_t *)base
                 + ((int64_t)(row_side ? m0 : n0) + lane * 4) * 4;
         x_step[j] = (int64_t)(row_side ? p.Mpad : p.Npad) * 4;
@@ -267,7 +281,11 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
                 const int q = ki * 2 + (lane >> 5);
                 const uint4 v = *(const uint4 *)(As + row * BK
                         + a_swz(row, q) * 16);
-                a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                if constexpr (SRC_ZP) // u8 source: s - 128 as s8
+                    a[i] = v4i {(int)(v.x ^ p.a_flip), (int)(v.y ^ p.a_flip),
+                            (int)(v.z ^ p.a_flip), (int)(v.w ^ p.a_flip)};
+                else
+                    a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
             }
 #pragma unroll
             for (int j = 0; j < FN; j++) {
@@ -300,7 +318,8 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
         for (int t = 1; t < p.tpg; t++)
             tile_mma(kt++, std::false_type {});
 
-        // ---- group end: res += (float)(acc [- z * rowsum]) * ss * sw ----
+        // ---- group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+        // (zw = -16 (z_w - offset); c2 = -16 (column sum - group * (z_w - offset)))
         // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
         // column l%32 of its fragment.
         const uint8_t *xs = lds + X_OFF + (g % STAGES) * XSLOT;
@@ -308,20 +327,30 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
         const float *swl = (const float *)(xs + X_BYTES);
         const int32_t *rsl = (const int32_t *)(xs + 2 * X_BYTES);
         const int32_t *zwl = (const int32_t *)(xs + 3 * X_BYTES);
+        const int32_t *zsl = (const int32_t *)(xs + 4 * X_BYTES);
+        const int32_t *c2l = (const int32_t *)(xs + 5 * X_BYTES);
         float sw[FN];
-        int zw[FN];
+        int zw[FN], c2[FN];
 #pragma unroll
         for (int j = 0; j < FN; j++) {
             sw[j] = swl[wn0 + j * 32 + (lane & 31)];
             zw[j] = HAS_ZP ? zwl[wn0 + j * 32 + (lane & 31)] : 0;
+            c2[j] = SRC_ZP ? c2l[wn0 + j * 32 + (lane & 31)] : 0;
         }
         static_for<FM>([&](auto I) {
             constexpr int i = decltype(I)::value;
             float ss[16];
-            int rs[16];
+            int rs[16], zs[16];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int row = wm0 + i * 32 + 8 * q + 4 * (lane >> 5);
+                if constexpr (SRC_ZP) {
+                    const int4 z4 = *(const int4 *)&zsl[row];
+                    zs[4 * q + 0] = z4.x;
+                    zs[4 * q + 1] = z4.y;
+                    zs[4 * q + 2] = z4.z;
+                    zs[4 * q + 3] = z4.w;
+                }
                 const float4 s4 = *(const float4 *)&ssl[row];
                 ss[4 * q + 0] = s4.x;
                 ss[4 * q + 1] = s4.y;
@@ -341,6 +370,7 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
                 for (int r = 0; r < 16; r++) {
                     int t = acc[i][j][r];
                     if constexpr (HAS_ZP) t += __mul24(zw[j], rs[r]);
+                    if constexpr (SRC_ZP) t += __mul24(zs[r], c2[j]);
                     res[i][j][r] = __builtin_fmaf(
                             (float)t * ss[r], sw[j], res[i][j][r]);
                 }
@@ -402,12 +432,19 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
                     ? load_float(p.ss_dt, p.ss,
                             m * p.ss_sm + (k0 / p.ss_g) * p.ss_sk)
                     : 1.f;
+            if (p.zsT) // source zero point of the (row, group), as s8 counts
+                p.zsT[(int64_t)g * p.Mpad + m]
+                        = (p.zs ? load_int(p.zs_dt, p.zs,
+                                   m * p.zs_sm + (k0 / p.zs_g) * p.zs_sk)
+                                : 0)
+                        - (p.a_flip ? 128 : 0);
             if (p.rsT) {
                 const uint8_t *a = p.A + (int64_t)m * p.lda + k0;
                 int sum = 0;
                 for (int k = 0; k < p.gk; k += 16) {
                     const uint4 v = *(const uint4 *)(a + k);
-                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                    const uint32_t w[4] = {v.x ^ p.a_flip, v.y ^ p.a_flip,
+                            v.z ^ p.a_flip, v.w ^ p.a_flip};
 #pragma unroll
                     for (int d = 0; d < 4; d++)
                         sum += (int)(int8_t)(w[d] & 0xff)
@@ -430,6 +467,36 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
                                       (k0 / p.zw_g) * p.zw_sk + n * p.zw_sn)
                                    : 0;
                 p.zwT[(int64_t)g * p.Npad + n] = -16 * (z - p.w_off);
+                if (p.c2T) {
+                    // column sum of the group's stored nibbles w' (signed):
+                    // the 64 k of a tile are the 16-byte pieces of lanes
+                    // n % 32 and n % 32 + 32 of the column block's tile
+                    const int tpg = p.gk / 64;
+                    const uint8_t *b = p.B
+                            + (((int64_t)(n >> 5) * p.kt64 + (int64_t)g * tpg) * 64
+                                      + (n & 31))
+                                    * 16;
+                    int sum = 0;
+                    for (int t = 0; t < tpg; t++) {
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const uint4 v = *(const uint4 *)(b + (int64_t)t * 1024
+                                    + h * 512);
+                            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                            for (int d = 0; d < 4; d++) {
+                                // nibble ^ 8 is w' + 8: bytewise sums of the
+                                // low and high nibbles, then of the four bytes
+                                const uint32_t y = w[d] ^ 0x88888888u;
+                                const uint32_t e = (y & 0x0F0F0F0Fu)
+                                        + ((y >> 4) & 0x0F0F0F0Fu);
+                                sum += (int)((e * 0x01010101u) >> 24) - 64;
+                            }
+                        }
+                    }
+                    p.c2T[(int64_t)g * p.Npad + n]
+                            = -16 * sum + p.gk * 16 * (z - p.w_off);
+                }
             }
         }
     }
@@ -1016,32 +1083,33 @@ static void launch_small_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         launch_small_cfg<FM, SC, true, 2>(p, stream);
 }
 
-template <int BM, int BN, int WGM, int WGN, bool HAS_ZP>
+template <int BM, int BN, int WGM, int WGN, int ZPM>
 static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
     // a tile is only 8 MFMAs per wave: five stages (four tiles in flight) are
     // what it takes to cover the L2 / HBM latency; two workgroups still fit
-    constexpr int STAGES = 5;
+    // (four stages with the six per-group arrays of ZPM = 2)
+    constexpr int STAGES = ZPM == 2 ? 4 : 5;
     w4a8_params_t q = p;
     q.tiles_m = (p.M + BM - 1) / BM;
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ntiles >= 64 ? ((ntiles + 7) / 8) * 8 : ntiles;
     constexpr size_t lds_main = (size_t)STAGES
-            * (BM * BK + BN * BK / 2 + (HAS_ZP ? 4 : 2) * X_BYTES);
+            * (BM * BK + BN * BK / 2 + (ZPM == 2 ? 6 : ZPM == 1 ? 4 : 2) * X_BYTES);
     constexpr size_t lds_ep
             = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
     constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
-    auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, HAS_ZP>;
+    auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, ZPM>;
     ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3(grid_x), dim3(WGM * WGN * 64), lds, stream, q);
 }
 
-template <bool HAS_ZP>
+template <int ZPM>
 static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
     switch (variant) {
-        case 1: launch_cfg<128, 128, 2, 2, HAS_ZP>(p, stream); break;
-        case 2: launch_cfg<64, 128, 2, 2, HAS_ZP>(p, stream); break;
-        default: launch_cfg<32, 64, 1, 2, HAS_ZP>(p, stream); break;
+        case 1: launch_cfg<128, 128, 2, 2, ZPM>(p, stream); break;
+        case 2: launch_cfg<64, 128, 2, 2, ZPM>(p, stream); break;
+        default: launch_cfg<32, 64, 1, 2, ZPM>(p, stream); break;
     }
 }
 
@@ -1049,18 +1117,23 @@ static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
 
 // The kernel families build in translation units of their own (QMM_W4A8_PART:
 // 1, 2 the tiled GEMM without / with zero points, 3 the split-K kernel and its
-// reduction, 4 the single-token kernel); the unit without the macro holds the
-// pre-pass and the dispatch.
+// reduction, 4 the single-token kernel, 5 the tiled GEMM with source zero
+// points); the unit without the macro holds the pre-pass and the dispatch.
 #if defined(QMM_W4A8_PART)
 #if QMM_W4A8_PART == 1
 void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
-    w4a8::launch_zp<false>(p, variant, stream);
+    w4a8::launch_zp<0>(p, variant, stream);
 }
 #elif QMM_W4A8_PART == 2
 void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
-    w4a8::launch_zp<true>(p, variant, stream);
+    w4a8::launch_zp<1>(p, variant, stream);
+}
+#elif QMM_W4A8_PART == 5
+void launch_gemm_w4a8_szp(const w4a8_params_t &p, int variant,
+        hipStream_t stream) {
+    w4a8::launch_zp<2>(p, variant, stream);
 }
 #elif QMM_W4A8_PART == 3
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
@@ -1103,6 +1176,8 @@ void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
 void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
         hipStream_t stream);
 void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
+        hipStream_t stream);
+void launch_gemm_w4a8_szp(const w4a8_params_t &p, int variant,
         hipStream_t stream);
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, hipStream_t stream);
@@ -1162,7 +1237,9 @@ void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream) {
         variant = big >= 256 ? 1 : ((mid >= 128 && p.M > 32) ? 2 : 3);
         if (variant == 3 && p.M > 64) variant = 2;
     }
-    if (p.zwT)
+    if (p.zsT)
+        launch_gemm_w4a8_szp(p, variant, stream);
+    else if (p.zwT)
         launch_gemm_w4a8_zp(p, variant, stream);
     else
         launch_gemm_w4a8_nozp(p, variant, stream);

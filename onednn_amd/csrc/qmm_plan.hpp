@@ -191,13 +191,17 @@ struct w4a8_params_t {
     const int32_t *rsT; // [ng][Mpad] source row sums per group, or nullptr
     const float *swT; // [ng][Npad] weights scales / 16
     const int32_t *zwT; // [ng][Npad] -16 * (zero point - offset), or nullptr
+    // source zero points / u8 source (both or neither): [ng][Mpad] the zero
+    // point of the source taken as s8, [ng][Npad] -16 * (column sum of the
+    // stored nibbles - group * (zero point - offset))
+    const int32_t *zsT, *c2T;
     int32_t M, N, K;
     int32_t Mpad, Npad;
     int32_t kt64, nb32;
     int32_t tpg; // 64-k tiles per group
     int32_t ng;
     int32_t tiles_m, tiles_n;
-    int32_t pad_;
+    uint32_t a_flip; // 0x80808080 for a u8 source (read as s8 = u8 - 128)
     epilogue_t ep;
 };
 
@@ -214,6 +218,14 @@ struct w4a8_prep_t {
     int32_t *rsT;
     float *swT;
     int32_t *zwT;
+    // source zero points / u8 source
+    const void *zs; // nullptr: 0
+    int32_t zs_dt, zs_g;
+    int64_t zs_sm, zs_sk;
+    uint32_t a_flip;
+    int32_t kt64;
+    const uint8_t *B; // packed weights (column sums)
+    int32_t *zsT, *c2T; // nullptr unless the source has zero points or is u8
 };
 
 // Rows <= 64 (decode): the K range is cut into `splits` slices of `gps` groups,

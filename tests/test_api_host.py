@@ -343,7 +343,7 @@ def test_generic_takes_what_the_tiled_kernels_do_not(eng):
     assert pd.impl_info_str() == "hip:gfx950:mfma_w4a8"
     assert pd.weights_desc().get_format_kind() == memory.format_kind.opaque
     assert pd.weights_desc().get_size() == 128 * 32 // 2
-    # ... and to the generic kernel otherwise (groups of 32, source zero points)
+    # ... and to the generic kernel otherwise (groups of 32, s32 source zero points)
     attr = dnnl.primitive_attr()
     attr.set_scales(dnnl.DNNL_ARG_SRC, 3, [1, 32], dt.f16)
     attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 3, [32, 1], dt.f16)
@@ -353,10 +353,17 @@ def test_generic_takes_what_the_tiled_kernels_do_not(eng):
     assert pd.weights_desc().get_format_kind() == memory.format_kind.blocked
     attr = dnnl.primitive_attr()
     attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 3, [64, 1], dt.f16)
-    attr.set_zero_points(dnnl.DNNL_ARG_SRC, 3, [1, 64], dt.s8)
+    attr.set_zero_points(dnnl.DNNL_ARG_SRC, 3, [1, 64], dt.s32)
     pd = dnnl.matmul.primitive_desc(eng, memory.desc([4, 128], dt.s8, T("ab")), memory.desc([128, 32], dt.s4, T("ab")),
                                     memory.desc([4, 32], dt.f32, T("ab")), attr=attr)
     assert pd.impl_info_str() == "hip:gfx950:generic"
+    # 8-bit source zero points per row and K group, and u8 sources, stay on the MFMA path
+    attr = dnnl.primitive_attr()
+    attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 3, [64, 1], dt.f16)
+    attr.set_zero_points(dnnl.DNNL_ARG_SRC, 3, [1, 64], dt.u8)
+    pd = dnnl.matmul.primitive_desc(eng, memory.desc([4, 128], dt.u8, T("ab")), memory.desc([128, 32], dt.s4, T("ab")),
+                                    memory.desc([4, 32], dt.f32, T("ab")), attr=attr)
+    assert pd.impl_info_str() == "hip:gfx950:mfma_w4a8"
     # transposed source
     pd = dnnl.matmul.primitive_desc(eng, memory.desc([64, 64], dt.s8, T("ba")), memory.desc([64, 64], dt.s8, T("ab")),
                                     memory.desc([64, 64], dt.s32, T("ab")))

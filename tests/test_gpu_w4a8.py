@@ -42,15 +42,18 @@ def variant(request):
 
 
 def dynamic_quant(M, K, N, seed, wei_dt=dt.s4, gs=128, gw=128, gz=None, zp_dt=dt.u8, exact=False,
-                  dst_dt=dt.f32, scale_dt=dt.f16, post_ops=None, wei_layout="ab", dst_init=None):
+                  dst_dt=dt.f32, scale_dt=dt.f16, post_ops=None, wei_layout="ab", dst_init=None,
+                  src_dt=dt.s8, src_zp=None, src_zp_dt=dt.u8):
     """s8 src with per-row K-grouped scales (1 x gs), int4 weights with K-grouped
     scales (gw x 1) and optional zero points (gz x 1): the layout of
     tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu:32-117."""
     r = np.random.default_rng(seed)
     s = np.clip(np.rint(r.standard_normal((M, K)) * 40), -128, 127)
+    if src_dt == dt.u8:
+        s = s + 128
     lo, hi = (0, 16) if wei_dt == dt.u4 else (-8, 8)
     w = r.integers(lo, hi, (K, N))
-    src = TensorSpec(dt.s8, [M, K], None, s)
+    src = TensorSpec(src_dt, [M, K], None, s)
     wei = TensorSpec(wei_dt, [K, N], wei_layout, w)
     dst = TensorSpec(dst_dt, [M, N], None, dst_init)
     if exact:
@@ -67,6 +70,16 @@ def dynamic_quant(M, K, N, seed, wei_dt=dt.s4, gs=128, gw=128, gz=None, zp_dt=dt
         else:
             z = r.integers(5, 12, (K // gz, N))
         zps["wei"] = (3, zp_dt, (gz, 1), z)
+    # source zero points: "common" (one value), "k" (per K group of src_zp[1]), "mk" (per row and K group)
+    if src_zp is not None:
+        kind, g = src_zp
+        zlo, zhi = (100, 156) if src_zp_dt == dt.u8 else (-20, 21)
+        if kind == "common":
+            zps["src"] = (0, src_zp_dt, None, r.integers(zlo, zhi, (1,)))
+        elif kind == "k":
+            zps["src"] = (2, src_zp_dt, (1, g), r.integers(zlo, zhi, (K // g,)))
+        else:
+            zps["src"] = (3, src_zp_dt, (1, g), r.integers(zlo, zhi, (M, K // g)))
     p = Problem(src, wei, dst, scales=scales, zps=zps, post_ops=post_ops)
     # magnitude of one group's term, for the relative bar
     p.term_scale = float(np.abs(s).mean() * 4 * np.sqrt(min(gs, gw)) * ss.mean() * sw.mean())
@@ -90,6 +103,17 @@ EXACT_CASES = {
     "m3_k2048_g64": dict(M=3, K=2048, N=70, gs=64, gw=64, gz=64, zp_dt=dt.s4),
     "m4_k8192": dict(M=4, K=8192, N=96),
     "edges": dict(M=129, K=320, N=162, gs=64, gw=64),
+    # source zero points / u8 sources: the tiled kernel's third mode at every M
+    "u8_src_no_zp": dict(M=70, K=256, N=100, src_dt=dt.u8),
+    "u8_src_common_zp": dict(M=130, K=384, N=96, src_dt=dt.u8, src_zp=("common", 0), wei_dt=dt.u4),
+    "u8_src_zp_per_row_group": dict(M=200, K=512, N=130, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128),
+    "s8_src_zp_s8_per_row_group64": dict(M=33, K=256, N=64, gs=64, gw=64, gz=64, zp_dt=dt.s4, src_zp=("mk", 64),
+                                         src_zp_dt=dt.s8),
+    "s8_src_zp_per_group_wider_than_scales": dict(M=17, K=512, N=48, gs=128, gw=128, src_zp=("k", 256),
+                                                  src_zp_dt=dt.s8, gz=128, zp_dt=dt.u8, wei_dt=dt.u4),
+    "u8_src_zp_m1": dict(M=1, K=512, N=160, src_dt=dt.u8, src_zp=("mk", 128)),
+    "u8_src_zp_m300_k2048": dict(M=300, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
+                                 zp_dt=dt.u4),
 }
 
 
