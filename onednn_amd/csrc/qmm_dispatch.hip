@@ -27,6 +27,9 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
+void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
+        int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
+        int src_zp_dt, hipStream_t stream);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream);
@@ -382,7 +385,7 @@ int64_t wei_batch(const qmm_matmul_desc_t &D) {
 
 int supports_gemm_b8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
-    const bool i8 = is_int8(D.src.dt) && D.wei.dt == dt_s8;
+    const bool i8 = is_int8(D.src.dt) && is_int8(D.wei.dt);
     const bool f8 = D.src.dt == dt_f8_e4m3 && D.wei.dt == dt_f8_e4m3;
     if (!i8 && !f8) return QMM_UNIMPLEMENTED;
     if (i8 && !one_of(D.dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s32, dt_s8, dt_u8}))
@@ -409,7 +412,14 @@ int supports_gemm_b8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     int64_t a_sb;
     if (!fold_batch(D.src, D.dst, a_sb) || a_sb % 16 != 0)
         return QMM_UNIMPLEMENTED;
-    if (D.zps[QMM_WEI].set) return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_WEI].set) {
+        // one zero point for the tensor or per column (no groups): applied
+        // through the source's row sums in the general kernel's epilogue
+        const qmm_quant_t &wz = D.zps[QMM_WEI];
+        if (!i8 || (wz.mask & ~(1 << (nd - 1))) || wz.has_groups)
+            return QMM_UNIMPLEMENTED;
+        if (!one_of(wz.dt, {dt_s32, dt_s8, dt_u8})) return QMM_UNIMPLEMENTED;
+    }
     if (D.zps[QMM_SRC].set) {
         if (!i8 || D.zps[QMM_SRC].mask != 0) return QMM_UNIMPLEMENTED;
         if (!one_of(D.zps[QMM_SRC].dt, {dt_s32, dt_s8, dt_u8}))
@@ -709,9 +719,24 @@ int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
 
 // Large u8-source problems go through the 256 x 256 kernel after a pre-pass
 // that rewrites the source as s8: room for that copy, behind the packed weights.
+// mfma_b8 with weights zero points or u8 weights: the source's row sums (s32
+// per batch and row) live in the scratchpad behind the packed weights
+static bool b8_needs_rowsum(const qmm_matmul_desc_t &D) {
+    return is_int8(D.src.dt) && (D.wei.dt == dt_u8 || D.zps[QMM_WEI].set);
+}
+static size_t b8_rowsum_bytes(const qmm_matmul_desc_t &D) {
+    if (!b8_needs_rowsum(D)) return 0;
+    const int nd = D.dst.ndims;
+    int64_t rows = D.dst.dims[nd - 2];
+    for (int d = 0; d < nd - 2; d++)
+        rows *= D.dst.dims[d];
+    return (size_t)rows * 4;
+}
+
 static size_t u8_copy_bytes(const qmm_matmul_desc_t *desc) {
     const int nd = desc->dst.ndims;
     if (desc->src.dt != dt_u8) return 0;
+    if (b8_needs_rowsum(*desc)) return 0; // never the 256 x 256 kernels
     const int64_t M = desc->dst.dims[nd - 2], N = desc->dst.dims[nd - 1];
     const int64_t K = desc->src.dims[nd - 1];
     int64_t batch = 1;
@@ -734,7 +759,7 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
                 ? qmm_packed_size(QMM_LAYOUT_MFMA_B8, desc->wei.dt,
                         wei_batch(*desc), K, N)
                 : 0;
-        const size_t copy = u8_copy_bytes(desc);
+        const size_t copy = u8_copy_bytes(desc) + b8_rowsum_bytes(*desc);
         return copy ? round256(packed) + copy : packed;
     }
     if (impl == impl_gemm_w4a8) {
@@ -914,6 +939,20 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.src_zp = D.zps[QMM_SRC].set ? args->zps[QMM_SRC] : nullptr;
         g.src_zp_dt = D.zps[QMM_SRC].dt;
         g.a_is_u8 = D.src.dt == dt_u8;
+        if (b8_needs_rowsum(D)) {
+            const qmm_quant_t &wz = D.zps[QMM_WEI];
+            int32_t *rs = (int32_t *)((uint8_t *)args->scratch
+                    + (D.wei_layout == QMM_LAYOUT_PLAIN
+                                    ? round256(geom.total_bytes)
+                                    : 0));
+            launch_rowsum_b8(g.A, rs, P.batch, P.M, P.K, g.lda, g.a_sb,
+                    D.src.dt == dt_u8, g.src_zp, g.src_zp_dt, stream);
+            g.rowsum = rs;
+            g.wei_zp = wz.set ? args->zps[QMM_WEI] : nullptr;
+            g.wei_zp_dt = wz.dt;
+            g.wei_zp_sn = wz.set && (wz.mask & (1 << (nd - 1))) ? 1 : 0;
+            g.w_off = D.wei.dt == dt_u8 ? 128 : 0;
+        }
         g.M = (int32_t)P.M;
         g.N = (int32_t)P.N;
         g.K = (int32_t)P.K;

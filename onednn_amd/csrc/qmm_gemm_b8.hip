@@ -301,14 +301,22 @@ gemm_b8_kernel(const gemm_params_t p) {
     // back row-wise, 4 neighbouring columns per lane, so that the post-op code
     // exists once (run-time loop) and every store is a dense vector.
     float *const stg = (float *)lds + wave * (32 * WN);
-    int cs[FN];
+    int cs[FN], zwn[FN];
+    const bool has_wz = !F8 && p.rowsum != nullptr; // block uniform
 #pragma unroll
     for (int j = 0; j < FN; j++) {
         cs[j] = 0;
+        zwn[j] = 0;
         if constexpr (!F8) {
             const int n = n0 + wn0 + j * 32 + (lane & 31);
             if (n < p.N && comp != 0 && p.colsum)
                 cs[j] = comp * p.colsum[(int64_t)bz * p.colsum_sb + n];
+            // zero point of the stored (s8) weights of the lane's column
+            if (has_wz && n < p.N)
+                zwn[j] = (p.wei_zp ? load_int(p.wei_zp_dt, p.wei_zp,
+                                  (int64_t)n * p.wei_zp_sn)
+                                   : 0)
+                        - p.w_off;
         }
     }
     constexpr int ROWS_PER_IT = 256 / WN; // 64 lanes x 4 columns
@@ -329,6 +337,19 @@ gemm_b8_kernel(const gemm_params_t p) {
     const float ws4[4] = {cols.ws[0], cols.ws[1], cols.ws[2], cols.ws[3]};
     static_for<FM>([&](auto I) {
         constexpr int i = decltype(I)::value;
+        // weights zero points: the row sums of the lane's 16 rows (s32
+        // arithmetic wraps as the reference's int accumulation does)
+        int rsr[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) rsr[r] = 0;
+        if (has_wz) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                const int m = min(m0 + wm0 + i * 32 + row, p.M - 1);
+                rsr[r] = p.rowsum[(int64_t)bz * p.M + m];
+            }
+        }
 #pragma unroll
         for (int j = 0; j < FN; j++) {
 #pragma unroll
@@ -339,7 +360,8 @@ gemm_b8_kernel(const gemm_params_t p) {
                     v = acc[i][j][r];
                 else
                     v = (float)(int32_t)((uint32_t)acc[i][j][r]
-                            + (uint32_t)cs[j]);
+                            + (uint32_t)cs[j]
+                            - (uint32_t)zwn[j] * (uint32_t)rsr[r]);
                 stg[row * WN + j * 32 + (lane & 31)] = v;
             }
         }

@@ -1488,6 +1488,7 @@ static bool short_k(const gemm_params_t &p) {
 
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     if (p.K % 64 != 0 || p.K < 64) return false;
+    if (p.rowsum) return false; // weights zero points: the general kernel
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
     if (p.a_is_u8 && !p.a_preflipped && !short_k(p)) return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;

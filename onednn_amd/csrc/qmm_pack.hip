@@ -33,13 +33,17 @@ pack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
         const int64_t nb = frag / g.kb32, kb = frag % g.kb32;
         const int64_t n = nb * 32 + (lane & 31);
         const int64_t k0 = kb * 32 + (lane >> 5) * 16;
+        const uint32_t flip = p.dt == dt_u8 ? 0x80u : 0u;
         uint32_t w[4] = {0, 0, 0, 0};
         if (n < p.N) {
             const uint8_t *s = p.src + b * p.sb + n * p.sn;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int64_t k = k0 + i;
-                const uint32_t v = k < p.K ? s[k * p.sk] : 0u;
+                // u8 weights are stored as s8 = u8 - 128 (top bit flipped);
+                // the padding stays 0
+                const uint32_t v
+                        = k < p.K ? (uint32_t)s[k * p.sk] ^ flip : 0u;
                 w[i / 4] |= v << (8 * (i % 4));
             }
         }
@@ -47,7 +51,8 @@ pack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
     }
 }
 
-// column sums of the (signed or unsigned) 8-bit weights: blockIdx.y cuts K into
+// column sums of the 8-bit weights as the kernels see them (s8; u8 weights
+// minus 128): blockIdx.y cuts K into
 // chunks of COLSUM_KCHUNK rows, a thread sums one column of its chunk and adds
 // the partial sum to the (zeroed) s32 result -- integer atomics, so the result
 // does not depend on the order
@@ -74,7 +79,9 @@ colsum_kernel(const pack_params_t p, const b8_geom_t g) {
         int32_t acc = 0;
         for (int64_t k = k0; k < k1; k++) {
             const uint8_t v = s[k * p.sk];
-            acc += p.dt == dt_s8 ? (int32_t)(int8_t)v : (int32_t)v;
+            acc += p.dt == dt_s8 ? (int32_t)(int8_t)v
+                    : p.dt == dt_u8 ? (int32_t)v - 128
+                                    : (int32_t)v;
         }
         atomicAdd((int32_t *)(p.dst + g.colsum_off) + i, acc);
     }
@@ -88,7 +95,8 @@ unpack_b8_kernel(const pack_params_t p, const b8_geom_t g) {
             i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t n = i % p.N, k = (i / p.N) % p.K, b = i / (p.N * p.K);
         p.dst[b * p.sb + k * p.sk + n * p.sn]
-                = p.src[b * g.batch_bytes + b8_offset(g, k, n)];
+                = p.src[b * g.batch_bytes + b8_offset(g, k, n)]
+                ^ (p.dt == dt_u8 ? 0x80 : 0);
     }
 }
 
@@ -269,6 +277,48 @@ void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
     hipLaunchKernelGGL(flip_u8_kernel, dim3(grid_for(batch * M * K / 16)),
             dim3(256), 0, stream, (const uint8_t *)src, (uint8_t *)dst,
             batch * M, K / 16, M, lda, a_sb);
+}
+
+// Row sums of the 8-bit source as the kernels see it (s8; a u8 source minus
+// 128), plus K times the source compensation (128 for a u8 source, minus the
+// source zero point): what a weights zero point multiplies,
+//   sum_k (s - z_s)(w - z_w) = P + comp * colsum[n] - z_w' * (rowsum[m] + K * comp)
+// with P the s8 x s8 product sum and z_w' the zero point of the stored s8
+// weights. One wave per row.
+__global__ void __launch_bounds__(256)
+rowsum_b8_kernel(const uint8_t *src, int32_t *dst, int64_t rows, int64_t M,
+        int64_t K, int64_t lda, int64_t a_sb, int a_is_u8, const void *src_zp,
+        int src_zp_dt) {
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const uint8_t *a = src + (r / M) * a_sb + (r % M) * lda;
+    const uint32_t flip = a_is_u8 ? 0x80808080u : 0u;
+    int sum = 0;
+    for (int64_t k = lane * 16; k < K; k += 64 * 16) { // K % 16 == 0
+        const uint4 v = *(const uint4 *)(a + k);
+        const uint32_t w[4] = {v.x ^ flip, v.y ^ flip, v.z ^ flip, v.w ^ flip};
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+            sum += (int)(int8_t)(w[d] & 0xff) + (int)(int8_t)((w[d] >> 8) & 0xff)
+                    + (int)(int8_t)((w[d] >> 16) & 0xff) + (int)(int8_t)(w[d] >> 24);
+    }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) sum += __shfl_xor(sum, o);
+    if (lane == 0) {
+        int comp = a_is_u8 ? 128 : 0;
+        if (src_zp) comp -= load_int(src_zp_dt, src_zp, 0);
+        dst[r] = sum + (int)K * comp;
+    }
+}
+
+void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
+        int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
+        int src_zp_dt, hipStream_t stream) {
+    const int64_t rows = batch * M;
+    hipLaunchKernelGGL(rowsum_b8_kernel, dim3((unsigned)((rows + 3) / 4)),
+            dim3(256), 0, stream, (const uint8_t *)src, dst, rows, M, K, lda,
+            a_sb, a_is_u8 ? 1 : 0, src_zp, src_zp_dt);
 }
 
 void launch_unpack_b8(const void *src, void *dst, int dt, int64_t batch,

@@ -156,6 +156,12 @@ struct gemm_params_t {
     int32_t nb32;
     int32_t tiles_m, tiles_n;
     int32_t a_preflipped; // u8 source already rewritten as s8 (x ^ 0x80)
+    // weights zero points / u8 weights (stored as s8 = u8 - 128): the zero
+    // point of the stored weights is zp[n * wei_zp_sn] - w_off, applied through
+    // rowsum (see rowsum_b8_kernel); nullptr rowsum: neither
+    const void *wei_zp; // nullptr: 0
+    int32_t wei_zp_dt, wei_zp_sn, w_off, pad2_;
+    const int32_t *rowsum; // [batch][M]
     epilogue_t ep;
 };
 
