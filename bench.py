@@ -242,21 +242,34 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
     G = 128
     r = np.random.default_rng(3)
     res = {}
-    w = O.pack4(r.integers(0, 16, (K, N)))
-    sc = O.from_f32(O.F16, r.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
-    zp = O.pack4(r.integers(6, 10, (K // G, N)))
-    for M in rows:
+    w4 = O.pack4(r.integers(0, 16, (K, N)))
+    sc4 = O.from_f32(O.F16, r.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
+    zp4 = O.pack4(r.integers(6, 10, (K // G, N)))
+    # the last entry: 8-bit weights-only quantization, one f16 scale and u8 zero point per column
+    # (tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu: --dt=f16:u8:f16, wei:per_oc)
+    for M, w8 in [(m, False) for m in rows] + [(1, True)]:
         attr = A.primitive_attr()
-        attr.set_fpmath_mode(A.fpmath_mode.bf16, True)
-        attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
-        attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.u4)
-        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.bf16, T("ab")), memory.desc([K, N], dt.u4, tag.any),
-                                     memory.desc([M, N], dt.bf16, T("ab")), attr=attr)
+        if w8:
+            w = r.integers(0, 256, (K, N)).astype(np.uint8)
+            sc = O.from_f32(O.F16, r.uniform(0.0005, 0.002, N).astype(np.float32))
+            zp = r.integers(100, 156, N).astype(np.uint8)
+            attr.set_fpmath_mode(A.fpmath_mode.f16, True)
+            attr.set_scales(A.DNNL_ARG_WEIGHTS, 2, [], dt.f16)
+            attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 2, [], dt.u8)
+            adt, wdt = dt.f16, dt.u8
+        else:
+            w, sc, zp = w4, sc4, zp4
+            attr.set_fpmath_mode(A.fpmath_mode.bf16, True)
+            attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
+            attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.u4)
+            adt, wdt = dt.bf16, dt.u4
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], adt, T("ab")), memory.desc([K, N], wdt, tag.any),
+                                     memory.desc([M, N], adt, T("ab")), attr=attr)
         prim = A.matmul(pd)
-        a = O.from_f32(O.BF16, r.standard_normal((M, K)).astype(np.float32))
+        a = O.from_f32(O.F16 if w8 else O.BF16, r.standard_normal((M, K)).astype(np.float32))
         m_src = memory(pd.src_desc(), eng).write(a)
         m_dst = memory(pd.dst_desc(), eng)
-        plain = memory(memory.desc([K, N], dt.u4, T("ab")), eng).write(w)
+        plain = memory(memory.desc([K, N], wdt, T("ab")), eng).write(w)
         first = memory(pd.weights_desc(), eng)
         A.reorder(plain, first).execute(strm, plain, first)
         strm.wait()
@@ -288,9 +301,9 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
         e1.record(hs)
         strm.wait()
         us = e1.elapsed_ms(e0) * 1e3 / (reps * sets)
-        nbytes = K * N // 2 + sc.nbytes + zp.nbytes + M * K * 2 + M * N * 2
+        nbytes = (K * N if w8 else K * N // 2) + sc.nbytes + zp.nbytes + M * K * 2 + M * N * 2
         floor = None
-        if M == 1:
+        if M == 1 and not w8:
             # the same bytes, the same weight sets and the same graph harness, read by a kernel that
             # does nothing else (qmm_stream_read): what the launch gaps and a cold 8.7 MB read cost alone
             from onednn_amd import _capi
@@ -315,7 +328,7 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
             f1.record(hs)
             strm.wait()
             floor = round(f1.elapsed_ms(f0) * 1e3 / (reps * sets), 3)
-        res["M%d" % M] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
+        res["M%d%s" % (M, "_u8_weights" if w8 else "")] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
                           "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
                           "impl": pd.impl_info_str(), "weight_sets": sets, "timing": "hip graph of %d launches x %d" % (sets, reps)}
         if floor is not None:

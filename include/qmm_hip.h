@@ -67,7 +67,12 @@ enum {
      * j = 4..7 as bytes holding 16 * value. Values are stored as signed
      * nibbles: s4 as is, u4 as (u - 8). K padded to 64 and N to 32 with
      * zeros. */
-    QMM_LAYOUT_MFMA_W4K64 = 3
+    QMM_LAYOUT_MFMA_W4K64 = 3,
+    /* 8-bit elements for the decode kernel, as two planes of nibbles: per
+     * batch, [N/16][K/128][2 planes][64 lanes][16 bytes]; plane 0 holds the
+     * high nibbles and plane 1 the low nibbles of the bytes, each in the
+     * order of QMM_LAYOUT_MFMA_W4. K padded to 128 and N to 16 with zeros. */
+    QMM_LAYOUT_MFMA_W8 = 4
 };
 
 typedef struct {

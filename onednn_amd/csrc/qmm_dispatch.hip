@@ -51,6 +51,12 @@ void launch_unpack_b8(const void *src, void *dst, int dt, int64_t batch,
 void launch_pack_w4(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
+void launch_pack_w8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
+void launch_unpack_w8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream);
 void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -571,7 +577,8 @@ w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
 int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
     if (nd != 2) return QMM_UNIMPLEMENTED;
-    if (!one_of(D.src.dt, {dt_bf16, dt_f16}) || !is_int4(D.wei.dt)
+    const bool w8 = is_int8(D.wei.dt);
+    if (!one_of(D.src.dt, {dt_bf16, dt_f16}) || !(is_int4(D.wei.dt) || w8)
             || !D.apply_to_int)
         return QMM_UNIMPLEMENTED;
     if (D.src.dt == dt_bf16 && !one_of(D.dst.dt, {dt_bf16, dt_f32}))
@@ -581,10 +588,31 @@ int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
     if (P.M > INT32_MAX || P.N > INT32_MAX || P.K > INT32_MAX)
         return QMM_UNIMPLEMENTED;
-    if (!one_of(D.wei_layout, {QMM_LAYOUT_PLAIN, QMM_LAYOUT_MFMA_W4}))
+    if (!one_of(D.wei_layout,
+                {QMM_LAYOUT_PLAIN, w8 ? QMM_LAYOUT_MFMA_W8 : QMM_LAYOUT_MFMA_W4}))
         return QMM_UNIMPLEMENTED;
     if (D.src.strides[1] != 1 || P.K % 8 != 0 || D.src.strides[0] % 8 != 0)
         return QMM_UNIMPLEMENTED;
+    if (w8) {
+        // 8-bit weights run in the kernel's all-unconditional-loads variant
+        // only: 16-bit scales, byte-sized zero points, K groups of 128 << s
+        // (or one group over all of K); the rest is the generic kernel's
+        const qmm_quant_t &s8 = D.scales[QMM_WEI], &z8 = D.zps[QMM_WEI];
+        if (!s8.set || !one_of(s8.dt, {dt_f16, dt_bf16})) return QMM_UNIMPLEMENTED;
+        if (z8.set && !one_of(z8.dt, {dt_s8, dt_u8, dt_s4, dt_u4}))
+            return QMM_UNIMPLEMENTED;
+        auto pow2_of_128 = [&](int64_t g) {
+            if (g >= round_up(P.K, 128)) return true;
+            if (g % 128) return false;
+            const int64_t q = g / 128;
+            return (q & (q - 1)) == 0;
+        };
+        if ((s8.mask & 1) && !pow2_of_128(P.q_wei_scale.g0)) return QMM_UNIMPLEMENTED;
+        if (z8.set && (z8.mask & 1) && !pow2_of_128(P.q_wei_zp.g0))
+            return QMM_UNIMPLEMENTED;
+        if (D.src.strides[0] >= ((int64_t)1 << 31) || P.M >= (1 << 23))
+            return QMM_UNIMPLEMENTED;
+    }
     if (D.zps[QMM_SRC].set || D.zps[QMM_DST].set) return QMM_UNIMPLEMENTED;
     if (D.scales[QMM_SRC].set && D.scales[QMM_SRC].mask != 0)
         return QMM_UNIMPLEMENTED;
@@ -699,6 +727,8 @@ size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N) 
         return (size_t)w4_geom(batch, K, N).total_bytes;
     if (layout == QMM_LAYOUT_MFMA_W4K64)
         return (size_t)w4k_geom(batch, K, N).total_bytes;
+    if (layout == QMM_LAYOUT_MFMA_W8)
+        return (size_t)w4_geom(batch, K, N).total_bytes * 2;
     return 0;
 }
 
@@ -714,6 +744,9 @@ int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
     d.wei_layout = QMM_LAYOUT_MFMA_W4;
     if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
         return QMM_LAYOUT_MFMA_W4;
+    d.wei_layout = QMM_LAYOUT_MFMA_W8;
+    if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
+        return QMM_LAYOUT_MFMA_W8;
     return QMM_LAYOUT_PLAIN;
 }
 
@@ -777,7 +810,9 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
     }
     if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     if (impl == impl_gemv_w4)
-        return qmm_packed_size(QMM_LAYOUT_MFMA_W4, desc->wei.dt, 1, K, N);
+        return qmm_packed_size(is_int8(desc->wei.dt) ? QMM_LAYOUT_MFMA_W8
+                                                     : QMM_LAYOUT_MFMA_W4,
+                desc->wei.dt, 1, K, N);
     return 0;
 }
 
@@ -1102,9 +1137,14 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
         const w4_geom_t geom = w4_geom(1, P.K, P.N);
         const uint8_t *packed = (const uint8_t *)args->wei;
+        g.w8 = is_int8(D.wei.dt);
         if (D.wei_layout == QMM_LAYOUT_PLAIN) {
-            launch_pack_w4(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N, 0,
-                    D.wei.strides[0], D.wei.strides[1], stream);
+            if (g.w8)
+                launch_pack_w8(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N,
+                        0, D.wei.strides[0], D.wei.strides[1], stream);
+            else
+                launch_pack_w4(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N,
+                        0, D.wei.strides[0], D.wei.strides[1], stream);
             packed = (const uint8_t *)args->scratch;
         }
         g.A = (const uint16_t *)args->src;
@@ -1125,7 +1165,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.K = (int32_t)P.K;
         g.kg128 = (int32_t)geom.kg128;
         g.nb16 = (int32_t)geom.nb16;
-        g.wei_signed = D.wei.dt == dt_s4;
+        g.wei_signed = D.wei.dt == dt_s4 || D.wei.dt == dt_s8;
         g.act_f16 = D.src.dt == dt_f16;
         g.m0 = 0;
         launch_gemv_w4(g, stream);
@@ -1201,6 +1241,8 @@ int qmm_reorder_supports(const qmm_reorder_desc_t *d) {
             return QMM_UNIMPLEMENTED;
         return QMM_OK;
     }
+    if (packed == QMM_LAYOUT_MFMA_W8)
+        return is_int8(pl.dt) ? QMM_OK : QMM_UNIMPLEMENTED;
     if (packed == QMM_LAYOUT_MFMA_W4 || packed == QMM_LAYOUT_MFMA_W4K64) {
         if (!is_int4(pl.dt)) return QMM_UNIMPLEMENTED;
         if (d->dst_layout == QMM_LAYOUT_PLAIN) {
@@ -1381,6 +1423,13 @@ int qmm_reorder_launch(const qmm_reorder_desc_t *d,
                         sn, pl.dt == dt_s8 || pl.dt == dt_u8, stream);
             else
                 launch_unpack_b8(args->src, args->dst, pl.dt, batch, K, N, sb,
+                        sk, sn, stream);
+        } else if (packed == QMM_LAYOUT_MFMA_W8) {
+            if (packing)
+                launch_pack_w8(args->src, args->dst, pl.dt, batch, K, N, sb, sk,
+                        sn, stream);
+            else
+                launch_unpack_w8(args->src, args->dst, pl.dt, batch, K, N, sb,
                         sk, sn, stream);
         } else if (packed == QMM_LAYOUT_MFMA_W4K64) {
             if (packing)

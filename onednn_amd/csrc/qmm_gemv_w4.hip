@@ -21,6 +21,8 @@
 //   * a block owns 16 columns and all of K; its waves take the k tiles round
 //     robin and issue their loads before touching the activations, which are
 //     staged once per block in LDS in MFMA operand order.
+#include <type_traits>
+
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
@@ -346,7 +348,12 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 //     4-bit, 3 zero points signed, 4 scales f16 (else bf16), 5 weights signed,
 //     6 zero points present, 7 plain store (see gemv_reduce_store);
 //     bits 8..: M
-template <bool F16, int ROWS, bool WSIGNED>
+// W8: 8-bit weights as two planes of nibbles (QMM_LAYOUT_MFMA_W8: a tile is
+// its high-nibble KiB followed by its low-nibble KiB). Both planes go through
+// the 4-bit arithmetic, w = 16 hi + lo:
+//     sum a * (w - z) = 16 P_hi + P_lo - (17 * offset + 16 * [8 if signed] + z) * S,
+// the sign of an s8 weight living in its high nibble.
+template <bool F16, int ROWS, bool WSIGNED, bool W8>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
@@ -387,7 +394,10 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     asm volatile("" : "+s"(NIB));
 
     v4f out = {0.f, 0.f, 0.f, 0.f};
-    const uint8_t *__restrict__ Bt = pB + ((int64_t)nb * kg128) * 1024 + lane * 16;
+    constexpr int NP = W8 ? 2 : 1; // planes per tile
+    constexpr int TILE_BYTES = 1024 * NP;
+    const uint8_t *__restrict__ Bt
+            = pB + ((int64_t)nb * kg128) * TILE_BYTES + lane * 16;
     const int64_t sN = scale_per_n ? N : 0, zN = zp_per_n ? N : 0;
 
     // Waves are independent until the final reduction: each one fetches its
@@ -421,12 +431,14 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         // u + 1 .. are still arriving. (Requesting all activations first and
         // the scales last, so that only the weights order the arithmetic, was
         // measured slower: the first weights request leaves later.)
-        uint4 wt[UNR], av[UNR][NA];
+        uint4 wt[UNR][NP], av[UNR][NA];
         uint32_t scp[UNR], zpp[UNR];
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             const int tc = tile_of(tb + uw + u * GEMV_WAVES);
-            wt[u] = ld_stream(Bt + (int64_t)tc * 1024);
+#pragma unroll
+            for (int pl = 0; pl < NP; pl++)
+                wt[u][pl] = ld_stream(Bt + (int64_t)tc * TILE_BYTES + pl * 1024);
 #pragma unroll
             for (int h = 0; h < NA; h++) {
                 // chunks past the row's end re-read its last one, rows past M
@@ -465,18 +477,30 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             v4f Pu = {0.f, 0.f, 0.f, 0.f}, Su = {0.f, 0.f, 0.f, 0.f};
+            v4f Pl = {0.f, 0.f, 0.f, 0.f}; // low-nibble plane (W8)
 #pragma unroll
             for (int s4 = 0; s4 < 4; s4++) {
-                const uint32_t d = (s4 == 0 ? wt[u].x
-                                : s4 == 1   ? wt[u].y
-                                : s4 == 2   ? wt[u].z
-                                            : wt[u].w)
+                const uint32_t d = (s4 == 0 ? wt[u][0].x
+                                : s4 == 1   ? wt[u][0].y
+                                : s4 == 2   ? wt[u][0].z
+                                            : wt[u][0].w)
                         ^ sflip;
                 v4u b;
                 b.x = (d & NIB) | MAGIC;
                 b.y = ((d >> 4) & NIB) | MAGIC;
                 b.z = ((d >> 8) & NIB) | MAGIC;
                 b.w = ((d >> 12) & NIB) | MAGIC;
+                v4u bl = b;
+                if constexpr (W8) {
+                    const uint32_t dl = s4 == 0 ? wt[u][NP - 1].x
+                            : s4 == 1           ? wt[u][NP - 1].y
+                            : s4 == 2           ? wt[u][NP - 1].z
+                                                : wt[u][NP - 1].w;
+                    bl.x = (dl & NIB) | MAGIC;
+                    bl.y = ((dl >> 4) & NIB) | MAGIC;
+                    bl.z = ((dl >> 8) & NIB) | MAGIC;
+                    bl.w = ((dl >> 12) & NIB) | MAGIC;
+                }
                 v4u a;
                 {
                     // operand row SPL j takes step s4's chunk from lane
@@ -495,6 +519,7 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                                 row_shl<3>(v.z), row_shl<3>(v.w)};
                 }
                 Pu = mfma16<F16>(a, b, Pu);
+                if constexpr (W8) Pl = mfma16<F16>(a, bl, Pl);
                 Su = mfma16<F16>(a, ones, Su);
             }
             const int t = tb + uw + u * GEMV_WAVES;
@@ -512,11 +537,14 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             const uint32_t zraw = (zpp[u] >> (4 * odd)) & ((1u << zbits) - 1u);
             const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
             const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
-            const float off = OFFSET + soff + zp;
+            const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp
+                                 : OFFSET + soff + zp;
             // a single row: only register 0 (row 0) is stored
 #pragma unroll
             for (int j = 0; j < 4; j += SPL)
-                out[j] = __builtin_fmaf(sc, Pu[j] - off * Su[j], out[j]);
+                out[j] = __builtin_fmaf(sc,
+                        (W8 ? 16.f * Pu[j] + Pl[j] : Pu[j]) - off * Su[j],
+                        out[j]);
         }
     }
     gemv_reduce_store<ROWS>(p, red, out, uw, lane, m_base, rows, n,
@@ -563,6 +591,7 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         return q == 1;
     };
     gemv_params_t q = p;
+    // 8-bit weights exist in the fast variant only (host-checked at creation)
     const bool fast = p.scales && fl % 128 == 0
             && (p.scale_dt == dt_f16 || p.scale_dt == dt_bf16)
             && (!p.zps || p.zp_dt != dt_s32) && shift_of(p.gs, q.gs_shift)
@@ -587,32 +616,38 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
                     (int)p.lda, shifts, flags_m, q);
         };
-        const int which = (p.act_f16 ? 8 : 0)
-                + (p.M == 1               ? 2
-                                : p.M <= 4 ? 4
-                                : p.M <= 8 ? 6
-                                           : 0)
-                + (p.wei_signed ? 1 : 0);
-        switch (which) {
-            case 0: go(gemv_w4_fast_kernel<false, 16, false>); break;
-            case 1: go(gemv_w4_fast_kernel<false, 16, true>); break;
-            case 2: go(gemv_w4_fast_kernel<false, 1, false>); break;
-            case 3: go(gemv_w4_fast_kernel<false, 1, true>); break;
-            case 4: go(gemv_w4_fast_kernel<false, 4, false>); break;
-            case 5: go(gemv_w4_fast_kernel<false, 4, true>); break;
-            case 6: go(gemv_w4_fast_kernel<false, 8, false>); break;
-            case 7: go(gemv_w4_fast_kernel<false, 8, true>); break;
-            case 8: go(gemv_w4_fast_kernel<true, 16, false>); break;
-            case 9: go(gemv_w4_fast_kernel<true, 16, true>); break;
-            case 10: go(gemv_w4_fast_kernel<true, 1, false>); break;
-            case 11: go(gemv_w4_fast_kernel<true, 1, true>); break;
-            case 12: go(gemv_w4_fast_kernel<true, 4, false>); break;
-            case 13: go(gemv_w4_fast_kernel<true, 4, true>); break;
-            case 14: go(gemv_w4_fast_kernel<true, 8, false>); break;
-            default: go(gemv_w4_fast_kernel<true, 8, true>); break;
-        }
+        // template arguments from the run-time choices, one level each
+        auto by_w8 = [&](auto f16, auto rows, auto sgn) {
+            constexpr bool F = decltype(f16)::value, S = decltype(sgn)::value;
+            constexpr int R = decltype(rows)::value;
+            if (p.w8)
+                go(gemv_w4_fast_kernel<F, R, S, true>);
+            else
+                go(gemv_w4_fast_kernel<F, R, S, false>);
+        };
+        auto by_sign = [&](auto f16, auto rows) {
+            if (p.wei_signed)
+                by_w8(f16, rows, std::true_type {});
+            else
+                by_w8(f16, rows, std::false_type {});
+        };
+        auto by_rows = [&](auto f16) {
+            if (p.M == 1)
+                by_sign(f16, std::integral_constant<int, 1> {});
+            else if (p.M <= 4)
+                by_sign(f16, std::integral_constant<int, 4> {});
+            else if (p.M <= 8)
+                by_sign(f16, std::integral_constant<int, 8> {});
+            else
+                by_sign(f16, std::integral_constant<int, 16> {});
+        };
+        if (p.act_f16)
+            by_rows(std::true_type {});
+        else
+            by_rows(std::false_type {});
         return;
     }
+    if (p.w8) return; // not reachable: creation admits fast-variant problems only
     auto launch = [&](auto kern) {
         ensure_dynamic_lds((const void *)kern, GEMV_LDS_BUDGET);
         hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, q,

@@ -130,6 +130,55 @@ pack_w4_kernel(const pack_params_t p, const w4_geom_t g) {
     }
 }
 
+// QMM_LAYOUT_MFMA_W8: one thread per packed dword (the high or the low
+// nibbles of 8 weights bytes); g is the 4-bit geometry of the same K and N, a
+// tile being its two 1 KiB planes
+__global__ void __launch_bounds__(256)
+pack_w8_kernel(const pack_params_t p, const w4_geom_t g) {
+    const int64_t per_b = g.batch_bytes / 2; // dwords: 2 planes of batch_bytes
+    const int64_t dwords = p.batch * per_b;
+    for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < dwords;
+            d += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t b = d / per_b, db = d % per_b;
+        const int s = (int)(db % 4);
+        const int lane = (int)((db / 4) % 64);
+        const int plane = (int)((db / 256) % 2);
+        const int64_t tile = db / 512;
+        const int64_t nbk = tile / g.kg128, kg = tile % g.kg128;
+        const int64_t n = nbk * 16 + (lane & 15);
+        const int64_t kbase = kg * 128 + 32 * s + 8 * (lane >> 4);
+        uint32_t w = 0;
+        if (n < p.N) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int64_t k = kbase + j;
+                if (k >= p.K) continue;
+                const uint32_t v = p.src[b * p.sb + k * p.sk + n * p.sn];
+                const uint32_t nib = plane ? (v & 15u) : (v >> 4);
+                const int pos = j / 2 + 4 * (j % 2);
+                w |= nib << (4 * pos);
+            }
+        }
+        ((uint32_t *)p.dst)[d] = w;
+    }
+}
+
+// one thread per destination byte
+__global__ void __launch_bounds__(256)
+unpack_w8_kernel(const pack_params_t p, const w4_geom_t g) {
+    const int64_t total = p.batch * p.K * p.N;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t n = i % p.N, k = (i / p.N) % p.K, b = i / (p.N * p.K);
+        // nibble index inside the 4-bit layout: 2048 nibbles per tile plane
+        const int64_t ni = w4_nibble_index(g, k, n);
+        const int64_t tile = ni / 2048, off = ni % 2048;
+        const uint8_t *t = p.src + b * g.batch_bytes * 2 + tile * 2048;
+        const int hi = nibble_at(t, off), lo = nibble_at(t + 1024, off);
+        p.dst[b * p.sb + k * p.sk + n * p.sn] = (uint8_t)((hi << 4) | lo);
+    }
+}
+
 // one thread per destination byte: the two nibbles are neighbours along the
 // plain tensor's stride-1 dim (n for ab, k for ba)
 __global__ void __launch_bounds__(256)
@@ -348,6 +397,26 @@ void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
     pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
             sn, dt, 0};
     hipLaunchKernelGGL(unpack_w4_kernel, dim3(grid_for(batch * K * N / 2)),
+            dim3(256), 0, stream, p, g);
+}
+
+void launch_pack_w8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4_geom_t g = w4_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(pack_w8_kernel, dim3(grid_for(batch * g.batch_bytes / 2)),
+            dim3(256), 0, stream, p, g);
+}
+
+void launch_unpack_w8(const void *src, void *dst, int dt, int64_t batch,
+        int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
+        hipStream_t stream) {
+    const w4_geom_t g = w4_geom(batch, K, N);
+    pack_params_t p {(const uint8_t *)src, (uint8_t *)dst, batch, K, N, sb, sk,
+            sn, dt, 0};
+    hipLaunchKernelGGL(unpack_w8_kernel, dim3(grid_for(batch * K * N)),
             dim3(256), 0, stream, p, g);
 }
 

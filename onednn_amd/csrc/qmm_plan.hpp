@@ -182,7 +182,7 @@ struct gemv_params_t {
     int32_t m0; // first row handled by this launch
     // fast variant: K groups are 128 << shift wide (host-checked); -1: single
     int32_t gs_shift, gz_shift;
-    int32_t pad_;
+    int32_t w8; // 8-bit weights, QMM_LAYOUT_MFMA_W8 (fast variant only)
     epilogue_t ep;
 };
 

@@ -75,19 +75,30 @@ def int8_linear(M, K, N, seed, src_dt=dt.u8, dst_dt=dt.f32, src_zp=128, src_scal
 
 
 def decode_w4(M, K, N, seed, G=128, act_dt=dt.bf16, wei_dt=dt.u4, zp_dt=dt.u4, scale_dt=dt.f16,
-              with_zp=True, zp_group=None, post_ops=None):
+              with_zp=True, zp_group=None, post_ops=None, per_column=False, wei_layout=None, dst_dt=None):
+    """per_column: one scale / zero point per column over all of K (the 8-bit weights-only entries of
+    tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu: --attr-scales=wei:per_oc:f16 --attr-zero-points=wei:per_oc:u8)."""
     r = rnd(seed)
     a = r.standard_normal((M, K)).astype(np.float32)
-    lo, hi = (0, 16) if wei_dt == dt.u4 else (-8, 8)
+    lo, hi = {dt.u4: (0, 16), dt.s4: (-8, 8), dt.u8: (0, 256), dt.s8: (-128, 128)}[wei_dt]
     w = r.integers(lo, hi, (K, N))
     src = TensorSpec(act_dt, [M, K], None, a)
-    wei = TensorSpec(wei_dt, [K, N], None, w)
-    dst = TensorSpec(act_dt, [M, N])
-    scales = {"wei": (3, scale_dt, (G, 1), r.uniform(0.005, 0.02, (K // G, N)))}
+    wei = TensorSpec(wei_dt, [K, N], wei_layout, w)
+    dst = TensorSpec(dst_dt or act_dt, [M, N])
+    wide = wei_dt in (dt.u8, dt.s8)
+    zlo, zhi = (6, 10) if zp_dt not in (dt.s4, dt.s8) else (-2, 3)
+    if wide and zp_dt == dt.u8:
+        zlo, zhi = 100, 156
     zps = {}
+    if per_column:
+        scales = {"wei": (2, scale_dt, None, r.uniform(0.0005 if wide else 0.005, 0.002 if wide else 0.02, N))}
+        if with_zp:
+            zps["wei"] = (2, zp_dt, None, r.integers(zlo, zhi, N))
+        return Problem(src, wei, dst, scales=scales, zps=zps, post_ops=post_ops, apply_to_int=True,
+                       fpmath=dnnl.fpmath_mode.bf16 if act_dt == dt.bf16 else dnnl.fpmath_mode.f16)
+    scales = {"wei": (3, scale_dt, (G, 1), r.uniform(0.0005 if wide else 0.005, 0.002 if wide else 0.02, (K // G, N)))}
     if with_zp:
         zg = zp_group or G
-        zlo, zhi = (6, 10) if zp_dt != dt.s4 else (-2, 3)
         zps["wei"] = (3, zp_dt, (zg, 1), r.integers(zlo, zhi, (K // zg, N)))
     return Problem(src, wei, dst, scales=scales, zps=zps, post_ops=post_ops, apply_to_int=True,
                    fpmath=dnnl.fpmath_mode.bf16 if act_dt == dt.bf16 else dnnl.fpmath_mode.f16)
@@ -111,11 +122,13 @@ def decode_term_scale(p):
     w = p.wei.logical().astype(np.float64)
     K, N = w.shape
     mask, code, groups, vals = p.scales["wei"]
-    sc = O.to_f32(code, Problem._quant_raw(code, vals)).astype(np.float64).reshape(K // groups[0], N)
+    g = groups[0] if groups else K  # no groups: one entry per column over all of K
+    sc = O.to_f32(code, Problem._quant_raw(code, vals)).astype(np.float64).reshape(K // g, N)
     if "wei" in p.zps:
         zm, zc, zg, zv = p.zps["wei"]
-        w = w - np.repeat(np.asarray(zv, np.float64).reshape(K // zg[0], N), zg[0], 0)
-    return a @ (np.abs(w) * np.repeat(sc, groups[0], 0))
+        zgk = zg[0] if zg else K
+        w = w - np.repeat(np.asarray(zv, np.float64).reshape(K // zgk, N), zgk, 0)
+    return a @ (np.abs(w) * np.repeat(sc, g, 0))
 
 
 def term_scale(p):
@@ -680,6 +693,62 @@ def test_decode_w4_variants(ctx, kw):
     code = kw.get("act_dt", dt.bf16)
     g, w = O.to_f32(code, got), O.to_f32(code, want)
     assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="decode variant")
+
+
+W8_CASES = {
+    "f16_u8_per_column_m1": dict(M=1, K=4096, N=1024, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8, per_column=True, wei_layout="ba"),
+    "f16_u8_per_column_m32_f32_dst": dict(M=32, K=1024, N=520, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8, per_column=True,
+                                          wei_layout="ba", dst_dt=dt.f32),
+    "f16_u8_per_column_m5": dict(M=5, K=512, N=272, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8, per_column=True),
+    "bf16_s8_groups_128_zp_s8": dict(M=3, K=512, N=160, act_dt=dt.bf16, wei_dt=dt.s8, zp_dt=dt.s8, scale_dt=dt.bf16),
+    "f16_s8_no_zp_groups_256": dict(M=8, K=1024, N=96, act_dt=dt.f16, wei_dt=dt.s8, with_zp=False, G=256),
+    "f16_u8_k_tail_m17": dict(M=17, K=200, N=48, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8, per_column=True),
+}
+
+
+@pytest.mark.parametrize("name", sorted(W8_CASES))
+@pytest.mark.parametrize("weights_any", [True, False])
+def test_decode_8bit_weights(ctx, name, weights_any):
+    """8-bit weights-only quantization on the decode kernel: the weights as two planes of nibbles."""
+    eng, strm = ctx
+    say("decode_w4 8-bit weights %s any=%s" % (name, weights_any))
+    kw = W8_CASES[name]
+    p = decode_w4(seed=90 + len(name), **kw)
+    got, pd = p.run_gpu(eng, strm, weights_any=weights_any, return_pd=True)
+    assert pd.impl_info_str() == DECODE
+    want = p.run_oracle()
+    code = kw.get("dst_dt") or kw["act_dt"]
+    g, w = O.to_f32(code, got).reshape(kw["M"], kw["N"]), O.to_f32(code, want).reshape(kw["M"], kw["N"])
+    assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="decode 8-bit")
+    if code == dt.f32:
+        # the offset form (16 P_hi + P_lo - offset * S) rounds relative to the summed magnitudes, not to the result
+        err = np.abs(g.astype(np.float64) - w) / decode_term_scale(p)
+        print("[decode 8-bit f32] max error %.2e of the summed magnitudes" % err.max())
+        assert err.max() <= 2e-5
+    elif code == dt.bf16:
+        assert_bf16_within_1ulp(got, want, "decode 8-bit bf16", abs_slack=2e-5 * decode_term_scale(p))
+
+
+def test_prepack_8bit_decode_weights_round_trip(ctx):
+    eng, strm = ctx
+    say("W8 prepack round trip")
+    r = rnd(92)
+    for code, dims, layout in ((dt.u8, [200, 48], "ab"), (dt.s8, [136, 34], "ba")):
+        vals = r.integers(0, 256, dims) if code == dt.u8 else r.integers(-128, 128, dims)
+        t = TensorSpec(code, dims, layout, vals)
+        attr = dnnl.primitive_attr()
+        attr.set_fpmath_mode(dnnl.fpmath_mode.f16, True)
+        attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 2, [], dt.f16)
+        pd = dnnl.matmul.primitive_desc(eng, memory.desc([1, dims[0]], dt.f16, T("ab")), memory.desc(dims, code, tag.any),
+                                        memory.desc([1, dims[1]], dt.f16, T("ab")), attr=attr)
+        assert pd.impl_info_str() == DECODE
+        plain = memory(t.md(), eng).write(t.raw)
+        packed = memory(pd.weights_desc(), eng)
+        back = memory(t.md(), eng).write(np.zeros_like(t.raw))
+        dnnl.reorder(plain, packed).execute(strm, plain, packed)
+        dnnl.reorder(packed, back).execute(strm, packed, back)
+        strm.wait()
+        assert_bit_exact(back.read(t.raw.dtype), t.raw, "W8 round trip %s" % layout)
 
 
 # ---------------------------------------------------------------------------
