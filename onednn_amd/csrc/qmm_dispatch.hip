@@ -472,8 +472,11 @@ int supports_gemm_w4a8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
         return QMM_UNIMPLEMENTED;
     // whole 64-k tiles per group, every buffer's K extent a whole number of
     // groups
+    // (or groups of 32 k, two per tile: the tiled kernel at every M)
     const int64_t gk = P.group_k;
-    if (P.K % 64 != 0 || gk % 64 != 0 || gk > 32768) return QMM_UNIMPLEMENTED;
+    if (P.K % 64 != 0 || (gk % 64 != 0 && gk != 32) || gk > 32768)
+        return QMM_UNIMPLEMENTED;
+    if (gk == 32 && w4a8_src_zp_mode(D)) return QMM_UNIMPLEMENTED;
     const qmm_quant_t &ss = D.scales[QMM_SRC], &ws = D.scales[QMM_WEI];
     const qmm_quant_t &wz = D.zps[QMM_WEI], &sz = D.zps[QMM_SRC];
     if (k_extent(ss, 1, 2, P.K) % gk || k_extent(ws, 0, 1, P.K) % gk
@@ -549,7 +552,7 @@ w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     w4a8_small_plan_t s;
     std::memset(&s, 0, sizeof(s));
     s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0
-            && !w4a8_src_zp_mode(P.desc);
+            && !w4a8_src_zp_mode(P.desc) && P.group_k >= 64;
     if (!s.use) return s;
     const int64_t ng = P.ngroups_k, tpg = P.group_k / 64;
     const int64_t nblk = (P.N + 127) / 128;

@@ -116,10 +116,14 @@ QMM_D int zp_value(int dt, uint32_t raw, int64_t idx) {
 // (the group's source row sums take part); 2 also source zero points or a u8
 // source (the group's weights column sums take part, and the source bytes
 // are shifted to s8 by flipping their top bit).
-template <int BM, int BN, int WGM, int WGN, int STAGES, int ZPM>
+// HALF: groups of 32 k, two per 64-k tile (each MFMA is a group of its own and
+// the group end runs after it); the per-group arrays then travel with the
+// tile, two slices each.
+template <int BM, int BN, int WGM, int WGN, int STAGES, int ZPM, bool HALF = false>
 __global__ void __launch_bounds__(WGM *WGN * 64, 2)
 gemm_w4a8_kernel(const w4a8_params_t p) {
     constexpr bool HAS_ZP = ZPM >= 1, SRC_ZP = ZPM == 2;
+    static_assert(!(HALF && SRC_ZP), "");
     constexpr int NW = WGM * WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int FM = WM / 32, FN = WN / 32;
@@ -127,7 +131,7 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     // per-group arrays: ss, sw [, rs, zw [, zs, c2]]
     constexpr int NX = SRC_ZP ? 6 : HAS_ZP ? 4 : 2;
-    constexpr int XSLOT = NX * X_BYTES;
+    constexpr int XSLOT = (HALF ? 2 : 1) * NX * X_BYTES;
     constexpr int X_OFF = STAGES * STAGE_BYTES;
     // wave-wide 1 KiB loads per tile / per group, spread over the waves; a
     // wave whose share runs past the end repeats earlier ones (same bytes to
@@ -220,7 +224,15 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     // issue state: tile number, its position in its group, the group
     int is_kt = 0, is_t = 0, is_g = 0;
     auto issue = [&]() {
-        if (is_t == 0) {
+        if constexpr (HALF) {
+            const uint32_t xs = lds_base + X_OFF + (is_kt % STAGES) * XSLOT;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int j = 0; j < PER_X; j++)
+                    load_to_lds16(x_ptr[j] + (2 * is_kt + h) * x_step[j],
+                            xs + h * NX * X_BYTES + x_lds[j]);
+        } else if (is_t == 0) {
             const uint32_t xs = lds_base + X_OFF + (is_g % STAGES) * XSLOT;
 #pragma unroll
             for (int j = 0; j < PER_X; j++)
@@ -253,76 +265,11 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
     for (int s = 0; s < STAGES - 1; s++)
         if (s < KT) issue();
 
-    // one 64-k tile: FIRST starts the group's s32 accumulators from zero
-    auto tile_mma = [&](int kt, auto first_tag) {
-        constexpr bool FIRST = decltype(first_tag)::value;
-        // the tile has landed once only younger tiles' loads are in flight (a
-        // younger tile may carry group loads too: then this waits a little
-        // longer than needed, never shorter)
-        if (kt + STAGES - 2 < KT)
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * PER_T));
-        else
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-        __syncthreads();
-        if (kt + STAGES - 1 < KT) issue();
-
-        const uint8_t *As = lds + (kt % STAGES) * STAGE_BYTES;
-        const uint8_t *Bs = As + A_BYTES;
-        uint4 braw[FN];
-#pragma unroll
-        for (int j = 0; j < FN; j++)
-            braw[j] = *(const uint4 *)(Bs + (((wn0 >> 5) + j) * 64 + lane) * 16);
-#pragma unroll
-        for (int ki = 0; ki < 2; ki++) {
-            v4i a[FM], b[FN];
-#pragma unroll
-            for (int i = 0; i < FM; i++) {
-                const int row = wm0 + i * 32 + (lane & 31);
-                const int q = ki * 2 + (lane >> 5);
-                const uint4 v = *(const uint4 *)(As + row * BK
-                        + a_swz(row, q) * 16);
-                if constexpr (SRC_ZP) // u8 source: s - 128 as s8
-                    a[i] = v4i {(int)(v.x ^ p.a_flip), (int)(v.y ^ p.a_flip),
-                            (int)(v.z ^ p.a_flip), (int)(v.w ^ p.a_flip)};
-                else
-                    a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-            }
-#pragma unroll
-            for (int j = 0; j < FN; j++) {
-                const uint32_t w0 = ki ? braw[j].z : braw[j].x;
-                const uint32_t w1 = ki ? braw[j].w : braw[j].y;
-                b[j] = v4i {(int)((w0 << 4) & 0xF0F0F0F0u),
-                        (int)(w0 & 0xF0F0F0F0u), (int)((w1 << 4) & 0xF0F0F0F0u),
-                        (int)(w1 & 0xF0F0F0F0u)};
-            }
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-#pragma unroll
-                for (int j = 0; j < FN; j++) {
-                    if (FIRST && ki == 0) {
-                        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
-                                0, 0, 0};
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                                a[i], b[j], zero, 0, 0, 0);
-                    } else {
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                                a[i], b[j], acc[i][j], 0, 0, 0);
-                    }
-                }
-        }
-    };
-
-    int kt = 0;
-    for (int g = 0; g < p.ng; g++) {
-        tile_mma(kt++, std::true_type {});
-        for (int t = 1; t < p.tpg; t++)
-            tile_mma(kt++, std::false_type {});
-
-        // ---- group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+    // ---- group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+    auto group_end = [&](const uint8_t *xs) {
         // (zw = -16 (z_w - offset); c2 = -16 (column sum - group * (z_w - offset)))
         // Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
         // column l%32 of its fragment.
-        const uint8_t *xs = lds + X_OFF + (g % STAGES) * XSLOT;
         const float *ssl = (const float *)xs;
         const float *swl = (const float *)(xs + X_BYTES);
         const int32_t *rsl = (const int32_t *)(xs + 2 * X_BYTES);
@@ -375,6 +322,81 @@ gemm_w4a8_kernel(const w4a8_params_t p) {
                             (float)t * ss[r], sw[j], res[i][j][r]);
                 }
         });
+    };
+
+    // one 64-k tile: FIRST starts the group's s32 accumulators from zero
+    auto tile_mma = [&](int kt, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
+        // the tile has landed once only younger tiles' loads are in flight (a
+        // younger tile may carry group loads too: then this waits a little
+        // longer than needed, never shorter)
+        if (kt + STAGES - 2 < KT)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * PER_T));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        __syncthreads();
+        if (kt + STAGES - 1 < KT) issue();
+
+        const uint8_t *As = lds + (kt % STAGES) * STAGE_BYTES;
+        const uint8_t *Bs = As + A_BYTES;
+        uint4 braw[FN];
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+            braw[j] = *(const uint4 *)(Bs + (((wn0 >> 5) + j) * 64 + lane) * 16);
+#pragma unroll
+        for (int ki = 0; ki < 2; ki++) {
+            v4i a[FM], b[FN];
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                const int row = wm0 + i * 32 + (lane & 31);
+                const int q = ki * 2 + (lane >> 5);
+                const uint4 v = *(const uint4 *)(As + row * BK
+                        + a_swz(row, q) * 16);
+                if constexpr (SRC_ZP) // u8 source: s - 128 as s8
+                    a[i] = v4i {(int)(v.x ^ p.a_flip), (int)(v.y ^ p.a_flip),
+                            (int)(v.z ^ p.a_flip), (int)(v.w ^ p.a_flip)};
+                else
+                    a[i] = v4i {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+            }
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                const uint32_t w0 = ki ? braw[j].z : braw[j].x;
+                const uint32_t w1 = ki ? braw[j].w : braw[j].y;
+                b[j] = v4i {(int)((w0 << 4) & 0xF0F0F0F0u),
+                        (int)(w0 & 0xF0F0F0F0u), (int)((w1 << 4) & 0xF0F0F0F0u),
+                        (int)(w1 & 0xF0F0F0F0u)};
+            }
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    if (HALF || (FIRST && ki == 0)) {
+                        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                0, 0, 0};
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                a[i], b[j], zero, 0, 0, 0);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                a[i], b[j], acc[i][j], 0, 0, 0);
+                    }
+                }
+            if constexpr (HALF)
+                group_end(lds + X_OFF + (kt % STAGES) * XSLOT
+                        + ki * NX * X_BYTES);
+        }
+    };
+
+    int kt = 0;
+    if constexpr (HALF) {
+        for (; kt < KT; kt++)
+            tile_mma(kt, std::true_type {});
+    } else
+    for (int g = 0; g < p.ng; g++) {
+        tile_mma(kt++, std::true_type {});
+        for (int t = 1; t < p.tpg; t++)
+            tile_mma(kt++, std::false_type {});
+
+        group_end(lds + X_OFF + (g % STAGES) * XSLOT);
     }
     __syncthreads(); // LDS is reused by the epilogue
 
@@ -1083,33 +1105,35 @@ static void launch_small_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         launch_small_cfg<FM, SC, true, 2>(p, stream);
 }
 
-template <int BM, int BN, int WGM, int WGN, int ZPM>
+template <int BM, int BN, int WGM, int WGN, int ZPM, bool HALF = false>
 static void launch_cfg(const w4a8_params_t &p, hipStream_t stream) {
     // a tile is only 8 MFMAs per wave: five stages (four tiles in flight) are
     // what it takes to cover the L2 / HBM latency; two workgroups still fit
-    // (four stages with the six per-group arrays of ZPM = 2)
-    constexpr int STAGES = ZPM == 2 ? 4 : 5;
+    // (four stages with the six per-group arrays of ZPM = 2, three where every
+    // tile carries two slices of each array)
+    constexpr int STAGES = HALF ? 3 : ZPM == 2 ? 4 : 5;
     w4a8_params_t q = p;
     q.tiles_m = (p.M + BM - 1) / BM;
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ntiles >= 64 ? ((ntiles + 7) / 8) * 8 : ntiles;
     constexpr size_t lds_main = (size_t)STAGES
-            * (BM * BK + BN * BK / 2 + (ZPM == 2 ? 6 : ZPM == 1 ? 4 : 2) * X_BYTES);
+            * (BM * BK + BN * BK / 2
+                    + (HALF ? 2 : 1) * (ZPM == 2 ? 6 : ZPM == 1 ? 4 : 2) * X_BYTES);
     constexpr size_t lds_ep
             = (size_t)WGM * WGN * 32 * (BN / WGN) * sizeof(float);
     constexpr size_t lds = lds_main > lds_ep ? lds_main : lds_ep;
-    auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, ZPM>;
+    auto kern = gemm_w4a8_kernel<BM, BN, WGM, WGN, STAGES, ZPM, HALF>;
     ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3(grid_x), dim3(WGM * WGN * 64), lds, stream, q);
 }
 
-template <int ZPM>
+template <int ZPM, bool HALF = false>
 static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
     switch (variant) {
-        case 1: launch_cfg<128, 128, 2, 2, ZPM>(p, stream); break;
-        case 2: launch_cfg<64, 128, 2, 2, ZPM>(p, stream); break;
-        default: launch_cfg<32, 64, 1, 2, ZPM>(p, stream); break;
+        case 1: launch_cfg<128, 128, 2, 2, ZPM, HALF>(p, stream); break;
+        case 2: launch_cfg<64, 128, 2, 2, ZPM, HALF>(p, stream); break;
+        default: launch_cfg<32, 64, 1, 2, ZPM, HALF>(p, stream); break;
     }
 }
 
@@ -1118,6 +1142,7 @@ static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
 // The kernel families build in translation units of their own (QMM_W4A8_PART:
 // 1, 2 the tiled GEMM without / with zero points, 3 the split-K kernel and its
 // reduction, 4 the single-token kernel, 5 the tiled GEMM with source zero
+// points, 6 and 7 the tiled GEMM with groups of 32 k without / with zero
 // points); the unit without the macro holds the pre-pass and the dispatch.
 #if defined(QMM_W4A8_PART)
 #if QMM_W4A8_PART == 1
@@ -1134,6 +1159,16 @@ void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
 void launch_gemm_w4a8_szp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
     w4a8::launch_zp<2>(p, variant, stream);
+}
+#elif QMM_W4A8_PART == 6
+void launch_gemm_w4a8_half_nozp(const w4a8_params_t &p, int variant,
+        hipStream_t stream) {
+    w4a8::launch_zp<0, true>(p, variant, stream);
+}
+#elif QMM_W4A8_PART == 7
+void launch_gemm_w4a8_half_zp(const w4a8_params_t &p, int variant,
+        hipStream_t stream) {
+    w4a8::launch_zp<1, true>(p, variant, stream);
 }
 #elif QMM_W4A8_PART == 3
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
@@ -1178,6 +1213,10 @@ void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
 void launch_gemm_w4a8_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream);
 void launch_gemm_w4a8_szp(const w4a8_params_t &p, int variant,
+        hipStream_t stream);
+void launch_gemm_w4a8_half_nozp(const w4a8_params_t &p, int variant,
+        hipStream_t stream);
+void launch_gemm_w4a8_half_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream);
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, hipStream_t stream);
@@ -1237,7 +1276,12 @@ void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream) {
         variant = big >= 256 ? 1 : ((mid >= 128 && p.M > 32) ? 2 : 3);
         if (variant == 3 && p.M > 64) variant = 2;
     }
-    if (p.zsT)
+    if (p.tpg == 0) { // groups of 32 k
+        if (p.zwT)
+            launch_gemm_w4a8_half_zp(p, variant, stream);
+        else
+            launch_gemm_w4a8_half_nozp(p, variant, stream);
+    } else if (p.zsT)
         launch_gemm_w4a8_szp(p, variant, stream);
     else if (p.zwT)
         launch_gemm_w4a8_zp(p, variant, stream);

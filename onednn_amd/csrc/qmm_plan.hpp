@@ -204,7 +204,7 @@ struct w4a8_params_t {
     int32_t M, N, K;
     int32_t Mpad, Npad;
     int32_t kt64, nb32;
-    int32_t tpg; // 64-k tiles per group
+    int32_t tpg; // 64-k tiles per group; 0: groups of 32 k, two per tile
     int32_t ng;
     int32_t tiles_m, tiles_n;
     uint32_t a_flip; // 0x80808080 for a u8 source (read as s8 = u8 - 128)

@@ -112,6 +112,13 @@ EXACT_CASES = {
     "s8_src_zp_per_group_wider_than_scales": dict(M=17, K=512, N=48, gs=128, gw=128, src_zp=("k", 256),
                                                   src_zp_dt=dt.s8, gz=128, zp_dt=dt.u8, wei_dt=dt.u4),
     "u8_src_zp_m1": dict(M=1, K=512, N=160, src_dt=dt.u8, src_zp=("mk", 128)),
+    # source scales per 32 k (--attr-scales=src0:per_ocic:f16:1x32+wei:per_ocic:f16:128x1 in the reference's list):
+    # groups of half a tile, the tiled kernel at every M
+    "src_g32_wei_g128_u4_zp": dict(M=70, K=256, N=100, gs=32, gw=128, wei_dt=dt.u4, gz=128),
+    "src_g32_wei_g64_s4": dict(M=33, K=512, N=64, gs=32, gw=64),
+    "src_g32_wei_g32_zp_s4_g32": dict(M=130, K=128, N=130, gs=32, gw=32, gz=32, zp_dt=dt.s4),
+    "src_g32_m1_k4096": dict(M=1, K=4096, N=96, gs=32, gw=128, wei_dt=dt.u4, gz=128),
+    "src_g32_m300_k1536": dict(M=300, K=1536, N=264, gs=32, gw=128, wei_dt=dt.u4, gz=128),
     "u8_src_zp_m300_k2048": dict(M=300, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
                                  zp_dt=dt.u4),
 }
