@@ -48,7 +48,7 @@ for v in GEMM_VARIANTS:
 # (even and odd numbers of k-steps), fp8 on 16 x 16 MFMAs
 for v in (1, 2, 3, 4, 5, 6):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
-for v in (1, 2, 3, 4, 5, 6, 7):
+for v in (1, 2, 3, 4, 5, 6, 7, 8, 9):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))
 # longest first, so that the pool finishes together
 UNITS.sort(key=lambda u: 0 if "w4a8" in u[0] else (1 if u[1] else 2))

@@ -36,6 +36,7 @@ void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
 bool gemm_w4a8_small_takes(const w4a8_prep_t &q);
 void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
         hipStream_t stream);
+int gemm_w4a8_tiny_max_groups(bool half);
 void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -1076,7 +1077,11 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             q.c2T = (int32_t *)(arrays + sc.c2_off);
         }
         const w4a8_small_plan_t sm = w4a8_small_plan(P, w4a8_variant);
-        if (sm.use && gemm_w4a8_small_takes(q)) {
+        // the single-token kernel also takes groups of 32 k and source zero
+        // points / u8 sources (which the split-K kernel does not)
+        const bool tiny_only = !sm.use && w4a8_variant == 0 && P.M <= 4
+                && (sc.src_zp || q.gk == 32);
+        if ((sm.use || tiny_only) && gemm_w4a8_small_takes(q)) {
             w4a8_small_t h;
             std::memset(&h, 0, sizeof(h));
             h.q = q;
@@ -1086,14 +1091,22 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             h.nb32 = (int32_t)geom.nb32;
             if (P.M <= 4) {
                 // single-token decode: the waves of a workgroup cut K between
-                // them, at most 16 groups and preferably 16 tiles per wave
+                // them, at most 16 groups (32 of 32 k) and preferably 16 tiles
+                // per wave
+                const bool half = q.gk == 32;
+                const int64_t maxg = gemm_w4a8_tiny_max_groups(half);
+                auto per_wave = [&](int n) {
+                    int64_t g = (q.ng + n - 1) / n;
+                    return half ? (g + 1) / 2 * 2 : g; // whole tiles per wave
+                };
+                auto tiles = [&](int64_t g) { return half ? g / 2 : g * h.tpg; };
                 int nwv = 4;
-                int64_t gpw = (q.ng + 3) / 4;
-                if (gpw * h.tpg > 16 || gpw > 16) {
+                int64_t gpw = per_wave(4);
+                if (tiles(gpw) > 16 || gpw > maxg) {
                     nwv = 8;
-                    gpw = (q.ng + 7) / 8;
+                    gpw = per_wave(8);
                 }
-                if (gpw <= 16) {
+                if (gpw <= maxg) {
                     h.gps = (int32_t)gpw;
                     h.ep = g.ep;
                     launch_gemm_w4a8_tiny(h, sc.has_zp, nwv, stream);
@@ -1102,15 +1115,17 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
                     return QMM_OK;
                 }
             }
-            h.gps = sm.gps;
-            h.splits = sm.splits;
-            h.ldp = sm.ldp;
-            h.part = (float *)arrays;
-            h.ep = g.ep;
-            launch_gemm_w4a8_small(h, sc.has_zp, stream);
-            const hipError_t e = hipGetLastError();
-            if (e != hipSuccess) return hip_fail(e, "kernel launch");
-            return QMM_OK;
+            if (!tiny_only) { // else (too many groups per wave): the tiled kernel
+                h.gps = sm.gps;
+                h.splits = sm.splits;
+                h.ldp = sm.ldp;
+                h.part = (float *)arrays;
+                h.ep = g.ep;
+                launch_gemm_w4a8_small(h, sc.has_zp, stream);
+                const hipError_t e = hipGetLastError();
+                if (e != hipSuccess) return hip_fail(e, "kernel launch");
+                return QMM_OK;
+            }
         }
         launch_w4a8_prep(q, stream);
         g.A = q.A;

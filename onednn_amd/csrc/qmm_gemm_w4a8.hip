@@ -817,28 +817,42 @@ w4a8_small_kernel(const w4a8_small_t p) {
 // summed through LDS in wave order (= K order) by wave 0, which also runs the
 // epilogue. Accumulator registers 0..3 of lanes 0..31 are rows 0..3: the only
 // ones looked at.
+// MODE 1: groups of 32 k (p.tpg == 0): every MFMA is a group of its own, twice
+// the groups per wave. MODE 2: source zero points / u8 source (with HAS_ZP):
+// the source bytes are flipped to s8, the column sums of the stored nibbles
+// come from dot products of the weights operand with ones, and the group end
+// adds z_s' * -(16 sum w' + group * zw) (see gemm_w4a8_kernel).
 constexpr int TN_ROWS = 4;
 constexpr int TN_AROW = SM_CH * BK + 16; // staged row, padded against conflicts
-constexpr int TN_MAXG = 16; // groups per wave
-constexpr int TN_WAVE_BYTES = TN_ROWS * TN_AROW + TN_MAXG * 4 * 4
-        + TN_MAXG * 32 * 4 + TN_MAXG * 32 * 4;
+constexpr int tn_maxg(int mode) { // groups per wave
+    return mode == 1 ? 32 : 16;
+}
+constexpr int tn_wave_bytes(int mode) {
+    // rows, source scales [, source zero points], weights scales, zero points
+    return TN_ROWS * TN_AROW + tn_maxg(mode) * 4 * 4 * (mode == 2 ? 2 : 1)
+            + tn_maxg(mode) * 32 * 4 + tn_maxg(mode) * 32 * 4;
+}
 
-template <int NWV, int SC, bool HAS_ZP, int ZPK>
+template <int NWV, int SC, bool HAS_ZP, int ZPK, int MODE = 0>
 __global__ void __launch_bounds__(NWV * 64)
 w4a8_tiny_kernel(const w4a8_small_t p) {
-    constexpr int SW_PER = TN_MAXG * 32 / 64;
+    constexpr bool HALF = MODE == 1, SZP = MODE == 2;
+    static_assert(!SZP || HAS_ZP, "");
+    constexpr int TN_MAXG = tn_maxg(MODE), TN_WAVE_BYTES = tn_wave_bytes(MODE);
+    constexpr int SW_PER = TN_MAXG * 32 / 64, SS_PER = TN_MAXG * 4 / 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const w4a8_prep_t &q = p.q;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n0 = blockIdx.x * 32;
-    const int g_begin = wave * p.gps;
+    const int g_begin = wave * p.gps; // p.gps is even with groups of 32 k
     const int g_cnt = max(0, min(p.gps, q.ng - g_begin));
-    const int T0 = g_begin * p.tpg;
-    const int KT = g_cnt * p.tpg; // tiles of this wave
+    const int T0 = HALF ? g_begin / 2 : g_begin * p.tpg;
+    const int KT = HALF ? g_cnt / 2 : g_cnt * p.tpg; // tiles of this wave
     uint8_t *wA = lds + wave * TN_WAVE_BYTES;
     float *wss = (float *)(wA + TN_ROWS * TN_AROW);
-    float *wsw = wss + TN_MAXG * 4;
+    int32_t *wzs = (int32_t *)(wss + TN_MAXG * 4); // SZP only
+    float *wsw = wss + TN_MAXG * 4 * (SZP ? 2 : 1);
     int32_t *wzw = (int32_t *)(wsw + TN_MAXG * 32);
     float *red = (float *)(lds + NWV * TN_WAVE_BYTES); // [NWV][4][32]
 
@@ -873,17 +887,29 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
 
         load_rows(0, min(SM_CH, KT));
         const bool has_ss = q.ss != nullptr, has_sw = q.sw != nullptr;
-        uint32_t rs_ = 0, rw_[SW_PER], rz_[SW_PER];
+        uint32_t rs_[SS_PER], rzs_[SS_PER], rw_[SW_PER], rz_[SW_PER];
         int64_t iz_[SW_PER];
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++)
+            rs_[j] = rzs_[j] = 0;
 #pragma unroll
         for (int j = 0; j < SW_PER; j++) {
             rw_[j] = rz_[j] = 0;
             iz_[j] = 0;
         }
-        if (has_ss) {
-            const int gl = min(lane >> 2, g_cnt - 1), r = min(lane & 3, q.M - 1);
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++) {
+            const int i = lane + j * 64;
+            const int gl = min(i >> 2, g_cnt - 1), r = min(i & 3, q.M - 1);
             const int k0 = (g_begin + gl) * q.gk;
-            rs_ = scale_raw<SC>(q.ss, r * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
+            if (has_ss)
+                rs_[j] = scale_raw<SC>(
+                        q.ss, r * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
+            if constexpr (SZP) {
+                if (q.zs) // one byte: s8 or u8 (host-checked)
+                    rzs_[j] = ((const uint8_t *)q.zs)[r * q.zs_sm
+                            + (k0 / q.zs_g) * q.zs_sk];
+            }
         }
         if (has_sw) {
 #pragma unroll
@@ -910,9 +936,16 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
         load_weights(0, min(SM_CH, KT));
 
         stage_rows();
-        {
-            const float v = scale_value<SC>(q.ss_dt, rs_);
-            wss[lane] = has_ss ? v : 1.f;
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++) {
+            const float v = scale_value<SC>(q.ss_dt, rs_[j]);
+            wss[lane + j * 64] = has_ss ? v : 1.f;
+            if constexpr (SZP) {
+                const int z = !q.zs ? 0
+                        : q.zs_dt == dt_s8 ? (int)(int8_t)rzs_[j]
+                                           : (int)rzs_[j];
+                wzs[lane + j * 64] = z - (q.a_flip ? 128 : 0);
+            }
         }
 #pragma unroll
         for (int j = 0; j < SW_PER; j++) {
@@ -930,9 +963,44 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
 #pragma unroll
         for (int r = 0; r < 16; r++)
             acc[r] = 0;
-        int rsum = 0;
+        int rsum = 0, csum = 0;
         int t_in_g = 0, gl = 0;
         const int arow = min(lane & 31, q.M - 1) * TN_AROW + (lane >> 5) * 16;
+        // group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+        auto group_end = [&]() {
+            const float sw = wsw[gl * 32 + (lane & 31)];
+            const float4 s4 = *(const float4 *)&wss[gl * 4];
+            const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+            int zw = 0, tot = 0, c2 = 0;
+            int zs[4] = {0, 0, 0, 0};
+            if constexpr (HAS_ZP) {
+                zw = wzw[gl * 32 + (lane & 31)];
+                // both k halves of a row: lanes l and l ^ 32;
+                // row r of the source sits in lane r
+                tot = rsum + __shfl_xor(rsum, 32);
+                rsum = 0;
+            }
+            if constexpr (SZP) {
+                // the column's 16 * sum w' of the group, both k halves
+                const int ctot = csum + __shfl_xor(csum, 32);
+                csum = 0;
+                c2 = -ctot - q.gk * zw;
+                const int4 z4 = *(const int4 *)&wzs[gl * 4];
+                zs[0] = z4.x;
+                zs[1] = z4.y;
+                zs[2] = z4.z;
+                zs[3] = z4.w;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int t = acc[r];
+                if constexpr (HAS_ZP)
+                    t += __mul24(zw, __builtin_amdgcn_readlane(tot, r));
+                if constexpr (SZP) t += __mul24(zs[r], c2);
+                res[r] = __builtin_fmaf((float)t * ss[r], sw, res[r]);
+            }
+            gl++;
+        };
         for (int t0 = 0; t0 < KT; t0 += SM_CH) {
             const int cnt = min(SM_CH, KT - t0);
             if (t0 > 0) {
@@ -954,7 +1022,18 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
                                 (int)(w1 & 0xF0F0F0F0u)};
                         const uint4 v = *(const uint4 *)(wA + arow
                                 + (j * 4 + ki * 2) * 16);
-                        const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        if constexpr (SZP) {
+                            // u8 source: s - 128 as s8
+                            a = v4i {(int)(v.x ^ q.a_flip), (int)(v.y ^ q.a_flip),
+                                    (int)(v.z ^ q.a_flip), (int)(v.w ^ q.a_flip)};
+                            int t = csum;
+                            t = __builtin_amdgcn_sdot4(b[0], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[1], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[2], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[3], 0x01010101, t, false);
+                            csum = t;
+                        }
                         if constexpr (HAS_ZP) {
                             int t = rsum;
                             t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
@@ -963,7 +1042,7 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
                             t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
                             rsum = t;
                         }
-                        if (ki == 0 && first) {
+                        if (HALF || (ki == 0 && first)) {
                             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
                                     0, 0, 0, 0};
                             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
@@ -972,30 +1051,13 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
                             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                     a, b, acc, 0, 0, 0);
                         }
+                        if constexpr (HALF) group_end();
                     }
-                    if (++t_in_g == p.tpg) {
-                        t_in_g = 0;
-                        const float sw = wsw[gl * 32 + (lane & 31)];
-                        const float4 s4 = *(const float4 *)&wss[gl * 4];
-                        const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
-                        int zw = 0, tot = 0;
-                        if constexpr (HAS_ZP) {
-                            zw = wzw[gl * 32 + (lane & 31)];
-                            // both k halves of a row: lanes l and l ^ 32;
-                            // row r of the source sits in lane r
-                            tot = rsum + __shfl_xor(rsum, 32);
-                            rsum = 0;
+                    if constexpr (!HALF) {
+                        if (++t_in_g == p.tpg) {
+                            t_in_g = 0;
+                            group_end();
                         }
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            int t = acc[r];
-                            if constexpr (HAS_ZP)
-                                t += __mul24(zw,
-                                        __builtin_amdgcn_readlane(tot, r));
-                            res[r] = __builtin_fmaf(
-                                    (float)t * ss[r], sw, res[r]);
-                        }
-                        gl++;
                     }
                 }
             }
@@ -1019,26 +1081,30 @@ w4a8_tiny_kernel(const w4a8_small_t p) {
     }
 }
 
-template <int NWV, int SC, bool HAS_ZP, int ZPK>
+template <int NWV, int SC, bool HAS_ZP, int ZPK, int MODE = 0>
 static void launch_tiny_cfg(const w4a8_small_t &p, hipStream_t stream) {
-    constexpr size_t lds = (size_t)NWV * TN_WAVE_BYTES + NWV * 4 * 32 * 4;
-    auto kern = w4a8_tiny_kernel<NWV, SC, HAS_ZP, ZPK>;
+    constexpr size_t lds = (size_t)NWV * tn_wave_bytes(MODE) + NWV * 4 * 32 * 4;
+    auto kern = w4a8_tiny_kernel<NWV, SC, HAS_ZP, ZPK, MODE>;
     ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern, dim3((p.q.N + 31) / 32), dim3(NWV * 64), lds,
             stream, p);
 }
 
-template <int NWV, int SC>
+template <int NWV, int SC, int MODE = 0>
 static void launch_tiny_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         hipStream_t stream) {
-    if (!has_zp)
-        launch_tiny_cfg<NWV, SC, false, 0>(p, stream);
-    else if (zpk == 0)
-        launch_tiny_cfg<NWV, SC, true, 0>(p, stream);
+    if constexpr (MODE != 2) {
+        if (!has_zp) {
+            launch_tiny_cfg<NWV, SC, false, 0, MODE>(p, stream);
+            return;
+        }
+    }
+    if (zpk == 0)
+        launch_tiny_cfg<NWV, SC, true, 0, MODE>(p, stream);
     else if (zpk == 1)
-        launch_tiny_cfg<NWV, SC, true, 1>(p, stream);
+        launch_tiny_cfg<NWV, SC, true, 1, MODE>(p, stream);
     else
-        launch_tiny_cfg<NWV, SC, true, 2>(p, stream);
+        launch_tiny_cfg<NWV, SC, true, 2, MODE>(p, stream);
 }
 
 #if defined(QMM_W4A8_PART) && QMM_W4A8_PART == 3
@@ -1191,19 +1257,31 @@ void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
             dim3(256), 0, stream, (const float *)p.part, p.splits, p.q.M, p.q.N,
             p.ldp, p.ep);
 }
-#elif QMM_W4A8_PART == 4
-void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
-        bool sc4, int nwv, hipStream_t stream) {
+#elif QMM_W4A8_PART == 4 || QMM_W4A8_PART == 8 || QMM_W4A8_PART == 9
+// the single-token kernel: whole tiles per group (4), groups of 32 k (8),
+// source zero points / u8 source (9)
+#if QMM_W4A8_PART == 4
+#define QMM_TINY_NAME launch_gemm_w4a8_tiny_part
+#define QMM_TINY_MODE 0
+#elif QMM_W4A8_PART == 8
+#define QMM_TINY_NAME launch_gemm_w4a8_tiny_half_part
+#define QMM_TINY_MODE 1
+#else
+#define QMM_TINY_NAME launch_gemm_w4a8_tiny_szp_part
+#define QMM_TINY_MODE 2
+#endif
+void QMM_TINY_NAME(const w4a8_small_t &p, bool has_zp, int zpk, bool sc4,
+        int nwv, hipStream_t stream) {
     if (nwv == 8) {
         if (sc4)
-            w4a8::launch_tiny_zp<8, 4>(p, has_zp, zpk, stream);
+            w4a8::launch_tiny_zp<8, 4, QMM_TINY_MODE>(p, has_zp, zpk, stream);
         else
-            w4a8::launch_tiny_zp<8, 2>(p, has_zp, zpk, stream);
+            w4a8::launch_tiny_zp<8, 2, QMM_TINY_MODE>(p, has_zp, zpk, stream);
     } else {
         if (sc4)
-            w4a8::launch_tiny_zp<4, 4>(p, has_zp, zpk, stream);
+            w4a8::launch_tiny_zp<4, 4, QMM_TINY_MODE>(p, has_zp, zpk, stream);
         else
-            w4a8::launch_tiny_zp<4, 2>(p, has_zp, zpk, stream);
+            w4a8::launch_tiny_zp<4, 2, QMM_TINY_MODE>(p, has_zp, zpk, stream);
     }
 }
 #endif
@@ -1222,6 +1300,10 @@ void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, hipStream_t stream);
 void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, int nwv, hipStream_t stream);
+void launch_gemm_w4a8_tiny_half_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, int nwv, hipStream_t stream);
+void launch_gemm_w4a8_tiny_szp_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, int nwv, hipStream_t stream);
 
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
     const int64_t total = (int64_t)p.ng * ((int64_t)p.M + p.N);
@@ -1252,12 +1334,26 @@ static int zp_storage(const w4a8_prep_t &q) {
 }
 
 // Single-token decode kernel: nwv waves per workgroup (4 or 8), p.gps groups
-// per wave; p.part / p.splits are unused.
+// per wave; p.part / p.splits are unused. p.tpg == 0: groups of 32 k;
+// p.q.zsT != nullptr stands for "source zero points / u8 source" (the pointer
+// itself is not used by this kernel).
 void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
         hipStream_t stream) {
     if (p.q.M <= 0 || p.q.N <= 0) return;
-    launch_gemm_w4a8_tiny_part(
-            p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+    if (p.tpg == 0)
+        launch_gemm_w4a8_tiny_half_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+    else if (p.q.zsT)
+        launch_gemm_w4a8_tiny_szp_part(
+                p, true, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+    else
+        launch_gemm_w4a8_tiny_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+}
+
+// groups one wave of the single-token kernel can hold (its LDS tables)
+int gemm_w4a8_tiny_max_groups(bool half) {
+    return w4a8::tn_maxg(half ? 1 : 0);
 }
 
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,

@@ -119,6 +119,14 @@ EXACT_CASES = {
     "src_g32_wei_g32_zp_s4_g32": dict(M=130, K=128, N=130, gs=32, gw=32, gz=32, zp_dt=dt.s4),
     "src_g32_m1_k4096": dict(M=1, K=4096, N=96, gs=32, gw=128, wei_dt=dt.u4, gz=128),
     "src_g32_m300_k1536": dict(M=300, K=1536, N=264, gs=32, gw=128, wei_dt=dt.u4, gz=128),
+    "src_g32_m4_zp_s4_g32": dict(M=4, K=1024, N=70, gs=32, gw=32, gz=32, zp_dt=dt.s4),
+    "src_g32_m2_k8192": dict(M=2, K=8192, N=64, gs=32, gw=128),
+    "src_g32_m1_k14336_tiled": dict(M=1, K=14336, N=64, gs=32, gw=128, wei_dt=dt.u4, gz=128),
+    "u8_src_no_zp_m3": dict(M=3, K=1024, N=100, src_dt=dt.u8, wei_dt=dt.u4),
+    "s8_src_zp_s8_m2_k4096": dict(M=2, K=4096, N=96, src_zp=("k", 256), src_zp_dt=dt.s8, gz=128, zp_dt=dt.u8,
+                                  wei_dt=dt.u4),
+    "u8_src_zp_common_m1": dict(M=1, K=2048, N=160, src_dt=dt.u8, src_zp=("common", 0), gz=64, gs=64, gw=64,
+                                zp_dt=dt.s4),
     "u8_src_zp_m300_k2048": dict(M=300, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
                                  zp_dt=dt.u4),
 }
