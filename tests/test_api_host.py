@@ -343,11 +343,18 @@ def test_generic_takes_what_the_tiled_kernels_do_not(eng):
     assert pd.impl_info_str() == "hip:gfx950:mfma_w4a8"
     assert pd.weights_desc().get_format_kind() == memory.format_kind.opaque
     assert pd.weights_desc().get_size() == 128 * 32 // 2
-    # ... and to the generic kernel otherwise (groups of 32, s32 source zero points)
+    # groups of 32 (half a tile) too
     attr = dnnl.primitive_attr()
     attr.set_scales(dnnl.DNNL_ARG_SRC, 3, [1, 32], dt.f16)
     attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 3, [32, 1], dt.f16)
     pd = dnnl.matmul.primitive_desc(eng, memory.desc([4, 128], dt.s8, T("ab")), memory.desc([128, 32], dt.u4, tag.any),
+                                    memory.desc([4, 32], dt.f16, T("ab")), attr=attr)
+    assert pd.impl_info_str() == "hip:gfx950:mfma_w4a8"
+    # ... and to the generic kernel otherwise (groups of 96, s32 source zero points)
+    attr = dnnl.primitive_attr()
+    attr.set_scales(dnnl.DNNL_ARG_SRC, 3, [1, 96], dt.f16)
+    attr.set_scales(dnnl.DNNL_ARG_WEIGHTS, 3, [96, 1], dt.f16)
+    pd = dnnl.matmul.primitive_desc(eng, memory.desc([4, 192], dt.s8, T("ab")), memory.desc([192, 32], dt.u4, tag.any),
                                     memory.desc([4, 32], dt.f16, T("ab")), attr=attr)
     assert pd.impl_info_str() == "hip:gfx950:generic"
     assert pd.weights_desc().get_format_kind() == memory.format_kind.blocked
