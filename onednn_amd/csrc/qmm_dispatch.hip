@@ -27,6 +27,7 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
+void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream);
 void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
         int src_zp_dt, hipStream_t stream);
@@ -978,6 +979,27 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.src_zp = D.zps[QMM_SRC].set ? args->zps[QMM_SRC] : nullptr;
         g.src_zp_dt = D.zps[QMM_SRC].dt;
         g.a_is_u8 = D.src.dt == dt_u8;
+        g.M = (int32_t)P.M;
+        g.N = (int32_t)P.N;
+        g.K = (int32_t)P.K;
+        g.batch = (int32_t)P.batch;
+        g.kb32 = (int32_t)geom.kb32;
+        g.nb32 = (int32_t)geom.nb32;
+        // at most 4 rows of one matrix: the single-token kernel (it forms the
+        // row sums a weights zero point needs itself)
+        if (!f8 && P.M <= 4 && P.batch == 1 && gemm_variant == 0) {
+            if (b8_needs_rowsum(D)) {
+                const qmm_quant_t &wz = D.zps[QMM_WEI];
+                g.wei_zp = wz.set ? args->zps[QMM_WEI] : nullptr;
+                g.wei_zp_dt = wz.dt;
+                g.wei_zp_sn = wz.set && (wz.mask & (1 << (nd - 1))) ? 1 : 0;
+                g.w_off = D.wei.dt == dt_u8 ? 128 : 0;
+            }
+            launch_gemv_b8(g, stream);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return hip_fail(e, "kernel launch");
+            return QMM_OK;
+        }
         if (b8_needs_rowsum(D)) {
             const qmm_quant_t &wz = D.zps[QMM_WEI];
             int32_t *rs = (int32_t *)((uint8_t *)args->scratch

@@ -1,0 +1,130 @@
+// hip:gfx950:mfma_b8, at most 4 source rows (the decode step of a W8A8 linear
+// layer): the launch is one read of the weights, so the kernel is organised
+// around memory parallelism instead of tiles. A workgroup owns 32 columns (one
+// block of QMM_LAYOUT_MFMA_B8, whose 1 KiB fragments already are the MFMA
+// operand per lane); its 8 waves cut K between them and each streams its
+// fragments straight into registers, 16 requested at a time together with the
+// matching source bytes, and multiplies them with v_mfma_i32_32x32x32_i8 (rows
+// 0..3 of the 32 x 32 result are the source rows; the others repeat the last
+// row and are dropped). The waves' s32 sums are added through LDS by wave 0 --
+// integer addition, so the result does not depend on the cut -- which then runs
+// the epilogue of qmm_gemm_b8.hip per element:
+//   (float)(P + comp * colsum[n] - z_w'[n] * (rowsum[m] + K * comp)),
+// source scale, weights scale, bias, post-ops, dst quantization
+// (src/cpu/matmul/ref_matmul_int8.cpp:165-259). The row sums that a weights
+// zero point needs come from dot products of the source fragments with ones.
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr int GB8_WAVES = 8;
+constexpr int GB8_CH = 16; // fragments in flight per wave
+
+__global__ void __launch_bounds__(GB8_WAVES * 64)
+gemv_b8_kernel(const gemm_params_t p) {
+    __shared__ int red[GB8_WAVES][4][32];
+    __shared__ int red_rs[GB8_WAVES][4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nb = blockIdx.x;
+    // the wave's fragments (32 k each): an even cut of the K / 32 that hold data
+    const int nfrag = (p.K + 31) / 32;
+    const int per = (nfrag + GB8_WAVES - 1) / GB8_WAVES;
+    const int f0 = min(wave * per, nfrag), f1 = min(f0 + per, nfrag);
+    const v4u *bsrc = (const v4u *)(p.B + (int64_t)nb * p.kb32 * 1024) + lane;
+    // A operand: lane l is row l % 32, bytes 16 (l / 32) .. + 15 of the fragment
+    const int row = min(lane & 31, p.M - 1);
+    const uint8_t *arow = p.A + (int64_t)row * p.lda;
+    const uint32_t flip = p.a_is_u8 && !p.a_preflipped ? 0x80808080u : 0u;
+    const bool need_rs = p.wei_zp != nullptr || p.w_off != 0;
+
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    int rsum = 0;
+    for (int fb = f0; fb < f1; fb += GB8_CH) {
+        v4u bq[GB8_CH];
+        uint4 av[GB8_CH];
+        // every request of the chunk before the first use; fragments past the
+        // wave's end repeat its last one and are skipped below
+#pragma unroll
+        for (int j = 0; j < GB8_CH; j++) {
+            const int f = min(fb + j, f1 - 1);
+            bq[j] = __builtin_nontemporal_load(bsrc + (int64_t)f * 64);
+            // K is a multiple of 16: a half fragment is inside the row or past it
+            const int k = f * 32 + (lane >> 5) * 16;
+            av[j] = *(const uint4 *)(arow + min(k, p.K - 16));
+            if (k >= p.K) av[j] = make_uint4(flip, flip, flip, flip); // zero after the flip
+        }
+#pragma unroll
+        for (int j = 0; j < GB8_CH; j++) {
+            if (fb + j < f1) {
+                const v4i a = {(int)(av[j].x ^ flip), (int)(av[j].y ^ flip),
+                        (int)(av[j].z ^ flip), (int)(av[j].w ^ flip)};
+                const v4i b = {(int)bq[j].x, (int)bq[j].y, (int)bq[j].z,
+                        (int)bq[j].w};
+                if (need_rs) {
+                    int t = rsum;
+                    t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
+                    t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
+                    rsum = t;
+                }
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+            }
+        }
+    }
+    // accumulator registers 0..3 of lanes 0..31 are rows 0..3, column = lane;
+    // the two k halves of row r's sum sit in lanes r and r + 32
+    if (lane < 32) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wave][r][lane] = acc[r];
+    }
+    const int tot = rsum + __shfl_xor(rsum, 32);
+    if (lane < 4) red_rs[wave][lane] = tot;
+    __syncthreads();
+    if (wave == 0 && lane < 32) {
+        const int n = nb * 32 + lane;
+        if (n < p.N) {
+            int comp = p.a_is_u8 ? 128 : 0;
+            if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+            const int cs = comp != 0 && p.colsum ? comp * p.colsum[n] : 0;
+            const int zw = need_rs
+                    ? (p.wei_zp ? load_int(p.wei_zp_dt, p.wei_zp,
+                               (int64_t)n * p.wei_zp_sn)
+                                : 0)
+                            - p.w_off
+                    : 0;
+            for (int r = 0; r < p.M; r++) {
+                uint32_t v = 0, rs = 0;
+#pragma unroll
+                for (int w = 0; w < GB8_WAVES; w++) {
+                    v += (uint32_t)red[w][r][lane];
+                    rs += (uint32_t)red_rs[w][r];
+                }
+                // s32 arithmetic that wraps as the reference's int accumulation
+                v += (uint32_t)cs
+                        - (uint32_t)zw * (rs + (uint32_t)p.K * (uint32_t)comp);
+                epilogue_apply_store(p.ep, (float)(int32_t)v, 0, r, n);
+            }
+        }
+    }
+}
+
+} // namespace
+
+// p.M <= 4, one batch, integer operands (the caller checks)
+void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream) {
+    if (p.M <= 0 || p.N <= 0) return;
+    hipLaunchKernelGGL(gemv_b8_kernel, dim3((unsigned)p.nb32),
+            dim3(GB8_WAVES * 64), 0, stream, p);
+}
+
+} // namespace qmm
