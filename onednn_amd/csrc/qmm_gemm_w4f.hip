@@ -1,0 +1,291 @@
+// hip:gfx950:decode_w4 at many rows (the prefill step of a weights-only
+// quantized linear layer): 16-bit activations [M,K] x 4-bit or 8-bit weights
+// [K,N] with K-grouped scales and zero points, f32 accumulation -- the
+// arithmetic of qmm_gemv_w4.hip (src/cpu/matmul/ref_matmul.cpp:140-173 with
+// fpmath_mode apply_to_int), tiled so that a weights tile is unpacked once for
+// BM rows:
+//   * a workgroup of 8 waves owns BM rows x 256 columns; a wave owns 32
+//     columns (two 16-column tiles of QMM_LAYOUT_MFMA_W4 / _W8 per 128 k,
+//     loaded straight into registers one k tile ahead) and all BM rows;
+//   * the activations of a k tile (BM x 128, 16-bit) are shared by the eight
+//     waves through LDS, double buffered, one barrier per k tile; they cross
+//     the CU's load path once per 256 columns;
+//   * per k tile and column: P = sum a * (offset + w) and S = sum a from
+//     16 x 16 x 32 MFMAs (the nibble -> float trick of the decode kernel: no
+//     integer-to-float conversion), then out += scale * (P - (offset + zp) * S);
+//     for 8-bit weights P = 16 P_hi + P_lo over the two nibble planes.
+// One 16-bit scale and at most one byte-sized zero point per column and k tile
+// (group widths 128 << s or all of K), as in the decode kernel's fast variant.
+#include <type_traits>
+
+#include "qmm_device.hpp"
+#include "qmm_plan.hpp"
+
+namespace qmm {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr int WF_WAVES = 8;
+constexpr int WF_BN = 32 * WF_WAVES;
+constexpr int WF_PITCH = 256 + 16; // bytes of a staged activation row
+
+template <bool F16>
+QMM_D v4f mfma16(const v4u &a, const v4u &b, const v4f &c) {
+    if constexpr (F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                __builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0,
+                0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0,
+                0, 0);
+}
+
+QMM_D uint4 ld_stream(const uint8_t *ptr) {
+    const v4u v = __builtin_nontemporal_load((const v4u *)ptr);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// flags_m / shifts: as gemv_w4_fast_kernel (qmm_gemv_w4.hip)
+template <bool F16, bool WSIGNED, bool W8, int BM>
+__global__ void __launch_bounds__(WF_WAVES * 64)
+gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
+    constexpr int RB = BM / 16; // row blocks of the MFMA
+    constexpr int NP = W8 ? 2 : 1;
+    constexpr int TILE_BYTES = 1024 * NP;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * WF_PITCH];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane >> 4, r = lane & 15;
+    const int N = p.N, K = p.K, M = p.M;
+    const int m0 = blockIdx.y * BM;
+    const int nb16 = p.nb16, tiles = p.kg128;
+    const int nb0 = (blockIdx.x * WF_WAVES + wave) * 2; // first 16-column block
+    const int gs_shift = (int8_t)(shifts & 0xff), gz_shift = (int8_t)(shifts >> 8);
+    const bool scale_per_n = flags_m & 1, zp_per_n = flags_m & 2;
+    const bool zp4 = flags_m & 4, zp_signed = flags_m & 8, sc_f16 = flags_m & 16;
+    const bool has_zp = flags_m & 64;
+    constexpr float OFFSET = F16 ? 1024.f : 128.f;
+    constexpr uint32_t ONE2 = F16 ? 0x3C003C00u : 0x3F803F80u;
+    const v4u ones = {ONE2, ONE2, ONE2, ONE2};
+    constexpr uint32_t sflip = WSIGNED ? 0x88888888u : 0u;
+    constexpr float soff = WSIGNED ? 8.f : 0.f;
+    constexpr uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    constexpr uint32_t NIB = 0x000F000Fu;
+
+    // column blocks past the last one repeat it and are never stored
+    const uint8_t *Bt[2];
+    const uint16_t *scn[2];
+    int zcol[2];
+    const int64_t sN = scale_per_n ? N : 0, zN = zp_per_n ? N : 0;
+    const uint8_t *pZP = p.zps ? (const uint8_t *)p.zps : p.B;
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++) {
+        Bt[cb] = p.B + ((int64_t)min(nb0 + cb, nb16 - 1) * tiles) * TILE_BYTES
+                + lane * 16;
+        const int nn = min((nb0 + cb) * 16 + r, N - 1);
+        scn[cb] = (const uint16_t *)p.scales + (scale_per_n ? nn : 0);
+        zcol[cb] = zp_per_n ? nn : 0;
+    }
+
+    // activations: thread t stages 16-byte chunk t % 16 of rows t / 16 + 32 i
+    // (a row of a k tile is 256 bytes = 16 chunks); rows past M repeat the
+    // last row, chunks past K are zero
+    constexpr int A_LD = BM * 16 / (WF_WAVES * 64);
+    static_assert(A_LD >= 1, "");
+    const int a_chunk = tid & 15, a_row = tid >> 4;
+    const uint16_t *a_src[A_LD];
+#pragma unroll
+    for (int i = 0; i < A_LD; i++)
+        a_src[i] = p.A + (int64_t)min(m0 + a_row + 32 * i, M - 1) * p.lda;
+    uint4 a_reg[A_LD], wt[2][NP];
+    uint32_t scp[2], zpp[2];
+    auto request = [&](int kt) { // global -> registers, tile kt
+        const int tc = min(kt, tiles - 1);
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int pl = 0; pl < NP; pl++)
+                wt[cb][pl] = ld_stream(Bt[cb] + (int64_t)tc * TILE_BYTES + pl * 1024);
+        const int k = tc * 128 + a_chunk * 8;
+#pragma unroll
+        for (int i = 0; i < A_LD; i++) {
+            a_reg[i] = *(const uint4 *)(a_src[i] + min(k, K - 8));
+            if (k >= K) a_reg[i] = make_uint4(0, 0, 0, 0);
+        }
+        const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
+        const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++) {
+            scp[cb] = scn[cb][(int64_t)gsc * sN];
+            const int64_t zi = has_zp ? (int64_t)gzp * zN + zcol[cb] : 0;
+            zpp[cb] = pZP[zp4 ? zi >> 1 : zi];
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_LD; i++)
+            *(uint4 *)(lds_a[buf] + (a_row + 32 * i) * WF_PITCH + a_chunk * 16)
+                    = a_reg[i];
+    };
+
+    v4f out[RB][2];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++) out[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
+
+    request(0);
+    for (int kt = 0; kt < tiles; kt++) {
+        // this tile's operands leave the request registers: activations to
+        // LDS, weights / scales / zero points to the compute registers
+        stage(kt & 1);
+        uint4 w_cur[2][NP];
+        uint32_t sc_cur[2], zp_cur[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++) {
+#pragma unroll
+            for (int pl = 0; pl < NP; pl++) w_cur[cb][pl] = wt[cb][pl];
+            sc_cur[cb] = scp[cb];
+            zp_cur[cb] = zpp[cb];
+        }
+        __syncthreads(); // the tile is staged; buffer (kt + 1) & 1 is free
+        if (kt + 1 < tiles) request(kt + 1);
+
+        v4f Pu[RB][2], Pl[RB][2], Su[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            Su[rb] = v4f {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++) {
+                Pu[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
+                Pl[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int s4 = 0; s4 < 4; s4++) {
+            v4u b[2], bl[2];
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++) {
+                const uint32_t d = (s4 == 0 ? w_cur[cb][0].x
+                                : s4 == 1   ? w_cur[cb][0].y
+                                : s4 == 2   ? w_cur[cb][0].z
+                                            : w_cur[cb][0].w)
+                        ^ sflip;
+                b[cb].x = (d & NIB) | MAGIC;
+                b[cb].y = ((d >> 4) & NIB) | MAGIC;
+                b[cb].z = ((d >> 8) & NIB) | MAGIC;
+                b[cb].w = ((d >> 12) & NIB) | MAGIC;
+                bl[cb] = b[cb];
+                if constexpr (W8) {
+                    const uint32_t dl = s4 == 0 ? w_cur[cb][NP - 1].x
+                            : s4 == 1           ? w_cur[cb][NP - 1].y
+                            : s4 == 2           ? w_cur[cb][NP - 1].z
+                                                : w_cur[cb][NP - 1].w;
+                    bl[cb].x = (dl & NIB) | MAGIC;
+                    bl[cb].y = ((dl >> 4) & NIB) | MAGIC;
+                    bl[cb].z = ((dl >> 8) & NIB) | MAGIC;
+                    bl[cb].w = ((dl >> 12) & NIB) | MAGIC;
+                }
+            }
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                // A operand: lane (r, c) holds row 16 rb + r, k = 32 s4 + 8 c ..
+                const uint4 v = *(const uint4 *)(lds_a[kt & 1]
+                        + (16 * rb + r) * WF_PITCH + (32 * s4 + 8 * c) * 2);
+                const v4u a = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++) {
+                    Pu[rb][cb] = mfma16<F16>(a, b[cb], Pu[rb][cb]);
+                    if constexpr (W8)
+                        Pl[rb][cb] = mfma16<F16>(a, bl[cb], Pl[rb][cb]);
+                }
+                Su[rb] = mfma16<F16>(a, ones, Su[rb]);
+            }
+        }
+        const int gzp = gz_shift < 0 ? 0 : kt >> gz_shift;
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++) {
+            const float sc = sc_f16
+                    ? (float)__builtin_bit_cast(_Float16, (uint16_t)sc_cur[cb])
+                    : u2f(sc_cur[cb] << 16);
+            const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol[cb]) & 1) : 0;
+            const int zbits = zp4 ? 4 : 8;
+            const uint32_t zraw = (zp_cur[cb] >> (4 * odd)) & ((1u << zbits) - 1u);
+            const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
+            const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
+            const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp
+                                 : OFFSET + soff + zp;
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    out[rb][cb][j] = __builtin_fmaf(sc,
+                            (W8 ? 16.f * Pu[rb][cb][j] + Pl[rb][cb][j]
+                                : Pu[rb][cb][j])
+                                    - off * Su[rb][j],
+                            out[rb][cb][j]);
+        }
+    }
+
+    // MFMA output: register j of lane l is row 4 * (l / 16) + j, column l % 16
+    const bool plain = (flags_m & 128) != 0;
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++) {
+        const int n = (nb0 + cb) * 16 + r;
+        if (nb0 + cb >= nb16 || n >= N) continue;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int m = m0 + 16 * rb + 4 * c + j;
+                if (m >= M) continue;
+                if (plain)
+                    store_float(p.ep.dst.dt, out[rb][cb][j], (void *)p.ep.dst.ptr,
+                            (int64_t)m * p.ep.dst.sm + n);
+                else
+                    epilogue_apply_store(p.ep, out[rb][cb][j], 0, m, n);
+            }
+    }
+}
+
+} // namespace
+
+// many rows (the caller decides), fast-variant attribute set (the caller
+// checks); flags_m and shifts as for gemv_w4_fast_kernel
+void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
+        hipStream_t stream) {
+    const dim3 grid((unsigned)((p.N + WF_BN - 1) / WF_BN),
+            (unsigned)((p.M + 63) / 64));
+    auto go = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, dim3(WF_WAVES * 64), 0, stream, p, shifts,
+                flags_m);
+    };
+    auto by_bm = [&](auto f16, auto sgn, auto w8) {
+        constexpr bool F = decltype(f16)::value, S = decltype(sgn)::value,
+                       W = decltype(w8)::value;
+        go(gemm_w4f_kernel<F, S, W, 64>);
+    };
+    auto by_w8 = [&](auto f16, auto sgn) {
+        if (p.w8)
+            by_bm(f16, sgn, std::true_type {});
+        else
+            by_bm(f16, sgn, std::false_type {});
+    };
+    auto by_sign = [&](auto f16) {
+        if (p.wei_signed)
+            by_w8(f16, std::true_type {});
+        else
+            by_w8(f16, std::false_type {});
+    };
+    if (p.act_f16)
+        by_sign(std::true_type {});
+    else
+        by_sign(std::false_type {});
+}
+
+} // namespace qmm

@@ -551,6 +551,9 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             (flags_m & 128) != 0, dst_ptr, dst_sm, dst_dt);
 }
 
+void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
+        hipStream_t stream);
+
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return;
     const int rows = p.M < 16 ? p.M : 16;
@@ -611,6 +614,14 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         // an absent zero-point buffer is never dereferenced past its first
         // byte: the weights stand in for it
         const uint8_t *zp = p.zps ? (const uint8_t *)p.zps : p.B;
+        // Enough rows that blocks of 64 rows x 256 columns fill half the chip:
+        // the tiled kernel (a weights tile unpacked once for 64 rows). Below
+        // that, this kernel once per block of 16 rows keeps more CUs reading.
+        if (p.M > 64
+                && (int64_t)((p.M + 63) / 64) * ((p.N + 255) / 256) >= 128) {
+            launch_gemm_w4f(q, shifts, flags_m, stream);
+            return;
+        }
         auto go = [&](auto kern) {
             hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), 0, stream, p.B,
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,

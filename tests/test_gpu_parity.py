@@ -729,6 +729,36 @@ def test_decode_8bit_weights(ctx, name, weights_any):
         assert_bf16_within_1ulp(got, want, "decode 8-bit bf16", abs_slack=2e-5 * decode_term_scale(p))
 
 
+TILED_CASES = {
+    "bf16_u4_g128_zp_u4": dict(M=1100, K=256, N=2048),
+    "f16_u8_per_column_row_and_column_tails": dict(M=1030, K=384, N=2040, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8,
+                                                   per_column=True, wei_layout="ba"),
+    "f16_s4_no_zp_k_tail_f32_dst": dict(M=1090, K=328, N=2048, act_dt=dt.f16, wei_dt=dt.s4, with_zp=False, G=328,
+                                        dst_dt=dt.f32, per_column=True),
+    "bf16_s8_g128_zp_s8": dict(M=1100, K=256, N=2064, wei_dt=dt.s8, zp_dt=dt.s8, scale_dt=dt.bf16),
+}
+
+
+@pytest.mark.parametrize("name", sorted(TILED_CASES))
+def test_decompression_at_many_rows(ctx, name):
+    """Enough rows for the tiled kernel (blocks of 64 rows x 256 columns, a weights tile unpacked once per block):
+    the prefill entries of the reference's LLM list (M = 1024 ... 1088) at a reduced K."""
+    eng, strm = ctx
+    say("decode_w4 tiled %s" % name)
+    kw = TILED_CASES[name]
+    p = decode_w4(seed=70 + len(name), **kw)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == DECODE
+    want = p.run_oracle()
+    code = kw.get("dst_dt") or kw.get("act_dt", dt.bf16)
+    g, w = O.to_f32(code, got).reshape(kw["M"], kw["N"]), O.to_f32(code, want).reshape(kw["M"], kw["N"])
+    assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="tiled decompression")
+    err = np.abs(g.astype(np.float64) - w) / decode_term_scale(p)
+    bar = {dt.f32: 2e-5, dt.f16: 2.0 ** -10, dt.bf16: 2.0 ** -7}[code]
+    print("[tiled decompression] max error %.2e of the summed magnitudes (bar %.1e)" % (err.max(), bar))
+    assert err.max() <= bar
+
+
 def test_prepack_8bit_decode_weights_round_trip(ctx):
     eng, strm = ctx
     say("W8 prepack round trip")
