@@ -102,35 +102,35 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
 #pragma unroll
     for (int i = 0; i < A_LD; i++)
         a_src[i] = p.A + (int64_t)min(m0 + a_row + 32 * i, M - 1) * p.lda;
-    uint4 a_reg[A_LD], wt[2][NP];
-    uint32_t scp[2], zpp[2];
-    auto request = [&](int kt) { // global -> registers, tile kt
+    // two request slots: a tile's operands are asked for two k tiles before
+    // they are used (one k tile of arithmetic is shorter than a trip to memory)
+    uint4 a_reg[2][A_LD], wt[2][2][NP];
+    // kept in their storage types: widening them here would make the request
+    // wait for the values
+    uint16_t scp[2][2];
+    uint8_t zpp[2][2];
+    auto request = [&](int kt, auto slot_tag) { // global -> registers, tile kt
+        constexpr int sl = decltype(slot_tag)::value;
         const int tc = min(kt, tiles - 1);
 #pragma unroll
         for (int cb = 0; cb < 2; cb++)
 #pragma unroll
             for (int pl = 0; pl < NP; pl++)
-                wt[cb][pl] = ld_stream(Bt[cb] + (int64_t)tc * TILE_BYTES + pl * 1024);
+                wt[sl][cb][pl] = ld_stream(
+                        Bt[cb] + (int64_t)tc * TILE_BYTES + pl * 1024);
         const int k = tc * 128 + a_chunk * 8;
 #pragma unroll
-        for (int i = 0; i < A_LD; i++) {
-            a_reg[i] = *(const uint4 *)(a_src[i] + min(k, K - 8));
-            if (k >= K) a_reg[i] = make_uint4(0, 0, 0, 0);
-        }
+        for (int i = 0; i < A_LD; i++) // (chunks past K are zeroed when staged:
+            // touching the value here would make the request wait for it)
+            a_reg[sl][i] = *(const uint4 *)(a_src[i] + min(k, K - 8));
         const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
         const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
 #pragma unroll
         for (int cb = 0; cb < 2; cb++) {
-            scp[cb] = scn[cb][(int64_t)gsc * sN];
+            scp[sl][cb] = scn[cb][(int64_t)gsc * sN];
             const int64_t zi = has_zp ? (int64_t)gzp * zN + zcol[cb] : 0;
-            zpp[cb] = pZP[zp4 ? zi >> 1 : zi];
+            zpp[sl][cb] = pZP[zp4 ? zi >> 1 : zi];
         }
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_LD; i++)
-            *(uint4 *)(lds_a[buf] + (a_row + 32 * i) * WF_PITCH + a_chunk * 16)
-                    = a_reg[i];
     };
 
     v4f out[RB][2];
@@ -139,22 +139,31 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
 #pragma unroll
         for (int cb = 0; cb < 2; cb++) out[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
 
-    request(0);
-    for (int kt = 0; kt < tiles; kt++) {
+    // one k tile; its operands sit in request slot kt % 2 (= LDS buffer)
+    auto k_tile = [&](int kt, auto slot_tag) {
+        constexpr int sl = decltype(slot_tag)::value;
         // this tile's operands leave the request registers: activations to
         // LDS, weights / scales / zero points to the compute registers
-        stage(kt & 1);
+        const bool past_k = kt * 128 + a_chunk * 8 >= K;
+#pragma unroll
+        for (int i = 0; i < A_LD; i++)
+            *(uint4 *)(lds_a[sl] + (a_row + 32 * i) * WF_PITCH + a_chunk * 16)
+                    = past_k ? make_uint4(0, 0, 0, 0) : a_reg[sl][i];
         uint4 w_cur[2][NP];
-        uint32_t sc_cur[2], zp_cur[2];
+        uint16_t sc_cur[2];
+        uint8_t zp_cur[2];
 #pragma unroll
         for (int cb = 0; cb < 2; cb++) {
 #pragma unroll
-            for (int pl = 0; pl < NP; pl++) w_cur[cb][pl] = wt[cb][pl];
-            sc_cur[cb] = scp[cb];
-            zp_cur[cb] = zpp[cb];
+            for (int pl = 0; pl < NP; pl++) w_cur[cb][pl] = wt[sl][cb][pl];
+            sc_cur[cb] = scp[sl][cb];
+            zp_cur[cb] = zpp[sl][cb];
         }
-        __syncthreads(); // the tile is staged; buffer (kt + 1) & 1 is free
-        if (kt + 1 < tiles) request(kt + 1);
+        // the tile is staged; every wave is past its reads of the other buffer
+        __syncthreads();
+        // unconditional (past the end: the last tile again, never used): a
+        // branch around the loads makes the compiler wait for them at its end
+        request(kt + 2, slot_tag);
 
         v4f Pu[RB][2], Pl[RB][2], Su[RB];
 #pragma unroll
@@ -195,7 +204,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++) {
                 // A operand: lane (r, c) holds row 16 rb + r, k = 32 s4 + 8 c ..
-                const uint4 v = *(const uint4 *)(lds_a[kt & 1]
+                const uint4 v = *(const uint4 *)(lds_a[sl]
                         + (16 * rb + r) * WF_PITCH + (32 * s4 + 8 * c) * 2);
                 const v4u a = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -211,11 +220,12 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
 #pragma unroll
         for (int cb = 0; cb < 2; cb++) {
             const float sc = sc_f16
-                    ? (float)__builtin_bit_cast(_Float16, (uint16_t)sc_cur[cb])
-                    : u2f(sc_cur[cb] << 16);
+                    ? (float)__builtin_bit_cast(_Float16, sc_cur[cb])
+                    : u2f((uint32_t)sc_cur[cb] << 16);
             const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol[cb]) & 1) : 0;
             const int zbits = zp4 ? 4 : 8;
-            const uint32_t zraw = (zp_cur[cb] >> (4 * odd)) & ((1u << zbits) - 1u);
+            const uint32_t zraw
+                    = ((uint32_t)zp_cur[cb] >> (4 * odd)) & ((1u << zbits) - 1u);
             const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
             const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
             const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp
@@ -230,6 +240,12 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                                     - off * Su[rb][j],
                             out[rb][cb][j]);
         }
+    };
+    request(0, std::integral_constant<int, 0> {});
+    request(1, std::integral_constant<int, 1> {});
+    for (int kt = 0; kt < tiles; kt += 2) {
+        k_tile(kt, std::integral_constant<int, 0> {});
+        if (kt + 1 < tiles) k_tile(kt + 1, std::integral_constant<int, 1> {});
     }
 
     // MFMA output: register j of lane l is row 4 * (l / 16) + j, column l % 16
