@@ -13,7 +13,8 @@
 //   * per k tile and column: P = sum a * (offset + w) and S = sum a from
 //     16 x 16 x 32 MFMAs (the nibble -> float trick of the decode kernel: no
 //     integer-to-float conversion), then out += scale * (P - (offset + zp) * S);
-//     for 8-bit weights P = 16 P_hi + P_lo over the two nibble planes.
+//     for 8-bit weights both nibble planes add into P, the high one behind
+//     the exponent of 16 * offset (P = sum a * (17 offset + w)).
 // One 16-bit scale and at most one byte-sized zero point per column and k tile
 // (group widths 128 << s or all of K), as in the decode kernel's fast variant.
 #include <type_traits>
@@ -57,7 +58,13 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     constexpr int RB = BM / 16; // row blocks of the MFMA
     constexpr int NP = W8 ? 2 : 1;
     constexpr int TILE_BYTES = 1024 * NP;
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * WF_PITCH];
+    // two activation buffers; after the k loop the same bytes stage the results
+    constexpr int A_BUF = BM * WF_PITCH, STG_PITCH = 36; // floats per staged row
+    constexpr int STG_WAVE = 32 * STG_PITCH * 4; // 32 rows x 32 columns of a wave
+    constexpr int LDS_BYTES
+            = 2 * A_BUF > WF_WAVES * STG_WAVE ? 2 * A_BUF : WF_WAVES * STG_WAVE;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    uint8_t *const lds_a[2] = {lds_raw, lds_raw + A_BUF};
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane >> 4, r = lane & 15;
@@ -75,6 +82,11 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     constexpr uint32_t sflip = WSIGNED ? 0x88888888u : 0u;
     constexpr float soff = WSIGNED ? 8.f : 0.f;
     constexpr uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    // 8-bit weights: the high nibbles behind the exponent of 16 * offset, where
+    // one unit of the last mantissa bit is 16 (f16: 0x7400 | h = 16384 + 16 h;
+    // bf16: 0x4500 | h = 2048 + 16 h), so both planes add into one accumulator:
+    // sum a * (16 (offset + h) + (offset + l)) = sum a * (17 offset + w)
+    constexpr uint32_t MAGIC_HI = W8 ? (F16 ? 0x74007400u : 0x45004500u) : MAGIC;
     constexpr uint32_t NIB = 0x000F000Fu;
 
     // column blocks past the last one repeat it and are never stored
@@ -165,14 +177,13 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         // branch around the loads makes the compiler wait for them at its end
         request(kt + 2, slot_tag);
 
-        v4f Pu[RB][2], Pl[RB][2], Su[RB];
+        v4f Pu[RB][2], Su[RB];
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             Su[rb] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int cb = 0; cb < 2; cb++) {
                 Pu[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
-                Pl[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
             }
         }
 #pragma unroll
@@ -185,10 +196,10 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                                 : s4 == 2   ? w_cur[cb][0].z
                                             : w_cur[cb][0].w)
                         ^ sflip;
-                b[cb].x = (d & NIB) | MAGIC;
-                b[cb].y = ((d >> 4) & NIB) | MAGIC;
-                b[cb].z = ((d >> 8) & NIB) | MAGIC;
-                b[cb].w = ((d >> 12) & NIB) | MAGIC;
+                b[cb].x = (d & NIB) | MAGIC_HI;
+                b[cb].y = ((d >> 4) & NIB) | MAGIC_HI;
+                b[cb].z = ((d >> 8) & NIB) | MAGIC_HI;
+                b[cb].w = ((d >> 12) & NIB) | MAGIC_HI;
                 bl[cb] = b[cb];
                 if constexpr (W8) {
                     const uint32_t dl = s4 == 0 ? w_cur[cb][NP - 1].x
@@ -211,7 +222,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                 for (int cb = 0; cb < 2; cb++) {
                     Pu[rb][cb] = mfma16<F16>(a, b[cb], Pu[rb][cb]);
                     if constexpr (W8)
-                        Pl[rb][cb] = mfma16<F16>(a, bl[cb], Pl[rb][cb]);
+                        Pu[rb][cb] = mfma16<F16>(a, bl[cb], Pu[rb][cb]);
                 }
                 Su[rb] = mfma16<F16>(a, ones, Su[rb]);
             }
@@ -235,10 +246,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     out[rb][cb][j] = __builtin_fmaf(sc,
-                            (W8 ? 16.f * Pu[rb][cb][j] + Pl[rb][cb][j]
-                                : Pu[rb][cb][j])
-                                    - off * Su[rb][j],
-                            out[rb][cb][j]);
+                            Pu[rb][cb][j] - off * Su[rb][j], out[rb][cb][j]);
         }
     };
     request(0, std::integral_constant<int, 0> {});
@@ -248,25 +256,41 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         if (kt + 1 < tiles) k_tile(kt + 1, std::integral_constant<int, 1> {});
     }
 
-    // MFMA output: register j of lane l is row 4 * (l / 16) + j, column l % 16
-    const bool plain = (flags_m & 128) != 0;
+    // Epilogue: the wave's 64 x 32 results go through a wave-private LDS tile,
+    // 32 rows at a time, and come back as four neighbouring columns of a row
+    // per lane, so that bias / post-ops / dst conversion exist once and every
+    // store is a vector. MFMA output: register j of lane l is row
+    // 4 * (l / 16) + j, column l % 16.
+    __syncthreads(); // every wave is done with the activation buffers
+    float *const stg = (float *)(lds_raw + wave * STG_WAVE);
+    const int n_w = nb0 * 16; // the wave's first column
+    static_assert(RB == 4, "two halves of 32 rows");
+    auto flush = [&](auto h_tag) { // rows 32 h .. 32 h + 31 (h a constant:
+        // the accumulators must stay in registers)
+        constexpr int h = decltype(h_tag)::value;
 #pragma unroll
-    for (int cb = 0; cb < 2; cb++) {
-        const int n = (nb0 + cb) * 16 + r;
-        if (nb0 + cb >= nb16 || n >= N) continue;
+        for (int rb2 = 0; rb2 < 2; rb2++)
 #pragma unroll
-        for (int rb = 0; rb < RB; rb++)
+            for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int m = m0 + 16 * rb + 4 * c + j;
-                if (m >= M) continue;
-                if (plain)
-                    store_float(p.ep.dst.dt, out[rb][cb][j], (void *)p.ep.dst.ptr,
-                            (int64_t)m * p.ep.dst.sm + n);
-                else
-                    epilogue_apply_store(p.ep, out[rb][cb][j], 0, m, n);
+                for (int j = 0; j < 4; j++)
+                    stg[(16 * rb2 + 4 * c + j) * STG_PITCH + 16 * cb + r]
+                            = out[2 * h + rb2][cb][j];
+        // (wave-private: the LDS writes above are ordered before the reads
+        // below by the compiler's waitcnt, no barrier needed)
+#pragma unroll 1
+        for (int it = 0; it < 4; it++) {
+            const int row = it * 8 + (lane >> 3), cg = (lane & 7) * 4;
+            const float4 t = *(const float4 *)&stg[row * STG_PITCH + cg];
+            const int m = m0 + 32 * h + row, n = n_w + cg;
+            if (m < M && n < N) {
+                float v[4] = {t.x, t.y, t.z, t.w};
+                epilogue_apply_store4(p.ep, v, 0, m, n, min(4, N - n));
             }
-    }
+        }
+    };
+    flush(std::integral_constant<int, 0> {});
+    flush(std::integral_constant<int, 1> {});
 }
 
 } // namespace

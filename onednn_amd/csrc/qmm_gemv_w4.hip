@@ -350,8 +350,9 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 //     bits 8..: M
 // W8: 8-bit weights as two planes of nibbles (QMM_LAYOUT_MFMA_W8: a tile is
 // its high-nibble KiB followed by its low-nibble KiB). Both planes go through
-// the 4-bit arithmetic, w = 16 hi + lo:
-//     sum a * (w - z) = 16 P_hi + P_lo - (17 * offset + 16 * [8 if signed] + z) * S,
+// the 4-bit arithmetic, w = 16 hi + lo, the high nibbles as 16 * (offset + hi)
+// so that both planes add into one accumulator:
+//     sum a * (w - z) = P - (17 * offset + 16 * [8 if signed] + z) * S,
 // the sign of an s8 weight living in its high nibble.
 template <bool F16, int ROWS, bool WSIGNED, bool W8>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
@@ -390,6 +391,11 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     // v_and_or_b32 (an instruction takes one scalar or literal operand only)
     uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
     asm volatile("" : "+v"(MAGIC));
+    // 8-bit weights: the high nibbles behind the exponent of 16 * offset, where
+    // one unit of the last mantissa bit is 16 (f16: 0x7400 | h = 16384 + 16 h;
+    // bf16: 0x4500 | h = 2048 + 16 h), so both planes add into one accumulator
+    uint32_t MAGIC_HI = W8 ? (F16 ? 0x74007400u : 0x45004500u) : MAGIC;
+    if constexpr (W8) asm volatile("" : "+v"(MAGIC_HI));
     uint32_t NIB = 0x000F000Fu;
     asm volatile("" : "+s"(NIB));
 
@@ -477,7 +483,6 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             v4f Pu = {0.f, 0.f, 0.f, 0.f}, Su = {0.f, 0.f, 0.f, 0.f};
-            v4f Pl = {0.f, 0.f, 0.f, 0.f}; // low-nibble plane (W8)
 #pragma unroll
             for (int s4 = 0; s4 < 4; s4++) {
                 const uint32_t d = (s4 == 0 ? wt[u][0].x
@@ -486,10 +491,10 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                                             : wt[u][0].w)
                         ^ sflip;
                 v4u b;
-                b.x = (d & NIB) | MAGIC;
-                b.y = ((d >> 4) & NIB) | MAGIC;
-                b.z = ((d >> 8) & NIB) | MAGIC;
-                b.w = ((d >> 12) & NIB) | MAGIC;
+                b.x = (d & NIB) | MAGIC_HI;
+                b.y = ((d >> 4) & NIB) | MAGIC_HI;
+                b.z = ((d >> 8) & NIB) | MAGIC_HI;
+                b.w = ((d >> 12) & NIB) | MAGIC_HI;
                 v4u bl = b;
                 if constexpr (W8) {
                     const uint32_t dl = s4 == 0 ? wt[u][NP - 1].x
@@ -519,7 +524,7 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                                 row_shl<3>(v.z), row_shl<3>(v.w)};
                 }
                 Pu = mfma16<F16>(a, b, Pu);
-                if constexpr (W8) Pl = mfma16<F16>(a, bl, Pl);
+                if constexpr (W8) Pu = mfma16<F16>(a, bl, Pu);
                 Su = mfma16<F16>(a, ones, Su);
             }
             const int t = tb + uw + u * GEMV_WAVES;
@@ -543,7 +548,7 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
 #pragma unroll
             for (int j = 0; j < 4; j += SPL)
                 out[j] = __builtin_fmaf(sc,
-                        (W8 ? 16.f * Pu[j] + Pl[j] : Pu[j]) - off * Su[j],
+                        Pu[j] - off * Su[j],
                         out[j]);
         }
     }
