@@ -233,7 +233,7 @@ def C_stream(strm):
     return p.value
 
 
-def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, K=4096, N=4096, rows=(1, 4, 8, 16)):
+def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, K=4096, N=4096, rows=(1, 4, 8, 16, 1024)):
     """Config 3: bf16 x u4 GEMV, G=128 f16 scales + u4 zero points. The 8.7 MB
     of one weights set would sit in the last-level cache, so `sets` distinct
     copies are cycled; the launches are replayed from a HIP graph so that the
@@ -331,6 +331,10 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
         res["M%d%s" % (M, "_u8_weights" if w8 else "")] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
                           "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
                           "impl": pd.impl_info_str(), "weight_sets": sets, "timing": "hip graph of %d launches x %d" % (sets, reps)}
+        if M > 64:  # the prefill step of the same layer: the tiled kernel, arithmetic-bound
+            key = "M%d%s" % (M, "_u8_weights" if w8 else "")
+            res[key]["TFLOPs"] = round(2.0 * M * K * N / us / 1e6, 1)
+            res[key]["frac_of_f16_peak"] = round(2.0 * M * K * N / us / 1e6 / 2500.0, 4)
         if floor is not None:
             res["M1"]["read_floor_us"] = floor
             res["M1"]["read_floor_kernel"] = ("qmm_stream_read: 256 workgroups x 512 lanes, 16-byte loads of the same "
