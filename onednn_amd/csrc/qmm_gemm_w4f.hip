@@ -113,7 +113,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     const uint16_t *a_src[A_LD];
 #pragma unroll
     for (int i = 0; i < A_LD; i++)
-        a_src[i] = p.A + (int64_t)min(m0 + a_row + 32 * i, M - 1) * p.lda;
+        a_src[i] = p.A + (int64_t)min(m0 + a_row + WF_WAVES * 4 * i, M - 1) * p.lda;
     // two request slots: a tile's operands are asked for two k tiles before
     // they are used (one k tile of arithmetic is shorter than a trip to memory)
     uint4 a_reg[2][A_LD], wt[2][2][NP];
@@ -159,7 +159,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         const bool past_k = kt * 128 + a_chunk * 8 >= K;
 #pragma unroll
         for (int i = 0; i < A_LD; i++)
-            *(uint4 *)(lds_a[sl] + (a_row + 32 * i) * WF_PITCH + a_chunk * 16)
+            *(uint4 *)(lds_a[sl] + (a_row + WF_WAVES * 4 * i) * WF_PITCH + a_chunk * 16)
                     = past_k ? make_uint4(0, 0, 0, 0) : a_reg[sl][i];
         uint4 w_cur[2][NP];
         uint16_t sc_cur[2];
