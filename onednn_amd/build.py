@@ -35,7 +35,7 @@ UNITS = [("qmm_generic.hip", "", []), ("qmm_gemv_w4.hip", "", PRELOAD),
          ("qmm_pack.hip", "", []), ("qmm_quantize.hip", "", []),
          ("qmm_dispatch.hip", "", []), ("qmm_measure.hip", "", PRELOAD), ("qmm_softmax.hip", "", []), ("qmm_sdpa.hip", "", []),
          ("qmm_gemm_b8.hip", "", []),
-         ("qmm_gemm_b8x.hip", "", []), ("qmm_gemm_w4a8.hip", "", []), ("qmm_gemv_b8.hip", "", []), ("qmm_gemm_w4f.hip", "", []),
+         ("qmm_gemm_b8x.hip", "", []), ("qmm_gemm_w4a8.hip", "", []), ("qmm_gemv_b8.hip", "", []), ("qmm_gemm_w4f.hip", "", []), ("qmm_gemm_f16.hip", "", []),
          ("dnnl_core.cpp", "", []), ("dnnl_primitives.cpp", "", [])]
 # the tiled GEMM is instantiated once per tile configuration, each in its own
 # object so the instantiations compile in parallel

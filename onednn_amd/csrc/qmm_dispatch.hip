@@ -28,6 +28,7 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream);
+void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream);
 void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
         int src_zp_dt, hipStream_t stream);
@@ -642,6 +643,31 @@ int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     return QMM_OK;
 }
 
+// plain 16-bit matmul: no quantization attributes, source rows K-contiguous,
+// weights and dst rows N-contiguous, batch dims that fold into one stride
+int supports_gemm_f16(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    const int nd = D.dst.ndims;
+    if (!one_of(D.src.dt, {dt_f16, dt_bf16}) || D.wei.dt != D.src.dt)
+        return QMM_UNIMPLEMENTED;
+    if (D.dst.dt != D.src.dt && D.dst.dt != dt_f32) return QMM_UNIMPLEMENTED;
+    if (D.wei_layout != QMM_LAYOUT_PLAIN) return QMM_UNIMPLEMENTED;
+    for (int i = 0; i < 3; i++)
+        if (D.scales[i].set || D.zps[i].set) return QMM_UNIMPLEMENTED;
+    if (P.M == 0 || P.N == 0 || P.K == 0) return QMM_UNIMPLEMENTED;
+    if (P.M > INT32_MAX || P.N > INT32_MAX || P.K > INT32_MAX
+            || P.batch > 65535 || (P.M + 63) / 64 > 65535)
+        return QMM_UNIMPLEMENTED;
+    if (D.src.strides[nd - 1] != 1 || D.wei.strides[nd - 1] != 1
+            || D.dst.strides[nd - 1] != 1)
+        return QMM_UNIMPLEMENTED;
+    int64_t sb;
+    if (!fold_batch(D.src, D.dst, sb) || !fold_batch(D.wei, D.dst, sb))
+        return QMM_UNIMPLEMENTED;
+    epilogue_t ep;
+    if (!build_epilogue(ep, P, nullptr)) return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
 int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     if (D.wei_layout != QMM_LAYOUT_PLAIN) return QMM_UNIMPLEMENTED;
     const int s = D.src.dt, w = D.wei.dt, d = D.dst.dt;
@@ -684,7 +710,8 @@ int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
 }
 
 const char *impl_names[impl_count] = {"hip:gfx950:mfma_b8",
-        "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:generic"};
+        "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:mfma_f16",
+        "hip:gfx950:generic"};
 
 std::atomic<int> g_gemm_variant {0};
 std::atomic<int> g_w4a8_variant {0};
@@ -719,6 +746,7 @@ int qmm_matmul_impl_supports(int impl, const qmm_matmul_desc_t *desc) {
         case impl_gemm_b8: return supports_gemm_b8(*desc, P);
         case impl_gemm_w4a8: return supports_gemm_w4a8(*desc, P);
         case impl_gemv_w4: return supports_gemv_w4(*desc, P);
+        case impl_gemm_f16: return supports_gemm_f16(*desc, P);
         case impl_generic: return supports_generic(*desc, P);
         default: return QMM_INVALID_ARGUMENTS;
     }
@@ -942,7 +970,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
     (void)gemm_variant;
     (void)w4a8_variant;
     int impl = plan->impl;
-    if (impl != impl_generic && !aligned16(args->src)) {
+    if (impl != impl_generic && impl != impl_gemm_f16 && !aligned16(args->src)) {
         if (!plan->dev)
             return fail(QMM_INVALID_ARGUMENTS,
                     "source pointer must be 16-byte aligned");
@@ -1170,6 +1198,25 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.tpg = q.gk / 64;
         g.ng = q.ng;
         launch_gemm_w4a8(g, w4a8_variant, stream);
+    } else if (impl == impl_gemm_f16) {
+        gemm16_params_t g;
+        std::memset(&g, 0, sizeof(g));
+        if (!build_epilogue(g.ep, P, args))
+            return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
+        g.A = (const uint16_t *)args->src;
+        g.B = (const uint16_t *)args->wei;
+        g.lda = D.src.strides[nd - 2];
+        g.ldb = D.wei.strides[nd - 2];
+        fold_batch(D.src, D.dst, g.a_sb);
+        fold_batch(D.wei, D.dst, g.b_sb);
+        g.M = (int32_t)P.M;
+        g.N = (int32_t)P.N;
+        g.K = (int32_t)P.K;
+        g.batch = (int32_t)P.batch;
+        g.bf = D.src.dt == dt_bf16;
+        g.a_vec = g.lda % 8 == 0 && g.a_sb % 8 == 0 && aligned16(args->src);
+        g.b_vec = g.ldb % 8 == 0 && g.b_sb % 8 == 0 && aligned16(args->wei);
+        launch_gemm_f16(g, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;
         std::memset(&g, 0, sizeof(g));

@@ -165,6 +165,17 @@ struct gemm_params_t {
     epilogue_t ep;
 };
 
+// ---- plain 16-bit batched matmul (qmm_gemm_f16.hip) ---------------------------
+struct gemm16_params_t {
+    const uint16_t *A, *B; // src rows K-contiguous, weights rows N-contiguous
+    int64_t lda, a_sb, ldb, b_sb; // elements
+    int32_t M, N, K, batch;
+    int32_t bf; // bf16 (else f16)
+    int32_t a_vec, b_vec; // rows and base on 16-byte boundaries: vector loads
+    int32_t pad_;
+    epilogue_t ep;
+};
+
 // ---- decode kernel (4-bit / 8-bit weights, 16-bit activations) -------------
 struct gemv_params_t {
     const uint16_t *A; // activations [M][K], bf16 or f16
@@ -274,9 +285,10 @@ struct quant_rows_params_t {
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
     impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales
-    impl_gemv_w4 = 2, // decode: 4-bit weights, 16-bit activations, M small
-    impl_generic = 3,
-    impl_count = 4
+    impl_gemv_w4 = 2, // decode: 4-bit / 8-bit weights, 16-bit activations
+    impl_gemm_f16 = 3, // plain f16 / bf16 batched matmul
+    impl_generic = 4,
+    impl_count = 5
 };
 
 } // namespace qmm

@@ -1,0 +1,93 @@
+"""GPU parity of hip:gfx950:mfma_f16 (plain f16 / bf16 batched matmul, f32 accumulation) against the CPU oracle
+(src/cpu/matmul/ref_matmul.cpp:130-233): the unfused attention products of the reference's LLM list
+(tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu, --dt=f16:f16:f16 --stag=abcd --wtag=abcd --dtag=abcd, K and N
+such as 998, 999, 1000 that are not multiples of the vector width). The kernel sums in another order than the oracle's
+k loop, so results are compared within one step of the dst type on the magnitude of the summed terms; integer-valued
+data, where every order gives the same bits, is compared bit for bit."""
+import sys
+
+import numpy as np
+import pytest
+
+import onednn_amd as dnnl
+import oracle as O
+from qmm_harness import Problem, TensorSpec, assert_bit_exact, assert_f32_close, dt
+
+pytestmark = pytest.mark.gpu
+A = dnnl.algorithm
+F16MM, GENERIC = "hip:gfx950:mfma_f16", "hip:gfx950:generic"
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    eng = dnnl.engine(dnnl.engine.kind.gpu, 0)
+    return eng, dnnl.stream(eng)
+
+
+def problem(sd, wd, seed, code=dt.f16, dst_dt=None, exact=False, post_ops=None, bias=False):
+    r = np.random.default_rng(seed)
+    nd = len(sd)
+    dd = [max(a, b) for a, b in zip(sd[:-2], wd[:-2])] + [sd[-2], wd[-1]]
+    if exact:
+        s, w = r.integers(-4, 5, sd).astype(np.float32), r.integers(-4, 5, wd).astype(np.float32)
+    else:
+        s, w = r.standard_normal(sd).astype(np.float32), r.standard_normal(wd).astype(np.float32)
+    b = None
+    if bias:
+        b = TensorSpec(dt.f32, [1] * (nd - 1) + [wd[-1]], None, r.integers(-3, 4, wd[-1]).astype(np.float32))
+    return Problem(TensorSpec(code, sd, None, s), TensorSpec(code, wd, None, w), TensorSpec(dst_dt or code, dd), bias=b,
+                   post_ops=post_ops)
+
+
+CASES = {
+    "decode_scores_clip": dict(sd=[1, 8, 1, 128], wd=[1, 8, 128, 999], post_ops=[{"kind": "eltwise", "alg": A.eltwise_clip, "alpha": -1.0, "beta": 1.0}]),
+    "decode_context_k999": dict(sd=[1, 8, 1, 999], wd=[1, 8, 999, 128]),
+    "prefill_scores_998": dict(sd=[1, 4, 198, 128], wd=[1, 4, 128, 198]),
+    "prefill_context_k198": dict(sd=[1, 4, 198, 198], wd=[1, 4, 198, 128]),
+    "two_dims_bf16_f32_dst": dict(sd=[70, 256], wd=[256, 100], code=dt.bf16, dst_dt=dt.f32),
+    "broadcast_weights_bias": dict(sd=[3, 2, 33, 64], wd=[1, 1, 64, 72], bias=True),
+    "tiny_k": dict(sd=[2, 5, 8], wd=[2, 8, 16]),
+    "odd_everything": dict(sd=[2, 67, 45], wd=[2, 45, 51]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+@pytest.mark.parametrize("exact", [True, False])
+def test_f16_matmul(ctx, name, exact):
+    eng, strm = ctx
+    say("mfma_f16 %s exact=%s" % (name, exact))
+    kw = CASES[name]
+    p = problem(seed=len(name), exact=exact, **kw)
+    got, pd = p.run_gpu(eng, strm, return_pd=True)
+    assert pd.impl_info_str() == F16MM
+    want = p.run_oracle()
+    if exact:
+        assert_bit_exact(got, want, name)
+        return
+    code = kw.get("dst_dt") or kw.get("code", dt.f16)
+    g, w = O.to_f32(code, got), O.to_f32(code, want)
+    K = kw["sd"][-1]
+    step = {dt.f16: 2.0 ** -10, dt.bf16: 2.0 ** -7, dt.f32: 1e-5}[code]
+    assert_f32_close(g, w, rel=step, scale=np.sqrt(K), what=name, max_slack_frac=1.0)
+
+
+def test_matches_the_per_element_kernel(ctx):
+    eng, strm = ctx
+    say("mfma_f16 vs generic")
+    p = problem([2, 3, 40, 96], [2, 3, 96, 80], 5, exact=True)
+    assert_bit_exact(p.run_gpu(eng, strm, impl=F16MM), p.run_gpu(eng, strm, impl=GENERIC), "vs generic")
+
+
+def test_what_it_does_not_take(ctx):
+    """Transposed weights (k contiguous) and f32 operands stay with the per-element kernel."""
+    eng, strm = ctx
+    p = Problem(TensorSpec(dt.f16, [16, 32], None, np.ones((16, 32), np.float32)),
+                TensorSpec(dt.f16, [32, 24], "ba", np.ones((32, 24), np.float32)), TensorSpec(dt.f16, [16, 24]))
+    got, pd = p.run_gpu(eng, strm, return_pd=True)
+    assert pd.impl_info_str() == GENERIC
+    assert_bit_exact(got, p.run_oracle(), "ba weights")
