@@ -117,7 +117,10 @@ def test_f16_chain_with_quantized_kv_cache(ctx, Qn):
              O.Tensor(dt.f32, [MB, H, Qn, S], want_s),
              post_ops=[{"kind": "binary", "alg": A.binary_mul, "src1": O.Tensor(dt.f32, [1, 1, 1, 1], scale)},
                        {"kind": "binary", "alg": A.binary_add, "src1": O.Tensor(dt.f32, [1, 1, Qn, S], mask)}])
-    assert np.array_equal(got_s, want_s), "scores"  # the generic kernel adds in the reference's order
+    # the 16-bit MFMA matmul sums in another order than the oracle's k loop: 1e-5 of the magnitude of the summed terms
+    err_s = np.abs(got_s.astype(np.float64) - want_s)
+    tol_s = 1e-5 * np.maximum(np.abs(want_s), np.sqrt(D) * np.abs(float(scale[0])))
+    assert np.all((err_s <= tol_s) | np.isinf(want_s)), ("scores", float(err_s[np.isfinite(want_s)].max()))
 
     # ---- stage 2: softmax over the keys, f32 -> f16
     p_md = memory.desc([MB, H, Qn, S], dt.f16, T("abcd"))
@@ -141,7 +144,9 @@ def test_f16_chain_with_quantized_kv_cache(ctx, Qn):
     want_o = np.zeros((MB, H, Qn, D), np.uint16)
     O.matmul(O.Tensor(dt.f16, [MB, H, Qn, S], got_p), O.Tensor(dt.f16, [MB, H, S, D], v_deq),
              O.Tensor(dt.f16, [MB, H, Qn, D], want_o))
-    assert np.array_equal(got_o, want_o), "output"
+    d_o = np.abs(got_o.astype(np.int32) - want_o.astype(np.int32))  # f16 codes: at most one step apart
+    near_zero = np.abs(O.to_f32(dt.f16, want_o).reshape(want_o.shape)) < 2.0 ** -10
+    assert np.all((d_o <= 1) | near_zero) and (d_o != 0).mean() < 0.05, ("output", int(d_o.max()), float((d_o != 0).mean()))
 
     # ---- end to end against float64 attention on the dequantized operands, the reference test's rule
     kf = O.to_f32(dt.f16, k_deq).reshape(MB, H, D, S).astype(np.float64)
