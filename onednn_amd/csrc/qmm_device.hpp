@@ -596,26 +596,36 @@ QMM_D void epilogue_store4(const epilogue_t &ep, const float (&d)[4],
     if (nvalid == 4 && ep.dst.sn == 1) {
         if (dt == dt_bf16 || dt == dt_f16) {
             uint16_t *q = (uint16_t *)dst + dst_off;
-            if (((uintptr_t)q & 7) == 0) {
-                uint16_t h[4];
-                if (dt == dt_bf16) {
+            uint16_t h[4];
+            if (dt == dt_bf16) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        h[i] = f32_to_bf16(d[i]);
-                } else if (d[0] != d[0] || d[1] != d[1] || d[2] != d[2]
-                        || d[3] != d[3]) {
+                for (int i = 0; i < 4; i++)
+                    h[i] = f32_to_bf16(d[i]);
+            } else if (d[0] != d[0] || d[1] != d[1] || d[2] != d[2]
+                    || d[3] != d[3]) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        h[i] = f32_to_f16(d[i]);
-                } else {
+                for (int i = 0; i < 4; i++)
+                    h[i] = f32_to_f16(d[i]);
+            } else {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        h[i] = f32_to_f16_hw(d[i]);
-                }
-                *(uint2 *)q = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16),
-                        (uint32_t)h[2] | ((uint32_t)h[3] << 16));
-                return;
+                for (int i = 0; i < 4; i++)
+                    h[i] = f32_to_f16_hw(d[i]);
             }
+            // the widest stores the address allows (rows of odd length start
+            // on 2- or 4-byte boundaries)
+            const uint32_t lo = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+            const uint32_t hi = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+            if (((uintptr_t)q & 7) == 0) {
+                *(uint2 *)q = make_uint2(lo, hi);
+            } else if (((uintptr_t)q & 3) == 0) {
+                *(uint32_t *)q = lo;
+                *(uint32_t *)(q + 2) = hi;
+            } else {
+                q[0] = h[0];
+                *(uint32_t *)(q + 1) = (uint32_t)h[1] | ((uint32_t)h[2] << 16);
+                q[3] = h[3];
+            }
+            return;
         } else if (dt == dt_f32) {
             float *q = (float *)dst + dst_off;
             if (((uintptr_t)q & 15) == 0) {

@@ -1214,8 +1214,15 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.K = (int32_t)P.K;
         g.batch = (int32_t)P.batch;
         g.bf = D.src.dt == dt_bf16;
-        g.a_vec = g.lda % 8 == 0 && g.a_sb % 8 == 0 && aligned16(args->src);
-        g.b_vec = g.ldb % 8 == 0 && g.b_sb % 8 == 0 && aligned16(args->wei);
+        // the widest aligned load every row start of the operand allows
+        auto granule = [](int64_t ld, int64_t sb, const void *ptr) {
+            for (int g = 8; g > 1; g >>= 1)
+                if (ld % g == 0 && sb % g == 0 && (uintptr_t)ptr % (2 * g) == 0)
+                    return g;
+            return 1;
+        };
+        g.a_vec = granule(g.lda, g.a_sb, args->src);
+        g.b_vec = granule(g.ldb, g.b_sb, args->wei);
         launch_gemm_f16(g, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;

@@ -19,6 +19,8 @@
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
+#include <type_traits>
+
 namespace qmm {
 namespace {
 
@@ -42,27 +44,87 @@ QMM_D v4f mma16(const v8s &a, const v8s &b, const v4f &c) {
                 __builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
 }
 
-// eight neighbouring 16-bit elements p[0..7] of a row of `len` elements
-// starting at element `at`: one 16-byte load where the row allows it, else
-// element by element; elements at or past `len` (or a row that is not there)
-// read as zero
-QMM_D uint4 load8(const uint16_t *row, int64_t at, int64_t len, bool row_ok,
-        bool vec) {
-    if (row_ok && vec && at + 8 <= len) return *(const uint4 *)(row + at);
-    uint32_t w[4] = {0, 0, 0, 0};
-    if (row_ok) {
+// Eight neighbouring 16-bit elements of a row of `len` elements, starting at
+// element `at` (a multiple of 8), in two steps so that nothing touches the
+// loaded registers before the tile is staged. G (8, 2 or 1) elements per load:
+// row starts are multiples of 2 G bytes and `len` is a multiple of G, so a
+// piece of G elements is inside the row or past it, never across its end.
+// `request8` only issues the 8 / G loads, a piece past the end re-reading the
+// row's first one; `finish8` packs them and zeroes what is not there.
+template <int G>
+struct req8_t {
+    uint32_t w[G == 8 ? 4 : 8 / G];
+};
+
+template <int G>
+QMM_D void request8(req8_t<G> &r, const uint16_t *row, int at, int len) {
+    if constexpr (G == 8) {
+        const uint4 v = *(const uint4 *)(row + (at < len ? at : 0));
+        r.w[0] = v.x, r.w[1] = v.y, r.w[2] = v.z, r.w[3] = v.w;
+    } else if constexpr (G == 2) {
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            if (at + i < len) w[i / 2] |= (uint32_t)row[at + i] << (16 * (i % 2));
+        for (int j = 0; j < 4; j++)
+            r.w[j] = *(const uint32_t *)(row + (at + 2 * j < len ? at + 2 * j : 0));
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) r.w[j] = row[at + j < len ? at + j : 0];
+    }
+}
+
+template <int G>
+QMM_D uint4 finish8(const req8_t<G> &r, int at, int len, bool row_ok) {
+    uint32_t w[4];
+    if constexpr (G == 8) {
+        const bool ok = row_ok && at < len;
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = ok ? r.w[j] : 0u;
+    } else if constexpr (G == 2) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = row_ok && at + 2 * j < len ? r.w[j] : 0u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t lo = row_ok && at + 2 * j < len ? r.w[2 * j] : 0u;
+            const uint32_t hi = row_ok && at + 2 * j + 1 < len ? r.w[2 * j + 1] : 0u;
+            w[j] = lo | (hi << 16);
+        }
     }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <bool BF>
+constexpr int F16_AHEAD = 4; // steps between an operand's request and its staging
+
+template <int N, typename F>
+QMM_D void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1> {});
+    }
+}
+
+constexpr int F16_A_BYTES = F16_BM * F16_A_PITCH, F16_B_BYTES = F16_BK * F16_B_PITCH;
+constexpr int F16_OUT_PITCH = F16_BN + 4; // words of a staged dst row
+constexpr int F16_LDS_BYTES = 2 * (F16_A_BYTES + F16_B_BYTES) > F16_BM * F16_OUT_PITCH * 4
+        ? 2 * (F16_A_BYTES + F16_B_BYTES)
+        : F16_BM * F16_OUT_PITCH * 4;
+
+// LIGHT: nothing follows the accumulation but at most one relu / linear / clip
+// (what the attention products carry). Everything else goes through the
+// post-op interpreter, whose register needs halve the waves a SIMD can hold.
+QMM_HD bool light_epilogue(const epilogue_t &ep) {
+    if (ep.bias.ptr || ep.src_scale.ptr || ep.wei_scale.ptr || ep.dst_scale || ep.dst_zp)
+        return false;
+    if (ep.npo == 0) return true;
+    return ep.npo == 1 && ep.po[0].kind == pk_eltwise
+            && (ep.po[0].alg == alg_relu || ep.po[0].alg == alg_linear
+                    || ep.po[0].alg == alg_clip || ep.po[0].alg == alg_clip_v2);
+}
+
+template <bool BF, bool LIGHT, int GA, int GB>
 __global__ void __launch_bounds__(256)
 gemm_f16_kernel(const gemm16_params_t p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][F16_BM * F16_A_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][F16_BK * F16_B_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[F16_LDS_BYTES];
+    uint8_t *const lds_a = lds, *const lds_b = lds + 2 * F16_A_BYTES;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, c = lane >> 4;
@@ -75,34 +137,38 @@ gemm_f16_kernel(const gemm16_params_t p) {
     const int bk = tid >> 3, bn = (tid & 7) * 8;
     const bool a_row_ok = m0 + ar < p.M;
     const uint16_t *a_row = A + (int64_t)min(m0 + ar, p.M - 1) * p.lda;
-    const bool b_cols_ok = n0 + bn < p.N;
     const int steps = (p.K + F16_BK - 1) / F16_BK;
 
-    uint4 ra, rb;
-    auto request = [&](int kt) {
-        const int k0 = kt * F16_BK;
-        ra = load8(a_row, k0 + ak, p.K, a_row_ok, p.a_vec != 0);
-        const bool b_row_ok = k0 + bk < p.K && b_cols_ok;
-        rb = load8(B + (int64_t)min(k0 + bk, p.K - 1) * p.ldb, n0 + bn, p.N,
-                b_row_ok, p.b_vec != 0);
+    // operands are requested F16_AHEAD steps before they are staged: one slot
+    // of registers per step in flight, named statically (the loop is unrolled
+    // by the slot count)
+    req8_t<GA> ra[F16_AHEAD];
+    req8_t<GB> rb[F16_AHEAD];
+    auto request = [&](int kt, auto S) {
+        constexpr int sl = decltype(S)::value;
+        const int k0 = min(kt, steps - 1) * F16_BK; // past the end: a re-read nobody stages
+        request8<GA>(ra[sl], a_row, k0 + ak, p.K);
+        request8<GB>(rb[sl], B + (int64_t)min(k0 + bk, p.K - 1) * p.ldb, n0 + bn, p.N);
     };
-    auto stage = [&](int buf) {
-        *(uint4 *)(lds_a[buf] + ar * F16_A_PITCH + ak * 2) = ra;
-        *(uint4 *)(lds_b[buf] + bk * F16_B_PITCH + bn * 2) = rb;
+    auto stage = [&](int kt, auto S) {
+        constexpr int sl = decltype(S)::value;
+        const int k0 = kt * F16_BK, buf = kt & 1;
+        *(uint4 *)(lds_a + buf * F16_A_BYTES + ar * F16_A_PITCH + ak * 2)
+                = finish8<GA>(ra[sl], k0 + ak, p.K, a_row_ok);
+        *(uint4 *)(lds_b + buf * F16_B_BYTES + bk * F16_B_PITCH + bn * 2)
+                = finish8<GB>(rb[sl], n0 + bn, p.N, k0 + bk < p.K);
     };
 
     v4f acc[4];
 #pragma unroll
     for (int mf = 0; mf < 4; mf++) acc[mf] = v4f {0.f, 0.f, 0.f, 0.f};
 
-    request(0);
-    stage(0);
-    __syncthreads();
-    for (int kt = 0; kt < steps; kt++) {
+    auto step = [&](int kt, auto S) {
+        constexpr int sl = decltype(S)::value;
         const int buf = kt & 1;
-        if (kt + 1 < steps) request(kt + 1);
+        request(kt + F16_AHEAD, S); // the slot's tile kt was staged a step ago
         // weights fragment of the wave's 16 columns, transposed out of LDS
-        const uint8_t *vb = lds_b[buf] + (4 * c + (r >> 2)) * F16_B_PITCH
+        const uint8_t *vb = lds_b + buf * F16_B_BYTES + (4 * c + (r >> 2)) * F16_B_PITCH
                 + (16 * wave + 4 * (r & 3)) * 2;
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                 (v4s __attribute__((address_space(3))) *)vb);
@@ -112,38 +178,273 @@ gemm_f16_kernel(const gemm16_params_t p) {
 #pragma unroll
         for (int mf = 0; mf < 4; mf++) {
             // source fragment: row 16 mf + r, the same eight k
-            const uint8_t *pa = lds_a[buf] + (16 * mf + r) * F16_A_PITCH;
+            const uint8_t *pa = lds_a + buf * F16_A_BYTES + (16 * mf + r) * F16_A_PITCH;
             const v4s x = *(const v4s *)(pa + (4 * c) * 2);
             const v4s y = *(const v4s *)(pa + (16 + 4 * c) * 2);
             const v8s af = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
             acc[mf] = mma16<BF>(bf, af, acc[mf]);
         }
-        if (kt + 1 < steps) stage(buf ^ 1);
+        if (kt + 1 < steps)
+            stage(kt + 1, std::integral_constant<int, (sl + 1) % F16_AHEAD> {});
         __syncthreads();
-    }
+    };
 
-    // register i of lane (r, c): dst[m0 + 16 mf + r][n0 + 16 wave + 4 c + i]
-    const int n = n0 + 16 * wave + 4 * c;
+    static_for<F16_AHEAD>([&](auto S) { request(decltype(S)::value, S); });
+    stage(0, std::integral_constant<int, 0> {});
+    __syncthreads();
+    for (int kt = 0; kt < steps; kt += F16_AHEAD)
+        static_for<F16_AHEAD>([&](auto S) {
+            if (kt + decltype(S)::value < steps) step(kt + decltype(S)::value, S);
+        });
+
+    // register i of lane (r, c) is dst[m0 + 16 mf + r][n0 + 16 wave + 4 c + i].
+    // The tile goes through LDS so that 16 neighbouring lanes store one whole
+    // 64-column row piece instead of 16 rows with 8 bytes each.
+    float *out = (float *)lds;
 #pragma unroll
-    for (int mf = 0; mf < 4; mf++) {
-        const int m = m0 + 16 * mf + r;
+    for (int mf = 0; mf < 4; mf++)
+        *(v4f *)(out + (16 * mf + r) * F16_OUT_PITCH + 16 * wave + 4 * c) = acc[mf];
+    __syncthreads();
+    const int n = n0 + (tid & 15) * 4;
+    // one copy of the interpreter is enough; the light form is four stores
+#pragma unroll 1
+    for (int i = 0; i < 4; i++) {
+        const int row = 16 * i + (tid >> 4), m = m0 + row;
         if (m < p.M && n < p.N) {
-            float v[4] = {acc[mf][0], acc[mf][1], acc[mf][2], acc[mf][3]};
-            epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
+            const v4f t = *(const v4f *)(out + row * F16_OUT_PITCH + (tid & 15) * 4);
+            float v[4] = {t[0], t[1], t[2], t[3]};
+            if constexpr (LIGHT) {
+                if (p.ep.npo) {
+                    const int alg = p.ep.po[0].alg;
+                    const float al = p.ep.po[0].alpha, be = p.ep.po[0].beta,
+                                sc = p.ep.po[0].scale;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float e = alg == alg_relu ? eltwise_one<alg_relu>(v[j], al, be)
+                                : alg == alg_linear     ? eltwise_one<alg_linear>(v[j], al, be)
+                                : alg == alg_clip       ? eltwise_one<alg_clip>(v[j], al, be)
+                                                  : eltwise_one<alg_clip_v2>(v[j], al, be);
+                        v[j] = e * sc;
+                    }
+                }
+                epilogue_store4(p.ep, v, bz * p.ep.dst.sb + (int64_t)m * p.ep.dst.sm + n,
+                        min(4, p.N - n));
+            } else {
+                epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
+            }
         }
     }
+}
+
+// ---- few rows per batch (M <= 4): the decode-time attention products ---------
+// One token's scores (1 x 128 by 128 x keys) and context (1 x keys by
+// keys x 128) per head are a few MB of weights read once; a 64 x 64 MFMA tile
+// would leave most of the chip idle. Here a workgroup owns `cw` columns of one
+// batch entry: `tpr` neighbouring lanes cover a weights row of the chunk (V
+// elements each: one 16-byte load where rows are 16-byte granular and N is a
+// multiple of 8, else one element), the 256 / tpr lane groups take every
+// (256 / tpr)-th k, requests run one unrolled block ahead of the arithmetic,
+// the activations wait in LDS as f32, and the partial sums of the lane groups
+// meet through lane permutes (within a wave) and LDS (across the four waves).
+constexpr int GV_THREADS = 256;
+constexpr int GV_MAX_ACT = 8192; // staged activation elements (rows x K)
+
+template <bool BF>
+QMM_D float up16(uint32_t h) {
+    if constexpr (BF) return __builtin_bit_cast(float, h << 16);
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+template <bool BF, int V, int MR>
+__global__ void __launch_bounds__(GV_THREADS)
+gemv_f16_kernel(const gemm16_params_t p, const int tpr_log2) {
+    constexpr int U = V == 8 ? 8 : 16; // loads per lane and block
+    typedef typename std::conditional<V == 8, uint4, uint16_t>::type wv_t;
+    extern __shared__ __attribute__((aligned(16))) float gv_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tpr = 1 << tpr_log2, cw = tpr * V, rpp = GV_THREADS >> tpr_log2;
+    const int col_l = (tid & (tpr - 1)) * V, phase = tid >> tpr_log2;
+    const int n0 = blockIdx.x * cw, n = n0 + col_l;
+    const int64_t bz = blockIdx.y;
+    const int K = p.K;
+    float *qtab = gv_lds; // [MR][K]
+    float *red = gv_lds + MR * K; // [4][MR][cw]
+    const uint16_t *wcol = p.B + bz * p.b_sb + (n < p.N ? n : 0);
+
+    auto request = [&](wv_t (&w)[U], int kb) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = min(kb + u * rpp + phase, K - 1);
+            w[u] = *(const wv_t *)(wcol + (int64_t)k * p.ldb);
+        }
+    };
+    wv_t wc[U], wn[U];
+    request(wc, 0);
+
+    // activations -> f32 table; rows past M stay zero
+    const uint16_t *A = p.A + bz * p.a_sb;
+#pragma unroll
+    for (int m = 0; m < MR; m++) {
+        const bool row_ok = m < p.M;
+        const uint16_t *arow = A + (int64_t)(row_ok ? m : 0) * p.lda;
+        for (int k0 = 0; k0 < K; k0 += 4 * GV_THREADS) {
+            uint16_t t[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                t[j] = arow[min(k0 + j * GV_THREADS + tid, K - 1)];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int k = k0 + j * GV_THREADS + tid;
+                if (k < K) qtab[m * K + k] = row_ok ? up16<BF>(t[j]) : 0.f;
+            }
+        }
+    }
+    __syncthreads();
+
+    float acc[MR][V];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int i = 0; i < V; i++) acc[m][i] = 0.f;
+
+    const int block = U * rpp;
+    for (int kb = 0; kb < K; kb += block) {
+        request(wn, min(kb + block, K - 1)); // clamped: past K it re-reads the last row
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = kb + u * rpp + phase;
+            const bool ok = k < K;
+            float q[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++) q[m] = ok ? qtab[m * K + min(k, K - 1)] : 0.f;
+            float wf[V];
+            if constexpr (V == 8) {
+                const uint32_t d[4] = {wc[u].x, wc[u].y, wc[u].z, wc[u].w};
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    wf[i] = up16<BF>((d[i / 2] >> (16 * (i % 2))) & 0xffffu);
+            } else {
+                wf[0] = up16<BF>(wc[u]);
+            }
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const float w = ok ? wf[i] : 0.f; // a clamped re-read counts as zero
+#pragma unroll
+                for (int m = 0; m < MR; m++) acc[m][i] = fmaf(q[m], w, acc[m][i]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) wc[u] = wn[u];
+    }
+
+    // lanes l, l + tpr, l + 2 tpr ... of a wave hold the same columns
+    for (int s = tpr; s < 64; s <<= 1) {
+#pragma unroll
+        for (int m = 0; m < MR; m++)
+#pragma unroll
+            for (int i = 0; i < V; i++) acc[m][i] += __shfl_xor(acc[m][i], s);
+    }
+    if (lane < tpr) {
+#pragma unroll
+        for (int m = 0; m < MR; m++)
+#pragma unroll
+            for (int i = 0; i < V; i++)
+                red[(wave * MR + m) * cw + col_l + i] = acc[m][i];
+    }
+    __syncthreads();
+    const int quads = cw >> 2;
+    if (tid < MR * quads) {
+        const int m = tid / quads, c4 = (tid - m * quads) * 4;
+        const int nn = n0 + c4;
+        if (m < p.M && nn < p.N) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float t = 0.f;
+#pragma unroll
+                for (int w = 0; w < 4; w++) t += red[(w * MR + m) * cw + c4 + i];
+                v[i] = t;
+            }
+            epilogue_apply_store4(p.ep, v, bz, m, nn, min(4, p.N - nn));
+        }
+    }
+}
+
+template <bool BF, int V, int MR>
+void launch_gemv_f16_as(const gemm16_params_t &p, int tpr_log2, hipStream_t stream) {
+    const int cw = (1 << tpr_log2) * V;
+    const size_t lds = sizeof(float) * ((size_t)MR * p.K + 4 * MR * cw);
+    hipLaunchKernelGGL((gemv_f16_kernel<BF, V, MR>),
+            dim3((unsigned)((p.N + cw - 1) / cw), (unsigned)p.batch),
+            dim3(GV_THREADS), lds, stream, p, tpr_log2);
 }
 
 } // namespace
 
 void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return;
+    const int mr = p.M == 1 ? 1 : 4;
+    if (p.M <= 4 && (int64_t)mr * p.K <= GV_MAX_ACT) {
+        // vector loads need whole 8-column chunks inside N as well
+        const bool vec = p.b_vec == 8 && p.N % 8 == 0;
+        int tpr_log2 = 6; // one element per lane: 64 columns per workgroup
+        if (vec) {
+            // the widest chunk (32 .. 256 columns) that still gives 256 workgroups
+            tpr_log2 = 5;
+            while (tpr_log2 > 2
+                    && ((int64_t)p.batch * ((p.N + (8 << tpr_log2) - 1) >> (tpr_log2 + 3)) < 256
+                            || (4 << tpr_log2) >= p.N))
+                tpr_log2--;
+        }
+        auto go = [&](auto bf, auto v) {
+            if (mr == 1)
+                launch_gemv_f16_as<decltype(bf)::value, decltype(v)::value, 1>(
+                        p, tpr_log2, stream);
+            else
+                launch_gemv_f16_as<decltype(bf)::value, decltype(v)::value, 4>(
+                        p, tpr_log2, stream);
+        };
+        auto by_bf = [&](auto v) {
+            if (p.bf) go(std::true_type {}, v);
+            else go(std::false_type {}, v);
+        };
+        if (vec) by_bf(std::integral_constant<int, 8> {});
+        else by_bf(std::integral_constant<int, 1> {});
+        return;
+    }
     const dim3 grid((unsigned)((p.N + F16_BN - 1) / F16_BN),
             (unsigned)((p.M + F16_BM - 1) / F16_BM), (unsigned)p.batch);
-    if (p.bf)
-        hipLaunchKernelGGL(gemm_f16_kernel<true>, grid, dim3(256), 0, stream, p);
-    else
-        hipLaunchKernelGGL(gemm_f16_kernel<false>, grid, dim3(256), 0, stream, p);
+    // loads of 8, 2 or 1 elements: the granule has to divide the row length too
+    auto pick = [](int g, int len) { return g >= 8 && len % 8 == 0 ? 8 : g >= 2 && len % 2 == 0 ? 2 : 1; };
+    int ga = pick(p.a_vec, p.K), gb = pick(p.b_vec, p.N);
+    const bool light = light_epilogue(p.ep) && p.ep.dst.sn == 1;
+    if (!light && !(ga == 8 && gb == 8)) ga = gb = 1; // the interpreter form exists twice
+    auto go = [&](auto bf, auto lt, auto a, auto b) {
+        hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
+                                   decltype(a)::value, decltype(b)::value>),
+                grid, dim3(256), 0, stream, p);
+    };
+    auto by_bf = [&](auto lt, auto a, auto b) {
+        if (p.bf) go(std::true_type {}, lt, a, b);
+        else go(std::false_type {}, lt, a, b);
+    };
+    using I8 = std::integral_constant<int, 8>;
+    using I2 = std::integral_constant<int, 2>;
+    using I1 = std::integral_constant<int, 1>;
+    if (!light) {
+        if (ga == 8) by_bf(std::false_type {}, I8 {}, I8 {});
+        else by_bf(std::false_type {}, I1 {}, I1 {});
+        return;
+    }
+    auto by_b = [&](auto a) {
+        if (gb == 8) by_bf(std::true_type {}, a, I8 {});
+        else if (gb == 2) by_bf(std::true_type {}, a, I2 {});
+        else by_bf(std::true_type {}, a, I1 {});
+    };
+    if (ga == 8) by_b(I8 {});
+    else if (ga == 2) by_b(I2 {});
+    else by_b(I1 {});
 }
 
 } // namespace qmm

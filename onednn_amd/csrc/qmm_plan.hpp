@@ -171,7 +171,7 @@ struct gemm16_params_t {
     int64_t lda, a_sb, ldb, b_sb; // elements
     int32_t M, N, K, batch;
     int32_t bf; // bf16 (else f16)
-    int32_t a_vec, b_vec; // rows and base on 16-byte boundaries: vector loads
+    int32_t a_vec, b_vec; // elements per aligned load the rows allow: 8, 4, 2 or 1
     int32_t pad_;
     epilogue_t ep;
 };

@@ -51,6 +51,14 @@ CASES = {
     "prefill_context_k198": dict(sd=[1, 4, 198, 198], wd=[1, 4, 198, 128]),
     "two_dims_bf16_f32_dst": dict(sd=[70, 256], wd=[256, 100], code=dt.bf16, dst_dt=dt.f32),
     "broadcast_weights_bias": dict(sd=[3, 2, 33, 64], wd=[1, 1, 64, 72], bias=True),
+    # M <= 4 per batch entry runs the lane-per-column kernel instead of the MFMA tile
+    "decode_scores_n1000_vector": dict(sd=[1, 8, 1, 128], wd=[1, 8, 128, 1000]),
+    "decode_scores_bf16": dict(sd=[1, 8, 1, 128], wd=[1, 8, 128, 1001], code=dt.bf16),
+    "three_rows_vector": dict(sd=[2, 6, 3, 200], wd=[2, 6, 200, 264], bias=True),
+    "four_rows_scalar_f32_dst": dict(sd=[5, 4, 2043], wd=[5, 2043, 77], dst_dt=dt.f32),
+    "two_rows_narrow": dict(sd=[3, 2, 64], wd=[3, 64, 8]),
+    "one_row_long_k": dict(sd=[1, 8192], wd=[8192, 520]),
+    "two_rows_k_past_the_table": dict(sd=[2, 4100], wd=[4100, 96]),
     "tiny_k": dict(sd=[2, 5, 8], wd=[2, 8, 16]),
     "odd_everything": dict(sd=[2, 67, 45], wd=[2, 45, 51]),
 }
