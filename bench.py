@@ -183,7 +183,7 @@ def main():
                                # what the reference's own CPU implementation reached where it could be built and run:
                                # a different, smaller host than the one timed here, quoted for scale only
                                "reference_brgemm_elsewhere": {
-                                   "where": "survey container, 8 vCPU, isa avx10_1_512_amx (brg_matmul:avx10_1_512_amx), benchdnn",
+                                   "where": "a CPU-only container (8 vCPU) where the reference was built, isa avx10_1_512_amx (brg_matmul:avx10_1_512_amx), benchdnn",
                                    "config2_TOPs": 11.3, "config1_TOPs": 17.7, "config4_TOPs": 1.9,
                                    "decode_common_zp_M1_ms": 20.1,
                                    "note": "config 2 there ran with one common src scale: the reference's brgemm has no "

@@ -50,8 +50,11 @@ for v in (1, 2, 3, 4, 5, 6):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
 for v in (1, 2, 3, 4, 5, 6, 7, 8, 9):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))
+# the tiled decompression kernel per activation type and weights width
+for v in (0, 1, 2, 3):
+    UNITS.append(("qmm_gemm_w4f.hip", "_p%d" % v, ["-DQMM_W4F_PART=%d" % v]))
 # longest first, so that the pool finishes together
-UNITS.sort(key=lambda u: 0 if "w4a8" in u[0] else (1 if u[1] else 2))
+UNITS.sort(key=lambda u: 0 if "w4a8" in u[0] or ("w4f" in u[0] and u[1]) else (1 if u[1] else 2))
 
 
 def _compile(unit):

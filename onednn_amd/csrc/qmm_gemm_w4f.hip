@@ -22,7 +22,12 @@
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
+// The kernel is instantiated per activation type and weights width in
+// translation units of their own (QMM_W4F_PART = 0..3: bit 0 f16 activations,
+// bit 1 8-bit weights), so that they compile in parallel; the unit without the
+// macro holds the launcher that picks one.
 namespace qmm {
+#if defined(QMM_W4F_PART)
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -31,7 +36,6 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 constexpr int WF_WAVES = 8;
-constexpr int WF_BN = 32 * WF_WAVES;
 constexpr int WF_PITCH = 256 + 16; // bytes of a staged activation row
 
 template <bool F16>
@@ -52,15 +56,17 @@ QMM_D uint4 ld_stream(const uint8_t *ptr) {
 }
 
 // flags_m / shifts: as gemv_w4_fast_kernel (qmm_gemv_w4.hip)
-template <bool F16, bool WSIGNED, bool W8, int BM>
+// BM rows (32 or 64) x 16 * CBW * 8 columns per workgroup; CBW = 1 where the
+// problem has too few columns to fill the chip with 256-column blocks
+template <bool F16, bool WSIGNED, bool W8, int BM, int CBW>
 __global__ void __launch_bounds__(WF_WAVES * 64)
 gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     constexpr int RB = BM / 16; // row blocks of the MFMA
     constexpr int NP = W8 ? 2 : 1;
     constexpr int TILE_BYTES = 1024 * NP;
     // two activation buffers; after the k loop the same bytes stage the results
-    constexpr int A_BUF = BM * WF_PITCH, STG_PITCH = 36; // floats per staged row
-    constexpr int STG_WAVE = 32 * STG_PITCH * 4; // 32 rows x 32 columns of a wave
+    constexpr int A_BUF = BM * WF_PITCH, STG_PITCH = 16 * CBW + 4; // floats per staged row
+    constexpr int STG_WAVE = 32 * STG_PITCH * 4; // 32 rows x the wave's columns
     constexpr int LDS_BYTES
             = 2 * A_BUF > WF_WAVES * STG_WAVE ? 2 * A_BUF : WF_WAVES * STG_WAVE;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
@@ -71,7 +77,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     const int N = p.N, K = p.K, M = p.M;
     const int m0 = blockIdx.y * BM;
     const int nb16 = p.nb16, tiles = p.kg128;
-    const int nb0 = (blockIdx.x * WF_WAVES + wave) * 2; // first 16-column block
+    const int nb0 = (blockIdx.x * WF_WAVES + wave) * CBW; // first 16-column block
     const int gs_shift = (int8_t)(shifts & 0xff), gz_shift = (int8_t)(shifts >> 8);
     const bool scale_per_n = flags_m & 1, zp_per_n = flags_m & 2;
     const bool zp4 = flags_m & 4, zp_signed = flags_m & 8, sc_f16 = flags_m & 16;
@@ -90,13 +96,13 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
     constexpr uint32_t NIB = 0x000F000Fu;
 
     // column blocks past the last one repeat it and are never stored
-    const uint8_t *Bt[2];
-    const uint16_t *scn[2];
-    int zcol[2];
+    const uint8_t *Bt[CBW];
+    const uint16_t *scn[CBW];
+    int zcol[CBW];
     const int64_t sN = scale_per_n ? N : 0, zN = zp_per_n ? N : 0;
     const uint8_t *pZP = p.zps ? (const uint8_t *)p.zps : p.B;
 #pragma unroll
-    for (int cb = 0; cb < 2; cb++) {
+    for (int cb = 0; cb < CBW; cb++) {
         Bt[cb] = p.B + ((int64_t)min(nb0 + cb, nb16 - 1) * tiles) * TILE_BYTES
                 + lane * 16;
         const int nn = min((nb0 + cb) * 16 + r, N - 1);
@@ -116,16 +122,16 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         a_src[i] = p.A + (int64_t)min(m0 + a_row + WF_WAVES * 4 * i, M - 1) * p.lda;
     // two request slots: a tile's operands are asked for two k tiles before
     // they are used (one k tile of arithmetic is shorter than a trip to memory)
-    uint4 a_reg[2][A_LD], wt[2][2][NP];
+    uint4 a_reg[2][A_LD], wt[2][CBW][NP];
     // kept in their storage types: widening them here would make the request
     // wait for the values
-    uint16_t scp[2][2];
-    uint8_t zpp[2][2];
+    uint16_t scp[2][CBW];
+    uint8_t zpp[2][CBW];
     auto request = [&](int kt, auto slot_tag) { // global -> registers, tile kt
         constexpr int sl = decltype(slot_tag)::value;
         const int tc = min(kt, tiles - 1);
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
+        for (int cb = 0; cb < CBW; cb++)
 #pragma unroll
             for (int pl = 0; pl < NP; pl++)
                 wt[sl][cb][pl] = ld_stream(
@@ -138,18 +144,18 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
         const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
+        for (int cb = 0; cb < CBW; cb++) {
             scp[sl][cb] = scn[cb][(int64_t)gsc * sN];
             const int64_t zi = has_zp ? (int64_t)gzp * zN + zcol[cb] : 0;
             zpp[sl][cb] = pZP[zp4 ? zi >> 1 : zi];
         }
     };
 
-    v4f out[RB][2];
+    v4f out[RB][CBW];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) out[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
+        for (int cb = 0; cb < CBW; cb++) out[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
 
     // one k tile; its operands sit in request slot kt % 2 (= LDS buffer)
     auto k_tile = [&](int kt, auto slot_tag) {
@@ -161,11 +167,11 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         for (int i = 0; i < A_LD; i++)
             *(uint4 *)(lds_a[sl] + (a_row + WF_WAVES * 4 * i) * WF_PITCH + a_chunk * 16)
                     = past_k ? make_uint4(0, 0, 0, 0) : a_reg[sl][i];
-        uint4 w_cur[2][NP];
-        uint16_t sc_cur[2];
-        uint8_t zp_cur[2];
+        uint4 w_cur[CBW][NP];
+        uint16_t sc_cur[CBW];
+        uint8_t zp_cur[CBW];
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
+        for (int cb = 0; cb < CBW; cb++) {
 #pragma unroll
             for (int pl = 0; pl < NP; pl++) w_cur[cb][pl] = wt[sl][cb][pl];
             sc_cur[cb] = scp[sl][cb];
@@ -177,20 +183,20 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         // branch around the loads makes the compiler wait for them at its end
         request(kt + 2, slot_tag);
 
-        v4f Pu[RB][2], Su[RB];
+        v4f Pu[RB][CBW], Su[RB];
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             Su[rb] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++) {
+            for (int cb = 0; cb < CBW; cb++) {
                 Pu[rb][cb] = v4f {0.f, 0.f, 0.f, 0.f};
             }
         }
 #pragma unroll
         for (int s4 = 0; s4 < 4; s4++) {
-            v4u b[2], bl[2];
+            v4u b[CBW], bl[CBW];
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++) {
+            for (int cb = 0; cb < CBW; cb++) {
                 const uint32_t d = (s4 == 0 ? w_cur[cb][0].x
                                 : s4 == 1   ? w_cur[cb][0].y
                                 : s4 == 2   ? w_cur[cb][0].z
@@ -219,7 +225,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                         + (16 * rb + r) * WF_PITCH + (32 * s4 + 8 * c) * 2);
                 const v4u a = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int cb = 0; cb < 2; cb++) {
+                for (int cb = 0; cb < CBW; cb++) {
                     Pu[rb][cb] = mfma16<F16>(a, b[cb], Pu[rb][cb]);
                     if constexpr (W8)
                         Pu[rb][cb] = mfma16<F16>(a, bl[cb], Pu[rb][cb]);
@@ -229,7 +235,7 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         }
         const int gzp = gz_shift < 0 ? 0 : kt >> gz_shift;
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
+        for (int cb = 0; cb < CBW; cb++) {
             const float sc = sc_f16
                     ? (float)__builtin_bit_cast(_Float16, sc_cur[cb])
                     : u2f((uint32_t)sc_cur[cb] << 16);
@@ -256,22 +262,23 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         if (kt + 1 < tiles) k_tile(kt + 1, std::integral_constant<int, 1> {});
     }
 
-    // Epilogue: the wave's 64 x 32 results go through a wave-private LDS tile,
-    // 32 rows at a time, and come back as four neighbouring columns of a row
-    // per lane, so that bias / post-ops / dst conversion exist once and every
-    // store is a vector. MFMA output: register j of lane l is row
-    // 4 * (l / 16) + j, column l % 16.
+    // Epilogue: the wave's results go through a wave-private LDS tile, 32 rows
+    // at a time, and come back as four neighbouring columns of a row per lane,
+    // so that bias / post-ops / dst conversion exist once and every store is a
+    // vector. MFMA output: register j of lane l is row 4 * (l / 16) + j,
+    // column l % 16.
     __syncthreads(); // every wave is done with the activation buffers
     float *const stg = (float *)(lds_raw + wave * STG_WAVE);
     const int n_w = nb0 * 16; // the wave's first column
-    static_assert(RB == 4, "two halves of 32 rows");
+    static_assert(RB == 2 || RB == 4, "halves of 32 rows");
+    constexpr int QPR = 4 * CBW; // lanes (four columns each) per staged row
     auto flush = [&](auto h_tag) { // rows 32 h .. 32 h + 31 (h a constant:
         // the accumulators must stay in registers)
         constexpr int h = decltype(h_tag)::value;
 #pragma unroll
         for (int rb2 = 0; rb2 < 2; rb2++)
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++)
+            for (int cb = 0; cb < CBW; cb++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     stg[(16 * rb2 + 4 * c + j) * STG_PITCH + 16 * cb + r]
@@ -279,8 +286,8 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         // (wave-private: the LDS writes above are ordered before the reads
         // below by the compiler's waitcnt, no barrier needed)
 #pragma unroll 1
-        for (int it = 0; it < 4; it++) {
-            const int row = it * 8 + (lane >> 3), cg = (lane & 7) * 4;
+        for (int it = 0; it < 32 * QPR / 64; it++) {
+            const int row = it * (64 / QPR) + lane / QPR, cg = (lane % QPR) * 4;
             const float4 t = *(const float4 *)&stg[row * STG_PITCH + cg];
             const int m = m0 + 32 * h + row, n = n_w + cg;
             if (m < M && n < N) {
@@ -290,42 +297,78 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         }
     };
     flush(std::integral_constant<int, 0> {});
-    flush(std::integral_constant<int, 1> {});
+    if constexpr (RB == 4) flush(std::integral_constant<int, 1> {});
 }
 
 } // namespace
 
-// many rows (the caller decides), fast-variant attribute set (the caller
-// checks); flags_m and shifts as for gemv_w4_fast_kernel
-void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
+// Which shape a problem runs as: 64 x 256 blocks where they fill at least half
+// the chip, else 128-column blocks of 32 or 64 rows.
+static void w4f_shape(const gemv_params_t &p, int &bm, int &cbw) {
+    const int64_t wide = (int64_t)((p.M + 63) / 64) * ((p.N + 255) / 256);
+    cbw = p.M > 64 && wide >= 128 ? 2 : 1;
+    bm = cbw == 1 && p.M <= 32 ? 32 : 64;
+}
+
+#define QMM_W4F_NAME2(n) launch_gemm_w4f_part##n
+#define QMM_W4F_NAME(n) QMM_W4F_NAME2(n)
+void QMM_W4F_NAME(QMM_W4F_PART)(const gemv_params_t &p, int shifts, int flags_m,
         hipStream_t stream) {
-    const dim3 grid((unsigned)((p.N + WF_BN - 1) / WF_BN),
-            (unsigned)((p.M + 63) / 64));
+    int bm, cbw;
+    w4f_shape(p, bm, cbw);
+    const int bn = 16 * cbw * WF_WAVES;
+    const dim3 grid((unsigned)((p.N + bn - 1) / bn), (unsigned)((p.M + bm - 1) / bm));
     auto go = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, dim3(WF_WAVES * 64), 0, stream, p, shifts,
                 flags_m);
     };
-    auto by_bm = [&](auto f16, auto sgn, auto w8) {
-        constexpr bool F = decltype(f16)::value, S = decltype(sgn)::value,
-                       W = decltype(w8)::value;
-        go(gemm_w4f_kernel<F, S, W, 64>);
+    constexpr bool F = (QMM_W4F_PART & 1) != 0, W = (QMM_W4F_PART & 2) != 0;
+    auto by_bm = [&](auto sgn) {
+        constexpr bool S = decltype(sgn)::value;
+        if (cbw == 2) go(gemm_w4f_kernel<F, S, W, 64, 2>);
+        else if (bm == 64) go(gemm_w4f_kernel<F, S, W, 64, 1>);
+        else go(gemm_w4f_kernel<F, S, W, 32, 1>);
     };
-    auto by_w8 = [&](auto f16, auto sgn) {
-        if (p.w8)
-            by_bm(f16, sgn, std::true_type {});
-        else
-            by_bm(f16, sgn, std::false_type {});
-    };
-    auto by_sign = [&](auto f16) {
-        if (p.wei_signed)
-            by_w8(f16, std::true_type {});
-        else
-            by_w8(f16, std::false_type {});
-    };
-    if (p.act_f16)
-        by_sign(std::true_type {});
-    else
-        by_sign(std::false_type {});
+    if (p.wei_signed) by_bm(std::true_type {});
+    else by_bm(std::false_type {});
 }
+
+#else // the launcher
+
+void launch_gemm_w4f_part0(const gemv_params_t &, int, int, hipStream_t);
+void launch_gemm_w4f_part1(const gemv_params_t &, int, int, hipStream_t);
+void launch_gemm_w4f_part2(const gemv_params_t &, int, int, hipStream_t);
+void launch_gemm_w4f_part3(const gemv_params_t &, int, int, hipStream_t);
+
+// Whether the tiled kernel is the better way to run p.M > 16 rows, against the
+// decode kernel once per block of 16 rows. Both walk K at about the same pace;
+// measured at K = 4096: a pass of the decode kernel over 4096 columns 4.3 us, a
+// round of 128-column workgroups 26 us (32 rows) or 40 us (64 rows).
+bool gemm_w4f_wins(const gemv_params_t &p) {
+    if (p.M <= 16) return false;
+    const int64_t wide = (int64_t)((p.M + 63) / 64) * ((p.N + 255) / 256);
+    if (p.M > 64 && wide >= 128) return true;
+    const int bm = p.M <= 32 ? 32 : 64;
+    const double wgs = (double)((p.M + bm - 1) / bm) * ((p.N + 127) / 128);
+    const double rounds = wgs <= 256 ? 1.0 : wgs / 256;
+    const double tiled = (bm == 32 ? 26.0 : 40.0) * rounds;
+    const double passes = (double)((p.M + 15) / 16) * 4.3 * p.N / 4096.0;
+    return tiled < passes;
+}
+
+// more than 16 rows (the caller decides with gemm_w4f_wins), fast-variant
+// attribute set (the caller checks); flags_m and shifts as for
+// gemv_w4_fast_kernel
+void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
+        hipStream_t stream) {
+    switch ((p.act_f16 ? 1 : 0) | (p.w8 ? 2 : 0)) {
+        case 0: launch_gemm_w4f_part0(p, shifts, flags_m, stream); break;
+        case 1: launch_gemm_w4f_part1(p, shifts, flags_m, stream); break;
+        case 2: launch_gemm_w4f_part2(p, shifts, flags_m, stream); break;
+        default: launch_gemm_w4f_part3(p, shifts, flags_m, stream); break;
+    }
+}
+
+#endif
 
 } // namespace qmm

@@ -558,6 +558,7 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
 
 void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
         hipStream_t stream);
+bool gemm_w4f_wins(const gemv_params_t &p);
 
 void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return;
@@ -619,11 +620,9 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         // an absent zero-point buffer is never dereferenced past its first
         // byte: the weights stand in for it
         const uint8_t *zp = p.zps ? (const uint8_t *)p.zps : p.B;
-        // Enough rows that blocks of 64 rows x 256 columns fill half the chip:
-        // the tiled kernel (a weights tile unpacked once for 64 rows). Below
-        // that, this kernel once per block of 16 rows keeps more CUs reading.
-        if (p.M > 64
-                && (int64_t)((p.M + 63) / 64) * ((p.N + 255) / 256) >= 128) {
+        // More than 16 rows: the tiled kernel (a weights tile unpacked once
+        // for 32 or 64 rows) where it beats this one once per block of 16 rows.
+        if (gemm_w4f_wins(p)) {
             launch_gemm_w4f(q, shifts, flags_m, stream);
             return;
         }

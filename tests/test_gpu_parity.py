@@ -736,13 +736,21 @@ TILED_CASES = {
     "f16_s4_no_zp_k_tail_f32_dst": dict(M=1090, K=328, N=2048, act_dt=dt.f16, wei_dt=dt.s4, with_zp=False, G=328,
                                         dst_dt=dt.f32, per_column=True),
     "bf16_s8_g128_zp_s8": dict(M=1100, K=256, N=2064, wei_dt=dt.s8, zp_dt=dt.s8, scale_dt=dt.bf16),
+    # fewer rows over many columns: blocks of 32 or 64 rows x 128 columns
+    "f16_u4_24_rows_wide": dict(M=24, K=256, N=12808, act_dt=dt.f16),
+    "bf16_u4_50_rows_wide": dict(M=50, K=384, N=9744),
+    "f16_u8_130_rows_per_column": dict(M=130, K=256, N=4616, act_dt=dt.f16, wei_dt=dt.u8, zp_dt=dt.u8,
+                                       per_column=True),
+    "f16_s4_32_rows_k_tail": dict(M=32, K=200, N=12800, act_dt=dt.f16, wei_dt=dt.s4, with_zp=False, G=200,
+                                  per_column=True),
 }
 
 
 @pytest.mark.parametrize("name", sorted(TILED_CASES))
 def test_decompression_at_many_rows(ctx, name):
-    """Enough rows for the tiled kernel (blocks of 64 rows x 256 columns, a weights tile unpacked once per block):
-    the prefill entries of the reference's LLM list (M = 1024 ... 1088) at a reduced K."""
+    """Shapes that take the tiled kernel (blocks of 64 rows x 256 columns, or 32 / 64 rows x 128 columns where rows are
+    few and columns many; a weights tile unpacked once per block): the prefill entries of the reference's LLM list
+    (M = 1024 ... 1088) and its 32-row entries over 14336 columns, at a reduced K."""
     eng, strm = ctx
     say("decode_w4 tiled %s" % name)
     kw = TILED_CASES[name]
