@@ -34,6 +34,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 
 constexpr int WF_WAVES = 8;
 constexpr int WF_PITCH = 256 + 16; // bytes of a staged activation row
@@ -183,6 +184,45 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
         // branch around the loads makes the compiler wait for them at its end
         request(kt + 2, slot_tag);
 
+        // scale and zero point of the tile's group, per column block
+        const int gzp = gz_shift < 0 ? 0 : kt >> gz_shift;
+        float sc[CBW], zp[CBW];
+#pragma unroll
+        for (int cb = 0; cb < CBW; cb++) {
+            sc[cb] = sc_f16 ? (float)__builtin_bit_cast(_Float16, sc_cur[cb])
+                            : u2f((uint32_t)sc_cur[cb] << 16);
+            const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol[cb]) & 1) : 0;
+            const int zbits = zp4 ? 4 : 8;
+            const uint32_t zraw
+                    = ((uint32_t)zp_cur[cb] >> (4 * odd)) & ((1u << zbits) - 1u);
+            const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
+            zp[cb] = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
+        }
+        // f16: the offsets leave the weights before the MFMA -- (1024 + w) -
+        // (1024 + z) and (16384 + 16 h) - 16384 are small integers, exact in a
+        // packed f16 subtraction -- so the products sum to a * (w - z) and no
+        // activation sums are needed. bf16 has no packed subtraction: there
+        // the sums S of the activations come from an MFMA against ones and the
+        // offsets leave in the fold, P - (offset + z) S.
+        uint32_t sub_hi[CBW], sub_lo[CBW];
+#pragma unroll
+        for (int cb = 0; cb < CBW; cb++) {
+            if constexpr (F16) {
+                const float lo = OFFSET + (W8 ? 0.f : soff) + zp[cb];
+                const float hi = W8 ? 16.f * OFFSET + 16.f * soff : lo;
+                const uint32_t l16 = __builtin_bit_cast(uint16_t, (_Float16)lo);
+                const uint32_t h16 = __builtin_bit_cast(uint16_t, (_Float16)hi);
+                sub_lo[cb] = l16 | (l16 << 16);
+                sub_hi[cb] = h16 | (h16 << 16);
+            } else {
+                sub_lo[cb] = sub_hi[cb] = 0;
+            }
+        }
+        auto pk_sub = [](uint32_t x, uint32_t y) {
+            return __builtin_bit_cast(uint32_t,
+                    __builtin_bit_cast(v2h, x) - __builtin_bit_cast(v2h, y));
+        };
+
         v4f Pu[RB][CBW], Su[RB];
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
@@ -206,6 +246,10 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                 b[cb].y = ((d >> 4) & NIB) | MAGIC_HI;
                 b[cb].z = ((d >> 8) & NIB) | MAGIC_HI;
                 b[cb].w = ((d >> 12) & NIB) | MAGIC_HI;
+                if constexpr (F16) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b[cb][e] = pk_sub(b[cb][e], sub_hi[cb]);
+                }
                 bl[cb] = b[cb];
                 if constexpr (W8) {
                     const uint32_t dl = s4 == 0 ? w_cur[cb][NP - 1].x
@@ -216,6 +260,11 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                     bl[cb].y = ((dl >> 4) & NIB) | MAGIC;
                     bl[cb].z = ((dl >> 8) & NIB) | MAGIC;
                     bl[cb].w = ((dl >> 12) & NIB) | MAGIC;
+                    if constexpr (F16) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            bl[cb][e] = pk_sub(bl[cb][e], sub_lo[cb]);
+                    }
                 }
             }
 #pragma unroll
@@ -230,29 +279,21 @@ gemm_w4f_kernel(const gemv_params_t p, const int shifts, const int flags_m) {
                     if constexpr (W8)
                         Pu[rb][cb] = mfma16<F16>(a, bl[cb], Pu[rb][cb]);
                 }
-                Su[rb] = mfma16<F16>(a, ones, Su[rb]);
+                if constexpr (!F16) Su[rb] = mfma16<F16>(a, ones, Su[rb]);
             }
         }
-        const int gzp = gz_shift < 0 ? 0 : kt >> gz_shift;
 #pragma unroll
         for (int cb = 0; cb < CBW; cb++) {
-            const float sc = sc_f16
-                    ? (float)__builtin_bit_cast(_Float16, sc_cur[cb])
-                    : u2f((uint32_t)sc_cur[cb] << 16);
-            const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol[cb]) & 1) : 0;
-            const int zbits = zp4 ? 4 : 8;
-            const uint32_t zraw
-                    = ((uint32_t)zp_cur[cb] >> (4 * odd)) & ((1u << zbits) - 1u);
-            const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
-            const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
-            const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp
-                                 : OFFSET + soff + zp;
+            const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp[cb]
+                                 : OFFSET + soff + zp[cb];
 #pragma unroll
             for (int rb = 0; rb < RB; rb++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    out[rb][cb][j] = __builtin_fmaf(sc,
-                            Pu[rb][cb][j] - off * Su[rb][j], out[rb][cb][j]);
+                    out[rb][cb][j] = F16
+                            ? __builtin_fmaf(sc[cb], Pu[rb][cb][j], out[rb][cb][j])
+                            : __builtin_fmaf(sc[cb],
+                                      Pu[rb][cb][j] - off * Su[rb][j], out[rb][cb][j]);
         }
     };
     request(0, std::integral_constant<int, 0> {});
