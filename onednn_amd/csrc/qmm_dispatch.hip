@@ -554,8 +554,9 @@ struct w4a8_small_plan_t {
 w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     w4a8_small_plan_t s;
     std::memset(&s, 0, sizeof(s));
-    s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0
-            && !w4a8_src_zp_mode(P.desc) && P.group_k >= 64;
+    // whole 64-k tiles per group, or groups of 32 k
+    const bool half = P.group_k == 32;
+    s.use = P.M <= W4A8_SMALL_MAX_M && variant == 0 && (P.group_k >= 64 || half);
     if (!s.use) return s;
     const int64_t ng = P.ngroups_k, tpg = P.group_k / 64;
     const int64_t nblk = (P.N + 127) / 128;
@@ -569,10 +570,12 @@ w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     if (want < 1) want = 1;
     if (want > ng) want = ng;
     int64_t gps = (ng + want - 1) / want;
+    if (half) gps = (gps + 1) / 2 * 2; // whole tiles per slice
     // a slice of at most one chunk of 16 tiles where the groups allow it
-    const int64_t one_chunk = 16 / tpg > 1 ? 16 / tpg : 1;
+    const int64_t one_chunk = half ? 32 : (16 / tpg > 1 ? 16 / tpg : 1);
     if (gps > one_chunk) gps = one_chunk;
-    if (gps > W4A8_SMALL_MAX_GPS) gps = W4A8_SMALL_MAX_GPS;
+    const int64_t max_gps = (half ? 2 : 1) * W4A8_SMALL_MAX_GPS;
+    if (gps > max_gps) gps = max_gps;
     s.gps = (int)gps;
     s.splits = (int)((ng + gps - 1) / gps);
     s.ldp = (int)round_up(P.N, 4);
@@ -1127,8 +1130,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             q.c2T = (int32_t *)(arrays + sc.c2_off);
         }
         const w4a8_small_plan_t sm = w4a8_small_plan(P, w4a8_variant);
-        // the single-token kernel also takes groups of 32 k and source zero
-        // points / u8 sources (which the split-K kernel does not)
+        // the single-token kernel where the split-K kernel is not used
         const bool tiny_only = !sm.use && w4a8_variant == 0 && P.M <= 4
                 && (sc.src_zp || q.gk == 32);
         if ((sm.use || tiny_only) && gemm_w4a8_small_takes(q)) {

@@ -541,15 +541,32 @@ __global__ void __launch_bounds__(256) w4a8_prep_kernel(const w4a8_prep_t p) {
 constexpr int SM_CH = 16; // 64-k tiles per chunk
 
 // HAS_ZP: zero points or u4 weights (row-sum path); ZPK: 0 = no zero-point
-// buffer (the constant u4 offset only), else its storage class.
-template <int FM, int SC, bool HAS_ZP, int ZPK>
+// buffer (the constant u4 offset only), else its storage class. MODE 1: groups
+// of 32 k (p.tpg == 0): every MFMA is a group of its own, twice the groups per
+// slice. MODE 2: source zero points / u8 source (with HAS_ZP), as in the
+// single-token kernel below: the source bytes are flipped to s8, the column
+// sums of the stored nibbles come from dot products of the weights operand
+// with ones, and the group end adds z_s' * -(16 sum w' + group * zw).
+constexpr int sm_maxg(int mode) { // groups per slice
+    return mode == 1 ? 2 * W4A8_SMALL_MAX_GPS : W4A8_SMALL_MAX_GPS;
+}
+constexpr size_t sm_lds_bytes(int fm, int mode) {
+    return (size_t)SM_CH * fm * 32 * BK
+            + (size_t)sm_maxg(mode) * (fm * 32 * 4 * (mode == 2 ? 2 : 1) + 128 * 4 + 128 * 4)
+            + 4 * fm * 32 * 4;
+}
+
+template <int FM, int SC, bool HAS_ZP, int ZPK, int MODE = 0>
 __global__ void __launch_bounds__(256)
 w4a8_small_kernel(const w4a8_small_t p) {
+    constexpr bool HALF = MODE == 1, SZP = MODE == 2;
+    static_assert(!SZP || HAS_ZP, "");
     constexpr int BM = FM * 32, BN = 128, NT = 256;
-    constexpr int MAXG = W4A8_SMALL_MAX_GPS;
+    constexpr int MAXG = sm_maxg(MODE);
     constexpr int A_BYTES = SM_CH * BM * BK; // [tile][row][64 B], swizzled
     constexpr int SS_OFF = A_BYTES;
-    constexpr int SW_OFF = SS_OFF + MAXG * BM * 4;
+    constexpr int ZS_OFF = SS_OFF + MAXG * BM * 4; // SZP only
+    constexpr int SW_OFF = ZS_OFF + (SZP ? MAXG * BM * 4 : 0);
     constexpr int ZW_OFF = SW_OFF + MAXG * BN * 4;
     constexpr int RS_OFF = ZW_OFF + MAXG * BN * 4; // [4 waves][BM] s32
     constexpr int A_PER = SM_CH * BM * 4 / NT; // 16-byte pieces per thread
@@ -563,10 +580,10 @@ w4a8_small_kernel(const w4a8_small_t p) {
     const int n0 = blockIdx.x * BN;
     const int m0 = blockIdx.z * BM;
     const int split = blockIdx.y;
-    const int g_begin = split * p.gps;
+    const int g_begin = split * p.gps; // p.gps is even with groups of 32 k
     const int g_cnt = min(p.gps, q.ng - g_begin);
-    const int T0 = g_begin * p.tpg; // first 64-k tile of the slice
-    const int KT = g_cnt * p.tpg; // tiles of this workgroup
+    const int T0 = HALF ? g_begin / 2 : g_begin * p.tpg; // first 64-k tile of the slice
+    const int KT = HALF ? g_cnt / 2 : g_cnt * p.tpg; // tiles of this workgroup
 
     // Request order = order of use: source rows, scales, then the weights tile
     // by tile, so that every wait below leaves the younger requests in flight.
@@ -607,12 +624,12 @@ w4a8_small_kernel(const w4a8_small_t p) {
     load_rows(0, min(SM_CH, KT));
     // scales and zero points of the slice (f32 / s32 in LDS, [group][row or
     // column]): all loads of a thread before the first conversion
-    uint32_t rs_[SS_PER], rw_[SW_PER], rz_[SW_PER];
+    uint32_t rs_[SS_PER], rzs_[SS_PER], rw_[SW_PER], rz_[SW_PER];
     int64_t iz_[SW_PER];
     const bool has_ss = q.ss != nullptr, has_sw = q.sw != nullptr;
 #pragma unroll
     for (int j = 0; j < SS_PER; j++)
-        rs_[j] = 0;
+        rs_[j] = rzs_[j] = 0;
 #pragma unroll
     for (int j = 0; j < SW_PER; j++) {
         rw_[j] = rz_[j] = 0;
@@ -626,6 +643,18 @@ w4a8_small_kernel(const w4a8_small_t p) {
             const int k0 = (g_begin + gl) * q.gk;
             const int m = min(m0 + r, q.M - 1);
             rs_[j] = scale_raw<SC>(q.ss, m * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
+        }
+    }
+    if constexpr (SZP) {
+        if (q.zs) { // one byte per value: s8 or u8 (host-checked)
+#pragma unroll
+            for (int j = 0; j < SS_PER; j++) {
+                const int i = tid + j * NT;
+                const int gl = min(i / BM, g_cnt - 1), r = i % BM;
+                const int k0 = (g_begin + gl) * q.gk;
+                const int m = min(m0 + r, q.M - 1);
+                rzs_[j] = ((const uint8_t *)q.zs)[m * q.zs_sm + (k0 / q.zs_g) * q.zs_sk];
+            }
         }
     }
     if (has_sw) {
@@ -660,7 +689,15 @@ w4a8_small_kernel(const w4a8_small_t p) {
         for (int j = 0; j < SS_PER; j++) {
             const int i = tid + j * NT;
             const float v = scale_value<SC>(q.ss_dt, rs_[j]);
-            if (i < g_cnt * BM) ssl[i] = has_ss ? v : 1.f;
+            if (i < g_cnt * BM) {
+                ssl[i] = has_ss ? v : 1.f;
+                if constexpr (SZP) {
+                    const int z = !q.zs      ? 0
+                            : q.zs_dt == dt_s8 ? (int)(int8_t)rzs_[j]
+                                               : (int)rzs_[j];
+                    ((int32_t *)(lds + ZS_OFF))[i] = z - (q.a_flip ? 128 : 0);
+                }
+            }
         }
 #pragma unroll
         for (int j = 0; j < SW_PER; j++) {
@@ -681,7 +718,7 @@ w4a8_small_kernel(const w4a8_small_t p) {
 
     v16i acc[FM];
     v16f res[FM];
-    int rsum[FM];
+    int rsum[FM], csum = 0;
 #pragma unroll
     for (int i = 0; i < FM; i++) {
         rsum[i] = 0;
@@ -695,8 +732,66 @@ w4a8_small_kernel(const w4a8_small_t p) {
     const float *swl = (const float *)(lds + SW_OFF);
     const int32_t *zwl = (const int32_t *)(lds + ZW_OFF);
     int32_t *rsw = (int32_t *)(lds + RS_OFF) + wave * BM;
+    const int32_t *zsl = (const int32_t *)(lds + ZS_OFF);
     int t_in_g = 0, gl = 0; // position of the next tile in its group; the group
     const int mrows = min(BM, q.M - m0);
+    // group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+    auto group_end = [&]() {
+        const float sw = swl[gl * BN + wave * 32 + (lane & 31)];
+        int zw = 0, c2 = 0;
+        if constexpr (HAS_ZP) {
+            zw = zwl[gl * BN + wave * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                // both k halves of a row: lanes l and l ^ 32
+                const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
+                rsw[i * 32 + (lane & 31)] = tot;
+                rsum[i] = 0;
+            }
+        }
+        if constexpr (SZP) {
+            // the column's 16 * sum w' of the group, both k halves
+            const int ctot = csum + __shfl_xor(csum, 32);
+            csum = 0;
+            c2 = -ctot - q.gk * zw;
+        }
+#pragma unroll
+        for (int i = 0; i < FM; i++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                // registers 4c..4c+3 are rows 8c..8c+7 of the fragment: skip
+                // those past the last row
+                if (i * 32 + 8 * c >= mrows) continue;
+                const int row = i * 32 + 8 * c + 4 * (lane >> 5);
+                const float4 s4 = *(const float4 *)&ssl[gl * BM + row];
+                const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+                int rs[4] = {0, 0, 0, 0}, zs[4] = {0, 0, 0, 0};
+                if constexpr (HAS_ZP) {
+                    const int4 r4 = *(const int4 *)&rsw[row];
+                    rs[0] = r4.x;
+                    rs[1] = r4.y;
+                    rs[2] = r4.z;
+                    rs[3] = r4.w;
+                }
+                if constexpr (SZP) {
+                    const int4 z4 = *(const int4 *)&zsl[gl * BM + row];
+                    zs[0] = z4.x;
+                    zs[1] = z4.y;
+                    zs[2] = z4.z;
+                    zs[3] = z4.w;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int t = acc[i][4 * c + e];
+                    if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
+                    if constexpr (SZP) t += __mul24(zs[e], c2);
+                    res[i][4 * c + e] = __builtin_fmaf(
+                            (float)t * ss[e], sw, res[i][4 * c + e]);
+                }
+            }
+        }
+        gl++;
+    };
 
     for (int t0 = 0; t0 < KT; t0 += SM_CH) {
         const int cnt = min(SM_CH, KT - t0);
@@ -720,13 +815,24 @@ w4a8_small_kernel(const w4a8_small_t p) {
                             (int)(w0 & 0xF0F0F0F0u),
                             (int)((w1 << 4) & 0xF0F0F0F0u),
                             (int)(w1 & 0xF0F0F0F0u)};
+                    if constexpr (SZP) {
+                        int t = csum;
+                        t = __builtin_amdgcn_sdot4(b[0], 0x01010101, t, false);
+                        t = __builtin_amdgcn_sdot4(b[1], 0x01010101, t, false);
+                        t = __builtin_amdgcn_sdot4(b[2], 0x01010101, t, false);
+                        t = __builtin_amdgcn_sdot4(b[3], 0x01010101, t, false);
+                        csum = t;
+                    }
 #pragma unroll
                     for (int i = 0; i < FM; i++) {
                         const int row = i * 32 + (lane & 31);
                         const int cq = ki * 2 + (lane >> 5);
                         const uint4 v = *(const uint4 *)(As + row * BK
                                 + a_swz(row, cq) * 16);
-                        const v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                        if constexpr (SZP) // u8 source: s - 128 as s8
+                            a = v4i {(int)(v.x ^ q.a_flip), (int)(v.y ^ q.a_flip),
+                                    (int)(v.z ^ q.a_flip), (int)(v.w ^ q.a_flip)};
                         if constexpr (HAS_ZP) {
                             int t = rsum[i];
                             t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
@@ -735,7 +841,7 @@ w4a8_small_kernel(const w4a8_small_t p) {
                             t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
                             rsum[i] = t;
                         }
-                        if (ki == 0 && first) {
+                        if (HALF || (ki == 0 && first)) {
                             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
                                     0, 0, 0, 0};
                             acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
@@ -745,51 +851,13 @@ w4a8_small_kernel(const w4a8_small_t p) {
                                     a, b, acc[i], 0, 0, 0);
                         }
                     }
+                    if constexpr (HALF) group_end();
                 }
-                if (++t_in_g == p.tpg) {
-                    // group end: res += (float)(acc [- z * rowsum]) * ss * sw
-                    t_in_g = 0;
-                    const float sw = swl[gl * BN + wave * 32 + (lane & 31)];
-                    int zw = 0;
-                    if constexpr (HAS_ZP) {
-                        zw = zwl[gl * BN + wave * 32 + (lane & 31)];
-#pragma unroll
-                        for (int i = 0; i < FM; i++) {
-                            // both k halves of a row: lanes l and l ^ 32
-                            const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
-                            rsw[i * 32 + (lane & 31)] = tot;
-                            rsum[i] = 0;
-                        }
+                if constexpr (!HALF) {
+                    if (++t_in_g == p.tpg) {
+                        t_in_g = 0;
+                        group_end();
                     }
-#pragma unroll
-                    for (int i = 0; i < FM; i++) {
-#pragma unroll
-                        for (int c = 0; c < 4; c++) {
-                            // registers 4c..4c+3 are rows 8c..8c+7 of the
-                            // fragment: skip those past the last row
-                            if (i * 32 + 8 * c >= mrows) continue;
-                            const int row = i * 32 + 8 * c + 4 * (lane >> 5);
-                            const float4 s4
-                                    = *(const float4 *)&ssl[gl * BM + row];
-                            const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
-                            int rs[4] = {0, 0, 0, 0};
-                            if constexpr (HAS_ZP) {
-                                const int4 r4 = *(const int4 *)&rsw[row];
-                                rs[0] = r4.x;
-                                rs[1] = r4.y;
-                                rs[2] = r4.z;
-                                rs[3] = r4.w;
-                            }
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                int t = acc[i][4 * c + e];
-                                if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
-                                res[i][4 * c + e] = __builtin_fmaf(
-                                        (float)t * ss[e], sw, res[i][4 * c + e]);
-                            }
-                        }
-                    }
-                    gl++;
                 }
             }
         }
@@ -1145,30 +1213,49 @@ w4a8_reduce_kernel(const float *part, int splits, int M, int N, int ldp,
 
 #endif // reduction
 
-template <int FM, int SC, bool HAS_ZP, int ZPK>
+template <int FM, int SC, bool HAS_ZP, int ZPK, int MODE>
 static void launch_small_cfg(const w4a8_small_t &p, hipStream_t stream) {
     constexpr int BM = FM * 32;
-    constexpr size_t lds = (size_t)SM_CH * BM * BK
-            + (size_t)W4A8_SMALL_MAX_GPS * (BM * 4 + 128 * 4 + 128 * 4)
-            + 4 * BM * 4;
-    auto kern = w4a8_small_kernel<FM, SC, HAS_ZP, ZPK>;
+    constexpr size_t lds = sm_lds_bytes(FM, MODE);
+    auto kern = w4a8_small_kernel<FM, SC, HAS_ZP, ZPK, MODE>;
     ensure_dynamic_lds((const void *)kern, (int)lds);
     hipLaunchKernelGGL(kern,
             dim3((p.q.N + 127) / 128, p.splits, (p.q.M + BM - 1) / BM),
             dim3(256), lds, stream, p);
 }
 
-template <int FM, int SC>
+template <int FM, int SC, int MODE>
 static void launch_small_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         hipStream_t stream) {
-    if (!has_zp)
-        launch_small_cfg<FM, SC, false, 0>(p, stream);
-    else if (zpk == 0)
-        launch_small_cfg<FM, SC, true, 0>(p, stream);
+    if constexpr (MODE != 2) {
+        if (!has_zp) {
+            launch_small_cfg<FM, SC, false, 0, MODE>(p, stream);
+            return;
+        }
+    }
+    if (zpk == 0)
+        launch_small_cfg<FM, SC, true, 0, MODE>(p, stream);
     else if (zpk == 1)
-        launch_small_cfg<FM, SC, true, 1>(p, stream);
+        launch_small_cfg<FM, SC, true, 1, MODE>(p, stream);
     else
-        launch_small_cfg<FM, SC, true, 2>(p, stream);
+        launch_small_cfg<FM, SC, true, 2, MODE>(p, stream);
+}
+
+// by rows (one or two 32-row fragments) and scale size
+template <int MODE>
+static void launch_small_mode(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, hipStream_t stream) {
+    if (p.q.M > 32) {
+        if (sc4)
+            launch_small_zp<2, 4, MODE>(p, has_zp, zpk, stream);
+        else
+            launch_small_zp<2, 2, MODE>(p, has_zp, zpk, stream);
+    } else {
+        if (sc4)
+            launch_small_zp<1, 4, MODE>(p, has_zp, zpk, stream);
+        else
+            launch_small_zp<1, 2, MODE>(p, has_zp, zpk, stream);
+    }
 }
 
 template <int BM, int BN, int WGM, int WGN, int ZPM, bool HALF = false>
@@ -1209,7 +1296,9 @@ static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
 // 1, 2 the tiled GEMM without / with zero points, 3 the split-K kernel and its
 // reduction, 4 the single-token kernel, 5 the tiled GEMM with source zero
 // points, 6 and 7 the tiled GEMM with groups of 32 k without / with zero
-// points); the unit without the macro holds the pre-pass and the dispatch.
+// points, 8 and 9 the single-token kernel and 10 and 11 the split-K kernel with
+// groups of 32 k / source zero points); the unit without the macro holds the
+// pre-pass and the dispatch.
 #if defined(QMM_W4A8_PART)
 #if QMM_W4A8_PART == 1
 void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
@@ -1236,20 +1325,23 @@ void launch_gemm_w4a8_half_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream) {
     w4a8::launch_zp<1, true>(p, variant, stream);
 }
+#elif QMM_W4A8_PART == 10
+void launch_gemm_w4a8_small_half_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, hipStream_t stream) {
+    w4a8::launch_small_mode<1>(p, has_zp, zpk, sc4, stream);
+}
+#elif QMM_W4A8_PART == 11
+void launch_gemm_w4a8_small_szp_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, hipStream_t stream) {
+    w4a8::launch_small_mode<2>(p, has_zp, zpk, sc4, stream);
+}
 #elif QMM_W4A8_PART == 3
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, hipStream_t stream) {
-    if (p.q.M > 32) {
-        if (sc4)
-            w4a8::launch_small_zp<2, 4>(p, has_zp, zpk, stream);
-        else
-            w4a8::launch_small_zp<2, 2>(p, has_zp, zpk, stream);
-    } else {
-        if (sc4)
-            w4a8::launch_small_zp<1, 4>(p, has_zp, zpk, stream);
-        else
-            w4a8::launch_small_zp<1, 2>(p, has_zp, zpk, stream);
-    }
+    w4a8::launch_small_mode<0>(p, has_zp, zpk, sc4, stream);
+}
+// the slices' partial results -> dst
+void launch_gemm_w4a8_reduce(const w4a8_small_t &p, hipStream_t stream) {
     const int64_t total = (int64_t)p.q.M * ((p.q.N + 3) / 4);
     int64_t blocks = (total + 255) / 256;
     if (blocks > 65535) blocks = 65535;
@@ -1298,6 +1390,11 @@ void launch_gemm_w4a8_half_zp(const w4a8_params_t &p, int variant,
         hipStream_t stream);
 void launch_gemm_w4a8_small_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, hipStream_t stream);
+void launch_gemm_w4a8_small_half_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, hipStream_t stream);
+void launch_gemm_w4a8_small_szp_part(const w4a8_small_t &p, bool has_zp,
+        int zpk, bool sc4, hipStream_t stream);
+void launch_gemm_w4a8_reduce(const w4a8_small_t &p, hipStream_t stream);
 void launch_gemm_w4a8_tiny_part(const w4a8_small_t &p, bool has_zp, int zpk,
         bool sc4, int nwv, hipStream_t stream);
 void launch_gemm_w4a8_tiny_half_part(const w4a8_small_t &p, bool has_zp,
@@ -1359,8 +1456,18 @@ int gemm_w4a8_tiny_max_groups(bool half) {
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream) {
     if (p.q.M <= 0 || p.q.N <= 0) return;
-    launch_gemm_w4a8_small_part(
-            p, has_zp, zp_storage(p.q), scales_are_f32(p.q), stream);
+    // p.tpg == 0: groups of 32 k; p.q.zsT != nullptr: source zero points / u8
+    // source (as for the single-token kernel)
+    if (p.tpg == 0)
+        launch_gemm_w4a8_small_half_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), stream);
+    else if (p.q.zsT)
+        launch_gemm_w4a8_small_szp_part(
+                p, true, zp_storage(p.q), scales_are_f32(p.q), stream);
+    else
+        launch_gemm_w4a8_small_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), stream);
+    launch_gemm_w4a8_reduce(p, stream);
 }
 
 // variant: 0 = by problem size; 1: 128 x 128, 2: 64 x 128, 3: 32 x 64 tiles

@@ -127,6 +127,15 @@ EXACT_CASES = {
                                   wei_dt=dt.u4),
     "u8_src_zp_common_m1": dict(M=1, K=2048, N=160, src_dt=dt.u8, src_zp=("common", 0), gz=64, gs=64, gw=64,
                                 zp_dt=dt.s4),
+    # 5 ... 64 rows with groups of 32 k / source zero points: the split-K kernel's second and third mode
+    "src_g32_m64_k4096_zp": dict(M=64, K=4096, N=200, gs=32, gw=128, wei_dt=dt.u4, gz=128),
+    "src_g32_m5_k2048_g32_everything": dict(M=5, K=2048, N=130, gs=32, gw=32, gz=32, zp_dt=dt.s4),
+    "src_g32_m24_k14336": dict(M=24, K=14336, N=64, gs=32, gw=128),
+    "u8_src_zp_m40_k2048": dict(M=40, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
+                                zp_dt=dt.u4),
+    "s8_src_zp_m64_k4096_common": dict(M=64, K=4096, N=96, src_zp=("common", 0), src_zp_dt=dt.s8, gs=4096, gw=64,
+                                       gz=64, zp_dt=dt.s8),
+    "u8_src_no_zp_m9_k512": dict(M=9, K=512, N=100, src_dt=dt.u8),
     "u8_src_zp_m300_k2048": dict(M=300, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
                                  zp_dt=dt.u4),
 }
