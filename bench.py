@@ -44,7 +44,8 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
-          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize"}
+          "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize",
+          "attention_products_f16": "bench_f16_products"}
 
 
 def main():
@@ -424,6 +425,40 @@ def bench_c1(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=200):
     ms = _time(prim, strm, hs, hiprt, ex, steps, warm=10)
     return {"us_per_launch": round(ms * 1e3, 2), "TOPs": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
             "impl": pd.impl_info_str(), "note": "back-to-back launches on one stream; launch-latency bound"}
+
+
+def bench_f16_products(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=100):
+    """The attention products as frameworks issue them unfused, shapes of the reference's LLM matmul list
+    (tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu: --dt=f16:f16:f16, abcd tags, 32 heads of 128): one token's
+    scores and context over about 1000 keys, and the prefill products at 998 tokens (rows that are only 4-byte
+    granular). No quantization attributes; the scores carry the list's clip post-op."""
+    out = {}
+    r = np.random.default_rng(9)
+    h16 = lambda x: x.astype(np.float16).view(np.uint16)
+    clip = A.post_ops()
+    clip.append_eltwise(A.algorithm.eltwise_clip, -65504.0, 65504.0)
+    for name, sd, wd, po in (("decode_scores_1x128x1000", [1, 32, 1, 128], [1, 32, 128, 1000], True),
+                             ("decode_context_1x1000x128", [1, 32, 1, 1000], [1, 32, 1000, 128], False),
+                             ("decode_scores_1x128x999", [1, 32, 1, 128], [1, 32, 128, 999], True),
+                             ("prefill_scores_998x128x998", [1, 32, 998, 128], [1, 32, 128, 998], True),
+                             ("prefill_context_998x998x128", [1, 32, 998, 998], [1, 32, 998, 128], False)):
+        dd = sd[:-1] + [wd[-1]]
+        attr = A.primitive_attr()
+        if po:
+            attr.set_post_ops(clip)
+        pd = A.matmul.primitive_desc(eng, memory.desc(sd, dt.f16, T("abcd")), memory.desc(wd, dt.f16, T("abcd")),
+                                     memory.desc(dd, dt.f16, T("abcd")), attr=attr)
+        prim = A.matmul(pd)
+        ex = {A.DNNL_ARG_SRC: memory(pd.src_desc(), eng).write(h16(r.standard_normal(sd))),
+              A.DNNL_ARG_WEIGHTS: memory(pd.weights_desc(), eng).write(h16(r.standard_normal(wd))),
+              A.DNNL_ARG_DST: memory(pd.dst_desc(), eng)}
+        ms = _time(prim, strm, hs, hiprt, ex, steps, warm=5)
+        nbytes = 2 * (int(np.prod(sd)) + int(np.prod(wd)) + int(np.prod(dd)))
+        out[name] = {"us_per_launch": round(ms * 1e3, 2), "TFLOPs": round(2.0 * np.prod(sd) * wd[-1] / (ms * 1e-3) / 1e12, 2),
+                     "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str()}
+    out["note"] = "back-to-back launches on one stream"
+    return out
 
 
 def bench_c4(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
