@@ -1,14 +1,15 @@
-// hip:gfx950:mfma_b8, at most 4 source rows (the decode step of a W8A8 linear
-// layer): the launch is one read of the weights, so the kernel is organised
+// hip:gfx950:mfma_b8, at most 32 source rows (the decode step of a W8A8 linear
+// layer, one token or a small batch of them): the launch is one read of the weights, so the kernel is organised
 // around memory parallelism instead of tiles. A workgroup owns 32 columns (one
 // block of QMM_LAYOUT_MFMA_B8, whose 1 KiB fragments already are the MFMA
 // operand per lane); its 8 waves cut K between them and each streams its
 // fragments straight into registers, 16 requested at a time together with the
-// matching source bytes, and multiplies them with v_mfma_i32_32x32x32_i8 (rows
-// 0..3 of the 32 x 32 result are the source rows; the others repeat the last
-// row and are dropped). The waves' s32 sums are added through LDS by wave 0 --
-// integer addition, so the result does not depend on the cut -- which then runs
-// the epilogue of qmm_gemm_b8.hip per element:
+// matching source bytes, and multiplies them with v_mfma_i32_32x32x32_i8 (the
+// first M rows of the 32 x 32 result are the source rows; the others repeat the
+// last row and are dropped: MR = 4 keeps only registers 0..3 of lanes 0..31,
+// MR = 32 everything). The waves' s32 sums are added through LDS -- integer
+// addition, so the result does not depend on the cut -- and the epilogue of
+// qmm_gemm_b8.hip runs per element:
 //   (float)(P + comp * colsum[n] - z_w'[n] * (rowsum[m] + K * comp)),
 // source scale, weights scale, bias, post-ops, dst quantization
 // (src/cpu/matmul/ref_matmul_int8.cpp:165-259). The row sums that a weights
@@ -26,10 +27,11 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 constexpr int GB8_WAVES = 8;
 constexpr int GB8_CH = 16; // fragments in flight per wave
 
+template <int MR>
 __global__ void __launch_bounds__(GB8_WAVES * 64)
 gemv_b8_kernel(const gemm_params_t p) {
-    __shared__ int red[GB8_WAVES][4][32];
-    __shared__ int red_rs[GB8_WAVES][4];
+    __shared__ int red[GB8_WAVES][MR][32];
+    __shared__ int red_rs[GB8_WAVES][MR];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nb = blockIdx.x;
@@ -81,50 +83,60 @@ gemv_b8_kernel(const gemm_params_t p) {
             }
         }
     }
-    // accumulator registers 0..3 of lanes 0..31 are rows 0..3, column = lane;
-    // the two k halves of row r's sum sit in lanes r and r + 32
-    if (lane < 32) {
+    // accumulator register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4,
+    // column l % 32; the two k halves of row r's sum sit in lanes r and r + 32
+    if constexpr (MR == 4) {
+        if (lane < 32) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[wave][r][lane] = acc[r];
+            for (int r = 0; r < 4; r++) red[wave][r][lane] = acc[r];
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            red[wave][8 * (r / 4) + 4 * (lane >> 5) + r % 4][lane & 31] = acc[r];
     }
     const int tot = rsum + __shfl_xor(rsum, 32);
-    if (lane < 4) red_rs[wave][lane] = tot;
+    if (lane < MR) red_rs[wave][lane] = tot;
     __syncthreads();
-    if (wave == 0 && lane < 32) {
-        const int n = nb * 32 + lane;
-        if (n < p.N) {
-            int comp = p.a_is_u8 ? 128 : 0;
-            if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
-            const int cs = comp != 0 && p.colsum ? comp * p.colsum[n] : 0;
-            const int zw = need_rs
-                    ? (p.wei_zp ? load_int(p.wei_zp_dt, p.wei_zp,
-                               (int64_t)n * p.wei_zp_sn)
-                                : 0)
-                            - p.w_off
-                    : 0;
-            for (int r = 0; r < p.M; r++) {
-                uint32_t v = 0, rs = 0;
+    // one thread per element: column t % 32, rows t / 32 + 16 i
+    const int tid = threadIdx.x;
+    const int n = nb * 32 + (tid & 31);
+    if (n >= p.N) return;
+    int comp = p.a_is_u8 ? 128 : 0;
+    if (p.src_zp) comp -= load_int(p.src_zp_dt, p.src_zp, 0);
+    const int cs = comp != 0 && p.colsum ? comp * p.colsum[n] : 0;
+    const int zw = need_rs
+            ? (p.wei_zp ? load_int(p.wei_zp_dt, p.wei_zp, (int64_t)n * p.wei_zp_sn) : 0)
+                    - p.w_off
+            : 0;
 #pragma unroll
-                for (int w = 0; w < GB8_WAVES; w++) {
-                    v += (uint32_t)red[w][r][lane];
-                    rs += (uint32_t)red_rs[w][r];
-                }
-                // s32 arithmetic that wraps as the reference's int accumulation
-                v += (uint32_t)cs
-                        - (uint32_t)zw * (rs + (uint32_t)p.K * (uint32_t)comp);
-                epilogue_apply_store(p.ep, (float)(int32_t)v, 0, r, n);
+    for (int i = 0; i < (MR + 15) / 16; i++) {
+        const int r = (tid >> 5) + 16 * i;
+        if (r < p.M && r < MR) {
+            uint32_t v = 0, rs = 0;
+#pragma unroll
+            for (int w = 0; w < GB8_WAVES; w++) {
+                v += (uint32_t)red[w][r][tid & 31];
+                rs += (uint32_t)red_rs[w][r];
             }
+            // s32 arithmetic that wraps as the reference's int accumulation
+            v += (uint32_t)cs - (uint32_t)zw * (rs + (uint32_t)p.K * (uint32_t)comp);
+            epilogue_apply_store(p.ep, (float)(int32_t)v, 0, r, n);
         }
     }
 }
 
 } // namespace
 
-// p.M <= 4, one batch, integer operands (the caller checks)
+// p.M <= 32, one batch, integer operands (the caller checks)
 void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return;
-    hipLaunchKernelGGL(gemv_b8_kernel, dim3((unsigned)p.nb32),
-            dim3(GB8_WAVES * 64), 0, stream, p);
+    if (p.M <= 4)
+        hipLaunchKernelGGL(gemv_b8_kernel<4>, dim3((unsigned)p.nb32),
+                dim3(GB8_WAVES * 64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(gemv_b8_kernel<32>, dim3((unsigned)p.nb32),
+                dim3(GB8_WAVES * 64), 0, stream, p);
 }
 
 } // namespace qmm
