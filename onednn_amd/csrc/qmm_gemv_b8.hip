@@ -27,13 +27,31 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 constexpr int GB8_WAVES = 8;
 constexpr int GB8_CH = 16; // fragments in flight per wave
 
+// MR = 32: the source bytes of a chunk go through a wave-private piece of LDS --
+// requested as whole 256-byte row pieces (16 lanes a row, 4 rows an
+// instruction) instead of one 16-byte piece per lane out of 32 different rows
+// -- and come back in operand order. The same bytes hold the wave's results
+// for the sum across waves afterwards.
+constexpr int GB8_CH32 = 8; // fragments per chunk with 32 rows
+constexpr int GB8_APITCH = GB8_CH32 * 32 + 16; // bytes of a staged row
+constexpr int GB8_WAVE_LDS = 32 * GB8_APITCH; // >= 32 x 32 s32 of results + row sums
+static_assert(GB8_WAVE_LDS >= 32 * 32 * 4 + 32 * 4, "");
+
 template <int MR>
 __global__ void __launch_bounds__(GB8_WAVES * 64)
 gemv_b8_kernel(const gemm_params_t p) {
-    __shared__ int red[GB8_WAVES][MR][32];
-    __shared__ int red_rs[GB8_WAVES][MR];
+    constexpr int CH = MR == 32 ? GB8_CH32 : GB8_CH;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int WAVE_LDS = MR == 32 ? GB8_WAVE_LDS : (4 * 32 + 4) * 4;
+    // a wave's results [MR][32] and row sums [MR], s32
+    auto red = [&](int w, int r, int c) -> int & {
+        return ((int *)(lds_raw + w * WAVE_LDS))[r * 32 + c];
+    };
+    auto red_rs = [&](int w, int r) -> int & {
+        return ((int *)(lds_raw + w * WAVE_LDS))[MR * 32 + r];
+    };
     const int nb = blockIdx.x;
     // the wave's fragments (32 k each): an even cut of the K / 32 that hold data
     const int nfrag = (p.K + 31) / 32;
@@ -45,27 +63,50 @@ gemv_b8_kernel(const gemm_params_t p) {
     const uint8_t *arow = p.A + (int64_t)row * p.lda;
     const uint32_t flip = p.a_is_u8 && !p.a_preflipped ? 0x80808080u : 0u;
     const bool need_rs = p.wei_zp != nullptr || p.w_off != 0;
+    uint8_t *const stage = lds_raw + wave * WAVE_LDS;
 
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
     int rsum = 0;
-    for (int fb = f0; fb < f1; fb += GB8_CH) {
-        v4u bq[GB8_CH];
-        uint4 av[GB8_CH];
+    for (int fb = f0; fb < f1; fb += CH) {
+        v4u bq[CH];
+        uint4 av[CH];
         // every request of the chunk before the first use; fragments past the
         // wave's end repeat its last one and are skipped below
+        if constexpr (MR == 32) {
+            // piece l % 16 of rows l / 16 + 4 i (K is a multiple of 16: a piece
+            // is inside the row or past it)
+            const int k = fb * 32 + (lane & 15) * 16;
 #pragma unroll
-        for (int j = 0; j < GB8_CH; j++) {
-            const int f = min(fb + j, f1 - 1);
-            bq[j] = __builtin_nontemporal_load(bsrc + (int64_t)f * 64);
-            // K is a multiple of 16: a half fragment is inside the row or past it
-            const int k = f * 32 + (lane >> 5) * 16;
-            av[j] = *(const uint4 *)(arow + min(k, p.K - 16));
-            if (k >= p.K) av[j] = make_uint4(flip, flip, flip, flip); // zero after the flip
+            for (int i = 0; i < CH; i++) {
+                const int r = min(4 * i + (lane >> 4), p.M - 1);
+                av[i] = *(const uint4 *)(p.A + (int64_t)r * p.lda + min(k, p.K - 16));
+            }
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                bq[j] = __builtin_nontemporal_load(bsrc + (int64_t)min(fb + j, f1 - 1) * 64);
+#pragma unroll
+            for (int i = 0; i < CH; i++)
+                *(uint4 *)(stage + (4 * i + (lane >> 4)) * GB8_APITCH + (lane & 15) * 16)
+                        = k >= p.K ? make_uint4(flip, flip, flip, flip) : av[i]; // zero after the flip
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                av[j] = *(const uint4 *)(stage + (lane & 31) * GB8_APITCH + j * 32
+                        + (lane >> 5) * 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < CH; j++) {
+                const int f = min(fb + j, f1 - 1);
+                bq[j] = __builtin_nontemporal_load(bsrc + (int64_t)f * 64);
+                // K is a multiple of 16: a half fragment is inside the row or past it
+                const int k = f * 32 + (lane >> 5) * 16;
+                av[j] = *(const uint4 *)(arow + min(k, p.K - 16));
+                if (k >= p.K) av[j] = make_uint4(flip, flip, flip, flip); // zero after the flip
+            }
         }
 #pragma unroll
-        for (int j = 0; j < GB8_CH; j++) {
+        for (int j = 0; j < CH; j++) {
             if (fb + j < f1) {
                 const v4i a = {(int)(av[j].x ^ flip), (int)(av[j].y ^ flip),
                         (int)(av[j].z ^ flip), (int)(av[j].w ^ flip)};
@@ -88,15 +129,15 @@ gemv_b8_kernel(const gemm_params_t p) {
     if constexpr (MR == 4) {
         if (lane < 32) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) red[wave][r][lane] = acc[r];
+            for (int r = 0; r < 4; r++) red(wave, r, lane) = acc[r];
         }
     } else {
 #pragma unroll
         for (int r = 0; r < 16; r++)
-            red[wave][8 * (r / 4) + 4 * (lane >> 5) + r % 4][lane & 31] = acc[r];
+            red(wave, 8 * (r / 4) + 4 * (lane >> 5) + r % 4, lane & 31) = acc[r];
     }
     const int tot = rsum + __shfl_xor(rsum, 32);
-    if (lane < MR) red_rs[wave][lane] = tot;
+    if (lane < MR) red_rs(wave, lane) = tot;
     __syncthreads();
     // one thread per element: column t % 32, rows t / 32 + 16 i
     const int tid = threadIdx.x;
@@ -116,8 +157,8 @@ gemv_b8_kernel(const gemm_params_t p) {
             uint32_t v = 0, rs = 0;
 #pragma unroll
             for (int w = 0; w < GB8_WAVES; w++) {
-                v += (uint32_t)red[w][r][tid & 31];
-                rs += (uint32_t)red_rs[w][r];
+                v += (uint32_t)red(w, r, tid & 31);
+                rs += (uint32_t)red_rs(w, r);
             }
             // s32 arithmetic that wraps as the reference's int accumulation
             v += (uint32_t)cs - (uint32_t)zw * (rs + (uint32_t)p.K * (uint32_t)comp);
@@ -131,12 +172,15 @@ gemv_b8_kernel(const gemm_params_t p) {
 // p.M <= 32, one batch, integer operands (the caller checks)
 void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return;
-    if (p.M <= 4)
+    if (p.M <= 4) {
         hipLaunchKernelGGL(gemv_b8_kernel<4>, dim3((unsigned)p.nb32),
-                dim3(GB8_WAVES * 64), 0, stream, p);
-    else
+                dim3(GB8_WAVES * 64), GB8_WAVES * (4 * 32 + 4) * 4, stream, p);
+    } else {
+        constexpr int lds = GB8_WAVES * GB8_WAVE_LDS;
+        ensure_dynamic_lds((const void *)gemv_b8_kernel<32>, lds);
         hipLaunchKernelGGL(gemv_b8_kernel<32>, dim3((unsigned)p.nb32),
-                dim3(GB8_WAVES * 64), 0, stream, p);
+                dim3(GB8_WAVES * 64), lds, stream, p);
+    }
 }
 
 } // namespace qmm
