@@ -1016,9 +1016,9 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.batch = (int32_t)P.batch;
         g.kb32 = (int32_t)geom.kb32;
         g.nb32 = (int32_t)geom.nb32;
-        // at most 32 rows of one matrix: the streaming kernel (it forms the
+        // at most 64 rows of one matrix: the streaming kernel (it forms the
         // row sums a weights zero point needs itself)
-        if (!f8 && P.M <= 32 && P.batch == 1 && gemm_variant == 0) {
+        if (!f8 && P.M <= 64 && P.batch == 1 && gemm_variant == 0) {
             if (b8_needs_rowsum(D)) {
                 const qmm_quant_t &wz = D.zps[QMM_WEI];
                 g.wei_zp = wz.set ? args->zps[QMM_WEI] : nullptr;

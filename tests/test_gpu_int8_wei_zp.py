@@ -79,11 +79,15 @@ CASES = {
     "m3_u8_src_zp_s8_weights_no_wzp": dict(M=3, K=1024, N=100, src_dt=dt.u8, wei_dt=dt.s8, wei_zp=None, src_zp=77),
     "m4_k208_half_fragment": dict(M=4, K=208, N=72, src_dt=dt.u8, src_zp=130, dst_dt=dt.s32),
     "m2_u8_u8_common_zp_s32_dst": dict(M=2, K=14336, N=64, src_dt=dt.u8, wei_zp="common", dst_dt=dt.s32, src_zp=3),
-    # 5 ... 32 rows of one matrix: the streaming kernel keeps all 32 rows of its MFMA
+    # 5 ... 64 rows of one matrix: the streaming kernel keeps all rows of one or two 32-row MFMA blocks
     "m32_k4096_zp_per_column": dict(M=32, K=4096, N=200),
     "m17_u8_src_both_zero_points_s32_dst": dict(M=17, K=1040, N=72, src_dt=dt.u8, src_zp=99, dst_dt=dt.s32),
     "m9_s8_s8_plain_k_tail_s32_dst": dict(M=9, K=208, N=130, wei_dt=dt.s8, wei_zp=None, dst_dt=dt.s32),
     "m31_s8_s8_zp_s8_bias": dict(M=31, K=512, N=96, wei_dt=dt.s8, wei_zp_dt=dt.s8, bias_dt=dt.f32),
+    "m33_k2048_zp_per_column": dict(M=33, K=2048, N=130),
+    "m64_u8_src_zp_s8_weights_zp": dict(M=64, K=1040, N=96, src_dt=dt.u8, wei_dt=dt.s8, wei_zp_dt=dt.s8, src_zp=131,
+                                        dst_dt=dt.s32),
+    "m48_s8_s8_plain_bias": dict(M=48, K=512, N=200, wei_dt=dt.s8, wei_zp=None, bias_dt=dt.f32),
     "m1_s8_s8_plain": dict(M=1, K=512, N=1000, wei_dt=dt.s8, wei_zp=None),
     "ab_weights_bias_s8_dst": dict(M=50, K=256, N=80, wei_layout="ab", bias_dt=dt.f32, dst_dt=dt.s8),
     "batched_broadcast_zp": dict(M=20, K=128, N=64, batch=(3,), dst_dt=dt.s32),
