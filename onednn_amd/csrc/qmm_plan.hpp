@@ -16,14 +16,14 @@ namespace qmm {
 // several host threads that launch concurrently.
 inline void ensure_dynamic_lds(const void *kern, int bytes) {
     static std::mutex mu;
-    static const void *seen[96];
+    static const void *seen[1024]; // (far more than the library has kernels)
     static int n = 0;
     std::lock_guard<std::mutex> lock(mu);
     for (int i = 0; i < n; i++)
         if (seen[i] == kern) return;
     (void)hipFuncSetAttribute(
             kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (n < 96) seen[n++] = kern;
+    if (n < 1024) seen[n++] = kern;
 }
 
 // A scales / zero-points buffer as the generic kernels index it: dense
