@@ -354,7 +354,11 @@ gemv_w4_kernel(const gemv_params_t p, const int MR, const int KC) {
 // so that both planes add into one accumulator:
 //     sum a * (w - z) = P - (17 * offset + 16 * [8 if signed] + z) * S,
 // the sign of an s8 weight living in its high nibble.
-template <bool F16, int ROWS, bool WSIGNED, bool W8>
+constexpr int GEMV_UNR = 4; // tiles of a wave in flight
+constexpr int GEMV_APITCH = 256 + 16; // bytes of a staged activation row of a tile
+constexpr int GEMV_STAGE_BYTES = GEMV_WAVES * GEMV_UNR * 16 * GEMV_APITCH;
+
+template <bool F16, int ROWS, bool WSIGNED, bool W8, bool STAGED = false>
 __global__ void __launch_bounds__(GEMV_WAVES * 64)
 gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
@@ -362,6 +366,9 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
         const int K, const int lda, const int shifts, const int flags_m,
         const gemv_params_t p) {
     __shared__ __attribute__((aligned(16))) float red[GEMV_WAVES * 64 * 4];
+    // STAGED: the activations of a wave's tiles pass through a wave-private
+    // piece of LDS (see below)
+    extern __shared__ __attribute__((aligned(16))) uint8_t act_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int uw = __builtin_amdgcn_readfirstlane(tid >> 6);
     // consecutive workgroups run on the 8 XCDs in turn: give each XCD a
@@ -418,13 +425,22 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
     const int tiles = kg128;
     constexpr int SPL = ROWS == 16 ? 1 : ROWS == 8 ? 2 : 4; // steps per load
     constexpr int NA = 4 / SPL; // activation loads per tile
-    const int rr = ROWS == 1 ? 0 : min(r / SPL, rows - 1);
+    // STAGED (16 rows, a launch of at most one workgroup per CU -- the 136 KiB
+    // leave room for one): requested as whole 256-byte row pieces (16 lanes a
+    // row, 4 rows an instruction: load h of lane l is piece l % 16 of row
+    // 4 h + l / 16) instead of 64-byte pieces of 16 different rows, and read
+    // back from LDS in operand order; wave-private, so no barrier. 4096 x 4096
+    // at 16 rows: 6.7 us against 7.5 us; with more workgroups than CUs the
+    // second resident workgroup is worth more (14336 columns: 19 against 21 us).
+    static_assert(!STAGED || ROWS == 16, "");
+    const int rr = ROWS == 1 ? 0 : STAGED ? 0 : min(r / SPL, rows - 1);
     const uint16_t *__restrict__ Arow = pA + (int64_t)(m_base + rr) * lda;
+    uint8_t *const stage_w = act_lds + uw * (GEMV_UNR * 16 * GEMV_APITCH);
     const int nn = min(n, N - 1);
     const uint16_t *const scn = pSC + (scale_per_n ? nn : 0);
     const int zcol = zp_per_n ? nn : 0;
     const bool k_tail = (K & 127) != 0;
-    constexpr int UNR = 4;
+    constexpr int UNR = GEMV_UNR;
     void *dst_ptr = nullptr;
     int64_t dst_sm = 0;
     int dst_dt = 0;
@@ -449,9 +465,15 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             for (int h = 0; h < NA; h++) {
                 // chunks past the row's end re-read its last one, rows past M
                 // the last row
-                const int k = min(
-                        tc * 128 + (h * SPL + r % SPL) * 32 + c * 8, K - 8);
-                av[u][h] = *(const uint4 *)(Arow + k);
+                if constexpr (STAGED) {
+                    const int row = min(4 * h + (lane >> 4), rows - 1);
+                    const int k = min(tc * 128 + (lane & 15) * 8, K - 8);
+                    av[u][h] = *(const uint4 *)(pA + (int64_t)(m_base + row) * lda + k);
+                } else {
+                    const int k = min(
+                            tc * 128 + (h * SPL + r % SPL) * 32 + c * 8, K - 8);
+                    av[u][h] = *(const uint4 *)(Arow + k);
+                }
             }
             const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
             scp[u] = scn[(int64_t)gsc * sN];
@@ -466,7 +488,9 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
                 const int tc = tile_of(tb + uw + u * GEMV_WAVES);
 #pragma unroll
                 for (int h = 0; h < NA; h++)
-                    if (tc * 128 + (h * SPL + r % SPL) * 32 + c * 8 >= K)
+                    if ((STAGED ? tc * 128 + (lane & 15) * 8
+                                : tc * 128 + (h * SPL + r % SPL) * 32 + c * 8)
+                            >= K)
                         av[u][h] = make_uint4(0, 0, 0, 0);
             }
         }
@@ -478,11 +502,27 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             dst_dt = p.ep.dst.dt;
             asm volatile("" ::"s"(dst_ptr), "s"(dst_sm), "s"(dst_dt));
         }
+        if constexpr (STAGED) {
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+#pragma unroll
+                for (int h = 0; h < NA; h++)
+                    *(uint4 *)(stage_w + ((u * 16 + 4 * h + (lane >> 4)) * GEMV_APITCH)
+                            + (lane & 15) * 16)
+                            = av[u][h];
+        }
         // the four tiles are independent accumulation chains: a tile past
         // the end is a repeat of the last one and is folded with scale 0
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             v4f Pu = {0.f, 0.f, 0.f, 0.f}, Su = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (STAGED) {
+                // lane (r, c): row r, k = 32 s + 8 c .. + 7 of the tile
+#pragma unroll
+                for (int h = 0; h < NA; h++)
+                    av[u][h] = *(const uint4 *)(stage_w + (u * 16 + r) * GEMV_APITCH
+                            + h * 64 + c * 16);
+            }
 #pragma unroll
             for (int s4 = 0; s4 < 4; s4++) {
                 const uint32_t d = (s4 == 0 ? wt[u][0].x
@@ -626,8 +666,13 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
             launch_gemm_w4f(q, shifts, flags_m, stream);
             return;
         }
+        // more than 8 rows in at most one workgroup per CU: the variant that
+        // stages its activations in LDS
+        const bool staged = p.M > 8 && (int64_t)grid.x * grid.y <= 256;
+        const int lds = staged ? GEMV_STAGE_BYTES : 0;
         auto go = [&](auto kern) {
-            hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), 0, stream, p.B,
+            if (lds) ensure_dynamic_lds((const void *)kern, lds);
+            hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, p.B,
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
                     (int)p.lda, shifts, flags_m, q);
         };
@@ -635,6 +680,15 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         auto by_w8 = [&](auto f16, auto rows, auto sgn) {
             constexpr bool F = decltype(f16)::value, S = decltype(sgn)::value;
             constexpr int R = decltype(rows)::value;
+            if constexpr (R == 16) {
+                if (staged) {
+                    if (p.w8)
+                        go(gemv_w4_fast_kernel<F, R, S, true, true>);
+                    else
+                        go(gemv_w4_fast_kernel<F, R, S, false, true>);
+                    return;
+                }
+            }
             if (p.w8)
                 go(gemv_w4_fast_kernel<F, R, S, true>);
             else
