@@ -45,7 +45,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 # side measurements reported next to the headline configuration: key -> function
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
           "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize",
-          "attention_products_f16": "bench_f16_products"}
+          "attention_products_f16": "bench_f16_products", "int8_decode_rows": "bench_int8_rows"}
 
 
 def main():
@@ -425,6 +425,45 @@ def bench_c1(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=200):
     ms = _time(prim, strm, hs, hiprt, ex, steps, warm=10)
     return {"us_per_launch": round(ms * 1e3, 2), "TOPs": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
             "impl": pd.impl_info_str(), "note": "back-to-back launches on one stream; launch-latency bound"}
+
+
+def bench_int8_rows(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=100, K=4096, N=14336):
+    """The decode step of config 2's layer (s8 x s8, per-token and per-column scales, bf16 dst) and of the W8A8 layers of
+    the reference's LLM list (--dt=s8:u8:f16, a u8 zero point per column) at 1, 32 and 64 rows: the streaming kernel.
+    The 59 MB of weights stay in the last-level cache between launches, so the rate is not an HBM figure."""
+    out = {}
+    r = np.random.default_rng(11)
+    for name, wdt, zp in (("s8_s8", dt.s8, False), ("s8_u8_zp_per_column", dt.u8, True)):
+        for M in (1, 32, 64):
+            attr = A.primitive_attr()
+            attr.set_scales(A.DNNL_ARG_SRC, 3, [1, K], dt.f32)  # per token, as in config 2
+            attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 2)
+            if zp:
+                attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 2, [], dt.u8)
+            pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.s8, T("ab")), memory.desc([K, N], wdt, tag.any),
+                                         memory.desc([M, N], dt.bf16, T("ab")), attr=attr)
+            prim = A.matmul(pd)
+            w = r.integers(0, 256, (K, N)).astype(np.uint8) if zp else r.integers(-127, 128, (K, N)).astype(np.int8)
+            plain = memory(memory.desc([K, N], wdt, T("ab")), eng).write(w)
+            m_wei = memory(pd.weights_desc(), eng)
+            A.reorder(plain, m_wei).execute(strm, plain, m_wei)
+            strm.wait()
+            ex = {A.DNNL_ARG_SRC: memory(pd.src_desc(), eng).write(r.integers(-127, 128, (M, K)).astype(np.int8)),
+                  A.DNNL_ARG_WEIGHTS: m_wei, A.DNNL_ARG_DST: memory(pd.dst_desc(), eng),
+                  A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: memory(memory.desc([M], dt.f32, T("a")), eng).write(
+                      r.uniform(0.005, 0.05, M).astype(np.float32)),
+                  A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: memory(memory.desc([N], dt.f32, T("a")), eng).write(
+                      r.uniform(0.0005, 0.005, N).astype(np.float32))}
+            if zp:
+                ex[A.DNNL_ARG_ATTR_ZERO_POINTS | A.DNNL_ARG_WEIGHTS] = memory(memory.desc([N], dt.u8, T("a")), eng).write(
+                    r.integers(100, 156, N).astype(np.uint8))
+            ms = _time(prim, strm, hs, hiprt, ex, steps, warm=5)
+            nbytes = K * N + M * K + 2 * M * N + 8 * N
+            out["%s_M%d" % (name, M)] = {"us_per_launch": round(ms * 1e3, 2), "TOPs": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
+                                         "algorithmic_bytes": nbytes, "GBps_from_cache": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                         "impl": pd.impl_info_str()}
+    out["note"] = "back-to-back launches on one stream, one weight set (resident in the last-level cache)"
+    return out
 
 
 def bench_f16_products(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=100):
