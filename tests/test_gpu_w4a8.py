@@ -136,6 +136,11 @@ EXACT_CASES = {
     "s8_src_zp_m64_k4096_common": dict(M=64, K=4096, N=96, src_zp=("common", 0), src_zp_dt=dt.s8, gs=4096, gw=64,
                                        gz=64, zp_dt=dt.s8),
     "u8_src_no_zp_m9_k512": dict(M=9, K=512, N=100, src_dt=dt.u8),
+    # 5 ... 32 rows, whole tiles per group (the decode batches of the LLM list: 31, 32 rows)
+    "m32_k4096_u4_zp_g128": dict(M=32, K=4096, N=200, wei_dt=dt.u4, gz=128),
+    "m31_k4096_s4_g64_everything": dict(M=31, K=4096, N=130, gs=64, gw=64, gz=64, zp_dt=dt.s8),
+    "m9_k1024_src_per_row_only": dict(M=9, K=1024, N=96, gs=1024, gw=128),
+    "m17_k512_u4_zp_u4_g256": dict(M=17, K=512, N=70, wei_dt=dt.u4, gs=256, gw=256, gz=256, zp_dt=dt.u4),
     "u8_src_zp_m300_k2048": dict(M=300, K=2048, N=264, src_dt=dt.u8, src_zp=("mk", 128), wei_dt=dt.u4, gz=128,
                                  zp_dt=dt.u4),
 }
