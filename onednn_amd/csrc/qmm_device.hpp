@@ -611,20 +611,12 @@ QMM_D void epilogue_store4(const epilogue_t &ep, const float (&d)[4],
                 for (int i = 0; i < 4; i++)
                     h[i] = f32_to_f16_hw(d[i]);
             }
-            // the widest stores the address allows (rows of odd length start
-            // on 2- or 4-byte boundaries)
+            // one 8-byte store whatever the address (rows of odd length start on
+            // 2- or 4-byte boundaries; global stores take any address)
+            typedef unsigned v2u_any __attribute__((ext_vector_type(2), aligned(2)));
             const uint32_t lo = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
             const uint32_t hi = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-            if (((uintptr_t)q & 7) == 0) {
-                *(uint2 *)q = make_uint2(lo, hi);
-            } else if (((uintptr_t)q & 3) == 0) {
-                *(uint32_t *)q = lo;
-                *(uint32_t *)(q + 2) = hi;
-            } else {
-                q[0] = h[0];
-                *(uint32_t *)(q + 1) = (uint32_t)h[1] | ((uint32_t)h[2] << 16);
-                q[3] = h[3];
-            }
+            *(v2u_any *)q = v2u_any {lo, hi};
             return;
         } else if (dt == dt_f32) {
             float *q = (float *)dst + dst_off;

@@ -46,14 +46,20 @@ QMM_D v4f mma16(const v8s &a, const v8s &b, const v4f &c) {
 
 // Eight neighbouring 16-bit elements of a row of `len` elements, starting at
 // element `at` (a multiple of 8), in two steps so that nothing touches the
-// loaded registers before the tile is staged. G (8, 2 or 1) elements per load:
-// row starts are multiples of 2 G bytes and `len` is a multiple of G, so a
-// piece of G elements is inside the row or past it, never across its end.
-// `request8` only issues the 8 / G loads, a piece past the end re-reading the
-// row's first one; `finish8` packs them and zeroes what is not there.
+// loaded registers before the tile is staged: `request8` only issues loads,
+// `finish8` zeroes what lies at or past `len` (or in a row that is not there).
+//   G = 8: rows start on 16-byte boundaries and `len` is a multiple of 8, so a
+//     chunk is inside the row or past it: one aligned 16-byte load.
+//   G = 0: any alignment, `len` >= 8: one 16-byte load that need not be aligned
+//     (global loads take any address), at min(at, len - 8); where that moved the
+//     window back, the chunk's elements are the window's upper ones and
+//     `finish8` shifts them down, which also zero-fills what is past `len`.
+//   G = 1: rows shorter than 8: element loads.
+typedef unsigned v4u_any __attribute__((ext_vector_type(4), aligned(2)));
+
 template <int G>
 struct req8_t {
-    uint32_t w[G == 8 ? 4 : 8 / G];
+    uint32_t w[G == 1 ? 8 : 4];
 };
 
 template <int G>
@@ -61,10 +67,9 @@ QMM_D void request8(req8_t<G> &r, const uint16_t *row, int at, int len) {
     if constexpr (G == 8) {
         const uint4 v = *(const uint4 *)(row + (at < len ? at : 0));
         r.w[0] = v.x, r.w[1] = v.y, r.w[2] = v.z, r.w[3] = v.w;
-    } else if constexpr (G == 2) {
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            r.w[j] = *(const uint32_t *)(row + (at + 2 * j < len ? at + 2 * j : 0));
+    } else if constexpr (G == 0) {
+        const auto v = *(const v4u_any *)(row + min(at, len - 8));
+        r.w[0] = v[0], r.w[1] = v[1], r.w[2] = v[2], r.w[3] = v[3];
     } else {
 #pragma unroll
         for (int j = 0; j < 8; j++) r.w[j] = row[at + j < len ? at + j : 0];
@@ -78,9 +83,21 @@ QMM_D uint4 finish8(const req8_t<G> &r, int at, int len, bool row_ok) {
         const bool ok = row_ok && at < len;
 #pragma unroll
         for (int j = 0; j < 4; j++) w[j] = ok ? r.w[j] : 0u;
-    } else if constexpr (G == 2) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) w[j] = row_ok && at + 2 * j < len ? r.w[j] : 0u;
+    } else if constexpr (G == 0) {
+        // the window started `back` elements before the chunk: shift the 128
+        // bits right by 16 * back (0 .. 112)
+        const int back = at - min(at, len - 8);
+        const uint64_t lo = (uint64_t)r.w[0] | ((uint64_t)r.w[1] << 32);
+        const uint64_t hi = (uint64_t)r.w[2] | ((uint64_t)r.w[3] << 32);
+        const int sh = 16 * (back & 3);
+        const uint64_t a = back < 4 ? lo : hi, b = back < 4 ? hi : 0ull;
+        const uint64_t nlo = sh ? (a >> sh) | (b << (64 - sh)) : a;
+        const uint64_t nhi = b >> sh;
+        const bool ok = row_ok && at < len;
+        w[0] = ok ? (uint32_t)nlo : 0u;
+        w[1] = ok ? (uint32_t)(nlo >> 32) : 0u;
+        w[2] = ok ? (uint32_t)nhi : 0u;
+        w[3] = ok ? (uint32_t)(nhi >> 32) : 0u;
     } else {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -415,8 +432,10 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     }
     const dim3 grid((unsigned)((p.N + F16_BN - 1) / F16_BN),
             (unsigned)((p.M + F16_BM - 1) / F16_BM), (unsigned)p.batch);
-    // loads of 8, 2 or 1 elements: the granule has to divide the row length too
-    auto pick = [](int g, int len) { return g >= 8 && len % 8 == 0 ? 8 : g >= 2 && len % 2 == 0 ? 2 : 1; };
+    // aligned 16-byte loads where rows start on 16-byte boundaries and hold a
+    // multiple of 8 elements, else unaligned ones (rows of 8 elements and
+    // more), else element loads
+    auto pick = [](int g, int len) { return g >= 8 && len % 8 == 0 ? 8 : len >= 8 ? 0 : 1; };
     int ga = pick(p.a_vec, p.K), gb = pick(p.b_vec, p.N);
     const bool light = light_epilogue(p.ep) && p.ep.dst.sn == 1;
     if (!light && !(ga == 8 && gb == 8)) ga = gb = 1; // the interpreter form exists twice
@@ -430,7 +449,7 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
         else go(std::false_type {}, lt, a, b);
     };
     using I8 = std::integral_constant<int, 8>;
-    using I2 = std::integral_constant<int, 2>;
+    using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     if (!light) {
         if (ga == 8) by_bf(std::false_type {}, I8 {}, I8 {});
@@ -439,11 +458,11 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     }
     auto by_b = [&](auto a) {
         if (gb == 8) by_bf(std::true_type {}, a, I8 {});
-        else if (gb == 2) by_bf(std::true_type {}, a, I2 {});
+        else if (gb == 0) by_bf(std::true_type {}, a, I0 {});
         else by_bf(std::true_type {}, a, I1 {});
     };
     if (ga == 8) by_b(I8 {});
-    else if (ga == 2) by_b(I2 {});
+    else if (ga == 0) by_b(I0 {});
     else by_b(I1 {});
 }
 
