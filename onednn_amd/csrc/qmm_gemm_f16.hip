@@ -258,8 +258,8 @@ gemm_f16_kernel(const gemm16_params_t p) {
 // keys x 128) per head are a few MB of weights read once; a 64 x 64 MFMA tile
 // would leave most of the chip idle. Here a workgroup owns `cw` columns of one
 // batch entry: `tpr` neighbouring lanes cover a weights row of the chunk (V
-// elements each: one 16-byte load where rows are 16-byte granular and N is a
-// multiple of 8, else one element), the 256 / tpr lane groups take every
+// elements each: one 16-byte load at any address, or one element for rows
+// shorter than 32), the 256 / tpr lane groups take every
 // (256 / tpr)-th k, requests run one unrolled block ahead of the arithmetic,
 // the activations wait in LDS as f32, and the partial sums of the lane groups
 // meet through lane permutes (within a wave) and LDS (across the four waves).
@@ -276,13 +276,17 @@ template <bool BF, int V, int MR>
 __global__ void __launch_bounds__(GV_THREADS)
 gemv_f16_kernel(const gemm16_params_t p, const int tpr_log2) {
     constexpr int U = V == 8 ? 8 : 16; // loads per lane and block
-    typedef typename std::conditional<V == 8, uint4, uint16_t>::type wv_t;
+    // (16-byte loads at any address: rows of any length and alignment)
+    typedef typename std::conditional<V == 8, v4u_any, uint16_t>::type wv_t;
     extern __shared__ __attribute__((aligned(16))) float gv_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tpr = 1 << tpr_log2, cw = tpr * V, rpp = GV_THREADS >> tpr_log2;
     const int col_l = (tid & (tpr - 1)) * V, phase = tid >> tpr_log2;
-    const int n0 = blockIdx.x * cw, n = n0 + col_l;
+    // V = 8: the last chunk moves back inside the row (N >= cw, the host
+    // checks), recomputing a few columns of its neighbour with the same result
+    const int n0 = V == 8 ? min((int)blockIdx.x * cw, p.N - cw) : blockIdx.x * cw;
+    const int n = n0 + col_l;
     const int64_t bz = blockIdx.y;
     const int K = p.K;
     float *qtab = gv_lds; // [MR][K]
@@ -337,7 +341,7 @@ gemv_f16_kernel(const gemm16_params_t p, const int tpr_log2) {
             for (int m = 0; m < MR; m++) q[m] = ok ? qtab[m * K + min(k, K - 1)] : 0.f;
             float wf[V];
             if constexpr (V == 8) {
-                const uint32_t d[4] = {wc[u].x, wc[u].y, wc[u].z, wc[u].w};
+                const uint32_t d[4] = {wc[u][0], wc[u][1], wc[u][2], wc[u][3]};
 #pragma unroll
                 for (int i = 0; i < 8; i++)
                     wf[i] = up16<BF>((d[i / 2] >> (16 * (i % 2))) & 0xffffu);
@@ -403,15 +407,15 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.batch <= 0) return;
     const int mr = p.M == 1 ? 1 : 4;
     if (p.M <= 4 && (int64_t)mr * p.K <= GV_MAX_ACT) {
-        // vector loads need whole 8-column chunks inside N as well
-        const bool vec = p.b_vec == 8 && p.N % 8 == 0;
+        // 16-byte loads (8 columns a lane) wherever a 32-column chunk fits the row
+        const bool vec = p.N >= 32;
         int tpr_log2 = 6; // one element per lane: 64 columns per workgroup
         if (vec) {
             // the widest chunk (32 .. 256 columns) that still gives 256 workgroups
             tpr_log2 = 5;
             while (tpr_log2 > 2
                     && ((int64_t)p.batch * ((p.N + (8 << tpr_log2) - 1) >> (tpr_log2 + 3)) < 256
-                            || (4 << tpr_log2) >= p.N))
+                            || (8 << tpr_log2) > p.N))
                 tpr_log2--;
         }
         auto go = [&](auto bf, auto v) {
