@@ -619,24 +619,22 @@ QMM_D void epilogue_store4(const epilogue_t &ep, const float (&d)[4],
             *(v2u_any *)q = v2u_any {lo, hi};
             return;
         } else if (dt == dt_f32) {
-            float *q = (float *)dst + dst_off;
-            if (((uintptr_t)q & 15) == 0) {
-                *(float4 *)q = make_float4(d[0], d[1], d[2], d[3]);
-                return;
-            }
+            // (one 16-byte store at any 4-byte address)
+            typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+            *(v4f_any *)((float *)dst + dst_off) = v4f_any {d[0], d[1], d[2], d[3]};
+            return;
         } else if (dt == dt_s8 || dt == dt_u8) {
-            uint8_t *q = (uint8_t *)dst + dst_off;
-            if (((uintptr_t)q & 3) == 0) {
-                uint32_t w = 0;
+            // (one 4-byte store at any address)
+            typedef uint32_t u32_any __attribute__((aligned(1)));
+            uint32_t w = 0;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int r = dt == dt_s8 ? round_sat(d[i], -128.f, 127.f)
-                                              : round_sat(d[i], 0.f, 255.f);
-                    w |= (uint32_t)(r & 0xff) << (8 * i);
-                }
-                *(uint32_t *)q = w;
-                return;
+            for (int i = 0; i < 4; i++) {
+                const int r = dt == dt_s8 ? round_sat(d[i], -128.f, 127.f)
+                                          : round_sat(d[i], 0.f, 255.f);
+                w |= (uint32_t)(r & 0xff) << (8 * i);
             }
+            *(u32_any *)((uint8_t *)dst + dst_off) = w;
+            return;
         }
     }
 #pragma unroll
