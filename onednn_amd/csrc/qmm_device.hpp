@@ -559,29 +559,25 @@ QMM_D void ep_load4(const ep_tensor_t &t, int64_t b, int64_t m, int64_t n,
         return;
     }
     if (t.sn == 1 && nvalid == 4) {
+        // one vector load at any address (global loads need no alignment)
         if (t.dt == dt_f32) {
-            const float *q = (const float *)t.ptr + off;
-            if (((uintptr_t)q & 15) == 0) {
-                const float4 v = *(const float4 *)q;
-                o[0] = v.x;
-                o[1] = v.y;
-                o[2] = v.z;
-                o[3] = v.w;
-                return;
-            }
+            typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+            const v4f_any v = *(const v4f_any *)((const float *)t.ptr + off);
+            o[0] = v[0];
+            o[1] = v[1];
+            o[2] = v[2];
+            o[3] = v[3];
+            return;
         } else if (t.dt == dt_f16 || t.dt == dt_bf16) {
-            const uint16_t *q = (const uint16_t *)t.ptr + off;
-            if (((uintptr_t)q & 7) == 0) {
-                const uint2 v = *(const uint2 *)q;
-                const uint16_t h[4] = {(uint16_t)v.x, (uint16_t)(v.x >> 16),
-                        (uint16_t)v.y, (uint16_t)(v.y >> 16)};
+            typedef unsigned v2u_any __attribute__((ext_vector_type(2), aligned(2)));
+            const v2u_any v = *(const v2u_any *)((const uint16_t *)t.ptr + off);
+            const uint16_t h[4] = {(uint16_t)v[0], (uint16_t)(v[0] >> 16),
+                    (uint16_t)v[1], (uint16_t)(v[1] >> 16)};
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    o[i] = t.dt == dt_f16
-                            ? (float)__builtin_bit_cast(_Float16, h[i])
-                            : bf16_to_f32(h[i]);
-                return;
-            }
+            for (int i = 0; i < 4; i++)
+                o[i] = t.dt == dt_f16 ? (float)__builtin_bit_cast(_Float16, h[i])
+                                      : bf16_to_f32(h[i]);
+            return;
         }
     }
 #pragma unroll
