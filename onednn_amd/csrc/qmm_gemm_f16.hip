@@ -442,7 +442,8 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     auto pick = [](int g, int len) { return g >= 8 && len % 8 == 0 ? 8 : len >= 8 ? 0 : 1; };
     int ga = pick(p.a_vec, p.K), gb = pick(p.b_vec, p.N);
     const bool light = light_epilogue(p.ep) && p.ep.dst.sn == 1;
-    if (!light && !(ga == 8 && gb == 8)) ga = gb = 1; // the interpreter form exists twice
+    // the interpreter form exists three times: aligned, any alignment, short rows
+    if (!light && !(ga == 8 && gb == 8)) ga = gb = (ga != 1 && gb != 1) ? 0 : 1;
     auto go = [&](auto bf, auto lt, auto a, auto b) {
         hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
                                    decltype(a)::value, decltype(b)::value>),
@@ -457,6 +458,7 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     using I1 = std::integral_constant<int, 1>;
     if (!light) {
         if (ga == 8) by_bf(std::false_type {}, I8 {}, I8 {});
+        else if (ga == 0) by_bf(std::false_type {}, I0 {}, I0 {});
         else by_bf(std::false_type {}, I1 {}, I1 {});
         return;
     }

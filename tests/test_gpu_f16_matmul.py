@@ -59,6 +59,8 @@ CASES = {
     "two_rows_narrow": dict(sd=[3, 2, 64], wd=[3, 64, 8]),
     "one_row_long_k": dict(sd=[1, 8192], wd=[8192, 520]),
     "two_rows_k_past_the_table": dict(sd=[2, 4100], wd=[4100, 96]),
+    "odd_rows_with_bias_and_f32_dst": dict(sd=[2, 70, 250], wd=[2, 250, 99], bias=True, dst_dt=dt.f32),
+    "odd_rows_with_bias_bf16": dict(sd=[3, 33, 77], wd=[3, 77, 51], bias=True, code=dt.bf16),
     "tiny_k": dict(sd=[2, 5, 8], wd=[2, 8, 16]),
     "odd_everything": dict(sd=[2, 67, 45], wd=[2, 45, 51]),
 }
