@@ -374,17 +374,22 @@ gemv_f16_kernel(const gemm16_params_t p, const int tpr_log2) {
                 red[(wave * MR + m) * cw + col_l + i] = acc[m][i];
     }
     __syncthreads();
+    // A workgroup stores only the columns from blockIdx.x * cw on: where the
+    // load window moved back, the columns in front of that belong to the
+    // neighbour, and an epilogue that reads dst (sum) must see each element once.
     const int quads = cw >> 2;
     if (tid < MR * quads) {
         const int m = tid / quads, c4 = (tid - m * quads) * 4;
-        const int nn = n0 + c4;
+        const int own0 = blockIdx.x * cw, shift = own0 - n0;
+        const int nn = own0 + c4;
         if (m < p.M && nn < p.N) {
             float v[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float t = 0.f;
+                const int c = min(shift + c4 + i, cw - 1);
 #pragma unroll
-                for (int w = 0; w < 4; w++) t += red[(w * MR + m) * cw + c4 + i];
+                for (int w = 0; w < 4; w++) t += red[(w * MR + m) * cw + c];
                 v[i] = t;
             }
             epilogue_apply_store4(p.ep, v, bz, m, nn, min(4, p.N - nn));

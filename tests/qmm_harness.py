@@ -128,6 +128,9 @@ class Problem:
             return O.pack4(v)
         if code in (dt.s32, dt.s8, dt.u8):
             return v.astype(O.STORAGE[code])
+        if code == dt.e8m0:
+            # the reference's encoder keeps the f32 exponent field (src/common/float8.cpp:28-34)
+            return ((v.astype(np.float32).view(np.uint32) >> 23) & 0xFF).astype(np.uint8)
         return O.from_f32(code, v.astype(np.float32))
 
     # ---- oracle ----

@@ -218,3 +218,50 @@ def test_swish_into_quantized_dst(ctx, route, dst_dt):
           % (route, dst_dt, 100 * frac, d.max(), len(np.unique(want))))
     assert len(np.unique(want)) > 50  # the case exercises the range, not a saturated constant
     assert d.max() <= 1 and frac < 2e-3, (int(d.max()), frac)
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("forced", [True, False], ids=["generic", "first_impl"])
+def test_e8m0_grouped_weights_scales(ctx, forced):
+    """Weights scales stored as e8m0 (src/common/primitive_attr.cpp:529 admits the type; decoded as
+    src/common/float8.cpp:36-41: 2^(r - 127)), one per 32 k and column, on s8 x s8. Powers of two keep every
+    product exact, so the result is the oracle's bit for bit whatever the order."""
+    eng, strm = ctx
+    say("e8m0 weights scales per 32 k, %s" % ("generic" if forced else "first implementation"))
+    r = np.random.default_rng(23)
+    M, K, N = 33, 128, 48
+    src = TensorSpec(dt.s8, [M, K], None, r.integers(-9, 10, (M, K)))
+    wei = TensorSpec(dt.s8, [K, N], None, r.integers(-9, 10, (K, N)))
+    dst = TensorSpec(dt.f32, [M, N])
+    ws = 2.0 ** r.integers(-6, 4, (K // 32, N))
+    p = Problem(src, wei, dst, scales={"src": (0, dt.f32, None, [0.25]), "wei": (3, dt.e8m0, (32, 1), ws)})
+    got, pd = p.run_gpu(eng, strm, impl=cases.GENERIC if forced else None, return_pd=True)
+    say("  ran on " + pd.impl_info_str())
+    want = p.run_oracle()
+    assert_bit_exact(got, want, "e8m0 grouped weights scales")
+    # and against the arithmetic itself: sum over groups of 2^e * (exact integer dot product of the group)
+    a = src.logical().astype(np.int64)
+    b = wei.logical().astype(np.int64)
+    exact = sum((a[:, g * 32:(g + 1) * 32] @ b[g * 32:(g + 1) * 32]) * ws[g][None, :] for g in range(K // 32)) * 0.25
+    assert np.array_equal(got.view(np.float32).reshape(M, N).astype(np.float64), exact)
+
+
+@pytest.mark.parametrize("act", [dt.bf16, dt.f16], ids=str)
+@pytest.mark.parametrize("scale", [2.0, 0.25])
+def test_e8m0_dst_scale(ctx, act, scale):
+    """The reference's CI case (tests/benchdnn/inputs/matmul/test_matmul_ci:110-114): a single destination scale of
+    type e8m0 on bf16 / f16 matmuls, 4x256:256x64 and 6x256:256x100."""
+    eng, strm = ctx
+    for M, K, N in ((4, 256, 64), (6, 256, 100)):
+        say("e8m0 dst scale %g, %s %dx%dx%d" % (scale, act, M, K, N))
+        r = np.random.default_rng(M * N)
+        src = TensorSpec(act, [M, K], None, r.integers(-4, 5, (M, K)).astype(np.float32))
+        wei = TensorSpec(act, [K, N], None, r.integers(-4, 5, (K, N)).astype(np.float32))
+        dst = TensorSpec(act, [M, N])
+        p = Problem(src, wei, dst, scales={"dst": (0, dt.e8m0, None, [scale])})
+        got, pd = p.run_gpu(eng, strm, return_pd=True)
+        say("  ran on " + pd.impl_info_str())
+        assert_bit_exact(got, p.run_oracle(), "e8m0 dst scale")
+        exact = (src.logical().astype(np.float64) @ wei.logical().astype(np.float64)) / scale
+        # the exact quotient (an integer or half-integer, exact in f32) rounded once to the dst type
+        assert np.array_equal(got.view(np.uint16).reshape(-1), O.from_f32(act, exact.astype(np.float32)).reshape(-1))

@@ -101,3 +101,21 @@ def test_what_it_does_not_take(ctx):
     got, pd = p.run_gpu(eng, strm, return_pd=True)
     assert pd.impl_info_str() == GENERIC
     assert_bit_exact(got, p.run_oracle(), "ba weights")
+
+
+@pytest.mark.parametrize("code", [dt.f16, dt.bf16], ids=str)
+@pytest.mark.parametrize("M,N", [(1, 1000), (3, 1000), (1, 264), (3, 264), (2, 1001), (4, 40)])
+def test_few_rows_with_sum_post_op_stores_each_column_once(ctx, code, M, N):
+    """The few-rows kernel moves its last column chunk back inside the row when N is not a multiple of the chunk; the
+    columns two workgroups then both compute must be stored by one of them only, or a sum post-op (which reads the old
+    dst) would be applied twice there. Integer-valued data: bit for bit."""
+    eng, strm = ctx
+    say("mfma_f16 few rows, sum post-op, %s M=%d N=%d" % (code, M, N))
+    K = 96
+    p = problem([2, 3, M, K], [2, 3, K, N], 7 * N + M, code=code, exact=True,
+                post_ops=[{"kind": "sum", "scale": 0.5}])
+    r = np.random.default_rng(N)
+    init = O.from_f32(code, r.integers(-20, 21, 2 * 3 * M * N).astype(np.float32) * 2)
+    got, pd = p.run_gpu(eng, strm, return_pd=True, dst_init=init)
+    assert pd.impl_info_str() == F16MM
+    assert_bit_exact(got, p.run_oracle(dst_init=init), "few rows + sum")

@@ -7,11 +7,11 @@ in f32, one k at a time (the oracle's KGROUP_LITERAL mode). The two agree bit
 for bit while every partial sum is exactly representable and differ by f32
 summation error otherwise. These tests measure that difference on the benchmark
 configurations and cap it:
-  * integer dst: never more than one unit apart, and rarely;
+  * integer dst: the same bytes;
   * f32 dst: the share of elements further than rel 1e-5 of |want| apart is
-    small, and every element is within 1e-5 of the magnitude of the summed
-    terms.
-The measured shares are printed ([literal] lines)."""
+    small, and every element is within a few percent of 1e-5 of the magnitude
+    of the summed terms.
+The measured shares are printed ([literal] lines); each cap is twice what was measured."""
 import sys
 
 import numpy as np
@@ -58,8 +58,9 @@ def test_config1_f32_against_literal(ctx):
     beyond, worst = f32_shares(got, want, cases.term_scale(p))
     print("[literal] config 1 f32: %.4f %% of the elements beyond rel 1e-5 of |want|; worst error %.3f x 1e-5 of the term scale"
           % (100 * beyond, worst), flush=True)
-    assert worst <= 1.0
-    assert beyond <= 0.05
+    # measured: 1.97 % beyond, worst 0.023 units; the caps are twice that (data and arithmetic are deterministic)
+    assert worst <= 0.05
+    assert beyond <= 0.04
 
 
 def test_config4_f32_against_literal(ctx):
@@ -93,8 +94,10 @@ def test_config4_f32_against_literal(ctx):
     beyond, worst = f32_shares(got, want, term)
     print("[literal] config 4 f32: %.4f %% of the elements beyond rel 1e-5 of |want|; worst error %.3f x 1e-5 of the term scale"
           % (100 * beyond, worst), flush=True)
-    assert worst <= 1.0
-    assert beyond <= 0.10  # scores cancel towards 0: relative to |want| alone many tiny results are "far"
+    # measured: 0.71 % beyond (scores cancel towards 0: relative to |want| alone tiny results are "far"), worst
+    # 0.029 units; the caps are twice that
+    assert worst <= 0.06
+    assert beyond <= 0.015
 
 
 def test_config2_slice_bf16_against_literal(ctx):
@@ -117,15 +120,17 @@ def test_config2_slice_bf16_against_literal(ctx):
           "(max distance %d, all of them within %.3f x 1e-5 of the term scale)"
           % (100 * share, 100 * float(far.mean()), int(d.max()),
              float((err[far] / (1e-5 * term[far])).max()) if far.any() else 0.0), flush=True)
-    assert (err[far] <= 1e-5 * term[far]).all()
-    assert float(far.mean()) <= 0.001
-    assert share <= 0.02
+    # measured: 0.082 % differ, 0.0051 % by more than one value, those within 0.006 units; caps are twice that
+    assert (err[far] <= 0.012 * 1e-5 * term[far]).all()
+    assert float(far.mean()) <= 0.0001
+    assert share <= 0.0017
 
 
 @pytest.mark.parametrize("name", ["u8_zp_7_s8_dst", "s8_u8_dst_relu"])
 def test_integer_dst_against_literal(ctx, name):
-    """s8 / u8 dst (dst scale, zero point, bias, relu): at most one unit from the
-    literal reference, on a small share of the elements."""
+    """s8 / u8 dst (dst scale, zero point, bias, relu): the same bytes as the literal reference (its f32 summation
+    error is far below the rounding step of an 8-bit result on these cases, and data and arithmetic are
+    deterministic)."""
     eng, strm = ctx
     say("integer dst %s vs the literal reference" % name)
     p = cases.MFMA_CASES[name][0]()
@@ -137,5 +142,4 @@ def test_integer_dst_against_literal(ctx, name):
     diff = np.abs(g - w)
     share = float((diff > 0).mean())
     print("[literal] %s: %.4f %% of the elements differ, max |diff| %d" % (name, 100 * share, int(diff.max())), flush=True)
-    assert diff.max() <= 1
-    assert share <= 0.01
+    assert diff.max() == 0 and share == 0.0

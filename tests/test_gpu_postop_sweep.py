@@ -93,7 +93,24 @@ def test_eltwise_algorithm(ctx, route, name):
         po, p.post_ops = p.post_ops, []
         term = 0.5 * np.abs(p.run_oracle().view(np.float32))
         p.post_ops = po
-    _check(_run(ctx, route, p), p.run_oracle(), exact, "%s %s" % (name, route), term)
+    got, want = _run(ctx, route, p), p.run_oracle()
+    _check(got, want, exact, "%s %s" % (name, route), term)
+    if name == "eltwise_gelu_erf":
+        # 0.5 x (1 + erf(x / sqrt 2)): for negative x the bracket is a difference of numbers near 1, so an erff that
+        # is good to an ulp or two of ITS result (2^-24) leaves the product good to that many units of 2^-24 x 0.5 |x|
+        # only. Both sides against the exact value (float64 erf): the device's erff must be as good as the host's.
+        from scipy.special import erf
+        po, p.post_ops = p.post_ops, []
+        x = p.run_oracle().view(np.float32).astype(np.float64).reshape(-1)
+        p.post_ops = po
+        exact64 = 0.5 * x * (1.0 + erf(x / np.sqrt(2.0)))
+        unit = 2.0 ** -24 * np.maximum(0.5 * np.abs(x), 1e-30)
+        e_gpu = np.abs(got.view(np.float32).astype(np.float64).reshape(-1) - exact64) / unit
+        e_ref = np.abs(want.view(np.float32).astype(np.float64).reshape(-1) - exact64) / unit
+        print("[gelu_erf] %s: distance from the exact value in units of 2^-24 x 0.5|x|: kernel max %.2f mean %.3f, "
+              "host libm (the oracle) max %.2f mean %.3f" % (route, e_gpu.max(), e_gpu.mean(), e_ref.max(), e_ref.mean()),
+              flush=True)
+        assert e_gpu.max() <= 6.0 and e_gpu.mean() <= 1.0, (e_gpu.max(), e_gpu.mean())
 
 
 @pytest.mark.parametrize("route", ROUTES)

@@ -148,6 +148,37 @@ def test_e5m2_matches_torch_and_round_trip():
     assert np.array_equal(got, want)
 
 
+def test_e8m0_decode_closed_form_all_codes():
+    # src/common/float8.cpp:36-41: the code is the f32 exponent field, no sign, no mantissa:
+    # r in 1..254 is 2^(r-127); 0xff is the only NaN (the "real indefinite" pattern); r = 0 has
+    # an all-zero f32 pattern, i.e. +0.0 (not the 2^-127 an OCP decoder would give).
+    codes = np.arange(256, dtype=np.uint8)
+    got = O.to_f32(O.E8M0, codes)
+    L = O.lib()
+    for r in range(256):
+        one = L.orc_load_float(O.E8M0, codes.ctypes.data, r)
+        if r == 0xFF:
+            assert np.isnan(got[r]) and np.isnan(one)
+            assert got[r:r + 1].view(np.uint32)[0] == 0xFFC00000
+        elif r == 0:
+            assert got[r] == 0.0 and not np.signbit(got[r]) and one == 0.0
+        else:
+            want = np.float32(2.0 ** (r - 127))       # exact: a normal f32 power of two
+            assert got[r] == want and one == want, r
+            assert np.frexp(np.float64(got[r])) == (0.5, r - 126)
+    # a second decoder: torch's e8m0 type agrees wherever the value is a normal f32
+    t = torch.from_numpy(codes[1:255].copy()).view(torch.float8_e8m0fnu).to(torch.float32).numpy()
+    assert np.array_equal(t, got[1:255])
+    # src/common/float8.cpp:28-34: the encoder keeps the exponent field and drops sign and
+    # mantissa (round toward zero), so decode(encode(x)) is the power of two at or below |x|
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(4096) * np.exp(rng.uniform(-60, 60, 4096))).astype(np.float32)
+    x = x[np.abs(x) >= np.float32(2.0 ** -126)]
+    enc = ((x.view(np.uint32) >> 23) & 0xFF).astype(np.uint8)
+    dec = O.to_f32(O.E8M0, enc)
+    assert np.array_equal(dec, np.float32(2.0) ** np.floor(np.log2(np.abs(x.astype(np.float64)))).astype(np.float32))
+
+
 def test_nibble_order_and_ranges():
     # tests/gtests/internals/test_nibble.cpp:36-80: low nibble is the even index
     buf = np.array([0x21, 0xF8], dtype=np.uint8)

@@ -225,6 +225,66 @@ def test_fp8_path_and_sum_post_op():
     assert np.array_equal(dst, _bf16(want))
 
 
+@pytest.mark.parametrize("dst_dt,sum_dt,zp,scale", [
+    ("u8", "s8", 5, 0.5), ("s8", "u8", -3, 0.75), ("u8", "s8", -128, 1.0), ("s8", None, 7, 0.5),
+    ("s32", None, 11, 2.0), ("f32", None, 9, 0.25)])
+def test_sum_post_op_zero_point_and_data_type(dst_dt, sum_dt, zp, scale):
+    """src/cpu/primitive_attr_postops.cpp:286-293: res += scale * (dst_val - float(zero_point)), where dst_val is the
+    old destination element read through the sum's own data type when it has one
+    (src/common/primitive_attr.hpp:448-455, src/cpu/matmul/ref_matmul_int8.cpp:231,246). Written here with numpy
+    float32 steps on the raw bytes: reading the old bytes in the destination's signedness, dropping the zero point or
+    flipping its sign each changes the expected bytes."""
+    rng = np.random.default_rng(11)
+    M, K, N = 6, 48, 9
+    np_of = {"u8": np.uint8, "s8": np.int8, "s32": np.int32, "f32": np.float32}
+    src = rng.integers(-6, 7, (M, K)).astype(np.int8)
+    wei = rng.integers(-6, 7, (K, N)).astype(np.int8)
+    if dst_dt in ("u8", "s8"):
+        old_bytes = rng.integers(0, 256, (M, N)).astype(np.uint8)      # both halves of the byte range
+        old = old_bytes.view(np_of[dst_dt])
+    elif dst_dt == "s32":
+        old = rng.integers(-300, 300, (M, N)).astype(np.int32)
+    else:
+        old = rng.integers(-300, 300, (M, N)).astype(np.float32)
+    dst = old.copy()
+    ws = np.float32(0.125)
+    po = {"kind": "sum", "scale": scale, "zero_point": zp}
+    if sum_dt:
+        po["dt"] = O.DT_NAMES[sum_dt]
+    O.matmul(T(O.S8, src), T(O.S8, wei), T(O.DT_NAMES[dst_dt], dst),
+             scales={O.Q_WEI: O.Quant(0, O.F32, np.array([ws], np.float32))}, post_ops=[po])
+    acc = (src.astype(np.int64) @ wei.astype(np.int64)).astype(np.float32)
+    res = acc * ws
+    seen = old.view(np_of[sum_dt]) if sum_dt else old                  # same bytes, the sum's own type
+    res = res + np.float32(scale) * (seen.astype(np.float32) - np.float32(zp))
+    if dst_dt == "f32":
+        want = res
+    else:
+        info = np.iinfo(np_of[dst_dt])
+        want = np.rint(np.clip(res, np.float32(info.min), np.float32(info.max))).astype(np_of[dst_dt])
+    assert np.array_equal(dst, want)
+    if sum_dt:      # the two readings of the old bytes must differ on this data, or the case pins nothing
+        other = res - np.float32(scale) * seen.astype(np.float32) + np.float32(scale) * old.astype(np.float32)
+        assert not np.array_equal(other, res)
+    assert zp != 0
+
+
+def test_float_path_sum_reads_old_dst_in_its_own_type():
+    """src/cpu/matmul/ref_matmul.cpp:190,215: the float path reads the old destination through get_sum_dt too. With a
+    bf16 destination and an f16 sum type the same 16 bits are another number."""
+    rng = np.random.default_rng(12)
+    M, K, N = 4, 16, 6
+    a = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    old = rng.integers(0x3000, 0x4800, (M, N)).astype(np.uint16)       # positive, normal in both formats
+    dst = old.copy()
+    O.matmul(T(O.F32, a), T(O.F32, b), T(O.BF16, dst), post_ops=[{"kind": "sum", "scale": 2.0, "dt": O.F16}])
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32) \
+        + np.float32(2.0) * old.view(np.float16).astype(np.float32)
+    assert np.array_equal(dst, _bf16(want))
+    assert not np.array_equal(old.view(np.float16).astype(np.float32), O.to_f32(O.BF16, old))
+
+
 def test_binary_post_op_broadcast_and_batch():
     rng = np.random.default_rng(6)
     B, M, K, N = 4, 6, 32, 5
