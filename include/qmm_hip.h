@@ -153,7 +153,10 @@ QMM_API int qmm_matmul_launch(const qmm_plan_t *plan,
  * GPU share the buffer: calls that overlap in time on one GPU (different
  * streams or threads) race; calls on one stream do not. Every kernel writes
  * the part of the buffer it later reads, so nothing has to be cleared between
- * calls. */
+ * calls. The buffer is the one of the stream's device (the current device for
+ * the null stream); its address is looked up once per device, when a plan that
+ * fits is created with that device current, else at the first such launch
+ * there (a mutex and one hipGetSymbolAddress). */
 #define QMM_STATIC_SCRATCH_BYTES (32u << 20)
 QMM_API int qmm_matmul_launch_static_scratch(const qmm_plan_t *plan,
         const qmm_matmul_args_t *args, void *hip_stream);
@@ -243,18 +246,16 @@ QMM_API size_t qmm_sdpa_scratch_size(const qmm_sdpa_desc_t *desc);
 QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
         const qmm_sdpa_args_t *args, void *hip_stream);
 
-/* ---- tuning / test hooks ----
- * Process-wide kernel-selection overrides for A/B measurements and for tests
- * that must reach a particular kernel at sizes the oracle finishes quickly.
- * Atomic; a launch reads each once. Production code leaves them alone.
- *   gemm variant: 0 by problem size (default); 1..3 a tile configuration of
+/* ---- kernel-selection overrides ----
+ * For A/B measurements and for tests that must reach a particular kernel at
+ * sizes the oracle finishes quickly. Environment variables, read once when a
+ * plan is created (qmm_matmul_plan_create) and fixed for that plan's life; a
+ * launch reads no process-wide state. Production code leaves them unset.
+ *   QMM_GEMM_VARIANT: 0 by problem size (default); 1..3 a tile configuration of
  *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible
- *   w4a8 variant: 0 by problem size (default); 1..3 a tile configuration
- *   b8x variant: MFMA shape of the 256 x 256 kernels: 1 = 16 x 16 (default),
+ *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration
+ *   QMM_B8X_VARIANT: MFMA shape of the 256 x 256 kernels: 1 = 16 x 16 (default),
  *     0 = 32 x 32 */
-QMM_API void qmm_set_gemm_variant(int v);
-QMM_API void qmm_set_w4a8_variant(int v);
-QMM_API void qmm_set_b8x_variant(int v);
 
 /* ---- measurement aid ----
  * Launches a kernel that only reads: up to three byte ranges (16-byte aligned,
@@ -266,6 +267,19 @@ QMM_API void qmm_set_b8x_variant(int v);
 #define QMM_STREAM_READ_GROUPS 256
 QMM_API int qmm_stream_read(const void *p0, size_t n0, const void *p1,
         size_t n1, const void *p2, size_t n2, void *sink, void *stream);
+
+/* Launches `groups` workgroups of four waves that issue nothing but the MFMAs
+ * of the 256 x 256 GEMM kernels' main loop (`ksteps` k-steps, even, of the
+ * 128 x 128 wave tile) on register-resident operands (data 0: uniformly random
+ * bytes, 1: zeros, 2: the value distributions of the int8 / fp8 benchmark
+ * configurations): kind 0 = v_mfma_i32_16x16x64_i8, 1 = v_mfma_i32_32x32x32_i8,
+ * 2 = v_mfma_f32_16x16x128_f8f6f4, 3 = v_mfma_f32_32x32x64_f8f6f4 (e4m3). One word
+ * per lane goes to `sink` (groups * 1024 bytes); *ops_per_launch receives the
+ * multiply-add operations (x 2) of a launch. No counterpart in the reference;
+ * benchmarks time it to state what the matrix cores sustain on this card next
+ * to the published peak. */
+QMM_API int qmm_mfma_ceiling(int kind, int ksteps, int groups, int data,
+        void *sink, void *hip_stream, double *ops_per_launch);
 
 /* ---- device queries used by the engine ---- */
 QMM_API int qmm_device_count(void);

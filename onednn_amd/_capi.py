@@ -4,6 +4,7 @@ The library must have been built (python -m onednn_amd.build, or
 __graft_entry__.build()); loading fails loudly otherwise. There is no CPU
 fallback of any kind.
 """
+import contextlib
 import ctypes as C
 import os
 
@@ -137,10 +138,8 @@ _SIGNATURES = {
     "qmm_matmul_impl_count": (_I, []),
     "qmm_matmul_impl_name": (C.c_char_p, [_I]),
     "qmm_reorder_impl_name": (C.c_char_p, [_P]),
-    "qmm_set_gemm_variant": (None, [_I]),
-    "qmm_set_w4a8_variant": (None, [_I]),
-    "qmm_set_b8x_variant": (None, [_I]),
     "qmm_stream_read": (_I, [_P, C.c_size_t, _P, C.c_size_t, _P, C.c_size_t, _P, _P]),
+    "qmm_mfma_ceiling": (_I, [_I, _I, _I, _I, _P, _P, C.POINTER(C.c_double)]),
 }
 
 _lib = None
@@ -159,11 +158,27 @@ def lib():
             f = getattr(L, name)
             f.argtypes = args
             f.restype = _I if res is None else res
-        L.qmm_set_gemm_variant.restype = None
-        L.qmm_set_w4a8_variant.restype = None
-        L.qmm_set_b8x_variant.restype = None
         _lib = L
     return _lib
+
+
+@contextlib.contextmanager
+def kernel_variants(gemm=None, w4a8=None, b8x=None):
+    """Kernel-selection overrides (include/qmm_hip.h) for the plans created inside the block: environment variables
+    the library reads at plan creation, restored on exit."""
+    names = {"QMM_GEMM_VARIANT": gemm, "QMM_W4A8_VARIANT": w4a8, "QMM_B8X_VARIANT": b8x}
+    old = {k: os.environ.get(k) for k in names}
+    try:
+        for k, v in names.items():
+            if v is not None:
+                os.environ[k] = str(int(v))
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
 
 
 def check(status, what):

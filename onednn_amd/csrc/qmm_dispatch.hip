@@ -24,7 +24,7 @@ void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, hipStream_t stream);
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream);
-void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
+bool launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream);
@@ -63,7 +63,6 @@ void launch_unpack_w8(const void *src, void *dst, int dt, int64_t batch,
 void launch_unpack_w4(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
-void set_gemm_b8x_variant(int v);
 } // namespace qmm
 
 using namespace qmm;
@@ -716,8 +715,16 @@ const char *impl_names[impl_count] = {"hip:gfx950:mfma_b8",
         "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:mfma_f16",
         "hip:gfx950:generic"};
 
-std::atomic<int> g_gemm_variant {0};
-std::atomic<int> g_w4a8_variant {0};
+// A kernel-selection override from the environment: an integer in [lo, hi],
+// else the default.
+int env_variant(const char *name, int lo, int hi, int dflt) {
+    const char *v = std::getenv(name);
+    if (!v || !*v) return dflt;
+    char *end = nullptr;
+    const long x = std::strtol(v, &end, 10);
+    if (end == v || *end || x < lo || x > hi) return dflt;
+    return (int)x;
+}
 
 } // namespace
 
@@ -852,6 +859,8 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
     return 0;
 }
 
+static void *static_scratch_ptr(hipStream_t stream);
+
 int qmm_matmul_plan_create(
         qmm_plan_t **plan, int impl, const qmm_matmul_desc_t *desc) {
     if (!plan || !desc) return QMM_INVALID_ARGUMENTS;
@@ -864,6 +873,14 @@ int qmm_matmul_plan_create(
     p->dev = nullptr;
     build_generic(p->host, *desc);
     p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
+    p->gemm_variant = env_variant("QMM_GEMM_VARIANT", 0, 6, 0);
+    p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 3, 0);
+    p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 1, 1);
+    // resolve the static scratch's address on the current device now, so that
+    // qmm_matmul_launch_static_scratch() finds it ready (a plan used on another
+    // device resolves it at its first launch there)
+    if (p->scratch_bytes && p->scratch_bytes <= (size_t)QMM_STATIC_SCRATCH_BYTES)
+        (void)static_scratch_ptr(nullptr);
     // the generic kernel reads its (large) descriptor from device memory; the
     // tiled kernels fall back to it for operands they cannot address (pointers
     // that are not 16-byte aligned), so every plan over plain weights keeps one
@@ -903,19 +920,32 @@ static bool aligned16(const void *p) {
 // once per device (with that device current) and kept.
 static __device__ __align__(256) unsigned char scratch[QMM_STATIC_SCRATCH_BYTES];
 
-static void *static_scratch_ptr() {
+// `stream`: the device is the stream's when it names one (a launch may target
+// a device that is not the calling thread's current one), else the current one.
+static void *static_scratch_ptr(hipStream_t stream) {
     constexpr int MAX_DEV = 64;
     static std::mutex mu;
     static void *ptr[MAX_DEV] = {};
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
-        g_last_error = "no current HIP device for the static scratch";
+    if (!stream || hipStreamGetDevice(stream, &dev) != hipSuccess) {
+        if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+    }
+    if (dev < 0 || dev >= MAX_DEV) {
+        g_last_error = "no HIP device for the static scratch";
         return nullptr;
     }
     std::lock_guard<std::mutex> lock(mu);
     if (!ptr[dev]) {
+        // the symbol's address is per device: ask with that device current
+        int cur = -1;
+        (void)hipGetDevice(&cur);
+        if (cur != dev && hipSetDevice(dev) != hipSuccess) {
+            g_last_error = "hipSetDevice for the static scratch failed";
+            return nullptr;
+        }
         void *q = nullptr;
         const hipError_t e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (cur != dev && cur >= 0) (void)hipSetDevice(cur);
         if (e != hipSuccess || !q) {
             g_last_error = std::string("hipGetSymbolAddress(scratch): ")
                     + hipGetErrorString(e);
@@ -936,7 +966,7 @@ int qmm_matmul_launch_static_scratch(const qmm_plan_t *plan,
     qmm_matmul_args_t a = *args;
     a.scratch = nullptr;
     if (plan->scratch_bytes) {
-        a.scratch = static_scratch_ptr();
+        a.scratch = static_scratch_ptr((hipStream_t)hip_stream);
         if (!a.scratch) return QMM_RUNTIME_ERROR;
     }
     return qmm_matmul_launch(plan, &a, hip_stream);
@@ -967,11 +997,8 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
     if (plan->scratch_bytes && !args->scratch)
         return fail(QMM_INVALID_ARGUMENTS, "scratch buffer is missing");
 
-    // one read per launch: a launch never sees two values of a tuning hook
-    const int gemm_variant = g_gemm_variant.load(std::memory_order_relaxed);
-    const int w4a8_variant = g_w4a8_variant.load(std::memory_order_relaxed);
-    (void)gemm_variant;
-    (void)w4a8_variant;
+    const int gemm_variant = plan->gemm_variant;
+    const int w4a8_variant = plan->w4a8_variant;
     int impl = plan->impl;
     if (impl != impl_generic && impl != impl_gemm_f16 && !aligned16(args->src)) {
         if (!plan->dev)
@@ -991,6 +1018,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
         g.A = (const uint8_t *)args->src;
         g.lda = D.src.strides[nd - 2];
+        g.b8x_mfma32 = plan->b8x_variant == 0;
         fold_batch(D.src, D.dst, g.a_sb);
         const int64_t wb = wei_batch(D);
         const b8_geom_t geom = b8_geom(wb, P.K, P.N);
@@ -1264,29 +1292,16 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.wei_signed = D.wei.dt == dt_s4 || D.wei.dt == dt_s8;
         g.act_f16 = D.src.dt == dt_f16;
         g.m0 = 0;
-        launch_gemv_w4(g, stream);
+        if (!launch_gemv_w4(g, stream))
+            return fail(QMM_RUNTIME_ERROR,
+                    "decode_w4: no kernel takes this problem (8-bit weights "
+                    "outside the forms the implementation admits)");
     } else {
         return fail(QMM_INVALID_ARGUMENTS, "unknown implementation");
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "kernel launch");
     return QMM_OK;
-}
-
-// Tuning / test hooks (declared in qmm_hip.h): process-wide, atomic, read once
-// per launch. The default of each (0, 0, 1) is what the implementations are
-// tuned and documented for.
-// tile configuration of mfma_b8
-QMM_API void qmm_set_gemm_variant(int v) {
-    g_gemm_variant = v;
-}
-// same for mfma_w4a8 (0: by problem size, 1..3: tile configuration)
-QMM_API void qmm_set_w4a8_variant(int v) {
-    g_w4a8_variant = v;
-}
-// the 256 x 256 int8 kernel's MFMA shape (0: 32 x 32 x 32, 1: 16 x 16 x 64)
-QMM_API void qmm_set_b8x_variant(int v) {
-    qmm::set_gemm_b8x_variant(v);
 }
 
 // ---------------------------------------------------------------------------

@@ -29,7 +29,6 @@
 // arithmetic as src/cpu/matmul/ref_matmul_int8.cpp:195-259); only epilogues of
 // the straight-line kinds (EP_FAST_*) are handled here, everything else stays
 // with the general kernel.
-#include <atomic>
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -1496,15 +1495,12 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
-// 0: the loops on 32 x 32 MFMAs; 1: int8 on 16 x 16 x 64 (at least 5 k-steps)
-// and fp8 on 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply
-static std::atomic<int> g_b8x_variant {1};
-void set_gemm_b8x_variant(int v) {
-    g_b8x_variant = v;
-}
-
+// By default int8 runs on 16 x 16 x 64 MFMAs (at least 5 k-steps) and fp8 on
+// 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply;
+// p.b8x_mfma32 (a plan-level override for A/B measurements) keeps the loops on
+// 32 x 32 MFMAs.
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
-    const int variant = g_b8x_variant.load(std::memory_order_relaxed);
+    const int variant = p.b8x_mfma32 ? 0 : 1;
     if (f8 && variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)

@@ -600,8 +600,9 @@ void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
         hipStream_t stream);
 bool gemm_w4f_wins(const gemv_params_t &p);
 
-void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
-    if (p.M <= 0 || p.N <= 0) return;
+// Returns false when no kernel takes the problem (nothing is launched then).
+bool launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
+    if (p.M <= 0 || p.N <= 0) return true;
     const int rows = p.M < 16 ? p.M : 16;
     int MR = 1;
     while (MR < rows) MR *= 2;
@@ -664,7 +665,7 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         // for 32 or 64 rows) where it beats this one once per block of 16 rows.
         if (gemm_w4f_wins(p)) {
             launch_gemm_w4f(q, shifts, flags_m, stream);
-            return;
+            return true;
         }
         // more than 8 rows in at most one workgroup per CU: the variant that
         // stages its activations in LDS
@@ -714,9 +715,12 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
             by_rows(std::true_type {});
         else
             by_rows(std::false_type {});
-        return;
+        return true;
     }
-    if (p.w8) return; // not reachable: creation admits fast-variant problems only
+    // 8-bit weights exist in the all-unconditional-loads form only; creation
+    // admits nothing else, and a drift between the two checks must not pass
+    // as a launch that wrote nothing
+    if (p.w8) return false;
     auto launch = [&](auto kern) {
         ensure_dynamic_lds((const void *)kern, GEMV_LDS_BUDGET);
         hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, q,
@@ -726,6 +730,7 @@ void launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         launch(gemv_w4_kernel<true>);
     else
         launch(gemv_w4_kernel<false>);
+    return true;
 }
 
 } // namespace qmm

@@ -160,7 +160,8 @@ struct gemm_params_t {
     // point of the stored weights is zp[n * wei_zp_sn] - w_off, applied through
     // rowsum (see rowsum_b8_kernel); nullptr rowsum: neither
     const void *wei_zp; // nullptr: 0
-    int32_t wei_zp_dt, wei_zp_sn, w_off, pad2_;
+    int32_t wei_zp_dt, wei_zp_sn, w_off;
+    int32_t b8x_mfma32; // host-side: the 256 x 256 loops on 32 x 32 MFMAs (QMM_B8X_VARIANT=0)
     const int32_t *rowsum; // [batch][M]
     epilogue_t ep;
 };
@@ -299,4 +300,8 @@ struct qmm_plan {
     qmm::generic_params_t *dev; // device copy, used by the generic kernel
     qmm_matmul_desc_t desc;
     size_t scratch_bytes;
+    // kernel-selection overrides (qmm_hip.h: QMM_GEMM_VARIANT, QMM_W4A8_VARIANT,
+    // QMM_B8X_VARIANT), read from the environment when the plan is created and
+    // fixed for the plan's life
+    int gemm_variant, w4a8_variant, b8x_variant;
 };

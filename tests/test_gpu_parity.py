@@ -343,9 +343,8 @@ def test_mfma_int8_against_literal_v38_reference(ctx):
 @pytest.fixture
 def tile256():
     from onednn_amd import _capi
-    _capi.lib().qmm_set_gemm_variant(6)
-    yield
-    _capi.lib().qmm_set_gemm_variant(0)
+    with _capi.kernel_variants(gemm=6):
+        yield
 
 
 def _tiny_scale_problem():
@@ -495,11 +494,8 @@ def test_mfma_int8_tile256_mi16_loop(ctx, tile256, name):
     got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
     assert pd.impl_info_str() == MFMA
     assert_bit_exact(got, p.run_oracle(), name)
-    _capi.lib().qmm_set_b8x_variant(0)
-    try:
+    with _capi.kernel_variants(b8x=0):
         other = p.run_gpu(eng, strm, weights_any=True)
-    finally:
-        _capi.lib().qmm_set_b8x_variant(1)
     assert_bit_exact(other, got, name + " (32x32x32 loop)")
 
 
@@ -567,8 +563,7 @@ def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
     shapes = ((256, 512, 256, dt.bf16, True), (300, 768, 260, dt.f32, False),
               (128, 1024, 512, dt.bf16, False), (512, 2048, 256, dt.f32, False))
     for variant in (1, 0):
-        _capi.lib().qmm_set_b8x_variant(variant)
-        try:
+        with _capi.kernel_variants(b8x=variant):
             for (M, K, N, dd, with_sum) in shapes:
                 say("mfma_b8 256x256 fp8 kernel, variant %d, %dx%dx%d" % (variant, M, K, N))
                 p = fp8_gemm(M, K, N, 178, dst_dt=dd, with_sum=with_sum)
@@ -582,8 +577,6 @@ def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
                     assert_f32_close(got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N),
                                      rel=1e-5, scale=a, what="fp8 f32", max_slack_frac=FP8_F32_SLACK)
                     assert_fp8_f32_error_against_exact(p, got, want, "256x256 kernel variant %d" % variant)
-        finally:
-            _capi.lib().qmm_set_b8x_variant(1)
 
 
 def test_mfma_fp8_tile256_f16_dst_bias_relu(ctx, tile256):

@@ -58,11 +58,8 @@ def _run(ctx, route, p):
     eng, strm = ctx
     if route == "generic":
         return p.run_gpu(eng, strm, impl=cases.GENERIC)
-    _capi.lib().qmm_set_gemm_variant(6 if route == "tile256" else 2)
-    try:
+    with _capi.kernel_variants(gemm=6 if route == "tile256" else 2):
         got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
-    finally:
-        _capi.lib().qmm_set_gemm_variant(0)
     assert pd.impl_info_str() == cases.MFMA
     return got
 

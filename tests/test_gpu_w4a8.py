@@ -36,9 +36,8 @@ def ctx():
 
 @pytest.fixture(params=[0, 1, 2, 3])
 def variant(request):
-    _capi.lib().qmm_set_w4a8_variant(request.param)
-    yield request.param
-    _capi.lib().qmm_set_w4a8_variant(0)
+    with _capi.kernel_variants(w4a8=request.param):
+        yield request.param
 
 
 def dynamic_quant(M, K, N, seed, wei_dt=dt.s4, gs=128, gw=128, gz=None, zp_dt=dt.u8, exact=False,
