@@ -187,6 +187,20 @@ struct pd_impl_t {
     bool runtime = false;
 };
 
+// A library-owned scratchpad is one buffer per primitive (or per cached shape
+// of a runtime-dims primitive), so launches of that primitive from different
+// streams (host threads) must not overlap on the device. The guard orders them:
+// under its mutex a launch on another stream than the previous one first waits
+// for an event recorded behind the previous launch. Launches on one stream pay
+// one event record each, and only when the primitive uses such a scratchpad.
+struct scratch_guard_t {
+    std::mutex mu;
+    void *event = nullptr; // hipEvent_t, created on first use
+    void *last_stream = nullptr;
+    bool used = false;
+    ~scratch_guard_t();
+};
+
 // One resolved shape of a runtime-dims matmul: the concrete descriptor, its
 // plan and a library-owned scratchpad. Owned by the primitive's cache.
 struct rt_entry_t {
@@ -194,6 +208,7 @@ struct rt_entry_t {
     std::shared_ptr<pd_impl_t> pd;
     qmm_plan_t *plan = nullptr;
     void *scratch = nullptr;
+    scratch_guard_t guard; // orders launches that share `scratch`
     uint64_t stamp = 0;
     ~rt_entry_t();
 };
@@ -207,6 +222,7 @@ struct dnnl_primitive {
     dnnl_primitive_desc pd_handle; // what dnnl_primitive_get_primitive_desc returns
     qmm_plan_t *plan = nullptr;
     void *lib_scratch = nullptr; // library-managed scratchpad
+    mutable scratch_guard_t guard; // orders launches that share lib_scratch
     // runtime dims: the shapes seen so far, least recently used evicted
     std::mutex rt_mutex;
     std::vector<std::shared_ptr<rt_entry_t>> rt;

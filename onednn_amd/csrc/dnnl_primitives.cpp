@@ -697,6 +697,46 @@ dnnl_status_t resolve_runtime_matmul(dnnl_primitive *prim,
 
 } // namespace
 
+scratch_guard_t::~scratch_guard_t() {
+    if (event) (void)hipEventDestroy((hipEvent_t)event);
+}
+
+namespace {
+// Holds the guard's mutex from before the launch until the event behind it is
+// recorded. A stream under capture is left alone (an event recorded outside the
+// capture cannot be waited for inside it): whoever captures orders the launches.
+struct scratch_order_t {
+    scratch_guard_t *g = nullptr;
+    hipStream_t stream = nullptr;
+    bool active = false;
+    scratch_order_t(scratch_guard_t *guard, void *hip_stream) {
+        if (!guard) return;
+        stream = (hipStream_t)hip_stream;
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &cs) == hipSuccess
+                && cs != hipStreamCaptureStatusNone)
+            return;
+        g = guard;
+        g->mu.lock();
+        active = true;
+        if (g->used && g->last_stream != hip_stream && g->event)
+            (void)hipStreamWaitEvent(stream, (hipEvent_t)g->event, 0);
+    }
+    ~scratch_order_t() {
+        if (!active) return;
+        if (!g->event) {
+            hipEvent_t e = nullptr;
+            if (hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess)
+                g->event = e;
+        }
+        if (g->event) (void)hipEventRecord((hipEvent_t)g->event, stream);
+        g->last_stream = (void *)stream;
+        g->used = true;
+        g->mu.unlock();
+    }
+};
+} // namespace
+
 // An evicted or destroyed shape: hipFree waits for the kernels that still use
 // the scratchpad.
 rt_entry_t::~rt_entry_t() {
@@ -1440,6 +1480,7 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
     const pd_impl_t *concrete = &upd;
     qmm_plan_t *plan = primitive->plan;
     void *lib_scratch = primitive->lib_scratch;
+    scratch_guard_t *guard = &primitive->guard;
     std::shared_ptr<rt_entry_t> rt_hold;
     if (upd.kind == dnnl_matmul && upd.runtime) {
         const dnnl_status_t rs = resolve_runtime_matmul(
@@ -1449,6 +1490,7 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         concrete = rt_hold->pd.get();
         plan = rt_hold->plan;
         lib_scratch = rt_hold->scratch;
+        guard = &rt_hold->guard;
     }
     const pd_impl_t &pd = *concrete;
 
@@ -1492,6 +1534,9 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         }
         A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
                                         : lib_scratch;
+        scratch_order_t order(
+                A.scratch && A.scratch == lib_scratch ? guard : nullptr,
+                stream->hip_stream);
         st = qmm_matmul_launch(plan, &A, stream->hip_stream);
     } else if (pd.kind == kind_sdpa) {
         if (pd.dst.has_zero_dim()) return dnnl_success;
@@ -1509,6 +1554,9 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive,
         A.v_zp = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_VALUES);
         A.scratch = pd.scratchpad.ndims ? handle(DNNL_ARG_SCRATCHPAD)
                                         : lib_scratch;
+        scratch_order_t order(
+                A.scratch && A.scratch == lib_scratch ? guard : nullptr,
+                stream->hip_stream);
         st = qmm_sdpa_launch(&pd.sd, &A, stream->hip_stream);
     } else if (pd.kind == dnnl_softmax) {
         if (pd.src.has_zero_dim()) return dnnl_success;
