@@ -46,7 +46,7 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
           "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize",
           "attention_products_f16": "bench_f16_products", "int8_decode_rows": "bench_int8_rows",
-          "mfma_ceiling": "bench_mfma_ceiling"}
+          "mfma_ceiling": "bench_mfma_ceiling", "gemm_anatomy": "bench_gemm_anatomy"}
 
 
 def main():
@@ -246,49 +246,68 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
     """Config 3: bf16 x u4 GEMV, G=128 f16 scales + u4 zero points. The 8.7 MB
     of one weights set would sit in the last-level cache, so `sets` distinct
     copies are cycled; the launches are replayed from a HIP graph so that the
-    host does not pace them."""
+    host does not pace them. After config 3's own shape: the same layer with 8-bit weights, and the decode shape of
+    the reference's LLM list (4096 x 14336, f16 and bf16 activations, 29 MB of weights per launch), where the launch
+    is long enough for bandwidth rather than launch latency to show."""
     import oracle as O
     G = 128
     r = np.random.default_rng(3)
     res = {}
-    w4 = O.pack4(r.integers(0, 16, (K, N)))
-    sc4 = O.from_f32(O.F16, r.uniform(0.005, 0.02, (K // G, N)).astype(np.float32))
-    zp4 = O.pack4(r.integers(6, 10, (K // G, N)))
-    # the last entry: 8-bit weights-only quantization, one f16 scale and u8 zero point per column
-    # (tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu: --dt=f16:u8:f16, wei:per_oc)
-    for M, w8 in [(m, False) for m in rows] + [(1, True)]:
+    cache = {}
+
+    def weights(Kx, Nx, w8):
+        key = (Kx, Nx, w8)
+        if key not in cache:
+            if w8:
+                # 8-bit weights-only quantization, one f16 scale and u8 zero point per column
+                # (tests/benchdnn/inputs/matmul/option_set_fwks_llm_gpu: --dt=f16:u8:f16, wei:per_oc)
+                cache[key] = (r.integers(0, 256, (Kx, Nx)).astype(np.uint8),
+                              O.from_f32(O.F16, r.uniform(0.0005, 0.002, Nx).astype(np.float32)),
+                              r.integers(100, 156, Nx).astype(np.uint8))
+            else:
+                cache[key] = (O.pack4(r.integers(0, 16, (Kx, Nx))),
+                              O.from_f32(O.F16, r.uniform(0.005, 0.02, (Kx // G, Nx)).astype(np.float32)),
+                              O.pack4(r.integers(6, 10, (Kx // G, Nx))))
+        return cache[key]
+
+    # (key, M, K, N, activations f16, 8-bit weights, weight sets)
+    cases = [("M%d" % m, m, K, N, False, False, sets) for m in rows]
+    cases.append(("M1_u8_weights", 1, K, N, True, True, sets))
+    for act16 in (True, False):
+        for m in (1, 16):
+            cases.append(("N14336_%s_M%d" % ("f16" if act16 else "bf16", m), m, 4096, 14336, act16, False, 20))
+    for key, M, Kx, Nx, act16, w8, nsets in cases:
+        w, sc, zp = weights(Kx, Nx, w8)
         attr = A.primitive_attr()
+        adt = dt.f16 if act16 else dt.bf16
+        attr.set_fpmath_mode(A.fpmath_mode.f16 if act16 else A.fpmath_mode.bf16, True)
         if w8:
-            w = r.integers(0, 256, (K, N)).astype(np.uint8)
-            sc = O.from_f32(O.F16, r.uniform(0.0005, 0.002, N).astype(np.float32))
-            zp = r.integers(100, 156, N).astype(np.uint8)
-            attr.set_fpmath_mode(A.fpmath_mode.f16, True)
             attr.set_scales(A.DNNL_ARG_WEIGHTS, 2, [], dt.f16)
             attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 2, [], dt.u8)
-            adt, wdt = dt.f16, dt.u8
+            wdt = dt.u8
         else:
-            w, sc, zp = w4, sc4, zp4
-            attr.set_fpmath_mode(A.fpmath_mode.bf16, True)
             attr.set_scales(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.f16)
             attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 3, [G, 1], dt.u4)
-            adt, wdt = dt.bf16, dt.u4
-        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], adt, T("ab")), memory.desc([K, N], wdt, tag.any),
-                                     memory.desc([M, N], adt, T("ab")), attr=attr)
+            wdt = dt.u4
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, Kx], adt, T("ab")), memory.desc([Kx, Nx], wdt, tag.any),
+                                     memory.desc([M, Nx], adt, T("ab")), attr=attr)
         prim = A.matmul(pd)
-        a = O.from_f32(O.F16 if w8 else O.BF16, r.standard_normal((M, K)).astype(np.float32))
+        a = O.from_f32(O.F16 if act16 else O.BF16, r.standard_normal((M, Kx)).astype(np.float32))
         m_src = memory(pd.src_desc(), eng).write(a)
         m_dst = memory(pd.dst_desc(), eng)
-        plain = memory(memory.desc([K, N], wdt, T("ab")), eng).write(w)
-        first = memory(pd.weights_desc(), eng)
-        A.reorder(plain, first).execute(strm, plain, first)
-        strm.wait()
-        wsets, ssets, zsets = [first], [], []
+        plain = memory(memory.desc([Kx, Nx], wdt, T("ab")), eng).write(w)
+        wsets, ssets, zsets = [], [], []
         nb = pd.weights_desc().get_size()
-        for i in range(sets):
-            if i:
-                m = memory(pd.weights_desc(), eng)
-                hiprt.memcpy_dtod(m.get_data_handle(), first.get_data_handle(), nb)
-                wsets.append(m)
+        ro = None
+        for i in range(nsets):
+            # every set is packed by the library's own reorder (a kernel on the stream): the bench issues no
+            # device-to-device copy through the HIP runtime
+            m = memory(pd.weights_desc(), eng)
+            ro = ro or A.reorder(plain, m)
+            ro.execute(strm, plain, m)
+            wsets.append(m)
+        strm.wait()
+        for i in range(nsets):
             ssets.append(memory(memory.desc([sc.nbytes], dt.u8, T("a")), eng).write(sc))
             zsets.append(memory(memory.desc([zp.nbytes], dt.u8, T("a")), eng).write(zp))
 
@@ -297,10 +316,10 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
                                 A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: ssets[i],
                                 A.DNNL_ARG_ATTR_ZERO_POINTS | A.DNNL_ARG_WEIGHTS: zsets[i]})
 
-        for i in range(sets):
+        for i in range(nsets):
             one(i)
         strm.wait()
-        graph = hiprt.Graph(hs, lambda: [one(i) for i in range(sets)])
+        graph = hiprt.Graph(hs, lambda: [one(i) for i in range(nsets)])
         graph.launch()
         strm.wait()
         e0, e1 = hiprt.Event(), hiprt.Event()
@@ -309,12 +328,12 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
             graph.launch()
         e1.record(hs)
         strm.wait()
-        us = e1.elapsed_ms(e0) * 1e3 / (reps * sets)
-        nbytes = (K * N if w8 else K * N // 2) + sc.nbytes + zp.nbytes + M * K * 2 + M * N * 2
+        us = e1.elapsed_ms(e0) * 1e3 / (reps * nsets)
+        nbytes = (Kx * Nx if w8 else Kx * Nx // 2) + sc.nbytes + zp.nbytes + M * Kx * 2 + M * Nx * 2
         floor = None
         if M == 1 and not w8:
             # the same bytes, the same weight sets and the same graph harness, read by a kernel that
-            # does nothing else (qmm_stream_read): what the launch gaps and a cold 8.7 MB read cost alone
+            # does nothing else (qmm_stream_read): what the launch gaps and a cold read cost alone
             from onednn_amd import _capi
             sink = memory(memory.desc([8192], dt.u8, T("a")), eng)
             L = _capi.lib()
@@ -324,10 +343,10 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
                                        zsets[i].get_data_handle(), zp.nbytes, sink.get_data_handle(), hs)
                 assert rc == 0, rc
 
-            for i in range(sets):
+            for i in range(nsets):
                 rd(i)
             strm.wait()
-            g2 = hiprt.Graph(hs, lambda: [rd(i) for i in range(sets)])
+            g2 = hiprt.Graph(hs, lambda: [rd(i) for i in range(nsets)])
             g2.launch()
             strm.wait()
             f0, f1 = hiprt.Event(), hiprt.Event()
@@ -336,18 +355,20 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
                 g2.launch()
             f1.record(hs)
             strm.wait()
-            floor = round(f1.elapsed_ms(f0) * 1e3 / (reps * sets), 3)
-        res["M%d%s" % (M, "_u8_weights" if w8 else "")] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
-                          "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
-                          "impl": pd.impl_info_str(), "weight_sets": sets, "timing": "hip graph of %d launches x %d" % (sets, reps)}
+            floor = round(f1.elapsed_ms(f0) * 1e3 / (reps * nsets), 3)
+        res[key] = {"us_per_launch": round(us, 3), "algorithmic_bytes": nbytes,
+                    "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM, 4),
+                    "impl": pd.impl_info_str(), "weight_sets": nsets, "timing": "hip graph of %d launches x %d" % (nsets, reps)}
+        if (Kx, Nx) != (K, N):
+            res[key]["shape"] = "%d x %d x %d" % (M, Kx, Nx)
         if M > 64:  # the prefill step of the same layer: the tiled kernel, arithmetic-bound
-            key = "M%d%s" % (M, "_u8_weights" if w8 else "")
-            res[key]["TFLOPs"] = round(2.0 * M * K * N / us / 1e6, 1)
-            res[key]["frac_of_f16_peak"] = round(2.0 * M * K * N / us / 1e6 / 2500.0, 4)
+            res[key]["TFLOPs"] = round(2.0 * M * Kx * Nx / us / 1e6, 1)
+            res[key]["frac_of_f16_peak"] = round(2.0 * M * Kx * Nx / us / 1e6 / 2500.0, 4)
         if floor is not None:
-            res["M1"]["read_floor_us"] = floor
-            res["M1"]["read_floor_kernel"] = ("qmm_stream_read: 256 workgroups x 512 lanes, 16-byte loads of the same "
-                                              "weights + scales + zero points, same graph of %d launches x %d" % (sets, reps))
+            res[key]["read_floor_us"] = floor
+            res[key]["read_floor_kernel"] = ("qmm_stream_read: 256 workgroups x 512 lanes, 16-byte loads of the same "
+                                              "weights + scales + zero points, same graph of %d launches x %d" % (nsets, reps))
+        del wsets, ssets, zsets, graph
     return res
 
 
@@ -409,6 +430,86 @@ def _settled_times(prim, strm, hs, hiprt, ex, steps, rounds, settle_s):
         e1.record(hs)
         strm.wait()
         out.append(e1.elapsed_ms(e0) / steps)
+    return out
+
+
+def _c2_primitive(A, memory, dt, tag, T, eng, strm, data):
+    """Config 2's primitive and execute arguments (weights prepacked); `data` = build_c2()."""
+    src, wei, ss, ws = data
+    M, K = src.shape
+    N = wei.shape[1]
+    attr = A.primitive_attr()
+    attr.set_scales(A.DNNL_ARG_SRC, 3, [1, K], dt.f32)
+    attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 2)
+    po = A.post_ops()
+    po.append_eltwise(A.algorithm.eltwise_swish, 1.0, 0.0)
+    attr.set_post_ops(po)
+    pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.s8, T("ab")), memory.desc([K, N], dt.s8, tag.any),
+                                 memory.desc([M, N], dt.bf16, T("ab")), attr=attr)
+    prim = A.matmul(pd)
+    m_plain = memory(memory.desc([K, N], dt.s8, T("ab")), eng).write(wei)
+    m_wei = memory(pd.weights_desc(), eng)
+    A.reorder(m_plain, m_wei).execute(strm, m_plain, m_wei)
+    strm.wait()
+    ex = {A.DNNL_ARG_SRC: memory(pd.src_desc(), eng).write(src), A.DNNL_ARG_WEIGHTS: m_wei,
+          A.DNNL_ARG_DST: memory(pd.dst_desc(), eng),
+          A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_SRC: memory(memory.desc([M], dt.f32, T("a")), eng).write(ss),
+          A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: memory(memory.desc([N], dt.f32, T("a")), eng).write(ws)}
+    return pd, prim, ex
+
+
+def bench_gemm_anatomy(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20, rounds=3, settle_s=1.5):
+    """Where a config-2 launch spends its time, from the kernels' own measurement switches (QMM_MEASURE): the launch as
+    it is, the same launch ending after the main loop (no epilogue, nothing stored), and per-tile time stamps (core
+    clock counter and a constant 100 MHz counter at kernel entry, loop entry, loop exit and the end of the epilogue),
+    which give the cycles per k-step and the clock each phase ran at. For the default kernel (256 x 256 tiles, one
+    workgroup per CU) and for the 256 x 128 kernel with two workgroups per CU (QMM_B8X_VARIANT=2)."""
+    import ctypes as C
+    from onednn_amd import _capi
+    data = build_c2(A, dt, T)
+    M, K, N = 4096, 4096, 14336
+    ops = 2.0 * M * K * N
+    out = {}
+    for label, b8x, tile_n, per_cu in (("tile_256x256", 1, 256, 1), ("tile_256x128_two_per_cu", 2, 128, 2)):
+        res = {}
+        for name, measure in (("as_is", 0), ("main_loop_only", 1)):
+            with _capi.kernel_variants(measure=measure, b8x=b8x):
+                pd, prim, ex = _c2_primitive(A, memory, dt, tag, T, eng, strm, data)
+            ms = float(np.median(_settled_times(prim, strm, hs, hiprt, ex, steps, rounds, settle_s)))
+            res[name] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / ms / 1e9, 1),
+                         "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8, 4)}
+            del prim, ex
+        res["epilogue_share_of_launch"] = round(1.0 - res["main_loop_only"]["ms_per_launch"] / res["as_is"]["ms_per_launch"], 4)
+        with _capi.kernel_variants(measure=2, b8x=b8x):
+            pd, prim, ex = _c2_primitive(A, memory, dt, tag, T, eng, strm, data)
+        _settled_times(prim, strm, hs, hiprt, ex, steps, 1, settle_s)       # the stamps kept are the last launch's
+        strm.wait()
+        ntiles = (M // 256) * (N // tile_n)
+        grid = min((ntiles + 7) // 8 * 8, 4096)
+        buf = (C.c_uint64 * (grid * 8))()
+        rc = _capi.lib().qmm_gemm_stamps_read(b8x, buf, C.sizeof(buf))
+        assert rc == 0, rc
+        t = np.frombuffer(buf, dtype=np.uint64).reshape(grid, 4, 2).astype(np.float64)
+        t = t[t[:, 3, 0] > 0]
+        cyc = np.diff(t[:, :, 0], axis=1)            # core-clock cycles per phase: prologue, main loop, epilogue
+        ns = np.diff(t[:, :, 1], axis=1) * 10.0      # the constant counter ticks at 100 MHz
+        ksteps = K // 64
+        ghz = cyc / np.maximum(ns, 1.0)
+        med = lambda a: float(np.median(a))
+        mfma_cycles = 1024 * tile_n // 256           # MFMA cycles of one wave per k-step
+        res["stamps"] = {
+            "tiles": int(t.shape[0]), "k_steps_per_tile": ksteps, "workgroups_per_cu": per_cu,
+            "prologue_us": round(med(ns[:, 0]) / 1e3, 2), "main_loop_us": round(med(ns[:, 1]) / 1e3, 2),
+            "epilogue_us": round(med(ns[:, 2]) / 1e3, 2),
+            "main_loop_cycles_per_k_step": round(med(cyc[:, 1]) / ksteps, 1),
+            "mfma_cycles_per_k_step_of_the_waves_sharing_a_simd": mfma_cycles * per_cu,
+            "main_loop_clock_GHz": round(med(ghz[:, 1]), 3), "epilogue_clock_GHz": round(med(ghz[:, 2]), 3),
+            "epilogue_cycles": round(med(cyc[:, 2]), 0),
+            "launch_span_us": round(float(t[:, 3, 1].max() - t[:, 0, 1].min()) * 10.0 / 1e3, 1)}
+        out[label] = res
+    out["note"] = ("stamps: medians over the block tiles of one launch; clock = core-clock cycles / time of the constant "
+                   "100 MHz counter (10 ns resolution); the stamp code costs a scalar branch per phase. With two workgroups "
+                   "per CU a phase's time includes what the SIMD gave the other workgroup's wave")
     return out
 
 
@@ -799,8 +900,9 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
             wsets = [first]
             for _ in range(7):
                 m = memory(pd.weights_desc(), eng)
-                hiprt.memcpy_dtod(m.get_data_handle(), first.get_data_handle(), pd.weights_desc().get_size())
+                A.reorder(plain, m).execute(strm, plain, m)
                 wsets.append(m)
+            strm.wait()
         a8 = np.clip(np.rint(r.standard_normal((M, K)) * 40), -128, 127)
         m_src = memory(pd.src_desc(), eng).write((a8 + 128).astype(np.uint8) if szp else a8.astype(np.int8))
         m_sz = memory(memory.desc([M * (K // G)], dt.u8, T("a")), eng).write(

@@ -139,6 +139,7 @@ _SIGNATURES = {
     "qmm_matmul_impl_name": (C.c_char_p, [_I]),
     "qmm_reorder_impl_name": (C.c_char_p, [_P]),
     "qmm_stream_read": (_I, [_P, C.c_size_t, _P, C.c_size_t, _P, C.c_size_t, _P, _P]),
+    "qmm_gemm_stamps_read": (_I, [_I, _P, C.c_size_t]),
     "qmm_mfma_ceiling": (_I, [_I, _I, _I, _I, _P, _P, C.POINTER(C.c_double)]),
 }
 
@@ -163,10 +164,10 @@ def lib():
 
 
 @contextlib.contextmanager
-def kernel_variants(gemm=None, w4a8=None, b8x=None):
+def kernel_variants(gemm=None, w4a8=None, b8x=None, measure=None):
     """Kernel-selection overrides (include/qmm_hip.h) for the plans created inside the block: environment variables
     the library reads at plan creation, restored on exit."""
-    names = {"QMM_GEMM_VARIANT": gemm, "QMM_W4A8_VARIANT": w4a8, "QMM_B8X_VARIANT": b8x}
+    names = {"QMM_GEMM_VARIANT": gemm, "QMM_W4A8_VARIANT": w4a8, "QMM_B8X_VARIANT": b8x, "QMM_MEASURE": measure}
     old = {k: os.environ.get(k) for k in names}
     try:
         for k, v in names.items():

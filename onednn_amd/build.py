@@ -45,8 +45,8 @@ for v in GEMM_VARIANTS:
         UNITS.append(("qmm_gemm_b8.hip", "_v%d_k%d" % (v, k),
                       ["-DQMM_GEMM_VARIANT=%d" % v, "-DQMM_GEMM_KIND=%d" % k]))
 # likewise the 256 x 256 kernels: int8, short-K int8, fp8, int8 on 16 x 16 MFMAs
-# (even and odd numbers of k-steps), fp8 on 16 x 16 MFMAs
-for v in (1, 2, 3, 4, 5, 6):
+# (even and odd numbers of k-steps), fp8 on 16 x 16 MFMAs, int8 with two workgroups per CU
+for v in (1, 2, 3, 4, 5, 6, 7):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
 for v in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))

@@ -875,7 +875,8 @@ int qmm_matmul_plan_create(
     p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
     p->gemm_variant = env_variant("QMM_GEMM_VARIANT", 0, 6, 0);
     p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 3, 0);
-    p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 1, 1);
+    p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 2, 1);
+    p->measure = env_variant("QMM_MEASURE", 0, 3, 0);
     // resolve the static scratch's address on the current device now, so that
     // qmm_matmul_launch_static_scratch() finds it ready (a plan used on another
     // device resolves it at its first launch there)
@@ -1018,7 +1019,10 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
             return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
         g.A = (const uint8_t *)args->src;
         g.lda = D.src.strides[nd - 2];
-        g.b8x_mfma32 = plan->b8x_variant == 0;
+        g.switches = (plan->b8x_variant == 0 ? GEMM_MFMA32 : 0)
+                | (plan->b8x_variant == 2 ? GEMM_TWO_PER_CU : 0)
+                | (plan->measure & 1 ? GEMM_SKIP_EPILOGUE : 0)
+                | (plan->measure & 2 ? GEMM_STAMPS : 0);
         fold_batch(D.src, D.dst, g.a_sb);
         const int64_t wb = wei_batch(D);
         const b8_geom_t geom = b8_geom(wb, P.K, P.N);

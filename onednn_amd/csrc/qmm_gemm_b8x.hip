@@ -44,6 +44,37 @@ namespace qmm {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
+// ---- measurement aid (QMM_MEASURE, qmm_hip.h) --------------------------------
+// With GEMM_STAMPS the first lane of a workgroup records (core clock counter,
+// constant 100 MHz counter) at four points of its block tile -- kernel entry,
+// main loop entry, main loop exit, end of the epilogue -- into a device array
+// that qmm_gemm_stamps_read() copies out; GEMM_SKIP_EPILOGUE ends the kernel
+// after the main loop. Both are a scalar branch on a kernel argument in the
+// normal path. Only the int8 16 x 16 x 64 kernel (even k-step count) has them:
+// the fp8 kernel has no registers to spare for the extra code.
+constexpr int STAMP_TILES = 4096;
+#if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5 || QMM_B8X_PART == 7)
+static __device__ unsigned long long g_gemm_stamps[STAMP_TILES * 8];
+#define QX_STAMP(slot) \
+    if ((p.switches & GEMM_STAMPS) && tid == 0) { \
+        const unsigned t = (blockIdx.x + gridDim.x * blockIdx.y) % STAMP_TILES; \
+        g_gemm_stamps[t * 8 + 2 * (slot)] = clock64(); \
+        g_gemm_stamps[t * 8 + 2 * (slot) + 1] = wall_clock64(); \
+    }
+// keeps the accumulators alive without storing them
+#define QX_SKIP_EPILOGUE(NI, NJ, NR) \
+    if (p.switches & GEMM_SKIP_EPILOGUE) { \
+        unsigned s = 0; \
+        for (int i = 0; i < NI; i++) \
+            for (int j = 0; j < NJ; j++) \
+                for (int r = 0; r < NR; r++) \
+                    s += __builtin_bit_cast(unsigned, acc[i][j][r]); \
+        if (s == 0x12345678u) ((unsigned *)p.ep.dst.ptr)[tid] = s; \
+        QX_STAMP(3) \
+        return; \
+    }
+#endif
+
 namespace b8x {
 
 constexpr int BM = 256, BN = 256, BK = 64, NT = 256;
@@ -236,11 +267,15 @@ QMM_D void epilogue_fast4_bf16(const epilogue_t &ep, float (&d)[4], bool has_ss,
 // (BATCHED), 4 in the others, whose register allocation does not survive more
 // (with 8 the compiler spills 2 KB per lane and moves scalar operands of the
 // direct loads into vector registers).
-template <int FAST, int DSTK, bool EXT, bool F8, int PITCH, bool BATCHED>
+// LPR: lanes that share a staged row (4 columns each): 32 for a wave tile of
+// 128 columns (two rows per pass over the 64 staged rows), 16 for one of 64.
+template <int FAST, int DSTK, bool EXT, bool F8, int PITCH, bool BATCHED,
+        int LPR = 32>
 QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         const float *ssl, int lane, const ep_cols_t &cols,
         const int (&cs4)[4], int64_t bz, int64_t m_first, int64_t en) {
-    const int ecol = (lane & 31) * 4;
+    constexpr int RPI = 64 / LPR, NIT = 64 / RPI; // rows per pass, passes
+    const int ecol = (lane & (LPR - 1)) * 4, lrow = lane / LPR;
     // rows in flight: fewer where a row is a long computation of its own
     constexpr int UNR = FAST == EP_FAST_GELU_ERF || FAST == EP_FAST_GELU_TANH
             ? 2
@@ -262,15 +297,15 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         // a batch of rows' operands requested before the first of their stores
         constexpr int BATCH = BATCHED ? 16 : 4;
 #pragma unroll 1
-        for (int it0 = 0; it0 < 32; it0 += BATCH) {
+        for (int it0 = 0; it0 < NIT; it0 += BATCH) {
             uint4 pre[BATCH];
 #pragma unroll
             for (int k = 0; k < BATCH; k++)
                 pre[k] = ep_operand_load<FAST, DSTK>(ep, cols, bz,
-                        m_first + (it0 + k) * 2 + (lane >> 5), en);
+                        m_first + (it0 + k) * RPI + lrow, en);
 #pragma unroll
             for (int k = 0; k < BATCH; k++) {
-                const int row = (it0 + k) * 2 + (lane >> 5);
+                const int row = (it0 + k) * RPI + lrow;
                 const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
                 const float ss = ssl[row];
                 float d[4];
@@ -282,8 +317,8 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
         return;
     }
 #pragma unroll UNR
-    for (int it = 0; it < 32; it++) {
-        const int row = it * 2 + (lane >> 5);
+    for (int it = 0; it < NIT; it++) {
+        const int row = it * RPI + lrow;
         const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
         const float ss = ssl[row];
         float d[4];
@@ -296,6 +331,8 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
 // scales, written to LDS by the first 256 threads before the main loop (the
 // loads' latency passes under the prologue): absent ones as 1.0 / 0, columns
 // past N likewise.
+// TABS: where the five 1 KiB tables start (SS_OFF in the 256 x 256 kernels).
+template <int TABS = b8x::SS_OFF>
 QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
         int m0, int n0, int bz) {
     using namespace b8x;
@@ -316,11 +353,11 @@ QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
         if (comp != 0 && p.colsum)
             cs = comp * p.colsum[(int64_t)bz * p.colsum_sb + n];
     }
-    ((float *)(lds + SS_OFF))[tid] = ss;
-    ((float *)(lds + WS_OFF))[tid] = ws;
-    ((int *)(lds + CS_OFF))[tid] = cs;
-    ((float *)(lds + BI_OFF))[tid] = bi;
-    ((float *)(lds + ZP_OFF))[tid] = zp;
+    ((float *)(lds + TABS))[tid] = ss;
+    ((float *)(lds + TABS + (WS_OFF - SS_OFF)))[tid] = ws;
+    ((int *)(lds + TABS + (CS_OFF - SS_OFF)))[tid] = cs;
+    ((float *)(lds + TABS + (BI_OFF - SS_OFF)))[tid] = bi;
+    ((float *)(lds + TABS + (ZP_OFF - SS_OFF)))[tid] = zp;
 }
 
 // Epilogue of one block tile, shared by the int8 and fp8 kernels.
@@ -328,15 +365,26 @@ QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
 // (fp8 and short-K launches; everything else they accept takes the row path)
 // The accumulators are NFI x NFJ fragments per wave: 4 x 4 of 32 x 32, or
 // 8 x NFJ of 16 x 16 (a wave tile of 128 x 16 NFJ).
-template <bool F8, bool LEAN, typename AccT, int NFI, int NFJ>
+// TABS: start of the operand tables (tile_operands_stage). NARROW: a wave tile
+// of 64 columns whose staged rows are shared by 16 lanes (pitch 68 words, four
+// rows per pass) -- the 256 x 128 kernel; otherwise a row takes 32 lanes and
+// lanes past the wave tile's columns idle.
+template <bool F8, bool LEAN, typename AccT, int NFI, int NFJ,
+        int TABS = b8x::SS_OFF, bool NARROW = false>
 QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
         uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
         int wm0, int wn0, int bz) {
     using namespace b8x;
     constexpr bool MI16 = NFI == 8;
     constexpr int WN = MI16 ? 16 * NFJ : 128; // columns of the wave tile
-    constexpr int PITCH = MI16 ? STG_PITCH16 : 128;
-    constexpr int STGW = MI16 ? STG_WAVE16 : STG_WAVE;
+    constexpr int PITCH = NARROW ? WN + 4 : (MI16 ? STG_PITCH16 : 128);
+    constexpr int STGW = NARROW ? 64 * PITCH * 4
+                                : (MI16 ? STG_WAVE16 : STG_WAVE);
+    constexpr int LPR = NARROW ? WN / 4 : 32; // lanes per staged row
+    constexpr int RPI = 64 / LPR; // rows per pass
+    static_assert(!NARROW || (MI16 && WN == 64), "narrow staging: 64 columns");
+    constexpr int WS_T = TABS + (WS_OFF - SS_OFF), CS_T = TABS + (CS_OFF - SS_OFF),
+                  BI_T = TABS + (BI_OFF - SS_OFF), ZP_T = TABS + (ZP_OFF - SS_OFF);
     // 32 x 32 fragments: accumulator register r of lane l is row
     // 8*(r/4) + 4*(l/32) + r%4, column l%32; written to LDS register by
     // register. 16 x 16 fragments are computed transposed (the kernels pass the
@@ -361,8 +409,8 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
                     : 4 * (lane >> 5) * 128 + (lane & 31))
                     * 4;
     const int *const stg_r = (const int *)lds + wave * (STGW / 4);
-    const float *const ssl = (const float *)(lds + SS_OFF) + wm0;
-    const int ecol = (lane & 31) * 4;
+    const float *const ssl = (const float *)(lds + TABS) + wm0;
+    const int ecol = (lane & (LPR - 1)) * 4;
     const bool lane_on = ecol < WN; // lanes past a 112-column wave tile idle
     const int en = n0 + wn0 + ecol;
     const int envalid = lane_on ? min(4, p.N - en) : 0;
@@ -382,10 +430,10 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
         // staged by tile_operands_stage()
         epilogue_cols_load(ep, cols, bz, en, 0);
         const int cw = lane_on ? wn0 + ecol : 0;
-        const float4 w4 = *(const float4 *)(lds + WS_OFF + cw * 4);
-        const int4 c4 = *(const int4 *)(lds + CS_OFF + cw * 4);
-        const float4 b4 = *(const float4 *)(lds + BI_OFF + cw * 4);
-        const float4 z4 = *(const float4 *)(lds + ZP_OFF + cw * 4);
+        const float4 w4 = *(const float4 *)(lds + WS_T + cw * 4);
+        const int4 c4 = *(const int4 *)(lds + CS_T + cw * 4);
+        const float4 b4 = *(const float4 *)(lds + BI_T + cw * 4);
+        const float4 z4 = *(const float4 *)(lds + ZP_T + cw * 4);
         cols.ws[0] = w4.x, cols.ws[1] = w4.y, cols.ws[2] = w4.z, cols.ws[3] = w4.w;
         cols.bias[0] = b4.x, cols.bias[1] = b4.y, cols.bias[2] = b4.z, cols.bias[3] = b4.w;
         cols.zp[0] = z4.x, cols.zp[1] = z4.y, cols.zp[2] = z4.z, cols.zp[3] = z4.w;
@@ -442,7 +490,7 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
 #define QX_EP_ROWS(F, D, X) \
     do { \
         if (lane_on) \
-            ep_rows_full<F, D, X, F8, PITCH, LEAN>( \
+            ep_rows_full<F, D, X, F8, PITCH, LEAN, LPR>( \
                     ep, stg_r, ssh, lane, cols, cs4, bz, m_first, en); \
     } while (0)
 #define QX_EP_DST(F) \
@@ -482,8 +530,8 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
 #undef QX_EP_CASE
         } else {
 #pragma unroll 2
-            for (int it = 0; it < 32; it++) {
-                const int row = it * 2 + (lane >> 5);
+            for (int it = 0; it < 64 / RPI; it++) {
+                const int row = it * RPI + lane / LPR;
                 const int4 t = *(const int4 *)&stg_r[row * PITCH + ecol];
                 const int lrow = h * 64 + row;
                 const int m = m0 + wm0 + lrow;
@@ -826,6 +874,7 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int KT = p.K / BK; // host guarantees K % 64 == 0, KT >= 5 and KT % 2 == ODD
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    if constexpr (!ODD) { QX_STAMP(0) }
 
     uint32_t a_vo[4], b_vo[4];
 #pragma unroll
@@ -904,6 +953,7 @@ gemm_b8y_kernel(const gemm_params_t p) {
         QX_SB(); \
         BODY \
     }
+    if constexpr (!ODD) { QX_STAMP(1) }
     // requesting steps kt = 1 .. KT-4, in pairs; an odd KT leaves one more
     constexpr int PAIRED_END = ODD ? 6 : 5;
     for (int kt = 1; kt <= KT - PAIRED_END; kt += 2) {
@@ -923,11 +973,266 @@ gemm_b8y_kernel(const gemm_params_t p) {
         QY_LAST(1)
     }
     __syncthreads();
+    if constexpr (!ODD) {
+        QX_STAMP(2)
+        QX_SKIP_EPILOGUE(8, NFJ, 4)
+    }
 
     tile_epilogue<false, false>(
             p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    if constexpr (!ODD) { QX_STAMP(3) }
 }
 #endif // int8, 16 x 16 x 64
+
+// ---- int8, two workgroups per CU -----------------------------------------------
+// The kernels above keep one wave per SIMD, so the matrix cores idle while a
+// workgroup runs its prologue and its epilogue (a sixth of a launch on a
+// 4096 x 4096 x 14336 problem with a swish epilogue). Here the block tile is
+// 256 x 128 (four waves of 128 x 64: 8 x 4 fragments of v_mfma_i32_16x16x64_i8,
+// 128 accumulator registers), a workgroup needs under 80 KiB of LDS and under
+// 256 registers per lane, and two workgroups share a CU: while one stages,
+// converts and stores its tile the other one's MFMAs have the matrix cores,
+// and in the main loop the two waves of a SIMD fill each other's gaps. The
+// price is operand traffic per MFMA: a k-step moves 24 KiB into LDS for 32 MFMAs
+// per wave (32 KiB for 64 above) and reads 12 fragments for them (16 for 64).
+// LDS ring of 3 stages x (A 256 x 64 + B 128 x 64 bytes); k-step kt multiplies
+// the fragments of tile kt-1 (read during the previous k-step), reads tile
+// kt's, and requests tile kt+2 into the stage tile kt-1 was read from; one
+// vmcnt + barrier per k-step. The MFMAs are inline assembly with the
+// accumulators constrained to the accumulator file (with the builtin and 128
+// accumulators the register allocator shuttles them between the two files
+// inside the loop), which wants ONE code path for all k-steps: the loop body
+// is a pair of k-steps (the two fragment buffers), the pair count is
+// ceil(k-steps / 2), a phantom last tile multiplies the zero padding of the
+// packed weights (K is padded to 128 there) against a re-read of the last
+// source tile, and request pointers stop advancing at the last tile.
+#if defined(QMM_B8X_PART) && QMM_B8X_PART == 7
+namespace b8w {
+constexpr int BM = 256, BN = 128, BK = 64, NT = 256;
+constexpr int STAGES = 3;
+constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+constexpr int STAGE_BYTES = A_BYTES + B_BYTES; // 24 KiB
+constexpr int RING = STAGES * STAGE_BYTES; // 72 KiB
+constexpr int STG_PITCH = 68, STG_WAVE = 64 * STG_PITCH * 4; // epilogue staging
+static_assert(4 * STG_WAVE <= RING, "the staging reuses the ring");
+constexpr int TABS = RING; // five 1 KiB operand tables (tile_operands_stage)
+constexpr int LDS_TOTAL = TABS + 5 * 1024;
+} // namespace b8w
+
+#define QW_MF(i, j, cb) \
+    { \
+        QX_SB(); \
+        asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" \
+                     : "+a"(acc[i][j]) \
+                     : "v"(fb[cb][j]), "v"(fa[cb][i])); \
+        QX_SB(); \
+    }
+#define QW_RA(nb, i) \
+    { \
+        fa[nb][i] = *(const v4i *)(ldsn + a_rel + (i)*1024); \
+        QX_SB(); \
+    }
+#define QW_RB(nb, j) \
+    { \
+        fb[nb][j] = *(const v4i *)(ldsn + b_rel + ((j) >> 1) * 2048 + ((j)&1) * 256); \
+        QX_SB(); \
+    }
+// advance to the next 64-k tile, staying on the last one once it is reached
+#define QW_ADV_A() \
+    { \
+        const int go = adv_a > 0; \
+        sa += go ? BK : 0; \
+        adv_a -= go; \
+        dA = dA + STAGE_BYTES >= lds_base + RING ? dA + STAGE_BYTES - RING \
+                                                 : dA + STAGE_BYTES; \
+    }
+#define QW_ADV_B() \
+    { \
+        const int go = adv_b > 0; \
+        sb += go ? 2048 : 0; \
+        adv_b -= go; \
+        dB = dB + STAGE_BYTES >= lds_base + A_BYTES + RING \
+                ? dB + STAGE_BYTES - RING \
+                : dB + STAGE_BYTES; \
+    }
+// row i of the fragment grid: 4 MFMAs with one other instruction after each
+#define QW_ROW(i, CB, X0, X1, X2, X3) \
+    QW_MF(i, 0, CB); X0; QW_MF(i, 1, CB); X1; QW_MF(i, 2, CB); X2; \
+    QW_MF(i, 3, CB); X3;
+// the B loads are two per wave: M0, load, M0, load
+#define QW_DB0() QX_M0(dB, 0 * 4096)
+#define QW_DB1() \
+    QX_DMA(b_vo[0], sb); \
+    QX_M0(dB, 1 * 4096)
+#define QW_DB2() QX_DMA(b_vo[1], sb)
+// one k-step: 32 MFMAs on buffer CB; the next tile's 12 fragments into buffer
+// NB and the 6 direct loads of the tile after next, one instruction per MFMA
+#define QW_STEP(CB, NB) \
+    QW_ROW(0, CB, QW_RA(NB, 0), QW_RB(NB, 0), QX_D0(a_vo, sa, dA), QW_RB(NB, 1)) \
+    QW_ROW(1, CB, QW_RB(NB, 2), QX_D1(a_vo, sa, dA), QW_RB(NB, 3), QW_RA(NB, 1)) \
+    QW_ROW(2, CB, QX_D2(a_vo, sa, dA), QW_RA(NB, 2), QW_RA(NB, 3), QX_D3(a_vo, sa, dA)) \
+    QW_ROW(3, CB, QW_RA(NB, 4), QX_D4(a_vo, sa, dA), QW_RA(NB, 5), QW_DB0()) \
+    QW_ROW(4, CB, QW_RA(NB, 6), QW_DB1(), QW_RA(NB, 7), QW_DB2()) \
+    QW_ROW(5, CB, , , , ) \
+    QW_ROW(6, CB, , , , ) \
+    QW_ROW(7, CB, , , , )
+
+__global__ void __launch_bounds__(b8w::NT, 2)
+gemm_b8w_kernel(const gemm_params_t p) {
+    using namespace b8w;
+    using b8x::a_swz16;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 64;
+
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int lt;
+    {
+        const int per = (ntiles + 7) / 8;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        lt = xcd * per + slot;
+        if (slot >= per || lt >= ntiles) return;
+    }
+    constexpr int GROUP_M = 8;
+    const int group = lt / (GROUP_M * p.tiles_n);
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int bz = blockIdx.y;
+
+    const int KT = p.K / BK; // host guarantees K % 64 == 0 and KT >= 4
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    QX_STAMP(0)
+
+    uint32_t a_vo[4], b_vo[2];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tid + j * NT;
+        const int row = c >> 2, cp = c & 3;
+        const int gm = min(m0 + row, p.M - 1) - m0;
+        a_vo[j] = (uint32_t)gm * (uint32_t)p.lda + a_swz16(row, cp) * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int c = tid + j * NT;
+        const int nbl = c >> 7, rem = c & 127;
+        const int nb = min(n0 / 32 + nbl, p.nb32 - 1) - n0 / 32;
+        b_vo[j] = (uint32_t)nb * (uint32_t)p.kb32 * 1024u + rem * 16;
+    }
+    auto sgpr_ptr = [](const uint8_t *q) {
+        const uint64_t v = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi
+                = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+    };
+    const uint8_t *sa = sgpr_ptr(
+            p.A + (int64_t)bz * p.a_sb + (int64_t)m0 * p.lda);
+    const uint8_t *sb = sgpr_ptr(p.B + (int64_t)bz * p.b_sb
+            + (int64_t)(n0 / 32) * p.kb32 * 1024);
+    uint32_t dA = lds_base + wave * 1024;
+    uint32_t dB = dA + A_BYTES;
+    // tile advances left: the source stops at its last tile, the packed weights
+    // at the last tile of their zero-padded K
+    int adv_a = KT - 1, adv_b = p.kb32 / 2 - 1;
+
+    const int g = lane >> 4;
+    const int arow = wm0 + (lane & 15);
+    const int a_rel = arow * BK + a_swz16(arow, g) * 16;
+    const int b_rel = A_BYTES + (wn0 >> 5) * 2048 + (g >> 1) * 1024
+            + ((g & 1) * 32 + (lane & 15)) * 16;
+
+    v4i acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                acc[i][j][r] = 0;
+    v4i fa[2][8], fb[2][4];
+
+    tile_operands_stage<TABS>(p, lds, tid, m0, n0, bz);
+
+    // ---- prologue: tiles 0..2 requested (the whole ring); tile 0's fragments
+    // read ----
+#define QW_FETCH_B() \
+    { \
+        QX_M0(dB, 0 * 4096); asm volatile("s_nop 0"); QX_DMA(b_vo[0], sb); \
+        QX_M0(dB, 1 * 4096); asm volatile("s_nop 0"); QX_DMA(b_vo[1], sb); \
+    }
+    QX_FETCH(a_vo, sa, dA); QW_ADV_A();
+    QW_FETCH_B(); QW_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QW_ADV_A();
+    QW_FETCH_B(); QW_ADV_B();
+    QX_FETCH(a_vo, sa, dA); QW_ADV_A();
+    QW_FETCH_B(); QW_ADV_B();
+    QX_WV(12);
+    __syncthreads();
+    uint32_t st = 0; // ring offset of the tile whose fragments are read next
+    {
+        const uint8_t *ldsn = lds;
+        QX_SB();
+        QW_RA(0, 0); QW_RB(0, 0); QW_RB(0, 1); QW_RB(0, 2); QW_RB(0, 3);
+        QW_RA(0, 1); QW_RA(0, 2); QW_RA(0, 3); QW_RA(0, 4); QW_RA(0, 5);
+        QW_RA(0, 6); QW_RA(0, 7);
+    }
+    // k-step: tile kt has landed for every wave (the 6 requests of tile kt+1
+    // may still be in flight), and every wave has read what it needed from the
+    // stage tile kt+2 goes to
+#define QW_KSTEP(CB, NB) \
+    { \
+        st = st + STAGE_BYTES >= (uint32_t)RING ? 0u : st + STAGE_BYTES; \
+        const uint8_t *ldsn = lds + st; \
+        QX_WV(6); \
+        __builtin_amdgcn_s_barrier(); \
+        QX_SB(); \
+        QW_STEP(CB, NB) \
+        QW_ADV_A(); \
+        QW_ADV_B(); \
+    }
+    const int pairs = (KT + 1) / 2;
+    QX_STAMP(1)
+    for (int it = 0; it < pairs; it++) {
+        QW_KSTEP(0, 1)
+        QW_KSTEP(1, 0)
+    }
+    // the last MFMAs are still writing, and the surplus requests must have
+    // landed before the ring is reused as staging
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    QX_WV(0);
+    __syncthreads();
+    QX_STAMP(2)
+    QX_SKIP_EPILOGUE(8, 4, 4)
+
+    tile_epilogue<false, false, v4i, 8, 4, TABS, true>(
+            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    QX_STAMP(3)
+}
+
+void launch_b8x_int8_two_per_cu(const gemm_params_t &p, hipStream_t stream) {
+    using namespace b8w;
+    gemm_params_t q = p;
+    q.tiles_m = (p.M + BM - 1) / BM;
+    q.tiles_n = (p.N + BN - 1) / BN;
+    const int ntiles = q.tiles_m * q.tiles_n;
+    const int grid_x = ((ntiles + 7) / 8) * 8;
+    ensure_dynamic_lds((const void *)gemm_b8w_kernel, LDS_TOTAL);
+    hipLaunchKernelGGL(gemm_b8w_kernel, dim3(grid_x, p.batch), dim3(NT),
+            LDS_TOTAL, stream, q);
+}
+int gemm_stamps_read_two_per_cu(void *host, size_t bytes) {
+    return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_stamps), bytes, 0,
+                   hipMemcpyDeviceToHost)
+            == hipSuccess;
+}
+#endif // int8, two workgroups per CU
 
 // ---- fp8 (e4m3 x e4m3 -> f32) ----------------------------------------------
 // Same tile, ring and epilogue. v_mfma_f32_32x32x64_f8f6f4 consumes a whole
@@ -1460,6 +1765,11 @@ void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream) {
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_b8y_kernel<false>, p, stream);
 }
+int gemm_stamps_read_int8(void *host, size_t bytes) {
+    return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_stamps), bytes, 0,
+                   hipMemcpyDeviceToHost)
+            == hipSuccess;
+}
 #elif QMM_B8X_PART == 5
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_b8y_kernel<true>, p, stream);
@@ -1468,9 +1778,13 @@ void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
 void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_f8y_kernel, p, stream);
 }
+
 #endif
 #else
 void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream);
+void launch_b8x_int8_two_per_cu(const gemm_params_t &p, hipStream_t stream);
+int gemm_stamps_read_int8(void *host, size_t bytes);
+int gemm_stamps_read_two_per_cu(void *host, size_t bytes);
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
@@ -1497,16 +1811,18 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
 
 // By default int8 runs on 16 x 16 x 64 MFMAs (at least 5 k-steps) and fp8 on
 // 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply;
-// p.b8x_mfma32 (a plan-level override for A/B measurements) keeps the loops on
+// GEMM_MFMA32 in p.switches (a plan-level override for A/B measurements) keeps the loops on
 // 32 x 32 MFMAs.
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
-    const int variant = p.b8x_mfma32 ? 0 : 1;
+    const int variant = (p.switches & GEMM_MFMA32) ? 0 : 1;
     if (f8 && variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)
         launch_b8x_fp8(p, stream);
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
+    else if ((p.switches & GEMM_TWO_PER_CU) && p.K >= 4 * 64)
+        launch_b8x_int8_two_per_cu(p, stream);
     else if (variant >= 1 && p.K >= 5 * 64) {
         if ((p.K / 64) & 1)
             launch_b8x_int8_mi16_odd(p, stream);
@@ -1519,3 +1835,13 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
 #endif
 
 } // namespace qmm
+
+#if !defined(QMM_B8X_PART)
+extern "C" int qmm_gemm_stamps_read(int which, void *host, size_t bytes) {
+    if (!host || bytes > sizeof(unsigned long long) * qmm::STAMP_TILES * 8)
+        return QMM_INVALID_ARGUMENTS;
+    const int ok = which == 2 ? qmm::gemm_stamps_read_two_per_cu(host, bytes)
+                              : qmm::gemm_stamps_read_int8(host, bytes);
+    return ok ? QMM_OK : QMM_RUNTIME_ERROR;
+}
+#endif

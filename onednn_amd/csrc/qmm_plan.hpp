@@ -141,6 +141,8 @@ QMM_HD int64_t w4k_nibble_index(const w4k_geom_t &g, int64_t k, int64_t n) {
 }
 
 // ---- MFMA GEMM (int8 / fp8) -----------------------------------------------
+enum { GEMM_MFMA32 = 1, GEMM_SKIP_EPILOGUE = 2, GEMM_STAMPS = 4, GEMM_TWO_PER_CU = 8 };
+
 struct gemm_params_t {
     const uint8_t *A; // src, rows K-contiguous
     int64_t lda, a_sb; // bytes
@@ -161,7 +163,13 @@ struct gemm_params_t {
     // rowsum (see rowsum_b8_kernel); nullptr rowsum: neither
     const void *wei_zp; // nullptr: 0
     int32_t wei_zp_dt, wei_zp_sn, w_off;
-    int32_t b8x_mfma32; // host-side: the 256 x 256 loops on 32 x 32 MFMAs (QMM_B8X_VARIANT=0)
+    // plan-level switches (qmm_hip.h, kernel-selection overrides and
+    // QMM_MEASURE): GEMM_MFMA32 keeps the 256 x 256 loops on 32 x 32 MFMAs;
+    // GEMM_SKIP_EPILOGUE ends the 256 x 256 kernels after the main loop (nothing
+    // is stored); GEMM_STAMPS makes them record time stamps per block tile;
+    // GEMM_TWO_PER_CU takes the int8 kernel with 256 x 128 block tiles and two
+    // workgroups per CU
+    int32_t switches;
     const int32_t *rowsum; // [batch][M]
     epilogue_t ep;
 };
@@ -304,4 +312,5 @@ struct qmm_plan {
     // QMM_B8X_VARIANT), read from the environment when the plan is created and
     // fixed for the plan's life
     int gemm_variant, w4a8_variant, b8x_variant;
+    int measure; // QMM_MEASURE: 1 skip the 256 x 256 kernels' epilogue, 2 time stamps
 };

@@ -499,6 +499,42 @@ def test_mfma_int8_tile256_mi16_loop(ctx, tile256, name):
     assert_bit_exact(other, got, name + " (32x32x32 loop)")
 
 
+
+# the int8 kernel with 256 x 128 block tiles and two workgroups per CU (QMM_B8X_VARIANT=2): same problems, same bits
+TWO_PER_CU_CASES = dict(MI16_CASES)
+TWO_PER_CU_CASES.update({k: v[0] for k, v in TILE256_CASES.items() if v[1] is True and not k.startswith("short_")})
+TWO_PER_CU_CASES.update({"ep_" + k: v[0] for k, v in TILE256_EPILOGUE_CASES.items() if v[1] is True and k != "f16_sum"})
+TWO_PER_CU_CASES["k256_min_f32"] = lambda: int8_linear(300, 256, 200, 121, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None)
+TWO_PER_CU_CASES["k4096_per_token_swish_rows"] = lambda: int8_linear(
+    256, 4096, 384, 122, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, per_token=True)
+
+
+@pytest.mark.parametrize("name", sorted(TWO_PER_CU_CASES))
+def test_mfma_int8_two_workgroups_per_cu(ctx, name):
+    """Bit-exact against the oracle (integer accumulation: the tiling cannot change a bit), and the kernel's own
+    uniform loop with its phantom last tile on odd k-step counts."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    say("mfma_b8 256x128 kernel, two workgroups per CU, %s" % name)
+    p = TWO_PER_CU_CASES[name]()
+    with _capi.kernel_variants(gemm=6, b8x=2):
+        got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    assert_bit_exact(got, p.run_oracle(), name)
+
+
+def test_mfma_int8_two_workgroups_per_cu_not_the_same_kernel(ctx):
+    """The override really selects another kernel: the two launches of one problem differ in time by construction
+    only, so check the selection through the plan-level switch instead: an impossible K for the 256 x 128 kernel
+    (below 4 k-steps) still runs (on the default kernels) and is exact."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    p = int8_linear(300, 128, 260, 123, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None)
+    with _capi.kernel_variants(gemm=6, b8x=2):
+        got = p.run_gpu(eng, strm, weights_any=True)
+    assert_bit_exact(got, p.run_oracle(), "short K under the two-per-CU override")
+
+
 def test_mfma_int8_large_u8_source_prepass_mi16(ctx):
     eng, strm = ctx
     say("mfma_b8 u8 source 4096x384x3072, 16x16x64 loop")
