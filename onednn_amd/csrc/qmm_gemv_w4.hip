@@ -596,6 +596,279 @@ gemv_w4_fast_kernel(const uint8_t *__restrict__ pB,
             (flags_m & 128) != 0, dst_ptr, dst_sm, dst_dt);
 }
 
+// gemv_w4_fast_kernel for wide weight matrices (4-bit weights, activations
+// straight from global memory): a workgroup owns CB column blocks of 16. The
+// activation fragments, their sums and the unpacking constants serve all of
+// them, and the launch has 1 / CB as many workgroups, each with CB times the
+// weights in flight: with more column blocks than the chip holds workgroups at
+// once that is fewer rounds of workgroups and 1 / CB of the activation traffic
+// (4096 x 14336 at 16 rows: 20.3 us with one block, 18.3 with two, 17.5 with four).
+template <bool F16, int ROWS, bool WSIGNED, int CB>
+__global__ void __launch_bounds__(GEMV_WAVES * 64)
+gemv_w4_fast_cb_kernel(const uint8_t *__restrict__ pB,
+        const uint16_t *__restrict__ pA, const uint16_t *__restrict__ pSC,
+        const uint8_t *__restrict__ pZP, const int kg128, const int N,
+        const int K, const int lda, const int shifts, const int flags_m,
+        const gemv_params_t p) {
+    constexpr bool W8 = false, STAGED = false;
+    __shared__ __attribute__((aligned(16))) float red[GEMV_WAVES * 64 * 4];
+    // STAGED: the activations of a wave's tiles pass through a wave-private
+    // piece of LDS (see below)
+    extern __shared__ __attribute__((aligned(16))) uint8_t act_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int uw = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // consecutive workgroups run on the 8 XCDs in turn: give each XCD a
+    // contiguous range of column blocks, so that a scale / zero-point line
+    // (64 and more neighbouring columns) is fetched into one L2 only
+    const int nbg = ((N + 15) >> 4) / CB; // groups of CB blocks (the host checks divisibility)
+    const int bx = blockIdx.x;
+    const int nb = ((nbg & 7) == 0 ? (bx & 7) * (nbg >> 3) + (bx >> 3) : bx) * CB;
+    const int M = (uint32_t)flags_m >> 8;
+    const int m_base = blockIdx.y * 16;
+    const int rows = min(16, M - m_base);
+    const int c = lane >> 4; // k chunk of the lane
+    const int r = lane & 15; // activation row (A operand) / column (B operand)
+    const int n = nb * 16 + r;
+    const int gs_shift = (int8_t)(shifts & 0xff), gz_shift = (int8_t)(shifts >> 8);
+    const bool scale_per_n = flags_m & 1, zp_per_n = flags_m & 2;
+    const bool zp4 = flags_m & 4, zp_signed = flags_m & 8, sc_f16 = flags_m & 16;
+    const bool has_zp = flags_m & 64;
+
+    constexpr float OFFSET = F16 ? 1024.f : 128.f;
+    constexpr uint32_t ONE2 = F16 ? 0x3C003C00u : 0x3F803F80u;
+    const v4u ones = {ONE2, ONE2, ONE2, ONE2};
+    constexpr uint32_t sflip = WSIGNED ? 0x88888888u : 0u;
+    constexpr float soff = WSIGNED ? 8.f : 0.f;
+    // the exponent pattern lives in a vector register and the nibble mask in a
+    // scalar one: (d >> 4 i) & mask | magic is then a shift and one
+    // v_and_or_b32 (an instruction takes one scalar or literal operand only)
+    uint32_t MAGIC = F16 ? 0x64006400u : 0x43004300u;
+    asm volatile("" : "+v"(MAGIC));
+    // 8-bit weights: the high nibbles behind the exponent of 16 * offset, where
+    // one unit of the last mantissa bit is 16 (f16: 0x7400 | h = 16384 + 16 h;
+    // bf16: 0x4500 | h = 2048 + 16 h), so both planes add into one accumulator
+    uint32_t MAGIC_HI = W8 ? (F16 ? 0x74007400u : 0x45004500u) : MAGIC;
+    if constexpr (W8) asm volatile("" : "+v"(MAGIC_HI));
+    uint32_t NIB = 0x000F000Fu;
+    asm volatile("" : "+s"(NIB));
+
+    v4f out[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) out[cb] = v4f {0.f, 0.f, 0.f, 0.f};
+    constexpr int NP = W8 ? 2 : 1; // planes per tile
+    constexpr int TILE_BYTES = 1024 * NP;
+    const uint8_t *__restrict__ Bt
+            = pB + ((int64_t)nb * kg128) * TILE_BYTES + lane * 16;
+    const int64_t BSTEP = (int64_t)kg128 * TILE_BYTES; // to the next column block
+    const int64_t sN = scale_per_n ? N : 0, zN = zp_per_n ? N : 0;
+
+    // Waves are independent until the final reduction: each one fetches its
+    // weight tiles, their scales / zero points AND its activation fragments
+    // (lane (r, c) holds row r, k = 32 s + 8 c .. + 7 of a tile) straight into
+    // registers, every load unconditional (clamped addresses), all issued
+    // before the first use. No LDS staging, no barrier before the arithmetic.
+    // Tile and group indices are wave uniform (scalar arithmetic, shifts
+    // instead of divisions). Rows past M compute on a repeated row and are
+    // never stored; only k past K has to be zeroed (the padded weights decode
+    // to the magic offset, not 0).
+    const int tiles = kg128;
+    constexpr int SPL = ROWS == 16 ? 1 : ROWS == 8 ? 2 : 4; // steps per load
+    constexpr int NA = 4 / SPL; // activation loads per tile
+    // STAGED (16 rows, a launch of at most one workgroup per CU -- the 136 KiB
+    // leave room for one): requested as whole 256-byte row pieces (16 lanes a
+    // row, 4 rows an instruction: load h of lane l is piece l % 16 of row
+    // 4 h + l / 16) instead of 64-byte pieces of 16 different rows, and read
+    // back from LDS in operand order; wave-private, so no barrier. 4096 x 4096
+    // at 16 rows: 6.7 us against 7.5 us; with more workgroups than CUs the
+    // second resident workgroup is worth more (14336 columns: 19 against 21 us).
+    static_assert(!STAGED || ROWS == 16, "");
+    const int rr = ROWS == 1 ? 0 : STAGED ? 0 : min(r / SPL, rows - 1);
+    const uint16_t *__restrict__ Arow = pA + (int64_t)(m_base + rr) * lda;
+    uint8_t *const stage_w = act_lds + uw * (GEMV_UNR * 16 * GEMV_APITCH);
+    // column of block cb: n + 16 cb
+    const uint16_t *scn[CB];
+    int zcol[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const int nn = min(n + 16 * cb, N - 1);
+        scn[cb] = pSC + (scale_per_n ? nn : 0);
+        zcol[cb] = zp_per_n ? nn : 0;
+    }
+    const bool k_tail = (K & 127) != 0;
+    constexpr int UNR = GEMV_UNR;
+    void *dst_ptr = nullptr;
+    int64_t dst_sm = 0;
+    int dst_dt = 0;
+    // steps past the end repeat the last tile and are folded with scale 0
+    auto tile_of = [&](int t) { return min(t, tiles - 1); };
+    for (int tb = 0; tb < tiles; tb += UNR * GEMV_WAVES) {
+        // Loads are issued tile by tile (weights, activations, scale, zero
+        // point) and consumed in the same order below: results return in
+        // issue order, so tile u is unpacked and multiplied while tiles
+        // u + 1 .. are still arriving. (Requesting all activations first and
+        // the scales last, so that only the weights order the arithmetic, was
+        // measured slower: the first weights request leaves later.)
+        uint4 wt[CB][UNR][NP], av[UNR][NA];
+        uint32_t scp[CB][UNR], zpp[CB][UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            const int tc = tile_of(tb + uw + u * GEMV_WAVES);
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                for (int pl = 0; pl < NP; pl++)
+                    wt[cb][u][pl] = ld_stream(Bt + cb * BSTEP
+                            + (int64_t)tc * TILE_BYTES + pl * 1024);
+#pragma unroll
+            for (int h = 0; h < NA; h++) {
+                // chunks past the row's end re-read its last one, rows past M
+                // the last row
+                if constexpr (STAGED) {
+                    const int row = min(4 * h + (lane >> 4), rows - 1);
+                    const int k = min(tc * 128 + (lane & 15) * 8, K - 8);
+                    av[u][h] = *(const uint4 *)(pA + (int64_t)(m_base + row) * lda + k);
+                } else {
+                    const int k = min(
+                            tc * 128 + (h * SPL + r % SPL) * 32 + c * 8, K - 8);
+                    av[u][h] = *(const uint4 *)(Arow + k);
+                }
+            }
+            const int gsc = gs_shift < 0 ? 0 : tc >> gs_shift;
+            const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                scp[cb][u] = scn[cb][(int64_t)gsc * sN];
+                const int64_t zi = has_zp ? (int64_t)gzp * zN + zcol[cb] : 0;
+                zpp[cb][u] = pZP[zp4 ? zi >> 1 : zi];
+            }
+        }
+        if (k_tail && tb + UNR * GEMV_WAVES >= tiles) {
+            // zero the activations past K (last tile of the matrix)
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int tc = tile_of(tb + uw + u * GEMV_WAVES);
+#pragma unroll
+                for (int h = 0; h < NA; h++)
+                    if ((STAGED ? tc * 128 + (lane & 15) * 8
+                                : tc * 128 + (h * SPL + r % SPL) * 32 + c * 8)
+                            >= K)
+                        av[u][h] = make_uint4(0, 0, 0, 0);
+            }
+        }
+        // what the final store needs from the (cold) parameter block is
+        // requested here, behind the loads and ahead of the arithmetic
+        if (tb == 0) {
+            dst_ptr = (void *)p.ep.dst.ptr;
+            dst_sm = p.ep.dst.sm;
+            dst_dt = p.ep.dst.dt;
+            asm volatile("" ::"s"(dst_ptr), "s"(dst_sm), "s"(dst_dt));
+        }
+        if constexpr (STAGED) {
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+#pragma unroll
+                for (int h = 0; h < NA; h++)
+                    *(uint4 *)(stage_w + ((u * 16 + 4 * h + (lane >> 4)) * GEMV_APITCH)
+                            + (lane & 15) * 16)
+                            = av[u][h];
+        }
+        // the four tiles are independent accumulation chains: a tile past
+        // the end is a repeat of the last one and is folded with scale 0
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            v4f Pu[CB], Su = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) Pu[cb] = v4f {0.f, 0.f, 0.f, 0.f};
+            if constexpr (STAGED) {
+                // lane (r, c): row r, k = 32 s + 8 c .. + 7 of the tile
+#pragma unroll
+                for (int h = 0; h < NA; h++)
+                    av[u][h] = *(const uint4 *)(stage_w + (u * 16 + r) * GEMV_APITCH
+                            + h * 64 + c * 16);
+            }
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+                v4u a;
+                {
+                    // operand row SPL j takes step s4's chunk from lane
+                    // (SPL j + s4 % SPL, c) of load s4 / SPL
+                    const uint4 v = av[u][s4 / SPL];
+                    if (s4 % SPL == 0)
+                        a = v4u {v.x, v.y, v.z, v.w};
+                    else if (s4 % SPL == 1)
+                        a = v4u {row_shl<1>(v.x), row_shl<1>(v.y),
+                                row_shl<1>(v.z), row_shl<1>(v.w)};
+                    else if (s4 % SPL == 2)
+                        a = v4u {row_shl<2>(v.x), row_shl<2>(v.y),
+                                row_shl<2>(v.z), row_shl<2>(v.w)};
+                    else
+                        a = v4u {row_shl<3>(v.x), row_shl<3>(v.y),
+                                row_shl<3>(v.z), row_shl<3>(v.w)};
+                }
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++) {
+                    const uint32_t d = (s4 == 0 ? wt[cb][u][0].x
+                                    : s4 == 1   ? wt[cb][u][0].y
+                                    : s4 == 2   ? wt[cb][u][0].z
+                                                : wt[cb][u][0].w)
+                            ^ sflip;
+                    v4u b;
+                    b.x = (d & NIB) | MAGIC_HI;
+                    b.y = ((d >> 4) & NIB) | MAGIC_HI;
+                    b.z = ((d >> 8) & NIB) | MAGIC_HI;
+                    b.w = ((d >> 12) & NIB) | MAGIC_HI;
+                    v4u bl = b;
+                    if constexpr (W8) {
+                        const uint32_t dl = s4 == 0 ? wt[cb][u][NP - 1].x
+                                : s4 == 1           ? wt[cb][u][NP - 1].y
+                                : s4 == 2           ? wt[cb][u][NP - 1].z
+                                                    : wt[cb][u][NP - 1].w;
+                        bl.x = (dl & NIB) | MAGIC;
+                        bl.y = ((dl >> 4) & NIB) | MAGIC;
+                        bl.z = ((dl >> 8) & NIB) | MAGIC;
+                        bl.w = ((dl >> 12) & NIB) | MAGIC;
+                    }
+                    Pu[cb] = mfma16<F16>(a, b, Pu[cb]);
+                    if constexpr (W8) Pu[cb] = mfma16<F16>(a, bl, Pu[cb]);
+                }
+                Su = mfma16<F16>(a, ones, Su);
+            }
+            const int t = tb + uw + u * GEMV_WAVES;
+            const int tc = tile_of(t);
+            const int gzp = gz_shift < 0 ? 0 : tc >> gz_shift;
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                // one scale and one zero point per column and tile
+                float sc = sc_f16
+                        ? (float)__builtin_bit_cast(_Float16, (uint16_t)scp[cb][u])
+                        : u2f(scp[cb][u] << 16);
+                if (t >= tiles) sc = 0.f;
+                // zero point: byte or nibble, signed or not, by shifts and selects
+                // (wave-uniform branches here cost more than the arithmetic)
+                const int odd = zp4 ? (int)(((int64_t)gzp * zN + zcol[cb]) & 1) : 0;
+                const int zbits = zp4 ? 4 : 8;
+                const uint32_t zraw = (zpp[cb][u] >> (4 * odd)) & ((1u << zbits) - 1u);
+                const int zsx = (int)(zraw << (32 - zbits)) >> (32 - zbits);
+                const float zp = has_zp ? (float)(zp_signed ? zsx : (int)zraw) : 0.f;
+                const float off = W8 ? 17.f * OFFSET + 16.f * soff + zp
+                                     : OFFSET + soff + zp;
+                // a single row: only register 0 (row 0) is stored
+#pragma unroll
+                for (int j = 0; j < 4; j += SPL)
+                    out[cb][j] = __builtin_fmaf(sc,
+                            Pu[cb][j] - off * Su[j],
+                            out[cb][j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        if (cb) __syncthreads(); // wave 0 has read the previous block's sums
+        gemv_reduce_store<ROWS>(p, red, out[cb], uw, lane, m_base, rows,
+                n + 16 * cb, (flags_m & 128) != 0, dst_ptr, dst_sm, dst_dt);
+    }
+}
+
 void launch_gemm_w4f(const gemv_params_t &p, int shifts, int flags_m,
         hipStream_t stream);
 bool gemm_w4f_wins(const gemv_params_t &p);
@@ -671,9 +944,20 @@ bool launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
         // stages its activations in LDS
         const bool staged = p.M > 8 && (int64_t)grid.x * grid.y <= 256;
         const int lds = staged ? GEMV_STAGE_BYTES : 0;
+        // two column blocks per workgroup where one block each would be more
+        // workgroups than the chip holds at once (two per CU)
+        // (5 .. 8 rows keep one block: with two, the 8-row form spills registers)
+        const bool two = !p.w8 && !staged && (p.nb16 & 1) == 0 && p.nb16 >= 512
+                && !(p.M > 4 && p.M <= 8);
+        // more than 8 rows: four blocks, for a quarter of the activation traffic
+        const bool four = two && p.M > 8 && (p.nb16 & 3) == 0 && p.nb16 >= 768;
         auto go = [&](auto kern) {
             if (lds) ensure_dynamic_lds((const void *)kern, lds);
-            hipLaunchKernelGGL(kern, grid, dim3(GEMV_WAVES * 64), lds, stream, p.B,
+            hipLaunchKernelGGL(kern,
+                    four       ? dim3(grid.x / 4, grid.y)
+                            : two ? dim3(grid.x / 2, grid.y)
+                                  : grid,
+                    dim3(GEMV_WAVES * 64), lds, stream, p.B,
                     p.A, (const uint16_t *)p.scales, zp, p.kg128, p.N, p.K,
                     (int)p.lda, shifts, flags_m, q);
         };
@@ -690,8 +974,16 @@ bool launch_gemv_w4(const gemv_params_t &p, hipStream_t stream) {
                     return;
                 }
             }
+            if constexpr (R == 16) {
+                if (four) {
+                    go(gemv_w4_fast_cb_kernel<F, R, S, 4>);
+                    return;
+                }
+            }
             if (p.w8)
                 go(gemv_w4_fast_kernel<F, R, S, true>);
+            else if (two)
+                go(gemv_w4_fast_cb_kernel<F, R, S, 2>);
             else
                 go(gemv_w4_fast_kernel<F, R, S, false>);
         };

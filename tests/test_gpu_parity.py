@@ -733,6 +733,29 @@ def test_decode_w4_config3(ctx, M, weights_any):
     assert_bf16_within_1ulp(got, want, "decode bf16", abs_slack=2e-5 * decode_term_scale(p))
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 13, 16])
+@pytest.mark.parametrize("kw", [dict(), dict(act_dt=dt.f16, wei_dt=dt.s4, zp_dt=dt.s8, G=128),
+                                dict(act_dt=dt.f16, with_zp=False, scale_dt=dt.bf16, G=256)])
+def test_decode_w4_wide_weights_two_column_blocks_per_workgroup(ctx, M, kw):
+    """8192 and more columns: a workgroup owns two column blocks (shared activation fragments). 8224 columns are
+    514 blocks and take two per workgroup; 8208 are 513, an odd count, and keep one."""
+    eng, strm = ctx
+    for N in (8224, 8208):
+        say("decode_w4 wide M=%d N=%d %r" % (M, N, kw))
+        p = decode_w4(M, 256, N, 300 + M, **kw)
+        got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+        assert pd.impl_info_str() == DECODE
+        want = p.run_oracle()
+        code = p.dst.dt
+        g, w = O.to_f32(code, got).reshape(M, N), O.to_f32(code, want).reshape(M, N)
+        assert_f32_close(g, w, rel=1e-2, scale=np.abs(w).mean(), what="decode wide")
+        if code == dt.bf16:
+            assert_bf16_within_1ulp(got, want, "decode wide", abs_slack=2e-5 * decode_term_scale(p))
+        else:  # one f16 step, or 2e-5 of the summed magnitudes where the result cancels
+            assert_f32_close(g, w, rel=2.0 ** -10, scale=np.abs(w) + 2e-5 * 1024 * decode_term_scale(p).reshape(M, N),
+                             what="decode wide f16")
+
+
 @pytest.mark.parametrize("kw", [
     dict(act_dt=dt.f16, wei_dt=dt.s4, zp_dt=dt.s8, scale_dt=dt.f32, G=64),
     dict(act_dt=dt.bf16, wei_dt=dt.u4, zp_dt=dt.u8, G=32, zp_group=128),
