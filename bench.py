@@ -486,11 +486,12 @@ def bench_gemm_anatomy(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20, ro
         strm.wait()
         ntiles = (M // 256) * (N // tile_n)
         grid = min((ntiles + 7) // 8 * 8, 4096)
-        buf = (C.c_uint64 * (grid * 8))()
+        buf = (C.c_uint64 * (grid * 16))()
         rc = _capi.lib().qmm_gemm_stamps_read(b8x, buf, C.sizeof(buf))
         assert rc == 0, rc
-        t = np.frombuffer(buf, dtype=np.uint64).reshape(grid, 4, 2).astype(np.float64)
-        t = t[t[:, 3, 0] > 0]
+        t8 = np.frombuffer(buf, dtype=np.uint64).reshape(grid, 8, 2).astype(np.float64)
+        t8 = t8[t8[:, 3, 0] > 0]
+        t = t8[:, :4]
         cyc = np.diff(t[:, :, 0], axis=1)            # core-clock cycles per phase: prologue, main loop, epilogue
         ns = np.diff(t[:, :, 1], axis=1) * 10.0      # the constant counter ticks at 100 MHz
         ksteps = K // 64
@@ -505,6 +506,11 @@ def bench_gemm_anatomy(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20, ro
             "mfma_cycles_per_k_step_of_the_waves_sharing_a_simd": mfma_cycles * per_cu,
             "main_loop_clock_GHz": round(med(ghz[:, 1]), 3), "epilogue_clock_GHz": round(med(ghz[:, 2]), 3),
             "epilogue_cycles": round(med(cyc[:, 2]), 0),
+            # inside the epilogue: staging of the first half, its rows (arithmetic + stores), staging of the second
+            # half, its rows
+            "epilogue_parts_cycles": {
+                "stage_half_0": round(med(t8[:, 4, 0] - t8[:, 2, 0]), 0), "rows_half_0": round(med(t8[:, 5, 0] - t8[:, 4, 0]), 0),
+                "stage_half_1": round(med(t8[:, 6, 0] - t8[:, 5, 0]), 0), "rows_half_1": round(med(t8[:, 3, 0] - t8[:, 6, 0]), 0)},
             "launch_span_us": round(float(t[:, 3, 1].max() - t[:, 0, 1].min()) * 10.0 / 1e3, 1)}
         out[label] = res
     out["note"] = ("stamps: medians over the block tiles of one launch; clock = core-clock cycles / time of the constant "
@@ -705,9 +711,31 @@ def bench_c4(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
           A.DNNL_ARG_ATTR_MULTIPLE_POST_OP(0) | A.DNNL_ARG_SRC_1: memory(mask_md, eng).write(mask)}
     ms = _time(prim, strm, hs, hiprt, ex, steps)
     nbytes = 2 * B * S * D + 4 * B * S * S + 4 * S * S
+    # what a launch that only writes the same 537 MB reaches (qmm_stream_write, the best of a few grid sizes): the
+    # practical ceiling of a destination-bound launch on this card, next to the published 8 TB/s
+    from onednn_amd import _capi
+    L = _capi.lib()
+    dst_bytes = 4 * B * S * S
+    dptr = ex[A.DNNL_ARG_DST].get_data_handle()
+    best = None
+    for groups in (1024, 2048, 4096, 8192):
+        for _ in range(3):
+            assert L.qmm_stream_write(dptr, dst_bytes, groups, hs) == 0
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record(hs)
+        for _ in range(steps):
+            L.qmm_stream_write(dptr, dst_bytes, groups, hs)
+        e1.record(hs)
+        strm.wait()
+        t = e1.elapsed_ms(e0) / steps
+        if best is None or t < best[0]:
+            best = (t, groups)
     return {"ms_per_launch": round(ms, 4), "TOPs": round(2.0 * B * S * S * D / (ms * 1e-3) / 1e12, 1),
             "algorithmic_bytes": nbytes, "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str()}
+            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 4), "impl": pd.impl_info_str(),
+            "write_only_floor": {"ms": round(best[0], 4), "GBps": round(dst_bytes / (best[0] * 1e-3) / 1e9, 1),
+                                 "kernel": "qmm_stream_write: %d workgroups x 256 lanes, 16-byte stores over the same 537 MB dst" % best[1]},
+            "frac_of_write_only_rate": round((nbytes / ms) / (dst_bytes / best[0]), 4)}
 
 
 def bench_attention_chain(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=10):

@@ -254,8 +254,10 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  *   QMM_GEMM_VARIANT: 0 by problem size (default); 1..3 a tile configuration of
  *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible
  *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration
- *   QMM_B8X_VARIANT: MFMA shape of the 256 x 256 kernels: 1 = 16 x 16 (default),
- *     0 = 32 x 32 */
+ *   QMM_B8X_VARIANT: the 256-row int8 / fp8 kernels: 1 = by shape (default: 16 x 16
+ *     MFMAs; int8 with 256 x 128 tiles and two workgroups per CU up to K 2048,
+ *     256 x 256 tiles and one per CU beyond), 2 = 256 x 128 two per CU wherever it
+ *     applies, 3 = 256 x 256 one per CU, 0 = the loops on 32 x 32 MFMAs */
 
 /* ---- measurement switches of the 256 x 256 GEMM kernels ----
  * QMM_MEASURE (environment, read at plan creation like the overrides above):
@@ -263,10 +265,11 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  * number of k-steps; 256 x 128 tiles, QMM_B8X_VARIANT=2) end after their main
  * loop and store nothing (what the loop alone costs); bit 1: the first lane of every workgroup records (core clock counter,
  * 100 MHz counter) at kernel entry, main-loop entry, main-loop exit and the end
- * of the epilogue. qmm_gemm_stamps_read() copies the records of the last such
+ * of the epilogue (slots 0..3), and inside the epilogue after each half of the
+ * tile is staged (slots 4, 6) and after the first half's rows are stored (5). qmm_gemm_stamps_read() copies the records of the last such
  * launch of the 256 x 256 kernel (which = 1) or the 256 x 128 kernel (which = 2)
- * out: 8 x uint64 per block tile, tile = (blockIdx.x + gridDim.x *
- * blockIdx.y) % 4096, at most 4096 * 64 bytes. No counterpart in the
+ * out: 8 slots x 2 x uint64 per block tile, tile = (blockIdx.x + gridDim.x *
+ * blockIdx.y) % 4096, at most 4096 * 128 bytes. No counterpart in the
  * reference. */
 QMM_API int qmm_gemm_stamps_read(int which, void *host, size_t bytes);
 
@@ -280,6 +283,12 @@ QMM_API int qmm_gemm_stamps_read(int which, void *host, size_t bytes);
 #define QMM_STREAM_READ_GROUPS 256
 QMM_API int qmm_stream_read(const void *p0, size_t n0, const void *p1,
         size_t n1, const void *p2, size_t n2, void *sink, void *stream);
+
+/* Launches a kernel that only writes: `groups` workgroups of 256 lanes store
+ * 16-byte vectors over `bytes` of dst (16-byte aligned) with a grid-stride
+ * loop. Benchmarks time it to state what a launch bound by its destination
+ * stream can reach on this card. No counterpart in the reference. */
+QMM_API int qmm_stream_write(void *dst, size_t bytes, int groups, void *hip_stream);
 
 /* Launches `groups` workgroups of four waves that issue nothing but the MFMAs
  * of the 256 x 256 GEMM kernels' main loop (`ksteps` k-steps, even, of the

@@ -460,10 +460,24 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream);
 // the tuning sweep; 6 = the 256 x 256 kernel where it applies)
 // true when launch_gemm_b8 would hand the problem to the 256 x 256 kernel
 bool gemm_b8_uses_tile256(const gemm_params_t &p, bool f8, int variant) {
-    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
-            * p.batch;
-    return (variant == 6 || (variant == 0 && tiles256 >= 192))
-            && gemm_b8x_eligible(p, f8);
+    if (!gemm_b8x_eligible(p, f8)) return false;
+    if (variant == 6) return true;
+    if (variant != 0) return false;
+    const int64_t tm = (p.M + 255) / 256;
+    const int64_t tiles256 = tm * ((p.N + 255) / 256) * p.batch;
+    if (tiles256 >= 192) return true;
+    // int8 with an s8 source also has the 256 x 128 kernel with two workgroups
+    // per CU, which beats the tiles below from 32 such tiles on, unless the row
+    // tiles are mostly padding and the tiles are few (measured with a swish /
+    // bf16 epilogue: 256 x 4096 x 4096 29 against 37 us, 2048 x 4096 x 4096 40
+    // against 67, 1024 x 512 x 1024 13 against 21; 512 x 1024 x 1024 (16 tiles)
+    // 15 against 10 and 128 x 4096 x 4096 (half-empty row tiles) 29 against 18)
+    if (f8 || (p.a_is_u8 && !p.a_preflipped)
+            || (p.switches & (GEMM_ONE_PER_CU | GEMM_MFMA32)))
+        return false;
+    const int64_t tiles128 = tm * ((p.N + 127) / 128) * p.batch;
+    const bool rows_full = 4 * (int64_t)p.M >= 3 * tm * 256;
+    return tiles128 >= 32 && (rows_full || tiles128 >= 96);
 }
 
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,

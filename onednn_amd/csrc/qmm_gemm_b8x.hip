@@ -52,15 +52,20 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 // after the main loop. Both are a scalar branch on a kernel argument in the
 // normal path. Only the int8 16 x 16 x 64 kernel (even k-step count) has them:
 // the fp8 kernel has no registers to spare for the extra code.
-constexpr int STAMP_TILES = 4096;
+[[maybe_unused]] constexpr int STAMP_TILES = 4096, STAMP_SLOTS = 8;
 #if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5 || QMM_B8X_PART == 7)
-static __device__ unsigned long long g_gemm_stamps[STAMP_TILES * 8];
-#define QX_STAMP(slot) \
-    if ((p.switches & GEMM_STAMPS) && tid == 0) { \
+#define QX_HAVE_STAMPS 1
+static __device__ unsigned long long g_gemm_stamps[STAMP_TILES * STAMP_SLOTS * 2];
+// slots: 0 kernel entry, 1 main loop entry, 2 main loop exit, 3 end of the
+// epilogue; inside the epilogue 4 / 6 after the first / second half of the tile
+// is staged and 5 after the first half's rows are stored
+#define QX_STAMP_IF(first, slot) \
+    if ((p.switches & GEMM_STAMPS) && (first)) { \
         const unsigned t = (blockIdx.x + gridDim.x * blockIdx.y) % STAMP_TILES; \
-        g_gemm_stamps[t * 8 + 2 * (slot)] = clock64(); \
-        g_gemm_stamps[t * 8 + 2 * (slot) + 1] = wall_clock64(); \
+        g_gemm_stamps[(t * STAMP_SLOTS + (slot)) * 2] = clock64(); \
+        g_gemm_stamps[(t * STAMP_SLOTS + (slot)) * 2 + 1] = wall_clock64(); \
     }
+#define QX_STAMP(slot) QX_STAMP_IF(tid == 0, slot)
 // keeps the accumulators alive without storing them
 #define QX_SKIP_EPILOGUE(NI, NJ, NR) \
     if (p.switches & GEMM_SKIP_EPILOGUE) { \
@@ -484,6 +489,9 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
                                              * 4)
                                      : "memory");
         }
+#ifdef QX_HAVE_STAMPS
+        QX_STAMP_IF(wave == 0 && lane == 0, 4 + 2 * h)
+#endif
         if (full) {
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
@@ -561,6 +569,9 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
                 }
             }
         }
+#ifdef QX_HAVE_STAMPS
+        if constexpr (h == 0) { QX_STAMP_IF(wave == 0 && lane == 0, 5) }
+#endif
     });
 }
 
@@ -1809,20 +1820,35 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     return true;
 }
 
-// By default int8 runs on 16 x 16 x 64 MFMAs (at least 5 k-steps) and fp8 on
-// 16 x 16 x 128 (K a multiple of 256, at least 512) where they apply;
-// GEMM_MFMA32 in p.switches (a plan-level override for A/B measurements) keeps the loops on
-// 32 x 32 MFMAs.
+// By default int8 runs on 16 x 16 x 64 MFMAs and fp8 on 16 x 16 x 128 (K a
+// multiple of 256, at least 512) where they apply. int8 with an s8 source has
+// two tilings: 256 x 256 with one workgroup per CU (the most MFMAs per byte
+// moved into LDS: the faster main loop, 1185 against 1240 cycles per 64 MFMAs
+// and SIMD) and 256 x 128 with two per CU (a workgroup's prologue, epilogue and
+// dst stream run under the other's MFMAs). Measured on 4096 x K x 14336 with a
+// swish / bf16 epilogue, two per CU over one per CU: K 128 0.77, 256 0.74, 512
+// 0.85, 1024 0.89, 2048 0.96, 4096 1.09, 8192 1.12 of the time; on the batched
+// attention scores (K 128, f32 dst bound by its write stream) 0.84; and 0.79
+// where the 256 x 256 tiles number half the CUs (2048 x 4096 x 4096). So: two
+// per CU up to K 2048, and beyond that where the large tiles would leave more
+// than a third of the CUs without one. Plan-level switches override the choice
+// (GEMM_MFMA32: the 32 x 32 loops; GEMM_TWO_PER_CU / GEMM_ONE_PER_CU).
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     const int variant = (p.switches & GEMM_MFMA32) ? 0 : 1;
+    const bool s8_src = !p.a_is_u8 || p.a_preflipped;
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
+            * p.batch;
+    const bool two_per_cu = !f8 && s8_src && variant >= 1
+            && !(p.switches & GEMM_ONE_PER_CU)
+            && ((p.switches & GEMM_TWO_PER_CU) || p.K <= 2048 || tiles256 <= 170);
     if (f8 && variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)
         launch_b8x_fp8(p, stream);
+    else if (two_per_cu)
+        launch_b8x_int8_two_per_cu(p, stream); // any K: surplus tiles are phantom
     else if (short_k(p))
         launch_b8x_short_k(p, stream);
-    else if ((p.switches & GEMM_TWO_PER_CU) && p.K >= 4 * 64)
-        launch_b8x_int8_two_per_cu(p, stream);
     else if (variant >= 1 && p.K >= 5 * 64) {
         if ((p.K / 64) & 1)
             launch_b8x_int8_mi16_odd(p, stream);
@@ -1838,7 +1864,9 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
 
 #if !defined(QMM_B8X_PART)
 extern "C" int qmm_gemm_stamps_read(int which, void *host, size_t bytes) {
-    if (!host || bytes > sizeof(unsigned long long) * qmm::STAMP_TILES * 8)
+    if (!host
+            || bytes > sizeof(unsigned long long) * qmm::STAMP_TILES
+                            * qmm::STAMP_SLOTS * 2)
         return QMM_INVALID_ARGUMENTS;
     const int ok = which == 2 ? qmm::gemm_stamps_read_two_per_cu(host, bytes)
                               : qmm::gemm_stamps_read_int8(host, bytes);

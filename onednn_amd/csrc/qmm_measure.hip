@@ -87,6 +87,8 @@ extern "C" int qmm_stream_read(const void *p0, size_t n0, const void *p1,
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }
 
+// (3) below: a kernel that only writes (the ceiling of a launch bound by its
+// destination stream).
 // (2) Matrix-core ceiling: a kernel that issues nothing but the MFMAs of the
 // 256 x 256 GEMM kernels' main loop -- one wave per SIMD, 256 accumulator
 // registers, 8 + 8 operand fragments held in registers and filled with
@@ -260,5 +262,27 @@ extern "C" int qmm_mfma_ceiling(int kind, int ksteps, int groups, int data,
         case 2: hipLaunchKernelGGL(mfma_ceiling_kernel<2>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
         default: hipLaunchKernelGGL(mfma_ceiling_kernel<3>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
     }
+    return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
+}
+
+// (3) A kernel that only writes: every lane stores 16-byte vectors with a
+// grid-stride loop, rows of a workgroup contiguous, as an epilogue that streams
+// a large destination does.
+namespace {
+__global__ void __launch_bounds__(256) stream_write_kernel(
+        uint4 *dst, size_t n16, uint32_t seed) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    uint4 v = {seed, seed ^ threadIdx.x, seed + blockIdx.x, ~seed};
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) {
+        dst[i] = v;
+        v.x += 0x9e3779b9u;
+    }
+}
+} // namespace
+
+extern "C" int qmm_stream_write(void *dst, size_t bytes, int groups, void *stream) {
+    if (!dst || ((uintptr_t)dst & 15) || groups < 1) return QMM_INVALID_ARGUMENTS;
+    hipLaunchKernelGGL(stream_write_kernel, dim3(groups), dim3(256), 0,
+            (hipStream_t)stream, (uint4 *)dst, bytes / 16, 0x12345u);
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }

@@ -141,7 +141,13 @@ QMM_HD int64_t w4k_nibble_index(const w4k_geom_t &g, int64_t k, int64_t n) {
 }
 
 // ---- MFMA GEMM (int8 / fp8) -----------------------------------------------
-enum { GEMM_MFMA32 = 1, GEMM_SKIP_EPILOGUE = 2, GEMM_STAMPS = 4, GEMM_TWO_PER_CU = 8 };
+enum {
+    GEMM_MFMA32 = 1,
+    GEMM_SKIP_EPILOGUE = 2,
+    GEMM_STAMPS = 4,
+    GEMM_TWO_PER_CU = 8,
+    GEMM_ONE_PER_CU = 16
+};
 
 struct gemm_params_t {
     const uint8_t *A; // src, rows K-contiguous
@@ -167,8 +173,8 @@ struct gemm_params_t {
     // QMM_MEASURE): GEMM_MFMA32 keeps the 256 x 256 loops on 32 x 32 MFMAs;
     // GEMM_SKIP_EPILOGUE ends the 256 x 256 kernels after the main loop (nothing
     // is stored); GEMM_STAMPS makes them record time stamps per block tile;
-    // GEMM_TWO_PER_CU takes the int8 kernel with 256 x 128 block tiles and two
-    // workgroups per CU
+    // GEMM_TWO_PER_CU / GEMM_ONE_PER_CU force the int8 tiling (256 x 128 with two
+    // workgroups per CU / 256 x 256 with one) that is otherwise chosen by shape
     int32_t switches;
     const int32_t *rowsum; // [batch][M]
     epilogue_t ep;

@@ -19,7 +19,7 @@ from qmm_harness import Problem, TensorSpec, assert_bit_exact, assert_f32_close,
 import test_gpu_parity as cases
 
 pytestmark = pytest.mark.gpu
-ROUTES = ["generic", "general", "tile256"]
+ROUTES = ["generic", "general", "tile256", "two_per_cu"]
 
 
 def say(msg):
@@ -37,7 +37,8 @@ def _run(ctx, route, p, dst_init=None):
     eng, strm = ctx
     if route == "generic":
         return p.run_gpu(eng, strm, impl=cases.GENERIC, dst_init=dst_init)
-    with _capi.kernel_variants(gemm=6 if route == "tile256" else 2):
+    # tile256: 256 x 256 tiles, one workgroup per CU; two_per_cu: 256 x 128 tiles; general: the 128 x 128 configuration
+    with _capi.kernel_variants(gemm=2 if route == "general" else 6, b8x=2 if route == "two_per_cu" else 3):
         got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True, dst_init=dst_init)
     assert pd.impl_info_str() == cases.MFMA
     return got
@@ -203,7 +204,7 @@ def test_swish_into_quantized_dst(ctx, route, dst_dt):
     host libm in the oracle), so a value within float rounding of a .5 boundary may land on the neighbouring
     integer: never further, and for few elements."""
     say("swish -> %s with dst scale and zero point via %s" % (dst_dt, route))
-    M, K, N = (512, 256, 512) if route == "tile256" else (300, 128, 130)
+    M, K, N = (512, 256, 512) if route in ("tile256", "two_per_cu") else (300, 128, 130)
     p = cases.int8_linear(M, K, N, 57, src_dt=dt.s8, dst_dt=dst_dt, src_zp=None, src_scale=0.01,
                           post_ops=[{"kind": "eltwise", "alg": dnnl.algorithm.eltwise_swish, "alpha": 1.0}],
                           dst_scale=0.05, dst_zp=[7])

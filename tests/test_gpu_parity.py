@@ -343,7 +343,7 @@ def test_mfma_int8_against_literal_v38_reference(ctx):
 @pytest.fixture
 def tile256():
     from onednn_amd import _capi
-    with _capi.kernel_variants(gemm=6):
+    with _capi.kernel_variants(gemm=6, b8x=3):      # the 256 x 256 tiles, one workgroup per CU
         yield
 
 
@@ -494,7 +494,7 @@ def test_mfma_int8_tile256_mi16_loop(ctx, tile256, name):
     got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
     assert pd.impl_info_str() == MFMA
     assert_bit_exact(got, p.run_oracle(), name)
-    with _capi.kernel_variants(b8x=0):
+    with _capi.kernel_variants(gemm=6, b8x=0):
         other = p.run_gpu(eng, strm, weights_any=True)
     assert_bit_exact(other, got, name + " (32x32x32 loop)")
 
@@ -599,7 +599,7 @@ def test_mfma_fp8_tile256_mi16_loop(ctx, tile256):
     shapes = ((256, 512, 256, dt.bf16, True), (300, 768, 260, dt.f32, False),
               (128, 1024, 512, dt.bf16, False), (512, 2048, 256, dt.f32, False))
     for variant in (1, 0):
-        with _capi.kernel_variants(b8x=variant):
+        with _capi.kernel_variants(gemm=6, b8x=variant):
             for (M, K, N, dd, with_sum) in shapes:
                 say("mfma_b8 256x256 fp8 kernel, variant %d, %dx%dx%d" % (variant, M, K, N))
                 p = fp8_gemm(M, K, N, 178, dst_dt=dd, with_sum=with_sum)

@@ -40,7 +40,7 @@ ELTWISE = {
 BINARY = ["binary_add", "binary_mul", "binary_max", "binary_min", "binary_div", "binary_sub", "binary_ge",
           "binary_gt", "binary_le", "binary_lt", "binary_eq", "binary_ne"]
 # sqrt, log and pow see negative accumulators (NaN in both); the routes are compared NaN for NaN
-ROUTES = ["generic", "general", "tile256"]
+ROUTES = ["generic", "general", "tile256", "two_per_cu"]
 
 
 def say(msg):
@@ -58,7 +58,8 @@ def _run(ctx, route, p):
     eng, strm = ctx
     if route == "generic":
         return p.run_gpu(eng, strm, impl=cases.GENERIC)
-    with _capi.kernel_variants(gemm=6 if route == "tile256" else 2):
+    # tile256: 256 x 256 tiles, one workgroup per CU; two_per_cu: 256 x 128 tiles; general: the 128 x 128 configuration
+    with _capi.kernel_variants(gemm=2 if route == "general" else 6, b8x=2 if route == "two_per_cu" else 3):
         got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
     assert pd.impl_info_str() == cases.MFMA
     return got
