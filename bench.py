@@ -459,64 +459,58 @@ def _c2_primitive(A, memory, dt, tag, T, eng, strm, data):
 
 
 def bench_gemm_anatomy(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20, rounds=3, settle_s=1.5):
-    """Where a config-2 launch spends its time, from the kernels' own measurement switches (QMM_MEASURE): the launch as
-    it is, the same launch ending after the main loop (no epilogue, nothing stored), and per-tile time stamps (core
-    clock counter and a constant 100 MHz counter at kernel entry, loop entry, loop exit and the end of the epilogue),
-    which give the cycles per k-step and the clock each phase ran at. For the default kernel (256 x 256 tiles, one
-    workgroup per CU) and for the 256 x 128 kernel with two workgroups per CU (QMM_B8X_VARIANT=2)."""
+    """Where a config-2 launch spends its time, from the 256 x 256 kernel's own measurement switches (QMM_MEASURE):
+    the launch as it is, the same launch ending after the main loop (no epilogue, nothing stored), and per-tile time
+    stamps (core clock counter and a constant 100 MHz counter at kernel entry, loop entry, loop exit and the end of
+    the epilogue, and inside the epilogue), which give the cycles per k-step and the clock each phase ran at. Next to
+    it the same problem on the 256 x 128 kernel with two workgroups per CU (the default up to K 2048), timed only."""
     import ctypes as C
     from onednn_amd import _capi
     data = build_c2(A, dt, T)
     M, K, N = 4096, 4096, 14336
     ops = 2.0 * M * K * N
-    out = {}
-    for label, b8x, tile_n, per_cu in (("tile_256x256", 1, 256, 1), ("tile_256x128_two_per_cu", 2, 128, 2)):
-        res = {}
-        for name, measure in (("as_is", 0), ("main_loop_only", 1)):
-            with _capi.kernel_variants(measure=measure, b8x=b8x):
-                pd, prim, ex = _c2_primitive(A, memory, dt, tag, T, eng, strm, data)
-            ms = float(np.median(_settled_times(prim, strm, hs, hiprt, ex, steps, rounds, settle_s)))
-            res[name] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / ms / 1e9, 1),
-                         "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8, 4)}
-            del prim, ex
-        res["epilogue_share_of_launch"] = round(1.0 - res["main_loop_only"]["ms_per_launch"] / res["as_is"]["ms_per_launch"], 4)
-        with _capi.kernel_variants(measure=2, b8x=b8x):
+    res = {}
+    for name, measure, b8x in (("as_is", 0, 3), ("main_loop_only", 1, 3), ("tile_256x128_two_per_cu", 0, 2)):
+        with _capi.kernel_variants(measure=measure, b8x=b8x):
             pd, prim, ex = _c2_primitive(A, memory, dt, tag, T, eng, strm, data)
-        _settled_times(prim, strm, hs, hiprt, ex, steps, 1, settle_s)       # the stamps kept are the last launch's
-        strm.wait()
-        ntiles = (M // 256) * (N // tile_n)
-        grid = min((ntiles + 7) // 8 * 8, 4096)
-        buf = (C.c_uint64 * (grid * 16))()
-        rc = _capi.lib().qmm_gemm_stamps_read(b8x, buf, C.sizeof(buf))
-        assert rc == 0, rc
-        t8 = np.frombuffer(buf, dtype=np.uint64).reshape(grid, 8, 2).astype(np.float64)
-        t8 = t8[t8[:, 3, 0] > 0]
-        t = t8[:, :4]
-        cyc = np.diff(t[:, :, 0], axis=1)            # core-clock cycles per phase: prologue, main loop, epilogue
-        ns = np.diff(t[:, :, 1], axis=1) * 10.0      # the constant counter ticks at 100 MHz
-        ksteps = K // 64
-        ghz = cyc / np.maximum(ns, 1.0)
-        med = lambda a: float(np.median(a))
-        mfma_cycles = 1024 * tile_n // 256           # MFMA cycles of one wave per k-step
-        res["stamps"] = {
-            "tiles": int(t.shape[0]), "k_steps_per_tile": ksteps, "workgroups_per_cu": per_cu,
-            "prologue_us": round(med(ns[:, 0]) / 1e3, 2), "main_loop_us": round(med(ns[:, 1]) / 1e3, 2),
-            "epilogue_us": round(med(ns[:, 2]) / 1e3, 2),
-            "main_loop_cycles_per_k_step": round(med(cyc[:, 1]) / ksteps, 1),
-            "mfma_cycles_per_k_step_of_the_waves_sharing_a_simd": mfma_cycles * per_cu,
-            "main_loop_clock_GHz": round(med(ghz[:, 1]), 3), "epilogue_clock_GHz": round(med(ghz[:, 2]), 3),
-            "epilogue_cycles": round(med(cyc[:, 2]), 0),
-            # inside the epilogue: staging of the first half, its rows (arithmetic + stores), staging of the second
-            # half, its rows
-            "epilogue_parts_cycles": {
-                "stage_half_0": round(med(t8[:, 4, 0] - t8[:, 2, 0]), 0), "rows_half_0": round(med(t8[:, 5, 0] - t8[:, 4, 0]), 0),
-                "stage_half_1": round(med(t8[:, 6, 0] - t8[:, 5, 0]), 0), "rows_half_1": round(med(t8[:, 3, 0] - t8[:, 6, 0]), 0)},
-            "launch_span_us": round(float(t[:, 3, 1].max() - t[:, 0, 1].min()) * 10.0 / 1e3, 1)}
-        out[label] = res
-    out["note"] = ("stamps: medians over the block tiles of one launch; clock = core-clock cycles / time of the constant "
-                   "100 MHz counter (10 ns resolution); the stamp code costs a scalar branch per phase. With two workgroups "
-                   "per CU a phase's time includes what the SIMD gave the other workgroup's wave")
-    return out
+        ms = float(np.median(_settled_times(prim, strm, hs, hiprt, ex, steps, rounds, settle_s)))
+        res[name] = {"ms_per_launch": round(ms, 4), "TOPs": round(ops / ms / 1e9, 1),
+                     "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8, 4)}
+        del prim, ex
+    res["epilogue_share_of_launch"] = round(1.0 - res["main_loop_only"]["ms_per_launch"] / res["as_is"]["ms_per_launch"], 4)
+    with _capi.kernel_variants(measure=2, b8x=3):
+        pd, prim, ex = _c2_primitive(A, memory, dt, tag, T, eng, strm, data)
+    _settled_times(prim, strm, hs, hiprt, ex, steps, 1, settle_s)       # the stamps kept are the last launch's
+    strm.wait()
+    ntiles = (M // 256) * (N // 256)
+    grid = min((ntiles + 7) // 8 * 8, 4096)
+    buf = (C.c_uint64 * (grid * 16))()
+    rc = _capi.lib().qmm_gemm_stamps_read(buf, C.sizeof(buf))
+    assert rc == 0, rc
+    t8 = np.frombuffer(buf, dtype=np.uint64).reshape(grid, 8, 2).astype(np.float64)
+    t8 = t8[t8[:, 3, 0] > 0]
+    t = t8[:, :4]
+    cyc = np.diff(t[:, :, 0], axis=1)            # core-clock cycles per phase: prologue, main loop, epilogue
+    ns = np.diff(t[:, :, 1], axis=1) * 10.0      # the constant counter ticks at 100 MHz
+    ksteps = K // 64
+    ghz = cyc / np.maximum(ns, 1.0)
+    med = lambda a: float(np.median(a))
+    res["stamps"] = {
+        "tiles": int(t.shape[0]), "k_steps_per_tile": ksteps,
+        "prologue_us": round(med(ns[:, 0]) / 1e3, 2), "main_loop_us": round(med(ns[:, 1]) / 1e3, 2),
+        "epilogue_us": round(med(ns[:, 2]) / 1e3, 2),
+        "main_loop_cycles_per_k_step": round(med(cyc[:, 1]) / ksteps, 1), "mfma_cycles_per_k_step": 1024,
+        "main_loop_clock_GHz": round(med(ghz[:, 1]), 3), "epilogue_clock_GHz": round(med(ghz[:, 2]), 3),
+        "epilogue_cycles": round(med(cyc[:, 2]), 0),
+        # inside the epilogue: staging of the first half of the tile, its rows (arithmetic + stores), staging of the
+        # second half, its rows
+        "epilogue_parts_cycles": {
+            "stage_half_0": round(med(t8[:, 4, 0] - t8[:, 2, 0]), 0), "rows_half_0": round(med(t8[:, 5, 0] - t8[:, 4, 0]), 0),
+            "stage_half_1": round(med(t8[:, 6, 0] - t8[:, 5, 0]), 0), "rows_half_1": round(med(t8[:, 3, 0] - t8[:, 6, 0]), 0)},
+        "launch_span_us": round(float(t[:, 3, 1].max() - t[:, 0, 1].min()) * 10.0 / 1e3, 1),
+        "note": "medians over the block tiles of one launch; clock = core-clock cycles / time of the constant 100 MHz counter "
+                "(10 ns resolution); the stamp code costs a scalar branch per phase"}
+    return res
 
 
 MFMA_KINDS = {"int8_16x16x64": 0, "int8_32x32x32": 1, "fp8_16x16x128": 2, "fp8_32x32x64": 3}

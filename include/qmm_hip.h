@@ -261,17 +261,16 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
 
 /* ---- measurement switches of the 256 x 256 GEMM kernels ----
  * QMM_MEASURE (environment, read at plan creation like the overrides above):
- * bit 0: the int8 kernels on 16 x 16 x 64 MFMAs (256 x 256 tiles with an even
- * number of k-steps; 256 x 128 tiles, QMM_B8X_VARIANT=2) end after their main
- * loop and store nothing (what the loop alone costs); bit 1: the first lane of every workgroup records (core clock counter,
+ * bit 0: the int8 kernel with 256 x 256 tiles on 16 x 16 x 64 MFMAs (even number
+ * of k-steps; QMM_B8X_VARIANT=3 selects it at any K) ends after its main loop
+ * and stores nothing (what the loop alone costs); bit 1: the first lane of every workgroup records (core clock counter,
  * 100 MHz counter) at kernel entry, main-loop entry, main-loop exit and the end
  * of the epilogue (slots 0..3), and inside the epilogue after each half of the
  * tile is staged (slots 4, 6) and after the first half's rows are stored (5). qmm_gemm_stamps_read() copies the records of the last such
- * launch of the 256 x 256 kernel (which = 1) or the 256 x 128 kernel (which = 2)
- * out: 8 slots x 2 x uint64 per block tile, tile = (blockIdx.x + gridDim.x *
+ * launch out: 8 slots x 2 x uint64 per block tile, tile = (blockIdx.x + gridDim.x *
  * blockIdx.y) % 4096, at most 4096 * 128 bytes. No counterpart in the
  * reference. */
-QMM_API int qmm_gemm_stamps_read(int which, void *host, size_t bytes);
+QMM_API int qmm_gemm_stamps_read(void *host, size_t bytes);
 
 /* ---- measurement aid ----
  * Launches a kernel that only reads: up to three byte ranges (16-byte aligned,

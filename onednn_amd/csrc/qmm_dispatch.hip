@@ -20,6 +20,7 @@ void launch_matmul_generic(const generic_params_t *dev_params,
 void launch_reorder_generic(const generic_reorder_params_t &params,
         const qmm_reorder_args_t &args, hipStream_t stream);
 bool gemm_b8_uses_tile256(const gemm_params_t &p, bool f8, int variant);
+bool gemm_b8x_two_per_cu(const gemm_params_t &p, bool f8);
 void launch_flip_u8(const void *src, void *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, hipStream_t stream);
 void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
@@ -1084,7 +1085,10 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.batch = (int32_t)P.batch;
         g.kb32 = (int32_t)geom.kb32;
         g.nb32 = (int32_t)geom.nb32;
-        if (g.a_is_u8 && u8_copy_bytes(&D) && args->scratch) {
+        // a u8 source is rewritten as s8 by a pre-pass only for the kernels that
+        // cannot read it as it is (the 256 x 256 ones with more than 4 k-steps)
+        if (g.a_is_u8 && u8_copy_bytes(&D) && args->scratch
+                && !gemm_b8x_two_per_cu(g, f8)) {
             gemm_params_t h = g;
             uint8_t *copy = (uint8_t *)args->scratch
                     + (D.wei_layout == QMM_LAYOUT_PLAIN

@@ -472,9 +472,7 @@ bool gemm_b8_uses_tile256(const gemm_params_t &p, bool f8, int variant) {
     // bf16 epilogue: 256 x 4096 x 4096 29 against 37 us, 2048 x 4096 x 4096 40
     // against 67, 1024 x 512 x 1024 13 against 21; 512 x 1024 x 1024 (16 tiles)
     // 15 against 10 and 128 x 4096 x 4096 (half-empty row tiles) 29 against 18)
-    if (f8 || (p.a_is_u8 && !p.a_preflipped)
-            || (p.switches & (GEMM_ONE_PER_CU | GEMM_MFMA32)))
-        return false;
+    if (f8 || (p.switches & (GEMM_ONE_PER_CU | GEMM_MFMA32))) return false;
     const int64_t tiles128 = tm * ((p.N + 127) / 128) * p.batch;
     const bool rows_full = 4 * (int64_t)p.M >= 3 * tm * 256;
     return tiles128 >= 32 && (rows_full || tiles128 >= 96);

@@ -50,10 +50,11 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 // main loop entry, main loop exit, end of the epilogue -- into a device array
 // that qmm_gemm_stamps_read() copies out; GEMM_SKIP_EPILOGUE ends the kernel
 // after the main loop. Both are a scalar branch on a kernel argument in the
-// normal path. Only the int8 16 x 16 x 64 kernel (even k-step count) has them:
-// the fp8 kernel has no registers to spare for the extra code.
+// normal path. Only the int8 256 x 256 kernel on 16 x 16 x 64 MFMAs (even
+// k-step count) has them: the fp8 kernel and the 256 x 128 kernel have no
+// registers to spare for the extra code.
 [[maybe_unused]] constexpr int STAMP_TILES = 4096, STAMP_SLOTS = 8;
-#if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5 || QMM_B8X_PART == 7)
+#if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5)
 #define QX_HAVE_STAMPS 1
 static __device__ unsigned long long g_gemm_stamps[STAMP_TILES * STAMP_SLOTS * 2];
 // slots: 0 kernel entry, 1 main loop entry, 2 main loop exit, 3 end of the
@@ -1067,6 +1068,18 @@ constexpr int LDS_TOTAL = TABS + 5 * 1024;
                 : dB + STAGE_BYTES; \
     }
 // row i of the fragment grid: 4 MFMAs with one other instruction after each
+// (u8 sources: a fragment's top bits are flipped in the k-step that reads it,
+// a row of MFMAs after its read was issued and a whole k-step before its use:
+// the MFMAs are inline assembly, so the compiler inserts no wait states between
+// a vector instruction that writes an operand and the MFMA that reads it)
+#define QW_FLIP(NB, i) \
+    if constexpr (U8) { \
+        fa[NB][i][0] ^= 0x80808080; \
+        fa[NB][i][1] ^= 0x80808080; \
+        fa[NB][i][2] ^= 0x80808080; \
+        fa[NB][i][3] ^= 0x80808080; \
+        QX_SB(); \
+    }
 #define QW_ROW(i, CB, X0, X1, X2, X3) \
     QW_MF(i, 0, CB); X0; QW_MF(i, 1, CB); X1; QW_MF(i, 2, CB); X2; \
     QW_MF(i, 3, CB); X3;
@@ -1084,10 +1097,14 @@ constexpr int LDS_TOTAL = TABS + 5 * 1024;
     QW_ROW(2, CB, QX_D2(a_vo, sa, dA), QW_RA(NB, 2), QW_RA(NB, 3), QX_D3(a_vo, sa, dA)) \
     QW_ROW(3, CB, QW_RA(NB, 4), QX_D4(a_vo, sa, dA), QW_RA(NB, 5), QW_DB0()) \
     QW_ROW(4, CB, QW_RA(NB, 6), QW_DB1(), QW_RA(NB, 7), QW_DB2()) \
-    QW_ROW(5, CB, , , , ) \
-    QW_ROW(6, CB, , , , ) \
+    QW_ROW(5, CB, QW_FLIP(NB, 0), QW_FLIP(NB, 1), QW_FLIP(NB, 2), QW_FLIP(NB, 3)) \
+    QW_ROW(6, CB, QW_FLIP(NB, 4), QW_FLIP(NB, 5), QW_FLIP(NB, 6), QW_FLIP(NB, 7)) \
     QW_ROW(7, CB, , , , )
 
+// U8: the source is u8: its fragments are turned into s8 = u8 - 128 by
+// flipping the top bit of every byte (the epilogue adds 128 x the weights'
+// column sums back).
+template <bool U8>
 __global__ void __launch_bounds__(b8w::NT, 2)
 gemm_b8w_kernel(const gemm_params_t p) {
     using namespace b8w;
@@ -1119,7 +1136,6 @@ gemm_b8w_kernel(const gemm_params_t p) {
     const int KT = p.K / BK; // host guarantees K % 64 == 0 and KT >= 4
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(lds_u8 *)lds);
-    QX_STAMP(0)
 
     uint32_t a_vo[4], b_vo[2];
 #pragma unroll
@@ -1193,6 +1209,8 @@ gemm_b8w_kernel(const gemm_params_t p) {
         QW_RA(0, 0); QW_RB(0, 0); QW_RB(0, 1); QW_RB(0, 2); QW_RB(0, 3);
         QW_RA(0, 1); QW_RA(0, 2); QW_RA(0, 3); QW_RA(0, 4); QW_RA(0, 5);
         QW_RA(0, 6); QW_RA(0, 7);
+        QW_FLIP(0, 0) QW_FLIP(0, 1) QW_FLIP(0, 2) QW_FLIP(0, 3)
+        QW_FLIP(0, 4) QW_FLIP(0, 5) QW_FLIP(0, 6) QW_FLIP(0, 7)
     }
     // k-step: tile kt has landed for every wave (the 6 requests of tile kt+1
     // may still be in flight), and every wave has read what it needed from the
@@ -1209,7 +1227,6 @@ gemm_b8w_kernel(const gemm_params_t p) {
         QW_ADV_B(); \
     }
     const int pairs = (KT + 1) / 2;
-    QX_STAMP(1)
     for (int it = 0; it < pairs; it++) {
         QW_KSTEP(0, 1)
         QW_KSTEP(1, 0)
@@ -1219,12 +1236,9 @@ gemm_b8w_kernel(const gemm_params_t p) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     QX_WV(0);
     __syncthreads();
-    QX_STAMP(2)
-    QX_SKIP_EPILOGUE(8, 4, 4)
 
     tile_epilogue<false, false, v4i, 8, 4, TABS, true>(
             p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
-    QX_STAMP(3)
 }
 
 void launch_b8x_int8_two_per_cu(const gemm_params_t &p, hipStream_t stream) {
@@ -1234,14 +1248,15 @@ void launch_b8x_int8_two_per_cu(const gemm_params_t &p, hipStream_t stream) {
     q.tiles_n = (p.N + BN - 1) / BN;
     const int ntiles = q.tiles_m * q.tiles_n;
     const int grid_x = ((ntiles + 7) / 8) * 8;
-    ensure_dynamic_lds((const void *)gemm_b8w_kernel, LDS_TOTAL);
-    hipLaunchKernelGGL(gemm_b8w_kernel, dim3(grid_x, p.batch), dim3(NT),
-            LDS_TOTAL, stream, q);
-}
-int gemm_stamps_read_two_per_cu(void *host, size_t bytes) {
-    return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_stamps), bytes, 0,
-                   hipMemcpyDeviceToHost)
-            == hipSuccess;
+    auto go = [&](auto kern) {
+        ensure_dynamic_lds((const void *)kern, LDS_TOTAL);
+        hipLaunchKernelGGL(kern, dim3(grid_x, p.batch), dim3(NT), LDS_TOTAL,
+                stream, q);
+    };
+    if (p.a_is_u8 && !p.a_preflipped)
+        go(gemm_b8w_kernel<true>);
+    else
+        go(gemm_b8w_kernel<false>);
 }
 #endif // int8, two workgroups per CU
 
@@ -1795,12 +1810,12 @@ void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream) {
 void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8_two_per_cu(const gemm_params_t &p, hipStream_t stream);
 int gemm_stamps_read_int8(void *host, size_t bytes);
-int gemm_stamps_read_two_per_cu(void *host, size_t bytes);
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_int8(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_short_k(const gemm_params_t &p, hipStream_t stream);
 void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream);
+bool gemm_b8x_two_per_cu(const gemm_params_t &p, bool f8);
 
 // Problems the kernels take: K a multiple of 64; s8 sources (u8 too when K is
 // at most 256, or rewritten as s8 by the caller), or fp8 sources with K a
@@ -1814,10 +1829,21 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     if (p.K % 64 != 0 || p.K < 64) return false;
     if (p.rowsum) return false; // weights zero points: the general kernel
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
-    if (p.a_is_u8 && !p.a_preflipped && !short_k(p)) return false;
+    if (p.a_is_u8 && !p.a_preflipped && !short_k(p)
+            && !gemm_b8x_two_per_cu(p, f8))
+        return false;
     if ((int64_t)256 * p.lda + 64 >= ((int64_t)1 << 32)) return false;
     if ((int64_t)8 * p.kb32 * 1024 >= ((int64_t)1 << 32)) return false;
     return true;
+}
+
+// Whether launch_gemm_b8x() takes the 256 x 128 kernel with two workgroups per
+// CU (which also reads u8 sources as they are).
+bool gemm_b8x_two_per_cu(const gemm_params_t &p, bool f8) {
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
+            * p.batch;
+    return !f8 && !(p.switches & (GEMM_MFMA32 | GEMM_ONE_PER_CU))
+            && ((p.switches & GEMM_TWO_PER_CU) || p.K <= 2048 || tiles256 <= 170);
 }
 
 // By default int8 runs on 16 x 16 x 64 MFMAs and fp8 on 16 x 16 x 128 (K a
@@ -1835,12 +1861,7 @@ bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
 // (GEMM_MFMA32: the 32 x 32 loops; GEMM_TWO_PER_CU / GEMM_ONE_PER_CU).
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     const int variant = (p.switches & GEMM_MFMA32) ? 0 : 1;
-    const bool s8_src = !p.a_is_u8 || p.a_preflipped;
-    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
-            * p.batch;
-    const bool two_per_cu = !f8 && s8_src && variant >= 1
-            && !(p.switches & GEMM_ONE_PER_CU)
-            && ((p.switches & GEMM_TWO_PER_CU) || p.K <= 2048 || tiles256 <= 170);
+    const bool two_per_cu = gemm_b8x_two_per_cu(p, f8);
     if (f8 && variant >= 1 && p.K % 256 == 0 && p.K >= 4 * 128)
         launch_b8x_fp8_mi16(p, stream);
     else if (f8)
@@ -1863,13 +1884,11 @@ void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
 } // namespace qmm
 
 #if !defined(QMM_B8X_PART)
-extern "C" int qmm_gemm_stamps_read(int which, void *host, size_t bytes) {
+extern "C" int qmm_gemm_stamps_read(void *host, size_t bytes) {
     if (!host
             || bytes > sizeof(unsigned long long) * qmm::STAMP_TILES
                             * qmm::STAMP_SLOTS * 2)
         return QMM_INVALID_ARGUMENTS;
-    const int ok = which == 2 ? qmm::gemm_stamps_read_two_per_cu(host, bytes)
-                              : qmm::gemm_stamps_read_int8(host, bytes);
-    return ok ? QMM_OK : QMM_RUNTIME_ERROR;
+    return qmm::gemm_stamps_read_int8(host, bytes) ? QMM_OK : QMM_RUNTIME_ERROR;
 }
 #endif

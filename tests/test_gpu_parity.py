@@ -504,6 +504,11 @@ def test_mfma_int8_tile256_mi16_loop(ctx, tile256, name):
 TWO_PER_CU_CASES = dict(MI16_CASES)
 TWO_PER_CU_CASES.update({k: v[0] for k, v in TILE256_CASES.items() if v[1] is True and not k.startswith("short_")})
 TWO_PER_CU_CASES.update({"ep_" + k: v[0] for k, v in TILE256_EPILOGUE_CASES.items() if v[1] is True and k != "f16_sum"})
+TWO_PER_CU_CASES["u8_source_zp121_k320"] = lambda: int8_linear(300, 320, 260, 124, src_zp=121)
+TWO_PER_CU_CASES["u8_source_no_zp_k1024_bf16"] = lambda: int8_linear(512, 1024, 256, 125, src_zp=None, dst_dt=dt.bf16,
+                                                                     per_token=True)
+TWO_PER_CU_CASES["u8_source_batched_k192_s32"] = lambda: int8_linear(256, 192, 130, 126, src_zp=7, src_scale=None,
+                                                                     dst_dt=dt.s32, batch=(3,))
 TWO_PER_CU_CASES["k256_min_f32"] = lambda: int8_linear(300, 256, 200, 121, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None)
 TWO_PER_CU_CASES["k4096_per_token_swish_rows"] = lambda: int8_linear(
     256, 4096, 384, 122, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, per_token=True)
