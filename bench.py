@@ -605,12 +605,14 @@ def bench_c1(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=200):
 
 def bench_int8_rows(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=100, K=4096, N=14336):
     """The decode step of config 2's layer (s8 x s8, per-token and per-column scales, bf16 dst) and of the W8A8 layers of
-    the reference's LLM list (--dt=s8:u8:f16, a u8 zero point per column) at 1, 32 and 64 rows: the streaming kernel.
-    The 59 MB of weights stay in the last-level cache between launches, so the rate is not an HBM figure."""
+    the reference's LLM list (--dt=s8:u8:f16, a u8 zero point per column) at 1, 32 and 64 rows: the streaming kernel;
+    and the same layers' prefill at 1024 rows (the MFMA kernels; a weights zero point costs a row-sum pre-pass and a
+    correction of the staged s32 sums in the epilogue). The 59 MB of weights stay in the last-level cache between
+    launches, so the rate is not an HBM figure."""
     out = {}
     r = np.random.default_rng(11)
     for name, wdt, zp in (("s8_s8", dt.s8, False), ("s8_u8_zp_per_column", dt.u8, True)):
-        for M in (1, 32, 64):
+        for M in (1, 32, 64, 1024):
             attr = A.primitive_attr()
             attr.set_scales(A.DNNL_ARG_SRC, 3, [1, K], dt.f32)  # per token, as in config 2
             attr.set_scales_mask(A.DNNL_ARG_WEIGHTS, 2)

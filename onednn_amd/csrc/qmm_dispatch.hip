@@ -333,12 +333,11 @@ bool build_epilogue(epilogue_t &ep, const generic_params_t &P,
     // straight-line shapes (see EP_FAST_* in qmm_device.hpp)
     ep.fast = EP_FAST_NONE;
     ep.fast_ext = 0;
-    const bool scales_f32 = (!ep.src_scale.ptr || ep.src_scale.dt == dt_f32)
-            && (!ep.wei_scale.ptr || ep.wei_scale.dt == dt_f32);
+    // (scales of any type: every kernel converts them to f32 as it loads them)
     const bool dst_base = ep.dst.dt == dt_bf16 || ep.dst.dt == dt_f32;
     const bool dst_more = one_of(ep.dst.dt, {dt_f16, dt_s8, dt_u8});
     const bool bias_ok = !ep.bias.ptr || ep.bias.sm == 0; // per column
-    if (scales_f32 && bias_ok && ep.dst.sn == 1 && (dst_base || dst_more)
+    if (bias_ok && ep.dst.sn == 1 && (dst_base || dst_more)
             && ep.npo <= 1) {
         if (ep.npo == 0) {
             ep.fast = EP_FAST_PLAIN;

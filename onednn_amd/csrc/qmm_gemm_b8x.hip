@@ -102,7 +102,10 @@ constexpr int WS_OFF = SS_OFF + 1024;
 constexpr int CS_OFF = WS_OFF + 1024;
 constexpr int BI_OFF = CS_OFF + 1024;
 constexpr int ZP_OFF = BI_OFF + 1024;
-constexpr int LDS_TOTAL = ZP_OFF + 1024;
+// per row: the source row's sum with its zero-point term (s32), read where the
+// weights have zero points
+constexpr int RS_OFF = ZP_OFF + 1024;
+constexpr int LDS_TOTAL = RS_OFF + 1024;
 
 template <int N, typename F>
 QMM_D void static_for(F &&f) {
@@ -337,7 +340,7 @@ QMM_D void ep_rows_full(const epilogue_t &ep, const int *stg_r,
 // scales, written to LDS by the first 256 threads before the main loop (the
 // loads' latency passes under the prologue): absent ones as 1.0 / 0, columns
 // past N likewise.
-// TABS: where the five 1 KiB tables start (SS_OFF in the 256 x 256 kernels).
+// TABS: where the six 1 KiB tables start (SS_OFF in the 256 x 256 kernels).
 template <int TABS = b8x::SS_OFF>
 QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
         int m0, int n0, int bz) {
@@ -364,6 +367,9 @@ QMM_D void tile_operands_stage(const gemm_params_t &p, uint8_t *lds, int tid,
     ((int *)(lds + TABS + (CS_OFF - SS_OFF)))[tid] = cs;
     ((float *)(lds + TABS + (BI_OFF - SS_OFF)))[tid] = bi;
     ((float *)(lds + TABS + (ZP_OFF - SS_OFF)))[tid] = zp;
+    if (p.rowsum)
+        ((int *)(lds + TABS + (RS_OFF - SS_OFF)))[tid]
+                = p.rowsum[(int64_t)bz * p.M + min(m0 + tid, p.M - 1)];
 }
 
 // Epilogue of one block tile, shared by the int8 and fp8 kernels.
@@ -462,6 +468,23 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
     if (to_bf16 && !ext && ep.fast != EP_FAST_NONE) epilogue_flush_denormals();
     // wave-uniform: whole wave tile inside the matrix, dst rows (and a binary
     // operand's rows) aligned for vector access
+    // Weights zero points (and u8 weights, stored as s8 = u8 - 128): the s32
+    // accumulator also loses z_w'[n] x rowsum[m], rowsum being the source row's
+    // sum with its zero-point term, one s32 per row from a pre-pass
+    // (rowsum_b8_kernel): sum (s - z_s)(w - z_w) = P + comp colsum[n]
+    // - z_w'[n] (rowsum[m] + K comp). The staged sums are corrected in LDS by
+    // the lanes that read them back, ahead of either row path.
+    const bool has_wz = MI16 && !F8 && p.rowsum != nullptr;
+    int zw4[4] = {0, 0, 0, 0};
+    if (has_wz) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < envalid)
+                zw4[i] = (p.wei_zp ? load_int(p.wei_zp_dt, p.wei_zp,
+                                  (int64_t)(en + i) * p.wei_zp_sn)
+                                   : 0)
+                        - p.w_off;
+    }
     const bool full = m0 + wm0 + 128 <= p.M && n0 + wn0 + WN <= p.N
             && ep.fast != EP_FAST_NONE && epilogue_full4_ok(ep)
             && (!LEAN || (ep.fast <= EP_FAST_SUM && dstk <= EP_DST_F16));
@@ -493,6 +516,23 @@ QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
 #ifdef QX_HAVE_STAMPS
         QX_STAMP_IF(wave == 0 && lane == 0, 4 + 2 * h)
 #endif
+        if (has_wz && lane_on) {
+            // s32 arithmetic that wraps like the reference's int sums
+            int *const stg_m = (int *)lds + wave * (STGW / 4);
+            const int *const rsl
+                    = (const int *)(lds + TABS + (RS_OFF - SS_OFF)) + wm0 + h * 64;
+#pragma unroll 4
+            for (int it = 0; it < 64 / RPI; it++) {
+                const int row = it * RPI + lane / LPR;
+                const uint32_t rs = (uint32_t)rsl[row];
+                int4 t = *(const int4 *)&stg_m[row * PITCH + ecol];
+                t.x = (int)((uint32_t)t.x - (uint32_t)zw4[0] * rs);
+                t.y = (int)((uint32_t)t.y - (uint32_t)zw4[1] * rs);
+                t.z = (int)((uint32_t)t.z - (uint32_t)zw4[2] * rs);
+                t.w = (int)((uint32_t)t.w - (uint32_t)zw4[3] * rs);
+                *(int4 *)&stg_m[row * PITCH + ecol] = t;
+            }
+        }
         if (full) {
             const int64_t m_first = m0 + wm0 + h * 64;
             const float *const ssh = ssl + h * 64;
@@ -1027,8 +1067,8 @@ constexpr int STAGE_BYTES = A_BYTES + B_BYTES; // 24 KiB
 constexpr int RING = STAGES * STAGE_BYTES; // 72 KiB
 constexpr int STG_PITCH = 68, STG_WAVE = 64 * STG_PITCH * 4; // epilogue staging
 static_assert(4 * STG_WAVE <= RING, "the staging reuses the ring");
-constexpr int TABS = RING; // five 1 KiB operand tables (tile_operands_stage)
-constexpr int LDS_TOTAL = TABS + 5 * 1024;
+constexpr int TABS = RING; // six 1 KiB operand tables (tile_operands_stage)
+constexpr int LDS_TOTAL = TABS + 6 * 1024;
 } // namespace b8w
 
 #define QW_MF(i, j, cb) \
@@ -1827,7 +1867,9 @@ static bool short_k(const gemm_params_t &p) {
 
 bool gemm_b8x_eligible(const gemm_params_t &p, bool f8) {
     if (p.K % 64 != 0 || p.K < 64) return false;
-    if (p.rowsum) return false; // weights zero points: the general kernel
+    // weights zero points: the kernels on 16 x 16 MFMAs (their epilogue's row path)
+    if (p.rowsum && (f8 || (p.switches & GEMM_MFMA32) || p.K < 5 * 64))
+        return false;
     if (f8 && (p.K % 128 != 0 || p.K < 6 * 64)) return false;
     if (p.a_is_u8 && !p.a_preflipped && !short_k(p)
             && !gemm_b8x_two_per_cu(p, f8))
@@ -1843,7 +1885,10 @@ bool gemm_b8x_two_per_cu(const gemm_params_t &p, bool f8) {
     const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256)
             * p.batch;
     return !f8 && !(p.switches & (GEMM_MFMA32 | GEMM_ONE_PER_CU))
-            && ((p.switches & GEMM_TWO_PER_CU) || p.K <= 2048 || tiles256 <= 170);
+            && ((p.switches & GEMM_TWO_PER_CU) || p.K <= 2048 || tiles256 <= 170
+                    || (p.rowsum != nullptr
+                            && (tiles256 >= 512
+                                    || (p.a_is_u8 && !p.a_preflipped))));
 }
 
 // By default int8 runs on 16 x 16 x 64 MFMAs and fp8 on 16 x 16 x 128 (K a
@@ -1857,7 +1902,12 @@ bool gemm_b8x_two_per_cu(const gemm_params_t &p, bool f8) {
 // attention scores (K 128, f32 dst bound by its write stream) 0.84; and 0.79
 // where the 256 x 256 tiles number half the CUs (2048 x 4096 x 4096). So: two
 // per CU up to K 2048, and beyond that where the large tiles would leave more
-// than a third of the CUs without one. Plan-level switches override the choice
+// than a third of the CUs without one. Weights with zero points (p.rowsum): two
+// per CU at any K once every CU gets two rounds of tiles, the epilogue's
+// correction pass over the staged sums then runs under the other workgroup's
+// MFMAs (s8:u8:f16 with a zero point per column, 4096 x 4096 x 14336: 200
+// against 213 us; 1024 rows: 66 against 63), and always for a u8 source, which
+// only that kernel reads as it is. Plan-level switches override the choice
 // (GEMM_MFMA32: the 32 x 32 loops; GEMM_TWO_PER_CU / GEMM_ONE_PER_CU).
 void launch_gemm_b8x(const gemm_params_t &p, bool f8, hipStream_t stream) {
     const int variant = (p.switches & GEMM_MFMA32) ? 0 : 1;

@@ -105,6 +105,37 @@ def test_weights_zero_points_exact(ctx, name, weights_any):
     assert_bit_exact(got, p.run_oracle(), name)
 
 
+TILE256_CASES = {
+    "s8_u8_zp_per_column_ragged": dict(M=300, K=320, N=200),
+    "s8_u8_zp_per_column_k3072": dict(M=300, K=3072, N=520),
+    "s8_u8_no_zp_s32_dst": dict(M=257, K=512, N=130, wei_zp=None, dst_dt=dt.s32),
+    "s8_s8_zp_s32_common_bias": dict(M=130, K=384, N=260, wei_dt=dt.s8, wei_zp="common", wei_zp_dt=dt.s32,
+                                     bias_dt=dt.f32),
+    "s8_u8_src_zp_f16_dst": dict(M=512, K=1024, N=256, src_zp=-5, dst_dt=dt.f16),
+    "s8_u8_batched_s32_dst": dict(M=140, K=320, N=136, batch=(2,), dst_dt=dt.s32),
+    # u8 sources: only the 256 x 128 kernel reads them as they are
+    "u8_u8_both_zero_points": dict(M=200, K=320, N=130, src_dt=dt.u8, src_zp=121),
+    "u8_s8_zp_s8_per_column_s32_dst": dict(M=384, K=576, N=128, src_dt=dt.u8, wei_dt=dt.s8, wei_zp_dt=dt.s8,
+                                           src_zp=7, dst_dt=dt.s32),
+}
+
+
+@pytest.mark.parametrize("name", sorted(TILE256_CASES))
+@pytest.mark.parametrize("tiling", ["two_per_cu", "one_per_cu"])
+def test_weights_zero_points_on_the_256_row_kernels(ctx, name, tiling):
+    """Forced onto the 256 x 128 and 256 x 256 tilings, whose epilogue takes z_w'[n] x rowsum[m] off the s32 sums in
+    its row path; a u8 source reaches the 256 x 256 kernels only as an s8 copy, which these problems do not make, so
+    there the general kernel answers (still bit-exact)."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    say("mfma_b8 weights zero points, 256-row kernels: %s %s" % (name, tiling))
+    p = w8a8(seed=900 + len(name), **TILE256_CASES[name])
+    with _capi.kernel_variants(gemm=6, b8x=2 if tiling == "two_per_cu" else 3):
+        got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    assert pd.impl_info_str() == MFMA
+    assert_bit_exact(got, p.run_oracle(), name)
+
+
 def test_matches_the_per_element_kernel(ctx):
     eng, strm = ctx
     say("mfma_b8 weights zero points vs generic")
