@@ -26,10 +26,35 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 PEAK_INT8 = 5000.0  # TOP/s, dense MFMA int8 (published MI355X figure)
 PEAK_FP8 = 5000.0  # TFLOP/s, dense MFMA fp8
 PEAK_HBM = 8000.0  # GB/s
-# HBM bytes per launch of the config-2 kernel: rocprofv3 FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch), each scaled by what the same counter reads for a 1 GiB
-# device copy (--calibrate-copy): 188,820 KiB x 2.000 + 114,690 KiB x 1.000
-TRAFFIC_C2_BYTES = 386.7e6 + 117.4e6
+# HBM bytes per launch of the config-2 kernel come from the committed rocprofv3
+# summary: its "traffic-record" line holds FETCH_SIZE and WRITE_SIZE (KiB per
+# dispatch), the factor each counter needs (what it reads for a 1 GiB device
+# copy, --calibrate-copy) and a hash of the kernel's source file at the time.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_b8y_config2_pmc.txt")
+TRAFFIC_SOURCE = os.path.join(ROOT, "onednn_amd", "csrc", "qmm_gemm_b8x.hip")
+
+
+def traffic_from_profile(kernel="gemm_b8y_kernel"):
+    """(bytes per launch or None, note): None when the summary is missing, has no record for the kernel, or was
+    taken from another version of the kernel's source file."""
+    import hashlib
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+        src_hash = hashlib.sha256(open(TRAFFIC_SOURCE, "rb").read()).hexdigest()[:16]
+    except OSError as e:
+        return None, "no traffic figure: %s" % e
+    for ln in lines:
+        tok = ln.split()
+        if len(tok) > 2 and tok[0] == "traffic-record:" and tok[1] == kernel:
+            kv = dict(t.split("=", 1) for t in tok[2:])
+            if kv.get("source_sha256") != src_hash:
+                return None, ("the counters in profiles/%s were read on another version of %s"
+                              % (os.path.basename(TRAFFIC_PROFILE), os.path.basename(TRAFFIC_SOURCE)))
+            nbytes = (float(kv["fetch_kib"]) * float(kv["fetch_factor"])
+                      + float(kv["write_kib"]) * float(kv["write_factor"])) * 1024.0
+            return nbytes, "profiles/%s: FETCH_SIZE %s KiB x %s + WRITE_SIZE %s KiB x %s" % (
+                os.path.basename(TRAFFIC_PROFILE), kv["fetch_kib"], kv["fetch_factor"], kv["write_kib"], kv["write_factor"])
+    return None, "no traffic-record for %s in profiles/%s" % (kernel, os.path.basename(TRAFFIC_PROFILE))
 
 
 def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
@@ -64,7 +89,7 @@ def main():
                     help="seconds of untimed launches of the same primitive before the timed steps (after --warmup)")
     ap.add_argument("--cpu-rows", type=int, default=640, help="rows of config 2 timed on the CPU oracle")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="run only a 1 GiB device-to-device copy (reference point for the rocprofv3 "
+                    help="run only a 1 GiB copy kernel (reference point for the rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -77,10 +102,11 @@ def main():
         n = 1 << 30
         a, b = H.malloc(n), H.malloc(n)
         H.memset(a, 0x5A, n)
+        from onednn_amd import _capi as CA
         for _ in range(3):
-            H.memcpy_dtod(b, a, n)
+            CA.call("qmm_stream_copy", b, a, n, 2048, None)  # stream_copy_kernel: n bytes in, n bytes out
         H.device_synchronize()
-        print(json.dumps({"calibrate_copy_bytes": n, "launches": 3}))
+        print(json.dumps({"calibrate_copy_bytes": n, "launches": 3, "kernel": "stream_copy_kernel"}))
         return
 
     import onednn_amd as dnnl
@@ -150,6 +176,7 @@ def main():
     tops = ops / (wall_ms * 1e-3) / 1e12
     kern_tops = ops / (ev_ms * 1e-3) / 1e12
 
+    traffic = traffic_from_profile()
     out = {
         "metric": "int8/fp8 matmul TOPS + % MFMA peak; int4-weight GEMV HBM GB/s, 1 MI355X",
         "value": round(tops, 2), "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -162,7 +189,7 @@ def main():
                                    "so the timed steps run at the settled clock" % args.clock_warmup_s},
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TOP/s",
                      "frac": round(kern_tops / PEAK_INT8, 4),
-                     "traffic": TRAFFIC_C2_BYTES if args.variant == 0 else None,
+                     "traffic": traffic[0] if args.variant == 0 else None, "traffic_source": traffic[1],
                      "kernel": "gemm_b8y_kernel (int8, 256x256 tile, 16x16x64 MFMA)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }

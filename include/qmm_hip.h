@@ -289,6 +289,13 @@ QMM_API int qmm_stream_read(const void *p0, size_t n0, const void *p1,
  * stream can reach on this card. No counterpart in the reference. */
 QMM_API int qmm_stream_write(void *dst, size_t bytes, int groups, void *hip_stream);
 
+/* Launches a plain copy kernel: `groups` workgroups of 256 lanes move `bytes`
+ * (both pointers 16-byte aligned) from src to dst, one 16-byte vector per lane
+ * and pass. A kernel of known traffic: profiler counters of HBM bytes are scaled
+ * by what they read for it. No counterpart in the reference. */
+QMM_API int qmm_stream_copy(void *dst, const void *src, size_t bytes, int groups,
+        void *hip_stream);
+
 /* Launches `groups` workgroups of four waves that issue nothing but the MFMAs
  * of the 256 x 256 GEMM kernels' main loop (`ksteps` k-steps, even, of the
  * 128 x 128 wave tile) on register-resident operands (data 0: uniformly random

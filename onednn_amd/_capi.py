@@ -140,6 +140,7 @@ _SIGNATURES = {
     "qmm_reorder_impl_name": (C.c_char_p, [_P]),
     "qmm_stream_read": (_I, [_P, C.c_size_t, _P, C.c_size_t, _P, C.c_size_t, _P, _P]),
     "qmm_stream_write": (_I, [_P, C.c_size_t, _I, _P]),
+    "qmm_stream_copy": (_I, [_P, _P, C.c_size_t, _I, _P]),
     "qmm_gemm_stamps_read": (_I, [_P, C.c_size_t]),
     "qmm_mfma_ceiling": (_I, [_I, _I, _I, _I, _P, _P, C.POINTER(C.c_double)]),
 }

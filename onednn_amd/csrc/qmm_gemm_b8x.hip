@@ -29,6 +29,7 @@
 // arithmetic as src/cpu/matmul/ref_matmul_int8.cpp:195-259); only epilogues of
 // the straight-line kinds (EP_FAST_*) are handled here, everything else stays
 // with the general kernel.
+#include <cstring>
 #include <type_traits>
 
 #include "qmm_device.hpp"
@@ -1832,9 +1833,16 @@ void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
     launch_b8x(gemm_b8y_kernel<false>, p, stream);
 }
 int gemm_stamps_read_int8(void *host, size_t bytes) {
-    return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_stamps), bytes, 0,
-                   hipMemcpyDeviceToHost)
+    // through pinned memory, as every other copy of the library to the host
+    void *pinned = nullptr;
+    if (hipHostMalloc(&pinned, bytes, hipHostMallocDefault) != hipSuccess)
+        return 0;
+    const bool ok = hipMemcpyFromSymbol(pinned, HIP_SYMBOL(g_gemm_stamps), bytes,
+                            0, hipMemcpyDeviceToHost)
             == hipSuccess;
+    if (ok) memcpy(host, pinned, bytes);
+    (void)hipHostFree(pinned);
+    return ok;
 }
 #elif QMM_B8X_PART == 5
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {

@@ -278,7 +278,22 @@ __global__ void __launch_bounds__(256) stream_write_kernel(
         v.x += 0x9e3779b9u;
     }
 }
+__global__ void __launch_bounds__(256) stream_copy_kernel(
+        uint4 *dst, const uint4 *src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
+        dst[i] = src[i];
+}
 } // namespace
+
+extern "C" int qmm_stream_copy(void *dst, const void *src, size_t bytes,
+        int groups, void *stream) {
+    if (!dst || !src || (((uintptr_t)dst | (uintptr_t)src) & 15) || groups < 1)
+        return QMM_INVALID_ARGUMENTS;
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(groups), dim3(256), 0,
+            (hipStream_t)stream, (uint4 *)dst, (const uint4 *)src, bytes / 16);
+    return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
+}
 
 extern "C" int qmm_stream_write(void *dst, size_t bytes, int groups, void *stream) {
     if (!dst || ((uintptr_t)dst & 15) || groups < 1) return QMM_INVALID_ARGUMENTS;
