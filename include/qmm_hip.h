@@ -252,7 +252,8 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  * plan is created (qmm_matmul_plan_create) and fixed for that plan's life; a
  * launch reads no process-wide state. Production code leaves them unset.
  *   QMM_GEMM_VARIANT: 0 by problem size (default); 1..3 a tile configuration of
- *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible
+ *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible;
+ *     for mfma_f16 plans 1 = 64 x 64 tiles, 2 = 128 x 128 tiles
  *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration
  *   QMM_B8X_VARIANT: the 256-row int8 / fp8 kernels: 1 = by shape (default: 16 x 16
  *     MFMAs; int8 with 256 x 128 tiles and two workgroups per CU up to K 2048,

@@ -30,9 +30,30 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef short v8s __attribute__((ext_vector_type(8)));
 
-constexpr int F16_BM = 64, F16_BN = 64, F16_BK = 32;
-constexpr int F16_A_PITCH = F16_BK * 2 + 16; // bytes of a staged source row
-constexpr int F16_B_PITCH = F16_BN * 2 + 16; // bytes of a staged weights row
+constexpr int F16_BK = 32;
+// Tile shapes: BM x BN of dst per workgroup of four waves arranged WGM x WGN.
+//   64 x 64, waves 1 x 4 (a wave owns 64 rows x 16 columns): small problems;
+//   128 x 128, waves 2 x 2 (64 x 64 per wave: 16 MFMAs per 32-k step for 8
+//   transposing and 8 plain fragment reads, four times the MFMAs per LDS read of
+//   the small tile): problems with enough such tiles to fill the chip.
+template <int BM_, int BN_, int WGM_, int WGN_>
+struct f16_tile {
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+    static constexpr int WM = BM / WGM, WN = BN / WGN; // wave tile
+    static constexpr int MF = WM / 16, NF = WN / 16; // 16 x 16 fragments of a wave
+    static constexpr int A_PITCH = F16_BK * 2 + 16; // bytes of a staged source row
+    static constexpr int B_PITCH = BN * 2 + 16; // bytes of a staged weights row
+    static constexpr int A_BYTES = BM * A_PITCH, B_BYTES = F16_BK * B_PITCH;
+    static constexpr int CA = BM * 4 / 256, CB = F16_BK * (BN / 8) / 256; // chunks a thread stages
+    static constexpr int OUT_PITCH = BN + 4; // words of a staged dst row
+    static constexpr int OUT_ROWS = WM; // dst rows staged at a time: one wave row
+    static constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) > OUT_ROWS * OUT_PITCH * 4
+            ? 2 * (A_BYTES + B_BYTES)
+            : OUT_ROWS * OUT_PITCH * 4;
+    static_assert(WM == 64 && CA >= 1 && CB >= 1, "tile shape");
+};
+typedef f16_tile<64, 64, 1, 4> f16_small_t;
+typedef f16_tile<128, 128, 2, 2> f16_big_t;
 
 template <bool BF>
 QMM_D v4f mma16(const v8s &a, const v8s &b, const v4f &c) {
@@ -119,12 +140,6 @@ QMM_D void static_for(F &&f) {
     }
 }
 
-constexpr int F16_A_BYTES = F16_BM * F16_A_PITCH, F16_B_BYTES = F16_BK * F16_B_PITCH;
-constexpr int F16_OUT_PITCH = F16_BN + 4; // words of a staged dst row
-constexpr int F16_LDS_BYTES = 2 * (F16_A_BYTES + F16_B_BYTES) > F16_BM * F16_OUT_PITCH * 4
-        ? 2 * (F16_A_BYTES + F16_B_BYTES)
-        : F16_BM * F16_OUT_PITCH * 4;
-
 // LIGHT: nothing follows the accumulation but at most one relu / linear / clip
 // (what the attention products carry). Everything else goes through the
 // post-op interpreter, whose register needs halve the waves a SIMD can hold.
@@ -137,69 +152,94 @@ QMM_HD bool light_epilogue(const epilogue_t &ep) {
                     || ep.po[0].alg == alg_clip || ep.po[0].alg == alg_clip_v2);
 }
 
-template <bool BF, bool LIGHT, int GA, int GB>
+template <bool BF, bool LIGHT, int GA, int GB, typename T>
 __global__ void __launch_bounds__(256)
 gemm_f16_kernel(const gemm16_params_t p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[F16_LDS_BYTES];
-    uint8_t *const lds_a = lds, *const lds_b = lds + 2 * F16_A_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_BYTES];
+    uint8_t *const lds_a = lds, *const lds_b = lds + 2 * T::A_BYTES;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wrow = wave / T::WGN, wcol = wave % T::WGN;
     const int r = lane & 15, c = lane >> 4;
-    const int m0 = blockIdx.y * F16_BM, n0 = blockIdx.x * F16_BN;
+    const int m0 = blockIdx.y * T::BM, n0 = blockIdx.x * T::BN;
     const int64_t bz = blockIdx.z;
     const uint16_t *A = p.A + bz * p.a_sb, *B = p.B + bz * p.b_sb;
-    // staging: thread t copies chunk (t % 4) of source row t / 4, and chunk
-    // (t % 8) of weights row t / 8 of the step (8 elements each)
-    const int ar = tid >> 2, ak = (tid & 3) * 8;
-    const int bk = tid >> 3, bn = (tid & 7) * 8;
-    const bool a_row_ok = m0 + ar < p.M;
-    const uint16_t *a_row = A + (int64_t)min(m0 + ar, p.M - 1) * p.lda;
+    // staging: chunk q = tid + 256 i (8 elements each) is chunk q % 4 of source
+    // row q / 4, and chunk q % (BN / 8) of weights row q / (BN / 8) of the step
+    constexpr int BCH = T::BN / 8;
     const int steps = (p.K + F16_BK - 1) / F16_BK;
 
     // operands are requested F16_AHEAD steps before they are staged: one slot
     // of registers per step in flight, named statically (the loop is unrolled
     // by the slot count)
-    req8_t<GA> ra[F16_AHEAD];
-    req8_t<GB> rb[F16_AHEAD];
+    req8_t<GA> ra[F16_AHEAD][T::CA];
+    req8_t<GB> rb[F16_AHEAD][T::CB];
     auto request = [&](int kt, auto S) {
         constexpr int sl = decltype(S)::value;
-        const int k0 = min(kt, steps - 1) * F16_BK; // past the end: a re-read nobody stages
-        request8<GA>(ra[sl], a_row, k0 + ak, p.K);
-        request8<GB>(rb[sl], B + (int64_t)min(k0 + bk, p.K - 1) * p.ldb, n0 + bn, p.N);
+        const int k0 = min(kt, steps - 1) * F16_BK; // (the prologue may ask past a short K)
+#pragma unroll
+        for (int i = 0; i < T::CA; i++) {
+            const int q = tid + 256 * i, ar = q >> 2, ak = (q & 3) * 8;
+            request8<GA>(ra[sl][i], A + (int64_t)min(m0 + ar, p.M - 1) * p.lda, k0 + ak, p.K);
+        }
+#pragma unroll
+        for (int i = 0; i < T::CB; i++) {
+            const int q = tid + 256 * i, bk = q / BCH, bn = (q % BCH) * 8;
+            request8<GB>(rb[sl][i], B + (int64_t)min(k0 + bk, p.K - 1) * p.ldb, n0 + bn, p.N);
+        }
     };
     auto stage = [&](int kt, auto S) {
         constexpr int sl = decltype(S)::value;
         const int k0 = kt * F16_BK, buf = kt & 1;
-        *(uint4 *)(lds_a + buf * F16_A_BYTES + ar * F16_A_PITCH + ak * 2)
-                = finish8<GA>(ra[sl], k0 + ak, p.K, a_row_ok);
-        *(uint4 *)(lds_b + buf * F16_B_BYTES + bk * F16_B_PITCH + bn * 2)
-                = finish8<GB>(rb[sl], n0 + bn, p.N, k0 + bk < p.K);
+#pragma unroll
+        for (int i = 0; i < T::CA; i++) {
+            const int q = tid + 256 * i, ar = q >> 2, ak = (q & 3) * 8;
+            *(uint4 *)(lds_a + buf * T::A_BYTES + ar * T::A_PITCH + ak * 2)
+                    = finish8<GA>(ra[sl][i], k0 + ak, p.K, m0 + ar < p.M);
+        }
+#pragma unroll
+        for (int i = 0; i < T::CB; i++) {
+            const int q = tid + 256 * i, bk = q / BCH, bn = (q % BCH) * 8;
+            *(uint4 *)(lds_b + buf * T::B_BYTES + bk * T::B_PITCH + bn * 2)
+                    = finish8<GB>(rb[sl][i], n0 + bn, p.N, k0 + bk < p.K);
+        }
     };
 
-    v4f acc[4];
+    v4f acc[T::MF][T::NF];
 #pragma unroll
-    for (int mf = 0; mf < 4; mf++) acc[mf] = v4f {0.f, 0.f, 0.f, 0.f};
+    for (int mf = 0; mf < T::MF; mf++)
+#pragma unroll
+        for (int nf = 0; nf < T::NF; nf++) acc[mf][nf] = v4f {0.f, 0.f, 0.f, 0.f};
 
     auto step = [&](int kt, auto S) {
         constexpr int sl = decltype(S)::value;
         const int buf = kt & 1;
-        request(kt + F16_AHEAD, S); // the slot's tile kt was staged a step ago
-        // weights fragment of the wave's 16 columns, transposed out of LDS
-        const uint8_t *vb = lds_b + buf * F16_B_BYTES + (4 * c + (r >> 2)) * F16_B_PITCH
-                + (16 * wave + 4 * (r & 3)) * 2;
-        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (v4s __attribute__((address_space(3))) *)vb);
-        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (v4s __attribute__((address_space(3))) *)(vb + 16 * F16_B_PITCH));
-        const v8s bf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        // the slot's tile kt was staged a step ago (short K: nothing left to ask
+        // for, and a dst-bound launch should not read its operands twice)
+        if (kt + F16_AHEAD < steps) request(kt + F16_AHEAD, S);
+        // weights fragments of the wave's columns, transposed out of LDS
+        v8s bf[T::NF];
 #pragma unroll
-        for (int mf = 0; mf < 4; mf++) {
-            // source fragment: row 16 mf + r, the same eight k
-            const uint8_t *pa = lds_a + buf * F16_A_BYTES + (16 * mf + r) * F16_A_PITCH;
+        for (int nf = 0; nf < T::NF; nf++) {
+            const uint8_t *vb = lds_b + buf * T::B_BYTES + (4 * c + (r >> 2)) * T::B_PITCH
+                    + (T::WN * wcol + 16 * nf + 4 * (r & 3)) * 2;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)vb);
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)(vb + 16 * T::B_PITCH));
+            bf[nf] = v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int mf = 0; mf < T::MF; mf++) {
+            // source fragment: row 16 mf + r of the wave's rows, the same eight k
+            const uint8_t *pa = lds_a + buf * T::A_BYTES
+                    + (T::WM * wrow + 16 * mf + r) * T::A_PITCH;
             const v4s x = *(const v4s *)(pa + (4 * c) * 2);
             const v4s y = *(const v4s *)(pa + (16 + 4 * c) * 2);
             const v8s af = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
-            acc[mf] = mma16<BF>(bf, af, acc[mf]);
+#pragma unroll
+            for (int nf = 0; nf < T::NF; nf++)
+                acc[mf][nf] = mma16<BF>(bf[nf], af, acc[mf][nf]);
         }
         if (kt + 1 < steps)
             stage(kt + 1, std::integral_constant<int, (sl + 1) % F16_AHEAD> {});
@@ -214,40 +254,51 @@ gemm_f16_kernel(const gemm16_params_t p) {
             if (kt + decltype(S)::value < steps) step(kt + decltype(S)::value, S);
         });
 
-    // register i of lane (r, c) is dst[m0 + 16 mf + r][n0 + 16 wave + 4 c + i].
-    // The tile goes through LDS so that 16 neighbouring lanes store one whole
-    // 64-column row piece instead of 16 rows with 8 bytes each.
+    // register i of lane (r, c) is dst[16 mf + r][16 nf + 4 c + i] of the wave
+    // tile. One wave row (64 dst rows) at a time goes through LDS, so that
+    // neighbouring lanes store whole row pieces of BN columns instead of 16
+    // rows with 8 bytes each.
     float *out = (float *)lds;
-#pragma unroll
-    for (int mf = 0; mf < 4; mf++)
-        *(v4f *)(out + (16 * mf + r) * F16_OUT_PITCH + 16 * wave + 4 * c) = acc[mf];
-    __syncthreads();
-    const int n = n0 + (tid & 15) * 4;
-    // one copy of the interpreter is enough; the light form is four stores
+    constexpr int TPR = T::BN / 4, RPI = 256 / TPR; // threads per row, rows per pass
+    const int n = n0 + (tid % TPR) * 4;
 #pragma unroll 1
-    for (int i = 0; i < 4; i++) {
-        const int row = 16 * i + (tid >> 4), m = m0 + row;
-        if (m < p.M && n < p.N) {
-            const v4f t = *(const v4f *)(out + row * F16_OUT_PITCH + (tid & 15) * 4);
-            float v[4] = {t[0], t[1], t[2], t[3]};
-            if constexpr (LIGHT) {
-                if (p.ep.npo) {
-                    const int alg = p.ep.po[0].alg;
-                    const float al = p.ep.po[0].alpha, be = p.ep.po[0].beta,
-                                sc = p.ep.po[0].scale;
+    for (int h = 0; h < T::WGM; h++) {
+        if (h) __syncthreads();
+        if (wrow == h) {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const float e = alg == alg_relu ? eltwise_one<alg_relu>(v[j], al, be)
-                                : alg == alg_linear     ? eltwise_one<alg_linear>(v[j], al, be)
-                                : alg == alg_clip       ? eltwise_one<alg_clip>(v[j], al, be)
-                                                  : eltwise_one<alg_clip_v2>(v[j], al, be);
-                        v[j] = e * sc;
+            for (int mf = 0; mf < T::MF; mf++)
+#pragma unroll
+                for (int nf = 0; nf < T::NF; nf++)
+                    *(v4f *)(out + (16 * mf + r) * T::OUT_PITCH + T::WN * wcol + 16 * nf + 4 * c)
+                            = acc[mf][nf];
+        }
+        __syncthreads();
+        // one copy of the interpreter is enough; the light form is four stores
+#pragma unroll 1
+        for (int i = 0; i < T::OUT_ROWS / RPI; i++) {
+            const int row = RPI * i + tid / TPR, m = m0 + T::WM * h + row;
+            if (m < p.M && n < p.N) {
+                const v4f t = *(const v4f *)(out + row * T::OUT_PITCH + (tid % TPR) * 4);
+                float v[4] = {t[0], t[1], t[2], t[3]};
+                if constexpr (LIGHT) {
+                    if (p.ep.npo) {
+                        const int alg = p.ep.po[0].alg;
+                        const float al = p.ep.po[0].alpha, be = p.ep.po[0].beta,
+                                    sc = p.ep.po[0].scale;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float e = alg == alg_relu ? eltwise_one<alg_relu>(v[j], al, be)
+                                    : alg == alg_linear     ? eltwise_one<alg_linear>(v[j], al, be)
+                                    : alg == alg_clip       ? eltwise_one<alg_clip>(v[j], al, be)
+                                                      : eltwise_one<alg_clip_v2>(v[j], al, be);
+                            v[j] = e * sc;
+                        }
                     }
+                    epilogue_store4(p.ep, v, bz * p.ep.dst.sb + (int64_t)m * p.ep.dst.sm + n,
+                            min(4, p.N - n));
+                } else {
+                    epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
                 }
-                epilogue_store4(p.ep, v, bz * p.ep.dst.sb + (int64_t)m * p.ep.dst.sm + n,
-                        min(4, p.N - n));
-            } else {
-                epilogue_apply_store4(p.ep, v, bz, m, n, min(4, p.N - n));
             }
         }
     }
@@ -439,8 +490,6 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
         else by_bf(std::integral_constant<int, 1> {});
         return;
     }
-    const dim3 grid((unsigned)((p.N + F16_BN - 1) / F16_BN),
-            (unsigned)((p.M + F16_BM - 1) / F16_BM), (unsigned)p.batch);
     // aligned 16-byte loads where rows start on 16-byte boundaries and hold a
     // multiple of 8 elements, else unaligned ones (rows of 8 elements and
     // more), else element loads
@@ -449,10 +498,30 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     const bool light = light_epilogue(p.ep) && p.ep.dst.sn == 1;
     // the interpreter form exists three times: aligned, any alignment, short rows
     if (!light && !(ga == 8 && gb == 8)) ga = gb = (ga != 1 && gb != 1) ? 0 : 1;
+    // 128 x 128 tiles once they give every CU a workgroup (the small tile's four
+    // times as many workgroups spread better below that) and K is long enough
+    // for the main loop to matter: 4096^3 421 -> 241 us, 32 x (2048 x 2048 x 128)
+    // 137 -> 80 us; with K = 128 (attention scores) a launch is its dst stream
+    // and the small tile's higher occupancy wins (998: 52 against 74 us). Not
+    // for the element-load forms.
+    const int64_t big_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+    const bool big = p.tile != 1 && ga != 1 && gb != 1 && p.M > 64 && p.N > 64
+            && (p.tile == 2 || (big_tiles >= 256 && p.K >= 256));
     auto go = [&](auto bf, auto lt, auto a, auto b) {
-        hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
-                                   decltype(a)::value, decltype(b)::value>),
-                grid, dim3(256), 0, stream, p);
+        if (big) {
+            const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)((p.M + 127) / 128),
+                    (unsigned)p.batch);
+            if constexpr (decltype(a)::value != 1 && decltype(b)::value != 1)
+                hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
+                                           decltype(a)::value, decltype(b)::value, f16_big_t>),
+                        grid, dim3(256), 0, stream, p);
+        } else {
+            const dim3 grid((unsigned)((p.N + 63) / 64), (unsigned)((p.M + 63) / 64),
+                    (unsigned)p.batch);
+            hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
+                                       decltype(a)::value, decltype(b)::value, f16_small_t>),
+                    grid, dim3(256), 0, stream, p);
+        }
     };
     auto by_bf = [&](auto lt, auto a, auto b) {
         if (p.bf) go(std::true_type {}, lt, a, b);

@@ -263,3 +263,28 @@ def test_e8m0_dst_scale(ctx, act, scale):
         exact = (src.logical().astype(np.float64) @ wei.logical().astype(np.float64)) / scale
         # the exact quotient (an integer or half-integer, exact in f32) rounded once to the dst type
         assert np.array_equal(got.view(np.uint16).reshape(-1), O.from_f32(act, exact.astype(np.float32)).reshape(-1))
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("route", ROUTES)
+@pytest.mark.parametrize("dst_dt", [dt.s8, dt.u8, dt.f32, dt.bf16, dt.s32], ids=str)
+@pytest.mark.parametrize("N", [999, 1001, 998])
+def test_rows_that_start_at_any_byte(ctx, route, dst_dt, N):
+    """dst rows of 999 / 1001 / 998 elements: a row starts at any byte (s8 / u8), at 2 mod 4 (bf16) or off its 16-byte
+    vector (f32 / s32), and the four-column stores of every epilogue are then vector stores at unaligned addresses,
+    which global memory instructions take. Integer data, a relu and a power-of-two dst scale: every route must give the
+    oracle's bits, in the last columns of a row and the first of the next one alike."""
+    say("odd row length %d, dst %s via %s" % (N, dst_dt, route))
+    M, K = (300, 320) if route in ("tile256", "two_per_cu") else (70, 128)
+    quant = dst_dt in (dt.s8, dt.u8)
+    p = cases.int8_linear(M, K, N, 91 + N, src_dt=dt.s8, dst_dt=dst_dt, src_zp=None,
+                          src_scale=None if dst_dt == dt.s32 else 2.0 ** -6,
+                          post_ops=None if dst_dt == dt.s32 else [{"kind": "eltwise", "alg": dnnl.algorithm.eltwise_relu,
+                                                                   "alpha": 0.25}],
+                          dst_scale=4.0 if quant else None, dst_zp=[3] if quant else None)
+    if dst_dt == dt.s32:
+        p.scales = {}
+    else:
+        r = np.random.default_rng(N)
+        p.scales["wei"] = (2, dt.f32, None, 2.0 ** r.integers(-7, -3, N))
+    assert_bit_exact(_run(ctx, route, p), p.run_oracle(), "odd rows %d %s %s" % (N, dst_dt, route))

@@ -86,6 +86,58 @@ def test_f16_matmul(ctx, name, exact):
     assert_f32_close(g, w, rel=step, scale=np.sqrt(K), what=name, max_slack_frac=1.0)
 
 
+BIG_TILE_CASES = {
+    "prefill_scores_198": CASES["prefill_scores_998"],
+    "prefill_context_k198": CASES["prefill_context_k198"],
+    "two_dims_bf16_f32_dst": CASES["two_dims_bf16_f32_dst"],
+    "odd_rows_with_bias_and_f32_dst": CASES["odd_rows_with_bias_and_f32_dst"],
+    "aligned_bias_clip_bf16": dict(sd=[2, 136, 256], wd=[2, 256, 200], bias=True, code=dt.bf16,
+                                   post_ops=[{"kind": "eltwise", "alg": A.eltwise_clip, "alpha": -2.0, "beta": 2.0}]),
+    "three_tiles_each_way_k520": dict(sd=[300, 520], wd=[520, 264],
+                                      post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0, "beta": 0.0}]),
+    "unaligned_rows_999": dict(sd=[2, 131, 999], wd=[2, 999, 999]),
+    "k_one_step_broadcast_weights": dict(sd=[3, 129, 24], wd=[1, 24, 130]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(BIG_TILE_CASES))
+@pytest.mark.parametrize("exact", [True, False])
+def test_f16_matmul_128x128_tiles(ctx, name, exact):
+    """The same products forced onto the 128 x 128 tiling (by default problems with at least 256 such tiles take it)."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    say("mfma_f16 128x128 tiles %s exact=%s" % (name, exact))
+    kw = BIG_TILE_CASES[name]
+    p = problem(seed=len(name) + 40, exact=exact, **kw)
+    with _capi.kernel_variants(gemm=2):
+        got, pd = p.run_gpu(eng, strm, return_pd=True)
+    assert pd.impl_info_str() == F16MM
+    want = p.run_oracle()
+    if exact:
+        assert_bit_exact(got, want, name)
+        with _capi.kernel_variants(gemm=1):
+            assert_bit_exact(p.run_gpu(eng, strm), want, name + " (64 x 64 tiles)")
+        return
+    code = kw.get("dst_dt") or kw.get("code", dt.f16)
+    g, w = O.to_f32(code, got), O.to_f32(code, want)
+    step = {dt.f16: 2.0 ** -10, dt.bf16: 2.0 ** -7, dt.f32: 1e-5}[code]
+    assert_f32_close(g, w, rel=step, scale=np.sqrt(kw["sd"][-1]), what=name, max_slack_frac=1.0)
+
+
+def test_f16_matmul_tilings_are_different_kernels(ctx):
+    """Forcing the tiling changes the summation grouping not at all (both sum 32 k per MFMA in the same order), so results
+    agree bit for bit on random data as well; what shows that the override took is the default choice: a problem with
+    256 tiles of 128 x 128 and one with fewer must both run, and the forced runs must equal the default ones."""
+    from onednn_amd import _capi
+    eng, strm = ctx
+    for sd, wd in (([16, 512, 64], [16, 64, 512]), ([2, 200, 64], [2, 64, 200])):
+        p = problem(sd, wd, 77)
+        base = p.run_gpu(eng, strm)
+        for v in (1, 2):
+            with _capi.kernel_variants(gemm=v):
+                assert_bit_exact(p.run_gpu(eng, strm), base, "tile variant %d" % v)
+
+
 def test_matches_the_per_element_kernel(ctx):
     eng, strm = ctx
     say("mfma_f16 vs generic")
