@@ -254,7 +254,9 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  *   QMM_GEMM_VARIANT: 0 by problem size (default); 1..3 a tile configuration of
  *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible;
  *     for mfma_f16 plans 1 = 64 x 64 tiles, 2 = 128 x 128 tiles
- *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration
+ *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration;
+ *     4 as 0 but with the split-K kernel instead of the one-launch kernel at
+ *     5 .. 64 rows
  *   QMM_B8X_VARIANT: the 256-row int8 / fp8 kernels: 1 = by shape (default: 16 x 16
  *     MFMAs; int8 with 256 x 128 tiles and two workgroups per CU up to K 2048,
  *     256 x 256 tiles and one per CU beyond), 2 = 256 x 128 two per CU wherever it

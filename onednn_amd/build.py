@@ -48,7 +48,7 @@ for v in GEMM_VARIANTS:
 # (even and odd numbers of k-steps), fp8 on 16 x 16 MFMAs, int8 with two workgroups per CU
 for v in (1, 2, 3, 4, 5, 6, 7):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
-for v in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11):
+for v in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))
 # the tiled decompression kernel per activation type and weights width
 for v in (0, 1, 2, 3):

@@ -40,6 +40,11 @@ bool gemm_w4a8_small_takes(const w4a8_prep_t &q);
 void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
         hipStream_t stream);
 int gemm_w4a8_tiny_max_groups(bool half);
+bool gemm_w4a8_mid_takes(int M, int group_k);
+int gemm_w4a8_mid_gpc(int M, int group_k);
+int gemm_w4a8_mid_wave_bytes(int M, int group_k, bool src_zp);
+void launch_gemm_w4a8_mid(const w4a8_small_t &p, bool has_zp, int nwv,
+        hipStream_t stream);
 void launch_pack_w4k(const void *src, void *dst, int dt, int64_t batch,
         int64_t K, int64_t N, int64_t sb, int64_t sk, int64_t sn,
         hipStream_t stream);
@@ -874,7 +879,7 @@ int qmm_matmul_plan_create(
     build_generic(p->host, *desc);
     p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
     p->gemm_variant = env_variant("QMM_GEMM_VARIANT", 0, 6, 0);
-    p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 3, 0);
+    p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 4, 0);
     p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 3, 1);
     p->measure = env_variant("QMM_MEASURE", 0, 3, 0);
     // resolve the static scratch's address on the current device now, so that
@@ -999,7 +1004,9 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         return fail(QMM_INVALID_ARGUMENTS, "scratch buffer is missing");
 
     const int gemm_variant = plan->gemm_variant;
-    const int w4a8_variant = plan->w4a8_variant;
+    // 4: as 0, but 5 .. 64 rows take the split-K kernel and its reduction
+    const bool w4a8_no_mid = plan->w4a8_variant == 4;
+    const int w4a8_variant = w4a8_no_mid ? 0 : plan->w4a8_variant;
     int impl = plan->impl;
     if (impl != impl_generic && impl != impl_gemm_f16 && !aligned16(args->src)) {
         if (!plan->dev)
@@ -1202,6 +1209,26 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
                     if (e != hipSuccess) return hip_fail(e, "kernel launch");
                     return QMM_OK;
                 }
+            }
+            if (!tiny_only && !w4a8_no_mid && gemm_w4a8_mid_takes((int)P.M, q.gk)) {
+                // 5 .. 64 rows: one launch, the waves of a workgroup cut K between
+                // them (8 waves while there are fewer 32-column blocks than CUs)
+                // eight waves where two such workgroups fit a CU's LDS or there
+                // are fewer 32-column blocks than CUs anyway
+                const int wb = gemm_w4a8_mid_wave_bytes((int)P.M, q.gk, sc.src_zp);
+                const int nwv = 8 * wb <= 80 * 1024
+                                || ((P.N + 31) / 32 < 256 && 8 * wb <= 160 * 1024)
+                        ? 8
+                        : 4;
+                h.splits = gemm_w4a8_mid_gpc((int)P.M, q.gk);
+                int64_t gpw = (q.ng + nwv - 1) / nwv;
+                if (q.gk == 32) gpw = (gpw + 1) / 2 * 2; // whole tiles per wave
+                h.gps = (int32_t)gpw;
+                h.ep = g.ep;
+                launch_gemm_w4a8_mid(h, sc.has_zp, nwv, stream);
+                const hipError_t e = hipGetLastError();
+                if (e != hipSuccess) return hip_fail(e, "kernel launch");
+                return QMM_OK;
             }
             if (!tiny_only) { // else (too many groups per wave): the tiled kernel
                 h.gps = sm.gps;

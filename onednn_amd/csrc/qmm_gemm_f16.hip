@@ -161,8 +161,19 @@ gemm_f16_kernel(const gemm16_params_t p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wrow = wave / T::WGN, wcol = wave % T::WGN;
     const int r = lane & 15, c = lane >> 4;
-    const int m0 = blockIdx.y * T::BM, n0 = blockIdx.x * T::BN;
-    const int64_t bz = blockIdx.z;
+    // Consecutive workgroups start on the 8 XCDs in turn. The launch is a flat
+    // list of tiles (columns fastest, then rows, then batch entries); XCD j takes
+    // the j-th eighth of it, so the tiles one L2 sees are neighbours: a few
+    // batch entries (attention heads) or a few row panels of one matrix, and
+    // their operands are fetched into that L2 only.
+    const int gx = (p.N + T::BN - 1) / T::BN, gy = (p.M + T::BM - 1) / T::BM;
+    int id = blockIdx.x;
+    {
+        const int total = gridDim.x;
+        if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    }
+    const int m0 = ((id / gx) % gy) * T::BM, n0 = (id % gx) * T::BN;
+    const int64_t bz = id / (gx * gy);
     const uint16_t *A = p.A + bz * p.a_sb, *B = p.B + bz * p.b_sb;
     // staging: chunk q = tid + 256 i (8 elements each) is chunk q % 4 of source
     // row q / 4, and chunk q % (BN / 8) of weights row q / (BN / 8) of the step
@@ -509,15 +520,13 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
             && (p.tile == 2 || (big_tiles >= 256 && p.K >= 256));
     auto go = [&](auto bf, auto lt, auto a, auto b) {
         if (big) {
-            const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)((p.M + 127) / 128),
-                    (unsigned)p.batch);
+            const dim3 grid((unsigned)(((p.N + 127) / 128) * ((p.M + 127) / 128) * p.batch));
             if constexpr (decltype(a)::value != 1 && decltype(b)::value != 1)
                 hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
                                            decltype(a)::value, decltype(b)::value, f16_big_t>),
                         grid, dim3(256), 0, stream, p);
         } else {
-            const dim3 grid((unsigned)((p.N + 63) / 64), (unsigned)((p.M + 63) / 64),
-                    (unsigned)p.batch);
+            const dim3 grid((unsigned)(((p.N + 63) / 64) * ((p.M + 63) / 64) * p.batch));
             hipLaunchKernelGGL((gemm_f16_kernel<decltype(bf)::value, decltype(lt)::value,
                                        decltype(a)::value, decltype(b)::value, f16_small_t>),
                     grid, dim3(256), 0, stream, p);

@@ -1175,6 +1175,359 @@ static void launch_tiny_zp(const w4a8_small_t &p, bool has_zp, int zpk,
         launch_tiny_cfg<NWV, SC, true, 2, MODE>(p, stream);
 }
 
+// ---- 5 .. 64 rows of one matrix: one launch, no partial results ----
+// The batched decode step (a few tens of tokens): still one read of the weights,
+// so the single-token kernel's shape with whole 32-row MFMA blocks. A workgroup
+// owns 32 columns; its NWV waves cut K between them in whole groups, and a wave
+// walks its range in chunks of MD_CH(RB) tiles: per chunk it requests the
+// weights tiles (straight into registers: the packed layout is the operand
+// order), its source rows as whole row pieces (16 lanes a row) and the chunk's
+// scales / zero points, one chunk ahead of the arithmetic; rows and tables wait
+// in a wave-private piece of LDS (no barrier before the end) and come back in
+// operand order. Group ends as in the kernels above. The waves' f32 results are
+// added through LDS in wave order (= K order) and every thread runs the
+// epilogue of a few elements. RB: blocks of 32 rows (1 or 2).
+// MODE as above: 1 groups of 32 k, 2 source zero points / u8 source.
+constexpr int md_ch(int rb) { return 8 / rb; } // 64-k tiles per chunk
+constexpr int md_gpc(int rb, int mode) { // most groups a chunk can hold
+    return (mode == 1 ? 2 : 1) * md_ch(rb);
+}
+constexpr int md_apitch(int rb) { return md_ch(rb) * BK + 16; } // staged row, bytes
+constexpr int md_wave_bytes(int rb, int mode, int gpc) {
+    // rows; source scales [, source zero points]; weights scales, zero points
+    // of the gpc groups a chunk holds; row sums
+    return rb * 32 * md_apitch(rb)
+            + gpc * (rb * 32 * 4 * (mode == 2 ? 2 : 1) + 32 * 4 * 2) + rb * 32 * 4;
+}
+static_assert(32 * md_apitch(1) >= 32 * 32 * 4 && 64 * md_apitch(2) >= 64 * 32 * 4,
+        "a wave's results fit where its rows were staged");
+
+template <int NWV, int RB, int SC, bool HAS_ZP, int ZPK, int MODE = 0>
+__global__ void __launch_bounds__(NWV * 64)
+w4a8_mid_kernel(const w4a8_small_t p) {
+    constexpr bool HALF = MODE == 1, SZP = MODE == 2;
+    static_assert(!SZP || HAS_ZP, "");
+    constexpr int R = RB * 32, CH = md_ch(RB), GPC = md_gpc(RB, MODE);
+    constexpr int APITCH = md_apitch(RB);
+    // p.splits: groups per full chunk (CH / p.tpg, or 2 CH of 32 k): the size of
+    // the wave's tables
+    const int gpc = p.splits;
+    const int WAVE_BYTES = md_wave_bytes(RB, MODE, gpc);
+    constexpr int PPR = CH * 4; // 16-byte pieces of a staged row
+    constexpr int A_PER = R * PPR / 64; // row pieces per lane and chunk
+    constexpr int SS_PER = GPC * R / 64, SW_PER = GPC * 32 / 64;
+    static_assert(A_PER == 16 && SS_PER >= 1 && SW_PER >= 1, "");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const w4a8_prep_t &q = p.q;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * 32;
+    const int g_begin = wave * p.gps; // p.gps: groups per wave, whole chunks' worth of tiles
+    const int g_cnt = max(0, min(p.gps, q.ng - g_begin));
+    const int T0 = HALF ? g_begin / 2 : g_begin * p.tpg; // first tile of the wave
+    const int KT = HALF ? g_cnt / 2 : g_cnt * p.tpg; // tiles of this wave
+    uint8_t *wA = lds + wave * WAVE_BYTES;
+    float *wss = (float *)(wA + R * APITCH); // [gpc][R]
+    int32_t *wzs = (int32_t *)(wss + gpc * R); // SZP only
+    float *wsw = wss + gpc * R * (SZP ? 2 : 1); // [gpc][32]
+    int32_t *wzw = (int32_t *)(wsw + gpc * 32);
+    int32_t *rsw = wzw + gpc * 32; // [R]
+    const int mrows = min(R, q.M);
+
+    v16f res[RB];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) res[i][r] = 0.f;
+
+    if (KT > 0) {
+        const bool has_ss = q.ss != nullptr, has_sw = q.sw != nullptr;
+        const int nb = min(n0 / 32, p.nb32 - 1);
+        const v4u *bsrc = (const v4u *)(p.B + (int64_t)nb * p.kt64 * 1024) + lane;
+        // what a chunk asks for, one chunk ahead of its use
+        uint4 av[A_PER];
+        v4u bn[CH];
+        uint32_t rs_[SS_PER], rzs_[SS_PER], rw_[SW_PER], rz_[SW_PER];
+        int64_t iz_[SW_PER];
+#pragma unroll
+        for (int j = 0; j < SS_PER; j++) rs_[j] = rzs_[j] = 0;
+#pragma unroll
+        for (int j = 0; j < SW_PER; j++) {
+            rw_[j] = rz_[j] = 0;
+            iz_[j] = 0;
+        }
+        // groups of the chunk that starts at tile t0 of the wave
+        auto first_group = [&](int t0) { return HALF ? 2 * t0 : t0 / p.tpg; };
+        auto request = [&](int t0, int cnt) {
+            // source rows: piece l % PPR of rows l / PPR + (64 / PPR) i
+#pragma unroll
+            for (int i = 0; i < A_PER; i++) {
+                const int row = min(lane / PPR + (64 / PPR) * i, q.M - 1);
+                const int pc = lane % PPR;
+                av[i] = make_uint4(0, 0, 0, 0);
+                if ((pc >> 2) < cnt)
+                    av[i] = *(const uint4 *)(q.A + (int64_t)row * q.lda
+                            + (int64_t)(T0 + t0) * BK + pc * 16);
+            }
+            const int gl0 = first_group(t0);
+#pragma unroll
+            for (int j = 0; j < SS_PER; j++) {
+                const int i = lane + j * 64;
+                const int gl = min(gl0 + i / R, g_cnt - 1), r = min(i % R, q.M - 1);
+                const int k0 = (g_begin + gl) * q.gk;
+                if (has_ss)
+                    rs_[j] = scale_raw<SC>(q.ss, r * q.ss_sm + (k0 / q.ss_g) * q.ss_sk);
+                if constexpr (SZP) {
+                    if (q.zs) // one byte: s8 or u8 (host-checked)
+                        rzs_[j] = ((const uint8_t *)q.zs)[r * q.zs_sm
+                                + (k0 / q.zs_g) * q.zs_sk];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < SW_PER; j++) {
+                const int i = lane + j * 64;
+                const int gl = min(gl0 + (i >> 5), g_cnt - 1), c = i & 31;
+                const int k0 = (g_begin + gl) * q.gk;
+                const int n = min(n0 + c, q.N - 1);
+                if (has_sw)
+                    rw_[j] = scale_raw<SC>(q.sw, (k0 / q.sw_g) * q.sw_sk + n * q.sw_sn);
+                if constexpr (ZPK != 0) {
+                    iz_[j] = (k0 / q.zw_g) * q.zw_sk + n * q.zw_sn;
+                    rz_[j] = zp_raw<ZPK>(q.zw, iz_[j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                bn[j] = __builtin_nontemporal_load(
+                        bsrc + (int64_t)(T0 + t0 + min(j, cnt - 1)) * 64);
+        };
+        auto stage = [&]() {
+#pragma unroll
+            for (int i = 0; i < A_PER; i++)
+                *(uint4 *)(wA + (lane / PPR + (64 / PPR) * i) * APITCH + (lane % PPR) * 16)
+                        = av[i];
+#pragma unroll
+            for (int j = 0; j < SS_PER; j++) {
+                const float v = scale_value<SC>(q.ss_dt, rs_[j]);
+                if (lane + j * 64 < gpc * R) {
+                    wss[lane + j * 64] = has_ss ? v : 1.f;
+                    if constexpr (SZP) {
+                        const int z = !q.zs ? 0
+                                : q.zs_dt == dt_s8 ? (int)(int8_t)rzs_[j]
+                                                   : (int)rzs_[j];
+                        wzs[lane + j * 64] = z - (q.a_flip ? 128 : 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < SW_PER; j++) {
+                const int i = lane + j * 64;
+                const float v = scale_value<SC>(q.sw_dt, rw_[j]);
+                if (i < gpc * 32) {
+                    wsw[i] = (has_sw ? v : 1.f) * 0.0625f;
+                    if constexpr (HAS_ZP) {
+                        int z = 0;
+                        if constexpr (ZPK != 0) z = zp_value<ZPK>(q.zw_dt, rz_[j], iz_[j]);
+                        wzw[i] = -16 * (z - q.w_off);
+                    }
+                }
+            }
+        };
+
+        v16i acc[RB];
+        int rsum[RB], csum = 0;
+#pragma unroll
+        for (int i = 0; i < RB; i++) {
+            rsum[i] = 0;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = 0;
+        }
+        int t_in_g = 0, gl = 0; // position in the group; group of the chunk
+        // group end: res += (float)(acc [+ zw * rowsum [+ zs * c2]]) * ss * sw
+        auto group_end = [&]() {
+            const float sw = wsw[gl * 32 + (lane & 31)];
+            int zw = 0, c2 = 0;
+            if constexpr (HAS_ZP) {
+                zw = wzw[gl * 32 + (lane & 31)];
+#pragma unroll
+                for (int i = 0; i < RB; i++) {
+                    // both k halves of a row: lanes l and l ^ 32
+                    const int tot = rsum[i] + __shfl_xor(rsum[i], 32);
+                    rsw[i * 32 + (lane & 31)] = tot;
+                    rsum[i] = 0;
+                }
+            }
+            if constexpr (SZP) {
+                // the column's 16 * sum w' of the group, both k halves
+                const int ctot = csum + __shfl_xor(csum, 32);
+                csum = 0;
+                c2 = -ctot - q.gk * zw;
+            }
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    // registers 4c .. 4c+3 are rows 8c + 4 (l / 32) .. + 3 of the block
+                    if (i * 32 + 8 * c >= mrows) continue;
+                    const int row = i * 32 + 8 * c + 4 * (lane >> 5);
+                    const float4 s4 = *(const float4 *)&wss[gl * R + row];
+                    const float ss[4] = {s4.x, s4.y, s4.z, s4.w};
+                    int rs[4] = {0, 0, 0, 0}, zs[4] = {0, 0, 0, 0};
+                    if constexpr (HAS_ZP) {
+                        const int4 r4 = *(const int4 *)&rsw[row];
+                        rs[0] = r4.x, rs[1] = r4.y, rs[2] = r4.z, rs[3] = r4.w;
+                    }
+                    if constexpr (SZP) {
+                        const int4 z4 = *(const int4 *)&wzs[gl * R + row];
+                        zs[0] = z4.x, zs[1] = z4.y, zs[2] = z4.z, zs[3] = z4.w;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int t = acc[i][4 * c + e];
+                        if constexpr (HAS_ZP) t += __mul24(zw, rs[e]);
+                        if constexpr (SZP) t += __mul24(zs[e], c2);
+                        res[i][4 * c + e] = __builtin_fmaf(
+                                (float)t * ss[e], sw, res[i][4 * c + e]);
+                    }
+                }
+            }
+            gl++;
+        };
+
+        request(0, min(CH, KT));
+        for (int t0 = 0; t0 < KT; t0 += CH) {
+            const int cnt = min(CH, KT - t0);
+            stage();
+            v4u bq[CH];
+#pragma unroll
+            for (int j = 0; j < CH; j++) bq[j] = bn[j];
+            if (t0 + CH < KT) request(t0 + CH, min(CH, KT - t0 - CH));
+            gl = 0;
+#pragma unroll
+            for (int j = 0; j < CH; j++) {
+                if (j < cnt) {
+                    const bool first = t_in_g == 0; // the group's accumulators start at 0
+#pragma unroll
+                    for (int ki = 0; ki < 2; ki++) {
+                        const uint32_t w0 = ki ? bq[j].z : bq[j].x;
+                        const uint32_t w1 = ki ? bq[j].w : bq[j].y;
+                        const v4i b = {(int)((w0 << 4) & 0xF0F0F0F0u),
+                                (int)(w0 & 0xF0F0F0F0u),
+                                (int)((w1 << 4) & 0xF0F0F0F0u),
+                                (int)(w1 & 0xF0F0F0F0u)};
+                        if constexpr (SZP) {
+                            int t = csum;
+                            t = __builtin_amdgcn_sdot4(b[0], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[1], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[2], 0x01010101, t, false);
+                            t = __builtin_amdgcn_sdot4(b[3], 0x01010101, t, false);
+                            csum = t;
+                        }
+#pragma unroll
+                        for (int i = 0; i < RB; i++) {
+                            const uint4 v = *(const uint4 *)(wA
+                                    + (i * 32 + (lane & 31)) * APITCH
+                                    + (j * 4 + ki * 2 + (lane >> 5)) * 16);
+                            v4i a = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                            if constexpr (SZP) // u8 source: s - 128 as s8
+                                a = v4i {(int)(v.x ^ q.a_flip), (int)(v.y ^ q.a_flip),
+                                        (int)(v.z ^ q.a_flip), (int)(v.w ^ q.a_flip)};
+                            if constexpr (HAS_ZP) {
+                                int t = rsum[i];
+                                t = __builtin_amdgcn_sdot4(a[0], 0x01010101, t, false);
+                                t = __builtin_amdgcn_sdot4(a[1], 0x01010101, t, false);
+                                t = __builtin_amdgcn_sdot4(a[2], 0x01010101, t, false);
+                                t = __builtin_amdgcn_sdot4(a[3], 0x01010101, t, false);
+                                rsum[i] = t;
+                            }
+                            if (HALF || (ki == 0 && first)) {
+                                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                        0, 0, 0, 0};
+                                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                        a, b, zero, 0, 0, 0);
+                            } else {
+                                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                        a, b, acc[i], 0, 0, 0);
+                            }
+                        }
+                        if constexpr (HALF) group_end();
+                    }
+                    if constexpr (!HALF) {
+                        if (++t_in_g == p.tpg) {
+                            t_in_g = 0;
+                            group_end();
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4 of its block,
+    // column l % 32; a wave's results go where its rows were staged
+    float *red = (float *)wA; // [R][32]
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            red[(i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4) * 32 + (lane & 31)]
+                    = res[i][r];
+    __syncthreads();
+    const int n = n0 + (threadIdx.x & 31);
+    if (n >= q.N) return;
+#pragma unroll 1
+    for (int row = threadIdx.x >> 5; row < mrows; row += NWV * 2) {
+        float v = ((const float *)lds)[row * 32 + (threadIdx.x & 31)];
+        for (int w = 1; w < NWV; w++)
+            v += ((const float *)(lds + w * WAVE_BYTES))[row * 32 + (threadIdx.x & 31)];
+        epilogue_apply_store(p.ep, v, 0, row, n);
+    }
+}
+
+template <int NWV, int RB, int SC, bool HAS_ZP, int ZPK, int MODE>
+static void launch_mid_cfg(const w4a8_small_t &p, hipStream_t stream) {
+    const size_t lds = (size_t)NWV * md_wave_bytes(RB, MODE, p.splits);
+    auto kern = w4a8_mid_kernel<NWV, RB, SC, HAS_ZP, ZPK, MODE>;
+    ensure_dynamic_lds((const void *)kern, (int)lds);
+    hipLaunchKernelGGL(kern, dim3((p.q.N + 31) / 32), dim3(NWV * 64), lds, stream, p);
+}
+
+template <int NWV, int RB, int SC, int MODE>
+static void launch_mid_zp(const w4a8_small_t &p, bool has_zp, int zpk,
+        hipStream_t stream) {
+    if constexpr (MODE != 2) {
+        if (!has_zp) {
+            launch_mid_cfg<NWV, RB, SC, false, 0, MODE>(p, stream);
+            return;
+        }
+    }
+    if (zpk == 0)
+        launch_mid_cfg<NWV, RB, SC, true, 0, MODE>(p, stream);
+    else if (zpk == 1)
+        launch_mid_cfg<NWV, RB, SC, true, 1, MODE>(p, stream);
+    else
+        launch_mid_cfg<NWV, RB, SC, true, 2, MODE>(p, stream);
+}
+
+// by waves per workgroup, rows (one or two blocks of 32) and scale size
+template <int MODE>
+static void launch_mid_mode(const w4a8_small_t &p, bool has_zp, int zpk, bool sc4,
+        int nwv, hipStream_t stream) {
+    auto by_sc = [&](auto W, auto B) {
+        constexpr int NWV = decltype(W)::value, RB = decltype(B)::value;
+        if (sc4)
+            launch_mid_zp<NWV, RB, 4, MODE>(p, has_zp, zpk, stream);
+        else
+            launch_mid_zp<NWV, RB, 2, MODE>(p, has_zp, zpk, stream);
+    };
+    auto by_rows = [&](auto W) {
+        if (p.q.M > 32) by_sc(W, std::integral_constant<int, 2> {});
+        else by_sc(W, std::integral_constant<int, 1> {});
+    };
+    if (nwv == 8) by_rows(std::integral_constant<int, 8> {});
+    else by_rows(std::integral_constant<int, 4> {});
+}
+
 #if defined(QMM_W4A8_PART) && QMM_W4A8_PART == 3
 // sum of the slices in slice order, then bias / post-ops / dst conversion:
 // one thread per four neighbouring columns of a row
@@ -1297,8 +1650,9 @@ static void launch_zp(const w4a8_params_t &p, int variant, hipStream_t stream) {
 // reduction, 4 the single-token kernel, 5 the tiled GEMM with source zero
 // points, 6 and 7 the tiled GEMM with groups of 32 k without / with zero
 // points, 8 and 9 the single-token kernel and 10 and 11 the split-K kernel with
-// groups of 32 k / source zero points); the unit without the macro holds the
-// pre-pass and the dispatch.
+// groups of 32 k / source zero points, 12 to 14 the one-launch kernel for 5 to 64
+// rows in its three modes); the unit without the macro holds the pre-pass and
+// the dispatch.
 #if defined(QMM_W4A8_PART)
 #if QMM_W4A8_PART == 1
 void launch_gemm_w4a8_nozp(const w4a8_params_t &p, int variant,
@@ -1348,6 +1702,21 @@ void launch_gemm_w4a8_reduce(const w4a8_small_t &p, hipStream_t stream) {
     hipLaunchKernelGGL(w4a8::w4a8_reduce_kernel, dim3((unsigned)blocks),
             dim3(256), 0, stream, (const float *)p.part, p.splits, p.q.M, p.q.N,
             p.ldp, p.ep);
+}
+#elif QMM_W4A8_PART == 12
+void launch_gemm_w4a8_mid_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream) {
+    w4a8::launch_mid_mode<0>(p, has_zp, zpk, sc4, nwv, stream);
+}
+#elif QMM_W4A8_PART == 13
+void launch_gemm_w4a8_mid_half_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream) {
+    w4a8::launch_mid_mode<1>(p, has_zp, zpk, sc4, nwv, stream);
+}
+#elif QMM_W4A8_PART == 14
+void launch_gemm_w4a8_mid_szp_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream) {
+    w4a8::launch_mid_mode<2>(p, true, zpk, sc4, nwv, stream);
 }
 #elif QMM_W4A8_PART == 4 || QMM_W4A8_PART == 8 || QMM_W4A8_PART == 9
 // the single-token kernel: whole tiles per group (4), groups of 32 k (8),
@@ -1401,6 +1770,12 @@ void launch_gemm_w4a8_tiny_half_part(const w4a8_small_t &p, bool has_zp,
         int zpk, bool sc4, int nwv, hipStream_t stream);
 void launch_gemm_w4a8_tiny_szp_part(const w4a8_small_t &p, bool has_zp,
         int zpk, bool sc4, int nwv, hipStream_t stream);
+void launch_gemm_w4a8_mid_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream);
+void launch_gemm_w4a8_mid_half_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream);
+void launch_gemm_w4a8_mid_szp_part(const w4a8_small_t &p, bool has_zp, int zpk,
+        bool sc4, int nwv, hipStream_t stream);
 
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream) {
     const int64_t total = (int64_t)p.ng * ((int64_t)p.M + p.N);
@@ -1445,6 +1820,39 @@ void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
                 p, true, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
     else
         launch_gemm_w4a8_tiny_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+}
+
+// 5 .. 64 rows in one launch: nwv waves per workgroup (4 or 8), p.gps groups per
+// wave. The kernel's chunks hold whole groups: groups of 32 k, or of 1, 2, 4 or
+// 8 tiles with at most 32 rows (up to 4 tiles with more).
+bool gemm_w4a8_mid_takes(int M, int group_k) {
+    if (M <= 4 || M > 64) return false;
+    if (group_k == 32) return true;
+    if (group_k % 64 != 0) return false;
+    const int tpg = group_k / 64, ch = w4a8::md_ch(M > 32 ? 2 : 1);
+    return tpg <= ch && ch % tpg == 0;
+}
+// groups per chunk (the kernel's p.splits) and the LDS a wave needs
+int gemm_w4a8_mid_gpc(int M, int group_k) {
+    const int ch = w4a8::md_ch(M > 32 ? 2 : 1);
+    return group_k == 32 ? 2 * ch : ch / (group_k / 64);
+}
+int gemm_w4a8_mid_wave_bytes(int M, int group_k, bool src_zp) {
+    return w4a8::md_wave_bytes(M > 32 ? 2 : 1, group_k == 32 ? 1 : (src_zp ? 2 : 0),
+            gemm_w4a8_mid_gpc(M, group_k));
+}
+void launch_gemm_w4a8_mid(const w4a8_small_t &p, bool has_zp, int nwv,
+        hipStream_t stream) {
+    if (p.q.M <= 0 || p.q.N <= 0) return;
+    if (p.tpg == 0)
+        launch_gemm_w4a8_mid_half_part(
+                p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+    else if (p.q.zsT)
+        launch_gemm_w4a8_mid_szp_part(
+                p, true, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
+    else
+        launch_gemm_w4a8_mid_part(
                 p, has_zp, zp_storage(p.q), scales_are_f32(p.q), nwv, stream);
 }
 
