@@ -1288,7 +1288,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         };
         g.a_vec = granule(g.lda, g.a_sb, args->src);
         g.b_vec = granule(g.ldb, g.b_sb, args->wei);
-        g.tile = gemm_variant == 1 || gemm_variant == 2 ? gemm_variant : 0;
+        g.tile = gemm_variant >= 1 && gemm_variant <= 3 ? gemm_variant : 0;
         launch_gemm_f16(g, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;

@@ -315,6 +315,234 @@ gemm_f16_kernel(const gemm16_params_t p) {
     }
 }
 
+// ---- short K over many columns (the attention scores: K = 64 / 128) ----------
+// Such a launch is its dst stream, and time stamps inside the kernels show where
+// it goes: a CU retires a store instruction of a wave only every 85 to 100
+// cycles whatever it carries, so the time is the number of store instructions --
+// four 16-bit results (8 bytes) a lane took 13.5 k cycles per 128 x 128 tile
+// against 4.4 k for its four k-steps; eight results (16 bytes) a lane 5.4 k. The
+// rest of this kernel keeps the CU storing: a workgroup owns 128 rows of one
+// batch entry, keeps them in LDS for all of K (at most 128) and WALKS a range
+// of column tiles; only the weights tiles stream (the next tile's k-step kt is
+// requested while this tile's is multiplied), so the next tile is never waited
+// for and a byte of dst costs half a byte of loads. A wave stores its 64 x 64
+// through a wave-private slice of LDS, 16 rows at a time (eight lanes a row
+// piece of 128 bytes), without a barrier. LIGHT epilogues only (what these
+// products carry). 32 x (2048 x 128 x 2048): 124 us against 165 us for the
+// 64 x 64 tiles (1000: 26 against 38 us).
+// A barrier that orders LDS traffic only. __syncthreads() also waits for every
+// global store the wave has issued (its fence covers global memory), which in a
+// kernel that keeps storing tiles while it multiplies the next one puts the full
+// latency of the stores in front of every k-step: 165 us instead of the time below.
+QMM_D void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+constexpr int F16_WALK_K = 128; // most k the resident rows hold
+constexpr int F16_WALK_APITCH = F16_WALK_K * 2 + 16; // bytes of a resident row
+constexpr int F16_WALK_SPITCH = 64 + 4; // words of a wave's staged dst row
+constexpr int F16_WALK_A = 128 * F16_WALK_APITCH;
+constexpr int F16_WALK_LDS
+        = F16_WALK_A + 2 * f16_big_t::B_BYTES + 4 * 16 * F16_WALK_SPITCH * 4;
+// STEPS: k-steps of a tile (2: K <= 64, 4: K <= 128; k past K multiplies zeros).
+// The weights of k-step kt of the NEXT tile are requested while this tile's are
+// multiplied: request slot and LDS buffer of a step are compile-time values.
+template <bool BF, int GA, int GB, int STEPS>
+__global__ void __launch_bounds__(256)
+gemm_f16_walk_kernel(const gemm16_params_t p, const int nseg) {
+    using T = f16_big_t;
+    static_assert(STEPS == 2 || STEPS == 4, "");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // F16_WALK_LDS bytes
+    uint8_t *const lds_a = lds, *const lds_b = lds + F16_WALK_A;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wrow = wave / T::WGN, wcol = wave % T::WGN;
+    const int r = lane & 15, c = lane >> 4;
+    float *const wout = (float *)(lds + F16_WALK_A + 2 * T::B_BYTES) + wave * 16 * F16_WALK_SPITCH;
+    // workgroup -> (batch entry, row block, segment of the column tiles); the
+    // XCDs take contiguous eighths of that list, as above
+    const int gx = (p.N + T::BN - 1) / T::BN, gy = (p.M + T::BM - 1) / T::BM;
+    int id = blockIdx.x;
+    {
+        const int total = gridDim.x;
+        if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    }
+    const int tps = (gx + nseg - 1) / nseg; // tiles per segment
+    const int tile0 = (id % nseg) * tps, ntile = min(tps, gx - tile0);
+    if (ntile <= 0) return; // (workgroup-uniform, before any barrier)
+    const int m0 = ((id / nseg) % gy) * T::BM;
+    const int64_t bz = id / (nseg * gy);
+    const uint16_t *A = p.A + bz * p.a_sb, *B = p.B + bz * p.b_sb;
+    constexpr int BCH = T::BN / 8;
+
+    req8_t<GB> rb[STEPS][T::CB];
+    auto request = [&](int n0, auto KT) __attribute__((always_inline)) {
+        constexpr int kt = decltype(KT)::value, k0 = kt * F16_BK;
+#pragma unroll
+        for (int i = 0; i < T::CB; i++) {
+            const int q = tid + 256 * i, bk = q / BCH, bn = (q % BCH) * 8;
+            request8<GB>(rb[kt][i], B + (int64_t)min(k0 + bk, p.K - 1) * p.ldb, n0 + bn, p.N);
+        }
+    };
+    auto stage = [&](int n0, auto KT) __attribute__((always_inline)) {
+        constexpr int kt = decltype(KT)::value, k0 = kt * F16_BK, buf = kt & 1;
+#pragma unroll
+        for (int i = 0; i < T::CB; i++) {
+            const int q = tid + 256 * i, bk = q / BCH, bn = (q % BCH) * 8;
+            *(uint4 *)(lds_b + buf * T::B_BYTES + bk * T::B_PITCH + bn * 2)
+                    = finish8<GB>(rb[kt][i], n0 + bn, p.N, k0 + bk < p.K);
+        }
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+
+    int n0 = tile0 * T::BN;
+    request(n0, S0 {});
+    request(n0, S1 {});
+    if constexpr (STEPS == 4) {
+        request(n0, S2 {});
+        request(n0, S3 {});
+    }
+    // the workgroup's rows, all of K: chunk q = tid + 256 i is chunk q % 16 of row q / 16
+    {
+        constexpr int NA = 128 * (STEPS * F16_BK / 8) / 256, CPR = STEPS * F16_BK / 8;
+        req8_t<GA> ra[NA];
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int q = tid + 256 * i, ar = q / CPR, ak = (q % CPR) * 8;
+            request8<GA>(ra[i], A + (int64_t)min(m0 + ar, p.M - 1) * p.lda, ak, p.K);
+        }
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int q = tid + 256 * i, ar = q / CPR, ak = (q % CPR) * 8;
+            *(uint4 *)(lds_a + ar * F16_WALK_APITCH + ak * 2)
+                    = finish8<GA>(ra[i], ak, p.K, m0 + ar < p.M);
+        }
+    }
+    stage(n0, S0 {});
+    lds_barrier();
+
+    v4f acc[T::MF][T::NF];
+    const int alg = p.ep.npo ? p.ep.po[0].alg : -1;
+    const float al = p.ep.po[0].alpha, be = p.ep.po[0].beta, sc = p.ep.po[0].scale;
+    const bool dst_bf = p.ep.dst.dt == dt_bf16;
+    const bool wide16 = (dst_bf || p.ep.dst.dt == dt_f16) && p.ep.dst.sn == 1;
+
+    // one k-step: the next tile's weights for this k-step requested, the MFMAs,
+    // the next step's weights staged, one barrier
+    auto step = [&](bool more, auto KT) __attribute__((always_inline)) {
+        constexpr int kt = decltype(KT)::value, buf = kt & 1;
+        constexpr bool last = kt == STEPS - 1;
+        if (more) request(n0 + T::BN, KT); // the slot's weights were staged a step ago
+        v8s bf[T::NF];
+#pragma unroll
+        for (int nf = 0; nf < T::NF; nf++) {
+            const uint8_t *vb = lds_b + buf * T::B_BYTES + (4 * c + (r >> 2)) * T::B_PITCH
+                    + (T::WN * wcol + 16 * nf + 4 * (r & 3)) * 2;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)vb);
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4s __attribute__((address_space(3))) *)(vb + 16 * T::B_PITCH));
+            bf[nf] = v8s {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int mf = 0; mf < T::MF; mf++) {
+            const uint8_t *pa = lds_a + (T::WM * wrow + 16 * mf + r) * F16_WALK_APITCH
+                    + kt * (F16_BK * 2);
+            const v4s x = *(const v4s *)(pa + (4 * c) * 2);
+            const v4s y = *(const v4s *)(pa + (16 + 4 * c) * 2);
+            const v8s af = {x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+#pragma unroll
+            for (int nf = 0; nf < T::NF; nf++)
+                acc[mf][nf] = mma16<BF>(bf[nf], af,
+                        kt == 0 ? v4f {0.f, 0.f, 0.f, 0.f} : acc[mf][nf]);
+        }
+        if constexpr (!last)
+            stage(n0, std::integral_constant<int, kt + 1> {});
+        else if (more)
+            stage(n0 + T::BN, S0 {});
+        lds_barrier();
+    };
+
+    for (int tile = 0; tile < ntile; tile++, n0 += T::BN) {
+        const bool more = tile + 1 < ntile;
+        step(more, S0 {});
+        step(more, S1 {});
+        if constexpr (STEPS == 4) {
+            step(more, S2 {});
+            step(more, S3 {});
+        }
+        // the wave's 64 x 64 results, 16 rows at a time through its own slice of
+        // LDS: lane (r, c) holds dst[16 mf + r][16 nf + 4 c + i]; 16 lanes then
+        // store a 64-column row piece
+        // (a fragment row per call with a compile-time index: left as a loop over
+        // mf the compiler kept it rolled and the accumulators in memory)
+        auto store_rows = [&](auto MFI) __attribute__((always_inline)) {
+            constexpr int mf = decltype(MFI)::value;
+#pragma unroll
+            for (int nf = 0; nf < T::NF; nf++)
+                *(v4f *)(wout + r * F16_WALK_SPITCH + 16 * nf + 4 * c) = acc[mf][nf];
+            // eight lanes a row, eight columns (16 bytes of a 16-bit dst) a lane:
+            // what a CU stores per cycle depends on the bytes per instruction
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int row = 8 * i + (lane >> 3), m = m0 + T::WM * wrow + 16 * mf + row;
+                const int n8 = n0 + T::WN * wcol + (lane & 7) * 8;
+                const v4f t0 = *(const v4f *)(wout + row * F16_WALK_SPITCH + (lane & 7) * 8);
+                const v4f t1 = *(const v4f *)(wout + row * F16_WALK_SPITCH + (lane & 7) * 8 + 4);
+                if (m < p.M && n8 < p.N) {
+                    float v[8] = {t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+                    if (alg >= 0) {
+#pragma unroll
+                        for (int j = 0; j < 8; j++) {
+                            const float e = alg == alg_relu ? eltwise_one<alg_relu>(v[j], al, be)
+                                    : alg == alg_linear     ? eltwise_one<alg_linear>(v[j], al, be)
+                                    : alg == alg_clip       ? eltwise_one<alg_clip>(v[j], al, be)
+                                                      : eltwise_one<alg_clip_v2>(v[j], al, be);
+                            v[j] = e * sc;
+                        }
+                    }
+                    const int64_t off = bz * p.ep.dst.sb + (int64_t)m * p.ep.dst.sm + n8;
+                    if (wide16 && n8 + 8 <= p.N) {
+                        uint16_t h[8];
+                        bool nan = false;
+#pragma unroll
+                        for (int j = 0; j < 8; j++) nan = nan || v[j] != v[j];
+                        if (dst_bf) {
+#pragma unroll
+                            for (int j = 0; j < 8; j++) h[j] = f32_to_bf16(v[j]);
+                        } else if (nan) { // (the reference's conversion of a NaN keeps its payload)
+#pragma unroll
+                            for (int j = 0; j < 8; j++) h[j] = f32_to_f16(v[j]);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 8; j++) h[j] = f32_to_f16_hw(v[j]);
+                        }
+                        uint32_t w[4];
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            w[j] = (uint32_t)h[2 * j] | ((uint32_t)h[2 * j + 1] << 16);
+                        typedef unsigned v4u_any2 __attribute__((ext_vector_type(4), aligned(2)));
+                        *(v4u_any2 *)((uint16_t *)p.ep.dst.ptr + off) = v4u_any2 {w[0], w[1], w[2], w[3]};
+                    } else {
+                        const float a4[4] = {v[0], v[1], v[2], v[3]}, b4[4] = {v[4], v[5], v[6], v[7]};
+                        epilogue_store4(p.ep, a4, off, min(4, p.N - n8));
+                        if (n8 + 4 < p.N) epilogue_store4(p.ep, b4, off + 4, min(4, p.N - n8 - 4));
+                    }
+                }
+            }
+        };
+        static_assert(T::MF == 4, "");
+        store_rows(S0 {});
+        store_rows(S1 {});
+        store_rows(S2 {});
+        store_rows(S3 {});
+    }
+}
+
 // ---- few rows per batch (M <= 4): the decode-time attention products ---------
 // One token's scores (1 x 128 by 128 x keys) and context (1 x keys by
 // keys x 128) per head are a few MB of weights read once; a 64 x 64 MFMA tile
@@ -518,6 +746,47 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream) {
     const int64_t big_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
     const bool big = p.tile != 1 && ga != 1 && gb != 1 && p.M > 64 && p.N > 64
             && (p.tile == 2 || (big_tiles >= 256 && p.K >= 256));
+    // short K over many column tiles with a light epilogue: the walking kernel,
+    // with the column tiles of a row block cut into as few segments as give
+    // every CU two workgroups
+    const int gx128 = (p.N + 127) / 128, gy128 = (p.M + 127) / 128;
+    // (by default only where a lane's eight results make one aligned 16-byte
+    // store: rows of a 16-bit dst that start on 16-byte boundaries; with rows of
+    // 998 elements the wide stores split and the kernel is no faster than the
+    // 64 x 64 tiles, 47.7 against 46.4 us)
+    const bool dst16 = (p.ep.dst.dt == dt_f16 || p.ep.dst.dt == dt_bf16) && p.ep.dst.sm % 8 == 0
+            && p.ep.dst.sb % 8 == 0 && (uintptr_t)p.ep.dst.ptr % 16 == 0;
+    const bool walk = p.tile != 1
+            && ((p.tile == 3 && p.K <= F16_WALK_K)
+                    || (p.tile == 0 && p.K <= F16_WALK_K && gx128 >= 4
+                            && (int64_t)gy128 * p.batch >= 64 && dst16))
+            && light && ga != 1 && gb != 1 && p.M > 64;
+    if (walk) {
+        int nseg = 1;
+        while ((int64_t)gy128 * p.batch * nseg < 512 && nseg * 2 <= gx128 / 2) nseg *= 2;
+        const dim3 grid((unsigned)(gy128 * p.batch * nseg));
+        auto gow = [&](auto bf, auto a, auto b) {
+            auto launch = [&](auto st) {
+                auto kern = gemm_f16_walk_kernel<decltype(bf)::value, decltype(a)::value,
+                        decltype(b)::value, decltype(st)::value>;
+                ensure_dynamic_lds((const void *)kern, F16_WALK_LDS);
+                hipLaunchKernelGGL(kern, grid, dim3(256), F16_WALK_LDS, stream, p, nseg);
+            };
+            if (p.K <= 64) launch(std::integral_constant<int, 2> {});
+            else launch(std::integral_constant<int, 4> {});
+        };
+        using W8 = std::integral_constant<int, 8>;
+        using W0 = std::integral_constant<int, 0>;
+        auto by_bfw = [&](auto a, auto b) {
+            if (p.bf) gow(std::true_type {}, a, b);
+            else gow(std::false_type {}, a, b);
+        };
+        if (ga == 8 && gb == 8) by_bfw(W8 {}, W8 {});
+        else if (ga == 8) by_bfw(W8 {}, W0 {});
+        else if (gb == 8) by_bfw(W0 {}, W8 {});
+        else by_bfw(W0 {}, W0 {});
+        return;
+    }
     auto go = [&](auto bf, auto lt, auto a, auto b) {
         if (big) {
             const dim3 grid((unsigned)(((p.N + 127) / 128) * ((p.M + 127) / 128) * p.batch));

@@ -187,7 +187,7 @@ struct gemm16_params_t {
     int32_t M, N, K, batch;
     int32_t bf; // bf16 (else f16)
     int32_t a_vec, b_vec; // elements per aligned load the rows allow: 8, 4, 2 or 1
-    int32_t tile; // 0: by problem size; 1: 64 x 64 tiles; 2: 128 x 128 tiles
+    int32_t tile; // 0: by problem size; 1: 64 x 64 tiles; 2: 128 x 128 tiles; 3: the walking kernel
     epilogue_t ep;
 };
 

@@ -288,3 +288,19 @@ def test_rows_that_start_at_any_byte(ctx, route, dst_dt, N):
         r = np.random.default_rng(N)
         p.scales["wei"] = (2, dt.f32, None, 2.0 ** r.integers(-7, -3, N))
     assert_bit_exact(_run(ctx, route, p), p.run_oracle(), "odd rows %d %s %s" % (N, dst_dt, route))
+
+
+@pytest.mark.parametrize("route", ROUTES)
+@pytest.mark.parametrize("op_dt", [dt.f32, dt.f16, dt.s8], ids=str)
+@pytest.mark.parametrize("N", [999, 1001])
+def test_binary_operand_rows_that_start_at_any_byte(ctx, route, op_dt, N):
+    """The same for the second tensor of a binary post-op: a dense [M, N] operand whose rows start off their vectors
+    (f32 at 4 mod 16, f16 at 2 mod 8, s8 at any byte), added to an f32 result. Integer data: bit for bit."""
+    say("binary add operand %s, odd row length %d via %s" % (op_dt, N, route))
+    M, K = (300, 320) if route in ("tile256", "two_per_cu") else (70, 128)
+    r = np.random.default_rng(7 * N + op_dt)
+    src1 = TensorSpec(op_dt, [M, N], None, r.integers(-50, 51, (M, N)).astype(np.float32))
+    p = cases.int8_linear(M, K, N, 17 + N, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None, src_scale=2.0 ** -6,
+                          post_ops=[{"kind": "binary", "alg": dnnl.algorithm.binary_add, "src1": src1}])
+    p.scales["wei"] = (2, dt.f32, None, 2.0 ** r.integers(-7, -3, N))
+    assert_bit_exact(_run(ctx, route, p), p.run_oracle(), "binary operand rows %d %s %s" % (N, op_dt, route))

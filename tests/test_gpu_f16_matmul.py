@@ -97,19 +97,29 @@ BIG_TILE_CASES = {
                                       post_ops=[{"kind": "eltwise", "alg": A.eltwise_relu, "alpha": 0.0, "beta": 0.0}]),
     "unaligned_rows_999": dict(sd=[2, 131, 999], wd=[2, 999, 999]),
     "k_one_step_broadcast_weights": dict(sd=[3, 129, 24], wd=[1, 24, 130]),
+    # many column tiles over a short K: what the walking kernel is for
+    "scores_k64_nine_column_tiles_clip_bf16": dict(sd=[1, 2, 300, 64], wd=[1, 2, 64, 1100], code=dt.bf16,
+                                                   post_ops=[{"kind": "eltwise", "alg": A.eltwise_clip, "alpha": -3.0,
+                                                              "beta": 3.0}]),
+    "scores_k128_unaligned_998": dict(sd=[1, 3, 260, 128], wd=[1, 3, 128, 998]),
+    "ragged_k40_n1000_f32_dst": dict(sd=[2, 150, 40], wd=[2, 40, 1000], dst_dt=dt.f32),
+    "k288_five_column_tiles": dict(sd=[131, 288], wd=[288, 600]),
 }
 
 
 @pytest.mark.parametrize("name", sorted(BIG_TILE_CASES))
 @pytest.mark.parametrize("exact", [True, False])
-def test_f16_matmul_128x128_tiles(ctx, name, exact):
-    """The same products forced onto the 128 x 128 tiling (by default problems with at least 256 such tiles take it)."""
+@pytest.mark.parametrize("tiling", [2, 3], ids=["tiles128", "walk"])
+def test_f16_matmul_128x128_tiles(ctx, name, exact, tiling):
+    """The same products forced onto the 128 x 128 tiling (by default problems with at least 256 such tiles and K >= 256
+    take it) and onto the kernel whose workgroups walk the column tiles of a 128-row block (the default for K <= 256 over
+    at least four column tiles; epilogues it does not take fall back to the tiled kernels)."""
     from onednn_amd import _capi
     eng, strm = ctx
-    say("mfma_f16 128x128 tiles %s exact=%s" % (name, exact))
+    say("mfma_f16 128x128 tiles %s exact=%s tiling=%d" % (name, exact, tiling))
     kw = BIG_TILE_CASES[name]
     p = problem(seed=len(name) + 40, exact=exact, **kw)
-    with _capi.kernel_variants(gemm=2):
+    with _capi.kernel_variants(gemm=tiling):
         got, pd = p.run_gpu(eng, strm, return_pd=True)
     assert pd.impl_info_str() == F16MM
     want = p.run_oracle()
@@ -133,7 +143,7 @@ def test_f16_matmul_tilings_are_different_kernels(ctx):
     for sd, wd in (([16, 512, 64], [16, 64, 512]), ([2, 200, 64], [2, 64, 200])):
         p = problem(sd, wd, 77)
         base = p.run_gpu(eng, strm)
-        for v in (1, 2):
+        for v in (1, 2, 3):
             with _capi.kernel_variants(gemm=v):
                 assert_bit_exact(p.run_gpu(eng, strm), base, "tile variant %d" % v)
 
