@@ -257,7 +257,7 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  *     workgroups that walk the column tiles (short K)
  *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration;
  *     4 as 0 but with the split-K kernel instead of the one-launch kernel at
- *     5 .. 64 rows
+ *     5 .. 64 rows, 5 as 0 but with the one-launch kernel wherever it applies
  *   QMM_B8X_VARIANT: the 256-row int8 / fp8 kernels: 1 = by shape (default: 16 x 16
  *     MFMAs; int8 with 256 x 128 tiles and two workgroups per CU up to K 2048,
  *     256 x 256 tiles and one per CU beyond), 2 = 256 x 128 two per CU wherever it

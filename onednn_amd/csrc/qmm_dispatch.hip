@@ -879,7 +879,7 @@ int qmm_matmul_plan_create(
     build_generic(p->host, *desc);
     p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
     p->gemm_variant = env_variant("QMM_GEMM_VARIANT", 0, 6, 0);
-    p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 4, 0);
+    p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 5, 0);
     p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 3, 1);
     p->measure = env_variant("QMM_MEASURE", 0, 3, 0);
     // resolve the static scratch's address on the current device now, so that
@@ -1004,9 +1004,10 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         return fail(QMM_INVALID_ARGUMENTS, "scratch buffer is missing");
 
     const int gemm_variant = plan->gemm_variant;
-    // 4: as 0, but 5 .. 64 rows take the split-K kernel and its reduction
-    const bool w4a8_no_mid = plan->w4a8_variant == 4;
-    const int w4a8_variant = w4a8_no_mid ? 0 : plan->w4a8_variant;
+    // 4: as 0, but 5 .. 64 rows take the split-K kernel and its reduction; 5: as
+    // 0, but they take the one-launch kernel wherever it applies
+    const bool w4a8_no_mid = plan->w4a8_variant == 4, w4a8_all_mid = plan->w4a8_variant == 5;
+    const int w4a8_variant = plan->w4a8_variant >= 4 ? 0 : plan->w4a8_variant;
     int impl = plan->impl;
     if (impl != impl_generic && impl != impl_gemm_f16 && !aligned16(args->src)) {
         if (!plan->dev)
@@ -1210,16 +1211,19 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
                     return QMM_OK;
                 }
             }
-            if (!tiny_only && !w4a8_no_mid && gemm_w4a8_mid_takes((int)P.M, q.gk)) {
-                // 5 .. 64 rows: one launch, the waves of a workgroup cut K between
-                // them (8 waves while there are fewer 32-column blocks than CUs)
+            // 5 .. 64 rows over at least 256 column blocks (one per CU and more:
+            // measured on 4096 x 14336 weights, with / without zero points, source
+            // scales per 32 k, a u8 source: 19.0 / 16.0 / 31.9 / 22.4 us against
+            // 24.9 / 24.5 / 41.8 / 30.4 us for the split-K kernel and its reduction;
+            // 48 rows 27.8 against 40.2; on 14336 x 4096 weights, 128 blocks, 27.6
+            // against 26.6): one launch, the waves of a workgroup cut K between them
+            if (!tiny_only && !w4a8_no_mid && gemm_w4a8_mid_takes((int)P.M, q.gk)
+                    && ((P.N + 31) / 32 >= 256 || w4a8_all_mid)) {
+                // (8 waves while there are fewer 32-column blocks than CUs)
                 // eight waves where two such workgroups fit a CU's LDS or there
                 // are fewer 32-column blocks than CUs anyway
                 const int wb = gemm_w4a8_mid_wave_bytes((int)P.M, q.gk, sc.src_zp);
-                const int nwv = 8 * wb <= 80 * 1024
-                                || ((P.N + 31) / 32 < 256 && 8 * wb <= 160 * 1024)
-                        ? 8
-                        : 4;
+                const int nwv = (P.N + 31) / 32 < 256 && 8 * wb <= 160 * 1024 ? 8 : 4;
                 h.splits = gemm_w4a8_mid_gpc((int)P.M, q.gk);
                 int64_t gpw = (q.ng + nwv - 1) / nwv;
                 if (q.gk == 32) gpw = (gpw + 1) / 2 * 2; // whole tiles per wave

@@ -1188,7 +1188,7 @@ static void launch_tiny_zp(const w4a8_small_t &p, bool has_zp, int zpk,
 // added through LDS in wave order (= K order) and every thread runs the
 // epilogue of a few elements. RB: blocks of 32 rows (1 or 2).
 // MODE as above: 1 groups of 32 k, 2 source zero points / u8 source.
-constexpr int md_ch(int rb) { return 8 / rb; } // 64-k tiles per chunk
+constexpr int md_ch(int rb) { return 4 / rb; } // 64-k tiles per chunk
 constexpr int md_gpc(int rb, int mode) { // most groups a chunk can hold
     return (mode == 1 ? 2 : 1) * md_ch(rb);
 }
@@ -1216,7 +1216,7 @@ w4a8_mid_kernel(const w4a8_small_t p) {
     constexpr int PPR = CH * 4; // 16-byte pieces of a staged row
     constexpr int A_PER = R * PPR / 64; // row pieces per lane and chunk
     constexpr int SS_PER = GPC * R / 64, SW_PER = GPC * 32 / 64;
-    static_assert(A_PER == 16 && SS_PER >= 1 && SW_PER >= 1, "");
+    static_assert(A_PER == 8 && SS_PER >= 1 && SW_PER >= 1, "");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const w4a8_prep_t &q = p.q;
     const int lane = threadIdx.x & 63;
@@ -1824,8 +1824,8 @@ void launch_gemm_w4a8_tiny(const w4a8_small_t &p, bool has_zp, int nwv,
 }
 
 // 5 .. 64 rows in one launch: nwv waves per workgroup (4 or 8), p.gps groups per
-// wave. The kernel's chunks hold whole groups: groups of 32 k, or of 1, 2, 4 or
-// 8 tiles with at most 32 rows (up to 4 tiles with more).
+// wave. The kernel's chunks hold whole groups: groups of 32 k, or of 1, 2 or 4
+// tiles with at most 32 rows (1 or 2 tiles with more).
 bool gemm_w4a8_mid_takes(int M, int group_k) {
     if (M <= 4 || M > 64) return false;
     if (group_k == 32) return true;

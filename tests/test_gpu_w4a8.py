@@ -34,7 +34,7 @@ def ctx():
     return eng, dnnl.stream(eng)
 
 
-@pytest.fixture(params=[0, 1, 2, 3, 4])
+@pytest.fixture(params=[0, 1, 2, 3, 4, 5])
 def variant(request):
     with _capi.kernel_variants(w4a8=request.param):
         yield request.param
