@@ -166,6 +166,10 @@ QMM_API int qmm_matmul_launch_static_scratch(const qmm_plan_t *plan,
 QMM_API size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N);
 /* Layout format_tag any resolves to for this problem, or QMM_LAYOUT_PLAIN. */
 QMM_API int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc);
+/* The same for one implementation (the packed layout `impl` takes this problem
+ * in, or QMM_LAYOUT_PLAIN): what format_tag any resolves to when the
+ * implementation list is walked past the first that applies. */
+QMM_API int qmm_matmul_impl_preferred_wei_layout(int impl, const qmm_matmul_desc_t *desc);
 
 /* ---- reorder ---- */
 typedef struct {

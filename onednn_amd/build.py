@@ -50,6 +50,9 @@ for v in (1, 2, 3, 4, 5, 6, 7):
     UNITS.append(("qmm_gemm_b8x.hip", "_p%d" % v, ["-DQMM_B8X_PART=%d" % v]))
 for v in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14):
     UNITS.append(("qmm_gemm_w4a8.hip", "_p%d" % v, ["-DQMM_W4A8_PART=%d" % v]))
+# f16 x 8-bit weights on the 256 x 256 design: even and odd numbers of k-steps
+for v in (0, 1):
+    UNITS.append(("qmm_gemm_f16w8.hip", "_p%d" % v, ["-DQMM_F16W8_PART=%d" % v]))
 # the tiled decompression kernel per activation type and weights width
 for v in (0, 1, 2, 3):
     UNITS.append(("qmm_gemm_w4f.hip", "_p%d" % v, ["-DQMM_W4F_PART=%d" % v]))

@@ -446,7 +446,7 @@ dnnl_status_t try_matmul_impl(pd_impl_t &pd, int impl) {
     if (wei_any) {
         // the implementation names its preferred weights layout
         qmm_matmul_desc_t probe = pd.mm;
-        const int want = qmm_matmul_preferred_wei_layout(&probe);
+        const int want = qmm_matmul_impl_preferred_wei_layout(impl, &probe);
         probe.wei_layout = want;
         if (want != QMM_LAYOUT_PLAIN
                 && qmm_matmul_impl_supports(impl, &probe) == QMM_OK) {

@@ -33,6 +33,7 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream);
 void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
         int src_zp_dt, hipStream_t stream);
+void launch_gemm_f16w8(const gemm_params_t &p, hipStream_t stream);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream);
@@ -587,6 +588,47 @@ w4a8_small_plan_t w4a8_small_plan(const generic_params_t &P, int variant) {
     return s;
 }
 
+// f16 activations x u8 / s8 weights whose scales and zero points do not vary
+// along K, at 256 rows and more (below that the decode implementation's
+// kernels, which work on blocks of 64 rows, waste less of a tile): the weights
+// in QMM_LAYOUT_MFMA_B8, converted to f16 in registers
+int supports_gemm_f16w8(const qmm_matmul_desc_t &D, const generic_params_t &P) {
+    if (D.dst.ndims != 2) return QMM_UNIMPLEMENTED;
+    if (D.src.dt != dt_f16 || !is_int8(D.wei.dt) || !D.apply_to_int)
+        return QMM_UNIMPLEMENTED;
+    if (!one_of(D.dst.dt, {dt_f16, dt_f32})) return QMM_UNIMPLEMENTED;
+    if (P.M < 256 || P.N == 0 || P.K < 5 * 32 || P.K % 32 != 0)
+        return QMM_UNIMPLEMENTED;
+    if (P.M > INT32_MAX || P.N > INT32_MAX || P.K > INT32_MAX)
+        return QMM_UNIMPLEMENTED;
+    if (!one_of(D.wei_layout, {QMM_LAYOUT_PLAIN, QMM_LAYOUT_MFMA_B8}))
+        return QMM_UNIMPLEMENTED;
+    if (D.src.strides[1] != 1 || D.src.strides[0] % 8 != 0)
+        return QMM_UNIMPLEMENTED;
+    // 32-bit offsets inside a block tile of the source / a column block of the
+    // packed weights
+    if (256 * 2 * D.src.strides[0] + 64 >= ((int64_t)1 << 32)
+            || 8 * b8_geom(1, P.K, P.N).kb32 * 1024 >= ((int64_t)1 << 32))
+        return QMM_UNIMPLEMENTED;
+    if (D.zps[QMM_SRC].set || D.zps[QMM_DST].set) return QMM_UNIMPLEMENTED;
+    if (D.scales[QMM_SRC].set && D.scales[QMM_SRC].mask != 0)
+        return QMM_UNIMPLEMENTED;
+    const qmm_quant_t &ws = D.scales[QMM_WEI], &wz = D.zps[QMM_WEI];
+    if (ws.set) {
+        if (!one_of(ws.dt, {dt_f32, dt_f16, dt_bf16})) return QMM_UNIMPLEMENTED;
+        if ((ws.mask & ~2) || P.q_wei_scale.g1 != 1) return QMM_UNIMPLEMENTED;
+    }
+    if (wz.set) {
+        // byte-sized zero points: 1152 - offset + zero point is then an integer
+        // that f16 holds exactly
+        if (!one_of(wz.dt, {dt_s8, dt_u8})) return QMM_UNIMPLEMENTED;
+        if ((wz.mask & ~2) || P.q_wei_zp.g1 != 1) return QMM_UNIMPLEMENTED;
+    }
+    epilogue_t ep;
+    if (!build_epilogue(ep, P, nullptr)) return QMM_UNIMPLEMENTED;
+    return QMM_OK;
+}
+
 int supports_gemv_w4(const qmm_matmul_desc_t &D, const generic_params_t &P) {
     const int nd = D.dst.ndims;
     if (nd != 2) return QMM_UNIMPLEMENTED;
@@ -717,8 +759,8 @@ int supports_generic(const qmm_matmul_desc_t &D, const generic_params_t &P) {
 }
 
 const char *impl_names[impl_count] = {"hip:gfx950:mfma_b8",
-        "hip:gfx950:mfma_w4a8", "hip:gfx950:decode_w4", "hip:gfx950:mfma_f16",
-        "hip:gfx950:generic"};
+        "hip:gfx950:mfma_w4a8", "hip:gfx950:mfma_f16w8", "hip:gfx950:decode_w4",
+        "hip:gfx950:mfma_f16", "hip:gfx950:generic"};
 
 // A kernel-selection override from the environment: an integer in [lo, hi],
 // else the default.
@@ -760,6 +802,7 @@ int qmm_matmul_impl_supports(int impl, const qmm_matmul_desc_t *desc) {
     switch (impl) {
         case impl_gemm_b8: return supports_gemm_b8(*desc, P);
         case impl_gemm_w4a8: return supports_gemm_w4a8(*desc, P);
+        case impl_gemm_f16w8: return supports_gemm_f16w8(*desc, P);
         case impl_gemv_w4: return supports_gemv_w4(*desc, P);
         case impl_gemm_f16: return supports_gemm_f16(*desc, P);
         case impl_generic: return supports_generic(*desc, P);
@@ -780,21 +823,24 @@ size_t qmm_packed_size(int layout, int dt, int64_t batch, int64_t K, int64_t N) 
     return 0;
 }
 
-int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
+int qmm_matmul_impl_preferred_wei_layout(
+        int impl, const qmm_matmul_desc_t *desc) {
+    if (!desc) return QMM_LAYOUT_PLAIN;
     qmm_matmul_desc_t d = *desc;
     // strides of an undecided weights tensor are not meaningful yet
-    d.wei_layout = QMM_LAYOUT_MFMA_B8;
-    if (qmm_matmul_impl_supports(impl_gemm_b8, &d) == QMM_OK)
-        return QMM_LAYOUT_MFMA_B8;
-    d.wei_layout = QMM_LAYOUT_MFMA_W4K64;
-    if (qmm_matmul_impl_supports(impl_gemm_w4a8, &d) == QMM_OK)
-        return QMM_LAYOUT_MFMA_W4K64;
-    d.wei_layout = QMM_LAYOUT_MFMA_W4;
-    if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
-        return QMM_LAYOUT_MFMA_W4;
-    d.wei_layout = QMM_LAYOUT_MFMA_W8;
-    if (qmm_matmul_impl_supports(impl_gemv_w4, &d) == QMM_OK)
-        return QMM_LAYOUT_MFMA_W8;
+    for (int layout : {QMM_LAYOUT_MFMA_B8, QMM_LAYOUT_MFMA_W4K64,
+                 QMM_LAYOUT_MFMA_W4, QMM_LAYOUT_MFMA_W8}) {
+        d.wei_layout = layout;
+        if (qmm_matmul_impl_supports(impl, &d) == QMM_OK) return layout;
+    }
+    return QMM_LAYOUT_PLAIN;
+}
+
+int qmm_matmul_preferred_wei_layout(const qmm_matmul_desc_t *desc) {
+    for (int impl = 0; impl < impl_generic; impl++) {
+        const int layout = qmm_matmul_impl_preferred_wei_layout(impl, desc);
+        if (layout != QMM_LAYOUT_PLAIN) return layout;
+    }
     return QMM_LAYOUT_PLAIN;
 }
 
@@ -857,6 +903,8 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
         return packed + (sm.use && sm.part_bytes > big ? sm.part_bytes : big);
     }
     if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
+    if (impl == impl_gemm_f16w8)
+        return qmm_packed_size(QMM_LAYOUT_MFMA_B8, desc->wei.dt, 1, K, N);
     if (impl == impl_gemv_w4)
         return qmm_packed_size(is_int8(desc->wei.dt) ? QMM_LAYOUT_MFMA_W8
                                                      : QMM_LAYOUT_MFMA_W4,
@@ -1294,6 +1342,40 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.b_vec = granule(g.ldb, g.b_sb, args->wei);
         g.tile = gemm_variant >= 1 && gemm_variant <= 3 ? gemm_variant : 0;
         launch_gemm_f16(g, stream);
+    } else if (impl == impl_gemm_f16w8) {
+        gemm_params_t g;
+        std::memset(&g, 0, sizeof(g));
+        if (!build_epilogue(g.ep, P, args))
+            return fail(QMM_RUNTIME_ERROR, "epilogue does not fold");
+        // the weights scales (left out of the epilogue for decompression
+        // problems, whose other kernels apply them to the weights): one per
+        // column or one in all, a factor of the f32 sum
+        const qmm_quant_t &ws = D.scales[QMM_WEI], &wz = D.zps[QMM_WEI];
+        if (ws.set
+                && !fold_quant(g.ep.wei_scale, P.q_wei_scale, ws, D.wei, D.dst,
+                        false, args->scales[QMM_WEI]))
+            return fail(QMM_RUNTIME_ERROR, "weights scales do not fold");
+        const b8_geom_t geom = b8_geom(1, P.K, P.N);
+        const uint8_t *packed = (const uint8_t *)args->wei;
+        if (D.wei_layout == QMM_LAYOUT_PLAIN) {
+            launch_pack_b8(args->wei, args->scratch, D.wei.dt, 1, P.K, P.N, 0,
+                    D.wei.strides[0], D.wei.strides[1], false, stream);
+            packed = (const uint8_t *)args->scratch;
+        }
+        g.A = (const uint8_t *)args->src;
+        g.lda = 2 * D.src.strides[0];
+        g.B = packed;
+        g.wei_zp = wz.set ? args->zps[QMM_WEI] : nullptr;
+        g.wei_zp_dt = wz.dt;
+        g.wei_zp_sn = wz.set && (wz.mask & 2) ? 1 : 0;
+        g.w_off = D.wei.dt == dt_u8 ? 128 : 0;
+        g.M = (int32_t)P.M;
+        g.N = (int32_t)P.N;
+        g.K = (int32_t)P.K;
+        g.batch = 1;
+        g.kb32 = (int32_t)geom.kb32;
+        g.nb32 = (int32_t)geom.nb32;
+        launch_gemm_f16w8(g, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;
         std::memset(&g, 0, sizeof(g));

@@ -300,10 +300,11 @@ struct quant_rows_params_t {
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
     impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales
-    impl_gemv_w4 = 2, // decode: 4-bit / 8-bit weights, 16-bit activations
-    impl_gemm_f16 = 3, // plain f16 / bf16 batched matmul
-    impl_generic = 4,
-    impl_count = 5
+    impl_gemm_f16w8 = 2, // f16 activations x 8-bit weights at many rows
+    impl_gemv_w4 = 3, // decode: 4-bit / 8-bit weights, 16-bit activations
+    impl_gemm_f16 = 4, // plain f16 / bf16 batched matmul
+    impl_generic = 5,
+    impl_count = 6
 };
 
 } // namespace qmm

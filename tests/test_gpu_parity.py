@@ -840,7 +840,8 @@ def test_decompression_at_many_rows(ctx, name):
     say("decode_w4 tiled %s" % name)
     kw = TILED_CASES[name]
     p = decode_w4(seed=70 + len(name), **kw)
-    got, pd = p.run_gpu(eng, strm, weights_any=True, return_pd=True)
+    # (asked for by name: f16 x 8-bit weights at 256 rows and more go to mfma_f16w8 first)
+    got, pd = p.run_gpu(eng, strm, weights_any=True, impl=DECODE, return_pd=True)
     assert pd.impl_info_str() == DECODE
     want = p.run_oracle()
     code = kw.get("dst_dt") or kw.get("act_dt", dt.bf16)
