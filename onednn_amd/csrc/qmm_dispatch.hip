@@ -33,7 +33,9 @@ void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream);
 void launch_rowsum_b8(const void *src, int32_t *dst, int64_t batch, int64_t M,
         int64_t K, int64_t lda, int64_t a_sb, bool a_is_u8, const void *src_zp,
         int src_zp_dt, hipStream_t stream);
-void launch_gemm_f16w8(const gemm_params_t &p, hipStream_t stream);
+void launch_gemm_f16w8(const gemm_params_t &p, int splits, float *part,
+        hipStream_t stream);
+int gemm_f16w8_splits(int64_t M, int64_t N, int64_t K);
 void launch_gemm_w4a8(const w4a8_params_t &p, int variant, hipStream_t stream);
 void launch_gemm_w4a8_small(const w4a8_small_t &p, bool has_zp,
         hipStream_t stream);
@@ -878,6 +880,13 @@ static size_t round256(size_t v) {
     return (v + 255) / 256 * 256;
 }
 
+// mfma_f16w8 with its K range cut into slices: the slices' f32 sums
+static size_t f16w8_part_bytes(const qmm_matmul_desc_t &D) {
+    const int64_t M = D.dst.dims[0], N = D.dst.dims[1], K = D.src.dims[1];
+    const int splits = gemm_f16w8_splits(M, N, K);
+    return splits > 1 ? (size_t)splits * M * round_up(N, 4) * 4 : 0;
+}
+
 size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
     const int nd = desc->wei.ndims;
     const int64_t K = desc->wei.dims[nd - 2], N = desc->wei.dims[nd - 1];
@@ -902,9 +911,12 @@ size_t qmm_matmul_scratch_size(int impl, const qmm_matmul_desc_t *desc) {
         // small-row kernel, so leave room for either
         return packed + (sm.use && sm.part_bytes > big ? sm.part_bytes : big);
     }
+    if (impl == impl_gemm_f16w8 && desc->wei_layout != QMM_LAYOUT_PLAIN)
+        return f16w8_part_bytes(*desc);
     if (desc->wei_layout != QMM_LAYOUT_PLAIN) return 0;
     if (impl == impl_gemm_f16w8)
-        return qmm_packed_size(QMM_LAYOUT_MFMA_B8, desc->wei.dt, 1, K, N);
+        return round256(qmm_packed_size(QMM_LAYOUT_MFMA_B8, desc->wei.dt, 1, K, N))
+                + f16w8_part_bytes(*desc);
     if (impl == impl_gemv_w4)
         return qmm_packed_size(is_int8(desc->wei.dt) ? QMM_LAYOUT_MFMA_W8
                                                      : QMM_LAYOUT_MFMA_W4,
@@ -1375,7 +1387,14 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.batch = 1;
         g.kb32 = (int32_t)geom.kb32;
         g.nb32 = (int32_t)geom.nb32;
-        launch_gemm_f16w8(g, stream);
+        // gemm_variant 1: never cut K into slices
+        const int splits
+                = gemm_variant == 1 ? 1 : gemm_f16w8_splits(P.M, P.N, P.K);
+        float *part = (float *)((uint8_t *)args->scratch
+                + (D.wei_layout == QMM_LAYOUT_PLAIN
+                                ? round256(geom.total_bytes)
+                                : 0));
+        launch_gemm_f16w8(g, splits, part, stream);
     } else if (impl == impl_gemv_w4) {
         gemv_params_t g;
         std::memset(&g, 0, sizeof(g));

@@ -295,6 +295,51 @@ void launch_f16w8_odd(const gemm_params_t &p, hipStream_t stream) {
 #if QMM_F16W8_PART == 0
 void launch_f16w8_odd(const gemm_params_t &p, hipStream_t stream);
 
+// Few block tiles, long K (1024 x 4096 dst over K 4096 ... 14336: 64 tiles on 256
+// CUs): the K range is cut into `splits` equal slices that run as the batch
+// dimension of one launch -- slice s reads the source from column s K/splits
+// and the packed weights from k block s K/splits / 32, and writes its f32 sums
+// to slice s of a scratch buffer -- and this kernel adds the slices in slice
+// order, then applies scales, bias, post-ops and the dst conversion: one
+// thread per four neighbouring columns of a row.
+// (S slices, a compile-time count: a thread's S loads are all in flight before
+// the first addition)
+template <int S>
+__global__ void __launch_bounds__(256)
+f16w8_reduce_kernel(const float *part, int M, int N, int ldp,
+        const epilogue_t ep) {
+    const int n4 = (N + 3) / 4;
+    const int64_t total = (int64_t)M * n4;
+    const bool has_ss = ep.src_scale.ptr != nullptr;
+    const bool has_ws = ep.wei_scale.ptr != nullptr;
+    const int64_t slice = (int64_t)M * ldp;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (int64_t)gridDim.x * blockDim.x) {
+        const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+        const float *q = part + (int64_t)m * ldp + n;
+        v4f t[S];
+#pragma unroll
+        for (int s = 0; s < S; s++)
+            t[s] = *(const v4f *)(q + s * slice);
+        float v[4] = {t[0].x, t[0].y, t[0].z, t[0].w};
+#pragma unroll
+        for (int s = 1; s < S; s++) {
+            v[0] += t[s].x;
+            v[1] += t[s].y;
+            v[2] += t[s].z;
+            v[3] += t[s].w;
+        }
+        const int nvalid = min(4, N - n);
+        ep_cols_t c;
+        epilogue_cols_load(ep, c, 0, n, nvalid);
+        const float ss = has_ss ? ep_load(ep.src_scale, 0, m, 0) : 1.f;
+        if (ep.fast != EP_FAST_NONE && !ep.fast_ext)
+            epilogue_fast4(ep, v, has_ss, ss, has_ws, c.ws, 0, m, n, nvalid);
+        else
+            epilogue_rows4(ep, c, v, has_ss, ss, 0, m, n, nvalid);
+    }
+}
+
 // Problems the kernel takes: K a multiple of 32 with at least 5 k-steps, source
 // rows of 16-byte granularity, tiles addressable with 32-bit offsets.
 bool gemm_f16w8_eligible(const gemm_params_t &p) {
@@ -304,11 +349,77 @@ bool gemm_f16w8_eligible(const gemm_params_t &p) {
     return true;
 }
 
-void launch_gemm_f16w8(const gemm_params_t &p, hipStream_t stream) {
+// How many K slices. Cost model in microseconds, fitted to measurements on
+// 1024 x K x 4096 and 512 x 4096 x 14336: a workgroup takes 0.6 per k-step plus
+// 10 for prologue and epilogue; slices add their f32 sums written (4 TB/s) and
+// read back by the second kernel (3 TB/s, plus 3 for its launch). Slices must
+// keep every workgroup in one round over the 256 CUs, divide the k-steps evenly
+// and have at least 16 of them; they are taken when the model promises a tenth
+// less time.
+int gemm_f16w8_splits(int64_t M, int64_t N, int64_t K) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const int64_t kt = K / 32;
+    if (tiles > 128) return 1;
+    const double one = 0.6 * (double)kt + 10.0;
+    double best_t = 0.9 * one;
+    int best = 1;
+    for (int s : {2, 3, 4, 6, 8}) {
+        if (kt % s != 0 || kt / s < 16 || tiles * s > 256) continue;
+        const double part = (double)s * (double)M * (double)N * 4.0;
+        const double t = 0.6 * (double)(kt / s) + 10.0 + part / 4e6 + 3.0
+                + (part + (double)M * (double)N * 4.0) / 3e6;
+        if (t < best_t) {
+            best_t = t;
+            best = s;
+        }
+    }
+    return best;
+}
+
+static void launch_one(const gemm_params_t &p, hipStream_t stream) {
     if ((p.K / 32) & 1)
         launch_f16w8_odd(p, stream);
     else
         launch_f16w8_even(p, stream);
+}
+
+// part: room for splits x M x round_up(N, 4) floats when splits > 1
+void launch_gemm_f16w8(const gemm_params_t &p, int splits, float *part,
+        hipStream_t stream) {
+    if (splits <= 1) {
+        launch_one(p, stream);
+        return;
+    }
+    const int ldp = (p.N + 3) / 4 * 4;
+    gemm_params_t q = p;
+    q.K = p.K / splits;
+    q.batch = splits;
+    q.a_sb = (int64_t)q.K * 2;
+    q.b_sb = (int64_t)(q.K / 32) * 1024;
+    std::memset(&q.ep, 0, sizeof(q.ep));
+    q.ep.dst.ptr = part;
+    q.ep.dst.dt = dt_f32;
+    q.ep.dst.sb = (int64_t)p.M * ldp;
+    q.ep.dst.sm = ldp;
+    q.ep.dst.sn = 1;
+    q.ep.fast = EP_FAST_PLAIN;
+    launch_one(q, stream);
+    const int64_t total = (int64_t)p.M * (ldp / 4);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+#define QH_REDUCE(S) \
+    case S: \
+        hipLaunchKernelGGL(f16w8_reduce_kernel<S>, dim3((unsigned)blocks), \
+                dim3(256), 0, stream, (const float *)part, p.M, p.N, ldp, p.ep); \
+        break;
+    switch (splits) {
+        QH_REDUCE(2)
+        QH_REDUCE(3)
+        QH_REDUCE(4)
+        QH_REDUCE(6)
+        default: QH_REDUCE(8)
+    }
+#undef QH_REDUCE
 }
 #endif
 

@@ -118,6 +118,12 @@ CASES = {
     # weights rows N-contiguous, source rows with a pitch, dst rows that start at odd elements
     "u8_ab_weights_pitched_source": dict(M=300, K=256, N=1001, wei_layout="ab", lda=264),
     "u8_gelu_f16": dict(M=270, K=256, N=272, post="gelu"),
+    # few tiles, long K: the K range runs as slices whose f32 sums a second kernel adds (8 slices for u8_k4096_f32
+    # above; here 3 of 16 k-steps, 2 of 17, 4 with a binary operand, 2 with odd dst rows)
+    "u8_k1536_three_slices_swish": dict(M=300, K=1536, N=520, post="swish"),
+    "s8_k1088_two_odd_slices": dict(M=256, K=1088, N=260, wei_dt=dt.s8, zp_dt=dt.s8, dst_dt=dt.f32),
+    "u8_k2048_four_slices_add": dict(M=512, K=2048, N=384, dst_dt=dt.f32, post="add"),
+    "u8_k1024_slices_gelu_odd_columns": dict(M=260, K=1024, N=1001, post="gelu", src_scale=0.5),
 }
 
 
@@ -153,6 +159,20 @@ def test_extreme_weights_and_zero_points_convert_exactly(ctx):
         g, r = got.view(np.float32).reshape(M, N), want.view(np.float32).reshape(M, N)
         # one product and one scale multiplication in either order: 2 f32 roundings at most
         assert np.all(np.abs(g - r) <= 2.0 ** -22 * np.abs(r)), "one-hot %s / %s" % (wei_dt, zp_dt)
+
+
+def test_slices_of_k_and_one_pass_agree(ctx, monkeypatch):
+    """QMM_GEMM_VARIANT=1 keeps K in one pass: same problem both ways, each against the oracle's bar."""
+    eng, strm = ctx
+    p = problem(256, 2048, 512, 11, dst_dt=dt.f32)
+    got_slices = p.run_gpu(eng, strm, weights_any=True)
+    monkeypatch.setenv("QMM_GEMM_VARIANT", "1")
+    got_one = p.run_gpu(eng, strm, weights_any=True)
+    want = p.run_oracle()
+    check(p, got_slices, want, "slices")
+    check(p, got_one, want, "one pass")
+    a, b = got_slices.view(np.float32), got_one.view(np.float32)
+    assert not np.array_equal(a, b), "the two paths sum in different orders: identical results mean one path ran twice"
 
 
 def test_fewer_than_256_rows_stay_with_the_decode_implementation(ctx):
