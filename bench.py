@@ -71,7 +71,8 @@ def build_c2(dnnl, dt, T, M=4096, K=4096, N=14336, seed=2):
 EXTRAS = {"decode_gemv": "bench_decode", "fp8_gemm": "bench_fp8", "int8_small": "bench_c1",
           "attention_scores": "bench_c4", "attention_chain": "bench_attention_chain", "attention_fused": "bench_attention_fused", "attention_decode": "bench_attention_decode", "int8_int4_grouped": "bench_w4a8", "quantize_reorder": "bench_quantize",
           "attention_products_f16": "bench_f16_products", "int8_decode_rows": "bench_int8_rows",
-          "mfma_ceiling": "bench_mfma_ceiling", "gemm_anatomy": "bench_gemm_anatomy"}
+          "mfma_ceiling": "bench_mfma_ceiling", "gemm_anatomy": "bench_gemm_anatomy",
+          "f16_u8_prefill": "bench_f16_u8_prefill"}
 
 
 def main():
@@ -668,6 +669,50 @@ def bench_int8_rows(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=100, K=40
                                          "algorithmic_bytes": nbytes, "GBps_from_cache": round(nbytes / (ms * 1e-3) / 1e9, 1),
                                          "impl": pd.impl_info_str()}
     out["note"] = "back-to-back launches on one stream, one weight set (resident in the last-level cache)"
+    return out
+
+
+PEAK_F16 = 2500.0  # TFLOP/s, dense MFMA f16
+
+
+def bench_f16_u8_prefill(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
+    """Prefill of the 8-bit weights-only layers of the reference's LLM list (tests/benchdnn/inputs/matmul/
+    option_set_fwks_llm_gpu: --dt=f16:u8:f16|f32 --attr-scales=wei:per_oc:f16 --attr-zero-points=wei:per_oc:u8
+    --attr-fpmath=f16:true): f16 activations, u8 weights prepacked through format_tag any, one scale and one zero point
+    per column. Bound: the f16 matrix cores (the weights are converted in registers between the MFMAs)."""
+    out = {}
+    r = np.random.default_rng(13)
+    for (M, K, N, dst, swish) in ((2176, 4096, 14336, dt.f16, True), (1024, 4096, 14336, dt.f16, False),
+                                  (1024, 4096, 4096, dt.f16, False), (1024, 11008, 4096, dt.f32, False),
+                                  (2048, 4096, 128256, dt.f32, False)):
+        attr = A.primitive_attr()
+        attr.set_fpmath_mode(A.fpmath_mode.f16, True)
+        attr.set_scales(A.DNNL_ARG_WEIGHTS, 2, [], dt.f16)
+        attr.set_zero_points(A.DNNL_ARG_WEIGHTS, 2, [], dt.u8)
+        if swish:
+            po = A.post_ops()
+            po.append_eltwise(A.algorithm.eltwise_swish, 1.0, 0.0)
+            attr.set_post_ops(po)
+        pd = A.matmul.primitive_desc(eng, memory.desc([M, K], dt.f16, T("ab")), memory.desc([K, N], dt.u8, tag.any),
+                                     memory.desc([M, N], dst, T("ab")), attr=attr)
+        prim = A.matmul(pd)
+        m_wei = memory(pd.weights_desc(), eng)
+        plain = memory(memory.desc([K, N], dt.u8, T("ba")), eng).write(r.integers(0, 256, K * N, dtype=np.uint8))
+        A.reorder(plain, m_wei).execute(strm, plain, m_wei)
+        strm.wait()
+        del plain
+        ex = {A.DNNL_ARG_SRC: memory(pd.src_desc(), eng).write(r.standard_normal((M, K)).astype(np.float16).view(np.uint16)),
+              A.DNNL_ARG_WEIGHTS: m_wei, A.DNNL_ARG_DST: memory(pd.dst_desc(), eng),
+              A.DNNL_ARG_ATTR_SCALES | A.DNNL_ARG_WEIGHTS: memory(memory.desc([N], dt.f16, T("a")), eng).write(
+                  r.uniform(0.0005, 0.002, N).astype(np.float16).view(np.uint16)),
+              A.DNNL_ARG_ATTR_ZERO_POINTS | A.DNNL_ARG_WEIGHTS: memory(memory.desc([N], dt.u8, T("a")), eng).write(
+                  r.integers(100, 156, N).astype(np.uint8))}
+        ms = _time(prim, strm, hs, hiprt, ex, steps, warm=5)
+        tf = 2.0 * M * K * N / (ms * 1e-3) / 1e12
+        out["%dx%dx%d_%s%s" % (M, K, N, "f16" if dst == dt.f16 else "f32", "_swish" if swish else "")] = {
+            "us_per_launch": round(ms * 1e3, 1), "TFLOPs": round(tf, 1), "frac_of_f16_peak": round(tf / PEAK_F16, 4),
+            "impl": pd.impl_info_str()}
+    out["note"] = "back-to-back launches on one stream; peak = 2.5 PFLOP/s dense f16"
     return out
 
 
