@@ -258,7 +258,8 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  *   QMM_GEMM_VARIANT: 0 by problem size (default); 1..3 a tile configuration of
  *     the general mfma_b8 kernel; 6 the 256 x 256 kernels wherever eligible;
  *     for mfma_f16 plans 1 = 64 x 64 tiles, 2 = 128 x 128 tiles, 3 = 128-row
- *     workgroups that walk the column tiles (short K)
+ *     workgroups that walk the column tiles (short K); for mfma_f16w8 plans
+ *     1 = K in one pass (no slices with a second, reducing kernel)
  *   QMM_W4A8_VARIANT: 0 by problem size (default); 1..3 a tile configuration;
  *     4 as 0 but with the split-K kernel instead of the one-launch kernel at
  *     5 .. 64 rows, 5 as 0 but with the one-launch kernel wherever it applies
