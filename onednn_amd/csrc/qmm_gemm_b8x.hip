@@ -29,6 +29,7 @@
 // arithmetic as src/cpu/matmul/ref_matmul_int8.cpp:195-259); only epilogues of
 // the straight-line kinds (EP_FAST_*) are handled here, everything else stays
 // with the general kernel.
+#include <algorithm>
 #include <cstring>
 #include <type_traits>
 
@@ -63,7 +64,7 @@ static __device__ unsigned long long g_gemm_stamps[STAMP_TILES * STAMP_SLOTS * 2
 // is staged and 5 after the first half's rows are stored
 #define QX_STAMP_IF(first, slot) \
     if ((p.switches & GEMM_STAMPS) && (first)) { \
-        const unsigned t = (blockIdx.x + gridDim.x * blockIdx.y) % STAMP_TILES; \
+        const unsigned t = (qx_stamp_id + gridDim.x * blockIdx.y) % STAMP_TILES; \
         g_gemm_stamps[(t * STAMP_SLOTS + (slot)) * 2] = clock64(); \
         g_gemm_stamps[(t * STAMP_SLOTS + (slot)) * 2 + 1] = wall_clock64(); \
     }
@@ -386,7 +387,7 @@ template <bool F8, bool LEAN, typename AccT, int NFI, int NFJ,
         int TABS = b8x::SS_OFF, bool NARROW = false>
 QMM_D void tile_epilogue(const gemm_params_t &p, AccT (&acc)[NFI][NFJ],
         uint8_t *lds, uint32_t lds_base, int wave, int lane, int m0, int n0,
-        int wm0, int wn0, int bz) {
+        int wm0, int wn0, int bz, [[maybe_unused]] unsigned qx_stamp_id = 0) {
     using namespace b8x;
     constexpr bool MI16 = NFI == 8;
     constexpr int WN = MI16 ? 16 * NFJ : 128; // columns of the wave tile
@@ -890,43 +891,22 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QY_ROW(6, CB, , , , ) QY_ROW(7, CB, , , , )
 
 #if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5)
+// One block tile of gemm_b8y_kernel.
 // ODD: an odd number of k-steps (the register buffers alternate per k-step, so
 // the two parities end on different buffers; one instantiation each keeps the
 // tail single and the accumulators out of scratch). A 224-column block tile
 // (wave tiles of 128 x 112, four equal rounds of workgroups on a 4096 x 14336
 // dst instead of three and a half) was measured at 0.6 % and is not kept.
 template <bool ODD>
-__global__ void __launch_bounds__(b8x::NT, 1)
-gemm_b8y_kernel(const gemm_params_t p) {
+QMM_D void gemm_b8y_tile(const gemm_params_t &p, uint8_t *lds,
+        const uint32_t lds_base, const int tid, const int lane, const int wave,
+        const int m0, const int n0, const int bz,
+        [[maybe_unused]] const unsigned qx_stamp_id) {
     using namespace b8x;
-    constexpr int NFJ = 8, BNY = BN;
-    typedef __attribute__((address_space(3))) uint8_t lds_u8;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int NFJ = 8;
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * (16 * NFJ);
 
-    const int ntiles = p.tiles_m * p.tiles_n;
-    int lt;
-    {
-        const int per = (ntiles + 7) / 8;
-        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-        lt = xcd * per + slot;
-        if (slot >= per || lt >= ntiles) return;
-    }
-    constexpr int GROUP_M = 8;
-    const int group = lt / (GROUP_M * p.tiles_n);
-    const int first_m = group * GROUP_M;
-    const int gsz = min(p.tiles_m - first_m, GROUP_M);
-    const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
-    const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
-    const int m0 = tile_m * BM, n0 = tile_n * BNY;
-    const int bz = blockIdx.y;
-
     const int KT = p.K / BK; // host guarantees K % 64 == 0, KT >= 5 and KT % 2 == ODD
-    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(lds_u8 *)lds);
     if constexpr (!ODD) { QX_STAMP(0) }
 
     uint32_t a_vo[4], b_vo[4];
@@ -1031,9 +1011,46 @@ gemm_b8y_kernel(const gemm_params_t p) {
         QX_SKIP_EPILOGUE(8, NFJ, 4)
     }
 
-    tile_epilogue<false, false>(
-            p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    tile_epilogue<false, false>(p, acc, lds, lds_base, wave, lane, m0, n0, wm0,
+            wn0, bz, qx_stamp_id);
     if constexpr (!ODD) { QX_STAMP(3) }
+}
+
+// Persistent: the grid is 8 x W workgroups, W per XCD (one per CU: the LDS ring
+// leaves no room for a second), and workgroup w of an XCD takes the tiles
+// w, w + W, ... of the XCD's share in turn: a tile starts when its predecessor
+// on the CU has stored its last row, without a trip through the dispatcher.
+template <bool ODD>
+__global__ void __launch_bounds__(b8x::NT, 1)
+gemm_b8y_kernel(const gemm_params_t p) {
+    using namespace b8x;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    const int bz = blockIdx.y;
+
+    const int ntiles = p.tiles_m * p.tiles_n;
+    const int per = (ntiles + 7) / 8;
+    const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
+    for (int slot = blockIdx.x >> 3, it = 0; slot < per; slot += W, it++) {
+        const int lt = xcd * per + slot;
+        if (lt >= ntiles) break;
+        constexpr int GROUP_M = 8;
+        const int group = lt / (GROUP_M * p.tiles_n);
+        const int first_m = group * GROUP_M;
+        const int gsz = min(p.tiles_m - first_m, GROUP_M);
+        const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
+        const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
+        gemm_b8y_tile<ODD>(p, lds, lds_base, tid, lane, wave, tile_m * BM,
+                tile_n * BN, bz, it * gridDim.x + blockIdx.x);
+        // the staging area and the operand tables are the next tile's ring
+        // and tables
+        __syncthreads();
+    }
 }
 #endif // int8, 16 x 16 x 64
 
@@ -1813,6 +1830,38 @@ static void launch_b8x(K kern, const gemm_params_t &p, hipStream_t stream) {
             stream, q);
 }
 
+// The persistent kernel: W workgroups per XCD, one per CU (fewer when an XCD's
+// share of the tiles is smaller). GEMM_NOT_PERSISTENT: one workgroup per tile.
+static int cus_per_xcd() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess
+                || hipDeviceGetAttribute(
+                           &cus, hipDeviceAttributeMultiprocessorCount, dev)
+                        != hipSuccess
+                || cus < 8)
+            cus = 256;
+        n = cus / 8;
+    }
+    return n;
+}
+template <typename K>
+static void launch_b8y_persistent(
+        K kern, const gemm_params_t &p, hipStream_t stream) {
+    using namespace b8x;
+    gemm_params_t q = p;
+    q.tiles_m = (p.M + BM - 1) / BM;
+    q.tiles_n = (p.N + BN - 1) / BN;
+    const int per = (q.tiles_m * q.tiles_n + 7) / 8;
+    const int W = (p.switches & GEMM_NOT_PERSISTENT)
+            ? per
+            : std::min(cus_per_xcd(), per);
+    ensure_dynamic_lds((const void *)kern, LDS_TOTAL);
+    hipLaunchKernelGGL(
+            kern, dim3(8 * W, p.batch), dim3(NT), LDS_TOTAL, stream, q);
+}
+
 // One kernel per translation unit (QMM_B8X_PART), so that they build in
 // parallel; the unit without the macro holds the dispatcher.
 #if defined(QMM_B8X_PART)
@@ -1830,7 +1879,7 @@ void launch_b8x_fp8(const gemm_params_t &p, hipStream_t stream) {
 }
 #elif QMM_B8X_PART == 4
 void launch_b8x_int8_mi16(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_b8y_kernel<false>, p, stream);
+    launch_b8y_persistent(gemm_b8y_kernel<false>, p, stream);
 }
 int gemm_stamps_read_int8(void *host, size_t bytes) {
     // through pinned memory, as every other copy of the library to the host
@@ -1846,7 +1895,7 @@ int gemm_stamps_read_int8(void *host, size_t bytes) {
 }
 #elif QMM_B8X_PART == 5
 void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_b8y_kernel<true>, p, stream);
+    launch_b8y_persistent(gemm_b8y_kernel<true>, p, stream);
 }
 #elif QMM_B8X_PART == 6
 void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream) {

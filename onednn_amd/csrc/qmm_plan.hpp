@@ -146,7 +146,10 @@ enum {
     GEMM_SKIP_EPILOGUE = 2,
     GEMM_STAMPS = 4,
     GEMM_TWO_PER_CU = 8,
-    GEMM_ONE_PER_CU = 16
+    GEMM_ONE_PER_CU = 16,
+    // the int8 256 x 256 kernel on 16 x 16 MFMAs: one workgroup per tile
+    // instead of one per CU walking its tiles (a measurement switch)
+    GEMM_NOT_PERSISTENT = 32
 };
 
 struct gemm_params_t {
