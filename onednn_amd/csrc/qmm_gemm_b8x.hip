@@ -1697,15 +1697,19 @@ gemm_f8y_kernel(const gemm_params_t p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(lds_u8 *)lds);
+    const int bz = blockIdx.y;
+    const int KS = p.K / 128; // host guarantees K % 256 == 0 and KS >= 4
 
+    // persistent, as gemm_b8y_kernel: workgroup w of an XCD walks the tiles
+    // w, w + W, ... of the XCD's share
     const int ntiles = p.tiles_m * p.tiles_n;
-    int lt;
-    {
-        const int per = (ntiles + 7) / 8;
-        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-        lt = xcd * per + slot;
-        if (slot >= per || lt >= ntiles) return;
-    }
+    const int per = (ntiles + 7) / 8;
+    const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
+    for (int slot = blockIdx.x >> 3; slot < per; slot += W) {
+    const int lt = xcd * per + slot;
+    if (lt >= ntiles) break;
     constexpr int GROUP_M = 8;
     const int group = lt / (GROUP_M * p.tiles_n);
     const int first_m = group * GROUP_M;
@@ -1713,11 +1717,6 @@ gemm_f8y_kernel(const gemm_params_t p) {
     const int tile_m = first_m + (lt % (GROUP_M * p.tiles_n)) % gsz;
     const int tile_n = (lt % (GROUP_M * p.tiles_n)) / gsz;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int bz = blockIdx.y;
-
-    const int KS = p.K / 128; // host guarantees K % 256 == 0 and KS >= 4
-    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(lds_u8 *)lds);
 
     uint32_t a_vo[4], b_vo[4];
 #pragma unroll
@@ -1813,6 +1812,10 @@ gemm_f8y_kernel(const gemm_params_t p) {
 
     tile_epilogue<true, true>(
             p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    // the staging area and the operand tables are the next tile's ring and
+    // tables
+    __syncthreads();
+    } // tiles of this workgroup
 }
 #endif // fp8, 16 x 16 x 128
 
@@ -1899,7 +1902,7 @@ void launch_b8x_int8_mi16_odd(const gemm_params_t &p, hipStream_t stream) {
 }
 #elif QMM_B8X_PART == 6
 void launch_b8x_fp8_mi16(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_f8y_kernel, p, stream);
+    launch_b8y_persistent(gemm_f8y_kernel, p, stream);
 }
 
 #endif
