@@ -781,7 +781,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
 }
 
 // the splits' states of one (head, query) -> dst. The weights of the splits
-// are formed once in LDS; a thread then owns one d and adds the splits'
+// are formed once in LDS; a thread then owns one d (two of 256) and adds the splits'
 // accumulators with independent loads.
 constexpr int SDPA_MAX_SPLIT = 256;
 __global__ void __launch_bounds__(128)
@@ -815,12 +815,12 @@ sdpa_combine_kernel(const sdpa_params_t p, const int D) {
     if ((t & 63) == 0) red[t >> 6] = l_part;
     __syncthreads();
     const float l_all = red[0] + red[1];
-    if (t < D) {
+    for (int d = t; d < D; d += 128) { // head sizes up to 256: two per thread
         float o = 0.f;
 #pragma unroll 8
         for (int s1 = 0; s1 < p.nsplit; s1++)
-            o += w_s[s1] * st[(int64_t)s1 * 16 * ST + t];
-        p.dst[b0 * p.o.b0 + b1 * p.o.b1 + (int64_t)q * p.o.row + t]
+            o += w_s[s1] * st[(int64_t)s1 * 16 * ST + d];
+        p.dst[b0 * p.o.b0 + b1 * p.o.b1 + (int64_t)q * p.o.row + d]
                 = p.bf ? f32_to_bf16(o / l_all)
                        : __builtin_bit_cast(uint16_t, (_Float16)(o / l_all));
     }
@@ -886,7 +886,10 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
     if (d.v.dims[nd - 1] != D) return false; // head size of V = head size of Q
     if (d.dst.dims[nd - 2] != Qn || d.dst.dims[nd - 1] != D) return false;
-    if (D != 64 && D != 128) return false;
+    // head sizes: 64 and 128 in every form; 32 and 256 with K / V in the
+    // queries' type (the 8-bit cache paths are instantiated for 64 and 128)
+    if (D != 64 && D != 128 && !((D == 32 || D == 256) && d.k.dt == d.q.dt))
+        return false;
     if (Qn < 1 || S < 1 || Qn > (1 << 30) || S > (1 << 30)) return false;
     // innermost-contiguous rows: Q [q][d], K as the transposed view of a
     // [keys][d] cache, V [keys][d], dst [q][d]
@@ -1044,7 +1047,8 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.k_zp = desc->k_zp.set ? args->k_zp : nullptr;
     p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
-    const bool d128 = desc->q.dims[desc->q.ndims - 1] == 128;
+    const int D = (int)desc->q.dims[desc->q.ndims - 1];
+    const bool d128 = D == 128;
     const bool qn = p.kv_dt != desc->q.dt, mk = p.mask != nullptr;
     const bool bf = p.bf != 0; // never together with qn
     if (p.Qn <= 16) {
@@ -1059,6 +1063,20 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
             hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
                     (hipStream_t)hip_stream, p);
         };
+        if (D == 32 || D == 256) {
+            // K / V in the queries' type only (supported())
+            switch ((D == 256 ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+                case 0: god(sdpa_decode_kernel<1, false, false, false>); break;
+                case 1: god(sdpa_decode_kernel<1, false, true, false>); break;
+                case 2: god(sdpa_decode_kernel<1, false, false, true>); break;
+                case 3: god(sdpa_decode_kernel<1, false, true, true>); break;
+                case 4: god(sdpa_decode_kernel<8, false, false, false>); break;
+                case 5: god(sdpa_decode_kernel<8, false, true, false>); break;
+                case 6: god(sdpa_decode_kernel<8, false, false, true>); break;
+                case 7: god(sdpa_decode_kernel<8, false, true, true>); break;
+                default: return QMM_UNIMPLEMENTED;
+            }
+        } else
         switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
             case 0: god(sdpa_decode_kernel<2, false, false, false>); break;
             case 1: god(sdpa_decode_kernel<2, false, true, false>); break;
@@ -1077,7 +1095,7 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         if (p.nsplit > 1)
             hipLaunchKernelGGL(sdpa_combine_kernel,
                     dim3((unsigned)(p.B0 * p.B1), (unsigned)p.Qn), dim3(128), 0,
-                    (hipStream_t)hip_stream, p, d128 ? 128 : 64);
+                    (hipStream_t)hip_stream, p, D);
         return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
     }
     const dim3 grid((unsigned)(p.B0 * p.B1),
@@ -1100,6 +1118,19 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);
     };
+    if (D == 32 || D == 256) {
+        switch ((D == 256 ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+            case 0: go(sdpa_f16_kernel<1, false, false, false>); break;
+            case 1: go(sdpa_f16_kernel<1, false, true, false>); break;
+            case 2: go(sdpa_f16_kernel<1, false, false, true>); break;
+            case 3: go(sdpa_f16_kernel<1, false, true, true>); break;
+            case 4: go(sdpa_f16_kernel<8, false, false, false>); break;
+            case 5: go(sdpa_f16_kernel<8, false, true, false>); break;
+            case 6: go(sdpa_f16_kernel<8, false, false, true>); break;
+            case 7: go(sdpa_f16_kernel<8, false, true, true>); break;
+            default: return QMM_UNIMPLEMENTED;
+        }
+    } else
     switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
         case 0: go(sdpa_f16_kernel<2, false, false, false>); break;
         case 1: go(sdpa_f16_kernel<2, false, true, false>); break;

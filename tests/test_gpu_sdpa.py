@@ -113,6 +113,14 @@ CASES = [
     ((4,), 0, 128, 128, 64, "causal", "none"),
     ((), 0, 77, 1000, 128, "2d", "mul"),
     ((1, 2), 0, 16, 33, 64, "none", "mul"),
+    # head sizes 32 and 256 (K / V in the queries' type): many queries, the few-queries form split over the keys, masks
+    ((1, 4), 0, 150, 200, 32, "2d", "mul"),
+    ((2, 2), 0, 8, 300, 32, "causal", "mul"),
+    ((3,), 0, 1, 1000, 32, "1d", "div"),
+    ((1, 2), 0, 130, 170, 256, "causal", "div"),
+    ((1, 3), 0, 1, 513, 256, "1d", "mul"),
+    ((1, 4), 2, 16, 700, 256, "none", "mul"),
+    ((2,), 0, 70, 96, 256, "2d", "none"),
 ]
 
 
@@ -303,6 +311,8 @@ def test_what_the_kernel_does_not_take_is_unimplemented(ctx):
 
     make()
     for bad in (dict(q=md([1, 2, 16, 96]), k=md([1, 2, 96, 32], t="abdc"), v=md([1, 2, 32, 96]), o=md([1, 2, 16, 96])),  # head size
+                dict(q=md([1, 2, 16, 32]), k=md([1, 2, 32, 32], dt.s8, t="abdc"), v=md([1, 2, 32, 32], dt.s8),
+                     o=md([1, 2, 16, 32])),                                    # an 8-bit cache at head size 32
                 dict(k=md([1, 2, 64, 32])),                                    # keys contiguous instead of head size
                 dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16)),  # bf16 queries on f16 keys
                 dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16),  # bf16 on an 8-bit cache
