@@ -276,7 +276,8 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
     copies are cycled; the launches are replayed from a HIP graph so that the
     host does not pace them. After config 3's own shape: the same layer with 8-bit weights, and the decode shape of
     the reference's LLM list (4096 x 14336, f16 and bf16 activations, 29 MB of weights per launch), where the launch
-    is long enough for bandwidth rather than launch latency to show."""
+    is long enough for bandwidth rather than launch latency to show, and the list's output projection over 128256
+    columns (525 MB of 8-bit weights), where nothing but bandwidth is left."""
     import oracle as O
     G = 128
     r = np.random.default_rng(3)
@@ -304,6 +305,9 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
     for act16 in (True, False):
         for m in (1, 16):
             cases.append(("N14336_%s_M%d" % ("f16" if act16 else "bf16", m), m, 4096, 14336, act16, False, 20))
+    # the output projection of the list's decode step (--dt=f16:u8:f32 1x4096:4096x128256, one f16 scale and u8 zero
+    # point per column): 525 MB of weights per launch, two sets alternating (one set is twice the last-level cache)
+    cases.append(("lm_head_f16_u8_M1", 1, 4096, 128256, True, True, 2))
     for key, M, Kx, Nx, act16, w8, nsets in cases:
         w, sc, zp = weights(Kx, Nx, w8)
         attr = A.primitive_attr()
