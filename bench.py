@@ -308,6 +308,10 @@ def bench_decode(A, memory, dt, tag, T, eng, strm, hs, hiprt, sets=64, reps=20, 
     # the output projection of the list's decode step (--dt=f16:u8:f32 1x4096:4096x128256, one f16 scale and u8 zero
     # point per column): 525 MB of weights per launch, two sets alternating (one set is twice the last-level cache)
     cases.append(("lm_head_f16_u8_M1", 1, 4096, 128256, True, True, 2))
+    # config 3's own format (bf16 x u4, groups of 128) at that width: 262 MB of weights and 12 MB of scales and zero
+    # points per launch, three sets in turn
+    cases.append(("lm_head_bf16_u4_M1", 1, 4096, 128256, False, False, 3))
+    cases.append(("lm_head_bf16_u4_M16", 16, 4096, 128256, False, False, 3))
     for key, M, Kx, Nx, act16, w8, nsets in cases:
         w, sc, zp = weights(Kx, Nx, w8)
         attr = A.primitive_attr()
