@@ -1046,15 +1046,17 @@ def bench_w4a8(A, memory, dt, tag, T, eng, strm, hs, hiprt):
 
 def bench_quantize(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20):
     """The reorder as a quantizer on the tensors of config 2: its weights f32 [4096,14336] -> s8 with per-column
-    scales (once per model), its activations bf16 [4096,4096] -> s8 with per-row scales (every step). A stream:
-    bytes read + written against HBM bandwidth."""
+    scales (once per model), its activations bf16 [4096,4096] -> s8 with per-row scales (every step), and the weights
+    again from their [N, K] storage (the transposing kernel). A stream: bytes read + written against HBM bandwidth."""
     r = np.random.default_rng(8)
     res = {}
-    for name, sdt, dims, mask, nsc in (("weights_f32_s8_per_column", dt.f32, [4096, 14336], 2, 14336),
-                                       ("activations_bf16_s8_per_row", dt.bf16, [4096, 4096], 1, 4096)):
+    for name, sdt, dims, mask, nsc, stag in (("weights_f32_s8_per_column", dt.f32, [4096, 14336], 2, 14336, "ab"),
+                                             ("activations_bf16_s8_per_row", dt.bf16, [4096, 4096], 1, 4096, "ab"),
+                                             # the same weights as a framework keeps them, [N, K]: a transposing pass
+                                             ("weights_f32_stored_n_k_s8_per_column", dt.f32, [4096, 14336], 2, 14336, "ba")):
         attr = A.primitive_attr()
         attr.set_scales_mask(A.DNNL_ARG_DST, mask)
-        s_md, d_md = memory.desc(dims, sdt, T("ab")), memory.desc(dims, dt.s8, T("ab"))
+        s_md, d_md = memory.desc(dims, sdt, T(stag)), memory.desc(dims, dt.s8, T("ab"))
         pd = A.reorder.primitive_desc(eng, s_md, eng, d_md, attr=attr)
         prim = A.reorder(pd)
         n = dims[0] * dims[1]

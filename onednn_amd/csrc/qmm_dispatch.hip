@@ -27,6 +27,7 @@ void launch_gemm_b8(const gemm_params_t &p, bool f8, int variant,
         hipStream_t stream);
 bool launch_gemv_w4(const gemv_params_t &p, hipStream_t stream);
 void launch_quantize_rows(const quant_rows_params_t &p, hipStream_t stream);
+void launch_quantize_transpose(const quant_tr_params_t &p, hipStream_t stream);
 void launch_w4a8_prep(const w4a8_prep_t &p, hipStream_t stream);
 void launch_gemv_b8(const gemm_params_t &p, hipStream_t stream);
 void launch_gemm_f16(const gemm16_params_t &p, hipStream_t stream);
@@ -1597,13 +1598,58 @@ static bool reorder_rows_plan(const qmm_reorder_desc_t *d,
     return true;
 }
 
+// The transposing quantizer (quantize_transpose_kernel): 2-D, a floating-point
+// source, one side with stride 1 over rows and the other over columns, the
+// quantization attributes of the row-wise pass; a 4-bit destination only where
+// its pairs along the stride-1 dim are whole and start on a byte.
+static bool reorder_transpose_plan(const qmm_reorder_desc_t *d,
+        quant_tr_params_t &p) {
+    std::memset(&p, 0, sizeof(p));
+    if (d->src_layout != QMM_LAYOUT_PLAIN || d->dst_layout != QMM_LAYOUT_PLAIN
+            || d->src.ndims != 2)
+        return false;
+    if (!one_of(d->src.dt, {dt_f32, dt_bf16, dt_f16})) return false;
+    if (!one_of(d->dst.dt, {dt_f32, dt_bf16, dt_f16, dt_s8, dt_u8, dt_s4,
+                dt_u4, dt_f8_e4m3, dt_f8_e5m2}))
+        return false;
+    const int64_t R = d->src.dims[0], C = d->src.dims[1];
+    if (R < 2 || C < 2 || R >= (int64_t(1) << 31) || C >= (int64_t(1) << 31))
+        return false;
+    const int64_t *ss = d->src.strides, *ds = d->dst.strides;
+    const bool src_cm = ss[0] == 1 && ss[1] >= R, src_rm = ss[1] == 1 && ss[0] >= C;
+    const bool dst_cm = ds[0] == 1 && ds[1] >= R, dst_rm = ds[1] == 1 && ds[0] >= C;
+    if (!((src_cm && !src_rm && dst_rm && !dst_cm)
+                || (src_rm && !src_cm && dst_cm && !dst_rm)))
+        return false;
+    if (d->dst.dt == dt_s4 || d->dst.dt == dt_u4) {
+        const int64_t pitch = dst_cm ? ds[1] : ds[0], run = dst_cm ? R : C;
+        if (pitch % 2 || run % 2) return false;
+    }
+    // tiles along the destination's stride-1 dim are the grid's y
+    if ((dst_cm ? R : C) > (int64_t)65535 * 128) return false;
+    if (!rows_quant(p.src_scale, d->src_scale, 2, d->src.dims)
+            || !rows_quant(p.dst_scale, d->dst_scale, 2, d->src.dims)
+            || !rows_quant(p.src_zp, d->src_zp, 2, d->src.dims))
+        return false;
+    if (d->dst_zp.set && d->dst_zp.mask != 0) return false;
+    p.rows = R;
+    p.cols = C;
+    p.src_sr = ss[0], p.src_sc = ss[1];
+    p.dst_sr = ds[0], p.dst_sc = ds[1];
+    p.src_dt = d->src.dt;
+    p.dst_dt = d->dst.dt;
+    return true;
+}
+
 const char *qmm_reorder_impl_name(const qmm_reorder_desc_t *d) {
     if (!d) return "";
     if (d->src_layout != QMM_LAYOUT_PLAIN || d->dst_layout != QMM_LAYOUT_PLAIN)
         return "hip:gfx950:prepack";
     quant_rows_params_t p;
-    return reorder_rows_plan(d, p) ? "hip:gfx950:quantize"
-                                   : "hip:gfx950:reorder";
+    quant_tr_params_t t;
+    return reorder_rows_plan(d, p)       ? "hip:gfx950:quantize"
+            : reorder_transpose_plan(d, t) ? "hip:gfx950:quantize_transpose"
+                                           : "hip:gfx950:reorder";
 }
 
 int qmm_reorder_launch(const qmm_reorder_desc_t *d,
@@ -1639,6 +1685,19 @@ int qmm_reorder_launch(const qmm_reorder_desc_t *d,
         qr.src_zp.ptr = d->src_zp.set ? args->src_zp : nullptr;
         qr.dst_zp = d->dst_zp.set ? (const int32_t *)args->dst_zp : nullptr;
         launch_quantize_rows(qr, stream);
+    } else if (quant_tr_params_t qt; reorder_transpose_plan(d, qt)) {
+        if ((d->src_scale.set && !args->src_scale)
+                || (d->dst_scale.set && !args->dst_scale)
+                || (d->src_zp.set && !args->src_zp)
+                || (d->dst_zp.set && !args->dst_zp))
+            return fail(QMM_INVALID_ARGUMENTS, "reorder attribute buffer missing");
+        qt.src = args->src;
+        qt.dst = args->dst;
+        qt.src_scale.ptr = d->src_scale.set ? args->src_scale : nullptr;
+        qt.dst_scale.ptr = d->dst_scale.set ? args->dst_scale : nullptr;
+        qt.src_zp.ptr = d->src_zp.set ? args->src_zp : nullptr;
+        qt.dst_zp = d->dst_zp.set ? (const int32_t *)args->dst_zp : nullptr;
+        launch_quantize_transpose(qt, stream);
     } else if (d->src_layout == QMM_LAYOUT_PLAIN
             && d->dst_layout == QMM_LAYOUT_PLAIN) {
         generic_reorder_params_t P;

@@ -300,6 +300,19 @@ struct quant_rows_params_t {
     int32_t col_groups, pad_; // set by the launcher
 };
 
+// ---- the same over a 2-D tensor whose two sides disagree on the dim order ----
+struct quant_tr_params_t {
+    const void *src;
+    void *dst;
+    int64_t rows, cols;
+    // element strides over (row, col): on each side one of them is 1, and not
+    // the same one on both
+    int64_t src_sr, src_sc, dst_sr, dst_sc;
+    int32_t src_dt, dst_dt;
+    quant_rows_q_t src_scale, dst_scale, src_zp;
+    const int32_t *dst_zp; // single value or nullptr
+};
+
 enum impl_id_t : int {
     impl_gemm_b8 = 0, // int8 / fp8 MFMA GEMM
     impl_gemm_w4a8 = 1, // s8 x int4 MFMA GEMM with K-grouped scales

@@ -6,9 +6,11 @@
 // elements of a row (32 or 16 bytes in, 4 to 32 bytes out) for 8 rows in turn,
 // so that per-column scales are fetched and inverted once. The arithmetic is the reference's, in its order:
 //     d = src_scale * (in - src_zp);  d = d * (1 / dst_scale) + dst_zp;
-// followed by the saturating / rounding store of the dst type. Everything else
-// (transposing reorders, scales over leading dims of tensors with more than
-// two dims) stays with the per-element kernel in qmm_generic.hip.
+// followed by the saturating / rounding store of the dst type. 2-D tensors
+// whose sides disagree on the dim order go through quantize_transpose_kernel
+// (a tile through LDS); everything else (scales over leading dims of tensors
+// with more than two dims, permutations of more dims) stays with the
+// per-element kernel in qmm_generic.hip.
 #include "qmm_device.hpp"
 #include "qmm_plan.hpp"
 
@@ -336,6 +338,144 @@ quantize8_cols_kernel(const quant_rows_params_t p) {
         *(uint2 *)((uint8_t *)p.dst + (row0 + r) * p.dst_pitch + col)
                 = make_uint2(o[0], o[1]);
     }
+}
+
+// The quantizer over a 2-D tensor that changes its dim order on the way (a
+// row-major f32 / bf16 / f16 source into a column-major quantized tensor or the
+// other way round: weights stored [N, K] quantized into [K, N], say). A
+// workgroup owns a tile: it reads along the source's stride-1 dim into LDS
+// (odd pitch: the transposed read-back is free of bank conflicts), then does
+// the arithmetic of quantize_rows_kernel per element (scales and zero points
+// addressed by the element's row and column, so every mask and group shape of
+// the row kernel is taken) and stores along the destination's stride-1 dim,
+// two neighbouring elements per thread (a 4-bit pair is one byte).
+// QT_FAST x QT_SLOW: the tile's extent along the destination's stride-1 dim
+// (128 elements: a whole 128-byte line of an 8-bit destination per row piece)
+// and along the source's (64 elements: 256 bytes of an f32 source)
+constexpr int QT_FAST = 128, QT_SLOW = 64;
+__global__ void __launch_bounds__(256)
+quantize_transpose_kernel(const quant_tr_params_t p) {
+    __shared__ float tile[QT_SLOW][QT_FAST + 1]; // [slow][fast] of the destination
+    const int tid = threadIdx.x;
+    const bool dst_col_major = p.dst_sr == 1; // else stride 1 over columns
+    // origin of the tile: blockIdx.x walks the SOURCE's stride-1 dim, so that
+    // the workgroups in flight together read neighbouring pieces of the same
+    // source lines' neighbourhood instead of pieces a whole (often power-of-two)
+    // pitch apart, which all fall on the same memory channels
+    const int64_t f0 = (int64_t)blockIdx.y * QT_FAST, s0 = (int64_t)blockIdx.x * QT_SLOW;
+    const int64_t r0 = dst_col_major ? f0 : s0, c0 = dst_col_major ? s0 : f0;
+    // the source values as f32, read along the source's stride-1 dim, which is
+    // the destination's slow one
+    // (every load of the thread is issued before the first value is used)
+    constexpr int NL = QT_FAST * QT_SLOW / 256;
+    const int ls = tid & (QT_SLOW - 1);
+    // the element of the tile's first line the thread reads, and the step to
+    // the next line: along the destination's stride-1 dim
+    const int64_t line = dst_col_major ? p.src_sr : p.src_sc;
+    const int64_t fmax = (dst_col_major ? p.rows : p.cols) - 1 - f0; // last valid line
+    const int64_t base = dst_col_major
+            ? r0 * p.src_sr + min(c0 + ls, p.cols - 1) * p.src_sc
+            : min(r0 + ls, p.rows - 1) * p.src_sr + c0 * p.src_sc;
+    uint32_t raw[NL];
+    if (p.src_dt == dt_f32) {
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            const int64_t lf = min((int64_t)(tid / QT_SLOW + (256 / QT_SLOW) * i), fmax);
+            raw[i] = ((const uint32_t *)p.src)[base + lf * line];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            const int64_t lf = min((int64_t)(tid / QT_SLOW + (256 / QT_SLOW) * i), fmax);
+            raw[i] = ((const uint16_t *)p.src)[base + lf * line];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const int lf = tid / QT_SLOW + (256 / QT_SLOW) * i;
+        tile[ls][lf] = p.src_dt == dt_f32 ? u2f(raw[i])
+                : p.src_dt == dt_f16
+                ? (float)__builtin_bit_cast(_Float16, (uint16_t)raw[i])
+                : u2f(raw[i] << 16);
+    }
+    __syncthreads();
+    const int ddt = p.dst_dt;
+    const bool nib = ddt == dt_s4 || ddt == dt_u4;
+    const float dst_zp = p.dst_zp ? (float)p.dst_zp[0] : 0.f;
+    // A thread's pair keeps its place along the destination's stride-1 dim
+    // through all its 8 steps: what does not depend on the other dim (a scale
+    // per column on the way into a row-major tensor, say) is fetched, and a
+    // dst scale inverted, once.
+    const int fast = (tid & (QT_FAST / 2 - 1)) * 2;
+    const auto along = [&](const quant_rows_q_t &q) { // varies with the slow dim?
+        return q.ptr && (dst_col_major ? q.sc != 0 : q.sr != 0);
+    };
+    const bool ss_var = along(p.src_scale), ds_var = along(p.dst_scale),
+               sz_var = along(p.src_zp);
+    const auto fetch = [&](int64_t r, int64_t c, bool second, float (&ss)[2],
+                               float (&ds)[2], float (&sz)[2], bool want_var) {
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int64_t re = min(r + (dst_col_major && e && second ? 1 : 0), p.rows - 1);
+            const int64_t ce = min(c + (!dst_col_major && e && second ? 1 : 0), p.cols - 1);
+            if (p.src_scale.ptr && ss_var == want_var)
+                ss[e] = load_float(p.src_scale.dt, p.src_scale.ptr,
+                        qr_off(p.src_scale, re, ce));
+            if (p.dst_scale.ptr && ds_var == want_var)
+                ds[e] = 1.f
+                        / load_float(p.dst_scale.dt, p.dst_scale.ptr,
+                                qr_off(p.dst_scale, re, ce));
+            // the zero point is an integer
+            if (p.src_zp.ptr && sz_var == want_var)
+                sz[e] = (float)(int)load_float(
+                        p.src_zp.dt, p.src_zp.ptr, qr_off(p.src_zp, re, ce));
+        }
+    };
+    float ss[2] = {1.f, 1.f}, ds[2] = {1.f, 1.f}, sz[2] = {0.f, 0.f};
+    {
+        const int64_t r = dst_col_major ? r0 + fast : r0, c = dst_col_major ? c0 : c0 + fast;
+        fetch(r, c, true, ss, ds, sz, false);
+    }
+    constexpr int SLOW_STEP = 256 / (QT_FAST / 2);
+#pragma unroll 4
+    for (int i = 0; i < QT_SLOW / SLOW_STEP; i++) {
+        const int slow = tid / (QT_FAST / 2) + SLOW_STEP * i;
+        const int64_t r = r0 + (dst_col_major ? fast : slow);
+        const int64_t c = c0 + (dst_col_major ? slow : fast);
+        if (r >= p.rows || c >= p.cols) continue;
+        // the pair's second element: the next row (column-major dst) or column
+        const bool second = dst_col_major ? r + 1 < p.rows : c + 1 < p.cols;
+        if (ss_var || ds_var || sz_var) fetch(r, c, second, ss, ds, sz, true);
+        // (the reference subtracts its default zero point 0 too)
+        const float d0 = ss[0] * (tile[slow][fast] - sz[0]) * ds[0] + dst_zp;
+        const float d1 = second ? ss[1] * (tile[slow][fast + 1] - sz[1]) * ds[1] + dst_zp : 0.f;
+        const int64_t o = r * p.dst_sr + c * p.dst_sc;
+        if (nib) {
+            // the host admits 4-bit destinations only where every pair starts
+            // on a byte and is whole
+            const float lo = ddt == dt_s4 ? -8.f : 0.f, hi = ddt == dt_s4 ? 7.f : 15.f;
+            ((uint8_t *)p.dst)[o >> 1] = (uint8_t)((round_sat(d0, lo, hi) & 0xf)
+                    | ((round_sat(d1, lo, hi) & 0xf) << 4));
+        } else if ((ddt == dt_s8 || ddt == dt_u8) && second) {
+            const float lo = ddt == dt_s8 ? -128.f : 0.f, hi = ddt == dt_s8 ? 127.f : 255.f;
+            // one two-byte store at any address
+            typedef uint16_t u16_any __attribute__((aligned(1)));
+            *(u16_any *)((uint8_t *)p.dst + o) = (uint16_t)((round_sat(d0, lo, hi) & 0xff)
+                    | ((round_sat(d1, lo, hi) & 0xff) << 8));
+        } else {
+            store_float(ddt, d0, p.dst, o);
+            if (second) store_float(ddt, d1, p.dst, o + 1);
+        }
+    }
+}
+
+void launch_quantize_transpose(const quant_tr_params_t &p, hipStream_t stream) {
+    if (p.rows <= 0 || p.cols <= 0) return;
+    const bool dst_col_major = p.dst_sr == 1;
+    const int64_t fast = dst_col_major ? p.rows : p.cols, slow = dst_col_major ? p.cols : p.rows;
+    const dim3 grid((unsigned)((slow + QT_SLOW - 1) / QT_SLOW),
+            (unsigned)((fast + QT_FAST - 1) / QT_FAST));
+    hipLaunchKernelGGL(quantize_transpose_kernel, grid, dim3(256), 0, stream, p);
 }
 
 // whether the 8-bit kernels cover the plan; how the dst scale runs (0: one

@@ -155,10 +155,11 @@ def test_three_dims_last_dim_scales(ctx):
 
 def test_other_shapes_stay_with_the_general_reorder(ctx):
     eng, strm = ctx
-    say("transposing / ragged reorders take the per-element kernel")
+    say("ragged rows, permutations of three dims and integer sources take the per-element kernel")
     N = 24
     sc = (2, dt.f32, None, np.random.default_rng(15).uniform(0.01, 0.1, N))
-    run_case(eng, strm, dt.f32, dt.s8, (64, N), 16, dst_scale=sc, layout="ab", dst_layout="ba", expect=REORDER)
+    run_case(eng, strm, dt.f32, dt.s8, (4, 16, N), 16, dst_scale=(4, dt.f32, None, sc[3]), layout="abc", dst_layout="acb",
+             expect=REORDER)
     run_case(eng, strm, dt.f32, dt.s8, (64, 20), 17, dst_scale=(0, dt.f32, None, [0.05]), expect=REORDER)
     run_case(eng, strm, dt.f32, dt.s8, (3, 8, 16), 18, dst_scale=(1, dt.f32, None, [0.05, 0.07, 0.09]), expect=REORDER)
 
@@ -184,3 +185,50 @@ def test_dequantize_int4_and_int8_weights_with_grouped_scales_and_zero_points(ct
     # groups along the last dim (activations quantized per row and 64 columns)
     run_case(eng, strm, dt.s8, dt.bf16, (40, K), 84, expect=REORDER, src_values=r.integers(-128, 128, (40, K)),
              src_scale=(3, dt.f32, (1, 64), r.uniform(0.01, 0.1, (40, K // 64))))
+
+
+TRANSPOSE = "hip:gfx950:quantize_transpose"
+
+
+@pytest.mark.parametrize("src_dt", [dt.f32, dt.bf16, dt.f16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("dims,src_layout,dst_dt,scale,zp", [
+    # weights stored [N, K] (column-major as a [K, N] tensor) quantized into row-major [K, N], one scale per column
+    ((256, 200), "ba", dt.s8, "col", None),
+    # tile tails on both dims, a dst zero point, scales per row
+    ((77, 130), "ba", dt.u8, "row", 5),
+    # row-major source into a column-major destination
+    ((130, 77), "ab", dt.s8, "col", -3),
+    # source scales per group of 32 rows and column (2-D mask with groups), 4-bit destination (pairs along the stride-1 dim)
+    ((128, 96), "ba", dt.s4, "grouped", None),
+    ((64, 192), "ab", dt.u4, "one", 8),
+    # 16-bit and fp8 destinations, a source scale on the way
+    ((100, 64), "ba", dt.bf16, "src", None),
+    ((66, 70), "ab", dt.f8_e4m3, "one", None),
+    ((2, 4098), "ba", dt.s8, "row", None), ((4098, 2), "ab", dt.u8, "none", 1),
+], ids=str)
+def test_transposing_quantizer(ctx, src_dt, dims, src_layout, dst_dt, scale, zp):
+    """The sides disagree on the dim order: a 64 x 64 tile through LDS, the row kernel's arithmetic per element. Bit for
+    bit against the oracle's reorder, with saturating values and a NaN in the source."""
+    eng, strm = ctx
+    say("transposing quantizer %s(%s) -> %s %s scale=%s zp=%s" % (src_dt, src_layout, dst_dt, dims, scale, zp))
+    r = np.random.default_rng(sum(dims) + src_dt + dst_dt)
+    amp = 3.0 if dst_dt in (dt.s4, dt.u4) else 40.0
+    x = (r.standard_normal(dims) * amp).astype(np.float32)
+    x.reshape(-1)[::97] *= 50
+    x.reshape(-1)[7 % x.size] = np.nan
+    R, C = dims
+    kw = {}
+    if scale == "col":
+        kw["dst_scale"] = (2, dt.f32, None, r.uniform(0.2, 0.9, C))
+    elif scale == "row":
+        kw["dst_scale"] = (1, dt.f32, None, r.uniform(0.2, 0.9, R))
+    elif scale == "one":
+        kw["dst_scale"] = (0, dt.f32, None, [0.37])
+    elif scale == "grouped":
+        kw["src_scale"] = (3, dt.f16, (32, 1), r.uniform(1.0, 3.0, (R // 32, C)))
+    elif scale == "src":
+        kw["src_scale"] = (2, dt.f32, None, r.uniform(0.5, 2.0, C))
+        kw["dst_scale"] = (0, dt.f32, None, [0.5])
+    dst_layout = "ab" if src_layout == "ba" else "ba"
+    run_case(eng, strm, src_dt, dst_dt, dims, 0, dst_zp=zp, layout=src_layout, dst_layout=dst_layout, expect=TRANSPOSE,
+             src_values=x, **kw)
