@@ -391,6 +391,8 @@ def test_reorder_descriptor_rules(eng):
     r = dnnl.reorder.primitive_desc(eng, pd.weights_desc(), eng, plain)
     assert r.impl_info_str() == "hip:gfx950:prepack"
     r = dnnl.reorder.primitive_desc(eng, memory.desc([8, 8], dt.f32, T("ab")), eng, memory.desc([8, 8], dt.s8, T("ba")))
+    assert r.impl_info_str() == "hip:gfx950:quantize_transpose"
+    r = dnnl.reorder.primitive_desc(eng, memory.desc([8, 8], dt.s8, T("ab")), eng, memory.desc([8, 8], dt.f32, T("ba")))
     assert r.impl_info_str() == "hip:gfx950:reorder"
     BAD = status.invalid_arguments
     expect(BAD, lambda: dnnl.reorder.primitive_desc(eng, memory.desc([8, 8], dt.f32, tag.any), eng, plain))
