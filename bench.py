@@ -549,7 +549,8 @@ def bench_gemm_anatomy(A, memory, dt, tag, T, eng, strm, hs, hiprt, steps=20, ro
     return res
 
 
-MFMA_KINDS = {"int8_16x16x64": 0, "int8_32x32x32": 1, "fp8_16x16x128": 2, "fp8_32x32x64": 3}
+MFMA_KINDS = {"int8_16x16x64": 0, "int8_32x32x32": 1, "fp8_16x16x128": 2, "fp8_32x32x64": 3,
+              "int8_16x16x64_weights_held": 4}
 
 
 def mfma_ceiling(hiprt, hs, kind, data=2, settle_s=1.0, steps=20, rounds=3, groups=256):
@@ -560,7 +561,7 @@ def mfma_ceiling(hiprt, hs, kind, data=2, settle_s=1.0, steps=20, rounds=3, grou
     import ctypes as C
     from onednn_amd import _capi
     L = _capi.lib()
-    ksteps = 112 if kind == 2 else (448 if kind == 1 else 224)
+    ksteps = 112 if kind == 2 else (448 if kind == 1 else 224)  # kinds 0 and 4: 224
     sink = hiprt.malloc(groups * 1024)
     ops = C.c_double()
 

@@ -311,7 +311,9 @@ QMM_API int qmm_stream_copy(void *dst, const void *src, size_t bytes, int groups
  * 128 x 128 wave tile) on register-resident operands (data 0: uniformly random
  * bytes, 1: zeros, 2: the value distributions of the int8 / fp8 benchmark
  * configurations): kind 0 = v_mfma_i32_16x16x64_i8, 1 = v_mfma_i32_32x32x32_i8,
- * 2 = v_mfma_f32_16x16x128_f8f6f4, 3 = v_mfma_f32_32x32x64_f8f6f4 (e4m3). One word
+ * 2 = v_mfma_f32_16x16x128_f8f6f4, 3 = v_mfma_f32_32x32x64_f8f6f4 (e4m3), 4 = kind 0
+ * with the weights fragment instead of the source fragment held over eight
+ * consecutive MFMAs. One word
  * per lane goes to `sink` (groups * 1024 bytes); *ops_per_launch receives the
  * multiply-add operations (x 2) of a launch. No counterpart in the reference;
  * benchmarks time it to state what the matrix cores sustain on this card next

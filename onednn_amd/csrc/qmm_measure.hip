@@ -165,9 +165,14 @@ __device__ inline uint32_t config_dword(bool f8, bool is_b, uint32_t h) {
 // data 0: uniformly random bytes; 1: all-zero operands (what the same loop
 // reaches when nothing toggles); 2: the distributions of the benchmark
 // configurations (config_dword).
-template <int KIND>
+// KIND 4: KIND 0 (int8 16 x 16 x 64) walking the fragment grid column by column:
+// eight consecutive MFMAs keep the weights fragment and change the source
+// fragment, where KIND 0 keeps the source fragment and changes the weights.
+template <int KIND0>
 __global__ void __launch_bounds__(256, 1)
 mfma_ceiling_kernel(uint32_t seed, int ksteps, int data, uint32_t *sink) {
+    constexpr int KIND = KIND0 == 4 ? 0 : KIND0;
+    constexpr bool BY_COLUMN = KIND0 == 4;
     constexpr bool F8 = KIND >= 2;
     constexpr bool SMALL = KIND == 0 || KIND == 2; // 16 x 16 fragments
     constexpr int NF = SMALL ? 8 : 4; // fragment grid NF x NF
@@ -206,9 +211,10 @@ mfma_ceiling_kernel(uint32_t seed, int ksteps, int data, uint32_t *sink) {
 #pragma unroll
         for (int s = 0; s < 2; s++)
 #pragma unroll
-            for (int i = 0; i < NF; i++)
+            for (int i0 = 0; i0 < NF; i0++)
 #pragma unroll
-                for (int j = 0; j < NF; j++) {
+                for (int j0 = 0; j0 < NF; j0++) {
+                    const int i = BY_COLUMN ? j0 : i0, j = BY_COLUMN ? i0 : j0;
                     if constexpr (KIND == 0)
                         // accumulators pinned to the accumulator file: with the
                         // builtin the allocator moves part of them through
@@ -246,7 +252,7 @@ mfma_ceiling_kernel(uint32_t seed, int ksteps, int data, uint32_t *sink) {
 
 extern "C" int qmm_mfma_ceiling(int kind, int ksteps, int groups, int data,
         void *sink, void *stream, double *ops_per_launch) {
-    if (kind < 0 || kind > 3 || data < 0 || data > 2 || ksteps < 2 || (ksteps & 1) || groups < 1 || !sink)
+    if (kind < 0 || kind > 4 || data < 0 || data > 2 || ksteps < 2 || (ksteps & 1) || groups < 1 || !sink)
         return QMM_INVALID_ARGUMENTS;
     // operations of one k-step of one wave: the fragment grid covers 128 x 128
     // outputs; a k-step contracts 64 k (int8, fp8 32 x 32 x 64) or 128 k
@@ -260,7 +266,8 @@ extern "C" int qmm_mfma_ceiling(int kind, int ksteps, int groups, int data,
         case 0: hipLaunchKernelGGL(mfma_ceiling_kernel<0>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
         case 1: hipLaunchKernelGGL(mfma_ceiling_kernel<1>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
         case 2: hipLaunchKernelGGL(mfma_ceiling_kernel<2>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
-        default: hipLaunchKernelGGL(mfma_ceiling_kernel<3>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
+        case 3: hipLaunchKernelGGL(mfma_ceiling_kernel<3>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
+        default: hipLaunchKernelGGL(mfma_ceiling_kernel<4>, g, b, 0, st, 0x9e3779b9u, ksteps, data, out); break;
     }
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }
