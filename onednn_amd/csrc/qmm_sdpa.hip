@@ -595,7 +595,8 @@ sdpa_decode_kernel(const sdpa_params_t p) {
             qsz[0] = sp ? ld_scale(up ? p.vs_dt : p.ks_dt, sp, qz_base + key) : 1.f;
             qsz[1] = zp ? ld_zp(up ? p.vz_dt : p.kz_dt, zp, qz_base + key) : 0.f;
         }
-        // V: lane l carries chunk (l % (D / 8)) of key (l / (D / 8)) + 64 / (D / 8) * n
+        // V: the tile's 8-element pieces in turn (piece i: key i / (D / 8), chunk
+        // i % (D / 8)), lane l carries the pieces l, l + 64, ...
 #pragma unroll
         for (int n = 0; n < D / 16; n++) {
             const int i = lane + 64 * n;
@@ -886,9 +887,10 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
     if (d.v.dims[nd - 1] != D) return false; // head size of V = head size of Q
     if (d.dst.dims[nd - 2] != Qn || d.dst.dims[nd - 1] != D) return false;
-    // head sizes: 64 and 128 in every form; 32 and 256 with K / V in the
+    // head sizes: 64 and 128 in every form; 32, 96 and 256 with K / V in the
     // queries' type (the 8-bit cache paths are instantiated for 64 and 128)
-    if (D != 64 && D != 128 && !((D == 32 || D == 256) && d.k.dt == d.q.dt))
+    if (D != 64 && D != 128
+            && !((D == 32 || D == 96 || D == 256) && d.k.dt == d.q.dt))
         return false;
     if (Qn < 1 || S < 1 || Qn > (1 << 30) || S > (1 << 30)) return false;
     // innermost-contiguous rows: Q [q][d], K as the transposed view of a
@@ -1063,9 +1065,13 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
             hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
                     (hipStream_t)hip_stream, p);
         };
-        if (D == 32 || D == 256) {
+        if (D == 32 || D == 96 || D == 256) {
             // K / V in the queries' type only (supported())
-            switch ((D == 256 ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+            switch ((D == 256 ? 4 : D == 96 ? 8 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+                case 8: god(sdpa_decode_kernel<3, false, false, false>); break;
+                case 9: god(sdpa_decode_kernel<3, false, true, false>); break;
+                case 10: god(sdpa_decode_kernel<3, false, false, true>); break;
+                case 11: god(sdpa_decode_kernel<3, false, true, true>); break;
                 case 0: god(sdpa_decode_kernel<1, false, false, false>); break;
                 case 1: god(sdpa_decode_kernel<1, false, true, false>); break;
                 case 2: god(sdpa_decode_kernel<1, false, false, true>); break;
@@ -1118,8 +1124,12 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);
     };
-    if (D == 32 || D == 256) {
-        switch ((D == 256 ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+    if (D == 32 || D == 96 || D == 256) {
+        switch ((D == 256 ? 4 : D == 96 ? 8 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
+            case 8: go(sdpa_f16_kernel<3, false, false, false>); break;
+            case 9: go(sdpa_f16_kernel<3, false, true, false>); break;
+            case 10: go(sdpa_f16_kernel<3, false, false, true>); break;
+            case 11: go(sdpa_f16_kernel<3, false, true, true>); break;
             case 0: go(sdpa_f16_kernel<1, false, false, false>); break;
             case 1: go(sdpa_f16_kernel<1, false, true, false>); break;
             case 2: go(sdpa_f16_kernel<1, false, false, true>); break;

@@ -115,6 +115,10 @@ CASES = [
     ((1, 2), 0, 16, 33, 64, "none", "mul"),
     # head sizes 32 and 256 (K / V in the queries' type): many queries, the few-queries form split over the keys, masks
     ((1, 4), 0, 150, 200, 32, "2d", "mul"),
+    ((1, 2), 0, 384, 384, 96, "2d", "mul"),
+    ((1, 2), 0, 1, 385, 96, "2d", "mul"),
+    ((2, 3), 0, 33, 259, 96, "causal", "div"),
+    ((1, 4), 2, 9, 129, 96, "none", "mul"),
     ((2, 2), 0, 8, 300, 32, "causal", "mul"),
     ((3,), 0, 1, 1000, 32, "1d", "div"),
     ((1, 2), 0, 130, 170, 256, "causal", "div"),
@@ -310,7 +314,7 @@ def test_what_the_kernel_does_not_take_is_unimplemented(ctx):
         return dnnl.sdpa.primitive_desc(eng, a["q"], a["k"], a["v"], None, dt.undef, a["o"])
 
     make()
-    for bad in (dict(q=md([1, 2, 16, 96]), k=md([1, 2, 96, 32], t="abdc"), v=md([1, 2, 32, 96]), o=md([1, 2, 16, 96])),  # head size
+    for bad in (dict(q=md([1, 2, 16, 80]), k=md([1, 2, 80, 32], t="abdc"), v=md([1, 2, 32, 80]), o=md([1, 2, 16, 80])),  # head size
                 dict(q=md([1, 2, 16, 32]), k=md([1, 2, 32, 32], dt.s8, t="abdc"), v=md([1, 2, 32, 32], dt.s8),
                      o=md([1, 2, 16, 32])),                                    # an 8-bit cache at head size 32
                 dict(k=md([1, 2, 64, 32])),                                    # keys contiguous instead of head size
