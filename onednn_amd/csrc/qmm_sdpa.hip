@@ -887,11 +887,8 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
     if (d.v.dims[nd - 1] != D) return false; // head size of V = head size of Q
     if (d.dst.dims[nd - 2] != Qn || d.dst.dims[nd - 1] != D) return false;
-    // head sizes: 64 and 128 in every form; 32, 96 and 256 with K / V in the
-    // queries' type (the 8-bit cache paths are instantiated for 64 and 128)
-    if (D != 64 && D != 128
-            && !((D == 32 || D == 96 || D == 256) && d.k.dt == d.q.dt))
-        return false;
+    // head sizes: 1, 2, 3, 4 or 8 chunks of 32
+    if (D != 32 && D != 64 && D != 96 && D != 128 && D != 256) return false;
     if (Qn < 1 || S < 1 || Qn > (1 << 30) || S > (1 << 30)) return false;
     // innermost-contiguous rows: Q [q][d], K as the transposed view of a
     // [keys][d] cache, V [keys][d], dst [q][d]
@@ -1050,7 +1047,6 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.v_scale = desc->v_scale.set ? args->v_scale : nullptr;
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
     const int D = (int)desc->q.dims[desc->q.ndims - 1];
-    const bool d128 = D == 128;
     const bool qn = p.kv_dt != desc->q.dt, mk = p.mask != nullptr;
     const bool bf = p.bf != 0; // never together with qn
     if (p.Qn <= 16) {
@@ -1065,37 +1061,24 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
             hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
                     (hipStream_t)hip_stream, p);
         };
-        if (D == 32 || D == 96 || D == 256) {
-            // K / V in the queries' type only (supported())
-            switch ((D == 256 ? 4 : D == 96 ? 8 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
-                case 8: god(sdpa_decode_kernel<3, false, false, false>); break;
-                case 9: god(sdpa_decode_kernel<3, false, true, false>); break;
-                case 10: god(sdpa_decode_kernel<3, false, false, true>); break;
-                case 11: god(sdpa_decode_kernel<3, false, true, true>); break;
-                case 0: god(sdpa_decode_kernel<1, false, false, false>); break;
-                case 1: god(sdpa_decode_kernel<1, false, true, false>); break;
-                case 2: god(sdpa_decode_kernel<1, false, false, true>); break;
-                case 3: god(sdpa_decode_kernel<1, false, true, true>); break;
-                case 4: god(sdpa_decode_kernel<8, false, false, false>); break;
-                case 5: god(sdpa_decode_kernel<8, false, true, false>); break;
-                case 6: god(sdpa_decode_kernel<8, false, false, true>); break;
-                case 7: god(sdpa_decode_kernel<8, false, true, true>); break;
-                default: return QMM_UNIMPLEMENTED;
-            }
-        } else
-        switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
-            case 0: god(sdpa_decode_kernel<2, false, false, false>); break;
-            case 1: god(sdpa_decode_kernel<2, false, true, false>); break;
-            case 2: god(sdpa_decode_kernel<2, true, false, false>); break;
-            case 3: god(sdpa_decode_kernel<2, true, true, false>); break;
-            case 4: god(sdpa_decode_kernel<4, false, false, false>); break;
-            case 5: god(sdpa_decode_kernel<4, false, true, false>); break;
-            case 6: god(sdpa_decode_kernel<4, true, false, false>); break;
-            case 7: god(sdpa_decode_kernel<4, true, true, false>); break;
-            case 8: god(sdpa_decode_kernel<2, false, false, true>); break;
-            case 9: god(sdpa_decode_kernel<2, false, true, true>); break;
-            case 12: god(sdpa_decode_kernel<4, false, false, true>); break;
-            case 13: god(sdpa_decode_kernel<4, false, true, true>); break;
+        // template arguments from the run-time choices (bf16 queries never
+        // come with an 8-bit cache: supported())
+#define SDPA_PICK(KERN, GO, DCV) \
+    switch ((qn ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) { \
+        case 0: GO(KERN<DCV, false, false, false>); break; \
+        case 1: GO(KERN<DCV, false, true, false>); break; \
+        case 2: GO(KERN<DCV, false, false, true>); break; \
+        case 3: GO(KERN<DCV, false, true, true>); break; \
+        case 4: GO(KERN<DCV, true, false, false>); break; \
+        case 5: GO(KERN<DCV, true, true, false>); break; \
+        default: return QMM_UNIMPLEMENTED; \
+    }
+        switch (D) {
+            case 32: SDPA_PICK(sdpa_decode_kernel, god, 1) break;
+            case 64: SDPA_PICK(sdpa_decode_kernel, god, 2) break;
+            case 96: SDPA_PICK(sdpa_decode_kernel, god, 3) break;
+            case 128: SDPA_PICK(sdpa_decode_kernel, god, 4) break;
+            case 256: SDPA_PICK(sdpa_decode_kernel, god, 8) break;
             default: return QMM_UNIMPLEMENTED;
         }
         if (p.nsplit > 1)
@@ -1124,38 +1107,15 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         hipLaunchKernelGGL(kern, grid, dim3(SDPA_WAVES * 64), 0,
                 (hipStream_t)hip_stream, p);
     };
-    if (D == 32 || D == 96 || D == 256) {
-        switch ((D == 256 ? 4 : D == 96 ? 8 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) {
-            case 8: go(sdpa_f16_kernel<3, false, false, false>); break;
-            case 9: go(sdpa_f16_kernel<3, false, true, false>); break;
-            case 10: go(sdpa_f16_kernel<3, false, false, true>); break;
-            case 11: go(sdpa_f16_kernel<3, false, true, true>); break;
-            case 0: go(sdpa_f16_kernel<1, false, false, false>); break;
-            case 1: go(sdpa_f16_kernel<1, false, true, false>); break;
-            case 2: go(sdpa_f16_kernel<1, false, false, true>); break;
-            case 3: go(sdpa_f16_kernel<1, false, true, true>); break;
-            case 4: go(sdpa_f16_kernel<8, false, false, false>); break;
-            case 5: go(sdpa_f16_kernel<8, false, true, false>); break;
-            case 6: go(sdpa_f16_kernel<8, false, false, true>); break;
-            case 7: go(sdpa_f16_kernel<8, false, true, true>); break;
-            default: return QMM_UNIMPLEMENTED;
-        }
-    } else
-    switch ((bf ? 8 : 0) | (d128 ? 4 : 0) | (qn ? 2 : 0) | (mk ? 1 : 0)) {
-        case 0: go(sdpa_f16_kernel<2, false, false, false>); break;
-        case 1: go(sdpa_f16_kernel<2, false, true, false>); break;
-        case 2: go(sdpa_f16_kernel<2, true, false, false>); break;
-        case 3: go(sdpa_f16_kernel<2, true, true, false>); break;
-        case 4: go(sdpa_f16_kernel<4, false, false, false>); break;
-        case 5: go(sdpa_f16_kernel<4, false, true, false>); break;
-        case 6: go(sdpa_f16_kernel<4, true, false, false>); break;
-        case 7: go(sdpa_f16_kernel<4, true, true, false>); break;
-        case 8: go(sdpa_f16_kernel<2, false, false, true>); break;
-        case 9: go(sdpa_f16_kernel<2, false, true, true>); break;
-        case 12: go(sdpa_f16_kernel<4, false, false, true>); break;
-        case 13: go(sdpa_f16_kernel<4, false, true, true>); break;
+    switch (D) {
+        case 32: SDPA_PICK(sdpa_f16_kernel, go, 1) break;
+        case 64: SDPA_PICK(sdpa_f16_kernel, go, 2) break;
+        case 96: SDPA_PICK(sdpa_f16_kernel, go, 3) break;
+        case 128: SDPA_PICK(sdpa_f16_kernel, go, 4) break;
+        case 256: SDPA_PICK(sdpa_f16_kernel, go, 8) break;
         default: return QMM_UNIMPLEMENTED;
     }
+#undef SDPA_PICK
     return hipGetLastError() == hipSuccess ? QMM_OK : QMM_RUNTIME_ERROR;
 }
 
