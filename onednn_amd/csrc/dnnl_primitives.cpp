@@ -341,6 +341,8 @@ void fill_quant(qmm_quant_t &q, const quant_entry_t &e, dnnl_data_type_t dflt) {
     }
 }
 
+bool collapse_broadcast_batch(qmm_matmul_desc_t &D);
+
 // Build the kernel-level description from resolved descriptors.
 void fill_mm_desc(pd_impl_t &pd) {
     qmm_matmul_desc_t &D = pd.mm;
@@ -381,6 +383,100 @@ void fill_mm_desc(pd_impl_t &pd) {
             default: break;
         }
     }
+    collapse_broadcast_batch(D);
+}
+
+// Weights that are one matrix for every batch entry ([1, .., 1, K, N]) under a
+// source and a destination whose batch dims nest densely over their rows: the
+// problem IS the 2-D product [batch x M, K] x [K, N], and as that it reaches the
+// kernels that take two dims only (weights decompression, int8 x int4, f16 x
+// 8-bit weights). Every tensor and attribute must read the same under the new
+// shape: operands of bias / binary post-ops and scales / zero points either do
+// not depend on (batch, M) at all or cover all of them densely; a prelu mask
+// names the last dim only. Returns false and leaves D alone otherwise.
+bool collapse_broadcast_batch(qmm_matmul_desc_t &D) {
+    const int nd = D.dst.ndims;
+    if (nd < 3) return false;
+    const int nb = nd - 2;
+    for (int d = 0; d < nb; d++)
+        if (D.wei.dims[d] != 1) return false;
+    // (batch .., M) as one row index with the M pitch
+    auto rows_nest = [&](const qmm_tensor_t &t) {
+        for (int d = 0; d < nb; d++)
+            if (t.dims[d] != 1
+                    && t.strides[d] != t.strides[d + 1] * t.dims[d + 1])
+                return false;
+        return true;
+    };
+    // an operand of dst's rank: 0 = no dependence on (batch, M), 1 = all of
+    // them as in dst and nesting, -1 = anything else
+    auto rows_kind = [&](const qmm_tensor_t &t) {
+        if (t.ndims != nd) return -1;
+        bool none = true, all = true;
+        for (int d = 0; d <= nb; d++) {
+            none = none && t.dims[d] == 1;
+            all = all && t.dims[d] == D.dst.dims[d];
+        }
+        if (none) return 0;
+        return all && rows_nest(t) ? 1 : -1;
+    };
+    if (!rows_nest(D.src) || !rows_nest(D.dst)) return false;
+    int bias_kind = 0;
+    if (D.bias.ndims && (bias_kind = rows_kind(D.bias)) < 0) return false;
+    int po_kind[QMM_MAX_POST_OPS] = {};
+    for (int i = 0; i < D.npo; i++) {
+        if (D.po[i].kind == dnnl_binary
+                && (po_kind[i] = rows_kind(D.po[i].src1)) < 0)
+            return false;
+        if (D.po[i].kind == dnnl_prelu && (D.po[i].mask & ~(1 << (nd - 1))))
+            return false;
+    }
+    const int row_bits = (1 << (nb + 1)) - 1; // batch dims and M
+    // scales / zero points: of the source and the destination over (batch, M)
+    // all or none, without a group over M; of the weights whatever their batch
+    // bits say (those dims are 1)
+    int new_mask[2][3];
+    for (int z = 0; z < 2; z++)
+        for (int a = 0; a < 3; a++) {
+            const qmm_quant_t &q = z ? D.zps[a] : D.scales[a];
+            new_mask[z][a] = 0;
+            if (!q.set) continue;
+            if (a == QMM_WEI) {
+                new_mask[z][a] = (q.mask >> nb) & 3;
+                continue;
+            }
+            const int rb = q.mask & row_bits;
+            if (rb != 0 && rb != row_bits) return false;
+            if (rb && q.has_groups && q.g0 != 1) return false;
+            new_mask[z][a] = (rb ? 1 : 0) | ((q.mask >> (nd - 1)) & 1 ? 2 : 0);
+        }
+    int64_t rows = 1;
+    for (int d = 0; d <= nb; d++)
+        rows *= D.dst.dims[d];
+    auto to2d = [&](qmm_tensor_t &t, bool over_rows) {
+        const int64_t d0 = over_rows ? rows : t.dims[nd - 2];
+        const int64_t s0 = t.strides[nd - 2], d1 = t.dims[nd - 1],
+                      s1 = t.strides[nd - 1];
+        t.ndims = 2;
+        t.dims[0] = d0, t.dims[1] = d1;
+        t.strides[0] = s0, t.strides[1] = s1;
+        for (int d = 2; d < QMM_MAX_NDIMS; d++)
+            t.dims[d] = t.strides[d] = 0;
+    };
+    to2d(D.src, true);
+    to2d(D.dst, true);
+    to2d(D.wei, false);
+    if (D.bias.ndims) to2d(D.bias, bias_kind == 1);
+    for (int i = 0; i < D.npo; i++) {
+        if (D.po[i].kind == dnnl_binary) to2d(D.po[i].src1, po_kind[i] == 1);
+        if (D.po[i].kind == dnnl_prelu) D.po[i].mask = D.po[i].mask ? 2 : 0;
+    }
+    for (int z = 0; z < 2; z++)
+        for (int a = 0; a < 3; a++) {
+            qmm_quant_t &q = z ? D.zps[a] : D.scales[a];
+            if (q.set) q.mask = new_mask[z][a];
+        }
+    return true;
 }
 
 int64_t batch_of(const dnnl_memory_desc &md) {
