@@ -191,7 +191,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kern_tops, 2), "peak": PEAK_INT8, "unit": "TOP/s",
                      "frac": round(kern_tops / PEAK_INT8, 4),
                      "traffic": traffic[0] if args.variant == 0 else None, "traffic_source": traffic[1],
-                     "kernel": "gemm_b8y_kernel (int8, 256x256 tile, 16x16x64 MFMA)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
+                     "kernel": "gemm_b8y_kernel (int8, 256x256 tile, 16x16x64 MFMA, persistent grid of one workgroup per CU)" if args.variant in (0, 6) else "gemm_b8_kernel (int8)", "kernel_ms": round(ev_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }
     # what the matrix cores sustain on this card in this run (MFMA-only loop, random operands), next to the published peak
