@@ -88,7 +88,7 @@ def main():
                     help="run one of the side measurements alone and print its JSON (for profiling)")
     ap.add_argument("--clock-warmup-s", type=float, default=2.0,
                     help="seconds of untimed launches of the same primitive before the timed steps (after --warmup)")
-    ap.add_argument("--cpu-rows", type=int, default=640, help="rows of config 2 timed on the CPU oracle")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of config 2 timed on the CPU oracle")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB copy kernel (reference point for the rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -204,11 +204,13 @@ def main():
     # ------------------------------------------------------- CPU baseline
     if not args.no_cpu_baseline:
         import oracle as O
-        rows = min(args.cpu_rows, M)
+        host = host_cpu()
+        # the whole problem where the oracle's K sums run on byte dot products (about a second), a sample of 640 rows
+        # (about 10 s) where they run scalar
+        rows = min(args.cpu_rows if host["oracle_isa"] != "scalar" else min(args.cpu_rows, 640), M)
         sel = np.linspace(0, M - 1, rows).astype(np.int64)
         s_sub = np.ascontiguousarray(src[sel])
         d_sub = np.zeros((rows, N), np.uint16)
-        host = host_cpu()
         ncores = min(host["usable_cpus"], int(os.environ.get("OMP_NUM_THREADS", "16")))
         t = time.perf_counter()
         O.matmul(O.Tensor(O.S8, [rows, K], s_sub), O.Tensor(O.S8, [K, N], wei), O.Tensor(O.BF16, [rows, N], d_sub),
@@ -225,8 +227,11 @@ def main():
                                    "decode_common_zp_M1_ms": 20.1,
                                    "note": "config 2 there ran with one common src scale: the reference's brgemm has no "
                                            "per-token src scales, and its scalar fallback was not timed"},
-                               "sample": "%d of the 4096 rows of config 2 (evenly spaced), full K and N, "
-                                         "scalar C oracle with OpenMP, %.1f s" % (rows, cpu_s)}
+                               "sample": "%d of the 4096 rows of config 2 (evenly spaced), full K and N, the C oracle with "
+                                         "OpenMP: its K sums on %s, everything else (scales, swish through libm, the bf16 "
+                                         "store) per element as the reference's scalar code, %.1f s"
+                                         % (rows, "AVX-512 VNNI byte dot products (64 products an instruction)"
+                                            if host["oracle_isa"] == "avx512_vnni" else "the scalar loop", cpu_s)}
         # the same rows double as a parity check of the timed kernel's output
         got = m_dst.read(np.uint16, (M, N))[sel]
         import contextlib
@@ -258,8 +263,11 @@ def host_cpu():
         usable = len(os.sched_getaffinity(0))
     except AttributeError:
         usable = os.cpu_count() or 1
+    vnni = {"avx512f", "avx512bw", "avx512_vnni"} <= flags and os.environ.get("QMM_ORACLE_SCALAR") != "1"
     return {"model": model, "logical_cpus": os.cpu_count(), "usable_cpus": usable, "widest_isa": isa,
-            "note": "the oracle is scalar C with OpenMP: it uses none of the vector ISAs named here"}
+            "oracle_isa": "avx512_vnni" if vnni else "scalar",
+            "note": "the oracle is C with OpenMP; the K sums of its integer path run on AVX-512 VNNI byte dot products where "
+                    "the host has them (bit-identical to its scalar loop), the rest is scalar"}
 
 
 def C_stream(strm):

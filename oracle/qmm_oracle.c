@@ -14,6 +14,7 @@
 #include <float.h>
 #include <limits.h>
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
 #include <omp.h>
@@ -632,6 +633,53 @@ static int is_wei_int(int dt) {
     return dt == ORC_S8 || dt == ORC_U8 || dt == ORC_S4 || dt == ORC_U4;
 }
 
+/* ---- the group's integer dot product on the host's byte dot-product
+ * instruction ------------------------------------------------------------
+ * Not another algorithm: the sum over a K group of s * w that the loop of
+ * matmul_int8 forms one product at a time, formed 64 products at a time where
+ * the CPU has AVX-512 VNNI (vpdpbusd: u8 x s8 -> s32). Integer sums wrap the
+ * same in any order, so the result is the scalar loop's bit for bit
+ * (tests/test_oracle_matmul.py runs both and compares). Taken for 2-D
+ * problems with an s8 or u8 source whose rows are contiguous, s8 weights and
+ * no zero points; the weights are copied once per call as [N][K] so that a
+ * column's k run is contiguous, with the group sums of every column next to
+ * them: an s8 source enters as s + 128 (one flipped bit), and 128 x the
+ * column's group sum leaves the product again. QMM_ORACLE_SCALAR=1 in the
+ * environment switches it off. This is what makes the oracle usable as a CPU
+ * baseline on the GPU box's host cores. */
+#if defined(__x86_64__)
+#include <immintrin.h>
+__attribute__((target("avx512f,avx512bw,avx512vnni")))
+static int32_t dot_u8s8(const uint8_t *a, const int8_t *b, int64_t n) {
+    __m512i acc = _mm512_setzero_si512();
+    int64_t i = 0;
+    for (; i + 64 <= n; i += 64)
+        acc = _mm512_dpbusd_epi32(acc, _mm512_loadu_si512((const void *)(a + i)),
+                _mm512_loadu_si512((const void *)(b + i)));
+    if (i < n) {
+        const __mmask64 m = (~(uint64_t)0) >> (64 - (n - i));
+        acc = _mm512_dpbusd_epi32(acc, _mm512_maskz_loadu_epi8(m, a + i),
+                _mm512_maskz_loadu_epi8(m, b + i));
+    }
+    return _mm512_reduce_add_epi32(acc);
+}
+static int have_vnni(void) {
+    const char *e = getenv("QMM_ORACLE_SCALAR");
+    if (e && e[0] == '1') return 0;
+    __builtin_cpu_init();
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw")
+            && __builtin_cpu_supports("avx512vnni");
+}
+#else
+static int32_t dot_u8s8(const uint8_t *a, const int8_t *b, int64_t n) {
+    (void)a, (void)b, (void)n;
+    return 0;
+}
+static int have_vnni(void) {
+    return 0;
+}
+#endif
+
 /* integer path: src/cpu/matmul/ref_matmul_int8.cpp:154-261 */
 static void matmul_int8(const orc_matmul_t *p, const mm_ctx_t *c,
         int32_t *acc_out) {
@@ -648,8 +696,75 @@ static void matmul_int8(const orc_matmul_t *p, const mm_ctx_t *c,
     const int sum_dt = sum_dt_of(p);
     const int64_t rows = c->batch * c->M;
 
+    /* the fast form of the group's dot product (see dot_u8s8) */
+    int8_t *wt = NULL; /* [N][K] */
+    int32_t *wsum = NULL; /* [N][groups]: sum of the column's weights per group */
+    const int fast = nd == 2 && c->K > 0 && is_int_dt(p->src.dt)
+            && p->wei.dt == ORC_S8 && !sz->set && !wz->set
+            && p->src.strides[1] == 1 && c->group_k >= 16 && have_vnni();
+    if (fast) {
+        wt = (int8_t *)malloc((size_t)c->N * c->K);
+        wsum = (int32_t *)malloc((size_t)c->N * c->ngroups_k * sizeof(int32_t));
+        if (wt && wsum) {
+            const int8_t *w = (const int8_t *)p->wei.ptr;
 #pragma omp parallel for schedule(static)
-    for (int64_t row = 0; row < rows; row++) {
+            for (int64_t n = 0; n < c->N; n++) {
+                for (int64_t k = 0; k < c->K; k++)
+                    wt[n * c->K + k]
+                            = w[k * p->wei.strides[0] + n * p->wei.strides[1]];
+                for (int64_t g = 0; g < c->ngroups_k; g++) {
+                    int32_t t = 0;
+                    for (int64_t k = 0; k < c->group_k; k++)
+                        t += wt[n * c->K + g * c->group_k + k];
+                    wsum[n * c->ngroups_k + g] = t;
+                }
+            }
+        }
+    }
+    const int use_fast = fast && wt && wsum;
+
+    /* rows are taken in blocks so that, in the fast form, a weights column
+     * read from memory serves a block's rows (the block's group sums are
+     * formed first, column by column, and the loop below picks them up) */
+    int64_t RB = 1;
+    if (use_fast) {
+        RB = 32;
+        while (RB > 1 && RB * c->N * c->ngroups_k * 4 > ((int64_t)8 << 20))
+            RB /= 2;
+    }
+    const int64_t nblocks = (rows + RB - 1) / RB;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t blk = 0; blk < nblocks; blk++) {
+    const int64_t row_lo = blk * RB, row_hi = row_lo + RB < rows ? row_lo + RB : rows;
+    uint8_t *urows = NULL; /* the block's rows as unsigned bytes: an s8 source
+                              with its top bit flipped */
+    int32_t *accb = NULL; /* [row in block][N][group] */
+    if (use_fast) {
+        urows = (uint8_t *)malloc((size_t)RB * c->K);
+        accb = (int32_t *)malloc((size_t)RB * c->N * c->ngroups_k * sizeof(int32_t));
+    }
+    if (urows && accb) {
+        const uint8_t flip = p->src.dt == ORC_S8 ? 0x80 : 0;
+        for (int64_t row = row_lo; row < row_hi; row++) {
+            const uint8_t *sr = (const uint8_t *)p->src.ptr + row * p->src.strides[0];
+            for (int64_t k = 0; k < c->K; k++)
+                urows[(row - row_lo) * c->K + k] = sr[k] ^ flip;
+        }
+        for (int64_t n = 0; n < c->N; n++)
+            for (int64_t g = 0; g < c->ngroups_k; g++) {
+                const int8_t *wc = wt + n * c->K + g * c->group_k;
+                const uint32_t back = p->src.dt == ORC_S8
+                        ? 128u * (uint32_t)wsum[n * c->ngroups_k + g]
+                        : 0u;
+                for (int64_t r = 0; r < row_hi - row_lo; r++)
+                    accb[(r * c->N + n) * c->ngroups_k + g] = (int32_t)(
+                            (uint32_t)dot_u8s8(urows + r * c->K + g * c->group_k,
+                                    wc, c->group_k)
+                            - back);
+            }
+    }
+    const int blk_fast = urows && accb;
+    for (int64_t row = row_lo; row < row_hi; row++) {
         const int64_t mb = row / c->M, m = row % c->M;
         for (int64_t n = 0; n < c->N; n++) {
             const int64_t l_offset = mb * c->M * c->N + m * c->N + n;
@@ -664,7 +779,13 @@ static void matmul_int8(const orc_matmul_t *p, const mm_ctx_t *c,
             float d = 0;
             for (int64_t g = 0; g < c->ngroups_k; g++) {
                 int32_t acc = 0;
-                for (int64_t k = 0; k < c->group_k; k++) {
+                if (blk_fast) {
+                    acc = accb[((row - row_lo) * c->N + n) * c->ngroups_k + g];
+                    /* the scale lookups below index by the group's last k */
+                    si[nd - 1] = (g + 1) * c->group_k - 1;
+                    wi[nd - 2] = (g + 1) * c->group_k - 1;
+                }
+                for (int64_t k = 0; k < (blk_fast ? 0 : c->group_k); k++) {
                     si[nd - 1] = k + g * c->group_k;
                     wi[nd - 2] = k + g * c->group_k;
                     int s = orc_load_int(p->src.dt, p->src.ptr,
@@ -718,6 +839,11 @@ static void matmul_int8(const orc_matmul_t *p, const mm_ctx_t *c,
             orc_store_float(p->dst.dt, d, p->dst.ptr, dst_off);
         }
     }
+    free(urows);
+    free(accb);
+    } /* row blocks */
+    free(wt);
+    free(wsum);
 }
 
 /* float / fp8 / weights-decompression path:

@@ -418,3 +418,44 @@ def test_reorder_every_quantization_entry_against_numpy_float32():
     outb = np.zeros((R, Ccols), np.uint16)
     O.reorder(T(O.F32, x), T(O.BF16, outb), dst_scale=O.Quant(2, O.F32, dsc))
     assert np.array_equal(outb, torch.from_numpy(scaled).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("src_dt", ["s8", "u8"])
+@pytest.mark.parametrize("M,K,N,gk,wei_t", [(5, 100, 7, None, False), (9, 256, 33, 64, False), (3, 4096, 20, 128, True),
+                                            (4, 16, 5, None, False), (2, 191, 3, None, True), (6, 512, 65, 32, False)])
+def test_byte_dot_product_instruction_gives_the_scalar_loops_bits(monkeypatch, src_dt, M, K, N, gk, wei_t):
+    """The integer path forms a K group's sum of products 64 at a time where the host has AVX-512 VNNI (u8 x s8 dot
+    products; an s8 source enters as s + 128 and 128 x the column's sum leaves again). Integer sums wrap the same in any
+    order: the destination (f32 with scales per row and per group and column, a swish behind them) and the raw s32
+    accumulators must be the scalar loop's bit for bit. Extreme values included (-128 x -128 four times in a row is the
+    instruction's largest intermediate sum)."""
+    rng = np.random.default_rng(M * 1000 + K + N)
+    if src_dt == "s8":
+        src = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        src[0, :8] = -128
+        sdt = O.S8
+    else:
+        src = rng.integers(0, 256, (M, K)).astype(np.uint8)
+        src[0, :8] = 255
+        sdt = O.U8
+    wei = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    wei[:8, 0] = -128
+    wt = O.Tensor(O.S8, [K, N], np.ascontiguousarray(wei.T), [1, K]) if wei_t else T(O.S8, wei)
+    if gk:
+        scales = {O.Q_SRC: O.Quant(3, O.F32, rng.uniform(0.01, 0.1, (M, K // gk)).astype(np.float32), (1, gk)),
+                  O.Q_WEI: O.Quant(3, O.F32, rng.uniform(0.01, 0.1, (K // gk, N)).astype(np.float32), (gk, 1))}
+    else:
+        scales = {O.Q_SRC: O.Quant(1, O.F32, rng.uniform(0.01, 0.1, M).astype(np.float32)),
+                  O.Q_WEI: O.Quant(2, O.F32, rng.uniform(0.01, 0.1, N).astype(np.float32))}
+    out = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("QMM_ORACLE_SCALAR", mode)
+        dst = np.zeros((M, N), np.float32)
+        O.matmul(T(sdt, src), wt, T(O.F32, dst), scales=scales)
+        acc = O.matmul_s32_acc(T(sdt, src), wt, T(O.S32, np.zeros((M, N), np.int32)))
+        out[mode] = (dst.view(np.uint32).copy(), acc.copy())
+    assert np.array_equal(out["0"][0], out["1"][0])
+    assert np.array_equal(out["0"][1], out["1"][1])
+    # and both are the integer product itself
+    exact = src.astype(np.int64) @ wei.astype(np.int64)
+    assert np.array_equal(out["0"][1].astype(np.int64), exact)
