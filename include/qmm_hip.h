@@ -267,7 +267,8 @@ QMM_API int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc,
  *     MFMAs; int8 with 256 x 128 tiles and two workgroups per CU up to K 2048,
  *     256 x 256 tiles and one per CU beyond), 2 = 256 x 128 two per CU wherever it
  *     applies, 3 = 256 x 256 one per CU, 4 = as 3 with one workgroup per tile
- *     instead of one per CU walking its tiles, 0 = the loops on 32 x 32 MFMAs */
+ *     instead of one per CU walking its tiles, 5 = as 3 with every workgroup
+ *     starting at once (no half-tile stagger), 0 = the loops on 32 x 32 MFMAs */
 
 /* ---- measurement switches of the 256 x 256 GEMM kernels ----
  * QMM_MEASURE (environment, read at plan creation like the overrides above):

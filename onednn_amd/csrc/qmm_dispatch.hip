@@ -941,7 +941,7 @@ int qmm_matmul_plan_create(
     p->scratch_bytes = qmm_matmul_scratch_size(impl, desc);
     p->gemm_variant = env_variant("QMM_GEMM_VARIANT", 0, 6, 0);
     p->w4a8_variant = env_variant("QMM_W4A8_VARIANT", 0, 5, 0);
-    p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 4, 1);
+    p->b8x_variant = env_variant("QMM_B8X_VARIANT", 0, 5, 1);
     p->measure = env_variant("QMM_MEASURE", 0, 3, 0);
     // resolve the static scratch's address on the current device now, so that
     // qmm_matmul_launch_static_scratch() finds it ready (a plan used on another
@@ -1092,6 +1092,7 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
                 | (plan->b8x_variant == 2 ? GEMM_TWO_PER_CU : 0)
                 | (plan->b8x_variant >= 3 ? GEMM_ONE_PER_CU : 0)
                 | (plan->b8x_variant == 4 ? GEMM_NOT_PERSISTENT : 0)
+                | (plan->b8x_variant == 5 ? GEMM_NO_STAGGER : 0)
                 | (plan->measure & 1 ? GEMM_SKIP_EPILOGUE : 0)
                 | (plan->measure & 2 ? GEMM_STAMPS : 0);
         fold_batch(D.src, D.dst, g.a_sb);

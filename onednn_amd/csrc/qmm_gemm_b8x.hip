@@ -1036,6 +1036,27 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int ntiles = p.tiles_m * p.tiles_n;
     const int per = (ntiles + 7) / 8;
     const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
+    // Out of step on purpose: when an XCD's share is F whole rounds and R more
+    // tiles, the workgroups without a tile in that last round start half a
+    // tile late (their CUs would idle at the end instead). The two groups then
+    // run their main loops and their epilogues half a tile apart for the
+    // whole launch: the power a CU does not draw while it converts and stores
+    // a tile is there for the main loops of the others, which run at a higher
+    // clock than when every CU multiplies at once.
+    {
+        const int F = per / W, R = per - F * W;
+        if (!(p.switches & GEMM_NO_STAGGER) && F >= 2 && R > 0
+                && (int)(blockIdx.x >> 3) >= R && gridDim.y == 1) {
+            if (tid == 0) {
+                // half of (prologue + epilogue ~ 12 us, 0.64 us a k-step), in
+                // ticks of the constant 100 MHz counter
+                const unsigned long long ticks = 600 + (p.K / BK) * 32;
+                const unsigned long long t0 = wall_clock64();
+                while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(64);
+            }
+            __syncthreads();
+        }
+    }
     for (int slot = blockIdx.x >> 3, it = 0; slot < per; slot += W, it++) {
         const int lt = xcd * per + slot;
         if (lt >= ntiles) break;

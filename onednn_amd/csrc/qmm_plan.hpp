@@ -149,7 +149,10 @@ enum {
     GEMM_ONE_PER_CU = 16,
     // the int8 256 x 256 kernel on 16 x 16 MFMAs: one workgroup per tile
     // instead of one per CU walking its tiles (a measurement switch)
-    GEMM_NOT_PERSISTENT = 32
+    GEMM_NOT_PERSISTENT = 32,
+    // the persistent int8 kernel with all its workgroups starting together
+    // (a measurement switch)
+    GEMM_NO_STAGGER = 64
 };
 
 struct gemm_params_t {
