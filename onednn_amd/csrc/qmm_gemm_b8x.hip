@@ -1043,10 +1043,16 @@ gemm_b8y_kernel(const gemm_params_t p) {
     // whole launch: the power a CU does not draw while it converts and stores
     // a tile is there for the main loops of the others, which run at a higher
     // clock than when every CU multiplies at once.
+    // The two groups no longer meet each other's operand slices in the L2, so
+    // where the split is 16 : 16 each group takes a 4 x 4 block of tiles (4 + 4
+    // operand panels) out of a round's 8 x 4 instead of 8 x 2 (8 + 2).
+    bool square_groups = false;
     {
         const int F = per / W, R = per - F * W;
-        if (!(p.switches & GEMM_NO_STAGGER) && F >= 2 && R > 0
-                && (int)(blockIdx.x >> 3) >= R && gridDim.y == 1) {
+        const bool late_half = !(p.switches & GEMM_NO_STAGGER) && F >= 2
+                && R > 0 && gridDim.y == 1;
+        square_groups = late_half && W == 32 && R == 16;
+        if (late_half && (int)(blockIdx.x >> 3) >= R) {
             if (tid == 0) {
                 // half of (prologue + epilogue ~ 12 us, 0.64 us a k-step), in
                 // ticks of the constant 100 MHz counter
@@ -1058,9 +1064,20 @@ gemm_b8y_kernel(const gemm_params_t p) {
         }
     }
     for (int slot = blockIdx.x >> 3, it = 0; slot < per; slot += W, it++) {
-        const int lt = xcd * per + slot;
-        if (lt >= ntiles) break;
         constexpr int GROUP_M = 8;
+        int lt = xcd * per + slot;
+        if (square_groups && it * W + 32 <= per) {
+            // a whole round: 32 consecutive tiles, 8 rows x 4 columns when they
+            // start on a row-group boundary and lie in one full row group
+            const int w = blockIdx.x >> 3, base = lt - w;
+            const int o = base % (GROUP_M * p.tiles_n);
+            const int rows_left
+                    = p.tiles_m - base / (GROUP_M * p.tiles_n) * GROUP_M;
+            if (o % GROUP_M == 0 && o + 32 <= GROUP_M * p.tiles_n
+                    && rows_left >= GROUP_M)
+                lt = base + ((w & 15) >> 2) * GROUP_M + (w >> 4) * 4 + (w & 3);
+        }
+        if (lt >= ntiles) break;
         const int group = lt / (GROUP_M * p.tiles_n);
         const int first_m = group * GROUP_M;
         const int gsz = min(p.tiles_m - first_m, GROUP_M);

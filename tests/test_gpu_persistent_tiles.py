@@ -52,6 +52,14 @@ CASES = {
     # two matrices of 4 x 40 tiles: an XCD's share (20) is smaller than its CUs, one grid row per matrix
     "batched_small_share_f32": lambda: cases.int8_linear(1024, 1024, 10240, 307, src_dt=dt.s8, dst_dt=dt.f32, src_zp=None,
                                                          batch=(2,)),
+    # 8 x 80 tiles, 80 per XCD = two whole rounds and 16 more: the 16 workgroups without a tile in the last round start
+    # late and the whole rounds hand each half of the workgroups a 4 x 4 block of tiles (another tile order)
+    "late_half_square_blocks_s8": lambda: cases.int8_linear(2048, 1024, 20480, 308, src_dt=dt.s8, dst_dt=dt.s8,
+                                                            src_zp=None, per_token=True),
+    # 12 x 53 tiles, 80 per XCD again, but rounds that straddle the 8-row groups or lie in the 4-row group keep the
+    # plain order
+    "late_half_partial_row_group_f32": lambda: cases.int8_linear(3072, 1024, 13568, 309, src_dt=dt.s8, dst_dt=dt.f32,
+                                                                 src_zp=None, per_token=True),
     "three_tiles_each_s8": lambda: cases.int8_linear(2048, 1024, 18432, 306, src_dt=dt.s8, dst_dt=dt.s8, src_zp=None,
                                                      per_token=True),
 }
