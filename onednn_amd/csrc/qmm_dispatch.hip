@@ -1380,6 +1380,8 @@ int qmm_matmul_launch(const qmm_plan_t *plan, const qmm_matmul_args_t *args,
         g.A = (const uint8_t *)args->src;
         g.lda = 2 * D.src.strides[0];
         g.B = packed;
+        g.switches = (plan->b8x_variant == 4 ? GEMM_NOT_PERSISTENT : 0)
+                | (plan->b8x_variant == 5 ? GEMM_NO_STAGGER : 0);
         g.wei_zp = wz.set ? args->zps[QMM_WEI] : nullptr;
         g.wei_zp_dt = wz.dt;
         g.wei_zp_sn = wz.set && (wz.mask & 2) ? 1 : 0;

@@ -890,6 +890,31 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QY_ROW(3, CB, , , , ) QY_ROW(4, CB, , , , ) QY_ROW(5, CB, , , , ) \
     QY_ROW(6, CB, , , , ) QY_ROW(7, CB, , , , )
 
+// The persistent kernels put their workgroups out of step on purpose: when an
+// XCD's share is F whole rounds and R more tiles, the workgroups without a tile
+// in that last round start half a tile late (their CUs would idle at the end
+// instead). The two groups then run their main loops and their epilogues half
+// a tile apart for the whole launch: the power a CU does not draw while it
+// converts and stores a tile is there for the main loops of the others, which
+// run at a higher clock than when every CU multiplies at once. Returns whether
+// the launch has such a late half; half_tile_ticks in ticks of the constant
+// 100 MHz counter (a bounded wait: every wave leaves it).
+QMM_D bool late_half_start(const gemm_params_t &p, int per, int W, int tid,
+        unsigned long long half_tile_ticks) {
+    const int F = per / W, R = per - F * W;
+    const bool late_half = !(p.switches & GEMM_NO_STAGGER) && F >= 2 && R > 0
+            && gridDim.y == 1;
+    if (late_half && (int)(blockIdx.x >> 3) >= R) {
+        if (tid == 0) {
+            const unsigned long long t0 = wall_clock64();
+            while (wall_clock64() - t0 < half_tile_ticks)
+                __builtin_amdgcn_s_sleep(64);
+        }
+        __syncthreads();
+    }
+    return late_half;
+}
+
 #if defined(QMM_B8X_PART) && (QMM_B8X_PART == 4 || QMM_B8X_PART == 5)
 // One block tile of gemm_b8y_kernel.
 // ODD: an odd number of k-steps (the register buffers alternate per k-step, so
@@ -1036,33 +1061,13 @@ gemm_b8y_kernel(const gemm_params_t p) {
     const int ntiles = p.tiles_m * p.tiles_n;
     const int per = (ntiles + 7) / 8;
     const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
-    // Out of step on purpose: when an XCD's share is F whole rounds and R more
-    // tiles, the workgroups without a tile in that last round start half a
-    // tile late (their CUs would idle at the end instead). The two groups then
-    // run their main loops and their epilogues half a tile apart for the
-    // whole launch: the power a CU does not draw while it converts and stores
-    // a tile is there for the main loops of the others, which run at a higher
-    // clock than when every CU multiplies at once.
-    // The two groups no longer meet each other's operand slices in the L2, so
-    // where the split is 16 : 16 each group takes a 4 x 4 block of tiles (4 + 4
-    // operand panels) out of a round's 8 x 4 instead of 8 x 2 (8 + 2).
-    bool square_groups = false;
-    {
-        const int F = per / W, R = per - F * W;
-        const bool late_half = !(p.switches & GEMM_NO_STAGGER) && F >= 2
-                && R > 0 && gridDim.y == 1;
-        square_groups = late_half && W == 32 && R == 16;
-        if (late_half && (int)(blockIdx.x >> 3) >= R) {
-            if (tid == 0) {
-                // half of (prologue + epilogue ~ 12 us, 0.64 us a k-step), in
-                // ticks of the constant 100 MHz counter
-                const unsigned long long ticks = 600 + (p.K / BK) * 32;
-                const unsigned long long t0 = wall_clock64();
-                while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(64);
-            }
-            __syncthreads();
-        }
-    }
+    // half of (prologue + epilogue ~ 12 us, 0.64 us a k-step). The two groups
+    // no longer meet each other's operand slices in the L2, so where the split
+    // is 16 : 16 each group takes a 4 x 4 block of tiles (4 + 4 operand panels)
+    // out of a round's 8 x 4 instead of 8 x 2 (8 + 2).
+    const bool square_groups
+            = late_half_start(p, per, W, tid, 600 + (p.K / BK) * 32) && W == 32
+            && per % 32 == 16;
     for (int slot = blockIdx.x >> 3, it = 0; slot < per; slot += W, it++) {
         constexpr int GROUP_M = 8;
         int lt = xcd * per + slot;

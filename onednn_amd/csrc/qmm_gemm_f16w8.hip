@@ -124,14 +124,16 @@ gemm_f16w8_kernel(const gemm_params_t p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
 
+    // persistent, as gemm_b8y_kernel: workgroup w of an XCD walks the tiles
+    // w, w + W, ... of the XCD's share, the workgroups without a tile in the
+    // last round half a tile behind the others
     const int ntiles = p.tiles_m * p.tiles_n;
-    int lt;
-    {
-        const int per = (ntiles + 7) / 8;
-        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-        lt = xcd * per + slot;
-        if (slot >= per || lt >= ntiles) return;
-    }
+    const int per = (ntiles + 7) / 8;
+    const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
+    late_half_start(p, per, W, tid, 600 + (p.K / 32) * 32);
+    for (int slot = blockIdx.x >> 3; slot < per; slot += W) {
+    const int lt = xcd * per + slot;
+    if (lt >= ntiles) break;
     constexpr int GROUP_M = 8;
     const int group = lt / (GROUP_M * p.tiles_n);
     const int first_m = group * GROUP_M;
@@ -280,15 +282,19 @@ gemm_f16w8_kernel(const gemm_params_t p) {
 
     tile_epilogue<true, false>(
             p, acc, lds, lds_base, wave, lane, m0, n0, wm0, wn0, bz);
+    // the staging area and the operand tables are the next tile's ring and
+    // tables
+    __syncthreads();
+    }
 }
 
 #if QMM_F16W8_PART == 0
 void launch_f16w8_even(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_f16w8_kernel<false>, p, stream);
+    launch_b8y_persistent(gemm_f16w8_kernel<false>, p, stream);
 }
 #else
 void launch_f16w8_odd(const gemm_params_t &p, hipStream_t stream) {
-    launch_b8x(gemm_f16w8_kernel<true>, p, stream);
+    launch_b8y_persistent(gemm_f16w8_kernel<true>, p, stream);
 }
 #endif
 
