@@ -4,9 +4,10 @@
 // semantics src/gpu/intel/ocl/ref_sdpa.cl:21-78; its test's gold path is the
 // matmul -> softmax -> matmul chain, tests/gtests/internals/test_sdpa.cpp:893-
 // 1043). Q, K, V, dst are f16 or bf16 (the kernels' BF flag; the text below
-// says f16 for both); with f16, K and V may instead be an s8 / u8 cache with
-// one scale (and zero point) per key, dequantized to f16 as the chain's reorder
-// does: f16(scale * (x - zero_point)).
+// says f16 for both); K and V may instead be an s8 / u8 cache with one scale
+// (and zero point) per key, dequantized to the queries' type as the chain's
+// reorder does: f16(scale * (x - zero_point)), in f32 arithmetic for bf16
+// queries and for f32 scales / s32 zero points.
 //
 // The scores never leave the CU. A workgroup owns 128 queries of one head (four
 // waves of 32) and walks the keys 32 at a time:
@@ -304,9 +305,9 @@ sdpa_f16_kernel(const sdpa_params_t p) {
                     const float kf = (float)((kw[j >> 2] >> (8 * (j & 3))) & 0xff);
                     const float vf = (float)((vw[j >> 2] >> (8 * (j & 3))) & 0xff);
                     kh[j] = __builtin_bit_cast(
-                            uint16_t, (_Float16)(pks[n] * (kf - kzb)));
+                            uint16_t, cvt16<BF>(pks[n] * (kf - kzb)));
                     vh[j] = __builtin_bit_cast(
-                            uint16_t, (_Float16)(pvs[n] * (vf - vzb)));
+                            uint16_t, cvt16<BF>(pvs[n] * (vf - vzb)));
                 }
                 kv = make_uint4(kh[0] | (kh[1] << 16), kh[2] | (kh[3] << 16),
                         kh[4] | (kh[5] << 16), kh[6] | (kh[7] << 16));
@@ -622,7 +623,7 @@ sdpa_decode_kernel(const sdpa_params_t p) {
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const float f = (float)((w[j >> 2] >> (8 * (j & 3))) & 0xff);
-            h[j] = __builtin_bit_cast(uint16_t, (_Float16)(s1 * (f - zb)));
+            h[j] = __builtin_bit_cast(uint16_t, cvt16<BF>(s1 * (f - zb)));
         }
         return make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16),
                 h[4] | (h[5] << 16), h[6] | (h[7] << 16));
@@ -878,10 +879,8 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     if (d.k.ndims != nd || d.v.ndims != nd || d.dst.ndims != nd) return false;
     if ((d.q.dt != dt_f16 && d.q.dt != dt_bf16) || d.dst.dt != d.q.dt) return false;
     if (d.k.dt != d.v.dt) return false;
-    // K / V in the queries' type, or (f16 only) an 8-bit cache
-    if (d.k.dt != d.q.dt
-            && !(d.q.dt == dt_f16 && (d.k.dt == dt_s8 || d.k.dt == dt_u8)))
-        return false;
+    // K / V in the queries' type, or an 8-bit cache
+    if (d.k.dt != d.q.dt && d.k.dt != dt_s8 && d.k.dt != dt_u8) return false;
     const int64_t Qn = d.q.dims[nd - 2], D = d.q.dims[nd - 1];
     const int64_t S = d.k.dims[nd - 1];
     if (d.k.dims[nd - 2] != D || d.v.dims[nd - 2] != S) return false;
@@ -981,7 +980,8 @@ bool supported(const qmm_sdpa_desc_t &d, sdpa_params_t *out) {
     p.causal = d.causal;
     p.kv_dt = d.k.dt;
     p.bf = d.q.dt == dt_bf16;
-    p.fastq = quant && (!d.k_scale.set || d.k_scale.dt == dt_f16)
+    p.fastq = quant && d.q.dt == dt_f16
+            && (!d.k_scale.set || d.k_scale.dt == dt_f16)
             && (!d.v_scale.set || d.v_scale.dt == dt_f16)
             && (!d.k_zp.set || d.k_zp.dt == dt_s8 || d.k_zp.dt == dt_u8)
             && (!d.v_zp.set || d.v_zp.dt == dt_s8 || d.v_zp.dt == dt_u8);
@@ -1048,7 +1048,7 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
     p.v_zp = desc->v_zp.set ? args->v_zp : nullptr;
     const int D = (int)desc->q.dims[desc->q.ndims - 1];
     const bool qn = p.kv_dt != desc->q.dt, mk = p.mask != nullptr;
-    const bool bf = p.bf != 0; // never together with qn
+    const bool bf = p.bf != 0;
     if (p.Qn <= 16) {
         const sdpa_split_t sp
                 = decode_split((int64_t)p.B0 * p.B1, p.S, p.Qn, p.causal != 0);
@@ -1061,8 +1061,7 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
             hipLaunchKernelGGL(kern, dgrid, dim3(SDPA_WAVES * 64), 0,
                     (hipStream_t)hip_stream, p);
         };
-        // template arguments from the run-time choices (bf16 queries never
-        // come with an 8-bit cache: supported())
+        // template arguments from the run-time choices
 #define SDPA_PICK(KERN, GO, DCV) \
     switch ((qn ? 4 : 0) | (bf ? 2 : 0) | (mk ? 1 : 0)) { \
         case 0: GO(KERN<DCV, false, false, false>); break; \
@@ -1071,6 +1070,8 @@ int qmm_sdpa_launch(const qmm_sdpa_desc_t *desc, const qmm_sdpa_args_t *args,
         case 3: GO(KERN<DCV, false, true, true>); break; \
         case 4: GO(KERN<DCV, true, false, false>); break; \
         case 5: GO(KERN<DCV, true, true, false>); break; \
+        case 6: GO(KERN<DCV, true, false, true>); break; \
+        case 7: GO(KERN<DCV, true, true, true>); break; \
         default: return QMM_UNIMPLEMENTED; \
     }
         switch (D) {

@@ -162,14 +162,16 @@ def test_f16_attention(ctx, case, qdt):
 
 @pytest.mark.parametrize("kv_dt,with_zp", [(dt.s8, True), (dt.u8, True), (dt.s8, False)], ids=str)
 @pytest.mark.parametrize("Qn", [1, 96])
-@pytest.mark.parametrize("D", [128, 32, 96, 256])
-def test_quantized_cache(ctx, kv_dt, with_zp, Qn, D):
+@pytest.mark.parametrize("D,qdt", [(128, dt.f16), (32, dt.f16), (96, dt.f16), (256, dt.f16), (128, dt.bf16), (64, dt.bf16),
+                                   (256, dt.bf16)], ids=str)
+def test_quantized_cache(ctx, kv_dt, with_zp, Qn, D, qdt):
     """K / V as an 8-bit cache with one f16 scale (and zero point) per head and key: the kernel dequantizes while
-    staging, to the same f16 values as the chain's reorder (checked through the oracle's reorder)."""
+    staging, to the same values of the queries' type (f16 or bf16) as the chain's reorder (checked through the
+    oracle's reorder)."""
     MB, H, S = 2, 4, 257
-    say("sdpa quantized cache %s zp=%s queries %d head size %d" % (kv_dt, with_zp, Qn, D))
+    say("sdpa quantized cache %s zp=%s queries %d head size %d %s" % (kv_dt, with_zp, Qn, D, qdt))
     r = np.random.default_rng(40 + Qn)
-    q = f16(r.standard_normal((MB, H, Qn, D)))
+    q = f16(r.standard_normal((MB, H, Qn, D)), qdt)
     lo, hi, npdt = (-128, 128, np.int8) if kv_dt == dt.s8 else (0, 256, np.uint8)
     kq = r.integers(lo, hi, (MB, H, S, D)).astype(npdt)
     vq = r.integers(lo, hi, (MB, H, S, D)).astype(npdt)
@@ -179,16 +181,17 @@ def test_quantized_cache(ctx, kv_dt, with_zp, Qn, D):
     vzp = r.integers(lo // 16 + (100 if kv_dt == dt.u8 else 0), hi // 16 + (100 if kv_dt == dt.u8 else 0), (H, S)).astype(npdt)
     kqa = (0b1110, (D, 1), dt.f16, ksc, zdt, kzp if with_zp else None)
     vqa = (0b1110, (1, D), dt.f16, vsc, zdt, vzp if with_zp else None)
-    got = run_sdpa(ctx, q, kq, vq, scale=1.0 / np.sqrt(D), causal=(Qn > 1), kv_dt=kv_dt, k_q=kqa, v_q=vqa)
-    # the dequantized cache as the reference chain's reorder produces it (oracle reorder, f16)
+    got = run_sdpa(ctx, q, kq, vq, scale=1.0 / np.sqrt(D), causal=(Qn > 1), kv_dt=kv_dt, k_q=kqa, v_q=vqa, qdt=qdt)
+    # the dequantized cache as the reference chain's reorder produces it (oracle reorder, to the queries' type)
     kd, vd = np.zeros((MB, H, S, D), np.uint16), np.zeros((MB, H, S, D), np.uint16)
     for raw, sc, zp, outd in ((kq, ksc, kzp, kd), (vq, vsc, vzp, vd)):
-        O.reorder(O.Tensor(kv_dt, [MB, H, S, D], raw), O.Tensor(dt.f16, [MB, H, S, D], outd),
+        O.reorder(O.Tensor(kv_dt, [MB, H, S, D], raw), O.Tensor(qdt, [MB, H, S, D], outd),
                   src_scale=O.Quant(0b1110, dt.f16, sc, (1, D)),
                   src_zp=O.Quant(0b1110, zdt, zp, (1, D)) if with_zp else None)
-    s_eff = float(f16_to_f64(f16(np.array([1.0 / np.sqrt(D)])))[0])
-    gold = attention64(f16_to_f64(q), np.swapaxes(f16_to_f64(kd), -1, -2), f16_to_f64(vd), s_eff, None, Qn > 1, 1)
-    bad, total, worst = reference_rule(f16_to_f64(got), gold)
+    s_eff = float(f16_to_f64(f16(np.array([1.0 / np.sqrt(D)]), qdt), qdt)[0])
+    gold = attention64(f16_to_f64(q, qdt), np.swapaxes(f16_to_f64(kd, qdt), -1, -2), f16_to_f64(vd, qdt), s_eff, None,
+                       Qn > 1, 1)
+    bad, total, worst = reference_rule(f16_to_f64(got, qdt), gold, 0.0079 if qdt == dt.bf16 else 0.001466)
     print("[sdpa quantized] %d of %d outside the threshold, max diff %.2e" % (bad, total, worst))
     assert bad <= total * 0.0006
 
@@ -318,8 +321,7 @@ def test_what_the_kernel_does_not_take_is_unimplemented(ctx):
     for bad in (dict(q=md([1, 2, 16, 80]), k=md([1, 2, 80, 32], t="abdc"), v=md([1, 2, 32, 80]), o=md([1, 2, 16, 80])),  # head size
                 dict(k=md([1, 2, 64, 32])),                                    # keys contiguous instead of head size
                 dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16)),  # bf16 queries on f16 keys
-                dict(q=md([1, 2, 16, 64], dt.bf16), o=md([1, 2, 16, 64], dt.bf16),  # bf16 on an 8-bit cache
-                     k=md([1, 2, 64, 32], dt.s8, t="abdc"), v=md([1, 2, 32, 64], dt.s8))):
+                dict(k=md([1, 2, 64, 32], dt.s32, t="abdc"), v=md([1, 2, 32, 64], dt.s32))):  # a 32-bit cache
         with pytest.raises(dnnl.error) as e:
             make(**bad)
         assert e.value.status == dnnl.status.unimplemented
