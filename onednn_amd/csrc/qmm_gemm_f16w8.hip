@@ -125,12 +125,11 @@ gemm_f16w8_kernel(const gemm_params_t p) {
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
 
     // persistent, as gemm_b8y_kernel: workgroup w of an XCD walks the tiles
-    // w, w + W, ... of the XCD's share, the workgroups without a tile in the
-    // last round half a tile behind the others
+    // w, w + W, ... of the XCD's share (all in step: the late half of that
+    // kernel measured 1 % slower here)
     const int ntiles = p.tiles_m * p.tiles_n;
     const int per = (ntiles + 7) / 8;
     const int xcd = blockIdx.x & 7, W = gridDim.x >> 3;
-    late_half_start(p, per, W, tid, 600 + (p.K / 32) * 32);
     for (int slot = blockIdx.x >> 3; slot < per; slot += W) {
     const int lt = xcd * per + slot;
     if (lt >= ntiles) break;
