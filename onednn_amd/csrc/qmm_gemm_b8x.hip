@@ -890,8 +890,8 @@ gemm_b8x_kernel(const gemm_params_t p) {
     QY_ROW(3, CB, , , , ) QY_ROW(4, CB, , , , ) QY_ROW(5, CB, , , , ) \
     QY_ROW(6, CB, , , , ) QY_ROW(7, CB, , , , )
 
-// The persistent kernels put their workgroups out of step on purpose: when an
-// XCD's share is F whole rounds and R more tiles, the workgroups without a tile
+// gemm_b8y_kernel puts its workgroups out of step on purpose: when an XCD's
+// share is F >= 1 whole rounds and R more tiles, the workgroups without a tile
 // in that last round start half a tile late (their CUs would idle at the end
 // instead). The two groups then run their main loops and their epilogues half
 // a tile apart for the whole launch: the power a CU does not draw while it
@@ -902,7 +902,7 @@ gemm_b8x_kernel(const gemm_params_t p) {
 QMM_D bool late_half_start(const gemm_params_t &p, int per, int W, int tid,
         unsigned long long half_tile_ticks) {
     const int F = per / W, R = per - F * W;
-    const bool late_half = !(p.switches & GEMM_NO_STAGGER) && F >= 2 && R > 0
+    const bool late_half = !(p.switches & GEMM_NO_STAGGER) && F >= 1 && R > 0
             && gridDim.y == 1;
     if (late_half && (int)(blockIdx.x >> 3) >= R) {
         if (tid == 0) {
